@@ -1,0 +1,231 @@
+/* mjt.h -- C ABI of libmjt.so: the MI355X (gfx950) execution path for
+ * Jittor's meta-operators.
+ *
+ * Every entry point returns 0 on success or a negative mjt_status; the text
+ * of the last failure on the calling thread is available from
+ * mjt_last_error().  Nothing throws or aborts across this boundary.  All
+ * tensor buffers are dense, row-major device memory owned by the caller
+ * (the reference allocates every group output before calling the kernel,
+ * python/jittor/src/executor.cc:575-577, and kernels only read
+ * Var::mem_ptr/shape/dtype, python/jittor/src/var.h:18-49).  Work is queued
+ * on one stream per device and is asynchronous; mjt_sync() waits for it.
+ *
+ * Paths in the citations below are relative to python/jittor/src/ of the
+ * reference tree.
+ */
+#ifndef MJT_H_
+#define MJT_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MJT_MAX_DIM 10 /* ops/reindex_op.cc:43: at most 10 dims */
+
+typedef enum {
+    MJT_OK = 0,
+    MJT_ERR_INVALID = -1,   /* bad descriptor (the reference's CHECK/ASSERT) */
+    MJT_ERR_UNSUPPORTED = -2,
+    MJT_ERR_COMPILE = -3,   /* runtime kernel specialisation failed */
+    MJT_ERR_DEVICE = -4,    /* HIP runtime error */
+    MJT_ERR_NOT_INIT = -5
+} mjt_status;
+
+/* dtype codes: order of misc/nano_string.h:17-31 */
+typedef enum {
+    MJT_VOID = 0, MJT_BOOL, MJT_INT8, MJT_INT16, MJT_INT32, MJT_INT64,
+    MJT_UINT8, MJT_UINT16, MJT_UINT32, MJT_UINT64, MJT_FLOAT16, MJT_FLOAT32,
+    MJT_FLOAT64, MJT_BFLOAT16, MJT_DTYPE_COUNT
+} mjt_dtype;
+
+/* op codes: order of misc/nano_string.h:33-89 (binary ops, then unary ops).
+ * MJT_OP_VOID is the "void" reduce op of ops/reindex_reduce_op.cc:34. */
+typedef enum {
+    MJT_OP_POW = 0, MJT_OP_MAXIMUM, MJT_OP_MINIMUM, MJT_OP_ADD,
+    MJT_OP_SUBTRACT, MJT_OP_MULTIPLY, MJT_OP_DIVIDE, MJT_OP_FLOOR_DIVIDE,
+    MJT_OP_MOD, MJT_OP_LESS, MJT_OP_LESS_EQUAL, MJT_OP_GREATER,
+    MJT_OP_GREATER_EQUAL, MJT_OP_EQUAL, MJT_OP_NOT_EQUAL, MJT_OP_LEFT_SHIFT,
+    MJT_OP_RIGHT_SHIFT, MJT_OP_LOGICAL_AND, MJT_OP_LOGICAL_OR,
+    MJT_OP_LOGICAL_XOR, MJT_OP_BITWISE_AND, MJT_OP_BITWISE_OR,
+    MJT_OP_BITWISE_XOR, MJT_OP_MEAN,
+    MJT_OP_ABS, MJT_OP_NEGATIVE, MJT_OP_LOGICAL_NOT, MJT_OP_BITWISE_NOT,
+    MJT_OP_LOG, MJT_OP_EXP, MJT_OP_SQRT, MJT_OP_ROUND, MJT_OP_FLOOR,
+    MJT_OP_CEIL, MJT_OP_ROUND_INT, MJT_OP_FLOOR_INT, MJT_OP_CEIL_INT,
+    MJT_OP_CAST, MJT_OP_SIN, MJT_OP_ASIN, MJT_OP_SINH, MJT_OP_ASINH,
+    MJT_OP_TAN, MJT_OP_ATAN, MJT_OP_TANH, MJT_OP_ATANH, MJT_OP_COS,
+    MJT_OP_ACOS, MJT_OP_COSH, MJT_OP_ACOSH, MJT_OP_ERF, MJT_OP_ERFINV,
+    MJT_OP_SIGMOID, MJT_OP_VOID, MJT_OP_COUNT
+} mjt_op;
+
+/* Dense row-major tensor: the fields a kernel reads from a reference Var
+ * (var.h:18-49: mem_ptr, shape, dtype; no strides). */
+typedef struct {
+    void*   ptr;
+    int32_t dtype;               /* mjt_dtype */
+    int32_t ndim;                /* 1..MJT_MAX_DIM */
+    int64_t shape[MJT_MAX_DIM];
+} mjt_tensor;
+
+typedef struct {
+    char     name[256];
+    char     arch[64];
+    int32_t  compute_units;
+    int32_t  clock_khz;
+    int32_t  mem_clock_khz;
+    int32_t  mem_bus_bits;
+    int32_t  lds_bytes_per_block;
+    int32_t  wavefront;
+    uint64_t hbm_bytes;
+    uint64_t l2_bytes;
+} mjt_device_info;
+
+/* ---- runtime ---------------------------------------------------------- */
+/* device >= 0: bind to that gfx950 device.  device == -1: compile-only mode
+ * for build checks on a machine without a GPU -- every entry point validates
+ * its descriptors and specialises + compiles its kernels for gfx950, but
+ * nothing is allocated or launched. */
+int         mjt_init(int device);
+void        mjt_shutdown(void);
+const char* mjt_last_error(void);
+int         mjt_get_device_info(mjt_device_info* out);
+const char* mjt_dtype_name(int dtype);
+const char* mjt_op_name(int op);
+int         mjt_dtype_from_name(const char* name);   /* <0 if unknown */
+int         mjt_op_from_name(const char* name);      /* <0 if unknown */
+
+/* Device memory.  Replaces Var::alloc / Allocator::alloc (var.cc:114-127). */
+int mjt_alloc(size_t bytes, void** out);
+int mjt_free(void* p);
+int mjt_h2d(void* dst, const void* src, size_t bytes);   /* synchronous */
+int mjt_d2h(void* dst, const void* src, size_t bytes);   /* synchronous */
+int mjt_d2d(void* dst, const void* src, size_t bytes);   /* copy kernel, async */
+int mjt_fill_u32(void* dst, uint32_t pattern, size_t n_words); /* async */
+int mjt_sync(void);
+
+/* Timing on the library's stream (the role of Profiler::record_and_run,
+ * profiler/profiler.cc:229-347). */
+int mjt_event_create(void** ev);
+int mjt_event_record(void* ev);
+int mjt_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for stop */
+int mjt_event_destroy(void* ev);
+
+/* ---- ReduceOp: ops/reduce_op.cc:374-399 -------------------------------
+ * y = reduce(x, op) over the axes set in reduce_mask (bit d = axis d of x is
+ * reduced, ops/reduce_op.h:14).  y->shape is the kept axes (with or without
+ * 1s for reduced axes: only the element count is checked).  Accumulation is
+ * in y->dtype starting from the identity init_OP
+ * (type/common_op_type.cc:116-117,142-151: lowest()/max() for max/min). */
+int mjt_reduce(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask);
+
+/* ---- ReindexOp: ops/reindex_op.cc:111-139 -----------------------------
+ * y[i..] = overflow ? Tx(overflow_value) : x[idx_0(i..), ..., idx_{XDIM-1}(i..)]
+ * indexes[d] and overflow_conditions[k] are C integer expressions over
+ * i0..i{YDIM-1}, xshapeK, yshapeK, xstrideK, ystrideK, XDIM, YDIM and
+ * @eK(a,b,..) = extras[K] at that coordinate (ops/reindex_op.h:58-68,
+ * op_compiler.cc:665-699).  n_indexes must equal x->ndim
+ * (ops/reindex_op.cc:83).  y->dtype must equal x->dtype. */
+int mjt_reindex(const mjt_tensor* x, const mjt_tensor* y,
+                int n_indexes, const char* const* indexes,
+                double overflow_value,
+                int n_overflow_conditions, const char* const* overflow_conditions,
+                int n_extras, const mjt_tensor* extras);
+
+/* ---- ReindexReduceOp: ops/reindex_reduce_op.cc:93-131 -----------------
+ * x (the output, shape given) is filled with init_OP, then for every
+ * coordinate of y (the input): x[idx(i..)] = OP(x[idx(i..)], y[i..]) unless
+ * overflow.  op is a binary op other than mean, or MJT_OP_VOID
+ * (ops/reindex_reduce_op.cc:34).  n_indexes must equal x->ndim (:66).
+ * Updates are applied with device atomics: for float add the summation
+ * order is not the reference's sequential order. */
+int mjt_reindex_reduce(const mjt_tensor* y, const mjt_tensor* x, int op,
+                       int n_indexes, const char* const* indexes,
+                       int n_overflow_conditions, const char* const* overflow_conditions,
+                       int n_extras, const mjt_tensor* extras);
+
+/* ---- fused element-wise group: fused_op.h:29-60 -----------------------
+ * One kernel for a group of broadcast / unary / binary / ternary ops
+ * (ops/broadcast_to_op.cc:177-194, ops/unary_op.cc:1021-1027,
+ * ops/binary_op.cc:563-570, ops/ternary_op.cc:84-95) over one iteration
+ * space.  vars[] mirrors FusedOp::vars (role 0 input / 1 intermediate /
+ * 2 output, fused_op.h:13-20) plus by-value scalars (ops/array_op.cc:56-60);
+ * ops[] is FusedOp::ops in topological order. */
+typedef enum {
+    MJT_VAR_INPUT = 0, MJT_VAR_INTERMEDIATE = 1, MJT_VAR_OUTPUT = 2,
+    MJT_VAR_SCALAR = 3
+} mjt_var_role;
+
+typedef struct {
+    int32_t role;        /* mjt_var_role */
+    int32_t dtype;
+    void*   ptr;         /* input / output */
+    double  fvalue;      /* scalar: value when dtype is floating */
+    int64_t ivalue;      /* scalar: value when dtype is integer / bool */
+    /* inputs only: axes (of the iteration space) along which this tensor has
+     * extent 1 and is broadcast; 0 for a full-size tensor */
+    uint32_t bcast_mask;
+    uint32_t reserved;
+} mjt_fused_var;
+
+typedef enum {
+    MJT_FOP_UNARY = 0, MJT_FOP_BINARY = 1, MJT_FOP_TERNARY = 2,
+    MJT_FOP_BROADCAST = 3
+} mjt_fused_kind;
+
+typedef struct {
+    int32_t kind;        /* mjt_fused_kind */
+    int32_t op;          /* mjt_op for unary / binary */
+    int32_t in[3];       /* indices into vars[]; ternary: cond, x, y */
+    int32_t out;         /* index into vars[] */
+} mjt_fused_op;
+
+typedef struct {
+    int32_t ndim;
+    int64_t shape[MJT_MAX_DIM];   /* iteration space = shape of every output */
+    int32_t n_vars;
+    const mjt_fused_var* vars;
+    int32_t n_ops;
+    const mjt_fused_op* ops;
+} mjt_fused_desc;
+
+int mjt_fused_elementwise(const mjt_fused_desc* desc);
+
+/* ---- meta-op convolution ----------------------------------------------
+ * The group reindex + broadcast + multiply + reduce.add that
+ * python/jittor/nn.py:1251-1262 builds and opt/tuner/conv_tuner.cc:218-411
+ * recognises; the parameters are the ones the matcher solves for
+ * (conv_tuner.cc:333-356).  x [N,C,H,W], w [K,C,R,S], y [N,K,OH,OW].
+ * x and w are bfloat16 or float32 (same dtype); y is float32 (the
+ * accumulator) or x's dtype (narrowed by truncation for bfloat16,
+ * type/fp16_compute.h:238-241).  Out-of-range taps contribute 0. */
+typedef struct {
+    int32_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+} mjt_conv_params;
+
+int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y,
+                    const mjt_conv_params* p);
+
+/* ---- index-expression helper ------------------------------------------
+ * Parses one index expression (the language of opt/expr.h:38-143 restricted
+ * to what ops/reindex_op.h:58-68 allows) and, when it is affine in i0..i9
+ * with integer coefficients, returns c0 and coef[0..9].  Used by the host
+ * side to recognise the convolution pattern the way ConvTuner does
+ * (conv_tuner.cc:312-338).  Returns 1 if affine, 0 if valid but not affine,
+ * <0 on a syntax error.  Shapes are needed to fold xshapeK / yshapeK. */
+int mjt_expr_affine(const char* expr, const mjt_tensor* x, const mjt_tensor* y,
+                    int64_t* c0, int64_t coef[MJT_MAX_DIM]);
+
+/* Number of kernels specialised at run time so far, and how many launches
+ * reused one (the role of jit_ops / jit_fused_ops, op.cc:30, fused_op.cc:18). */
+int mjt_jit_stats(int64_t* compiled, int64_t* cache_hits);
+
+/* Name of the device kernel the most recent entry-point call on this thread
+ * launched (for profiles). */
+const char* mjt_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MJT_H_ */

@@ -1,0 +1,164 @@
+// Axis-set reduction kernels (reference semantics:
+// python/jittor/src/ops/reduce_op.cc:374-399 -- identity, then
+// y[kept] = OP(y[kept], x[kept, reduced]) with the accumulator in Ty).
+//
+// Specialised at run time through these macros:
+//   TX, TY          element types of x and y
+//   index_t         int or long long
+//   NK, NR          number of merged kept / reduced axes (each 0..5, NR >= 1)
+//   VEC             elements per vector load
+//   G               lanes that cooperate on one output (row kernel), power of 2 <= 64
+//   SPLIT           1: several workgroup rows share one output and write partials
+//   COMBINE(a, x)   first-level update, a is TY, x is TX
+//   MERGE(a, b)     update between two partial results, both TY
+//   INIT            identity, TY
+//   ROW             1: innermost merged axis is reduced; 0: it is kept
+//
+// The host merges adjacent axes of equal kind, so kept and reduced axes
+// alternate.  Row kernel: G lanes stride over the contiguous reduced run with
+// VEC-wide loads and finish with a cross-lane xor-shuffle tree, no LDS.
+// Column kernel: each lane owns VEC adjacent outputs and walks the reduced
+// coordinates; lanes of a wave read one contiguous run per step.
+// When SPLIT is set the partials go to a scratch buffer and a second launch of
+// the same kernel family folds them (two-pass grid reduce).
+
+struct Params { unsigned long long a[8 + 6 * 5]; };
+// a[0] x, a[1] y or partials, a[2] O (outputs), a[3] S (splits), a[4] rcount (double bits),
+// a[5] work items per split, a[6] total work items,
+// a[8+0*5..]  kshape   a[8+1*5..] kstride (in x)   a[8+2*5..] kdiv
+// a[8+3*5..]  rshape   a[8+4*5..] rstride (in x)   a[8+5*5..] rdiv
+
+#if USE64
+#define MJT_DIVQ(n, k, tab) ((n) / (index_t)p.a[8 + ((tab)-2) * 5 + (k)])
+#else
+#define MJT_DIVQ(n, k, tab) ((index_t)mjt_div((unsigned)(n), mjt_unpack_divmod(p.a[8 + (tab) * 5 + (k)], 0)))
+#endif
+
+template <class T> __device__ __forceinline__ T mjt_shfl_xor_any(T v, int off) {
+    if constexpr (sizeof(T) == 8) {
+        long long t;
+        __builtin_memcpy(&t, &v, 8);
+        t = __shfl_xor(t, off, 64);
+        __builtin_memcpy(&v, &t, 8);
+        return v;
+    } else {
+        int t = 0;
+        __builtin_memcpy(&t, &v, sizeof(T));
+        t = __shfl_xor(t, off, 64);
+        __builtin_memcpy(&v, &t, sizeof(T));
+        return v;
+    }
+}
+
+__device__ __forceinline__ index_t mjt_kept_offset(const Params& p, index_t o) {
+    index_t off = 0;
+#pragma unroll
+    for (int k = NK - 1; k >= 0; k--) {
+        index_t shape = (index_t)p.a[8 + 0 * 5 + k];
+        index_t q = (k == 0) ? 0 : MJT_DIVQ(o, k, 2);
+        index_t c = (k == 0) ? o : o - q * shape;
+        off += c * (index_t)p.a[8 + 1 * 5 + k];
+        o = q;
+    }
+    return off;
+}
+
+// offset of reduced coordinate `r` counted over the first `nd` reduced axes
+template <int ND> __device__ __forceinline__ index_t mjt_red_offset(const Params& p, index_t r) {
+    index_t off = 0;
+#pragma unroll
+    for (int k = ND - 1; k >= 0; k--) {
+        index_t shape = (index_t)p.a[8 + 3 * 5 + k];
+        index_t q = (k == 0) ? 0 : MJT_DIVQ(r, k, 5);
+        index_t c = (k == 0) ? r : r - q * shape;
+        off += c * (index_t)p.a[8 + 4 * 5 + k];
+        r = q;
+    }
+    return off;
+}
+
+#if ROW
+extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
+    const TX* __restrict__ xp = (const TX*)p.a[0];
+    TY* __restrict__ yp = (TY*)p.a[1];
+    const index_t O = (index_t)p.a[2];
+    const index_t S = (index_t)p.a[3];
+    const TY rcount = (TY)__longlong_as_double((long long)p.a[4]);
+    (void)rcount;
+    const unsigned lane = threadIdx.x % G;
+    const index_t o = (index_t)blockIdx.x * (256 / G) + threadIdx.x / G;
+    const index_t s = blockIdx.y;
+    TY acc[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++) acc[k] = INIT;
+    if (o < O) {
+        const index_t kbase = mjt_kept_offset(p, o);
+        const index_t L = (index_t)p.a[8 + 3 * 5 + (NR - 1)];
+        const index_t nL = (L + (G * VEC) - 1) / (G * VEC);
+        const index_t per = (index_t)p.a[5];
+        const index_t total = (index_t)p.a[6];
+        index_t it = s * per;
+        index_t it_end = it + per < total ? it + per : total;
+        index_t ro = (NR == 1) ? 0 : it / nL;
+        index_t lc = (NR == 1) ? it : it - ro * nL;
+        while (it < it_end) {
+            const TX* __restrict__ row = xp + kbase + ((NR == 1) ? 0 : mjt_red_offset<(NR > 1 ? NR - 1 : 1)>(p, ro));
+            index_t lc_end = nL - lc < it_end - it ? nL : lc + (it_end - it);
+            it += lc_end - lc;
+#pragma unroll 4
+            for (; lc < lc_end; lc++) {
+                index_t l = (lc * G + lane) * VEC;
+                if (l < L) {
+                    mjt_pack<TX, VEC> v;
+                    mjt_load(v, row + l);
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v.v[k]));
+                }
+            }
+            lc = 0;
+            ro++;
+        }
+    }
+    TY r = acc[0];
+#pragma unroll
+    for (int k = 1; k < VEC; k++) r = (TY)(MERGE(r, acc[k]));
+#pragma unroll
+    for (int off = G / 2; off > 0; off >>= 1) {
+        TY other = mjt_shfl_xor_any(r, off);
+        r = (TY)(MERGE(r, other));
+    }
+    if (lane == 0 && o < O) yp[SPLIT ? o * S + s : o] = r;
+}
+#else
+extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
+    const TX* __restrict__ xp = (const TX*)p.a[0];
+    TY* __restrict__ yp = (TY*)p.a[1];
+    const index_t O = (index_t)p.a[2];
+    const TY rcount = (TY)__longlong_as_double((long long)p.a[4]);
+    (void)rcount;
+    const index_t o = ((index_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    const index_t s = blockIdx.y;
+    if (o >= O) return;
+    const index_t kbase = mjt_kept_offset(p, o);
+    const index_t per = (index_t)p.a[5];
+    const index_t total = (index_t)p.a[6];
+    index_t r = s * per;
+    const index_t r_end = r + per < total ? r + per : total;
+    TY acc[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++) acc[k] = INIT;
+    const TX* __restrict__ col = xp + kbase;
+#pragma unroll 4
+    for (; r < r_end; r++) {
+        index_t roff = (NR == 1) ? r * (index_t)p.a[8 + 4 * 5] : mjt_red_offset<NR>(p, r);
+        mjt_pack<TX, VEC> v;
+        mjt_load(v, col + roff);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v.v[k]));
+    }
+    mjt_pack<TY, VEC> out;
+#pragma unroll
+    for (int k = 0; k < VEC; k++) out.v[k] = acc[k];
+    mjt_store(yp + (SPLIT ? s * O : 0) + o, out);
+}
+#endif

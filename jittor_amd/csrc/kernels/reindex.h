@@ -1,0 +1,54 @@
+// Generic gather / scatter kernels for arbitrary index expressions
+// (reference: python/jittor/src/ops/reindex_op.cc:111-139 and
+// python/jittor/src/ops/reindex_reduce_op.cc:93-131).
+//
+// Constants and fragments supplied by the host:
+//   TX, index_t, VEC, NPARAM, SCATTER (0 gather, 1 scatter), LDIM
+//   MJT_RX_SETUP    shapes, strides and extras pointers under the names the
+//                   index language uses (xshapeK, yshapeK, xstrideK, ystrideK,
+//                   XDIM, YDIM, eKp, eKstrideJ)
+//   MJT_RX_DECODE   loop coordinates i0..i{LDIM-1} of flat element e; the
+//                   innermost one is named ilast_ (the lane's first element)
+//   MJT_RX_LASTVAR  name of the innermost coordinate (iN)
+//   MJT_RX_INDEX    per element: xid0.., flat xid, bool ov_
+//   ATOMIC_UPDATE(addr, v)   scatter only
+//
+// The loop runs over y: the output of a gather, the input of a scatter.  Each
+// lane owns VEC adjacent elements of y's innermost axis so that y moves as
+// one vector per lane; the x side is accessed element by element.
+
+struct Params { unsigned long long a[NPARAM]; };
+
+extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
+#if SCATTER
+    TX* __restrict__ xp = (TX*)p.a[0];
+    const TX* __restrict__ yp = (const TX*)p.a[1];
+#else
+    const TX* __restrict__ xp = (const TX*)p.a[0];
+    TX* __restrict__ yp = (TX*)p.a[1];
+    const TX ovalue_ = (TX)__longlong_as_double((long long)p.a[3]);
+#endif
+    const index_t nvec = (index_t)p.a[2];
+    MJT_RX_SETUP
+    const index_t j = (index_t)blockIdx.x * 256 + threadIdx.x;
+    if (j >= nvec) return;
+    const index_t e = j * VEC;
+    MJT_RX_DECODE
+    mjt_pack<TX, VEC> yv;
+#if SCATTER
+    mjt_load(yv, yp + e);
+#endif
+#pragma unroll
+    for (int k = 0; k < VEC; k++) {
+        const index_t MJT_RX_LASTVAR = ilast_ + k;
+        MJT_RX_INDEX
+#if SCATTER
+        if (!ov_) { ATOMIC_UPDATE(xp + xid, yv.v[k]); }
+#else
+        if (ov_) yv.v[k] = ovalue_; else yv.v[k] = xp[xid];
+#endif
+    }
+#if !SCATTER
+    mjt_store(yp + e, yv);
+#endif
+}

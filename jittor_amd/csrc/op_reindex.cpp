@@ -1,0 +1,316 @@
+// mjt_reindex / mjt_reindex_reduce: host side of the gather and scatter ops
+// (reference: python/jittor/src/ops/reindex_op.cc:82-139,
+// python/jittor/src/ops/reindex_reduce_op.cc:65-131).
+//
+// Index strings are parsed once per distinct op description (the role of the
+// reference's jit key, ops/reindex_op.cc:93-108) and kept in a plan: the
+// parsed expressions, their affine form when they have one, and the kernel
+// that was specialised for them.  A plan first tries the hand-written fast
+// kernels (sliding-window gather, one-axis scatter with LDS-privatised bins)
+// and otherwise uses the generic kernel with the expressions pasted in.
+#include "common.h"
+#include "expr.h"
+#include <mutex>
+#include <unordered_map>
+
+namespace mjt {
+
+// fast paths, aot_kernels.hip
+bool try_window_gather(const mjt_tensor* x, const mjt_tensor* y, const std::vector<Affine>& aff, double overflow_value);
+bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_tensor* index);
+void launch_fill_pattern(void* dst, uint64_t pattern, int elem_size, size_t n);
+
+namespace {
+
+struct Plan {
+    std::vector<std::unique_ptr<Expr>> idx, ofc;
+    bool all_affine = false;      // every index is affine and there are no overflow conditions / extras
+    bool plain_e0 = false;        // scatter: indexes == ["@e0(i0)"] style one-axis lookup of a 1-d extra
+    std::unordered_map<std::string, JitKernel*> kernels;   // by (vec, use64)
+};
+
+std::mutex g_mu;
+std::unordered_map<std::string, std::unique_ptr<Plan>> g_plans;
+
+std::string plan_key(bool scatter, int op, const mjt_tensor* x, const mjt_tensor* y, int n_idx, const char* const* idx,
+                     int n_ofc, const char* const* ofc, int n_ex, const mjt_tensor* ex) {
+    std::string k;
+    k.reserve(256);
+    k += scatter ? "S" : "G";
+    k += std::to_string(op) + "|" + std::to_string(x->dtype) + "|" + std::to_string(x->ndim) + "|" + std::to_string(y->ndim);
+    for (int i = 0; i < n_idx; i++) {
+        k += "\x1f";
+        k += idx[i];
+    }
+    k += "\x1e";
+    for (int i = 0; i < n_ofc; i++) {
+        k += "\x1f";
+        k += ofc[i];
+    }
+    k += "\x1e";
+    for (int i = 0; i < n_ex; i++) k += std::to_string(ex[i].dtype) + ":" + std::to_string(ex[i].ndim) + ",";
+    return k;
+}
+
+Plan* get_plan(const std::string& key, const mjt_tensor* x, const mjt_tensor* y, int loop_rank, int n_idx,
+               const char* const* idx, int n_ofc, const char* const* ofc, int n_ex, const mjt_tensor* ex) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_plans.find(key);
+    if (it != g_plans.end()) return it->second.get();
+    auto plan = std::make_unique<Plan>();
+    ExprEnv env;
+    env.n_loop = loop_rank;
+    env.xdim = x->ndim;
+    env.ydim = y->ndim;
+    for (int i = 0; i < n_ex; i++) env.extra_rank.push_back(ex[i].ndim);
+    bool pure = n_ofc == 0;
+    for (int i = 0; i < n_idx; i++) {
+        MJT_CHECK(idx[i], "null index expression");
+        plan->idx.push_back(parse_expr(idx[i]));
+        validate_expr(*plan->idx.back(), env);
+        pure = pure && is_pure(*plan->idx.back());
+    }
+    for (int i = 0; i < n_ofc; i++) {
+        MJT_CHECK(ofc[i], "null overflow condition");
+        plan->ofc.push_back(parse_expr(ofc[i]));
+        validate_expr(*plan->ofc.back(), env);
+    }
+    plan->all_affine = pure;
+    if (n_idx == 1 && n_ofc == 0 && n_ex >= 1 && ex[0].ndim == 1 && loop_rank == 1) {
+        const Expr& e = *plan->idx[0];
+        plan->plain_e0 = e.kind == Expr::EXTRA && e.extra == 0 && e.kids.size() == 1 && e.kids[0]->kind == Expr::VAR &&
+                         e.kids[0]->text == "i0";
+    }
+    Plan* raw = plan.get();
+    g_plans.emplace(key, std::move(plan));
+    return raw;
+}
+
+int pick_vec(int elem_size, int64_t last, const void* p) {
+    int vec = std::min(8, 16 / elem_size);
+    while (vec > 1 && (last % vec != 0 || ((uintptr_t)p % (size_t)(vec * elem_size)) != 0)) vec /= 2;
+    return vec;
+}
+
+// Specialises (once per plan and variant) and launches the generic kernel.
+void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mjt_tensor* y, double overflow_value,
+                 int n_ex, const mjt_tensor* ex) {
+    // the loop runs over y (gather output / scatter input)
+    const int LD = y->ndim, XD = x->ndim;
+    int64_t yn = numel(y), xn = numel(x);
+    if (yn == 0) return;
+    int64_t biggest = std::max(xn, yn);
+    for (int i = 0; i < n_ex; i++) biggest = std::max(biggest, numel(&ex[i]));
+    bool use64 = biggest >= (int64_t(1) << 31);   // index_t rule of op.cc:158-192
+    int vec = pick_vec(dtype_size(x->dtype), y->shape[LD - 1], y->ptr);
+
+    // parameter block: a[0] x, a[1] y, a[2] nvec, a[3] overflow value,
+    // then yshape[LD], ydiv[LD], xshape[XD], per extra: pointer, shape[rank]
+    std::vector<uint64_t> args{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), (uint64_t)(yn / vec), bits_of(overflow_value)};
+    int p_ys = (int)args.size();
+    for (int i = 0; i < LD; i++) args.push_back((uint64_t)y->shape[i]);
+    int p_yd = (int)args.size();
+    for (int i = 0; i < LD; i++) args.push_back(pack_divmod((uint64_t)y->shape[i]));
+    int p_xs = (int)args.size();
+    for (int i = 0; i < XD; i++) args.push_back((uint64_t)x->shape[i]);
+    std::vector<int> p_ex(n_ex);
+    for (int k = 0; k < n_ex; k++) {
+        p_ex[k] = (int)args.size();
+        args.push_back(bits_of_ptr(ex[k].ptr));
+        for (int i = 0; i < ex[k].ndim; i++) args.push_back((uint64_t)ex[k].shape[i]);
+    }
+
+    std::string vkey = std::to_string(vec) + (use64 ? "L" : "I");
+    JitKernel* kern = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        auto it = plan->kernels.find(vkey);
+        if (it != plan->kernels.end()) kern = it->second;
+    }
+    if (!kern) {
+        const char* IT = use64 ? "long long" : "int";
+        std::ostringstream setup, dec, index;
+        setup << "const index_t XDIM = " << XD << "; const index_t YDIM = " << LD << "; (void)XDIM; (void)YDIM; ";
+        auto shapes = [&](const char* n, int rank, int base) {
+            for (int i = 0; i < rank; i++)
+                setup << "const index_t " << n << "shape" << i << " = (index_t)p.a[" << base + i << "]; (void)" << n
+                      << "shape" << i << "; ";
+            setup << "const index_t " << n << "stride" << rank - 1 << " = 1; (void)" << n << "stride" << rank - 1 << "; ";
+            for (int i = rank - 2; i >= 0; i--)
+                setup << "const index_t " << n << "stride" << i << " = " << n << "stride" << i + 1 << " * " << n << "shape"
+                      << i + 1 << "; (void)" << n << "stride" << i << "; ";
+        };
+        shapes("y", LD, p_ys);
+        shapes("x", XD, p_xs);
+        for (int k = 0; k < n_ex; k++) {
+            std::string n = "e" + std::to_string(k);
+            setup << "const " << dtype_cname(ex[k].dtype) << "* __restrict__ " << n << "p = (const "
+                  << dtype_cname(ex[k].dtype) << "*)p.a[" << p_ex[k] << "]; (void)" << n << "p; ";
+            shapes(n.c_str(), ex[k].ndim, p_ex[k] + 1);
+        }
+        dec << IT << " rem_ = e; ";
+        for (int a = LD - 1; a >= 0; a--) {
+            std::string cname = a == LD - 1 ? std::string("ilast_") : "i" + std::to_string(a);
+            if (a == 0) {
+                dec << "const " << IT << " " << cname << " = rem_; ";
+            } else if (use64) {
+                dec << "const " << IT << " q" << a << "_ = rem_ / yshape" << a << "; const " << IT << " " << cname
+                    << " = rem_ - q" << a << "_ * yshape" << a << "; rem_ = q" << a << "_; ";
+            } else {
+                dec << "const int q" << a << "_ = (int)mjt_div((unsigned)rem_, mjt_unpack_divmod(p.a[" << p_yd + a
+                    << "], 0)); const int " << cname << " = rem_ - q" << a << "_ * yshape" << a << "; rem_ = q" << a
+                    << "_; ";
+            }
+            if (a != LD - 1) dec << "(void)" << cname << "; ";
+        }
+        for (int dd = 0; dd < XD; dd++)
+            index << "const index_t xid" << dd << " = (index_t)(" << emit_c(*plan->idx[dd]) << "); ";
+        index << "const index_t xid = 0";
+        for (int dd = 0; dd < XD; dd++) index << " + xid" << dd << " * xstride" << dd;
+        index << "; bool ov_ = false";
+        for (int dd = 0; dd < XD; dd++) index << " || xid" << dd << " < 0 || xid" << dd << " >= xshape" << dd;
+        for (auto& c : plan->ofc) index << " || (" << emit_c(*c) << ")";
+        index << "; ";
+
+        std::ostringstream frag;
+        frag << "#define TX " << dtype_cname(x->dtype) << "\n#define index_t " << IT << "\n#define VEC " << vec
+             << "\n#define NPARAM " << args.size() << "\n#define SCATTER " << (scatter ? 1 : 0) << "\n";
+        frag << "#define MJT_RX_LASTVAR i" << LD - 1 << "\n";
+        frag << "#define MJT_RX_SETUP " << setup.str() << "\n";
+        frag << "#define MJT_RX_DECODE " << dec.str() << "\n";
+        frag << "#define MJT_RX_INDEX " << index.str() << "\n";
+        if (scatter) frag << "#define ATOMIC_UPDATE(addr, v) mjt_atomic_" << mjt_op_name(op) << "<TX>((addr), (v))\n";
+        uint64_t h = 1469598103934665603ull;
+        for (unsigned char ch : frag.str()) {
+            h ^= ch;
+            h *= 1099511628211ull;
+        }
+        char name[96];
+        snprintf(name, sizeof(name), "mjt_%s_%016llx", scatter ? (std::string("reindex_reduce_") + mjt_op_name(op)).c_str() : "reindex",
+                 (unsigned long long)h);
+        std::string src = std::string("#define ENTRY ") + name + "\n" + frag.str() + embedded_source("prelude.h") + "\n" +
+                          (scatter ? std::string(embedded_source("atomics.h")) + "\n" : std::string()) +
+                          embedded_source("reindex.h") + "\n";
+        kern = jit_get(src, name);
+        std::lock_guard<std::mutex> lock(g_mu);
+        plan->kernels.emplace(vkey, kern);
+    }
+    int64_t nvec = yn / vec;
+    int64_t blocks = (nvec + 255) / 256;
+    MJT_CHECK(blocks < (int64_t(1) << 31), "reindex: launch too large");
+    jit_launch(kern, (unsigned)blocks, 1, 256, 0, args);
+}
+
+void check_extras(int n_ex, const mjt_tensor* ex) {
+    MJT_CHECK(n_ex >= 0 && n_ex <= 16, "too many extras");
+    MJT_CHECK(n_ex == 0 || ex, "null extras");
+    for (int i = 0; i < n_ex; i++) check_tensor(&ex[i], "extras");
+}
+
+// bit pattern of init_OP for dtype (type/common_op_type.cc:116-117,142-151;
+// 16-bit floats: type/fp16_op_type.cc:111-112)
+uint64_t identity_bits(int op, int dtype) {
+    auto fbits = [&](double v) -> uint64_t {
+        if (dtype == MJT_FLOAT64) return bits_of(v);
+        float f = (float)v;
+        uint32_t u;
+        memcpy(&u, &f, 4);
+        if (dtype == MJT_FLOAT32) return u;
+        if (dtype == MJT_BFLOAT16) return u >> 16;
+        // float16: only 0, 1 and +-32768 are needed
+        if (v == 0) return 0;
+        if (v == 1) return 0x3c00;
+        return v > 0 ? 0x7800 : 0xf800;
+    };
+    bool fl = dtype_is_float(dtype);
+    int sz = dtype_size(dtype);
+    uint64_t ones = sz == 8 ? ~0ull : ((1ull << (8 * sz)) - 1);
+    switch (op) {
+        case MJT_OP_MULTIPLY: return fl ? fbits(1.0) : 1;
+        case MJT_OP_MAXIMUM:
+            if (dtype == MJT_FLOAT32) return fbits(-3.402823466e+38);
+            if (dtype == MJT_FLOAT64) return fbits(-1.7976931348623157e+308);
+            if (fl) return fbits(-32768.0);
+            if (dtype == MJT_BOOL || dtype_is_unsigned(dtype)) return 0;
+            return 1ull << (8 * sz - 1);
+        case MJT_OP_MINIMUM:
+            if (dtype == MJT_FLOAT32) return fbits(3.402823466e+38);
+            if (dtype == MJT_FLOAT64) return fbits(1.7976931348623157e+308);
+            if (fl) return fbits(32768.0);
+            if (dtype == MJT_BOOL) return 1;
+            if (dtype_is_unsigned(dtype)) return ones;
+            return ones >> 1;
+        case MJT_OP_LOGICAL_AND: return fl ? fbits(1.0) : 1;
+        case MJT_OP_BITWISE_AND: return dtype == MJT_BOOL ? 1 : (fl ? fbits(-1.0) : ones);
+        default: return 0;   // add, subtract, void, logical_or/xor, bitwise_or/xor and the rest start from 0
+    }
+}
+
+}  // namespace
+
+void reindex_impl(const mjt_tensor* x, const mjt_tensor* y, int n_idx, const char* const* idx, double overflow_value,
+                  int n_ofc, const char* const* ofc, int n_ex, const mjt_tensor* ex) {
+    require_init();
+    check_tensor(x, "reindex x");
+    check_tensor(y, "reindex y");
+    check_extras(n_ex, ex);
+    MJT_CHECK(n_idx == x->ndim, "Number of x's shape and indexes should be the same. (x rank " << x->ndim << ", "
+                                                                                             << n_idx << " indexes)");
+    MJT_CHECK(n_idx == 0 || idx, "null indexes");
+    MJT_CHECK(n_ofc >= 0 && (n_ofc == 0 || ofc), "null overflow conditions");
+    MJT_CHECK(x->dtype == y->dtype, "reindex: y dtype must equal x dtype");
+    std::string key = plan_key(false, 0, x, y, n_idx, idx, n_ofc, ofc, n_ex, ex);
+    Plan* plan = get_plan(key, x, y, y->ndim, n_idx, idx, n_ofc, ofc, n_ex, ex);
+    if (numel(y) == 0) return;
+    if (plan->all_affine && numel(x) > 0) {
+        std::vector<int64_t> xs(x->shape, x->shape + x->ndim), ys(y->shape, y->shape + y->ndim);
+        std::vector<Affine> aff(n_idx);
+        bool ok = true;
+        for (int i = 0; i < n_idx && ok; i++) ok = affine_of(*plan->idx[i], xs, ys, &aff[i]);
+        if (ok && try_window_gather(x, y, aff, overflow_value)) return;
+    }
+    run_generic(plan, false, 0, x, y, overflow_value, n_ex, ex);
+}
+
+void reindex_reduce_impl(const mjt_tensor* y, const mjt_tensor* x, int op, int n_idx, const char* const* idx, int n_ofc,
+                         const char* const* ofc, int n_ex, const mjt_tensor* ex) {
+    require_init();
+    check_tensor(y, "reindex_reduce y");
+    check_tensor(x, "reindex_reduce x");
+    check_extras(n_ex, ex);
+    // ASSERT((ns.is_binary() && ns!=ns_mean) || ns == ns_void), ops/reindex_reduce_op.cc:34
+    MJT_CHECK((op >= MJT_OP_POW && op < MJT_OP_MEAN) || op == MJT_OP_VOID,
+              "reindex_reduce: op must be a binary op other than mean, or void");
+    MJT_CHECK(n_idx == x->ndim, "Number of shape and indexes should be the same. (shape rank " << x->ndim << ", " << n_idx
+                                                                                              << " indexes)");
+    MJT_CHECK(n_idx == 0 || idx, "null indexes");
+    MJT_CHECK(n_ofc >= 0 && (n_ofc == 0 || ofc), "null overflow conditions");
+    MJT_CHECK(x->dtype == y->dtype, "reindex_reduce: x dtype must equal y dtype");
+    std::string key = plan_key(true, op, x, y, n_idx, idx, n_ofc, ofc, n_ex, ex);
+    Plan* plan = get_plan(key, x, y, y->ndim, n_idx, idx, n_ofc, ofc, n_ex, ex);
+    int64_t xn = numel(x);
+    if (xn == 0) return;
+    if (plan->plain_e0 && numel(y) > 0 && numel(&ex[0]) == numel(y) && try_scatter_1d(y, x, op, &ex[0])) return;
+    if (op != MJT_OP_VOID) launch_fill_pattern(x->ptr, identity_bits(op, x->dtype), dtype_size(x->dtype), (size_t)xn);
+    run_generic(plan, true, op, x, y, 0.0, n_ex, ex);
+}
+
+}  // namespace mjt
+
+extern "C" int mjt_reindex(const mjt_tensor* x, const mjt_tensor* y, int n_indexes, const char* const* indexes,
+                           double overflow_value, int n_overflow_conditions, const char* const* overflow_conditions,
+                           int n_extras, const mjt_tensor* extras) {
+    return mjt::guarded([&] {
+        mjt::reindex_impl(x, y, n_indexes, indexes, overflow_value, n_overflow_conditions, overflow_conditions, n_extras,
+                          extras);
+    });
+}
+
+extern "C" int mjt_reindex_reduce(const mjt_tensor* y, const mjt_tensor* x, int op, int n_indexes,
+                                  const char* const* indexes, int n_overflow_conditions,
+                                  const char* const* overflow_conditions, int n_extras, const mjt_tensor* extras) {
+    return mjt::guarded([&] {
+        mjt::reindex_reduce_impl(y, x, op, n_indexes, indexes, n_overflow_conditions, overflow_conditions, n_extras,
+                                 extras);
+    });
+}
