@@ -1,0 +1,171 @@
+"""jittor_amd: the meta-operator execution path of Jittor on MI355X (gfx950).
+
+Keeps Jittor's Python signatures for this path -- jt.array, jt.reindex,
+jt.reindex_reduce, Var.sum / max / min, jt.broadcast, unary / binary / ternary
+ops -- on a small lazy Var graph that executes through libmjt.so
+(include/mjt.h) into hand-written HIP kernels.  Signatures follow
+python/jittor/__init__.pyi:203-206,280-285,368,823-891,1201-1263,2168,
+4122-4190,4258 of the reference.
+"""
+import numbers as _numbers
+
+import numpy as np
+
+from . import _lib
+from ._lib import MjtError, init, shutdown, sync as _device_sync, device_info
+from .core import (Var, array, unary, binary, ternary, broadcast, broadcast_var,
+                   reduce, reindex, reindex_var, reindex_reduce, make_number)
+from .executor import run_sync, stats as executor_stats, flags
+from . import dtypes
+from . import nn
+
+__all__ = ["Var", "array", "unary", "binary", "ternary", "broadcast", "broadcast_var",
+           "reduce", "reindex", "reindex_var", "reindex_reduce", "nn", "sync", "sync_all",
+           "fetch_sync", "MjtError"]
+
+
+def sync(vars, device_sync=False):
+    """jt.sync(vars): computes the given Vars (var_holder.cc:269-274)."""
+    run_sync(list(vars), device_sync)
+
+
+def sync_all(device_sync=True):
+    if device_sync and _lib.device() is not None:
+        _device_sync()
+
+
+def fetch_sync(vars):
+    vars = list(vars)
+    run_sync(vars)
+    return [v.numpy() for v in vars]
+
+
+def clean():
+    core.pool.release_all()
+
+
+# ---- creation helpers --------------------------------------------------------
+def zeros(shape, dtype="float32"):
+    if isinstance(shape, _numbers.Integral):
+        shape = [shape]
+    return array(np.zeros(shape, dtype=np.float32), dtypes.normalize_dtype(dtype))
+
+
+def ones(shape, dtype="float32"):
+    if isinstance(shape, _numbers.Integral):
+        shape = [shape]
+    return array(np.ones(shape, dtype=np.float32), dtypes.normalize_dtype(dtype))
+
+
+_rng = [np.random.default_rng(0)]
+
+
+def set_seed(seed):
+    _rng[0] = np.random.default_rng(seed)
+
+
+def random(shape, dtype="float32", type="uniform"):
+    """Host-generated random Var (the reference's generator,
+    python/jittor/src/init.cc:78-84, is not reproduced: tests seed numpy)."""
+    if isinstance(shape, _numbers.Integral):
+        shape = [shape]
+    if type == "normal":
+        a = _rng[0].standard_normal(shape)
+    else:
+        a = _rng[0].random(shape)
+    return array(a.astype(np.float32), dtypes.normalize_dtype(dtype))
+
+
+def randn(*shape):
+    if len(shape) == 1 and isinstance(shape[0], (list, tuple)):
+        shape = shape[0]
+    return random(list(shape), "float32", "normal")
+
+
+def index(shape, dim, dtype="int32"):
+    """jt.index(shape, dim): Var of `shape` holding the coordinate along `dim`."""
+    shape = list(shape)
+    a = array(np.arange(shape[dim]), dtype)
+    return broadcast(a, shape, [d for d in range(len(shape)) if d != dim])
+
+
+# ---- named ops ----------------------------------------------------------------
+def _make_binary(name):
+    def f(x, y):
+        return binary(x, y, name)
+    f.__name__ = name
+    return f
+
+
+def _make_unary(name):
+    def f(x):
+        return unary(x, name)
+    f.__name__ = name
+    return f
+
+
+def _make_reduce(name):
+    def f(x, dims=(), keepdims=False, dim=None):
+        return reduce(x, name, dims if dim is None else dim, keepdims)
+    f.__name__ = "reduce_" + name
+    return f
+
+
+for _n in _lib.BINARY_OPS:
+    if _n != "mean":
+        globals()[_n] = _make_binary(_n)
+for _n in _lib.UNARY_OPS:
+    if _n != "cast":
+        globals()[_n] = _make_unary(_n)
+for _n in _lib.DTYPES[1:]:
+    globals()[_n] = (lambda n: lambda x: array(x, n) if not isinstance(x, Var) else unary(x, n))(_n)
+for _n in dtypes.REDUCE_OPS:
+    globals()["reduce_" + _n] = _make_reduce(_n)
+float = float32  # noqa: F821
+int = int32  # noqa: F821
+
+
+def cast(x, dtype):
+    return unary(x, dtypes.normalize_dtype(dtype))
+
+
+def sum(x, dims=(), keepdims=False, dim=None):
+    return reduce(x, "add", dims if dim is None else dim, keepdims)
+
+
+def max(x, dims=(), keepdims=False, dim=None):
+    return reduce(x, "maximum", dims if dim is None else dim, keepdims)
+
+
+def min(x, dims=(), keepdims=False, dim=None):
+    return reduce(x, "minimum", dims if dim is None else dim, keepdims)
+
+
+def mean(x, dims=(), keepdims=False, dim=None):
+    return reduce(x, "mean", dims if dim is None else dim, keepdims)
+
+
+def prod(x, dims=(), keepdims=False, dim=None):
+    return reduce(x, "multiply", dims if dim is None else dim, keepdims)
+
+
+def ternary_out_hint(cond, x, y):
+    return ternary(cond, x, y)
+
+
+def histc(input, bins, min=0.0, max=0.0):
+    """python/jittor/misc.py:2212-2235: scatter-add of ones by bin index.
+    `input` is a 1-d Var."""
+    if input.ndim != 1:
+        raise ValueError("histc expects a 1-d Var")
+    if min == 0 and max == 0:
+        lo, hi = input.min().item(), input.max().item()
+    else:
+        lo, hi = min, max
+    assert lo <= hi
+    if hi - lo < 1e-5:
+        hi, lo = hi + 1e-5, lo - 1e-5
+    pos = (input - lo) * (bins / (hi - lo))
+    idx = unary(pos, "floor_int").minimum(bins - 1)
+    one = ones(input.shape, "float32")
+    return reindex_reduce(one, "add", [bins], ["@e0(i0)"], extras=[idx])

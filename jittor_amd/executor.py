@@ -1,0 +1,351 @@
+"""Executes pending Var graphs through libmjt.so.
+
+Mirror of the part of Executor::run_sync that matters for this path
+(python/jittor/src/executor.cc:200-716): collect the pending ops behind the
+requested Vars, partition them into fused groups (element / broadcast ops
+share a kernel, executor.cc:555; reduce, reindex and reindex_reduce start a
+new one), recognise the convolution pattern the way ConvTuner does
+(opt/tuner/conv_tuner.cc:218-411), allocate outputs and launch each group
+once.  Everything runs on the device; there is no host path.
+"""
+import ctypes
+
+from . import _lib
+from . import core
+from .core import (Var, Buffer, UnaryOp, BinaryOp, TernaryOp, BroadcastOp,
+                   ReduceOp, ReindexOp, ReindexReduceOp)
+from ._lib import MjtError
+
+stats = {"launches": 0, "fused_groups": 0, "conv_matches": 0, "syncs": 0}
+flags = {"enable_conv_match": True}
+
+
+class ConvUnit:
+    """reindex + broadcast + multiply + reduce.add matched as one convolution."""
+    kind = "conv"
+    fusable = False
+
+    def __init__(self, reduce_op, x, w, params, absorbed):
+        self.out = reduce_op.out
+        self.inputs = [x, w]
+        self.params = params
+        self.absorbed = absorbed
+        self.id = reduce_op.id
+
+
+def _pending_ops(targets):
+    """Pending producers behind `targets`, in topological order."""
+    order, seen = [], set()
+    stack = [(v, False) for v in targets]
+    while stack:
+        v, done = stack.pop()
+        if v.materialised:
+            continue
+        op = v._op
+        if done:
+            if op.id not in seen:
+                seen.add(op.id)
+                order.append(op)
+            continue
+        if op.id in seen:
+            continue
+        stack.append((v, True))
+        for u in op.inputs:
+            if not u.materialised and u._op.id not in seen:
+                stack.append((u, False))
+    return order
+
+
+def _affine(expr, xshape, yshape):
+    return _lib.expr_affine(expr, xshape, yshape)
+
+
+def _match_conv(red, consumers, targets):
+    """reduce.add <- multiply <- {reindex(x), broadcast(w)} with
+    xx = x.reindex([N,K,C,OH,OW,R,S], ['i0','i2','i3*s-p+i5*d','i4*s-p+i6*d']),
+    ww = w.broadcast(xx.shape, [0,3,4]), sum over [2,5,6]
+    (python/jittor/nn.py:1251-1262; matcher conv_tuner.cc:312-356)."""
+    if red.op != "add" or red.reduce_mask != 0b1100100:
+        return None
+    yy = red.inputs[0]
+    if yy.materialised or yy.ndim != 7 or not isinstance(yy._op, BinaryOp) or yy._op.op != "multiply":
+        return None
+    if yy.id in targets or len(consumers.get(yy.id, ())) != 1:
+        return None
+    a, b = yy._op.inputs
+    for xx, ww in ((a, b), (b, a)):
+        if xx.materialised or ww.materialised:
+            continue
+        ro, bo = xx._op, ww._op
+        if not isinstance(ro, ReindexOp) or not isinstance(bo, BroadcastOp):
+            continue
+        if xx.id in targets or ww.id in targets:
+            continue
+        if len(consumers.get(xx.id, ())) != 1 or len(consumers.get(ww.id, ())) != 1:
+            continue
+        if len(ro.inputs) != 1 or ro.overflow_conditions or ro.overflow_value != 0.0:
+            continue
+        x, w = ro.inputs[0], bo.inputs[0]
+        if x.ndim != 4 or w.ndim != 4 or bo.bcast_mask != 0b0011001:
+            continue
+        if x.dtype != w.dtype or x.dtype not in ("float32", "bfloat16"):
+            continue
+        N, K, C, OH, OW, R, S = xx.shape
+        if list(w.shape) != [K, C, R, S] or x.shape[0] != N or x.shape[1] != C:
+            continue
+        aff = [_affine(s, x.shape, xx.shape) for s in ro.indexes]
+        if any(a_ is None for a_ in aff):
+            continue
+        def only(co, allowed):
+            return all(co[k] == 0 for k in range(10) if k not in allowed)
+        (c0n, con), (c0c, coc), (c0h, coh), (c0w, cow) = aff
+        if c0n or c0c or con[0] != 1 or coc[2] != 1 or not only(con, (0,)) or not only(coc, (2,)):
+            continue
+        if not only(coh, (3, 5)) or not only(cow, (4, 6)):
+            continue
+        sh, dh, sw, dw = coh[3], coh[5], cow[4], cow[6]
+        ph, pw = -c0h, -c0w
+        if min(sh, dh, sw, dw) < 1 or ph < 0 or pw < 0:
+            continue
+        H, W = x.shape[2], x.shape[3]
+        # the matcher checks oh / ow against the solved parameters (conv_tuner.cc:349-355)
+        if OH != (H + 2 * ph - dh * (R - 1) - 1) // sh + 1 or OW != (W + 2 * pw - dw * (S - 1) - 1) // sw + 1:
+            continue
+        if red.out.dtype != "float32" and red.out.dtype != x.dtype:
+            continue
+        return ConvUnit(red, x, w, (sh, sw, ph, pw, dh, dw), {red.id, yy._op.id, ro.id, bo.id})
+    return None
+
+
+def run_sync(targets, device_sync=False):
+    targets = [t for t in targets if isinstance(t, Var)]
+    stats["syncs"] += 1
+    _lib.ensure_init()
+    ops = _pending_ops(targets)
+    if ops:
+        _execute(ops, {t.id for t in targets})
+    for t in targets:
+        t._device_ptr()
+    if device_sync:
+        _lib.sync()
+
+
+def _execute(ops, target_ids):
+    consumers = {}
+    for op in ops:
+        for u in op.inputs:
+            consumers.setdefault(u.id, []).append(op)
+
+    # ---- convolution pattern -------------------------------------------------
+    units = []
+    absorbed = set()
+    if flags["enable_conv_match"]:
+        for op in ops:
+            if isinstance(op, ReduceOp):
+                cu = _match_conv(op, consumers, target_ids)
+                if cu is not None:
+                    absorbed |= cu.absorbed
+                    units.append(cu)
+                    stats["conv_matches"] += 1
+    conv_by_id = {u.id: u for u in units}
+    sched = []
+    for op in ops:
+        if op.id in conv_by_id:
+            sched.append(conv_by_id[op.id])
+        elif op.id not in absorbed:
+            sched.append(op)
+
+    # ---- stages: an op can share a kernel with its producer only inside a stage ---------
+    producer = {}
+    for op in sched:
+        producer[op.out.id] = op
+    stage = {}
+    for op in sched:
+        s = 0
+        for u in op.inputs:
+            p = producer.get(u.id)
+            if p is None:
+                continue
+            step = 0
+            if not p.fusable or not op.fusable:
+                step = 1 if not p.fusable else 0
+            if isinstance(op, BroadcastOp) or (op.fusable and p.fusable and p.out.shape != op.out.shape):
+                step = 1
+            if getattr(u, "_stop_fuse", False):
+                step = 1
+            s = max(s, stage[p.id] + step)
+        stage[op.id] = s
+
+    # ---- union element ops into groups ---------------------------------------------
+    parent = {}
+
+    def find(a):
+        while parent[a] != a:
+            parent[a] = parent[parent[a]]
+            a = parent[a]
+        return a
+
+    for op in sched:
+        parent[op.id] = op.id
+    for op in sched:
+        if not op.fusable:
+            continue
+        for u in op.inputs:
+            p = producer.get(u.id)
+            if p is not None and p.fusable and stage[p.id] == stage[op.id] and p.out.shape == op.out.shape \
+                    and not isinstance(op, BroadcastOp) and not getattr(u, "_stop_fuse", False):
+                parent[find(op.id)] = find(p.id)
+    groups = {}
+    for op in sched:
+        if op.fusable:
+            groups.setdefault(find(op.id), []).append(op)
+
+    # ---- run stage by stage: element groups first, then the other ops ---------------------
+    nstage = max(stage.values()) + 1 if stage else 0
+    by_stage_groups = [[] for _ in range(nstage)]
+    by_stage_other = [[] for _ in range(nstage)]
+    for root, members in groups.items():
+        by_stage_groups[stage[members[0].id]].append(members)
+    for op in sched:
+        if not op.fusable:
+            by_stage_other[stage[op.id]].append(op)
+    for s in range(nstage):
+        for members in by_stage_groups[s]:
+            _run_group(members, consumers, target_ids)
+        for op in by_stage_other[s]:
+            _run_single(op)
+    # materialised vars become leaves: the graph behind them can be dropped
+    for op in sched:
+        if op.out._buf is not None:
+            op.out._op = None
+            op.inputs = []
+
+
+def _alloc_out(v):
+    if v._buf is None:
+        v._buf = Buffer(max(v.nbytes, 1))
+    return v._buf.ptr
+
+
+def _tensor_of(v):
+    return _lib.tensor(v._device_ptr(), v.dtype, v.shape)
+
+
+def _run_single(op):
+    lib = _lib.ensure_init()
+    out = op.out
+    stats["launches"] += 1
+    if isinstance(op, ReduceOp):
+        x = op.inputs[0]
+        tx = _tensor_of(x)
+        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        _lib.check(lib.mjt_reduce(ctypes.byref(tx), ctypes.byref(ty), _lib.OP_CODE[op.op], op.reduce_mask))
+    elif isinstance(op, ReindexOp):
+        x, extras = op.inputs[0], op.inputs[1:]
+        tx = _tensor_of(x)
+        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        ex = (_lib.Tensor * max(1, len(extras)))(*[_tensor_of(e) for e in extras])
+        _lib.check(lib.mjt_reindex(ctypes.byref(tx), ctypes.byref(ty), len(op.indexes), _lib.c_strings(op.indexes),
+                                   op.overflow_value, len(op.overflow_conditions),
+                                   _lib.c_strings(op.overflow_conditions), len(extras), ex))
+    elif isinstance(op, ReindexReduceOp):
+        y, extras = op.inputs[0], op.inputs[1:]
+        ty = _tensor_of(y)
+        tx = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        ex = (_lib.Tensor * max(1, len(extras)))(*[_tensor_of(e) for e in extras])
+        _lib.check(lib.mjt_reindex_reduce(ctypes.byref(ty), ctypes.byref(tx), _lib.OP_CODE[op.op], len(op.indexes),
+                                          _lib.c_strings(op.indexes), len(op.overflow_conditions),
+                                          _lib.c_strings(op.overflow_conditions), len(extras), ex))
+    elif isinstance(op, ConvUnit):
+        x, w = op.inputs
+        tx, tw = _tensor_of(x), _tensor_of(w)
+        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        p = _lib.ConvParams(*op.params)
+        _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
+    else:
+        raise MjtError(-2, "no kernel for op %r" % (op,))
+
+
+def _run_group(members, consumers, target_ids):
+    """One launch for a group of element / broadcast ops."""
+    lib = _lib.ensure_init()
+    member_ids = {op.id for op in members}
+    shape = members[-1].out.shape
+    fvars, fops = [], []
+    index = {}           # (var id, bcast mask) -> fused var index
+    keep = []            # keeps arrays alive
+
+    def add_var(role, dtype, ptr=None, fvalue=0.0, ivalue=0, mask=0):
+        fv = _lib.FusedVar()
+        fv.role, fv.dtype, fv.ptr = role, _lib.DTYPE_CODE[dtype], ptr
+        fv.fvalue, fv.ivalue, fv.bcast_mask = float(fvalue), int(ivalue), mask
+        fvars.append(fv)
+        return len(fvars) - 1
+
+    def external(u, mask):
+        key = (u.id, mask)
+        if key in index:
+            return index[key]
+        if u._op is None and u._host is not None and u.num == 1:
+            # one-element host array: by-value kernel argument (ops/array_op.cc:56-60)
+            h = u._host.reshape(-1)[0]
+            if u.dtype == "bfloat16":
+                from .dtypes import bf16_bits_to_f32
+                val = float(bf16_bits_to_f32(u._host).reshape(-1)[0])
+                i = add_var(_lib.VAR_SCALAR, u.dtype, fvalue=val)
+            elif u.is_float():
+                i = add_var(_lib.VAR_SCALAR, u.dtype, fvalue=float(h))
+            else:
+                i = add_var(_lib.VAR_SCALAR, u.dtype, ivalue=int(h))
+        else:
+            i = add_var(_lib.VAR_INPUT, u.dtype, ptr=u._device_ptr(), mask=mask)
+        index[key] = i
+        return i
+
+    outputs = []
+    for op in members:
+        ins = []
+        if isinstance(op, BroadcastOp):
+            u = op.inputs[0]
+            full = (1 << len(shape)) - 1
+            ins.append(external(u, op.bcast_mask & full))
+        else:
+            for u in op.inputs:
+                p = u._op
+                if p is not None and p.id in member_ids and u._buf is None:
+                    ins.append(index[(u.id, 0)])
+                else:
+                    ins.append(external(u, 0))
+        out = op.out
+        used_outside = out.id in target_ids or any(c.id not in member_ids for c in consumers.get(out.id, ()))
+        if used_outside:
+            oi = add_var(_lib.VAR_OUTPUT, out.dtype, ptr=_alloc_out(out))
+            outputs.append(out)
+        else:
+            oi = add_var(_lib.VAR_INTERMEDIATE, out.dtype)
+        index[(out.id, 0)] = oi
+        fo = _lib.FusedOp()
+        if isinstance(op, UnaryOp):
+            fo.kind, fo.op = _lib.FOP_UNARY, _lib.OP_CODE[op.op]
+        elif isinstance(op, BinaryOp):
+            fo.kind, fo.op = _lib.FOP_BINARY, _lib.OP_CODE[op.op]
+        elif isinstance(op, TernaryOp):
+            fo.kind, fo.op = _lib.FOP_TERNARY, 0
+        else:
+            fo.kind, fo.op = _lib.FOP_BROADCAST, 0
+        for j, v in enumerate(ins):
+            fo.inp[j] = v
+        fo.out = oi
+        fops.append(fo)
+    if not outputs:
+        return
+    desc = _lib.FusedDesc()
+    desc.ndim = len(shape)
+    for i, s in enumerate(shape):
+        desc.shape[i] = s
+    varr = (_lib.FusedVar * len(fvars))(*fvars)
+    oarr = (_lib.FusedOp * len(fops))(*fops)
+    desc.n_vars, desc.vars, desc.n_ops, desc.ops = len(fvars), varr, len(fops), oarr
+    stats["launches"] += 1
+    stats["fused_groups"] += 1
+    _lib.check(lib.mjt_fused_elementwise(ctypes.byref(desc)))

@@ -1,0 +1,403 @@
+"""GPU parity: the HIP path (through the C-ABI, via the ctypes front end)
+against the CPU oracle on the same seeded inputs.  Bar: bit-exact for reindex
+and integer work; 1e-5 relative for fp32 reduce / element-wise; 1e-4 relative
+for atomic scatter-add.  Full-size benchmark shapes are checked through
+closed forms and size-independent properties."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import jittor_amd as jt
+from jittor_amd import _lib as L
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+G = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "vectors.json")))
+
+
+def bits(a):
+    a = np.ascontiguousarray(a)
+    return a.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize])
+
+
+def exact(a, b):
+    return a.shape == b.shape and a.dtype == b.dtype and np.array_equal(bits(a), bits(b))
+
+
+# ---- golden vectors ------------------------------------------------------------------
+def test_golden_vectors(gpu):
+    g = G["reindex_shift"]
+    assert jt.array(np.array(g["x"], np.int32)).reindex(g["shape"], g["indexes"]).data.tolist() == g["y"]
+    g = G["reduce_negative_dim"]
+    a = jt.array(g["x"])
+    assert a.sum(-1).data.tolist() == g["sum_m1"] and a.sum(-2).data.tolist() == g["sum_m2"]
+    g = G["broadcast_dims"]
+    b = jt.array(g["x"])
+    assert b.broadcast(g["shape"], [-1]).data.tolist() == g["dims_m1"]
+    assert b.broadcast(g["shape"], [-2]).data.tolist() == g["dims_m2"]
+    g = G["add_scalar"]
+    assert (jt.array(g["x"]) + 1).data.tolist() == g["plus1"]
+    g = G["gather"]
+    t, idx = jt.array(g["t"]), jt.array(g["index"])
+    assert t.reindex(idx.shape, ["i0", "@e0(i0,i1)"], extras=[idx]).data.tolist() == g["dim1"]
+    assert t.reindex(idx.shape, ["@e0(i0,i1)", "i1"], extras=[idx]).data.tolist() == g["dim0"]
+    g = G["scatter_void"]
+    src = np.array(g["src"], np.int32)
+    out = jt.array(src[:1, :4]).reindex_reduce("void", [3, 5], ["@e0(i0,i1)", "i1"], extras=[jt.array(g["index0"])])
+    assert out.data.tolist() == g["out0"]
+    out = jt.array(src[:2, :3]).reindex_reduce("void", [3, 5], ["i0", "@e0(i0,i1)"], extras=[jt.array(g["index1"])])
+    assert out.data.tolist() == g["out1"]
+    g = G["bool_reduce"]
+    assert bool((jt.array(np.array(g["a"], bool)) | jt.array(np.array(g["b"], bool))).all().item()) is g["or_all"]
+    assert bool((jt.array(np.array(g["a"], bool)) & jt.array(np.array(g["b"], bool))).any().item()) is g["and_any"]
+
+
+# ---- reduce -------------------------------------------------------------------------------
+@pytest.mark.parametrize("keepdims", [False, True])
+def test_reduce_integer_exact(gpu, keepdims):
+    a = np.arange(2 * 3 * 4 * 5).reshape(2, 3, 4, 5).astype(np.int32)
+    ja = jt.array(a)
+    for dims in [(), (0,), (1,), (2,), (3,), (0, 2), (1, 3), (1, 2, 3), 2, 3]:
+        for op in ["add", "multiply", "maximum", "minimum", "logical_and", "logical_or", "logical_xor",
+                   "bitwise_and", "bitwise_or", "bitwise_xor"]:
+            if dims not in ((), (0,)) and op != "add":
+                continue
+            got = jt.reduce(ja, op, dims, keepdims).data
+            ref = O.reduce(a, op, dims, keepdims)
+            assert exact(got, ref), (op, dims, got, ref)
+
+
+@pytest.mark.parametrize("shape,dims", [((64, 33, 5), (1,)), ((64, 33, 5), (0, 2)), ((64, 33, 5), ()),
+                                        ((7, 1000), (1,)), ((1000, 7), (0,)), ((3, 5, 7, 9, 2), (1, 3)),
+                                        ((2, 70000), (1,)), ((70000, 4), (0,)), ((5, 0), (1,)), ((4, 6, 8), (2,))])
+def test_reduce_float(gpu, shape, dims):
+    rng = np.random.default_rng(7)
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    n_red = max(1, x.size // max(1, int(np.prod(O.reduce_shape(shape, dims, False)[0]))))
+    for op in ["add", "maximum", "minimum", "mean"]:
+        got = jt.reduce(jt.array(x), op, dims).data
+        ref = O.reduce(x, op, dims)
+        assert got.shape == ref.shape and got.dtype == ref.dtype
+        if op in ("maximum", "minimum"):
+            assert exact(got, ref), op
+        else:
+            # tolerance: 1e-5 relative, with the absolute floor a reordered fp32 sum of n terms needs
+            assert np.allclose(got, ref, rtol=1e-5, atol=1e-5 * np.sqrt(n_red)), (op, np.abs(got - ref).max())
+
+
+def test_reduce_other_dtypes(gpu):
+    rng = np.random.default_rng(8)
+    for dtype in ["int8", "uint8", "int16", "int64", "float64", "bool"]:
+        x = (rng.integers(0, 2, (6, 40)) if dtype == "bool" else rng.integers(0, 5, (6, 40))).astype(L.NP_STORAGE[dtype])
+        for op in ["add", "maximum"]:
+            got = jt.reduce(jt.array(x, dtype), op, 1).data
+            ref = O.reduce(x, op, 1)
+            assert got.dtype == ref.dtype and np.array_equal(got, ref), (dtype, op)
+    h = rng.standard_normal((4, 64)).astype(np.float32)
+    got = jt.array(h).bfloat16().sum(1).data          # cast -> float32 sum -> cast (truncation)
+    hb = O.BF16(O.f32_to_bf16_bits(h)).to_f32()
+    want = O.BF16(O.f32_to_bf16_bits(O.reduce(hb, "add", 1))).to_f32()
+    assert np.allclose(got, want, rtol=2 ** -7)
+
+
+def test_reduce_full_size_c1(gpu):
+    x = np.random.default_rng(0).uniform(-1, 1, (8192, 4096)).astype(np.float32)
+    got = jt.array(x).sum(1).data
+    assert L.last_kernel().startswith("mjt_reduce_row_add_float32")
+    ref = x.astype(np.float64).sum(1)
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-5 * np.sqrt(4096))
+    # linearity: sum(2x) == 2 sum(x) exactly (power-of-two scaling commutes with rounding)
+    assert np.array_equal(jt.array(2 * x).sum(1).data, 2 * got)
+
+
+# ---- reindex ----------------------------------------------------------------------------------
+def test_reindex_pad_matmul_and_conditions(gpu):
+    rng = np.random.default_rng(9)
+    a = rng.random(10).astype(np.float32)
+    assert exact(jt.array(a).reindex([17], ["i0-3"], -1).data, O.reindex(a, [17], ["i0-3"], -1))
+    n = 10
+    A, B = rng.random((n, n)).astype(np.float32), rng.random((n, n)).astype(np.float32)
+    cc = jt.array(A).reindex([n, n, n], ["i0", "i1"]) * jt.array(B).reindex([n, n, n], ["i1", "i2"])
+    assert np.allclose(cc.sum(1).data, A @ B, rtol=1e-5)
+    x = rng.random((2, 4, 4, 2)).astype(np.float32)
+    shape, idx, ofc = [2, 10, 10, 3, 3, 2], ["i0", "(i1-i3)/2", "(i2-i4)/2", "i5"], ["(i1-i3)%2", "(i2-i4)%2"]
+    assert exact(jt.array(x).reindex(shape, idx, 0, ofc).data, O.reindex(x, shape, idx, 0, ofc))
+    # reflect-style ternary expression and shape names
+    e = ["i0<2 ? 2-i0 : (i0>=xshape0+2 ? 2*xshape0-i0 : i0-2)"]
+    assert exact(jt.array(a).reindex([14], e).data, O.reindex(a, [14], e))
+
+
+def test_reindex_extras_and_dtypes(gpu):
+    rng = np.random.default_rng(10)
+    a = rng.random((10, 10)).astype(np.float32)
+    b = np.array([2], np.int32)
+    e1 = rng.integers(0, 10, (10, 10)).astype(np.float32)
+    idx = ["@e0(0)", "@e1(0,i0 / @e0(0))"]
+    assert exact(jt.array(a).reindex([8, 8], idx, extras=[jt.array(b), jt.array(e1)]).data,
+                 O.reindex(a, [8, 8], idx, extras=[b, e1]))
+    iv = rng.integers(-3, 13, (6, 7)).astype(np.int64)          # out of range on both sides -> overflow value
+    for dtype in ["int8", "int16", "int32", "int64", "uint8", "float64", "bool", "float16"]:
+        x = (rng.random(10) * 10).astype(L.NP_STORAGE[dtype])
+        got = jt.array(x, dtype).reindex_var([jt.array(iv, "int64")], 1).data
+        assert exact(got, O.reindex(x, [6, 7], ["@e0(i0,i1)"], 1, extras=[iv])), dtype
+    xb = jt.array(rng.standard_normal(10).astype(np.float32)).bfloat16()
+    got = xb.reindex([6, 7], ["@e0(i0,i1)"], 1.5, extras=[jt.array(iv, "int64")]).raw()
+    assert np.array_equal(got, O.reindex(O.BF16(xb.raw()), [6, 7], ["@e0(i0,i1)"], 1.5, extras=[iv]).bits)
+    assert jt.array(a).reindex([0, 4], ["i0", "i1"]).data.shape == (0, 4)
+
+
+@pytest.mark.parametrize("case", [
+    dict(x=(2, 3, 7, 6), k=(3, 3), s=(1, 1), d=(1, 1), p=(1, 1)),
+    dict(x=(3, 9, 11), k=(3, 2), s=(2, 1), d=(1, 2), p=(0, 1)),
+    dict(x=(13, 17), k=(5, 5), s=(1, 1), d=(1, 1), p=(2, 2)),
+    dict(x=(2, 2, 70, 64), k=(3, 3), s=(1, 1), d=(1, 1), p=(1, 1)),
+    dict(x=(1, 200, 8), k=(2, 2), s=(2, 2), d=(1, 1), p=(0, 0)),
+])
+@pytest.mark.parametrize("dtype", ["float32", "int16", "float64"])
+def test_window_gather_fast_path_matches_oracle_and_generic(gpu, case, dtype):
+    rng = np.random.default_rng(11)
+    xs, (kh, kw), (sh, sw), (dh, dw), (ph, pw) = case["x"], case["k"], case["s"], case["d"], case["p"]
+    H, W = xs[-2], xs[-1]
+    oh = (H + 2 * ph - dh * (kh - 1) - 1) // sh + 1
+    ow = (W + 2 * pw - dw * (kw - 1) - 1) // sw + 1
+    nb = len(xs) - 2
+    x = (rng.standard_normal(xs) * 50).astype(L.NP_STORAGE[dtype])
+    shape = list(xs[:nb]) + [oh, ow, kh, kw]
+    idx = ["i%d" % i for i in range(nb)] + ["i%d*%d+i%d*%d-%d" % (nb, sh, nb + 2, dh, ph),
+                                            "i%d*%d+i%d*%d-%d" % (nb + 1, sw, nb + 3, dw, pw)]
+    ref = O.reindex(x, shape, idx, 3)
+    got = jt.array(x, dtype).reindex(shape, idx, 3).data
+    fast = L.last_kernel()
+    assert exact(got, ref)
+    os.environ["MJT_NO_FASTPATH"] = "1"
+    try:
+        got2 = jt.array(x, dtype).reindex(shape, idx, 3).data
+        assert L.last_kernel().startswith("mjt_reindex_")
+    finally:
+        del os.environ["MJT_NO_FASTPATH"]
+    assert exact(got2, ref)
+    assert fast.startswith("mjt_window_gather"), fast
+
+
+def test_reindex_full_size_c2_bit_exact(gpu):
+    x = np.random.default_rng(0).standard_normal((32, 64, 56, 56)).astype(np.float32)
+    y = jt.array(x).reindex([32, 64, 56, 56, 3, 3], ["i0", "i1", "i2+i4-1", "i3+i5-1"], 0).data
+    assert L.last_kernel().startswith("mjt_window_gather")
+    ref = np.lib.stride_tricks.sliding_window_view(np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1))), (3, 3), axis=(2, 3))
+    assert np.array_equal(bits(y), bits(ref))
+
+
+# ---- reindex_reduce ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("op", ["maximum", "minimum", "multiply", "add"])
+def test_reindex_reduce_pool(gpu, op):
+    x = np.random.default_rng(12).random((3, 10, 10, 4)).astype(np.float32)
+    idx = ["i0", "i1/3", "i2/3", "i3"]
+    got = jt.array(x).reindex_reduce(op, [3, 4, 4, 4], idx).data
+    ref = O.reindex_reduce(x, op, [3, 4, 4, 4], idx)
+    if op in ("maximum", "minimum"):
+        assert exact(got, ref)
+    else:
+        assert np.allclose(got, ref, rtol=1e-4)
+
+
+def test_reindex_reduce_dtypes_and_overflow(gpu):
+    rng = np.random.default_rng(13)
+    n, bins = 4000, 50
+    idx = (rng.integers(0, bins + 6, n) - 3).astype(np.int32)
+    for dtype in ["int32", "int64", "uint32", "int8", "int16", "float64"]:
+        v = rng.integers(0, 3, n).astype(L.NP_STORAGE[dtype])
+        for op in ["add", "maximum", "minimum", "bitwise_or"]:
+            if dtype == "float64" and op == "bitwise_or":
+                continue
+            got = jt.array(v, dtype).reindex_reduce(op, [bins], ["@e0(i0)"], extras=[jt.array(idx)]).data
+            ref = O.reindex_reduce(v, op, [bins], ["@e0(i0)"], extras=[idx])
+            assert got.dtype == ref.dtype and np.array_equal(got, ref), (dtype, op)
+    # two-axis target, extras of another shape (test/test_reindex_reduce_op.py:79-90)
+    a = np.array([1, 2, 3, 0], np.int32)
+    b = rng.random((3, 3)).astype(np.float32)
+    got = jt.array(b).reindex_reduce("add", [4, 4], ["@e0(i0)", "@e0(i1)"], extras=[jt.array(a)]).data
+    assert np.allclose(got, O.reindex_reduce(b, "add", [4, 4], ["@e0(i0)", "@e0(i1)"], extras=[a]))
+
+
+@pytest.mark.parametrize("n,bins", [(1 << 16, 300), (100003, 1 << 17), (5, 3), (1 << 18, 40000)])
+def test_scatter_1d_fast_path(gpu, n, bins):
+    rng = np.random.default_rng(14)
+    v = rng.random(n).astype(np.float32)
+    v[::97] = np.nan if n > 100 else v[::97]
+    vi = np.nan_to_num(v)
+    idx = np.minimum((rng.pareto(1.0, n) * 3).astype(np.int64), bins + 2).astype(np.int32) - 1   # skewed, some out of range
+    ok = (idx >= 0) & (idx < bins)
+    jv, ji = jt.array(vi), jt.array(idx)
+    got = jv.reindex_reduce("add", [bins], ["@e0(i0)"], extras=[ji]).data
+    assert L.last_kernel().startswith("mjt_scatter1d_add")
+    ref = np.bincount(idx[ok], weights=vi[ok].astype(np.float64), minlength=bins)
+    assert np.allclose(got, ref, rtol=1e-4, atol=1e-6)
+    for op, at in (("maximum", np.maximum), ("minimum", np.minimum)):
+        got = jt.array(v).reindex_reduce(op, [bins], ["@e0(i0)"], extras=[ji]).data      # NaN values never win
+        assert exact(got, O.reindex_reduce(v, op, [bins], ["@e0(i0)"], extras=[idx])), op
+    i64 = jt.array(idx.astype(np.int64), "int64")
+    got = jt.array(np.ones(n, np.int32)).reindex_reduce("add", [bins], ["@e0(i0)"], extras=[i64]).data
+    assert np.array_equal(got, np.bincount(idx[ok], minlength=bins).astype(np.int32))
+
+
+def _zipf_indices(n, bins):
+    w = np.arange(1, bins + 1, dtype=np.float64) ** -1.1
+    cdf = np.cumsum(w) / w.sum()
+    return np.minimum(np.searchsorted(cdf, np.random.default_rng(1).random(n)), bins - 1).astype(np.int32)
+
+
+def test_scatter_full_size_c3(gpu):
+    n, bins = 1 << 24, 1 << 20
+    v = np.random.default_rng(0).random(n, dtype=np.float32)
+    idx = _zipf_indices(n, bins)
+    jv, ji = jt.array(v), jt.array(idx)
+    got = jv.reindex_reduce("add", [bins], ["@e0(i0)"], extras=[ji]).data
+    ref = np.bincount(idx, weights=v.astype(np.float64), minlength=bins)
+    assert np.allclose(got, ref, rtol=1e-4, atol=0)                     # empty bins are exactly 0
+    assert abs(got.astype(np.float64).sum() - ref.sum()) <= 1e-6 * ref.sum()
+    got = jv.reindex_reduce("maximum", [bins], ["@e0(i0)"], extras=[ji]).data
+    ref = np.full(bins, np.finfo(np.float32).min, np.float32)
+    np.maximum.at(ref, idx, v)
+    assert np.array_equal(got, ref)
+    # a shifted hot region must give the same answer (the LDS window follows the data)
+    shifted = ((idx.astype(np.int64) + 700001) % bins).astype(np.int32)
+    got = jv.reindex_reduce("add", [bins], ["@e0(i0)"], extras=[jt.array(shifted)]).data
+    ref = np.bincount(shifted, weights=v.astype(np.float64), minlength=bins)
+    assert np.allclose(got, ref, rtol=1e-4, atol=0)
+
+
+# ---- element-wise and fused chains ------------------------------------------------------------------------
+UNARY_RANGES = {"log": (0.1, 5), "sqrt": (0, 5), "asin": (-1, 1), "acos": (-1, 1), "acosh": (1, 5), "atanh": (-0.99, 0.99),
+                "erfinv": (-0.99, 0.99), "exp": (-5, 5), "sinh": (-5, 5), "cosh": (-5, 5)}
+
+
+@pytest.mark.parametrize("op", L.UNARY_OPS)
+def test_unary_ops(gpu, op):
+    if op == "cast":
+        pytest.skip("covered by test_casts")
+    rng = np.random.default_rng(15)
+    lo, hi = UNARY_RANGES.get(op, (-4, 4))
+    x = rng.uniform(lo, hi, 1031).astype(np.float32)
+    if op in ("logical_not", "bitwise_not"):
+        xi = rng.integers(-5, 5, 1031).astype(np.int32)
+        got, ref = jt.unary(jt.array(xi), op).data, O.unary(xi, op)
+        assert exact(got, ref)
+        return
+    got, ref = jt.unary(jt.array(x), op).data, O.unary(x, op)
+    assert got.dtype == ref.dtype
+    if ref.dtype.kind != "f" or op in ("abs", "negative", "floor", "ceil", "round"):
+        assert exact(got, ref), op
+    else:
+        assert np.allclose(got, ref, rtol=1e-5, atol=1e-6), (op, np.abs(got - ref).max())
+
+
+@pytest.mark.parametrize("op", [o for o in L.BINARY_OPS if o != "mean"])
+def test_binary_ops(gpu, op):
+    rng = np.random.default_rng(16)
+    if op in ("left_shift", "right_shift", "bitwise_and", "bitwise_or", "bitwise_xor"):
+        pairs = [(rng.integers(0, 100, 515).astype(np.int32), rng.integers(0, 5, 515).astype(np.int32))]
+    else:
+        xf, yf = rng.uniform(0.5, 4, 515).astype(np.float32), rng.uniform(-3, 3, 515).astype(np.float32)
+        yf[np.abs(yf) < 0.1] = 1.0
+        xi, yi = rng.integers(-20, 20, 515).astype(np.int32), rng.integers(1, 7, 515).astype(np.int32) * rng.choice([-1, 1], 515).astype(np.int32)
+        pairs = [(xf, yf), (xi, yi)] if op != "pow" else [(xf, yf)]
+        if op in ("add", "multiply", "maximum", "less"):
+            pairs.append((xi.astype(np.int8), yf))            # mixed widths / kinds
+    for x, y in pairs:
+        got, ref = jt.binary(jt.array(x), jt.array(y), op).data, O.binary(x, y, op)
+        assert got.dtype == ref.dtype, (op, got.dtype, ref.dtype)
+        if ref.dtype.kind == "f":
+            assert np.allclose(got, ref, rtol=1e-5, atol=1e-6), (op, x.dtype)
+        else:
+            assert np.array_equal(got, ref), (op, x.dtype)
+
+
+def test_casts(gpu):
+    rng = np.random.default_rng(17)
+    x = (rng.standard_normal(300) * 40).astype(np.float32)
+    for dtype in ["bool", "int8", "int16", "int32", "int64", "uint8", "float16", "float64", "bfloat16"]:
+        j = jt.array(x).cast(dtype)
+        ref = O.c_cast(np.clip(x, 0, 100) if dtype == "uint8" else x, dtype)
+        if dtype == "uint8":
+            j = jt.array(np.clip(x, 0, 100)).cast(dtype)
+        if dtype == "bfloat16":
+            assert np.array_equal(j.raw(), ref.bits)           # truncation, not rounding
+        else:
+            assert exact(j.data, ref), dtype
+    b = jt.array(x).bfloat16()
+    assert np.array_equal(b.float32().data, O.BF16(b.raw()).to_f32())
+
+
+def _c4(x, s, b):
+    return jt.exp(-jt.nn.relu(x * s + b)) * jt.sigmoid(x)
+
+
+def _c4_oracle(x, s, b):
+    t = O.binary(O.binary(x, O.broadcast_to(s, x.shape), "multiply"), O.broadcast_to(b, x.shape), "add")
+    zero = np.zeros(1, np.float32)
+    r = O.ternary(O.binary(t, O.broadcast_to(zero, x.shape), "greater"), t, O.broadcast_to(zero, x.shape))
+    return O.binary(O.unary(O.unary(r, "negative"), "exp"), O.unary(x, "sigmoid"), "multiply")
+
+
+@pytest.mark.parametrize("shape", [(4, 6, 8), (3, 5, 7), (2, 512, 1024)])
+def test_fused_chain_c4_small(gpu, shape):
+    x = np.random.default_rng(0).standard_normal(shape).astype(np.float32)
+    s = np.random.default_rng(1).standard_normal((shape[1], 1)).astype(np.float32)
+    b = np.random.default_rng(2).standard_normal((1, shape[2])).astype(np.float32)
+    before = jt.executor_stats["launches"]
+    got = _c4(jt.array(x), jt.array(s), jt.array(b)).data
+    assert jt.executor_stats["launches"] == before + 1            # one kernel for the whole chain
+    assert L.last_kernel().startswith("mjt_fused_")
+    ref = _c4_oracle(x, s, b)
+    assert np.allclose(got, ref, rtol=1e-5, atol=0), np.abs(got / ref - 1).max()
+
+
+def test_fused_chain_full_size_c4(gpu):
+    shape = (64, 512, 1024)
+    x = np.random.default_rng(0).standard_normal(shape).astype(np.float32)
+    s = np.random.default_rng(1).standard_normal((512, 1)).astype(np.float32)
+    b = np.random.default_rng(2).standard_normal((1, 1024)).astype(np.float32)
+    got = _c4(jt.array(x), jt.array(s), jt.array(b)).data
+    x64 = x.astype(np.float64)
+    ref = np.exp(-np.maximum(x64 * s + b, 0)) / (1 + np.exp(np.minimum(-x64, 30)))
+    assert np.abs(got / ref - 1).max() < 1e-5                     # all outputs are positive
+    sl = (slice(0, 64, 9), slice(0, 512, 37), slice(None))
+    assert np.allclose(got[sl], _c4_oracle(x[sl], s[sl[1]], b), rtol=1e-5, atol=0)
+
+
+def test_fused_groups_outputs_scalars_and_bool(gpu):
+    rng = np.random.default_rng(18)
+    x = rng.standard_normal((33, 17)).astype(np.float32)
+    y = rng.standard_normal((33, 17)).astype(np.float32)
+    jx, jy = jt.array(x), jt.array(y)
+    a = jx * 2.0 + jy                       # shared by both outputs
+    m = a > 0.5
+    z = jt.ternary(m, a, jy * 0.25)
+    before = jt.executor_stats["launches"]
+    jt.sync([a, m, z])
+    assert jt.executor_stats["launches"] == before + 1
+    ra = x * np.float32(2.0) + y
+    assert np.allclose(a.data, ra, rtol=1e-6) and np.array_equal(m.data, ra > 0.5)
+    assert np.allclose(z.data, np.where(ra > 0.5, ra, y * np.float32(0.25)), rtol=1e-6)
+    # a [1]-shaped computed Var (a full reduce) broadcasts as a tensor input
+    t = jx - jx.mean()
+    assert np.allclose(t.data, x - x.mean(), rtol=1e-5, atol=1e-6)
+    # relu(NaN) = 0 (python/jittor/nn.py:182-183)
+    assert jt.nn.relu(jt.array(np.array([np.nan, -1.0, 2.0], np.float32))).data.tolist() == [0.0, 0.0, 2.0]
+    # broadcast alone materialises through the same kernel family
+    assert np.array_equal(jt.array(x[:, :1]).broadcast([33, 17]).data, np.broadcast_to(x[:, :1], (33, 17)))
+    assert jt.zeros([0, 3]).exp().data.shape == (0, 3)
+
+
+def test_lazy_graph_recomputes_fused_intermediates(gpu):
+    x = np.random.default_rng(19).random(100).astype(np.float32)
+    c = jt.array(x) * 3.0
+    d = c + 1.0
+    assert np.allclose(d.data, x * 3 + 1)
+    assert np.allclose(c.data, x * 3)          # c was fused away; asking for it later still works
+    s = (jt.array(x).reindex([100, 3], ["i0"]) * 2.0).sum(1)      # element group feeding a reduce
+    assert np.allclose(s.data, x * 6, rtol=1e-6)
+    h = jt.histc(jt.array(x), 10, 0.0, 1.0).data
+    assert np.array_equal(h, np.histogram(x, 10, (0, 1))[0].astype(np.float32))

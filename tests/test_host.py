@@ -1,0 +1,248 @@
+"""Host-side logic without a GPU: the C-ABI library loads and exports every
+symbol include/mjt.h declares, descriptors are validated, index expressions
+parse as the reference's language, the front end reproduces the constructor
+rewrites / dtype rules, and kernels specialise + compile for gfx950."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+import jittor_amd as jt
+from jittor_amd import _lib as L
+
+G = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "vectors.json")))
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+P = 0x100000     # fake, aligned device pointer: nothing is launched in compile-only mode
+
+
+def test_library_exports_every_declared_symbol():
+    lib = L.load()
+    header = open(os.path.join(ROOT, "include", "mjt.h")).read()
+    declared = set(re.findall(r"\b(mjt_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(L.EXPORTS), declared ^ set(L.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+
+
+def test_names_and_codes():
+    lib = L.load()
+    for i, n in enumerate(L.DTYPES):
+        assert lib.mjt_dtype_name(i).decode() == n
+    for i, n in enumerate(L.OPS):
+        assert lib.mjt_op_name(i).decode() == n
+    assert lib.mjt_op_from_name(b"add") == L.OP_CODE["add"]
+    assert lib.mjt_op_from_name(b"nope") < 0
+    assert lib.mjt_dtype_from_name(b"bfloat16") == L.DTYPE_CODE["bfloat16"]
+
+
+def test_calls_fail_cleanly_without_init():
+    L.shutdown()
+    lib = L.load()
+    x = L.tensor(P, "float32", [4])
+    assert lib.mjt_reduce(ctypes.byref(x), ctypes.byref(x), 3, 1) == -5
+    assert b"mjt_init" in lib.mjt_last_error()
+
+
+def test_expr_affine_and_errors():
+    assert L.expr_affine("i3*2-1+i5*3", (4, 5, 6, 7), (1, 2, 3, 4, 5, 6)) == (-1, [0, 0, 0, 2, 0, 3, 0, 0, 0, 0])
+    assert L.expr_affine("xshape0-1-i0", (4,), (4,)) == (3, [-1] + [0] * 9)
+    assert L.expr_affine("(i1-i3)/2", (4, 4), (4, 4, 4, 4)) is None
+    assert L.expr_affine("7/2*i0 + (0-7)/2", (4,), (4,)) == (-3, [3] + [0] * 9)   # C division truncates
+    assert L.expr_affine("0x10 + 0b11", (4,), (4,)) == (19, [0] * 10)
+    assert L.expr_affine("@e0(i0)", (4,), (4,)) is None
+    with pytest.raises(L.MjtError):
+        L.expr_affine("i0 // 2", (4,), (4,))
+    with pytest.raises(L.MjtError):
+        L.expr_affine("i0 +", (4,), (4,))
+
+
+def test_descriptor_validation(compile_only):
+    lib = compile_only.load()
+    e = L.c_strings([])
+    x, y = L.tensor(P, "float32", [10, 10]), L.tensor(P, "float32", [8, 8])
+    # number of indexes must equal x rank (ops/reindex_op.cc:83)
+    assert lib.mjt_reindex(ctypes.byref(x), ctypes.byref(y), 1, L.c_strings(["i0"]), 0.0, 0, e, 0, None) == -1
+    # '//' is rejected (opt/pass/loop_var_analyze_pass.cc:298-309)
+    ex = (L.Tensor * 1)(L.tensor(P, "int32", [1]))
+    assert lib.mjt_reindex(ctypes.byref(x), ctypes.byref(y), 2, L.c_strings(["@e0(0) // 1", "@e0(0)"]), 0.0, 0, e, 1, ex) == -1
+    # unknown identifier, @eK arity, missing extra
+    assert lib.mjt_reindex(ctypes.byref(x), ctypes.byref(y), 2, L.c_strings(["i5", "i0"]), 0.0, 0, e, 0, None) == -1
+    assert lib.mjt_reindex(ctypes.byref(x), ctypes.byref(y), 2, L.c_strings(["@e0(i0,i1)", "i0"]), 0.0, 0, e, 1, ex) == -1
+    assert lib.mjt_reindex(ctypes.byref(x), ctypes.byref(y), 2, L.c_strings(["@e1(0)", "i0"]), 0.0, 0, e, 1, ex) == -1
+    # reindex_reduce: op must be binary and not mean; indexes == rank of the output
+    v, o = L.tensor(P, "float32", [3]), L.tensor(P, "float32", [3])
+    assert lib.mjt_reindex_reduce(ctypes.byref(v), ctypes.byref(o), L.OP_CODE["mean"], 1, L.c_strings(["i0"]), 0, e, 0, None) == -1
+    assert lib.mjt_reindex_reduce(ctypes.byref(v), ctypes.byref(o), L.OP_CODE["exp"], 1, L.c_strings(["i0"]), 0, e, 0, None) == -1
+    assert lib.mjt_reindex_reduce(ctypes.byref(v), ctypes.byref(o), L.OP_CODE["add"], 2, L.c_strings(["i0", "i0"]), 0, e, 0, None) == -1
+    # reduce: mask must fit, element counts must agree, op must be associative
+    big, small = L.tensor(P, "float32", [4, 5]), L.tensor(P, "float32", [4])
+    assert lib.mjt_reduce(ctypes.byref(big), ctypes.byref(small), L.OP_CODE["add"], 0b100) == -1
+    assert lib.mjt_reduce(ctypes.byref(big), ctypes.byref(small), L.OP_CODE["add"], 0b01) == -1
+    assert lib.mjt_reduce(ctypes.byref(big), ctypes.byref(small), L.OP_CODE["subtract"], 0b10) == -1
+    assert lib.mjt_reduce(ctypes.byref(big), ctypes.byref(small), L.OP_CODE["add"], 0b10) == 0
+
+
+def _fused(lib, shape, vars_, ops_):
+    va = (L.FusedVar * len(vars_))()
+    for i, (role, dt_, mask) in enumerate(vars_):
+        va[i].role, va[i].dtype, va[i].ptr, va[i].bcast_mask = role, L.DTYPE_CODE[dt_], P, mask
+    oa = (L.FusedOp * len(ops_))()
+    for i, (kind, op, ins, out) in enumerate(ops_):
+        oa[i].kind, oa[i].op, oa[i].out = kind, L.OP_CODE[op] if op else 0, out
+        for j, v in enumerate(ins):
+            oa[i].inp[j] = v
+    d = L.FusedDesc()
+    d.ndim = len(shape)
+    for i, s in enumerate(shape):
+        d.shape[i] = s
+    d.n_vars, d.vars, d.n_ops, d.ops = len(vars_), va, len(ops_), oa
+    return lib.mjt_fused_elementwise(ctypes.byref(d))
+
+
+def test_kernels_specialise_for_gfx950(compile_only):
+    """Compile-only mode builds the same kernels a GPU run would launch."""
+    lib = compile_only.load()
+    e = L.c_strings([])
+    before = L.jit_stats()[0]
+    os.environ["MJT_NO_DISK_CACHE"] = "1"
+    try:
+        # the five benchmark shapes
+        x, y = L.tensor(P, "float32", [8192, 4096]), L.tensor(P, "float32", [8192])
+        assert lib.mjt_reduce(ctypes.byref(x), ctypes.byref(y), L.OP_CODE["add"], 0b10) == 0, lib.mjt_last_error()
+        assert L.last_kernel().startswith("mjt_reduce_row_add")
+        x, y = L.tensor(P, "float32", [32, 64, 56, 56]), L.tensor(P, "float32", [32, 64, 56, 56, 3, 3])
+        assert lib.mjt_reindex(ctypes.byref(x), ctypes.byref(y), 4, L.c_strings(["i0", "i1", "i2+i4-1", "i3+i5-1"]),
+                               0.0, 0, e, 0, None) == 0, lib.mjt_last_error()
+        assert L.last_kernel().startswith("mjt_window_gather")
+        v, o = L.tensor(P, "float32", [1 << 24]), L.tensor(P, "float32", [1 << 20])
+        ex = (L.Tensor * 1)(L.tensor(P, "int32", [1 << 24]))
+        for op in ("add", "maximum"):
+            assert lib.mjt_reindex_reduce(ctypes.byref(v), ctypes.byref(o), L.OP_CODE[op], 1, L.c_strings(["@e0(i0)"]),
+                                          0, e, 1, ex) == 0, lib.mjt_last_error()
+            assert L.last_kernel().startswith("mjt_scatter1d_" + op)
+        vars_ = [(0, "float32", 0), (0, "float32", 0b101), (0, "float32", 0b011), (3, "float32", 0),
+                 (1, "float32", 0), (1, "float32", 0), (1, "bool", 0), (1, "float32", 0), (1, "float32", 0),
+                 (1, "float32", 0), (1, "float32", 0), (2, "float32", 0)]
+        ops_ = [(1, "multiply", [0, 1], 4), (1, "add", [4, 2], 5), (1, "greater", [5, 3], 6), (2, None, [6, 5, 3], 7),
+                (0, "negative", [7], 8), (0, "exp", [8], 9), (0, "sigmoid", [0], 10), (1, "multiply", [9, 10], 11)]
+        assert _fused(lib, [64, 512, 1024], vars_, ops_) == 0, lib.mjt_last_error()
+        # a generic gather with extras and a generic scatter
+        x, y = L.tensor(P, "float32", [10, 10]), L.tensor(P, "float32", [8, 8])
+        ex2 = (L.Tensor * 2)(L.tensor(P, "int32", [1]), L.tensor(P, "float32", [10, 10]))
+        assert lib.mjt_reindex(ctypes.byref(x), ctypes.byref(y), 2, L.c_strings(["@e0(0)", "@e1(0,i0 / @e0(0))"]),
+                               0.0, 0, e, 2, ex2) == 0, lib.mjt_last_error()
+        yy, xx = L.tensor(P, "int16", [3, 10, 10, 4]), L.tensor(P, "int16", [3, 4, 4, 4])
+        assert lib.mjt_reindex_reduce(ctypes.byref(yy), ctypes.byref(xx), L.OP_CODE["multiply"], 4,
+                                      L.c_strings(["i0", "i1/3", "i2/3", "i3"]), 0, e, 0, None) == 0, lib.mjt_last_error()
+    finally:
+        del os.environ["MJT_NO_DISK_CACHE"]
+    assert L.jit_stats()[0] >= before + 7
+
+
+def test_fused_graph_validation(compile_only):
+    lib = compile_only.load()
+    # op reads a var that is produced later
+    assert _fused(lib, [8], [(0, "float32", 0), (1, "float32", 0), (2, "float32", 0)],
+                  [(0, "exp", [1], 2), (0, "exp", [0], 1)]) == -1
+    # output never produced
+    assert _fused(lib, [8], [(0, "float32", 0), (2, "float32", 0), (2, "float32", 0)], [(0, "exp", [0], 1)]) == -1
+    # binary op code in a unary slot
+    assert _fused(lib, [8], [(0, "float32", 0), (2, "float32", 0)], [(0, "add", [0], 1)]) == -1
+
+
+# ---- front end: constructor rewrites, shapes, dtypes, errors ---------------------------
+def _count_ops(v, kind):
+    seen, stack, n = set(), [v], 0
+    while stack:
+        u = stack.pop()
+        if u._op is None or u._op.id in seen:
+            continue
+        seen.add(u._op.id)
+        n += u._op.kind == kind
+        stack.extend(u._op.inputs)
+    return n
+
+
+def test_binary_inserts_broadcasts_like_the_reference():
+    # test/test_broadcast_to_op.py:64-101: 0, 1 or 2 broadcast ops
+    a = jt.array([1, 2, 3])
+    assert _count_ops(a + 1, "broadcast") == 1
+    assert _count_ops(a + a, "broadcast") == 0
+    x, y = jt.zeros([3, 1]), jt.zeros([1, 4])
+    z = x + y
+    assert z.shape == [3, 4] and _count_ops(z, "broadcast") == 2
+    assert (jt.zeros([5, 4]) + jt.zeros([4])).shape == [5, 4]
+    with pytest.raises(ValueError):
+        jt.zeros([3, 4]) + jt.zeros([3, 5])
+
+
+def test_broadcast_shapes_and_forwarding():
+    a = jt.array([1, 2])
+    assert a.broadcast([2, 2], [-1]).shape == [2, 2]
+    assert a.broadcast([2]) is a                              # forward(x): nothing to broadcast
+    assert jt.zeros([512, 1]).broadcast([64, 512, 1024])._op.bcast_mask == 0b101
+    assert jt.zeros([1, 1024]).broadcast([64, 512, 1024])._op.bcast_mask == 0b011
+    w = jt.zeros([256, 256, 3, 3]).broadcast([64, 256, 256, 56, 56, 3, 3], [0, 3, 4])
+    assert w.shape == [64, 256, 256, 56, 56, 3, 3] and w._op.bcast_mask == 0b0011001
+    with pytest.raises(ValueError):
+        a.broadcast([2, 2], [5])
+
+
+def test_reduce_shapes_rewrites_and_errors():
+    a = jt.array([[1, 2], [3, 4]])
+    assert a.sum(-1).shape == [2] and a.sum(-1)._op.reduce_mask == 0b10
+    assert a.sum(-2)._op.reduce_mask == 0b01
+    assert a.sum().shape == [1] and a.sum().is_scalar
+    assert a.sum(1, keepdims=True).shape == [2, 1]
+    assert jt.zeros([2, 3, 4, 5]).sum([1, 3]).shape == [2, 4]
+    with pytest.raises(ValueError):
+        jt.reduce_add(jt.array([1, 2, 3]), 2)                 # test/test_reduce_op.py:50
+    h = jt.zeros([4, 4]).bfloat16().sum(1)                    # cast -> reduce(float32) -> cast
+    assert h.dtype == "bfloat16" and h._op.kind == "unary" and h._op.inputs[0].dtype == "float32"
+    assert jt.array([True, False]).sum().dtype == "int32"
+    assert len([n for n in dir(jt) if n.startswith("reduce_")]) >= 10
+
+
+def test_dtype_rules_of_the_front_end():
+    for op, x, y, xs, ys, want in G["dtype_table"]["rows"]:
+        assert jt.dtypes.binary_dtype_infer(op, x, y, xs, ys) == want
+    a = jt.array([1.0, 2.0, 3.0]).bfloat16()
+    assert (a * 1).dtype == "bfloat16"                        # test/test_bf16.py:275-281
+    assert (a * jt.array([1.0, 2.0, 3.0])).dtype == "float32"
+    assert (a * jt.array([1.0, 2.0, 3.0]).sum()).dtype == "bfloat16"
+    assert jt.array([0, 1, 0]).ternary(a, jt.array(1.0)).dtype == "bfloat16"
+    assert (a ** a).dtype == "float32"
+    i = jt.array([1, 2, 3])
+    assert i.dtype == "int32" and jt.array([1.5]).dtype == "float32" and jt.array(np.arange(4, dtype=np.uint8)).dtype == "uint8"
+    assert (i / 2).dtype == "float32" and (i // 2).dtype == "int32" and (i < 2).dtype == "bool"
+    assert i.sqrt().dtype == "float32" and i.float16().exp().dtype == "float32" and i.float32().round_int().dtype == "int32"
+    assert (i.float64() + 1).dtype == "float64"
+    assert i.int32() is i                                      # unary_op.cc:867-870 forwards
+
+
+def test_reindex_constructor_checks():
+    x = jt.zeros([10, 10])
+    with pytest.raises(ValueError):
+        x.reindex([8, 8], ["i0"])
+    y = x.reindex_var([jt.zeros([4, 5]).int32(), jt.zeros([4, 5]).int32()])
+    assert y.shape == [4, 5] and y._op.indexes == ["@e0(i0,i1)", "@e1(i0,i1)"]
+    v = jt.zeros([3])
+    v.reindex_reduce("add", [3], ["i0"])
+    for bad in (lambda: v.reindex_reduce("add", [3], []), lambda: v.reindex_reduce("add", [3], ["i0", "i0"]),
+                lambda: v.reindex_reduce("???", [3], ["i0"]), lambda: v.reindex_reduce("add", [-1], ["i0"])):
+        with pytest.raises(ValueError):
+            bad()                                              # test/test_reindex_reduce_op.py:92-97
+
+
+def test_conv2d_builds_the_meta_op_group():
+    x, w = jt.zeros([2, 3, 8, 8]), jt.zeros([4, 3, 3, 3])
+    y = jt.nn.conv2d(x, w, padding=1)
+    assert y.shape == [2, 4, 8, 8] and y._op.kind == "reduce" and y._op.reduce_mask == 0b1100100
+    mul = y._op.inputs[0]._op
+    assert mul.kind == "binary" and {i._op.kind for i in mul.inputs} == {"reindex", "broadcast"}
+    r = [i for i in mul.inputs if i._op.kind == "reindex"][0]._op
+    assert r.indexes == ["i0", "i2", "i3*1-1+i5*1", "i4*1-1+i6*1"]
+    assert jt.nn.conv2d(x, w, stride=2, padding=1).shape == [2, 4, 4, 4]

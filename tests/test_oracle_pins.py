@@ -1,0 +1,301 @@
+"""Pins the CPU oracle (oracle/oracle.py) against the known-answer vectors the
+reference's tests hold, numpy/scipy closed forms and brute-force loops, chosen
+so that a wrong sign, index or operand order fails one of them.  No GPU."""
+import json
+import os
+
+import numpy as np
+import pytest
+from scipy import special
+
+from oracle import oracle as O
+
+G = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "vectors.json")))
+rng = np.random.default_rng(1234)
+
+
+# ---- golden vectors of the reference ---------------------------------------------
+def test_golden_reindex_shift():
+    g = G["reindex_shift"]
+    y = O.reindex(np.array(g["x"], np.int32), g["shape"], g["indexes"], g["overflow_value"])
+    assert y.tolist() == g["y"]
+
+
+def test_golden_pad_with_overflow_value():
+    # test/test_reindex_op.py:181-190: b = a.reindex([size+l+r], ["i0-l"], -1)
+    size, l, r = 10, 3, 4
+    a = rng.random(size).astype(np.float32)
+    b = O.reindex(a, [size + l + r], ["i0-%d" % l], -1)
+    assert (b[l:l + size] == a).all() and (b[:l] == -1).all() and (b[-r:] == -1).all()
+
+
+def test_golden_reduce_and_broadcast():
+    g = G["reduce_negative_dim"]
+    x = np.array(g["x"], np.int32)
+    assert O.reduce(x, "add", -1).tolist() == g["sum_m1"]
+    assert O.reduce(x, "add", -2).tolist() == g["sum_m2"]
+    g = G["broadcast_dims"]
+    x = np.array(g["x"], np.int32)
+    assert O.broadcast_to(x, g["shape"], [-1]).tolist() == g["dims_m1"]
+    assert O.broadcast_to(x, g["shape"], [-2]).tolist() == g["dims_m2"]
+    g = G["add_scalar"]
+    assert O.binary(np.array(g["x"], np.int32), np.array([1], np.int32), "add", yscalar=True).tolist() == g["plus1"]
+
+
+def test_golden_gather_scatter_tables():
+    g = G["gather"]
+    t, idx = np.array(g["t"], np.int32), np.array(g["index"], np.int32)
+    assert O.reindex(t, idx.shape, ["i0", "@e0(i0,i1)"], extras=[idx]).tolist() == g["dim1"]
+    assert O.reindex(t, idx.shape, ["@e0(i0,i1)", "i1"], extras=[idx]).tolist() == g["dim0"]
+    g = G["scatter_void"]
+    src = np.array(g["src"], np.int32)
+    i0 = np.array(g["index0"], np.int32)
+    out = O.reindex_reduce(src[:1, :4], "void", [3, 5], ["@e0(i0,i1)", "i1"], extras=[i0])
+    assert out.tolist() == g["out0"]
+    i1 = np.array(g["index1"], np.int32)
+    out = O.reindex_reduce(src[:2, :3], "void", [3, 5], ["i0", "@e0(i0,i1)"], extras=[i1])
+    assert out.tolist() == g["out1"]
+
+
+def test_golden_dtype_table():
+    for op, x, y, xs, ys, want in G["dtype_table"]["rows"]:
+        assert O.binary_dtype_infer(op, x, y, xs, ys) == want
+    # test/test_bf16.py:280: ternary(int cond, bf16, float32 scalar) -> bfloat16
+    assert O.dtype_infer("bfloat16", "float32", False, True) == "bfloat16"
+    # test/test_bf16.py:250-255: a**a on bfloat16 is float32 (white list)
+    assert O.binary_dtype_infer("pow", "bfloat16", "bfloat16") == "float32"
+    assert O.reduce_dtype_infer("add", "bfloat16") == "float32"
+    assert O.unary_dtype_infer("sqrt", "int32") == "float32"
+    assert O.unary_dtype_infer("exp", "float16") == "float32"
+    assert O.binary_dtype_infer("divide", "int32", "int32") == "float32"
+    assert O.binary_dtype_infer("floor_divide", "int32", "int32") == "int32"
+    assert O.binary_dtype_infer("less", "float32", "float32") == "bool"
+    assert O.reduce_dtype_infer("add", "bool") == "int32"
+
+
+def test_golden_bool_reduce():
+    g = G["bool_reduce"]
+    a, b = np.array(g["a"], bool), np.array(g["b"], bool)
+    assert bool(O.reduce(O.binary(a, b, "bitwise_or"), "logical_and")[0]) is g["or_all"]
+    assert bool(O.reduce(O.binary(a, b, "bitwise_and"), "logical_or")[0]) is g["and_any"]
+
+
+# ---- reindex: closed forms and brute force ----------------------------------------
+def test_reindex_im2col_closed_form():
+    x = rng.standard_normal((2, 3, 7, 6)).astype(np.float32)
+    y = O.reindex(x, [2, 3, 7, 6, 3, 3], ["i0", "i1", "i2+i4-1", "i3+i5-1"], 0)
+    ref = np.lib.stride_tricks.sliding_window_view(np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1))), (3, 3), axis=(2, 3))
+    assert np.array_equal(y, ref)
+
+
+def test_reindex_matmul_identity():
+    # test/test_reindex_op.py:192-204: two reindexes, multiply, sum == np.matmul
+    n = 6
+    a, b = rng.random((n, n)).astype(np.float32), rng.random((n, n)).astype(np.float32)
+    cc = O.binary(O.reindex(a, [n, n, n], ["i0", "i1"]), O.reindex(b, [n, n, n], ["i1", "i2"]), "multiply")
+    c = O.reduce(cc, "add", 1)
+    assert np.allclose(c, a @ b)
+
+
+def test_reindex_brute_force_with_conditions():
+    # transposed-convolution indices with C truncating division and overflow conditions
+    x = rng.random((2, 4, 4, 2)).astype(np.float32)
+    shape = [2, 10, 10, 3, 3, 2]
+    idx = ["i0", "(i1-i3)/2", "(i2-i4)/2", "i5"]
+    ofc = ["(i1-i3)%2", "(i2-i4)%2"]
+    y = O.reindex(x, shape, idx, 0, ofc)
+    ref = np.zeros(shape, np.float32)
+    for c in np.ndindex(*shape):
+        i0, i1, i2, i3, i4, i5 = c
+        h, w = int((i1 - i3) / 2), int((i2 - i4) / 2)     # C division truncates toward zero
+        if (i1 - i3) % 2 or (i2 - i4) % 2:
+            continue
+        if 0 <= h < 4 and 0 <= w < 4:
+            ref[c] = x[i0, h, w, i5]
+    assert np.array_equal(y, ref)
+
+
+def test_reindex_nested_extras():
+    # test/test_reindex_op.py:297-303 shape of expression: "@e0(0)", "@e1(0,i0 / @e0(0))"
+    a = rng.random((10, 10)).astype(np.float32)
+    b = np.array([2], np.int32)
+    e1 = rng.integers(0, 10, (10, 10)).astype(np.float32)
+    y = O.reindex(a, [8, 8], ["@e0(0)", "@e1(0,i0 / @e0(0))"], extras=[b, e1])
+    ref = np.zeros((8, 8), np.float32)
+    for i0 in range(8):
+        for i1 in range(8):
+            ref[i0, i1] = a[2, int(e1[0, i0 // 2])]
+    assert np.array_equal(y, ref)
+
+
+def test_reindex_errors():
+    a = np.zeros((10, 10), np.float32)
+    with pytest.raises(ValueError):
+        O.reindex(a, [8, 8], ["@e0(0) // 1", "@e0(0)"], extras=[np.array([1]), np.array([1])])
+    with pytest.raises(ValueError):
+        O.reindex(a, [8, 8], ["i0"])
+
+
+# ---- reindex_reduce ------------------------------------------------------------------
+@pytest.mark.parametrize("op", ["maximum", "minimum", "multiply", "add"])
+def test_reindex_reduce_pooling_brute_force(op):
+    N, H, W, C, size = 2, 7, 7, 3, 3
+    x = rng.random((N, H, W, C)).astype(np.float32)
+    h, w = (H + size - 1) // size, (W + size - 1) // size
+    y = O.reindex_reduce(x, op, [N, h, w, C], ["i0", "i1/%d" % size, "i2/%d" % size, "i3"])
+    init = {"maximum": -1e100, "minimum": 1e100, "multiply": 1.0, "add": 0.0}[op]
+    f = {"maximum": max, "minimum": min, "multiply": lambda a, b: a * b, "add": lambda a, b: a + b}[op]
+    ref = np.full((N, h, w, C), init)
+    for i0, i1, i2, i3 in np.ndindex(N, H, W, C):
+        ref[i0, i1 // size, i2 // size, i3] = f(ref[i0, i1 // size, i2 // size, i3], float(x[i0, i1, i2, i3]))
+    assert np.allclose(y, ref)
+
+
+def test_reindex_reduce_histogram_closed_forms():
+    n, bins = 5000, 37
+    v = rng.random(n).astype(np.float32)
+    idx = rng.integers(0, bins + 5, n).astype(np.int32) - 2      # some out of range on both sides
+    ok = (idx >= 0) & (idx < bins)
+    add = O.reindex_reduce(v, "add", [bins], ["@e0(i0)"], extras=[idx])
+    assert np.allclose(add, np.bincount(idx[ok], weights=v[ok].astype(np.float64), minlength=bins), rtol=1e-5)
+    mx = O.reindex_reduce(v, "maximum", [bins + 8], ["@e0(i0)"], extras=[idx])
+    ok8 = (idx >= 0) & (idx < bins + 8)
+    ref = np.full(bins + 8, np.finfo(np.float32).min, np.float32)
+    np.maximum.at(ref, idx[ok8], v[ok8])
+    assert np.array_equal(mx, ref)
+    assert (mx[bins + 3:] == np.finfo(np.float32).min).all()      # empty bins keep lowest(), not -inf
+    # invariants: total mass, permutation invariance (integers: exact)
+    vi = rng.integers(0, 100, n).astype(np.int32)
+    a1 = O.reindex_reduce(vi, "add", [bins], ["@e0(i0)"], extras=[idx])
+    p = rng.permutation(n)
+    a2 = O.reindex_reduce(vi[p], "add", [bins], ["@e0(i0)"], extras=[idx[p]])
+    assert np.array_equal(a1, a2) and a1.sum() == vi[ok].sum()
+
+
+def test_reindex_reduce_errors():
+    v = np.zeros(3, np.float32)
+    O.reindex_reduce(v, "add", [3], ["i0"])
+    for bad in (lambda: O.reindex_reduce(v, "add", [3], []),
+                lambda: O.reindex_reduce(v, "add", [3], ["i0", "i0"]),
+                lambda: O.reindex_reduce(v, "???", [3], ["i0"]),
+                lambda: O.reindex_reduce(v, "add", [-1], ["i0"])):
+        with pytest.raises(ValueError):
+            bad()
+
+
+# ---- reduce ---------------------------------------------------------------------------
+@pytest.mark.parametrize("keepdims", [False, True])
+def test_reduce_integer_exact(keepdims):
+    # test/test_reduce_op.py:12-50: arange data, 10 ops x 10 dim sets, exact
+    a = np.arange(2 * 3 * 4 * 5).reshape(2, 3, 4, 5).astype(np.int32)
+    ops = {"add": np.add, "multiply": np.multiply, "maximum": np.maximum, "minimum": np.minimum,
+           "logical_and": np.logical_and, "logical_or": np.logical_or, "logical_xor": np.logical_xor,
+           "bitwise_and": np.bitwise_and, "bitwise_or": np.bitwise_or, "bitwise_xor": np.bitwise_xor}
+    for dims in [(), (0,), (1,), (2,), (3,), (0, 2), (1, 3), (1, 2, 3), 2, 3]:
+        nd = tuple(range(4)) if dims == () else dims
+        for name, uf in ops.items():
+            ref = uf.reduce(a, nd, keepdims=keepdims)
+            ref = np.array([ref]) if ref.ndim == 0 else ref
+            got = O.reduce(a, name, dims, keepdims)
+            assert got.shape == ref.shape and (got == ref.astype(np.int32)).all(), (name, dims)
+
+
+def test_reduce_float_and_mean():
+    x = rng.uniform(-1, 1, (64, 33, 5)).astype(np.float32)
+    for dims in [(1,), (0, 2), ()]:
+        nd = tuple(range(3)) if dims == () else dims
+        ref = x.astype(np.float64).sum(nd)
+        assert np.allclose(O.reduce(x, "add", dims).reshape(-1), np.reshape(ref, -1), rtol=1e-5, atol=1e-4)
+        refm = x.astype(np.float64).mean(nd)
+        assert np.allclose(O.reduce(x, "mean", dims).reshape(-1), np.reshape(refm, -1), rtol=1e-4, atol=1e-5)
+    assert O.reduce(np.zeros((3, 0), np.float32), "maximum", 1).tolist() == [np.finfo(np.float32).min] * 3
+    with pytest.raises(ValueError):
+        O.reduce(np.array([1, 2, 3]), "add", 2)
+
+
+# ---- element-wise -------------------------------------------------------------------------
+def test_unary_closed_forms():
+    x = rng.uniform(0.1, 3, 257).astype(np.float32)
+    for op, f in [("log", np.log), ("exp", np.exp), ("sqrt", np.sqrt), ("sin", np.sin), ("tanh", np.tanh),
+                  ("atan", np.arctan), ("erf", special.erf), ("floor", np.floor), ("ceil", np.ceil),
+                  ("abs", np.abs), ("negative", np.negative)]:
+        assert np.allclose(O.unary(x, op), f(x.astype(np.float64)), rtol=2e-6), op
+    y = rng.uniform(-0.99, 0.99, 200).astype(np.float32)
+    assert np.allclose(O.unary(y, "erfinv"), special.erfinv(y.astype(np.float64)), rtol=1e-5, atol=1e-6)
+    # std::round is half away from zero (numpy rounds half to even)
+    assert O.unary(np.array([0.5, 1.5, 2.5, -0.5, -2.5], np.float32), "round").tolist() == [1, 2, 3, -1, -3]
+    assert O.unary(np.array([2.5, -2.5], np.float32), "round_int").dtype == np.int32
+    # test/test_unary_op.py:68-73: no NaN for large |x|; clamp makes sigmoid(-150) = 1/(1+e^30)
+    s = O.unary(np.arange(-150, 150, 10).astype(np.float32), "sigmoid")
+    assert not np.isnan(s).any() and np.isclose(s[0], 1 / (1 + np.exp(30.0)), rtol=1e-6) and s[-1] == 1.0
+    assert O.unary(np.array([1.7, -1.7], np.float32), "int32").tolist() == [1, -1]      # cast truncates
+    assert O.unary(np.array([0.0, 0.3], np.float32), "bool").tolist() == [False, True]
+    assert O.unary(np.array([1, 2], np.int32), "sqrt").dtype == np.float32
+
+
+def test_binary_rules():
+    a = np.array([7, -7, 7, -7], np.int32)
+    b = np.array([2, 2, -2, -2], np.int32)
+    assert O.binary(a, b, "floor_divide").tolist() == [3, -3, -3, 3]        # C division, not floor
+    assert O.binary(a, b, "mod").tolist() == [1, -1, 1, -1]                  # C remainder
+    af, bf = a.astype(np.float32), b.astype(np.float32)
+    assert O.binary(af, bf, "mod").tolist() == [1.0, 1.0, -1.0, -1.0]        # x - floor(x/y)*y
+    assert O.binary(a, b, "divide").dtype == np.float32
+    assert np.allclose(O.binary(a, b, "divide"), a / b)
+    assert O.binary(a, b, "less").dtype == np.bool_
+    t, f = np.array([True, True, False]), np.array([True, False, False])
+    assert O.binary(t, f, "add").tolist() == [True, True, False]             # bool arithmetic stays bool
+    assert O.binary(t, f, "subtract").tolist() == [False, True, False]
+    assert O.binary(t, f, "multiply").tolist() == [True, False, False]
+    x = rng.uniform(0.5, 2, 64).astype(np.float32)
+    y = rng.uniform(-2, 2, 64).astype(np.float32)
+    assert np.allclose(O.binary(x, y, "pow"), np.power(x.astype(np.float64), y), rtol=1e-6)
+    assert np.array_equal(O.binary(x, y, "maximum"), np.maximum(x, y))
+    assert np.array_equal(O.ternary(x > 1, x, y), np.where(x > 1, x, y))
+    # relu = ternary(x > 0, x, 0): NaN -> 0 (python/jittor/nn.py:182-183)
+    z = np.array([np.nan, -1, 2], np.float32)
+    assert O.ternary(O.binary(z, np.float32([0]), "greater"), z, np.zeros(3, np.float32)).tolist() == [0, 0, 2]
+
+
+def test_bf16_truncation():
+    f = np.array([1.0, 1.00390625, 1.0078125, -3.1415926], np.float32)
+    bits = O.f32_to_bf16_bits(f)
+    back = O.BF16(bits).to_f32()
+    assert back[0] == 1.0 and back[1] == 1.0 and back[2] == 1.0078125          # 1+2^-8 truncates down
+    assert abs(back[3]) <= abs(f[3])                                          # toward zero
+    assert O.c_cast(f, "bfloat16").bits.tolist() == bits.tolist()
+
+
+# ---- convolution -----------------------------------------------------------------------------
+def _conv_f64(x, w, stride, pad, dil):
+    N, C, H, W = x.shape
+    K, _, R, S = w.shape
+    oh = (H + 2 * pad - dil * (R - 1) - 1) // stride + 1
+    ow = (W + 2 * pad - dil * (S - 1) - 1) // stride + 1
+    xp = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+    y = np.zeros((N, K, oh, ow))
+    for r in range(R):
+        for s in range(S):
+            patch = xp[:, :, r * dil:r * dil + (oh - 1) * stride + 1:stride, s * dil:s * dil + (ow - 1) * stride + 1:stride]
+            y += np.einsum("nchw,kc->nkhw", patch, w[:, :, r, s].astype(np.float64))
+    return y
+
+
+@pytest.mark.parametrize("stride,pad,dil", [(1, 1, 1), (2, 1, 1), (1, 2, 2), (1, 0, 1)])
+def test_conv_meta_vs_float64(stride, pad, dil):
+    x = rng.standard_normal((2, 3, 9, 8)).astype(np.float32)
+    w = rng.standard_normal((4, 3, 3, 3)).astype(np.float32)
+    y = O.conv_meta(x, w, stride, pad, dil)
+    assert np.allclose(y, _conv_f64(x, w, stride, pad, dil), rtol=1e-5, atol=1e-5)
+
+
+def test_conv_meta_one_hot_kernel_is_a_shift():
+    x = O.BF16(O.f32_to_bf16_bits(rng.standard_normal((1, 2, 6, 6)).astype(np.float32)))
+    w = np.zeros((2, 2, 3, 3), np.float32)
+    w[0, 0, 0, 2] = 1.0       # y[0,0,h,w] = x[0,0,h-1,w+1]
+    w[1, 1, 1, 1] = 1.0       # identity on channel 1
+    y = O.conv_meta(x, O.BF16(O.f32_to_bf16_bits(w)), 1, 1, 1)
+    xf = x.to_f32()
+    ref0 = np.zeros((6, 6), np.float32)
+    ref0[1:, :5] = xf[0, 0, :5, 1:]
+    assert np.array_equal(y[0, 0], ref0) and np.array_equal(y[0, 1], xf[0, 1])
