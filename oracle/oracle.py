@@ -212,7 +212,7 @@ def _c_mod(a, b):
 def _round_half_away(a):
     """std::round."""
     r = np.trunc(a)
-    return r + np.where(np.abs(a - r) >= 0.5, np.sign(a), 0).astype(a.dtype)
+    return np.copysign(r + np.where(np.abs(a - r) >= 0.5, np.sign(a), 0).astype(a.dtype), a)
 
 
 # --------------------------------------------------------------------------
@@ -499,7 +499,7 @@ def reduce(x, op, dims=(), keepdims=False):
         if op in ("add", "mean"):
             v = m.astype(T)
             if op == "mean":
-                v = v * T(K * 1.0 / (K * R))          # Ty(x) * Ty(rcount)
+                v = v * T(np.float64(K) / np.float64(K * R))          # Ty(x) * Ty(rcount); rcount = y.num*1.0/x.num
             acc = np.cumsum(np.concatenate([init, v], 1), axis=1, dtype=T)[:, -1]
         elif op == "multiply":
             acc = np.cumprod(np.concatenate([init, m.astype(T)], 1), axis=1, dtype=T)[:, -1]

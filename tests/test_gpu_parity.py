@@ -301,6 +301,8 @@ def test_binary_ops(gpu, op):
     else:
         xf, yf = rng.uniform(0.5, 4, 515).astype(np.float32), rng.uniform(-3, 3, 515).astype(np.float32)
         yf[np.abs(yf) < 0.1] = 1.0
+        if op == "floor_divide":
+            yf[np.abs(yf) < 1] = 1.5          # int(y) == 0 would be an integer division by zero (undefined in C)
         xi, yi = rng.integers(-20, 20, 515).astype(np.int32), rng.integers(1, 7, 515).astype(np.int32) * rng.choice([-1, 1], 515).astype(np.int32)
         pairs = [(xf, yf), (xi, yi)] if op != "pow" else [(xf, yf)]
         if op in ("add", "multiply", "maximum", "less"):

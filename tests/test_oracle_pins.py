@@ -225,6 +225,7 @@ def test_unary_closed_forms():
     # std::round is half away from zero (numpy rounds half to even)
     assert O.unary(np.array([0.5, 1.5, 2.5, -0.5, -2.5], np.float32), "round").tolist() == [1, 2, 3, -1, -3]
     assert O.unary(np.array([2.5, -2.5], np.float32), "round_int").dtype == np.int32
+    assert np.signbit(O.unary(np.array([-0.3, -0.0], np.float32), "round")).all()      # C: round(-0.3) is -0.0
     # test/test_unary_op.py:68-73: no NaN for large |x|; clamp makes sigmoid(-150) = 1/(1+e^30)
     s = O.unary(np.arange(-150, 150, 10).astype(np.float32), "sigmoid")
     assert not np.isnan(s).any() and np.isclose(s[0], 1 / (1 + np.exp(30.0)), rtol=1e-6) and s[-1] == 1.0
