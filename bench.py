@@ -1,0 +1,330 @@
+#!/usr/bin/env python3
+"""Benchmark of the meta-operator path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only C2]
+
+A step is one pass of one workload's hot path (one C-ABI call = one kernel, or
+a fill + kernel pair for the scatter) over synthetic input that is already
+resident in HBM.  The headline line is BASELINE.json's configs[1] (C2, the
+im2col reindex); the other configurations are reported inside the same JSON
+line under "workloads".  Each workload rotates over several buffer sets whose
+total size exceeds the 256 MB memory-side cache, so the rates are HBM rates.
+
+For every workload the line carries
+  roofline     algorithmic bytes (or flops) per launch / average launch time,
+               timed with HIP events on the library's stream, against the
+               published peak (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s)
+  cpu_baseline the CPU restatement of the reference's kernel
+               (oracle/oracle_kernels.cc) timed on this box's host cores.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+CACHE_BYTES = 256 << 20
+
+
+def zipf_indices(n, bins, seed=1):
+    w = np.arange(1, bins + 1, dtype=np.float64) ** -1.1
+    cdf = np.cumsum(w) / w.sum()
+    return np.minimum(np.searchsorted(cdf, np.random.default_rng(seed).random(n)), bins - 1).astype(np.int32)
+
+
+class Dev:
+    """Plain device buffers for the timed loops (no front-end objects)."""
+
+    def __init__(self, L):
+        self.L = L
+        self.ptrs = []
+
+    def put(self, arr):
+        p = self.L.alloc(max(arr.nbytes, 256))
+        self.L.h2d(p, arr)
+        self.ptrs.append(p)
+        return p
+
+    def empty(self, nbytes):
+        p = self.L.alloc(nbytes)
+        self.ptrs.append(p)
+        return p
+
+    def release(self):
+        for p in self.ptrs:
+            self.L.free(p)
+        self.ptrs = []
+
+
+def time_calls(L, calls, steps, warmup):
+    """calls: list of zero-argument launch functions used round-robin.
+    Returns (average device ms per step, wall ms per step)."""
+    n = len(calls)
+    for i in range(warmup):
+        calls[i % n]()
+    L.sync()
+    e0, e1 = L.Event(), L.Event()
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        calls[i % n]()
+    e1.record()
+    L.sync()
+    t1 = time.perf_counter()
+    return e1.elapsed_ms_since(e0) / steps, (t1 - t0) * 1e3 / steps
+
+
+def roofline(bound, work, ms, traffic=None):
+    if bound == "hbm":
+        achieved = work / (ms * 1e-3) / 1e9
+        return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic}
+    achieved = work / (ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic}
+
+
+def cpu_time(fn, repeat=3):
+    fn()
+    ts = []
+    for _ in range(repeat):
+        t = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t)
+    return float(np.median(ts))
+
+
+# ---- workloads -----------------------------------------------------------------
+def wl_c1(L, lib, steps, warmup, with_cpu):
+    from oracle import kernels as K
+    shape = (8192, 4096)
+    work = 134250496
+    sets = max(2, CACHE_BYTES * 2 // (shape[0] * shape[1] * 4) + 1)
+    dev = Dev(L)
+    x = np.random.default_rng(0).uniform(-1, 1, shape).astype(np.float32)
+    calls = []
+    for s in range(sets):
+        tx = L.tensor(dev.put(x), "float32", shape)
+        ty = L.tensor(dev.empty(shape[0] * 4), "float32", [shape[0]])
+        calls.append(lambda tx=tx, ty=ty: L.check(lib.mjt_reduce(ctypes.byref(tx), ctypes.byref(ty), L.OP_CODE["add"], 0b10)))
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out = {"workload": "C1 ReduceOp sum axis 1, fp32 [8192,4096]", "kernel": L.last_kernel(), "dtype": "f32",
+           "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5), "roofline": roofline("hbm", work, ms)}
+    dev.release()
+    if with_cpu:
+        t1 = cpu_time(lambda: K.reduce_sum_axis1(x, 1))
+        nt = K.max_threads()
+        tn = cpu_time(lambda: K.reduce_sum_axis1(x, nt))
+        out["cpu_baseline"] = {"value": round(work / t1 / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": "full C1 input, median of 3", "all_cores": {"value": round(work / tn / 1e9, 2), "cores": nt}}
+    return out
+
+
+def wl_c2(L, lib, steps, warmup, with_cpu):
+    from oracle import kernels as K
+    xs, ys = (32, 64, 56, 56), (32, 64, 56, 56, 3, 3)
+    work = 256901120
+    dev = Dev(L)
+    x = np.random.default_rng(0).standard_normal(xs).astype(np.float32)
+    idx, e = L.c_strings(["i0", "i1", "i2+i4-1", "i3+i5-1"]), L.c_strings([])
+    calls = []
+    for s in range(3):
+        tx = L.tensor(dev.put(x), "float32", xs)
+        ty = L.tensor(dev.empty(int(np.prod(ys)) * 4), "float32", ys)
+        calls.append(lambda tx=tx, ty=ty: L.check(lib.mjt_reindex(ctypes.byref(tx), ctypes.byref(ty), 4, idx, 0.0, 0, e, 0, None)))
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out = {"workload": "C2 ReindexOp im2col gather, fp32 [32,64,56,56] -> [32,64,56,56,3,3], 3x3 stride 1 pad 1",
+           "kernel": L.last_kernel(), "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+           "roofline": roofline("hbm", work, ms)}
+    dev.release()
+    if with_cpu:
+        buf = np.empty(ys, np.float32)
+        t1 = cpu_time(lambda: K.reindex_im2col3x3(x, 1, buf))
+        nt = K.max_threads()
+        tn = cpu_time(lambda: K.reindex_im2col3x3(x, nt, buf))
+        out["cpu_baseline"] = {"value": round(work / t1 / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": "full C2 input, median of 3", "all_cores": {"value": round(work / tn / 1e9, 2), "cores": nt}}
+    return out
+
+
+def wl_c3(L, lib, steps, warmup, with_cpu, op):
+    from oracle import kernels as K
+    n, bins = 1 << 24, 1 << 20
+    work = 138412032
+    dev = Dev(L)
+    v = np.random.default_rng(0).random(n, dtype=np.float32)
+    idx = zipf_indices(n, bins)
+    s1, e = L.c_strings(["@e0(i0)"]), L.c_strings([])
+    calls = []
+    for s in range(4):
+        tv = L.tensor(dev.put(v), "float32", [n])
+        ti = (L.Tensor * 1)(L.tensor(dev.put(idx), "int32", [n]))
+        tx = L.tensor(dev.empty(bins * 4), "float32", [bins])
+        calls.append(lambda tv=tv, ti=ti, tx=tx: L.check(lib.mjt_reindex_reduce(
+            ctypes.byref(tv), ctypes.byref(tx), L.OP_CODE[op], 1, s1, 0, e, 1, ti)))
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out = {"workload": "C3 ReindexReduceOp scatter-%s, 2^24 fp32 values into 2^20 bins, int32 Zipf(1.1) indices" % op,
+           "kernel": L.last_kernel(), "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+           "roofline": roofline("hbm", work, ms),
+           "note": "a step = identity fill of the bins + window sampling pass + scatter kernel"}
+    dev.release()
+    if with_cpu:
+        t1 = cpu_time(lambda: K.scatter_1d(v, idx, bins, op))
+        out["cpu_baseline"] = {"value": round(work / t1 / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": "full C3 input, median of 3 (the update loop is sequential in the reference)"}
+    return out
+
+
+def c4_desc(L, shape, xp, sp, bp, zp):
+    """FusedOp descriptor of exp(-relu(x*scale+bias)) * sigmoid(x) exactly as the
+    front end builds it (two broadcasts of the inputs, relu's 0.0 scalar)."""
+    V, F = L.FusedVar, L.FusedOp
+    spec = [(0, "float32", xp, 0), (0, "float32", sp, 0b101), (0, "float32", bp, 0b011), (3, "float32", None, 0),
+            (1, "float32", None, 0), (1, "float32", None, 0), (1, "float32", None, 0), (1, "float32", None, 0),
+            (1, "bool", None, 0), (1, "float32", None, 0), (1, "float32", None, 0), (1, "float32", None, 0),
+            (1, "float32", None, 0), (1, "float32", None, 0), (2, "float32", zp, 0)]
+    va = (V * len(spec))()
+    for i, (role, dt_, ptr, mask) in enumerate(spec):
+        va[i].role, va[i].dtype, va[i].ptr, va[i].bcast_mask = role, L.DTYPE_CODE[dt_], ptr, mask
+    ops = [(3, None, [1], 4), (1, "multiply", [0, 4], 5), (3, None, [2], 6), (1, "add", [5, 6], 7), (3, None, [3], 9),
+           (1, "greater", [7, 9], 8), (2, None, [8, 7, 9], 10), (0, "negative", [10], 11), (0, "exp", [11], 12),
+           (0, "sigmoid", [0], 13), (1, "multiply", [12, 13], 14)]
+    oa = (F * len(ops))()
+    for i, (kind, op, ins, out) in enumerate(ops):
+        oa[i].kind, oa[i].op, oa[i].out = kind, L.OP_CODE[op] if op else 0, out
+        for j, u in enumerate(ins):
+            oa[i].inp[j] = u
+    d = L.FusedDesc()
+    d.ndim = 3
+    for i, s in enumerate(shape):
+        d.shape[i] = s
+    d.n_vars, d.vars, d.n_ops, d.ops = len(spec), va, len(ops), oa
+    return d, (va, oa)
+
+
+def wl_c4(L, lib, steps, warmup, with_cpu):
+    from oracle import kernels as K
+    shape = (64, 512, 1024)
+    work = 268441600
+    dev = Dev(L)
+    x = np.random.default_rng(0).standard_normal(shape).astype(np.float32)
+    sc = np.random.default_rng(1).standard_normal((512, 1)).astype(np.float32)
+    bi = np.random.default_rng(2).standard_normal((1, 1024)).astype(np.float32)
+    sp, bp = dev.put(sc), dev.put(bi)
+    calls, keep = [], []
+    for s in range(3):
+        d, k = c4_desc(L, shape, dev.put(x), sp, bp, dev.empty(x.nbytes))
+        keep.append((d, k))
+        calls.append(lambda d=d: L.check(lib.mjt_fused_elementwise(ctypes.byref(d))))
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out = {"workload": "C4 fused exp(-relu(x*scale+bias))*sigmoid(x), x fp32 [64,512,1024], scale [512,1], bias [1,1024]",
+           "kernel": L.last_kernel(), "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+           "roofline": roofline("hbm", work, ms)}
+    dev.release()
+    if with_cpu:
+        sub = x[:8]                                    # 1/8 of the batch axis, scaled
+        buf = np.empty_like(sub)
+        t1 = cpu_time(lambda: K.fused_chain(sub, sc, bi, 1, buf)) * 8
+        nt = K.max_threads()
+        buf2 = np.empty_like(x)
+        tn = cpu_time(lambda: K.fused_chain(x, sc, bi, nt, buf2))
+        out["cpu_baseline"] = {"value": round(work / t1 / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": "x[:8] of 64 (1/8 of the elements), time scaled by 8, median of 3",
+                               "all_cores": {"value": round(work / tn / 1e9, 2), "cores": nt, "sample": "full C4 input"}}
+    return out
+
+
+def wl_c5(L, lib, steps, warmup, with_cpu):
+    from oracle import kernels as K
+    from jittor_amd.dtypes import f32_to_bf16_bits
+    xs, ws, ys = (64, 256, 56, 56), (256, 256, 3, 3), (64, 256, 56, 56)
+    flops = 236760072192
+    dev = Dev(L)
+    xb = f32_to_bf16_bits(np.random.default_rng(0).standard_normal(xs).astype(np.float32))
+    wb = f32_to_bf16_bits((np.random.default_rng(1).standard_normal(ws) * np.sqrt(2.0 / (256 * 9))).astype(np.float32))
+    p = L.ConvParams(1, 1, 1, 1, 1, 1)
+    calls = []
+    tw = L.tensor(dev.put(wb), "bfloat16", ws)
+    for s in range(2):
+        tx = L.tensor(dev.put(xb), "bfloat16", xs)
+        ty = L.tensor(dev.empty(int(np.prod(ys)) * 4), "float32", ys)
+        calls.append(lambda tx=tx, ty=ty: L.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p))))
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out = {"workload": "C5 meta-op conv, x bf16 [64,256,56,56], w bf16 [256,256,3,3], 3x3 s1 p1, fp32 accumulate and output",
+           "kernel": L.last_kernel(), "dtype": "bf16", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+           "roofline": roofline("mfma", flops, ms), "note": "a step = weight repack + convolution kernel"}
+    dev.release()
+    if with_cpu:
+        nt = K.max_threads()
+        sub = xb[:1, :, :14, :]                      # one image, 14 of 56 rows: 1/256 of the MACs (edge rows differ slightly)
+        t0 = time.perf_counter()
+        K.conv_meta_bf16(sub, wb, 1, 1, 1, nt)
+        tn = time.perf_counter() - t0
+        sub_flops = 2.0 * 1 * 256 * 14 * 56 * 256 * 9
+        out["cpu_baseline"] = {"value": round(sub_flops / tn / 1e12, 5), "unit": "TFLOP/s", "cores": nt, "kind": "port",
+                               "sample": "x[:1,:,:14,:] (1 image, 14 rows), all cores, one run"}
+    return out
+
+
+WORKLOADS = {
+    "C1": wl_c1,
+    "C2": wl_c2,
+    "C3add": lambda *a: wl_c3(*a, op="add"),
+    "C3max": lambda *a: wl_c3(*a, op="maximum"),
+    "C4": wl_c4,
+    "C5": wl_c5,
+}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", default="", help="comma-separated subset of " + ",".join(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (every box of this run has one GPU); "
+              "got --gpus %d" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    from jittor_amd import _lib as L
+    lib = L.init(0)
+    di = L.device_info()
+    only = [s for s in args.only.split(",") if s] or list(WORKLOADS)
+    results = {}
+    for name in only:
+        try:
+            results[name] = WORKLOADS[name](L, lib, args.steps, args.warmup, not args.no_cpu)
+        except L.MjtError as err:
+            results[name] = {"error": str(err)}
+        print("[bench] %s: %s" % (name, json.dumps(results[name])), file=sys.stderr, flush=True)
+    head = results.get("C2") or next(iter(results.values()))
+    line = {
+        "metric": "achieved HBM GB/s (% peak) for reduce/reindex/fused ops; conv TFLOP/s",
+        "value": head.get("roofline", {}).get("achieved"),
+        "unit": head.get("roofline", {}).get("unit", "GB/s"),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head.get("ms_per_step"),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": head.get("dtype", "f32"), "data": "synthetic",
+        "config": {"workload": head.get("workload"), "buffer_sets": "rotating, > 256 MB in total"},
+        "roofline": head.get("roofline"),
+        "cpu_baseline": head.get("cpu_baseline"),
+        "device": {"arch": di.arch.decode(), "compute_units": di.compute_units, "clock_khz": di.clock_khz,
+                   "mem_clock_khz": di.mem_clock_khz, "mem_bus_bits": di.mem_bus_bits},
+        "workloads": results,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
