@@ -19,10 +19,10 @@
 // 256*VEC-element runs, which keeps UNROLL independent loads in flight per
 // lane.
 
-struct Params { unsigned long long a[NPARAM]; };
+struct Params { void* a[NPARAM]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
 
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
-    const index_t nvec = (index_t)p.a[0];
+    const index_t nvec = (index_t)(unsigned long long)p.a[0];
     MJT_FUSED_SCALARS
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {

@@ -22,16 +22,16 @@
 // When SPLIT is set the partials go to a scratch buffer and a second launch of
 // the same kernel family folds them (two-pass grid reduce).
 
-struct Params { unsigned long long a[8 + 6 * 5]; };
+struct Params { void* a[8 + 6 * 5]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
 // a[0] x, a[1] y or partials, a[2] O (outputs), a[3] S (splits), a[4] rcount (double bits),
 // a[5] work items per split, a[6] total work items,
 // a[8+0*5..]  kshape   a[8+1*5..] kstride (in x)   a[8+2*5..] kdiv
 // a[8+3*5..]  rshape   a[8+4*5..] rstride (in x)   a[8+5*5..] rdiv
 
 #if USE64
-#define MJT_DIVQ(n, k, tab) ((n) / (index_t)p.a[8 + ((tab)-2) * 5 + (k)])
+#define MJT_DIVQ(n, k, tab) ((n) / (index_t)(unsigned long long)p.a[8 + ((tab)-2) * 5 + (k)])
 #else
-#define MJT_DIVQ(n, k, tab) ((index_t)mjt_div((unsigned)(n), mjt_unpack_divmod(p.a[8 + (tab) * 5 + (k)], 0)))
+#define MJT_DIVQ(n, k, tab) ((index_t)mjt_div((unsigned)(n), mjt_unpack_divmod((unsigned long long)p.a[8 + (tab) * 5 + (k)], 0)))
 #endif
 
 template <class T> __device__ __forceinline__ T mjt_shfl_xor_any(T v, int off) {
@@ -54,10 +54,10 @@ __device__ __forceinline__ index_t mjt_kept_offset(const Params& p, index_t o) {
     index_t off = 0;
 #pragma unroll
     for (int k = NK - 1; k >= 0; k--) {
-        index_t shape = (index_t)p.a[8 + 0 * 5 + k];
+        index_t shape = (index_t)(unsigned long long)p.a[8 + 0 * 5 + k];
         index_t q = (k == 0) ? 0 : MJT_DIVQ(o, k, 2);
         index_t c = (k == 0) ? o : o - q * shape;
-        off += c * (index_t)p.a[8 + 1 * 5 + k];
+        off += c * (index_t)(unsigned long long)p.a[8 + 1 * 5 + k];
         o = q;
     }
     return off;
@@ -68,10 +68,10 @@ template <int ND> __device__ __forceinline__ index_t mjt_red_offset(const Params
     index_t off = 0;
 #pragma unroll
     for (int k = ND - 1; k >= 0; k--) {
-        index_t shape = (index_t)p.a[8 + 3 * 5 + k];
+        index_t shape = (index_t)(unsigned long long)p.a[8 + 3 * 5 + k];
         index_t q = (k == 0) ? 0 : MJT_DIVQ(r, k, 5);
         index_t c = (k == 0) ? r : r - q * shape;
-        off += c * (index_t)p.a[8 + 4 * 5 + k];
+        off += c * (index_t)(unsigned long long)p.a[8 + 4 * 5 + k];
         r = q;
     }
     return off;
@@ -81,9 +81,9 @@ template <int ND> __device__ __forceinline__ index_t mjt_red_offset(const Params
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const TX* __restrict__ xp = (const TX*)p.a[0];
     TY* __restrict__ yp = (TY*)p.a[1];
-    const index_t O = (index_t)p.a[2];
-    const index_t S = (index_t)p.a[3];
-    const TY rcount = (TY)__longlong_as_double((long long)p.a[4]);
+    const index_t O = (index_t)(unsigned long long)p.a[2];
+    const index_t S = (index_t)(unsigned long long)p.a[3];
+    const TY rcount = (TY)__longlong_as_double((long long)(unsigned long long)p.a[4]);
     (void)rcount;
     const unsigned lane = threadIdx.x % G;
     const index_t o = (index_t)blockIdx.x * (256 / G) + threadIdx.x / G;
@@ -93,10 +93,10 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     for (int k = 0; k < VEC; k++) acc[k] = INIT;
     if (o < O) {
         const index_t kbase = mjt_kept_offset(p, o);
-        const index_t L = (index_t)p.a[8 + 3 * 5 + (NR - 1)];
+        const index_t L = (index_t)(unsigned long long)p.a[8 + 3 * 5 + (NR - 1)];
         const index_t nL = (L + (G * VEC) - 1) / (G * VEC);
-        const index_t per = (index_t)p.a[5];
-        const index_t total = (index_t)p.a[6];
+        const index_t per = (index_t)(unsigned long long)p.a[5];
+        const index_t total = (index_t)(unsigned long long)p.a[6];
         index_t it = s * per;
         index_t it_end = it + per < total ? it + per : total;
         index_t ro = (NR == 1) ? 0 : it / nL;
@@ -133,15 +133,15 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const TX* __restrict__ xp = (const TX*)p.a[0];
     TY* __restrict__ yp = (TY*)p.a[1];
-    const index_t O = (index_t)p.a[2];
-    const TY rcount = (TY)__longlong_as_double((long long)p.a[4]);
+    const index_t O = (index_t)(unsigned long long)p.a[2];
+    const TY rcount = (TY)__longlong_as_double((long long)(unsigned long long)p.a[4]);
     (void)rcount;
     const index_t o = ((index_t)blockIdx.x * 256 + threadIdx.x) * VEC;
     const index_t s = blockIdx.y;
     if (o >= O) return;
     const index_t kbase = mjt_kept_offset(p, o);
-    const index_t per = (index_t)p.a[5];
-    const index_t total = (index_t)p.a[6];
+    const index_t per = (index_t)(unsigned long long)p.a[5];
+    const index_t total = (index_t)(unsigned long long)p.a[6];
     index_t r = s * per;
     const index_t r_end = r + per < total ? r + per : total;
     TY acc[VEC];
@@ -150,7 +150,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const TX* __restrict__ col = xp + kbase;
 #pragma unroll 4
     for (; r < r_end; r++) {
-        index_t roff = (NR == 1) ? r * (index_t)p.a[8 + 4 * 5] : mjt_red_offset<NR>(p, r);
+        index_t roff = (NR == 1) ? r * (index_t)(unsigned long long)p.a[8 + 4 * 5] : mjt_red_offset<NR>(p, r);
         mjt_pack<TX, VEC> v;
         mjt_load(v, col + roff);
 #pragma unroll

@@ -17,7 +17,7 @@
 // lane owns VEC adjacent elements of y's innermost axis so that y moves as
 // one vector per lane; the x side is accessed element by element.
 
-struct Params { unsigned long long a[NPARAM]; };
+struct Params { void* a[NPARAM]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
 
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 #if SCATTER
@@ -26,9 +26,9 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 #else
     const TX* __restrict__ xp = (const TX*)p.a[0];
     TX* __restrict__ yp = (TX*)p.a[1];
-    const TX ovalue_ = (TX)__longlong_as_double((long long)p.a[3]);
+    const TX ovalue_ = (TX)__longlong_as_double((long long)(unsigned long long)p.a[3]);
 #endif
-    const index_t nvec = (index_t)p.a[2];
+    const index_t nvec = (index_t)(unsigned long long)p.a[2];
     MJT_RX_SETUP
     const index_t j = (index_t)blockIdx.x * 256 + threadIdx.x;
     if (j >= nvec) return;

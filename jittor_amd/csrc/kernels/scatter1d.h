@@ -15,7 +15,7 @@
 // read from device memory: a sampling pass picks the window that holds the
 // most updates.  x must hold the identity before this kernel runs.
 
-struct Params { unsigned long long a[8]; };
+struct Params { void* a[8]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
 // a[0] x, a[1] y, a[2] idx, a[3] n, a[4] bins, a[5] &lo (int), a[6] elements per workgroup
 
 #if MODE == 0
@@ -48,10 +48,10 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY(Params p) {
     TX* __restrict__ xp = (TX*)p.a[0];
     const TX* __restrict__ yp = (const TX*)p.a[1];
     const TE* __restrict__ ip = (const TE*)p.a[2];
-    const long long n = (long long)p.a[3];
-    const long long bins = (long long)p.a[4];
+    const long long n = (long long)(unsigned long long)p.a[3];
+    const long long bins = (long long)(unsigned long long)p.a[4];
     const long long lo = *(const int*)p.a[5];
-    const long long per = (long long)p.a[6];
+    const long long per = (long long)(unsigned long long)p.a[6];
     __shared__ TX win[WBINS];
     TX ident;
     {
@@ -99,8 +99,8 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY(Params p) {
 // bins; the start of the fullest window is written to *lo.
 extern "C" __global__ __launch_bounds__(1024) void ENTRY_SAMPLE(Params p) {
     const TE* __restrict__ ip = (const TE*)p.a[2];
-    const long long n = (long long)p.a[3];
-    const long long bins = (long long)p.a[4];
+    const long long n = (long long)(unsigned long long)p.a[3];
+    const long long bins = (long long)(unsigned long long)p.a[4];
     int* lo = (int*)p.a[5];
     __shared__ int votes[1024];
     __shared__ int best_votes, best_tile;

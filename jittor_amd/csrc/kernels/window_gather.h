@@ -15,12 +15,12 @@
 // vectors l, l+256, ... of that run and finds (row, ow, kh, kw) of each
 // element by constant division.
 
-struct Params { unsigned long long a[4]; };   // x, y, overflow bits, number of planes
+struct Params { void* a[4]; };   // 8-byte words; typed as pointers so loads/stores use the global address space   // x, y, overflow bits, number of planes
 
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const TB* __restrict__ xp = (const TB*)p.a[0];
     TB* __restrict__ yp = (TB*)p.a[1];
-    const TB ov = (TB)p.a[2];
+    const TB ov = (TB)(unsigned long long)p.a[2];
     __shared__ TB tile[LH * LW];
     constexpr int TILES = (OH + TH - 1) / TH;
     const unsigned plane = blockIdx.x / TILES;

@@ -1,4 +1,145 @@
+// mjt_conv2d_meta: host side of the meta-op convolution (the group
+// python/jittor/nn.py:1251-1262 builds; parameters as solved by
+// python/jittor/src/opt/tuner/conv_tuner.cc:312-356).
 #include "common.h"
+#include <mutex>
+#include <unordered_map>
+
+namespace mjt {
+
+namespace {
+std::mutex g_mu;
+std::unordered_map<std::string, JitKernel*> g_kernels;
+JitKernel* cached(const std::string& key) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_kernels.find(key);
+    return it == g_kernels.end() ? nullptr : it->second;
+}
+void remember(const std::string& key, JitKernel* k) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_kernels.emplace(key, k);
+}
+void* g_wpack = nullptr;
+size_t g_wpack_bytes = 0;
+}  // namespace
+
+void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p) {
+    require_init();
+    check_tensor(x, "conv x");
+    check_tensor(w, "conv w");
+    check_tensor(y, "conv y");
+    MJT_CHECK(p, "conv: null parameters");
+    MJT_CHECK(x->ndim == 4 && w->ndim == 4 && y->ndim == 4, "conv: x, w and y must have rank 4");
+    MJT_CHECK(x->dtype == w->dtype && (x->dtype == MJT_BFLOAT16 || x->dtype == MJT_FLOAT32),
+              "conv: x and w must both be bfloat16 or float32");
+    MJT_CHECK(y->dtype == MJT_FLOAT32 || y->dtype == x->dtype, "conv: y must be float32 or the input dtype");
+    const int64_t N = x->shape[0], C = x->shape[1], H = x->shape[2], W = x->shape[3];
+    const int64_t K = w->shape[0], R = w->shape[2], S = w->shape[3];
+    MJT_CHECK(w->shape[1] == C, "conv: weight channels " << w->shape[1] << " != input channels " << C);
+    MJT_CHECK(p->stride_h >= 1 && p->stride_w >= 1 && p->dil_h >= 1 && p->dil_w >= 1 && p->pad_h >= 0 && p->pad_w >= 0,
+              "conv: bad stride / padding / dilation");
+    const int64_t OH = (H + 2 * p->pad_h - p->dil_h * (R - 1) - 1) / p->stride_h + 1;
+    const int64_t OW = (W + 2 * p->pad_w - p->dil_w * (S - 1) - 1) / p->stride_w + 1;
+    MJT_CHECK(OH >= 1 && OW >= 1, "conv: empty output");
+    MJT_CHECK(y->shape[0] == N && y->shape[1] == K && y->shape[2] == OH && y->shape[3] == OW,
+              "conv: y shape " << shape_str(y) << " != [" << N << "," << K << "," << OH << "," << OW << "]");
+    if (N == 0 || K == 0) return;
+    MJT_CHECK(numel(x) < (int64_t(1) << 40) && numel(y) < (int64_t(1) << 40), "conv: too large");
+    Context& c = ctx();
+
+    std::ostringstream geo;
+    geo << "#define C_ " << C << "\n#define H_ " << H << "\n#define W_ " << W << "\n#define K_ " << K << "\n#define R_ " << R
+        << "\n#define S_ " << S << "\n#define OH_ " << OH << "\n#define OW_ " << OW << "\n#define SH " << p->stride_h
+        << "\n#define SW " << p->stride_w << "\n#define PH " << p->pad_h << "\n#define PW " << p->pad_w << "\n#define DH "
+        << p->dil_h << "\n#define DW " << p->dil_w << "\n";
+
+    // ---- MFMA path ----------------------------------------------------------------
+    int64_t TRW = OW <= 112 ? 112 / OW : 0;
+    if (TRW > OH) TRW = OH;
+    while (TRW > 1 && 2 * TRW > OH && (OH % (2 * TRW)) != 0 && (2 * (TRW - 1)) >= OH) TRW--;
+    const int64_t NT = TRW ? (TRW * OW + 15) / 16 : 0;
+    const int64_t LROWS = (2 * TRW - 1) * p->stride_h + (R - 1) * p->dil_h + 1;
+    const int64_t LCOLS = (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1 > W + 2 * p->pad_w
+                              ? (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1
+                              : W + 2 * p->pad_w;
+    const bool mfma_ok = x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 128 == 0 &&
+                         W % 8 == 0 && TRW >= 1 && NT <= 7 && LROWS * LCOLS * 128 <= 64 * 1024 &&
+                         (uintptr_t)x->ptr % 16 == 0 && R * S <= 49;
+    if (mfma_ok) {
+        const int64_t items = LROWS * (W / 8);
+        const int64_t items_per_wave = (items + 3) / 4;
+        std::ostringstream key;
+        key << "mfma|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16);
+        JitKernel* k = cached(key.str());
+        JitKernel* kp = cached(key.str() + "|pack");
+        if (!k || !kp) {
+            std::ostringstream name;
+            name << "mjt_conv_mfma_bf16_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s"
+                 << p->stride_h << "x" << p->stride_w << "_p" << p->pad_h << "x" << p->pad_w << "_d" << p->dil_h << "x"
+                 << p->dil_w << (y->dtype == MJT_BFLOAT16 ? "_obf16" : "_of32");
+            std::ostringstream src;
+            src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo.str()
+                << "#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
+                << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
+                << "\n";
+            src << embedded_source("conv_mfma.h") << "\n";
+            k = jit_get(src.str(), name.str());
+            kp = new JitKernel();
+            kp->name = name.str() + "_pack";
+            kp->module = k->module;
+            if (!c.dry_run) HIP_CHECK(hipModuleGetFunction(&kp->fn, k->module, kp->name.c_str()));
+            remember(key.str(), k);
+            remember(key.str() + "|pack", kp);
+        }
+        size_t wbytes = (size_t)numel(w) * 2;
+        if (!c.dry_run && wbytes > g_wpack_bytes) {
+            if (g_wpack) {
+                HIP_CHECK(hipStreamSynchronize(c.stream));
+                HIP_CHECK(hipFree(g_wpack));
+            }
+            HIP_CHECK(hipMalloc(&g_wpack, wbytes));
+            g_wpack_bytes = wbytes;
+        }
+        std::vector<uint64_t> pa{bits_of_ptr(w->ptr), bits_of_ptr(g_wpack), 0, 0};
+        int64_t pblocks = (numel(w) + 255) / 256;
+        if (pblocks > 2048) pblocks = 2048;
+        jit_launch(kp, (unsigned)pblocks, 1, 256, 0, pa);
+        const int64_t TR = 2 * TRW;
+        const int64_t tiles_r = (OH + TR - 1) / TR;
+        const int64_t ptiles = N * tiles_r;
+        const int64_t ptiles8 = (ptiles + 7) / 8 * 8;
+        const int64_t blocks = ptiles8 * (K / 128);
+        MJT_CHECK(blocks < (int64_t(1) << 31), "conv: launch too large");
+        std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(g_wpack), bits_of_ptr(y->ptr), (uint64_t)N};
+        jit_launch(k, (unsigned)blocks, 1, 256, 0, a);
+        return;
+    }
+
+    // ---- direct path ----------------------------------------------------------------
+    std::ostringstream key;
+    key << "direct|" << geo.str() << x->dtype << "|" << y->dtype;
+    JitKernel* k = cached(key.str());
+    if (!k) {
+        std::ostringstream name;
+        name << "mjt_conv_direct_" << mjt_dtype_name(x->dtype) << "_" << mjt_dtype_name(y->dtype) << "_c" << C << "_k" << K
+             << "_" << H << "x" << W << "_r" << R << "x" << S << "_s" << p->stride_h << "x" << p->stride_w << "_p" << p->pad_h
+             << "x" << p->pad_w << "_d" << p->dil_h << "x" << p->dil_w;
+        std::ostringstream src;
+        src << "#define ENTRY " << name.str() << "\n#define TIN " << dtype_cname(x->dtype) << "\n#define TOUT "
+            << dtype_cname(y->dtype) << "\n" << geo.str();
+        src << embedded_source("prelude.h") << "\n" << embedded_source("conv_direct.h") << "\n";
+        k = jit_get(src.str(), name.str());
+        remember(key.str(), k);
+    }
+    const int64_t total = numel(y);
+    const int64_t blocks = (total + 255) / 256;
+    MJT_CHECK(blocks < (int64_t(1) << 31), "conv: launch too large");
+    std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(w->ptr), bits_of_ptr(y->ptr), (uint64_t)total};
+    jit_launch(k, (unsigned)blocks, 1, 256, 0, a);
+}
+
+}  // namespace mjt
+
 extern "C" int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p) {
-    return mjt::guarded([&] { MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv2d_meta: not built yet"); });
+    return mjt::guarded([&] { mjt::conv_impl(x, w, y, p); });
 }

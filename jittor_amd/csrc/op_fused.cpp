@@ -189,10 +189,10 @@ void fused_impl(const mjt_fused_desc* d) {
             if (fv.role != MJT_VAR_SCALAR) continue;
             const char* T = dtype_cname(fv.dtype);
             if (dtype_is_float(fv.dtype))
-                scal << "const " << T << " " << vname(i) << " = (" << T << ")__longlong_as_double((long long)p.a["
+                scal << "const " << T << " " << vname(i) << " = (" << T << ")__longlong_as_double((long long)(unsigned long long)p.a["
                      << p_var[i] << "]); ";
             else
-                scal << "const " << T << " " << vname(i) << " = (" << T << ")(long long)p.a[" << p_var[i] << "]; ";
+                scal << "const " << T << " " << vname(i) << " = (" << T << ")(long long)(unsigned long long)p.a[" << p_var[i] << "]; ";
         }
         if (need_decode) {
             dec << IT << " rem_ = e; ";
@@ -200,12 +200,12 @@ void fused_impl(const mjt_fused_desc* d) {
                 if (a == 0) {
                     dec << "const " << IT << " c0 = rem_; ";
                 } else if (use64) {
-                    dec << "const " << IT << " q" << a << " = rem_ / (" << IT << ")p.a[" << p_dim[a] << "]; const " << IT
-                        << " c" << a << " = rem_ - q" << a << " * (" << IT << ")p.a[" << p_dim[a] << "]; rem_ = q" << a
+                    dec << "const " << IT << " q" << a << " = rem_ / (" << IT << ")(unsigned long long)p.a[" << p_dim[a] << "]; const " << IT
+                        << " c" << a << " = rem_ - q" << a << " * (" << IT << ")(unsigned long long)p.a[" << p_dim[a] << "]; rem_ = q" << a
                         << "; ";
                 } else {
-                    dec << "const int q" << a << " = (int)mjt_div((unsigned)rem_, mjt_unpack_divmod(p.a[" << p_dim[a] + 1
-                        << "], 0)); const int c" << a << " = rem_ - q" << a << " * (int)p.a[" << p_dim[a] << "]; rem_ = q"
+                    dec << "const int q" << a << " = (int)mjt_div((unsigned)rem_, mjt_unpack_divmod((unsigned long long)p.a[" << p_dim[a] + 1
+                        << "], 0)); const int c" << a << " = rem_ - q" << a << " * (int)(unsigned long long)p.a[" << p_dim[a] << "]; rem_ = q"
                         << a << "; ";
                 }
             }
@@ -218,7 +218,7 @@ void fused_impl(const mjt_fused_desc* d) {
                 off = "(";
                 for (int a = 0; a < nd; a++) {
                     if (dims[a].bcast[k]) continue;
-                    off += "c" + std::to_string(a) + " * (" + IT + ")p.a[" + std::to_string(p_stride[k][a]) + "] + ";
+                    off += "c" + std::to_string(a) + " * (" + IT + ")(unsigned long long)p.a[" + std::to_string(p_stride[k][a]) + "] + ";
                 }
                 off += "0)";
             }

@@ -133,7 +133,7 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
         setup << "const index_t XDIM = " << XD << "; const index_t YDIM = " << LD << "; (void)XDIM; (void)YDIM; ";
         auto shapes = [&](const char* n, int rank, int base) {
             for (int i = 0; i < rank; i++)
-                setup << "const index_t " << n << "shape" << i << " = (index_t)p.a[" << base + i << "]; (void)" << n
+                setup << "const index_t " << n << "shape" << i << " = (index_t)(unsigned long long)p.a[" << base + i << "]; (void)" << n
                       << "shape" << i << "; ";
             setup << "const index_t " << n << "stride" << rank - 1 << " = 1; (void)" << n << "stride" << rank - 1 << "; ";
             for (int i = rank - 2; i >= 0; i--)
@@ -157,7 +157,7 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
                 dec << "const " << IT << " q" << a << "_ = rem_ / yshape" << a << "; const " << IT << " " << cname
                     << " = rem_ - q" << a << "_ * yshape" << a << "; rem_ = q" << a << "_; ";
             } else {
-                dec << "const int q" << a << "_ = (int)mjt_div((unsigned)rem_, mjt_unpack_divmod(p.a[" << p_yd + a
+                dec << "const int q" << a << "_ = (int)mjt_div((unsigned)rem_, mjt_unpack_divmod((unsigned long long)p.a[" << p_yd + a
                     << "], 0)); const int " << cname << " = rem_ - q" << a << "_ * yshape" << a << "; rem_ = q" << a
                     << "_; ";
             }

@@ -190,6 +190,11 @@ JitKernel* jit_get(const std::string& source, const std::string& entry) {
         std::ifstream f(path, std::ios::binary);
         if (f) code.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
     }
+    if (const char* dump = getenv("MJT_DUMP_DIR")) {
+        // development aid: keep the generated source next to its name
+        std::ofstream f(std::string(dump) + "/" + entry + ".hip");
+        f << source;
+    }
     if (code.empty()) {
         code = compile_source(source, entry + ".hip");
         g_jit_compiled++;

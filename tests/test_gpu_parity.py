@@ -403,3 +403,141 @@ def test_lazy_graph_recomputes_fused_intermediates(gpu):
     assert np.allclose(s.data, x * 6, rtol=1e-6)
     h = jt.histc(jt.array(x), 10, 0.0, 1.0).data
     assert np.array_equal(h, np.histogram(x, 10, (0, 1))[0].astype(np.float32))
+
+
+# ---- meta-op convolution ---------------------------------------------------------------------------------
+def _bf16(a):
+    return O.f32_to_bf16_bits(np.asarray(a, np.float32))
+
+
+def _conv_call(xbits, wbits, params, out_dtype="float32", in_dtype="bfloat16"):
+    import ctypes
+    N, C, H, W = xbits.shape
+    Kc, _, R, S = wbits.shape
+    sh, sw, ph, pw, dh, dw = params
+    oh = (H + 2 * ph - dh * (R - 1) - 1) // sh + 1
+    ow = (W + 2 * pw - dw * (S - 1) - 1) // sw + 1
+    x, w = jt.array(xbits, in_dtype), jt.array(wbits, in_dtype)
+    y = jt.zeros([N, Kc, oh, ow], out_dtype)
+    tx, tw = L.tensor(x.raw_ptr(), in_dtype, x.shape), L.tensor(w.raw_ptr(), in_dtype, w.shape)
+    ty = L.tensor(y.raw_ptr(), out_dtype, y.shape)
+    p = L.ConvParams(*params)
+    L.check(L.load().mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
+    return L.d2h(y.raw_ptr(), y.shape, L.NP_STORAGE[out_dtype]), L.last_kernel()
+
+
+@pytest.mark.parametrize("case", [
+    dict(x=(2, 64, 16, 16), w=(128, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),      # partial last row tile
+    dict(x=(1, 128, 56, 56), w=(128, 128, 3, 3), p=(1, 1, 1, 1, 1, 1)),    # the benchmark geometry, fewer channels
+    dict(x=(3, 64, 28, 24), w=(256, 64, 3, 3), p=(2, 2, 1, 1, 1, 1)),      # stride 2
+    dict(x=(2, 64, 20, 32), w=(128, 64, 3, 3), p=(1, 1, 2, 2, 2, 2)),      # dilation 2
+    dict(x=(2, 192, 14, 8), w=(128, 192, 1, 1), p=(1, 1, 0, 0, 1, 1)),     # 1x1, three channel blocks
+    dict(x=(1, 64, 9, 40), w=(128, 64, 5, 3), p=(1, 1, 2, 1, 1, 1)),       # 5x3 taps, odd height
+])
+def test_conv_mfma_matches_oracle(gpu, case):
+    from oracle import kernels as K
+    rng = np.random.default_rng(20)
+    xb = _bf16(rng.standard_normal(case["x"]))
+    wb = _bf16(rng.standard_normal(case["w"]) * 0.05)
+    sh, sw, ph, pw, dh, dw = case["p"]
+    got, kern = _conv_call(xb, wb, case["p"])
+    assert kern.startswith("mjt_conv_mfma_bf16"), kern
+    if sh == sw and ph == pw and dh == dw:
+        ref = K.conv_meta_bf16(xb, wb, sh, ph, dh, 8)
+    else:
+        ref = None
+    if ref is None:
+        xf, wf = O.BF16(xb).to_f32().astype(np.float64), O.BF16(wb).to_f32().astype(np.float64)
+        N, C, H, W = xf.shape
+        Kc, _, R, S = wf.shape
+        oh, ow = got.shape[2], got.shape[3]
+        xp = np.pad(xf, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+        ref = np.zeros(got.shape)
+        for r in range(R):
+            for s in range(S):
+                patch = xp[:, :, r * dh:r * dh + (oh - 1) * sh + 1:sh, s * dw:s * dw + (ow - 1) * sw + 1:sw]
+                ref += np.einsum("nchw,kc->nkhw", patch, wf[:, :, r, s])
+    # fp32 accumulation in a different order than the reference's (c, kh, kw) loop: 1e-4 relative to the
+    # magnitude of the accumulated terms
+    scale = np.abs(ref).max()
+    assert np.abs(got - ref).max() <= 1e-4 * scale, (np.abs(got - ref).max(), scale)
+    # the direct kernel follows the reference's loop order exactly
+    os.environ["MJT_NO_FASTPATH"] = "1"
+    try:
+        got2, kern2 = _conv_call(xb, wb, case["p"])
+    finally:
+        del os.environ["MJT_NO_FASTPATH"]
+    assert kern2.startswith("mjt_conv_direct")
+    assert np.abs(got2 - ref).max() <= 1e-4 * scale
+
+
+def test_conv_direct_small_shapes_and_fp32(gpu):
+    rng = np.random.default_rng(21)
+    for xs, ws, st, pd, dl in [((2, 3, 9, 8), (4, 3, 3, 3), 1, 1, 1), ((2, 3, 9, 8), (4, 3, 3, 3), 2, 1, 1),
+                               ((1, 5, 11, 7), (2, 5, 3, 3), 1, 2, 2), ((1, 2, 6, 6), (3, 2, 1, 1), 1, 0, 1)]:
+        x = rng.standard_normal(xs).astype(np.float32)
+        w = rng.standard_normal(ws).astype(np.float32)
+        got, kern = _conv_call(x, w, (st, st, pd, pd, dl, dl), in_dtype="float32")
+        assert kern.startswith("mjt_conv_direct_float32")
+        assert np.allclose(got, O.conv_meta(x, w, st, pd, dl), rtol=1e-5, atol=1e-5)
+        got, _ = _conv_call(_bf16(x), _bf16(w), (st, st, pd, pd, dl, dl))
+        assert np.allclose(got, O.conv_meta(O.BF16(_bf16(x)), O.BF16(_bf16(w)), st, pd, dl), rtol=1e-5, atol=1e-5)
+
+
+def test_conv_front_end_pattern_match(gpu):
+    rng = np.random.default_rng(22)
+    x = jt.array(rng.standard_normal((2, 64, 14, 16)).astype(np.float32)).bfloat16()
+    w = jt.array((rng.standard_normal((128, 64, 3, 3)) * 0.05).astype(np.float32)).bfloat16()
+    before = dict(jt.executor_stats)
+    y = jt.nn.conv2d(x, w, padding=1)              # reindex + broadcast + multiply + sum, bf16 output
+    got = y.data
+    assert jt.executor_stats["conv_matches"] == before["conv_matches"] + 1
+    assert y.dtype == "bfloat16" and L.last_kernel().startswith("mjt_fused_")     # trailing cast of the fp32 sum
+    from oracle import kernels as K
+    acc = K.conv_meta_bf16(x.raw(), w.raw(), 1, 1, 1, 8)
+    want = O.BF16(O.f32_to_bf16_bits(acc)).to_f32()
+    assert np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max()
+    # without the matcher the same graph runs through the generic kernels (7-d intermediate materialised)
+    jt.flags["enable_conv_match"] = False
+    try:
+        xs = jt.array(rng.standard_normal((1, 2, 6, 6)).astype(np.float32))
+        ws = jt.array(rng.standard_normal((3, 2, 3, 3)).astype(np.float32))
+        got = jt.nn.conv2d(xs, ws, padding=1).data
+    finally:
+        jt.flags["enable_conv_match"] = True
+    assert np.allclose(got, O.conv_meta(xs.data, ws.data, 1, 1, 1), rtol=1e-5, atol=1e-5)
+    got = jt.nn.conv2d(xs, ws, padding=1).data      # matched, fp32 -> direct kernel
+    assert L.last_kernel().startswith("mjt_conv_direct_float32")
+    assert np.allclose(got, O.conv_meta(xs.data, ws.data, 1, 1, 1), rtol=1e-5, atol=1e-5)
+
+
+def test_conv_full_size_c5_properties(gpu):
+    rng = np.random.default_rng(0)
+    xs, ws = (64, 256, 56, 56), (256, 256, 3, 3)
+    xb = _bf16(rng.standard_normal(xs))
+    wb = _bf16(np.random.default_rng(1).standard_normal(ws) * np.sqrt(2.0 / (256 * 9)))
+    got, kern = _conv_call(xb, wb, (1, 1, 1, 1, 1, 1))
+    assert kern.startswith("mjt_conv_mfma_bf16")
+    xf, wf = O.BF16(xb).to_f32(), O.BF16(wb).to_f32().astype(np.float64)
+    xp = np.pad(xf, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    # sampled outputs against float64 dot products
+    pts = np.random.default_rng(2).integers(0, [64, 256, 56, 56], (4000, 4))
+    err = 0.0
+    mag = 0.0
+    for n, k, h, w_ in pts:
+        patch = xp[n, :, h:h + 3, w_:w_ + 3].astype(np.float64)
+        ref = float((patch * wf[k]).sum())
+        err = max(err, abs(ref - got[n, k, h, w_]))
+        mag = max(mag, float(np.abs(patch * wf[k]).sum()))
+    assert err <= 1e-4 * mag, (err, mag)
+    # padding taps contribute exactly 0 and a one-hot kernel is a shift (bit-exact)
+    w1 = np.zeros(ws, np.float32)
+    for k in range(256):
+        w1[k, k, 0, 2] = 1.0                       # y[n,k,h,w] = x[n,k,h-1,w+1]
+    got1, _ = _conv_call(xb[:8], _bf16(w1), (1, 1, 1, 1, 1, 1))
+    ref1 = np.zeros((8, 256, 56, 56), np.float32)
+    ref1[:, :, 1:, :55] = xf[:8, :, :55, 1:]
+    assert np.array_equal(got1, ref1)
+    # linearity in w: conv(x, 2w) == 2 conv(x, w) exactly
+    got2, _ = _conv_call(xb[:4], _bf16(2 * O.BF16(wb).to_f32()), (1, 1, 1, 1, 1, 1))
+    assert np.array_equal(got2, 2 * got[:4])
