@@ -437,6 +437,17 @@ def array(data, dtype=None):
     return v
 
 
+def from_storage(raw, dtype):
+    """Var from data already in storage format (bfloat16: uint16 bit patterns)."""
+    name = dt.normalize_dtype(dtype)
+    host = np.ascontiguousarray(raw, dtype=_lib.NP_STORAGE[name])
+    v = Var(host.shape, name)
+    v._host = host.reshape(v.shape)
+    if v.num == 1:
+        v.is_scalar = True
+    return v
+
+
 def unary_clone(x):
     # jt.array(var) clones; data-wise an identity broadcast-free copy
     return unary(x, "cast", force_dtype=x.dtype, allow_forward=False)

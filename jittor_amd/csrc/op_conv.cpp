@@ -57,11 +57,13 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     int64_t TRW = OW <= 112 ? 112 / OW : 0;
     if (TRW > OH) TRW = OH;
     while (TRW > 1 && 2 * TRW > OH && (OH % (2 * TRW)) != 0 && (2 * (TRW - 1)) >= OH) TRW--;
-    const int64_t NT = TRW ? (TRW * OW + 15) / 16 : 0;
-    const int64_t LROWS = (2 * TRW - 1) * p->stride_h + (R - 1) * p->dil_h + 1;
+    auto lds_rows = [&](int64_t trw) { return (2 * trw - 1) * p->stride_h + (R - 1) * p->dil_h + 1; };
     const int64_t LCOLS = (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1 > W + 2 * p->pad_w
                               ? (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1
                               : W + 2 * p->pad_w;
+    while (TRW > 1 && lds_rows(TRW) * LCOLS * 128 > 64 * 1024) TRW--;
+    const int64_t NT = TRW ? (TRW * OW + 15) / 16 : 0;
+    const int64_t LROWS = lds_rows(TRW);
     const bool mfma_ok = x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 128 == 0 &&
                          W % 8 == 0 && TRW >= 1 && NT <= 7 && LROWS * LCOLS * 128 <= 64 * 1024 &&
                          (uintptr_t)x->ptr % 16 == 0 && R * S <= 49;

@@ -68,6 +68,13 @@ def _match_conv(red, consumers, targets):
     if red.op != "add" or red.reduce_mask != 0b1100100:
         return None
     yy = red.inputs[0]
+    extra = set()
+    if (not yy.materialised and isinstance(yy._op, UnaryOp) and yy._op.op == "cast" and yy.dtype == "float32"
+            and yy.id not in targets and len(consumers.get(yy.id, ())) == 1):
+        # 16-bit inputs: the sum was rewritten to cast -> reduce(float32) -> cast (ops/reduce_op.cc:259-266);
+        # fused, the product is an exact float temporary (opt/kernel_ir.cc:958-968), so the cast is a no-op
+        extra.add(yy._op.id)
+        yy = yy._op.inputs[0]
     if yy.materialised or yy.ndim != 7 or not isinstance(yy._op, BinaryOp) or yy._op.op != "multiply":
         return None
     if yy.id in targets or len(consumers.get(yy.id, ())) != 1:
@@ -113,7 +120,7 @@ def _match_conv(red, consumers, targets):
             continue
         if red.out.dtype != "float32" and red.out.dtype != x.dtype:
             continue
-        return ConvUnit(red, x, w, (sh, sw, ph, pw, dh, dw), {red.id, yy._op.id, ro.id, bo.id})
+        return ConvUnit(red, x, w, (sh, sw, ph, pw, dh, dw), {red.id, yy._op.id, ro.id, bo.id} | extra)
     return None
 
 

@@ -417,7 +417,7 @@ def _conv_call(xbits, wbits, params, out_dtype="float32", in_dtype="bfloat16"):
     sh, sw, ph, pw, dh, dw = params
     oh = (H + 2 * ph - dh * (R - 1) - 1) // sh + 1
     ow = (W + 2 * pw - dw * (S - 1) - 1) // sw + 1
-    x, w = jt.array(xbits, in_dtype), jt.array(wbits, in_dtype)
+    x, w = jt.from_storage(xbits, in_dtype), jt.from_storage(wbits, in_dtype)
     y = jt.zeros([N, Kc, oh, ow], out_dtype)
     tx, tw = L.tensor(x.raw_ptr(), in_dtype, x.shape), L.tensor(w.raw_ptr(), in_dtype, w.shape)
     ty = L.tensor(y.raw_ptr(), out_dtype, y.shape)
