@@ -6,7 +6,7 @@
 // opt/pass/remove_intermediate_pass.cc:26-47).
 //
 // The host generates four code fragments and the constants below:
-//   VEC, UNROLL, index_t, NPARAM
+//   VEC, UNROLL, BLOCK, index_t, NPARAM, MJT_LD / MJT_ST (plain or non-temporal access)
 //   MJT_FUSED_DECODE   coordinates c0..c{n-1} of element e (only when a
 //                      broadcast input needs them)
 //   MJT_FUSED_LOADS    one vector (or scalar, when broadcast along the
@@ -16,17 +16,17 @@
 //
 // Each lane owns VEC adjacent elements of the innermost axis, so full-size
 // tensors move as 16-byte vectors; a workgroup covers UNROLL contiguous
-// 256*VEC-element runs, which keeps UNROLL independent loads in flight per
+// BLOCK*VEC-element runs, which keeps UNROLL independent loads in flight per
 // lane.
 
 struct Params { void* a[NPARAM]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
 
-extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
+extern "C" __global__ __launch_bounds__(BLOCK) void ENTRY(Params p) {
     const index_t nvec = (index_t)(unsigned long long)p.a[0];
     MJT_FUSED_SCALARS
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
-        const index_t j = ((index_t)blockIdx.x * UNROLL + u) * 256 + threadIdx.x;
+        const index_t j = ((index_t)blockIdx.x * UNROLL + u) * BLOCK + threadIdx.x;
         if (j < nvec) {
             const index_t e = j * VEC;
             MJT_FUSED_DECODE

@@ -13,6 +13,8 @@
 //   MERGE(a, b)     update between two partial results, both TY
 //   INIT            identity, TY
 //   ROW             1: innermost merged axis is reduced; 0: it is kept
+//   UNR             independent loads per lane and step (row kernel)
+//   MJT_LD          mjt_load or mjt_load_nt (streaming input)
 //
 // The host merges adjacent axes of equal kind, so kept and reduced axes
 // alternate.  Row kernel: G lanes stride over the contiguous reduced run with
@@ -105,12 +107,22 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
             const TX* __restrict__ row = xp + kbase + ((NR == 1) ? 0 : mjt_red_offset<(NR > 1 ? NR - 1 : 1)>(p, ro));
             index_t lc_end = nL - lc < it_end - it ? nL : lc + (it_end - it);
             it += lc_end - lc;
-#pragma unroll 4
+            // full steps: every lane in range, UNR independent loads in flight
+            const index_t nfull = L / (G * VEC);
+            for (; lc + UNR <= lc_end && lc + UNR <= nfull; lc += UNR) {
+                mjt_pack<TX, VEC> v[UNR];
+#pragma unroll
+                for (int u = 0; u < UNR; u++) MJT_LD(v[u], row + ((lc + u) * G + lane) * VEC);
+#pragma unroll
+                for (int u = 0; u < UNR; u++)
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v[u].v[k]));
+            }
             for (; lc < lc_end; lc++) {
                 index_t l = (lc * G + lane) * VEC;
                 if (l < L) {
                     mjt_pack<TX, VEC> v;
-                    mjt_load(v, row + l);
+                    MJT_LD(v, row + l);
 #pragma unroll
                     for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v.v[k]));
                 }
@@ -152,7 +164,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     for (; r < r_end; r++) {
         index_t roff = (NR == 1) ? r * (index_t)(unsigned long long)p.a[8 + 4 * 5] : mjt_red_offset<NR>(p, r);
         mjt_pack<TX, VEC> v;
-        mjt_load(v, col + roff);
+        MJT_LD(v, col + roff);
 #pragma unroll
         for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v.v[k]));
     }

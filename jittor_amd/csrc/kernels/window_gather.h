@@ -17,7 +17,7 @@
 
 struct Params { void* a[4]; };   // 8-byte words; typed as pointers so loads/stores use the global address space   // x, y, overflow bits, number of planes
 
-extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
+extern "C" __global__ __launch_bounds__(WTHREADS) void ENTRY(Params p) {
     const TB* __restrict__ xp = (const TB*)p.a[0];
     TB* __restrict__ yp = (TB*)p.a[1];
     const TB ov = (TB)(unsigned long long)p.a[2];
@@ -28,7 +28,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const int rows = (OH - oh0) < TH ? (OH - oh0) : TH;
     const int ih0 = oh0 * SH + CH;          // input row of LDS row 0
     const TB* __restrict__ xplane = xp + (size_t)plane * (H * W);
-    for (int t = threadIdx.x; t < LH * LW; t += 256) {
+    for (int t = threadIdx.x; t < LH * LW; t += WTHREADS) {
         const int lr = t / LW, lc = t - lr * LW;
         const int ih = ih0 + lr, iw = CW + lc;
         TB v = ov;
@@ -40,7 +40,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     constexpr int ROWLEN = OW * KK;
     const int nvec = rows * ROWLEN / VEC;
     TB* __restrict__ yrun = yp + ((size_t)plane * OH + oh0) * ROWLEN;
-    for (int q = threadIdx.x; q < nvec; q += 256) {
+    for (int q = threadIdx.x; q < nvec; q += WTHREADS) {
         const int t0 = q * VEC;
         int r = t0 / ROWLEN;
         int rem = t0 - r * ROWLEN;

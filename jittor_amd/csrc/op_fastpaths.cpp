@@ -62,23 +62,33 @@ bool try_window_gather(const mjt_tensor* x, const mjt_tensor* y, const std::vect
     const int64_t rowlen = OW * KH * KW;
     int vec = 16 / esz;
     while (vec > 1 && (rowlen % vec != 0 || (uintptr_t)y->ptr % (size_t)(vec * esz) != 0)) vec /= 2;
-    // rows per workgroup: LDS tile <= 24 KB, and at least ~4 workgroups per CU when possible
+    // rows per workgroup: aim at ~16 KB of output per workgroup (many workgroups in flight), keep the
+    // lanes of the last store round busy, and start every workgroup's run of y on a vector boundary
     const int64_t LW = (OW - 1) * SW + (KW - 1) * DW + 1;
-    int64_t TH = OH;
     auto tile_rows = [&](int64_t th) { return (th - 1) * SH + (KH - 1) * DH + 1; };
-    while (TH > 1 && tile_rows(TH) * LW * esz > 24 * 1024) TH = (TH + 1) / 2;
-    if (tile_rows(TH) * LW * esz > 48 * 1024) return false;
-    const int64_t cu = ctx().prop.multiProcessorCount;
-    while (TH > 4 && planes * ((OH + TH - 1) / TH) < cu * 4) TH = (TH + 1) / 2;
-    // a workgroup's run of y must start on a vector boundary
-    while (TH < OH && (TH * rowlen) % vec != 0) TH++;
+    const int wthreads = env_int("MJT_WINDOW_THREADS", 256);
+    int64_t TH = 0;
+    double best = -1.0;
+    for (int64_t th = 1; th <= OH; th++) {
+        if ((th * rowlen) % vec != 0 && th != OH) continue;
+        if (tile_rows(th) * LW * esz > 48 * 1024) break;
+        const int64_t nv = th * rowlen / vec;
+        const double lanes = (double)nv / (double)(((nv + wthreads - 1) / wthreads) * wthreads);
+        const double bytes = (double)(th * rowlen * esz);
+        const double size_score = bytes < 16384.0 ? bytes / 16384.0 : 16384.0 / bytes;
+        const double tail = (double)OH / (double)(((OH + th - 1) / th) * th);     // rows wasted in the last tile
+        const double score = lanes * tail * (0.5 + 0.5 * size_score);
+        if (score > best) { best = score; TH = th; }
+    }
+    if (TH == 0) return false;
+    if (env_int("MJT_WINDOW_TH", 0) > 0 && env_int("MJT_WINDOW_TH", 0) <= OH) TH = env_int("MJT_WINDOW_TH", 0);
     const int64_t LH = tile_rows(TH);
     const int64_t tiles = (OH + TH - 1) / TH;
     if (planes * tiles >= (int64_t(1) << 31)) return false;
 
     std::ostringstream key;
     key << "win|" << esz << "|" << vec << "|" << H << "," << W << "," << OH << "," << OW << "," << KH << "," << KW << ","
-        << SH << "," << SW << "," << DH << "," << DW << "," << CH << "," << CW << "," << TH;
+        << SH << "," << SW << "," << DH << "," << DW << "," << CH << "," << CW << "," << TH << "," << wthreads;
     JitKernel* k = cached(key.str());
     if (!k) {
         std::ostringstream name;
@@ -89,7 +99,7 @@ bool try_window_gather(const mjt_tensor* x, const mjt_tensor* y, const std::vect
             << "\n#define VEC " << vec << "\n#define H " << H << "\n#define W " << W << "\n#define OH " << OH
             << "\n#define OW " << OW << "\n#define KH " << KH << "\n#define KW " << KW << "\n#define SH " << SH
             << "\n#define SW " << SW << "\n#define DH " << DH << "\n#define DW " << DW << "\n#define CH (" << CH
-            << ")\n#define CW (" << CW << ")\n#define TH " << TH << "\n#define LH " << LH << "\n#define LW " << LW << "\n";
+            << ")\n#define CW (" << CW << ")\n#define WTHREADS " << wthreads << "\n#define TH " << TH << "\n#define LH " << LH << "\n#define LW " << LW << "\n";
         src << embedded_source("prelude.h") << "\n" << embedded_source("window_gather.h") << "\n";
         k = jit_get(src.str(), name.str());
         remember(key.str(), k);
@@ -107,14 +117,12 @@ bool try_window_gather(const mjt_tensor* x, const mjt_tensor* y, const std::vect
     }
     if (esz < 8) ovbits &= (1ull << (8 * esz)) - 1;
     std::vector<uint64_t> args{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), ovbits, (uint64_t)planes};
-    jit_launch(k, (unsigned)(planes * tiles), 1, 256, 0, args);
+    jit_launch(k, (unsigned)(planes * tiles), 1, (unsigned)wthreads, 0, args);
     return true;
 }
 
 // x[idx[i]] = OP(x[idx[i]], y[i]); fills x with the identity first.
 void launch_fill_pattern(void* dst, uint64_t pattern, int elem_size, size_t n);
-
-static void* g_lo = nullptr;   // device int: start of the privatised window
 
 bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_tensor* index) {
     if (getenv("MJT_NO_FASTPATH")) return false;
@@ -124,13 +132,20 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     if (index->dtype != MJT_INT32 && index->dtype != MJT_INT64) return false;
     if (x->ndim != 1 || y->ndim != 1) return false;
     const int64_t n = numel(y), bins = numel(x);
-    if (bins >= (int64_t(1) << 31)) return false;
-    if ((uintptr_t)y->ptr % 16 || (uintptr_t)index->ptr % 32) return false;
+    if (bins >= (int64_t(1) << 31) || n >= (int64_t(1) << 40)) return false;
+    if ((uintptr_t)y->ptr % 16 || (uintptr_t)index->ptr % 32 || (uintptr_t)x->ptr % 4) return false;
     Context& c = ctx();
-    int wbins = env_int("MJT_SCATTER_WBINS", 16384);
-    while (wbins > 256 && wbins / 2 >= bins) wbins /= 2;
-    int nthreads = env_int("MJT_SCATTER_THREADS", 1024);
-    int per_cu = env_int("MJT_SCATTER_WG_PER_CU", 2);
+    int logw = env_int("MJT_SCATTER_LOGW", 14);              // 16384 bins = 64 KB of LDS per private copy
+    while (logw > 8 && (int64_t(1) << (logw - 1)) >= bins) logw--;
+    const int64_t W = int64_t(1) << logw;
+    const int64_t NB = (bins + W - 1) / W;
+    if (NB > 4096) return false;                              // list cursors live in LDS
+    int64_t nbmax = 1;
+    while (nbmax < NB) nbmax *= 2;
+    const int nthreads = env_int("MJT_SCATTER_THREADS", 1024);
+    const int per_cu = env_int("MJT_SCATTER_WG_PER_CU", 1);
+    const int64_t cold_target = env_int("MJT_SCATTER_COLD_TARGET", 8192);   // list entries per cold workgroup
+    const int nhot = env_int("MJT_SCATTER_NHOT", mode == 0 ? 8 : 4);
     // identity
     uint32_t ident = 0;
     if (mode) {
@@ -138,45 +153,65 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
         else if (x->dtype == MJT_INT32) ident = mode == 1 ? 0x80000000u : 0x7fffffffu;
         else ident = mode == 1 ? 0u : 0xffffffffu;
     }
+    // geometry of the main pass
+    int64_t G1 = (int64_t)c.prop.multiProcessorCount * per_cu;
+    if (G1 > 512) G1 = 512;
+    const int64_t chunk = (int64_t)nthreads * 4;
+    const int64_t per = ((n + G1 - 1) / G1 + chunk - 1) / chunk * chunk;
+    G1 = n ? (n + per - 1) / per : 1;
+    // cold workgroups: one per bucket plus population / cold_target (see mjt_make_plan)
+    const int64_t cold_wgs = NB > 1 ? NB + n / cold_target + 1 : 0;
+    int64_t CAP = NB > 1 ? (4 * per / NB + 63) / 64 * 64 : 64;
+    if (CAP < 64) CAP = 64;
+    if (CAP > per) CAP = (per + 63) / 64 * 64;
+
     std::ostringstream key;
-    key << "sc1|" << x->dtype << "|" << index->dtype << "|" << mode << "|" << wbins << "|" << nthreads;
-    JitKernel* k = cached(key.str());
-    JitKernel* ks = cached(key.str() + "|sample");
-    if (!k || !ks) {
+    key << "sc1|" << x->dtype << "|" << index->dtype << "|" << mode << "|" << logw << "|" << nbmax << "|" << nthreads << "|" << nhot << "|" << cold_target;
+    static const char* parts[] = {"sample", "main", "cold", "final"};
+    JitKernel* ks[4];
+    bool have = true;
+    for (int i = 0; i < 4; i++) have = (ks[i] = cached(key.str() + "|" + parts[i])) != nullptr && have;
+    if (!have) {
         std::ostringstream name;
         name << "mjt_scatter1d_" << mjt_op_name(op) << "_" << mjt_dtype_name(x->dtype) << "_" << mjt_dtype_name(index->dtype)
-             << "_w" << wbins << "_t" << nthreads;
+             << "_w" << W << "_b" << nbmax << "_t" << nthreads;
         std::ostringstream src;
-        src << "#define ENTRY " << name.str() << "\n#define ENTRY_SAMPLE " << name.str() << "_sample\n#define TX "
-            << dtype_cname(x->dtype) << "\n#define TE " << dtype_cname(index->dtype) << "\n#define WBINS " << wbins
-            << "\n#define NTHREADS " << nthreads << "\n#define MODE " << mode << "\n#define IDENT_BITS " << ident << "u\n";
+        src << "#define ENTRY_SAMPLE " << name.str() << "_sample\n#define ENTRY_MAIN " << name.str() << "_main\n#define ENTRY_COLD "
+            << name.str() << "_cold\n#define ENTRY_FINAL " << name.str() << "_final\n#define COLD_TARGET " << cold_target
+            << "u\n#define TX " << dtype_cname(x->dtype) << "\n#define TE " << dtype_cname(index->dtype) << "\n#define WBINS "
+            << W << "\n#define LOGW " << logw << "\n#define NBMAX " << nbmax << "\n#define NTHREADS " << nthreads
+            << "\n#define NHOT " << nhot << "\n#define MODE " << mode << "\n#define IDENT_BITS " << ident << "u\n";
         src << embedded_source("prelude.h") << "\n" << embedded_source("atomics.h") << "\n" << embedded_source("scatter1d.h")
             << "\n";
-        k = jit_get(src.str(), name.str());
-        // second entry point of the same module
-        ks = new JitKernel();
-        ks->name = name.str() + "_sample";
-        ks->module = k->module;
-        if (!c.dry_run) HIP_CHECK(hipModuleGetFunction(&ks->fn, k->module, ks->name.c_str()));
-        remember(key.str(), k);
-        remember(key.str() + "|sample", ks);
+        JitKernel* first = jit_get(src.str(), name.str() + "_sample");
+        for (int i = 0; i < 4; i++) {
+            JitKernel* k = i == 0 ? first : new JitKernel();
+            if (i) {
+                k->name = name.str() + "_" + parts[i];
+                k->module = first->module;
+                if (!c.dry_run) HIP_CHECK(hipModuleGetFunction(&k->fn, first->module, k->name.c_str()));
+            }
+            ks[i] = k;
+            remember(key.str() + "|" + parts[i], k);
+        }
     }
-    if (!g_lo && !c.dry_run) {
-        HIP_CHECK(hipMalloc(&g_lo, 256));
-    }
-    launch_fill_pattern(x->ptr, ident, 4, (size_t)bins);
-    int64_t groups = (int64_t)c.prop.multiProcessorCount * per_cu;
-    int64_t chunk = (int64_t)nthreads * 4;
-    int64_t per = ((n + groups - 1) / groups + chunk - 1) / chunk * chunk;
-    groups = (n + per - 1) / per;
-    std::vector<uint64_t> args{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), bits_of_ptr(index->ptr), (uint64_t)n,
-                               (uint64_t)bins,      bits_of_ptr(g_lo),   (uint64_t)per,            0};
-    if (bins > wbins) {
-        jit_launch(ks, 1, 1, 1024, 0, args);
-    } else {
-        launch_fill_pattern(g_lo, 0, 4, 1);
-    }
-    jit_launch(k, (unsigned)groups, 1, (unsigned)nthreads, 0, args);
+    // scratch layout
+    auto align = [](size_t v) { return (v + 255) / 256 * 256; };
+    const size_t off_counts = 32768;                          // control block: 64 words + one word per bucket
+    const size_t off_pmain = off_counts + align((size_t)G1 * NB * 4);
+    const size_t off_pcold = off_pmain + align((size_t)G1 * W * 4);
+    const size_t off_lists = off_pcold + align((size_t)cold_wgs * W * 4);
+    const size_t off_ovf = off_lists + align(NB > 1 ? (size_t)G1 * NB * CAP * 8 : 0);
+    const size_t total = off_ovf + align(NB > 1 ? (size_t)n * 8 : 0);
+    char* base = (char*)scratch(total);
+    std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), bits_of_ptr(index->ptr), (uint64_t)n, (uint64_t)bins,
+                            bits_of_ptr(base), (uint64_t)per, (uint64_t)G1, (uint64_t)NB, (uint64_t)CAP,
+                            bits_of_ptr(base + off_counts), bits_of_ptr(base + off_lists), bits_of_ptr(base + off_pmain),
+                            bits_of_ptr(base + off_pcold), 0, bits_of_ptr(base + off_ovf)};
+    jit_launch(ks[0], 1, 1, 1024, 0, a);
+    jit_launch(ks[1], (unsigned)G1, 1, (unsigned)nthreads, 0, a);
+    if (NB > 1) jit_launch(ks[2], (unsigned)cold_wgs, 1, (unsigned)nthreads, 0, a);
+    jit_launch(ks[3], (unsigned)(NB * (W / 256)), 1, 256, 0, a);
     return true;
 }
 

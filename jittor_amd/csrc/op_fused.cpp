@@ -118,7 +118,12 @@ void fused_impl(const mjt_fused_desc* d) {
     };
     while (vec > 1 && !aligned(vec)) vec /= 2;
     int64_t nvec = total / vec;
-    int unroll = nvec >= (int64_t)ctx().prop.multiProcessorCount * 256 * 8 ? 4 : 1;
+    auto env_int = [](const char* n, int d) { const char* v = getenv(n); return v && *v ? atoi(v) : d; };
+    int block = env_int("MJT_FUSED_BLOCK", 256);
+    // measured on MI355X: one vector per lane and plain (cached) access is fastest for the chain
+    // workloads; more vectors per lane cost registers and occupancy
+    int unroll = env_int("MJT_FUSED_UNROLL", 1);
+    bool nt = env_int("MJT_FUSED_NT", 0) != 0;
 
     // ---- parameter block layout ---------------------------------------------------
     // a[0] nvec | per merged axis: extent, divider | per var: pointer or scalar bits
@@ -164,7 +169,7 @@ void fused_impl(const mjt_fused_desc* d) {
 
     // ---- static key -----------------------------------------------------------------
     std::ostringstream key;
-    key << nd << "|" << vec << "|" << unroll << "|" << use64 << "|";
+    key << nd << "|" << vec << "|" << unroll << "|" << use64 << "|" << block << "|" << nt << "|";
     for (int a = 0; a < nd; a++) {
         for (int b : dims[a].bcast) key << b;
         key << ",";
@@ -225,7 +230,7 @@ void fused_impl(const mjt_fused_desc* d) {
             if (dims.back().bcast[k] && vec > 1) {
                 loads << "const " << T << " s" << id << " = ((const " << T << "*)p.a[" << p_var[id] << "])[" << off << "]; ";
             } else {
-                loads << "mjt_pack<" << T << ", VEC> in" << id << "; mjt_load(in" << id << ", (const " << T << "*)p.a["
+                loads << "mjt_pack<" << T << ", VEC> in" << id << "; MJT_LD(in" << id << ", (const " << T << "*)p.a["
                       << p_var[id] << "] + " << off << "); ";
             }
         }
@@ -267,11 +272,12 @@ void fused_impl(const mjt_fused_desc* d) {
         }
         for (int i = 0; i < nv; i++)
             if (d->vars[i].role == MJT_VAR_OUTPUT)
-                stores << "mjt_store((" << dtype_cname(d->vars[i].dtype) << "*)p.a[" << p_var[i] << "] + e, out" << i << "); ";
+                stores << "MJT_ST((" << dtype_cname(d->vars[i].dtype) << "*)p.a[" << p_var[i] << "] + e, out" << i << "); ";
 
         std::ostringstream frag;
         frag << "#define VEC " << vec << "\n#define UNROLL " << unroll << "\n#define index_t " << IT << "\n#define NPARAM "
-             << args.size() << "\n";
+             << args.size() << "\n#define BLOCK " << block << "\n#define MJT_LD " << (nt ? "mjt_load_nt" : "mjt_load")
+             << "\n#define MJT_ST " << (nt ? "mjt_store_nt" : "mjt_store") << "\n";
         frag << "#define MJT_FUSED_SCALARS " << scal.str() << "\n";
         frag << "#define MJT_FUSED_DECODE " << dec.str() << "\n";
         frag << "#define MJT_FUSED_LOADS " << loads.str() << "\n";
@@ -290,10 +296,10 @@ void fused_impl(const mjt_fused_desc* d) {
         std::lock_guard<std::mutex> lock(g_mu);
         g_kernels.emplace(key.str(), kern);
     }
-    int64_t per_block = (int64_t)256 * unroll;
+    int64_t per_block = (int64_t)block * unroll;
     int64_t blocks = (nvec + per_block - 1) / per_block;
     MJT_CHECK(blocks < (int64_t(1) << 31), "fused: launch too large");
-    jit_launch(kern, (unsigned)blocks, 1, 256, 0, args);
+    jit_launch(kern, (unsigned)blocks, 1, (unsigned)block, 0, args);
 }
 
 }  // namespace mjt

@@ -28,15 +28,20 @@ bool reducible(int op) {
     }
 }
 
+int env_int(const char* n, int d) {
+    const char* v = getenv(n);
+    return v && *v ? atoi(v) : d;
+}
+
 struct Variant {
-    int tx, ty, op, nk, nr, vec, g;
+    int tx, ty, op, nk, nr, vec, g, unr, nt;
     bool row, split, use64, second;   // second: folding partials (TX == TY, plain merge)
 };
 
 JitKernel* get_kernel(const Variant& v) {
     std::ostringstream key;
     key << v.tx << "," << v.ty << "," << v.op << "," << v.nk << "," << v.nr << "," << v.vec << "," << v.g << ","
-        << v.row << v.split << v.use64 << v.second;
+        << v.row << v.split << v.use64 << v.second << "," << v.unr << "," << v.nt;
     std::lock_guard<std::mutex> lock(g_mu);
     auto it = g_kernels.find(key.str());
     if (it != g_kernels.end()) return it->second;
@@ -52,6 +57,7 @@ JitKernel* get_kernel(const Variant& v) {
     src << "#define index_t " << (v.use64 ? "long long" : "int") << "\n#define USE64 " << (v.use64 ? 1 : 0) << "\n";
     src << "#define NK " << v.nk << "\n#define NR " << v.nr << "\n#define VEC " << v.vec << "\n#define G " << v.g
         << "\n#define SPLIT " << (v.split ? 1 : 0) << "\n#define ROW " << (v.row ? 1 : 0) << "\n";
+    src << "#define UNR " << v.unr << "\n#define MJT_LD " << (v.nt ? "mjt_load_nt" : "mjt_load") << "\n";
     src << "#define MERGE(a, b) mjt_" << merge_op << "<TY>((a), (b))\n";
     if (v.second || v.op != MJT_OP_MEAN)
         src << "#define COMBINE(a, x) mjt_" << (v.second ? merge_op : std::string(opn)) << "<TY>((a), (x))\n";
@@ -90,8 +96,10 @@ void fill_axes(std::vector<uint64_t>& a, const std::vector<Axis>& kept, const st
 // S > 1) are written to `out` as [O, S] (row) or [S, O] (column).
 void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* out, int64_t O, int64_t S,
             const std::vector<Axis>& kept, const std::vector<Axis>& red, double rcount, bool use64, int vec, int g,
-            int64_t per, int64_t total) {
-    Variant v{tx, ty, op, (int)kept.size(), (int)red.size(), vec, g, row, S > 1, use64, second};
+            int64_t per, int64_t total, bool stream = false) {
+    // inputs larger than the caches are streamed (read once, non-temporal loads)
+    Variant v{tx, ty, op, (int)kept.size(), (int)red.size(), vec, g, env_int("MJT_REDUCE_UNR", 8),
+              env_int("MJT_REDUCE_NT", stream ? 1 : 0), row, S > 1, use64, second};
     JitKernel* k = get_kernel(v);
     std::vector<uint64_t> a(8 + 6 * 5, 0);
     a[0] = bits_of_ptr(x);
@@ -165,6 +173,7 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
     }
     bool use64 = xn >= (int64_t(1) << 31);
     bool row = red.back().stride == 1;   // innermost merged axis is reduced
+    const bool stream = xn * (int64_t)dtype_size(tx) >= (int64_t(64) << 20);
     const int64_t cu = c.prop.multiProcessorCount;
 
     if (row) {
@@ -191,10 +200,10 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         int64_t per = (total + S - 1) / S;
         S = (total + per - 1) / per;
         if (S == 1) {
-            launch(true, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, g, per, total);
+            launch(true, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, g, per, total, stream);
         } else {
             void* part = scratch((size_t)O * S * tsz);
-            launch(true, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, g, per, total);
+            launch(true, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, g, per, total, stream);
             // fold [O, S] along the last axis
             std::vector<Axis> k2{Axis{O, S}}, r2{Axis{S, 1}};
             int vec2 = pick_vec(tsz, S, part, nullptr, 0);
@@ -222,10 +231,10 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         int64_t per = (R + S - 1) / S;
         S = (R + per - 1) / per;
         if (S == 1) {
-            launch(false, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, 1, per, R);
+            launch(false, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, 1, per, R, stream);
         } else {
             void* part = scratch((size_t)O * S * tsz);
-            launch(false, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R);
+            launch(false, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R, stream);
             std::vector<Axis> k2{Axis{O, 1}}, r2{Axis{S, O}};
             int vec2 = pick_vec(tsz, O, part, y->ptr, tsz);
             launch(false, ty, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, 1, S, S);
