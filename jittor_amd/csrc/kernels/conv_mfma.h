@@ -8,71 +8,83 @@
 // contribute 0 (overflow value 0 times w).
 //
 // All geometry is baked in by the host: C_, H_, W_, K_, R_, S_, OH_, OW_, SH, SW,
-// PH, PW, DH, DW, TRW (output rows per wave), NT (16-pixel tiles per wave),
-// LROWS x LCOLS (input tile held in LDS), ITEMS_PER_WAVE, Y_BF16.
+// PH, PW, DH, DW, TRW (output rows per wave), NT (16-pixel tiles per wave), WKO
+// (groups of 64 output channels per workgroup), WPX (row groups per workgroup), LROWS x LCOLS (input tile held in LDS), ITEMS_PER_WAVE, Y_BF16.
 //
 // Mapping.  v_mfma_f32_16x16x32_bf16 computes D[16 ko][16 px] += A[16 ko][32 c] *
-// B[32 c][16 px].  A workgroup of 4 waves owns 128 output channels x (2*TRW
-// output rows) of one image; wave (wko, wpx) owns 64 channels x TRW rows =
+// B[32 c][16 px].  A workgroup of WPX*WKO waves owns 64*WKO output channels x
+// (WPX*TRW output rows) of one image; wave (wko, wpx) owns 64 channels x TRW rows =
 // 4 x NT accumulator tiles.  Channels are consumed 64 at a time:
 //   * the input rows the tile touches are staged through LDS as
 //     [row][col][64 c] (channel innermost) so that a B fragment is one 16-byte
-//     LDS read per lane; the NCHW -> channel-innermost transpose happens in the
-//     LDS write (lane = channel, so the 2-byte writes of a wave fill whole
-//     128-byte rows and the 16-byte chunk index is XOR-swizzled with the column
-//     to keep fragment reads conflict-free);
+//     LDS read per lane.  The NCHW -> channel-innermost transpose happens in the
+//     LDS write: a lane loads 8 columns of one channel, swaps halves with its
+//     neighbour lane so that it owns two channels x four columns, packs the two
+//     channels of a column into one dword, and the dwords of a wave fill whole
+//     128-byte rows; positions are padded to 144 bytes so that fragment reads
+//     are conflict-free.  The tile is double
+//     buffered: the loads of the next 64 channels are issued before the MFMAs of
+//     the current 64 and written to the other buffer after them (one barrier per
+//     channel block);
 //   * A fragments come straight from the re-packed weights
-//     Wp[tap][c/64][k-step][ko][32 c] (1 KB contiguous per fragment, L2 resident);
-//   * the A fragments of the next step are loaded while the MFMAs of the
-//     current step run; two workgroups per CU overlap one's staging with the
-//     other's MFMAs.
+//     Wp[tap][c/64][k-step][ko][32 c] (1 KB contiguous per fragment, L2
+//     resident) and are loaded one step before the MFMAs that use them.
 // Halo cells (padding, rows outside the image) are zeroed once: they are the
 // same for every channel block.
 
 typedef __bf16 mjt_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float mjt_f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned short mjt_u16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned mjt_u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
 
-struct Params { void* a[4]; };   // 8-byte words; typed as pointers so loads/stores use the global address space   // x, packed w, y, number of images
+struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as pointers: global address space)
 
 #define CB 64
-#define KO_WG 128
+#define KO_WG (64 * WKO)
+#define NWAVES (WPX * WKO)
+#define NTHR (64 * NWAVES)
 #define MT 4
-#define TR (2 * TRW)
+#define TR (WPX * TRW)
 #define TILES_R ((OH_ + TR - 1) / TR)
 #define NCB (C_ / CB)
-#define GROUPS (W_ / 8)
-#define ITEMS (LROWS * GROUPS)
+#define GROUPS (W_ / 8)                 // groups of 8 columns
+#define ITEMS (LROWS * GROUPS)          // (row, column group); a wave moves the 64 channels of an item
+#define TILE_ELEMS (LROWS * LCOLS * PSTRIDE)
 
+// LDS tile: position (row, col) holds its 64 channels in 128 bytes followed by 16 bytes of padding.
+// With a 144-byte stride, 8 neighbouring positions read by 8 lanes (one 16-byte chunk each) fall on 8
+// different groups of 4 banks, so fragment reads are conflict-free, and the address of a fragment is
+// linear in the tap: it folds into the immediate offset of the LDS read.
+#define PSTRIDE 72
 __device__ __forceinline__ int mjt_lds_off(int pos, int chunk) {
     // element offset (in bf16) of 16-byte chunk `chunk` (0..7) of position `pos`
-    return pos * CB + ((chunk ^ (pos & 7)) << 3);
+    return pos * PSTRIDE + (chunk << 3);
 }
 
-extern "C" __global__ __launch_bounds__(256, 2) void ENTRY(Params p) {
+extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const unsigned short* __restrict__ xp = (const unsigned short*)p.a[0];
     const unsigned short* __restrict__ wp = (const unsigned short*)p.a[1];
     const int n_img = (int)(unsigned long long)p.a[3];
-    __shared__ __attribute__((aligned(16))) unsigned short xs[LROWS * LCOLS * CB];
+    __shared__ __attribute__((aligned(16))) unsigned short xs[2][TILE_ELEMS];
 
-    // tile id: the two channel halves of one pixel tile are 8 workgroups apart,
-    // so they land on the same XCD (workgroups go round-robin over 8 XCDs) and
+    // tile id: the channel groups of one pixel tile are 8 workgroups apart, so
+    // they land on the same XCD (workgroups go round-robin over 8 XCDs) and
     // share the input rows in that XCD's L2
     const int id = blockIdx.x;
     const int xcd = id & 7, j = id >> 3;
-    const int khalf = j % (K_ / KO_WG);
+    const int kpart = j % (K_ / KO_WG);
     const int ptile = (j / (K_ / KO_WG)) * 8 + xcd;
     if (ptile >= n_img * TILES_R) return;
     const int n = ptile / TILES_R;
     const int r0 = (ptile % TILES_R) * TR;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wpx = wave & 1, wko = wave >> 1;
-    const int ko_base = khalf * KO_WG + wko * 64;
+    const int wpx = wave % WPX, wko = wave / WPX;
+    const int ko_base = kpart * KO_WG + wko * 64;
     const int l16 = lane & 15, lg = lane >> 4;
 
-    // zero the whole tile once (halo cells stay zero)
-    for (int t = tid; t < LROWS * LCOLS * CB / 8; t += 256) ((mjt_u16x8*)xs)[t] = (mjt_u16x8)(0);
+    // zero both buffers once (halo cells stay zero)
+    for (int t = tid; t < 2 * TILE_ELEMS / 8; t += NTHR) ((mjt_u32x4v*)&xs[0][0])[t] = (mjt_u32x4v)(0u);
 
     // per-lane pixel of each of the NT tiles
     int bpos[NT];
@@ -90,35 +102,51 @@ extern "C" __global__ __launch_bounds__(256, 2) void ENTRY(Params p) {
 #pragma unroll
         for (int t = 0; t < NT; t++) acc[m][t] = (mjt_f32x4)(0.0f);
 
-    // staging: item = (tile row, group of 8 columns); a wave moves 64 channels of an item
+    // staging: item = (tile row, group of 8 columns); a wave moves the 64 channels of an item, lane l
+    // loading 16 bytes (8 columns) of channel l -- one scattered load per lane is what the address unit
+    // is charged for, so it should be as wide as possible.  Adjacent lanes (channels 2k, 2k+1) then swap
+    // halves so that each owns 4 columns of both channels, and write one dword (channel pair) per column.
     const int ir0 = r0 * SH - PH;
-    auto stage_in = [&](int cb) {
-        mjt_u16x8 stage[ITEMS_PER_WAVE];
+    const int odd = lane & 1;
+    mjt_u32x4v stage[ITEMS_PER_WAVE];
+    auto fetch = [&](int cb) {
 #pragma unroll
         for (int it = 0; it < ITEMS_PER_WAVE; it++) {
-            const int item = it * 4 + wave;
+            const int item = it * NWAVES + wave;
             const int lr = item / GROUPS, g = item - lr * GROUPS;
             const int ir = ir0 + lr;
-            mjt_u16x8 v = (mjt_u16x8)(0);
+            mjt_u32x4v v = (mjt_u32x4v)(0u);
             if (item < ITEMS && ir >= 0 && ir < H_)
-                v = *(const mjt_u16x8*)(xp + (((size_t)n * C_ + cb * CB + lane) * H_ + ir) * W_ + g * 8);
+                v = *(const mjt_u32x4v*)(xp + (((size_t)n * C_ + cb * CB + lane) * H_ + ir) * W_ + g * 8);
             stage[it] = v;
         }
-        __syncthreads();              // zero fill / the previous channel block's reads are done
+    };
+    auto commit = [&](int buf) {
 #pragma unroll
         for (int it = 0; it < ITEMS_PER_WAVE; it++) {
-            const int item = it * 4 + wave;
+            const int item = it * NWAVES + wave;
             const int lr = item / GROUPS, g = item - lr * GROUPS;
             const int ir = ir0 + lr;
+            // even lane keeps its columns 0..3 and receives columns 0..3 of the odd lane; the odd lane
+            // keeps columns 4..7 and receives columns 4..7 of the even lane
+            const unsigned give0 = odd ? stage[it][0] : stage[it][2];
+            const unsigned give1 = odd ? stage[it][1] : stage[it][3];
+            const unsigned got0 = (unsigned)__shfl_xor((int)give0, 1, 64);
+            const unsigned got1 = (unsigned)__shfl_xor((int)give1, 1, 64);
+            const unsigned mine0 = odd ? stage[it][2] : stage[it][0];
+            const unsigned mine1 = odd ? stage[it][3] : stage[it][1];
+            const unsigned lo0 = odd ? got0 : mine0, hi0 = odd ? mine0 : got0;   // lo = even channel, hi = odd channel
+            const unsigned lo1 = odd ? got1 : mine1, hi1 = odd ? mine1 : got1;
             if (item < ITEMS && ir >= 0 && ir < H_) {
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const int pos = lr * LCOLS + PW + g * 8 + e;
-                    xs[mjt_lds_off(pos, lane >> 3) + (lane & 7)] = stage[it][e];
-                }
+                const int c = lane & ~1;                     // first channel of the pair
+                const int pos0 = lr * LCOLS + PW + g * 8 + odd * 4;
+                unsigned* dst = (unsigned*)&xs[buf][0];
+                dst[(mjt_lds_off(pos0 + 0, c >> 3) + (c & 7)) >> 1] = (lo0 & 0xffffu) | (hi0 << 16);
+                dst[(mjt_lds_off(pos0 + 1, c >> 3) + (c & 7)) >> 1] = (lo0 >> 16) | (hi0 & 0xffff0000u);
+                dst[(mjt_lds_off(pos0 + 2, c >> 3) + (c & 7)) >> 1] = (lo1 & 0xffffu) | (hi1 << 16);
+                dst[(mjt_lds_off(pos0 + 3, c >> 3) + (c & 7)) >> 1] = (lo1 >> 16) | (hi1 & 0xffff0000u);
             }
         }
-        __syncthreads();
     };
 
     // A fragments: Wp[step][ko][32 c], step = (tap * NCB + cb) * 2 + ks; 16 rows x 64 B per fragment
@@ -129,13 +157,14 @@ extern "C" __global__ __launch_bounds__(256, 2) void ENTRY(Params p) {
 #pragma unroll
         for (int m = 0; m < MT; m++) a[m] = *(const mjt_bf16x8*)(f + m * 16 * 32);
     };
-    auto compute = [&](const mjt_bf16x8 (&a)[MT], int s) {
+    auto compute = [&](const mjt_bf16x8 (&a)[MT], int s, int buf) {
         const int tap = s >> 1, ks = s & 1;
         const int kh = tap / S_, kw = tap - kh * S_;
         const int tap_pos = kh * DH * LCOLS + kw * DW;
+        const unsigned short* tile = &xs[buf][0];
         mjt_bf16x8 b[NT];
 #pragma unroll
-        for (int t = 0; t < NT; t++) b[t] = *(const mjt_bf16x8*)(xs + mjt_lds_off(bpos[t] + tap_pos, ks * 4 + lg));
+        for (int t = 0; t < NT; t++) b[t] = *(const mjt_bf16x8*)(tile + mjt_lds_off(bpos[t] + tap_pos, ks * 4 + lg));
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
@@ -143,18 +172,27 @@ extern "C" __global__ __launch_bounds__(256, 2) void ENTRY(Params p) {
                 acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[m], b[t], acc[m][t], 0, 0, 0);
     };
 
-    // the weights of step s+1 are in flight while the MFMAs of step s run
-    mjt_bf16x8 a0[MT], a1[MT];
-    load_a(a0, 0, 0);
-    for (int cb = 0; cb < NCB; cb++) {
-        stage_in(cb);
+    constexpr int STEPS = 2 * R_ * S_;            // steps per channel block (even)
+    mjt_bf16x8 ring[2][MT];                       // weights of the next step are in flight during a step
+    load_a(ring[0], 0, 0);
+    fetch(0);
+    __syncthreads();                              // zero fill done
+    commit(0);
+    __syncthreads();
+    // two steps per iteration (the ring has two slots); the tap is a run-time value
 #pragma unroll 1
-        for (int s = 0; s < 2 * R_ * S_; s += 2) {
-            load_a(a1, cb, s + 1);
-            compute(a0, s);
-            if (s + 2 < 2 * R_ * S_) load_a(a0, cb, s + 2);
-            else if (cb + 1 < NCB) load_a(a0, cb + 1, 0);
-            compute(a1, s + 1);
+    for (int g0 = 0; g0 < NCB * STEPS; g0 += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int g = g0 + u;
+            const int cb = g / STEPS, st = g - cb * STEPS;
+            if (st == 0 && cb + 1 < NCB) fetch(cb + 1);      // in flight during this block's MFMAs
+            if (g + 1 < NCB * STEPS) load_a(ring[u ^ 1], (g + 1) / STEPS, (g + 1) % STEPS);
+            compute(ring[u], st, cb & 1);
+            if (st == STEPS - 1 && cb + 1 < NCB) {
+                commit((cb + 1) & 1);                        // the other buffer: nobody reads it now
+                __syncthreads();
+            }
         }
     }
 

@@ -54,24 +54,29 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         << p->dil_h << "\n#define DW " << p->dil_w << "\n";
 
     // ---- MFMA path ----------------------------------------------------------------
-    int64_t TRW = OW <= 112 ? 112 / OW : 0;
+    const char* wpx_env = getenv("MJT_CONV_WPX");
+    const int64_t WPX = wpx_env && *wpx_env ? atoi(wpx_env) : 2;
+    const int64_t max_px = WPX == 1 ? 224 : 112;            // pixels per wave: 16 per accumulator tile
+    int64_t TRW = OW <= max_px ? max_px / OW : 0;
     if (TRW > OH) TRW = OH;
-    while (TRW > 1 && 2 * TRW > OH && (OH % (2 * TRW)) != 0 && (2 * (TRW - 1)) >= OH) TRW--;
-    auto lds_rows = [&](int64_t trw) { return (2 * trw - 1) * p->stride_h + (R - 1) * p->dil_h + 1; };
+    while (TRW > 1 && WPX * TRW > OH && (OH % (WPX * TRW)) != 0 && (WPX * (TRW - 1)) >= OH) TRW--;
+    auto lds_rows = [&](int64_t trw) { return (WPX * trw - 1) * p->stride_h + (R - 1) * p->dil_h + 1; };
     const int64_t LCOLS = (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1 > W + 2 * p->pad_w
                               ? (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1
                               : W + 2 * p->pad_w;
-    while (TRW > 1 && lds_rows(TRW) * LCOLS * 128 > 64 * 1024) TRW--;
+    while (TRW > 1 && lds_rows(TRW) * LCOLS * 144 > 72 * 1024) TRW--;   // two buffers of this size live in LDS
     const int64_t NT = TRW ? (TRW * OW + 15) / 16 : 0;
     const int64_t LROWS = lds_rows(TRW);
-    const bool mfma_ok = x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 128 == 0 &&
-                         W % 8 == 0 && TRW >= 1 && NT <= 7 && LROWS * LCOLS * 128 <= 64 * 1024 &&
+    // output channels per workgroup: 64 per pair of waves, up to 256
+    const int64_t WKO = K % 256 == 0 ? 4 : K % 128 == 0 ? 2 : 1;
+    const bool mfma_ok = x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 64 == 0 &&
+                         W % 8 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 144 <= 72 * 1024 &&
                          (uintptr_t)x->ptr % 16 == 0 && R * S <= 49;
     if (mfma_ok) {
-        const int64_t items = LROWS * (W / 8);
-        const int64_t items_per_wave = (items + 3) / 4;
+        const int64_t items = LROWS * (W / 8);                   // (row, 8 columns); a wave moves one item
+        const int64_t items_per_wave = (items + WPX * WKO - 1) / (WPX * WKO);
         std::ostringstream key;
-        key << "mfma|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16);
+        key << "mfma|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX;
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
@@ -81,7 +86,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                  << p->dil_w << (y->dtype == MJT_BFLOAT16 ? "_obf16" : "_of32");
             std::ostringstream src;
             src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo.str()
-                << "#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
+                << "#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
                 << "\n";
             src << embedded_source("conv_mfma.h") << "\n";
@@ -106,14 +111,14 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         int64_t pblocks = (numel(w) + 255) / 256;
         if (pblocks > 2048) pblocks = 2048;
         jit_launch(kp, (unsigned)pblocks, 1, 256, 0, pa);
-        const int64_t TR = 2 * TRW;
+        const int64_t TR = WPX * TRW;
         const int64_t tiles_r = (OH + TR - 1) / TR;
         const int64_t ptiles = N * tiles_r;
         const int64_t ptiles8 = (ptiles + 7) / 8 * 8;
-        const int64_t blocks = ptiles8 * (K / 128);
+        const int64_t blocks = ptiles8 * (K / (64 * WKO));
         MJT_CHECK(blocks < (int64_t(1) << 31), "conv: launch too large");
         std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(g_wpack), bits_of_ptr(y->ptr), (uint64_t)N};
-        jit_launch(k, (unsigned)blocks, 1, 256, 0, a);
+        jit_launch(k, (unsigned)blocks, 1, (unsigned)(64 * WPX * WKO), 0, a);
         return;
     }
 
