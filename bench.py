@@ -274,6 +274,33 @@ def wl_c5(L, lib, steps, warmup, with_cpu):
     return out
 
 
+def wl_copy(L, lib, steps, warmup, with_cpu):
+    """The library's device copy kernel on 256 MiB: the known-size launch that
+    calibrates the FETCH_SIZE / WRITE_SIZE counters (not part of the default run)."""
+    n = 256 << 20
+    dev = Dev(L)
+    bufs = [dev.empty(n) for _ in range(3)]
+    calls = [lambda a=bufs[i], b=bufs[(i + 1) % 3]: L.check(lib.mjt_d2d(a, b, n)) for i in range(3)]
+    ms, wall = time_calls(L, calls, steps, warmup)
+    dev.release()
+    return {"workload": "COPY device copy of 268435456 bytes (reads 268435456 B, writes 268435456 B)",
+            "kernel": L.last_kernel(), "dtype": "u8", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+            "roofline": roofline("hbm", 2 * n, ms)}
+
+
+# HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# runs of this file (KiB per dispatch), each scaled by what the same counter reads for the COPY workload
+# (FETCH_SIZE reads 131082 KiB for 262144 KiB fetched: factor 2.0; WRITE_SIZE reads 262144 KiB: factor 1.0).
+# Summaries: profiles/hbm_traffic_all_workloads.txt
+MEASURED_TRAFFIC = {
+    "C1": 2.0 * 65557.6 * 1024 + 64.0 * 1024,
+    "C2": 2.0 * 15635.8 * 1024 + 225838.1 * 1024,
+    "C3add": 2.0 * 65633.8 * 1024 + 41213.3 * 1024,
+    "C3max": 2.0 * 65614.6 * 1024 + 41223.5 * 1024,
+    "C4": 2.0 * 65584.3 * 1024 + 131072.0 * 1024,
+    "C5": 2.0 * 102488.2 * 1024 + 211400.0 * 1024,
+}
+
 WORKLOADS = {
     "C1": wl_c1,
     "C2": wl_c2,
@@ -281,7 +308,9 @@ WORKLOADS = {
     "C3max": lambda *a: wl_c3(*a, op="maximum"),
     "C4": wl_c4,
     "C5": wl_c5,
+    "COPY": wl_copy,
 }
+DEFAULT = ["C1", "C2", "C3add", "C3max", "C4", "C5"]
 
 
 def main():
@@ -299,11 +328,13 @@ def main():
     from jittor_amd import _lib as L
     lib = L.init(0)
     di = L.device_info()
-    only = [s for s in args.only.split(",") if s] or list(WORKLOADS)
+    only = [s for s in args.only.split(",") if s] or DEFAULT
     results = {}
     for name in only:
         try:
             results[name] = WORKLOADS[name](L, lib, args.steps, args.warmup, not args.no_cpu)
+            if name in MEASURED_TRAFFIC and "roofline" in results[name]:
+                results[name]["roofline"]["traffic"] = int(MEASURED_TRAFFIC[name])
         except L.MjtError as err:
             results[name] = {"error": str(err)}
         print("[bench] %s: %s" % (name, json.dumps(results[name])), file=sys.stderr, flush=True)

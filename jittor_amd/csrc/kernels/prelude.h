@@ -134,10 +134,27 @@ template <> struct mjt_mt<float16> { typedef float type; };
 template <> struct mjt_mt<bfloat16> { typedef float type; };
 #define MJT_M(T) typename mjt_mt<T>::type
 
+// exp in float, branch-free: n = rint(x*log2(e)); the reduced argument
+// x*log2(e) - n comes from two fused multiply-adds with log2(e) split in two
+// floats, so it carries one rounding of 2^-25; then the hardware exp2 and a
+// scaling by 2^n (about 1.5 ulp in all).  Beyond |x| = 150, where e^x and 2^x
+// are both 0 or inf, and for NaN, exp2(x) itself is the answer.
+__device__ __forceinline__ float mjt_expf(float x) {
+    const bool far = !(__builtin_fabsf(x) <= 150.0f);
+    const float n = __builtin_rintf(x * 0x1.715476p+0f);
+    const float f = __builtin_fmaf(x, 0x1.4ae0c0p-26f, __builtin_fmaf(x, 0x1.715476p+0f, -n));
+    return __builtin_ldexpf(__builtin_amdgcn_exp2f(far ? x : f), far ? 0 : (int)n);
+}
+// 1/d for finite d >= 1: hardware reciprocal and one Newton step (within 1 ulp)
+__device__ __forceinline__ float mjt_rcp_ge1(float d) {
+    const float r = __builtin_amdgcn_rcpf(d);
+    return __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+}
+
 #define MJT_MATH1(NAME, F32, F64) \
     __device__ __forceinline__ float mjt_m_##NAME(float x) { return F32(x); } \
     __device__ __forceinline__ double mjt_m_##NAME(double x) { return F64(x); }
-MJT_MATH1(log, logf, log) MJT_MATH1(exp, expf, exp) MJT_MATH1(sqrt, sqrtf, sqrt)
+MJT_MATH1(log, logf, log) MJT_MATH1(exp, mjt_expf, exp) MJT_MATH1(sqrt, sqrtf, sqrt)
 MJT_MATH1(round, roundf, round) MJT_MATH1(floor, floorf, floor) MJT_MATH1(ceil, ceilf, ceil)
 MJT_MATH1(sin, sinf, sin) MJT_MATH1(asin, asinf, asin) MJT_MATH1(sinh, sinhf, sinh)
 MJT_MATH1(asinh, asinhf, asinh) MJT_MATH1(tan, tanf, tan) MJT_MATH1(atan, atanf, atan)
@@ -203,7 +220,8 @@ MJT_UN(sigmoid) {
     M t = (M)(Tz(-x));
     M lim = (M)(Tz(mjt_is_f32<Tz>::v ? 30 : 300));
     M m = (lim < t) ? lim : t;
-    return Tz(1.0f / (1.0f + mjt_m_exp(m)));
+    if constexpr (mjt_is_f32<Tz>::v) return mjt_rcp_ge1(1.0f + mjt_expf(m));   // denominator in [1, 1+e^30]
+    else return Tz(1.0f / (1.0f + mjt_m_exp(m)));
 }
 
 #define MJT_BIN(NAME) template <class Tz, class X, class Y> __device__ __forceinline__ auto mjt_##NAME(X x, Y y)

@@ -120,10 +120,11 @@ void fused_impl(const mjt_fused_desc* d) {
     int64_t nvec = total / vec;
     auto env_int = [](const char* n, int d) { const char* v = getenv(n); return v && *v ? atoi(v) : d; };
     int block = env_int("MJT_FUSED_BLOCK", 256);
-    // measured on MI355X: one vector per lane and plain (cached) access is fastest for the chain
-    // workloads; more vectors per lane cost registers and occupancy
+    // measured on MI355X: one vector per lane is fastest for the chain workloads (more vectors per
+    // lane cost registers and occupancy); outputs too large to be re-read from cache are stored
+    // non-temporally, loads stay plain
     int unroll = env_int("MJT_FUSED_UNROLL", 1);
-    bool nt = env_int("MJT_FUSED_NT", 0) != 0;
+    int nt = env_int("MJT_FUSED_NT", total * maxsize >= (int64_t(32) << 20) ? 2 : 0);   // bit 0: non-temporal loads, bit 1: non-temporal stores
 
     // ---- parameter block layout ---------------------------------------------------
     // a[0] nvec | per merged axis: extent, divider | per var: pointer or scalar bits
@@ -276,8 +277,8 @@ void fused_impl(const mjt_fused_desc* d) {
 
         std::ostringstream frag;
         frag << "#define VEC " << vec << "\n#define UNROLL " << unroll << "\n#define index_t " << IT << "\n#define NPARAM "
-             << args.size() << "\n#define BLOCK " << block << "\n#define MJT_LD " << (nt ? "mjt_load_nt" : "mjt_load")
-             << "\n#define MJT_ST " << (nt ? "mjt_store_nt" : "mjt_store") << "\n";
+             << args.size() << "\n#define BLOCK " << block << "\n#define MJT_LD " << ((nt & 1) ? "mjt_load_nt" : "mjt_load")
+             << "\n#define MJT_ST " << ((nt & 2) ? "mjt_store_nt" : "mjt_store") << "\n";
         frag << "#define MJT_FUSED_SCALARS " << scal.str() << "\n";
         frag << "#define MJT_FUSED_DECODE " << dec.str() << "\n";
         frag << "#define MJT_FUSED_LOADS " << loads.str() << "\n";
