@@ -8,12 +8,18 @@
 // contribute 0 (overflow value 0 times w).
 //
 // All geometry is baked in by the host: C_, H_, W_, K_, R_, S_, OH_, OW_, SH, SW,
-// PH, PW, DH, DW, TRW (output rows per wave), NT (16-pixel tiles per wave), WKO
-// (groups of 64 output channels per workgroup), WPX (row groups per workgroup), LROWS x LCOLS (input tile held in LDS), ITEMS_PER_WAVE, Y_BF16.
+// PH, PW, DH, DW, WKO (groups of 64 output channels per workgroup), WPX (row
+// groups per workgroup), TRW / NT / LROWS (output rows per wave, 16-pixel tiles per
+// wave and input rows in LDS of a full tile), RPW (output rows a workgroup owns),
+// NFULL full tiles followed, when TAIL_TRW > 0, by one shorter tile (TAIL_TRW,
+// TAIL_NT, TAIL_LROWS), LCOLS, ITEMS_PER_WAVE, Y_BF16.
 //
 // Mapping.  v_mfma_f32_16x16x32_bf16 computes D[16 ko][16 px] += A[16 ko][32 c] *
-// B[32 c][16 px].  A workgroup of WPX*WKO waves owns 64*WKO output channels x
-// (WPX*TRW output rows) of one image; wave (wko, wpx) owns 64 channels x TRW rows =
+// B[32 c][16 px].  A workgroup of WPX*WKO waves owns 64*WKO output channels x RPW
+// consecutive output rows of one image and walks them tile by tile (WPX*TRW rows
+// each), so that the number of workgroups can match the number of compute units
+// whatever the row count, and the stores of one tile and the loads of the next
+// overlap the MFMAs.  Within a tile wave (wko, wpx) owns 64 channels x TRW rows =
 // 4 x NT accumulator tiles.  Channels are consumed 64 at a time:
 //   * the input rows the tile touches are staged through LDS as
 //     [row][col][64 c] (channel innermost) so that a B fragment is one 16-byte
@@ -21,16 +27,15 @@
 //     LDS write: a lane loads 8 columns of one channel, swaps halves with its
 //     neighbour lane so that it owns two channels x four columns, packs the two
 //     channels of a column into one dword, and the dwords of a wave fill whole
-//     128-byte rows; positions are padded to 144 bytes so that fragment reads
-//     are conflict-free.  The tile is double
-//     buffered: the loads of the next 64 channels are issued before the MFMAs of
-//     the current 64 and written to the other buffer after them (one barrier per
-//     channel block);
+//     128-byte rows; positions are padded to 144 bytes, which makes the address
+//     of a fragment linear in the tap.  The tile is double buffered across
+//     channel blocks and across tiles: the loads of the next block are issued
+//     before the MFMAs of the current one and written to the other buffer after
+//     them (one barrier per channel block);
 //   * A fragments come straight from the re-packed weights
 //     Wp[tap][c/64][k-step][ko][32 c] (1 KB contiguous per fragment, L2
 //     resident) and are loaded one step before the MFMAs that use them.
-// Halo cells (padding, rows outside the image) are zeroed once: they are the
-// same for every channel block.
+// Padding columns are zeroed once; rows outside the image are written as zeros.
 
 typedef __bf16 mjt_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float mjt_f32x4 __attribute__((ext_vector_type(4)));
@@ -45,10 +50,9 @@ struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as p
 #define NTHR (64 * NWAVES)
 #define MT 4
 #define TR (WPX * TRW)
-#define TILES_R ((OH_ + TR - 1) / TR)
+#define SPLITS ((OH_ + RPW - 1) / RPW)      // row ranges per image
 #define NCB (C_ / CB)
 #define GROUPS (W_ / 8)                 // groups of 8 columns
-#define ITEMS (LROWS * GROUPS)          // (row, column group); a wave moves the 64 channels of an item
 #define TILE_ELEMS (LROWS * LCOLS * PSTRIDE)
 
 // LDS tile: position (row, col) holds its 64 channels in 128 bytes followed by 16 bytes of padding.
@@ -61,72 +65,63 @@ __device__ __forceinline__ int mjt_lds_off(int pos, int chunk) {
     return pos * PSTRIDE + (chunk << 3);
 }
 
+template <int V> struct mjt_ic { static constexpr int v = V; };
+
 extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const unsigned short* __restrict__ xp = (const unsigned short*)p.a[0];
     const unsigned short* __restrict__ wp = (const unsigned short*)p.a[1];
     const int n_img = (int)(unsigned long long)p.a[3];
     __shared__ __attribute__((aligned(16))) unsigned short xs[2][TILE_ELEMS];
 
-    // tile id: the channel groups of one pixel tile are 8 workgroups apart, so
+    // range id: the channel groups of one row range are 8 workgroups apart, so
     // they land on the same XCD (workgroups go round-robin over 8 XCDs) and
     // share the input rows in that XCD's L2
     const int id = blockIdx.x;
     const int xcd = id & 7, j = id >> 3;
     const int kpart = j % (K_ / KO_WG);
-    const int ptile = (j / (K_ / KO_WG)) * 8 + xcd;
-    if (ptile >= n_img * TILES_R) return;
-    const int n = ptile / TILES_R;
-    const int r0 = (ptile % TILES_R) * TR;
+    const int range = (j / (K_ / KO_WG)) * 8 + xcd;
+    if (range >= n_img * SPLITS) return;
+    const int n = range / SPLITS;
+    const int row_begin = (range % SPLITS) * RPW;
+    const int row_end = row_begin + RPW < OH_ ? row_begin + RPW : OH_;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: what depends on it alone stays scalar
     const int wpx = wave % WPX, wko = wave / WPX;
     const int ko_base = kpart * KO_WG + wko * 64;
     const int l16 = lane & 15, lg = lane >> 4;
 
-    // zero both buffers once (halo cells stay zero)
+    // zero both buffers once (padding columns stay zero)
     for (int t = tid; t < 2 * TILE_ELEMS / 8; t += NTHR) ((mjt_u32x4v*)&xs[0][0])[t] = (mjt_u32x4v)(0u);
-
-    // per-lane pixel of each of the NT tiles
-    int bpos[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
-        int q = t * 16 + l16;
-        int r = q / OW_, col = q - r * OW_;
-        if (q >= TRW * OW_) { r = 0; col = 0; }
-        bpos[t] = ((wpx * TRW + r) * SH) * LCOLS + col * SW;
-    }
-
-    mjt_f32x4 acc[MT][NT];
-#pragma unroll
-    for (int m = 0; m < MT; m++)
-#pragma unroll
-        for (int t = 0; t < NT; t++) acc[m][t] = (mjt_f32x4)(0.0f);
 
     // staging: item = (tile row, group of 8 columns); a wave moves the 64 channels of an item, lane l
     // loading 16 bytes (8 columns) of channel l -- one scattered load per lane is what the address unit
     // is charged for, so it should be as wide as possible.  Adjacent lanes (channels 2k, 2k+1) then swap
     // halves so that each owns 4 columns of both channels, and write one dword (channel pair) per column.
-    const int ir0 = r0 * SH - PH;
     const int odd = lane & 1;
     mjt_u32x4v stage[ITEMS_PER_WAVE];
-    auto fetch = [&](int cb) {
+    const unsigned x_lane_off = (unsigned)lane * (H_ * W_ * 2);   // byte offset of the lane's channel
+    auto fetch = [&](int r0, int lrows, int cb) {            // input rows of the tile whose first output row is r0
+        const int ir0 = r0 * SH - PH;
 #pragma unroll
         for (int it = 0; it < ITEMS_PER_WAVE; it++) {
             const int item = it * NWAVES + wave;
             const int lr = item / GROUPS, g = item - lr * GROUPS;
             const int ir = ir0 + lr;
             mjt_u32x4v v = (mjt_u32x4v)(0u);
-            if (item < ITEMS && ir >= 0 && ir < H_)
-                v = *(const mjt_u32x4v*)(xp + (((size_t)n * C_ + cb * CB + lane) * H_ + ir) * W_ + g * 8);
+            if (lr < lrows && ir >= 0 && ir < H_) {
+                const char* base = (const char*)(xp + (((size_t)n * C_ + cb * CB) * H_ + ir) * W_ + g * 8);   // uniform
+                v = *(const mjt_u32x4v*)(base + x_lane_off);
+            }
             stage[it] = v;
         }
     };
-    auto commit = [&](int buf) {
+    const int commit_lane_off = (odd * 4 * PSTRIDE + (lane & ~1)) >> 1;   // in dwords: 4 columns on for odd lanes, channel pair
+    auto commit = [&](int lrows, int buf) {
 #pragma unroll
         for (int it = 0; it < ITEMS_PER_WAVE; it++) {
             const int item = it * NWAVES + wave;
             const int lr = item / GROUPS, g = item - lr * GROUPS;
-            const int ir = ir0 + lr;
             // even lane keeps its columns 0..3 and receives columns 0..3 of the odd lane; the odd lane
             // keeps columns 4..7 and receives columns 4..7 of the even lane
             const unsigned give0 = odd ? stage[it][0] : stage[it][2];
@@ -137,86 +132,129 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
             const unsigned mine1 = odd ? stage[it][3] : stage[it][1];
             const unsigned lo0 = odd ? got0 : mine0, hi0 = odd ? mine0 : got0;   // lo = even channel, hi = odd channel
             const unsigned lo1 = odd ? got1 : mine1, hi1 = odd ? mine1 : got1;
-            if (item < ITEMS && ir >= 0 && ir < H_) {
-                const int c = lane & ~1;                     // first channel of the pair
-                const int pos0 = lr * LCOLS + PW + g * 8 + odd * 4;
-                unsigned* dst = (unsigned*)&xs[buf][0];
-                dst[(mjt_lds_off(pos0 + 0, c >> 3) + (c & 7)) >> 1] = (lo0 & 0xffffu) | (hi0 << 16);
-                dst[(mjt_lds_off(pos0 + 1, c >> 3) + (c & 7)) >> 1] = (lo0 >> 16) | (hi0 & 0xffff0000u);
-                dst[(mjt_lds_off(pos0 + 2, c >> 3) + (c & 7)) >> 1] = (lo1 & 0xffffu) | (hi1 << 16);
-                dst[(mjt_lds_off(pos0 + 3, c >> 3) + (c & 7)) >> 1] = (lo1 >> 16) | (hi1 & 0xffff0000u);
+            if (lr < lrows) {                                // rows outside the image carry zeros
+                // uniform part of the address (row, column group, buffer) + the lane's part (column half, channel pair)
+                unsigned* dst = (unsigned*)&xs[buf][0] + ((lr * LCOLS + PW + g * 8) * PSTRIDE >> 1) + commit_lane_off;
+                dst[0 * (PSTRIDE >> 1)] = (lo0 & 0xffffu) | (hi0 << 16);
+                dst[1 * (PSTRIDE >> 1)] = (lo0 >> 16) | (hi0 & 0xffff0000u);
+                dst[2 * (PSTRIDE >> 1)] = (lo1 & 0xffffu) | (hi1 << 16);
+                dst[3 * (PSTRIDE >> 1)] = (lo1 >> 16) | (hi1 & 0xffff0000u);
             }
         }
     };
 
     // A fragments: Wp[step][ko][32 c], step = (tap * NCB + cb) * 2 + ks; 16 rows x 64 B per fragment
-    const unsigned short* __restrict__ wlane = wp + (size_t)(ko_base + l16) * 32 + lg * 8;
+    const unsigned a_lane_off = (unsigned)(((wko * 64 + l16) * 32 + lg * 8) * 2);   // bytes
     auto load_a = [&](mjt_bf16x8 (&a)[MT], int cb, int s) {
         const int tap = s >> 1, ks = s & 1;
-        const unsigned short* f = wlane + (size_t)((tap * NCB + cb) * 2 + ks) * (K_ * 32);
+        const char* f = (const char*)(wp + (size_t)((tap * NCB + cb) * 2 + ks) * (K_ * 32) + (size_t)kpart * KO_WG * 32);   // uniform
 #pragma unroll
-        for (int m = 0; m < MT; m++) a[m] = *(const mjt_bf16x8*)(f + m * 16 * 32);
-    };
-    auto compute = [&](const mjt_bf16x8 (&a)[MT], int s, int buf) {
-        const int tap = s >> 1, ks = s & 1;
-        const int kh = tap / S_, kw = tap - kh * S_;
-        const int tap_pos = kh * DH * LCOLS + kw * DW;
-        const unsigned short* tile = &xs[buf][0];
-        mjt_bf16x8 b[NT];
-#pragma unroll
-        for (int t = 0; t < NT; t++) b[t] = *(const mjt_bf16x8*)(tile + mjt_lds_off(bpos[t] + tap_pos, ks * 4 + lg));
-#pragma unroll
-        for (int t = 0; t < NT; t++)
-#pragma unroll
-            for (int m = 0; m < MT; m++)
-                acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[m], b[t], acc[m][t], 0, 0, 0);
+        for (int m = 0; m < MT; m++) a[m] = *(const mjt_bf16x8*)(f + a_lane_off + m * 16 * 32 * 2);
     };
 
     constexpr int STEPS = 2 * R_ * S_;            // steps per channel block (even)
     mjt_bf16x8 ring[2][MT];                       // weights of the next step are in flight during a step
-    load_a(ring[0], 0, 0);
-    fetch(0);
-    __syncthreads();                              // zero fill done
-    commit(0);
-    __syncthreads();
-    // two steps per iteration (the ring has two slots); the tap is a run-time value
-#pragma unroll 1
-    for (int g0 = 0; g0 < NCB * STEPS; g0 += 2) {
+    int buf = 0;                                  // LDS buffer that holds the current channel block
+
+    // One tile: TRW_ output rows per wave starting at r0, NT_ accumulator tiles per wave, LR_ input rows
+    // in LDS.  On entry its first channel block is in xs[buf] and its first A fragments are in ring[0];
+    // when another tile follows (next_lrows > 0) its first block and fragments are prepared the same way.
+    auto run_tile = [&](auto trw_c, auto nt_c, auto lr_c, const int r0, const int next_r0, const int next_lrows) {
+        constexpr int TRW_ = decltype(trw_c)::v, NT_ = decltype(nt_c)::v, LR_ = decltype(lr_c)::v;
+        // per-lane pixel of each of the NT_ tiles
+        unsigned baddr[NT_];                                 // byte address in a buffer of the fragment at tap (0,0), k-step 0
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
-            const int g = g0 + u;
-            const int cb = g / STEPS, st = g - cb * STEPS;
-            if (st == 0 && cb + 1 < NCB) fetch(cb + 1);      // in flight during this block's MFMAs
-            if (g + 1 < NCB * STEPS) load_a(ring[u ^ 1], (g + 1) / STEPS, (g + 1) % STEPS);
-            compute(ring[u], st, cb & 1);
-            if (st == STEPS - 1 && cb + 1 < NCB) {
-                commit((cb + 1) & 1);                        // the other buffer: nobody reads it now
-                __syncthreads();
+        for (int t = 0; t < NT_; t++) {
+            int q = t * 16 + l16;
+            int r = q / OW_, col = q - r * OW_;
+            if (q >= TRW_ * OW_) { r = 0; col = 0; }
+            baddr[t] = (unsigned)mjt_lds_off(((wpx * TRW_ + r) * SH) * LCOLS + col * SW, lg) * 2;
+        }
+        mjt_f32x4 acc[MT][NT_];
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int t = 0; t < NT_; t++) acc[m][t] = (mjt_f32x4)(0.0f);
+
+        auto compute = [&](const mjt_bf16x8 (&a)[MT], int s, int b_) {
+            const int tap = s >> 1, ks = s & 1;
+            const int kh = tap / S_, kw = tap - kh * S_;
+            const char* tile = (const char*)&xs[b_][0] + mjt_lds_off(kh * DH * LCOLS + kw * DW, ks * 4) * 2;   // uniform
+            mjt_bf16x8 b[NT_];
+#pragma unroll
+            for (int t = 0; t < NT_; t++) b[t] = *(const mjt_bf16x8*)(tile + baddr[t]);
+#pragma unroll
+            for (int t = 0; t < NT_; t++)
+#pragma unroll
+                for (int m = 0; m < MT; m++)
+                    acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[m], b[t], acc[m][t], 0, 0, 0);
+        };
+
+        // two steps per iteration (the ring has two slots); the tap is a run-time value
+#pragma unroll 1
+        for (int g0 = 0; g0 < NCB * STEPS; g0 += 2) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int g = g0 + u;
+                const int cb = g / STEPS, st = g - cb * STEPS;
+                const bool more = cb + 1 < NCB;
+                if (st == 0) {                                   // in flight during this block's MFMAs
+                    if (more) fetch(r0, LR_, cb + 1);
+                    else if (next_lrows) fetch(next_r0, next_lrows, 0);
+                }
+                if (g + 1 < NCB * STEPS) load_a(ring[u ^ 1], (g + 1) / STEPS, (g + 1) % STEPS);
+                else if (next_lrows) load_a(ring[u ^ 1], 0, 0);
+                compute(ring[u], st, buf);
+                if (st == STEPS - 1 && (more || next_lrows)) {
+                    commit(more ? LR_ : next_lrows, buf ^ 1);    // the other buffer: nobody reads it now
+                    __syncthreads();
+                    buf ^= 1;
+                }
             }
         }
-    }
 
-    // epilogue: lane holds D[ko = 4*(lane/16)+i][px = lane%16] of each tile
+        // epilogue: lane holds D[ko = 4*(lane/16)+i][px = lane%16] of each tile
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const int q = t * 16 + l16;
-        const int r = q / OW_, col = q - r * OW_;
-        const int orow = r0 + wpx * TRW + r;
-        if (q < TRW * OW_ && orow < OH_) {
+        for (int t = 0; t < NT_; t++) {
+            const int q = t * 16 + l16;
+            const int r = q / OW_, col = q - r * OW_;
+            const int orow = r0 + wpx * TRW_ + r;
+            if (q < TRW_ * OW_ && orow < row_end) {
 #pragma unroll
-            for (int m = 0; m < MT; m++)
+                for (int m = 0; m < MT; m++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int ko = ko_base + m * 16 + lg * 4 + i;
-                    const size_t o = (((size_t)n * K_ + ko) * OH_ + orow) * OW_ + col;
+                    for (int i = 0; i < 4; i++) {
+                        const int ko = ko_base + m * 16 + lg * 4 + i;
+                        const size_t o = (((size_t)n * K_ + ko) * OH_ + orow) * OW_ + col;
 #if Y_BF16
-                    ((unsigned short*)p.a[2])[o] = (unsigned short)(__float_as_uint(acc[m][t][i]) >> 16);
+                        ((unsigned short*)p.a[2])[o] = (unsigned short)(__float_as_uint(acc[m][t][i]) >> 16);
 #else
-                    ((float*)p.a[2])[o] = acc[m][t][i];
+                        ((float*)p.a[2])[o] = acc[m][t][i];
 #endif
-                }
+                    }
+            }
         }
+    };
+
+    // tiles of this workgroup: full tiles while they start inside the row range, then the short one
+    int nfull = (row_end - row_begin + TR - 1) / TR;
+    if (nfull > NFULL) nfull = NFULL;
+    const bool tail = TAIL_TRW > 0 && row_begin + NFULL * TR < row_end;
+    const int first_lrows = nfull ? LROWS : TAIL_LROWS;
+
+    load_a(ring[0], 0, 0);
+    fetch(row_begin, first_lrows, 0);
+    __syncthreads();                              // zero fill done
+    commit(first_lrows, 0);
+    __syncthreads();
+    for (int s = 0; s < nfull; s++) {
+        const int r0 = row_begin + s * TR;
+        const int next_lrows = s + 1 < nfull ? LROWS : tail ? TAIL_LROWS : 0;
+        run_tile(mjt_ic<TRW>(), mjt_ic<NT>(), mjt_ic<LROWS>(), r0, r0 + TR, next_lrows);
     }
+#if TAIL_TRW > 0
+    if (tail) run_tile(mjt_ic<TAIL_TRW>(), mjt_ic<TAIL_NT>(), mjt_ic<TAIL_LROWS>(), row_begin + NFULL * TR, 0, 0);
+#endif
 }
 
 // Weight re-pack: w[ko][c][kh][kw] -> Wp[tap][c/64][k-step][ko][32 c]

@@ -75,19 +75,49 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     if (mfma_ok) {
         const int64_t items = LROWS * (W / 8);                   // (row, 8 columns); a wave moves one item
         const int64_t items_per_wave = (items + WPX * WKO - 1) / (WPX * WKO);
+        // Rows per workgroup: a workgroup walks RPW output rows as NFULL tiles of TR rows plus one
+        // shorter tile.  Pick the RPW that minimises (rounds of workgroups over the compute units) x
+        // (accumulator tiles a workgroup computes, plus a per-tile overhead worth half a tile column).
+        const int64_t TR = WPX * TRW, KPARTS = K / (64 * WKO);
+        const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
+        auto tail_of = [&](int64_t rpw, int64_t* trw_t, int64_t* nt_t) {
+            const int64_t t = rpw % TR;
+            *trw_t = (t + WPX - 1) / WPX;
+            *nt_t = (*trw_t * OW + 15) / 16;
+        };
+        int64_t RPW = TR;
+        {
+            double best = 1e300;
+            for (int64_t r = TR; r <= OH || r == TR; r++) {
+                int64_t trw_t, nt_t;
+                tail_of(r, &trw_t, &nt_t);
+                const int64_t wgs = N * ((OH + r - 1) / r) * KPARTS;
+                const int64_t rounds = (wgs + cus - 1) / cus;
+                const int64_t ntiles = r / TR + (trw_t ? 1 : 0);
+                const double cost = (double)rounds * ((double)(r / TR) * NT + nt_t + 0.5 * ntiles);
+                if (cost < best - 1e-9) { best = cost; RPW = r; }
+            }
+            const char* e = getenv("MJT_CONV_RPW");
+            if (e && *e && atoi(e) >= TR) RPW = atoi(e);
+        }
+        int64_t TAIL_TRW, TAIL_NT;
+        tail_of(RPW, &TAIL_TRW, &TAIL_NT);
+        const int64_t NFULL = RPW / TR;
+        const int64_t TAIL_LROWS = TAIL_TRW ? lds_rows(TAIL_TRW) : 0;
         std::ostringstream key;
-        key << "mfma|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX;
+        key << "mfma|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX << "|" << RPW;
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
             std::ostringstream name;
             name << "mjt_conv_mfma_bf16_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s"
                  << p->stride_h << "x" << p->stride_w << "_p" << p->pad_h << "x" << p->pad_w << "_d" << p->dil_h << "x"
-                 << p->dil_w << (y->dtype == MJT_BFLOAT16 ? "_obf16" : "_of32");
+                 << p->dil_w << "_rows" << RPW << (y->dtype == MJT_BFLOAT16 ? "_obf16" : "_of32");
             std::ostringstream src;
             src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo.str()
                 << "#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
-                << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
+                << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
+                << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
                 << "\n";
             src << embedded_source("conv_mfma.h") << "\n";
             k = jit_get(src.str(), name.str());
@@ -111,11 +141,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         int64_t pblocks = (numel(w) + 255) / 256;
         if (pblocks > 2048) pblocks = 2048;
         jit_launch(kp, (unsigned)pblocks, 1, 256, 0, pa);
-        const int64_t TR = WPX * TRW;
-        const int64_t tiles_r = (OH + TR - 1) / TR;
-        const int64_t ptiles = N * tiles_r;
-        const int64_t ptiles8 = (ptiles + 7) / 8 * 8;
-        const int64_t blocks = ptiles8 * (K / (64 * WKO));
+        const int64_t ranges = N * ((OH + RPW - 1) / RPW);
+        const int64_t ranges8 = (ranges + 7) / 8 * 8;
+        const int64_t blocks = ranges8 * KPARTS;
         MJT_CHECK(blocks < (int64_t(1) << 31), "conv: launch too large");
         std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(g_wpack), bits_of_ptr(y->ptr), (uint64_t)N};
         jit_launch(k, (unsigned)blocks, 1, (unsigned)(64 * WPX * WKO), 0, a);
