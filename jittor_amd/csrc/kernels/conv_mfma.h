@@ -53,6 +53,7 @@ struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as p
 #define SPLITS ((OH_ + RPW - 1) / RPW)      // row ranges per image
 #define NCB (C_ / CB)
 #define GROUPS (W_ / 8)                 // groups of 8 columns
+#define SEGS ((GROUPS + 7) / 8)         // segments of 64 columns
 #define TILE_ELEMS (LROWS * LCOLS * PSTRIDE)
 
 // LDS tile: position (row, col) holds its 64 channels in 128 bytes followed by 16 bytes of padding.
@@ -66,6 +67,32 @@ __device__ __forceinline__ int mjt_lds_off(int pos, int chunk) {
 }
 
 template <int V> struct mjt_ic { static constexpr int v = V; };
+template <int I, int N, class F> __device__ __forceinline__ void mjt_static_for(F&& f) {
+    if constexpr (I < N) {
+        f(mjt_ic<I>());
+        mjt_static_for<I + 1, N>(f);
+    }
+}
+// byte offset inside the LDS tile of step s = (tap, k-step): row/column shift of the tap, 64 bytes per k-step
+__device__ constexpr int mjt_frag_off(int s) {
+    return ((((s >> 1) / S_) * DH * LCOLS + ((s >> 1) % S_) * DW) * PSTRIDE + (s & 1) * 32) * 2;
+}
+// value of lane ^ 1, ^ 2, ^ 4 through data-parallel-primitive moves (quad permutes; ^ 4 is a mirror
+// of each group of 8 lanes followed by a reversal inside each quad)
+__device__ __forceinline__ unsigned mjt_xor1(unsigned v) { return (unsigned)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xf, 0xf, true); }
+__device__ __forceinline__ unsigned mjt_xor2(unsigned v) { return (unsigned)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xf, 0xf, true); }
+__device__ __forceinline__ float mjt_xor1f(float v) { return __uint_as_float(mjt_xor1(__float_as_uint(v))); }
+__device__ __forceinline__ float mjt_xor2f(float v) { return __uint_as_float(mjt_xor2(__float_as_uint(v))); }
+__device__ __forceinline__ unsigned mjt_xor4(unsigned v) {
+    return (unsigned)__builtin_amdgcn_mov_dpp(__builtin_amdgcn_mov_dpp((int)v, 0x141, 0xf, 0xf, true), 0x1B, 0xf, 0xf, true);
+}
+template <int OFF> __device__ __forceinline__ void mjt_ds_read(mjt_u32x4v& dst, unsigned addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+// wait until at most N LDS operations issued after the one that fills x are outstanding (LDS returns in order)
+template <int N> __device__ __forceinline__ void mjt_lds_wait(mjt_u32x4v& x) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
+}
 
 extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const unsigned short* __restrict__ xp = (const unsigned short*)p.a[0];
@@ -90,55 +117,80 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const int wpx = wave % WPX, wko = wave / WPX;
     const int ko_base = kpart * KO_WG + wko * 64;
     const int l16 = lane & 15, lg = lane >> 4;
+    const unsigned xs_base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned short*)&xs[0][0];
 
     // zero both buffers once (padding columns stay zero)
     for (int t = tid; t < 2 * TILE_ELEMS / 8; t += NTHR) ((mjt_u32x4v*)&xs[0][0])[t] = (mjt_u32x4v)(0u);
 
-    // staging: item = (tile row, group of 8 columns); a wave moves the 64 channels of an item, lane l
-    // loading 16 bytes (8 columns) of channel l -- one scattered load per lane is what the address unit
-    // is charged for, so it should be as wide as possible.  Adjacent lanes (channels 2k, 2k+1) then swap
-    // halves so that each owns 4 columns of both channels, and write one dword (channel pair) per column.
-    const int odd = lane & 1;
+    // Staging.  An item is (tile row, segment of 64 columns, 8 channels); a wave moves one item per
+    // load: lane (g = lane / 8, r = lane % 8) loads the 16 bytes of columns 8g..8g+7 of channel r, so
+    // that a wave touches 8 cache lines per load instead of 64 (the address unit handles one line per
+    // cycle).  The 8 lanes of a column group then transpose their 8 channels x 8 columns among
+    // themselves with three butterfly exchanges (lane ^ 4, ^ 2, ^ 1; data-parallel-primitive moves,
+    // no LDS), after which lane r owns column 8g + r for the 8 channels in order: one 16-byte LDS
+    // write, at a lane stride of one position.
+    const int sg = lane >> 3, sr = lane & 7;
+    const bool b2 = lane & 4, b1 = lane & 2, b0 = lane & 1;
+    // byte selectors of v_perm_b32 (bytes 0-3 = second operand, 4-7 = first operand):
+    //   sel_t  what the lane gives away: the high halves of two dwords (even lane) or the low halves (odd lane)
+    //   sel_a  even lane: own low half | received low half << 16;  odd lane: received low half | own high half << 16
+    //   sel_b  even lane: own low half | received high half << 16; odd lane: received high half | own high half << 16
+    const unsigned sel_t = b0 ? 0x05040100u : 0x07060302u;
+    const unsigned sel_a = b0 ? 0x03020504u : 0x05040100u;
+    const unsigned sel_b = b0 ? 0x03020706u : 0x07060100u;
     mjt_u32x4v stage[ITEMS_PER_WAVE];
-    const unsigned x_lane_off = (unsigned)lane * (H_ * W_ * 2);   // byte offset of the lane's channel
+    const unsigned x_lane_off = (unsigned)sr * (H_ * W_ * 2);
+    auto item_of = [&](int it, int& lr, int& seg, int& cg) {
+        const int item = wave * ITEMS_PER_WAVE + it;
+        cg = item & 7;
+        const int rest = item >> 3;
+        lr = rest / SEGS;
+        seg = rest - lr * SEGS;
+    };
+    // The loads are unconditional (rows outside the image and idle lanes read a clamped address and
+    // are zeroed or skipped when written): a load under a branch would make every later wait for a
+    // weight fragment wait for all staging loads as well.
     auto fetch = [&](int r0, int lrows, int cb) {            // input rows of the tile whose first output row is r0
         const int ir0 = r0 * SH - PH;
 #pragma unroll
         for (int it = 0; it < ITEMS_PER_WAVE; it++) {
-            const int item = it * NWAVES + wave;
-            const int lr = item / GROUPS, g = item - lr * GROUPS;
-            const int ir = ir0 + lr;
-            mjt_u32x4v v = (mjt_u32x4v)(0u);
-            if (lr < lrows && ir >= 0 && ir < H_) {
-                const char* base = (const char*)(xp + (((size_t)n * C_ + cb * CB) * H_ + ir) * W_ + g * 8);   // uniform
-                v = *(const mjt_u32x4v*)(base + x_lane_off);
-            }
-            stage[it] = v;
+            int lr, seg, cg;
+            item_of(it, lr, seg, cg);
+            int ir = ir0 + (lr < lrows ? lr : lrows - 1);
+            ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
+            const char* base = (const char*)(xp + (((size_t)n * C_ + cb * CB + cg * 8) * H_ + ir) * W_);   // uniform
+            int grp = seg * 8 + sg;
+            grp = grp < GROUPS ? grp : GROUPS - 1;
+            stage[it] = *(const mjt_u32x4v*)(base + x_lane_off + (unsigned)grp * 16);
         }
     };
-    const int commit_lane_off = (odd * 4 * PSTRIDE + (lane & ~1)) >> 1;   // in dwords: 4 columns on for odd lanes, channel pair
-    auto commit = [&](int lrows, int buf) {
+    auto commit = [&](int r0, int lrows, int buf) {
+        const int ir0 = r0 * SH - PH;
 #pragma unroll
         for (int it = 0; it < ITEMS_PER_WAVE; it++) {
-            const int item = it * NWAVES + wave;
-            const int lr = item / GROUPS, g = item - lr * GROUPS;
-            // even lane keeps its columns 0..3 and receives columns 0..3 of the odd lane; the odd lane
-            // keeps columns 4..7 and receives columns 4..7 of the even lane
-            const unsigned give0 = odd ? stage[it][0] : stage[it][2];
-            const unsigned give1 = odd ? stage[it][1] : stage[it][3];
-            const unsigned got0 = (unsigned)__shfl_xor((int)give0, 1, 64);
-            const unsigned got1 = (unsigned)__shfl_xor((int)give1, 1, 64);
-            const unsigned mine0 = odd ? stage[it][2] : stage[it][0];
-            const unsigned mine1 = odd ? stage[it][3] : stage[it][1];
-            const unsigned lo0 = odd ? got0 : mine0, hi0 = odd ? mine0 : got0;   // lo = even channel, hi = odd channel
-            const unsigned lo1 = odd ? got1 : mine1, hi1 = odd ? mine1 : got1;
-            if (lr < lrows) {                                // rows outside the image carry zeros
-                // uniform part of the address (row, column group, buffer) + the lane's part (column half, channel pair)
-                unsigned* dst = (unsigned*)&xs[buf][0] + ((lr * LCOLS + PW + g * 8) * PSTRIDE >> 1) + commit_lane_off;
-                dst[0 * (PSTRIDE >> 1)] = (lo0 & 0xffffu) | (hi0 << 16);
-                dst[1 * (PSTRIDE >> 1)] = (lo0 >> 16) | (hi0 & 0xffff0000u);
-                dst[2 * (PSTRIDE >> 1)] = (lo1 & 0xffffu) | (hi1 << 16);
-                dst[3 * (PSTRIDE >> 1)] = (lo1 >> 16) | (hi1 & 0xffff0000u);
+            int lr, seg, cg;
+            item_of(it, lr, seg, cg);
+            mjt_u32x4v d = stage[it];                        // d[k] = columns 2k (low half), 2k+1 (high half) of channel r
+            if (ir0 + lr < 0 || ir0 + lr >= H_) d = (mjt_u32x4v)(0u);   // uniform: a row outside the image
+            // lane ^ 4: keep one half of the columns, get the same half from the channel 4 away
+            const unsigned g0 = mjt_xor4(b2 ? d[0] : d[2]), g1 = mjt_xor4(b2 ? d[1] : d[3]);
+            const unsigned a0 = b2 ? g0 : d[0], a1 = b2 ? g1 : d[1];      // channel r & 3:       column pairs 0, 1 of the half
+            const unsigned a2 = b2 ? d[2] : g0, a3 = b2 ? d[3] : g1;      // channel (r & 3) + 4
+            // lane ^ 2: keep one column pair, get it from the channel 2 away
+            const unsigned h0 = mjt_xor2(b1 ? a0 : a1), h1 = mjt_xor2(b1 ? a2 : a3);
+            const unsigned c0 = b1 ? h0 : a0, c1 = b1 ? a1 : h0;          // channels q, q+2 (q = r & 1), one column pair
+            const unsigned c2 = b1 ? h1 : a2, c3 = b1 ? a3 : h1;          // channels q+4, q+6
+            // lane ^ 1: keep one column, get it from the neighbouring channels (two 16-bit values per
+            // move; byte permutes with per-lane selectors keep this free of branches)
+            const unsigned s0 = mjt_xor1(__builtin_amdgcn_perm(c1, c0, sel_t)), s1 = mjt_xor1(__builtin_amdgcn_perm(c3, c2, sel_t));
+            mjt_u32x4v f;                                    // channels (0,1) (2,3) (4,5) (6,7) of column 8g + r
+            f[0] = __builtin_amdgcn_perm(s0, c0, sel_a);
+            f[1] = __builtin_amdgcn_perm(s0, c1, sel_b);
+            f[2] = __builtin_amdgcn_perm(s1, c2, sel_a);
+            f[3] = __builtin_amdgcn_perm(s1, c3, sel_b);
+            if (lr < lrows && seg * 8 + sg < GROUPS) {       // rows outside the image carry zeros
+                unsigned short* dst = &xs[buf][0] + mjt_lds_off(lr * LCOLS + PW + seg * 64, cg) + lane * PSTRIDE;
+                *(mjt_u32x4v*)dst = f;
             }
         }
     };
@@ -152,6 +204,13 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
         for (int m = 0; m < MT; m++) a[m] = *(const mjt_bf16x8*)(f + a_lane_off + m * 16 * 32 * 2);
     };
 
+#if DBG & 512
+    int tsn = 0;
+    __shared__ unsigned long long tsl[NWAVES][256];
+#define MJT_TS() do { if (lane == 0 && tsn < 256) tsl[wave][tsn] = __builtin_readcyclecounter(); tsn++; } while (0)
+#else
+#define MJT_TS() do {} while (0)
+#endif
     constexpr int STEPS = 2 * R_ * S_;            // steps per channel block (even)
     mjt_bf16x8 ring[2][MT];                       // weights of the next step are in flight during a step
     int buf = 0;                                  // LDS buffer that holds the current channel block
@@ -162,13 +221,13 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     auto run_tile = [&](auto trw_c, auto nt_c, auto lr_c, const int r0, const int next_r0, const int next_lrows) {
         constexpr int TRW_ = decltype(trw_c)::v, NT_ = decltype(nt_c)::v, LR_ = decltype(lr_c)::v;
         // per-lane pixel of each of the NT_ tiles
-        unsigned baddr[NT_];                                 // byte address in a buffer of the fragment at tap (0,0), k-step 0
+        unsigned baddr[NT_];                                 // LDS byte address of the fragment at tap (0,0), k-step 0, in the current buffer
 #pragma unroll
         for (int t = 0; t < NT_; t++) {
             int q = t * 16 + l16;
             int r = q / OW_, col = q - r * OW_;
             if (q >= TRW_ * OW_) { r = 0; col = 0; }
-            baddr[t] = (unsigned)mjt_lds_off(((wpx * TRW_ + r) * SH) * LCOLS + col * SW, lg) * 2;
+            baddr[t] = xs_base + (unsigned)(buf * TILE_ELEMS * 2) + (unsigned)mjt_lds_off(((wpx * TRW_ + r) * SH) * LCOLS + col * SW, lg) * 2;
         }
         mjt_f32x4 acc[MT][NT_];
 #pragma unroll
@@ -176,50 +235,110 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
 #pragma unroll
             for (int t = 0; t < NT_; t++) acc[m][t] = (mjt_f32x4)(0.0f);
 
-        auto compute = [&](const mjt_bf16x8 (&a)[MT], int s, int b_) {
-            const int tap = s >> 1, ks = s & 1;
-            const int kh = tap / S_, kw = tap - kh * S_;
-            const char* tile = (const char*)&xs[b_][0] + mjt_lds_off(kh * DH * LCOLS + kw * DW, ks * 4) * 2;   // uniform
-            mjt_bf16x8 b[NT_];
-#pragma unroll
-            for (int t = 0; t < NT_; t++) b[t] = *(const mjt_bf16x8*)(tile + baddr[t]);
-#pragma unroll
-            for (int t = 0; t < NT_; t++)
-#pragma unroll
-                for (int m = 0; m < MT; m++)
-                    acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[m], b[t], acc[m][t], 0, 0, 0);
-        };
-
-        // two steps per iteration (the ring has two slots); the tap is a run-time value
+        // Main loop.  Per channel block the STEPS x NT_ B fragments form one stream; fragment f is
+        // requested BQ_DIST fragments before the four MFMAs that use it (a ring of BQ_DIST + 1
+        // registers), so the LDS latency hides behind 4 * BQ_DIST MFMAs of this wave.  The reads and
+        // the waits for them are written out so that this order is what runs: tap and k-step are
+        // compile-time here and fold into the offset field of the read.
+        constexpr int NF = STEPS * NT_;
+        mjt_u32x4v bq[BQ_DIST + 1];
 #pragma unroll 1
-        for (int g0 = 0; g0 < NCB * STEPS; g0 += 2) {
-#pragma unroll
-            for (int u = 0; u < 2; u++) {
-                const int g = g0 + u;
-                const int cb = g / STEPS, st = g - cb * STEPS;
-                const bool more = cb + 1 < NCB;
-                if (st == 0) {                                   // in flight during this block's MFMAs
-                    if (more) fetch(r0, LR_, cb + 1);
+        for (int cb = 0; cb < NCB; cb++) {
+            const bool more = cb + 1 < NCB;
+            MJT_TS();
+            mjt_static_for<0, BQ_DIST>([&](auto fc) {
+                constexpr int f = decltype(fc)::v;
+                mjt_ds_read<mjt_frag_off(f / NT_)>(bq[f % (BQ_DIST + 1)], baddr[f % NT_]);
+            });
+            mjt_static_for<0, STEPS>([&](auto sc) {
+                constexpr int st = decltype(sc)::v;
+#if !(DBG & 1)
+                if (st + 1 < STEPS) load_a(ring[(st + 1) & 1], cb, st + 1);
+                else if (more) load_a(ring[0], cb + 1, 0);
+                else if (next_lrows) load_a(ring[0], 0, 0);
+#endif
+#if !(DBG & (2 | 16))
+                if (st == FETCH_STEP) {                          // in flight during this block's MFMAs; after the weight loads,
+                    if (more) fetch(r0, LR_, cb + 1);            // so that the wait for those does not include these
                     else if (next_lrows) fetch(next_r0, next_lrows, 0);
                 }
-                if (g + 1 < NCB * STEPS) load_a(ring[u ^ 1], (g + 1) / STEPS, (g + 1) % STEPS);
-                else if (next_lrows) load_a(ring[u ^ 1], 0, 0);
-                compute(ring[u], st, buf);
-                if (st == STEPS - 1 && (more || next_lrows)) {
-                    commit(more ? LR_ : next_lrows, buf ^ 1);    // the other buffer: nobody reads it now
-                    __syncthreads();
-                    buf ^= 1;
-                }
+#endif
+                mjt_static_for<0, NT_>([&](auto tc) {
+                    constexpr int t = decltype(tc)::v;
+                    constexpr int f = st * NT_ + t;
+                    if constexpr (f + BQ_DIST < NF && !(DBG & 8))
+                        mjt_ds_read<mjt_frag_off((f + BQ_DIST) / NT_)>(bq[(f + BQ_DIST) % (BQ_DIST + 1)], baddr[(f + BQ_DIST) % NT_]);
+                    mjt_lds_wait<(DBG & 8) ? 0 : (NF - 1 - f < BQ_DIST ? NF - 1 - f : BQ_DIST)>(bq[f % (BQ_DIST + 1)]);
+                    const mjt_bf16x8 b = __builtin_bit_cast(mjt_bf16x8, bq[f % (BQ_DIST + 1)]);
+#pragma unroll
+                    for (int m = 0; m < MT; m++)
+                        acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[st & 1][m], b, acc[m][t], 0, 0, 0);
+                });
+                if (st == 0 || st == 1 || st == 2 || st == 3 || st == 8 || st == 17) MJT_TS();
+            });
+            if (more || next_lrows) {
+#if !(DBG & (2 | 32))
+                commit(more ? r0 : next_r0, more ? LR_ : next_lrows, buf ^ 1);        // the other buffer: nobody reads it now
+#endif
+                MJT_TS();
+#if !(DBG & (2 | 64))
+                __syncthreads();
+#endif
+                MJT_TS();
+                buf ^= 1;
+#pragma unroll
+                for (int t = 0; t < NT_; t++) baddr[t] += buf ? (unsigned)(TILE_ELEMS * 2) : (unsigned)(-(TILE_ELEMS * 2));
             }
         }
 
         // epilogue: lane holds D[ko = 4*(lane/16)+i][px = lane%16] of each tile
+#if OW_ % 4 == 0
+        // The four lanes of a quad (4 pixels x 4 channels) transpose among themselves, after which lane j
+        // of the quad owns channel 4*(lane/16)+j for the quad's 4 consecutive pixels: one 16-byte (or
+        // 8-byte bfloat16) store instead of four scattered 4-byte stores.  Four pixels never straddle
+        // an output row because OW is a multiple of 4.
+        const int qj = lane & 3;
+#pragma unroll
+        for (int t = 0; t < NT_; t++) {
+            const int q0 = t * 16 + (l16 & ~3);
+            const int r = q0 / OW_, col = q0 - r * OW_;
+            const int orow = r0 + wpx * TRW_ + r;
+            const bool ok = q0 < TRW_ * OW_ && orow < row_end && (!(DBG & 4) || acc[0][t][0] == 123.456f);
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const mjt_f32x4 v = acc[m][t];
+                // lane ^ 1: rows (0,1) and (2,3) trade pixels
+                const float g0 = mjt_xor1f(b0 ? v[0] : v[1]), g1 = mjt_xor1f(b0 ? v[2] : v[3]);
+                const float a0 = b0 ? g0 : v[0], a1 = b0 ? v[1] : g0;     // row (j & 1):     pixel pair of this lane pair
+                const float a2 = b0 ? g1 : v[2], a3 = b0 ? v[3] : g1;     // row (j & 1) + 2
+                // lane ^ 2: row pairs trade pixel pairs
+                const float h0 = mjt_xor2f(b1 ? a0 : a2), h1 = mjt_xor2f(b1 ? a1 : a3);
+                mjt_f32x4 y4;                                             // row j, pixels 0..3 of the quad
+                y4[0] = b1 ? h0 : a0;
+                y4[1] = b1 ? h1 : a1;
+                y4[2] = b1 ? a2 : h0;
+                y4[3] = b1 ? a3 : h1;
+                if (ok) {
+                    const int ko = ko_base + m * 16 + lg * 4 + qj;
+                    const size_t o = (((size_t)n * K_ + ko) * OH_ + orow) * OW_ + col;
+#if Y_BF16
+                    mjt_u32x2 pk;
+                    pk[0] = (__float_as_uint(y4[0]) >> 16) | (__float_as_uint(y4[1]) & 0xffff0000u);
+                    pk[1] = (__float_as_uint(y4[2]) >> 16) | (__float_as_uint(y4[3]) & 0xffff0000u);
+                    *(mjt_u32x2*)((unsigned short*)p.a[2] + o) = pk;
+#else
+                    *(mjt_f32x4*)((float*)p.a[2] + o) = y4;
+#endif
+                }
+            }
+        }
+#else
 #pragma unroll
         for (int t = 0; t < NT_; t++) {
             const int q = t * 16 + l16;
             const int r = q / OW_, col = q - r * OW_;
             const int orow = r0 + wpx * TRW_ + r;
-            if (q < TRW_ * OW_ && orow < row_end) {
+            if (q < TRW_ * OW_ && orow < row_end && (!(DBG & 4) || acc[0][t][0] == 123.456f)) {
 #pragma unroll
                 for (int m = 0; m < MT; m++)
 #pragma unroll
@@ -234,6 +353,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
                     }
             }
         }
+#endif
     };
 
     // tiles of this workgroup: full tiles while they start inside the row range, then the short one
@@ -245,7 +365,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     load_a(ring[0], 0, 0);
     fetch(row_begin, first_lrows, 0);
     __syncthreads();                              // zero fill done
-    commit(first_lrows, 0);
+    commit(row_begin, first_lrows, 0);
     __syncthreads();
     for (int s = 0; s < nfull; s++) {
         const int r0 = row_begin + s * TR;
@@ -254,6 +374,10 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     }
 #if TAIL_TRW > 0
     if (tail) run_tile(mjt_ic<TAIL_TRW>(), mjt_ic<TAIL_NT>(), mjt_ic<TAIL_LROWS>(), row_begin + NFULL * TR, 0, 0);
+#endif
+#if DBG & 512
+    __syncthreads();
+    if (blockIdx.x == 8) for (int i = tid; i < NWAVES * 256; i += NTHR) ((unsigned long long*)p.a[2])[i] = tsl[i >> 8][i & 255];
 #endif
 }
 

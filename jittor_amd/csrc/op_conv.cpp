@@ -71,9 +71,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t WKO = K % 256 == 0 ? 4 : K % 128 == 0 ? 2 : 1;
     const bool mfma_ok = x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 64 == 0 &&
                          W % 8 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 144 <= 72 * 1024 &&
-                         (uintptr_t)x->ptr % 16 == 0 && R * S <= 49;
+                         (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49;
     if (mfma_ok) {
-        const int64_t items = LROWS * (W / 8);                   // (row, 8 columns); a wave moves one item
+        const int64_t items = LROWS * ((W / 8 + 7) / 8) * 8;     // (row, 64 columns, 8 channels); a wave moves one item per load
         const int64_t items_per_wave = (items + WPX * WKO - 1) / (WPX * WKO);
         // Rows per workgroup: a workgroup walks RPW output rows as NFULL tiles of TR rows plus one
         // shorter tile.  Pick the RPW that minimises (rounds of workgroups over the compute units) x
@@ -104,8 +104,11 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         tail_of(RPW, &TAIL_TRW, &TAIL_NT);
         const int64_t NFULL = RPW / TR;
         const int64_t TAIL_LROWS = TAIL_TRW ? lds_rows(TAIL_TRW) : 0;
+        const char* bq_env = getenv("MJT_CONV_BQ");
+        const int BQ = bq_env && *bq_env ? atoi(bq_env) : 3;   // B fragments requested ahead of use
+        const int DBG = getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0;
         std::ostringstream key;
-        key << "mfma|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX << "|" << RPW;
+        key << "mfma|" << (getenv("MJT_CONV_FS") ? getenv("MJT_CONV_FS") : "") << "|" << DBG << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX << "|" << RPW;
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
@@ -117,7 +120,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo.str()
                 << "#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
-                << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
+                << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS << "\n#define FETCH_STEP " << (getenv("MJT_CONV_FS") ? atoi(getenv("MJT_CONV_FS")) : 0) << "\n#define DBG " << DBG << "\n#define BQ_DIST " << BQ << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
                 << "\n";
             src << embedded_source("conv_mfma.h") << "\n";
             k = jit_get(src.str(), name.str());
