@@ -45,10 +45,9 @@ typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
 struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as pointers: global address space)
 
 #define CB 64
-#define KO_WG (64 * WKO)
+#define KO_WG (16 * MT * WKO)
 #define NWAVES (WPX * WKO)
 #define NTHR (64 * NWAVES)
-#define MT 4
 #define TR (WPX * TRW)
 #define SPLITS ((OH_ + RPW - 1) / RPW)      // row ranges per image
 #define NCB (C_ / CB)
@@ -115,7 +114,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: what depends on it alone stays scalar
     const int wpx = wave % WPX, wko = wave / WPX;
-    const int ko_base = kpart * KO_WG + wko * 64;
+    const int ko_base = kpart * KO_WG + wko * (16 * MT);
     const int l16 = lane & 15, lg = lane >> 4;
     const unsigned xs_base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned short*)&xs[0][0];
 
@@ -139,6 +138,10 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const unsigned sel_a = b0 ? 0x03020504u : 0x05040100u;
     const unsigned sel_b = b0 ? 0x03020706u : 0x07060100u;
     mjt_u32x4v stage[ITEMS_PER_WAVE];
+    // buffer descriptors (base, size in bytes): addresses are a scalar offset plus a 32-bit lane offset,
+    // so no per-item 64-bit address lives in vector registers
+    const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(xp + (size_t)n * C_ * H_ * W_), 0, C_ * H_ * W_ * 2, 0x00020000);
     const unsigned x_lane_off = (unsigned)sr * (H_ * W_ * 2);
     auto item_of = [&](int it, int& lr, int& seg, int& cg) {
         const int item = wave * ITEMS_PER_WAVE + it;
@@ -158,10 +161,10 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
             item_of(it, lr, seg, cg);
             int ir = ir0 + (lr < lrows ? lr : lrows - 1);
             ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
-            const char* base = (const char*)(xp + (((size_t)n * C_ + cb * CB + cg * 8) * H_ + ir) * W_);   // uniform
+            const int soff = (((cb * CB + cg * 8) * H_ + ir) * W_) * 2;     // uniform: channel group and row inside the image
             int grp = seg * 8 + sg;
             grp = grp < GROUPS ? grp : GROUPS - 1;
-            stage[it] = *(const mjt_u32x4v*)(base + x_lane_off + (unsigned)grp * 16);
+            stage[it] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)(x_lane_off + (unsigned)grp * 16), soff, 0);
         }
     };
     auto commit = [&](int r0, int lrows, int buf) {
@@ -196,12 +199,15 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     };
 
     // A fragments: Wp[step][ko][32 c], step = (tap * NCB + cb) * 2 + ks; 16 rows x 64 B per fragment
-    const unsigned a_lane_off = (unsigned)(((wko * 64 + l16) * 32 + lg * 8) * 2);   // bytes
+    const unsigned a_lane_off = (unsigned)(((wko * (16 * MT) + l16) * 32 + lg * 8) * 2);   // bytes
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(wp + (size_t)kpart * KO_WG * 32), 0, (R_ * S_ * C_ * K_ - kpart * KO_WG * 32) * 2, 0x00020000);
     auto load_a = [&](mjt_bf16x8 (&a)[MT], int cb, int s) {
         const int tap = s >> 1, ks = s & 1;
-        const char* f = (const char*)(wp + (size_t)((tap * NCB + cb) * 2 + ks) * (K_ * 32) + (size_t)kpart * KO_WG * 32);   // uniform
+        const int soff = ((tap * NCB + cb) * 2 + ks) * (K_ * 32 * 2);   // uniform
 #pragma unroll
-        for (int m = 0; m < MT; m++) a[m] = *(const mjt_bf16x8*)(f + a_lane_off + m * 16 * 32 * 2);
+        for (int m = 0; m < MT; m++)
+            a[m] = __builtin_bit_cast(mjt_bf16x8, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)a_lane_off + (m & 3) * 1024, soff + (m >> 2) * 4096, 0));
     };
 
 #if DBG & 512

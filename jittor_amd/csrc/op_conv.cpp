@@ -68,7 +68,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t NT = TRW ? (TRW * OW + 15) / 16 : 0;
     const int64_t LROWS = lds_rows(TRW);
     // output channels per workgroup: 64 per pair of waves, up to 256
-    const int64_t WKO = K % 256 == 0 ? 4 : K % 128 == 0 ? 2 : 1;
+    // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
+    const int64_t MT = getenv("MJT_CONV_MT") ? atoi(getenv("MJT_CONV_MT")) : 4;
+    const int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
     const bool mfma_ok = x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 64 == 0 &&
                          W % 8 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 144 <= 72 * 1024 &&
                          (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49;
@@ -78,7 +80,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         // Rows per workgroup: a workgroup walks RPW output rows as NFULL tiles of TR rows plus one
         // shorter tile.  Pick the RPW that minimises (rounds of workgroups over the compute units) x
         // (accumulator tiles a workgroup computes, plus a per-tile overhead worth half a tile column).
-        const int64_t TR = WPX * TRW, KPARTS = K / (64 * WKO);
+        const int64_t TR = WPX * TRW, KPARTS = K / (16 * MT * WKO);
         const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
         auto tail_of = [&](int64_t rpw, int64_t* trw_t, int64_t* nt_t) {
             const int64_t t = rpw % TR;
@@ -108,7 +110,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int BQ = bq_env && *bq_env ? atoi(bq_env) : 3;   // B fragments requested ahead of use
         const int DBG = getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0;
         std::ostringstream key;
-        key << "mfma|" << (getenv("MJT_CONV_FS") ? getenv("MJT_CONV_FS") : "") << "|" << DBG << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX << "|" << RPW;
+        key << "mfma|" << (getenv("MJT_CONV_FS") ? getenv("MJT_CONV_FS") : "") << "|" << DBG << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT;
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
@@ -118,7 +120,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                  << p->dil_w << "_rows" << RPW << (y->dtype == MJT_BFLOAT16 ? "_obf16" : "_of32");
             std::ostringstream src;
             src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo.str()
-                << "#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
+                << "#define MT " << MT << "\n#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
                 << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS << "\n#define FETCH_STEP " << (getenv("MJT_CONV_FS") ? atoi(getenv("MJT_CONV_FS")) : 0) << "\n#define DBG " << DBG << "\n#define BQ_DIST " << BQ << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
                 << "\n";
