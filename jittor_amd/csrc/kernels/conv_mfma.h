@@ -210,13 +210,6 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
             a[m] = __builtin_bit_cast(mjt_bf16x8, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)a_lane_off + (m & 3) * 1024, soff + (m >> 2) * 4096, 0));
     };
 
-#if DBG & 512
-    int tsn = 0;
-    __shared__ unsigned long long tsl[NWAVES][256];
-#define MJT_TS() do { if (lane == 0 && tsn < 256) tsl[wave][tsn] = __builtin_readcyclecounter(); tsn++; } while (0)
-#else
-#define MJT_TS() do {} while (0)
-#endif
     constexpr int STEPS = 2 * R_ * S_;            // steps per channel block (even)
     mjt_bf16x8 ring[2][MT];                       // weights of the next step are in flight during a step
     int buf = 0;                                  // LDS buffer that holds the current channel block
@@ -251,46 +244,34 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
 #pragma unroll 1
         for (int cb = 0; cb < NCB; cb++) {
             const bool more = cb + 1 < NCB;
-            MJT_TS();
             mjt_static_for<0, BQ_DIST>([&](auto fc) {
                 constexpr int f = decltype(fc)::v;
                 mjt_ds_read<mjt_frag_off(f / NT_)>(bq[f % (BQ_DIST + 1)], baddr[f % NT_]);
             });
             mjt_static_for<0, STEPS>([&](auto sc) {
                 constexpr int st = decltype(sc)::v;
-#if !(DBG & 1)
                 if (st + 1 < STEPS) load_a(ring[(st + 1) & 1], cb, st + 1);
                 else if (more) load_a(ring[0], cb + 1, 0);
                 else if (next_lrows) load_a(ring[0], 0, 0);
-#endif
-#if !(DBG & (2 | 16))
-                if (st == FETCH_STEP) {                          // in flight during this block's MFMAs; after the weight loads,
+                if (st == 0) {                                   // in flight during this block's MFMAs; after the weight loads,
                     if (more) fetch(r0, LR_, cb + 1);            // so that the wait for those does not include these
                     else if (next_lrows) fetch(next_r0, next_lrows, 0);
                 }
-#endif
                 mjt_static_for<0, NT_>([&](auto tc) {
                     constexpr int t = decltype(tc)::v;
                     constexpr int f = st * NT_ + t;
-                    if constexpr (f + BQ_DIST < NF && !(DBG & 8))
+                    if constexpr (f + BQ_DIST < NF)
                         mjt_ds_read<mjt_frag_off((f + BQ_DIST) / NT_)>(bq[(f + BQ_DIST) % (BQ_DIST + 1)], baddr[(f + BQ_DIST) % NT_]);
-                    mjt_lds_wait<(DBG & 8) ? 0 : (NF - 1 - f < BQ_DIST ? NF - 1 - f : BQ_DIST)>(bq[f % (BQ_DIST + 1)]);
+                    mjt_lds_wait<(NF - 1 - f < BQ_DIST ? NF - 1 - f : BQ_DIST)>(bq[f % (BQ_DIST + 1)]);
                     const mjt_bf16x8 b = __builtin_bit_cast(mjt_bf16x8, bq[f % (BQ_DIST + 1)]);
 #pragma unroll
                     for (int m = 0; m < MT; m++)
                         acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[st & 1][m], b, acc[m][t], 0, 0, 0);
                 });
-                if (st == 0 || st == 1 || st == 2 || st == 3 || st == 8 || st == 17) MJT_TS();
             });
             if (more || next_lrows) {
-#if !(DBG & (2 | 32))
                 commit(more ? r0 : next_r0, more ? LR_ : next_lrows, buf ^ 1);        // the other buffer: nobody reads it now
-#endif
-                MJT_TS();
-#if !(DBG & (2 | 64))
                 __syncthreads();
-#endif
-                MJT_TS();
                 buf ^= 1;
 #pragma unroll
                 for (int t = 0; t < NT_; t++) baddr[t] += buf ? (unsigned)(TILE_ELEMS * 2) : (unsigned)(-(TILE_ELEMS * 2));
@@ -309,7 +290,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
             const int q0 = t * 16 + (l16 & ~3);
             const int r = q0 / OW_, col = q0 - r * OW_;
             const int orow = r0 + wpx * TRW_ + r;
-            const bool ok = q0 < TRW_ * OW_ && orow < row_end && (!(DBG & 4) || acc[0][t][0] == 123.456f);
+            const bool ok = q0 < TRW_ * OW_ && orow < row_end;
 #pragma unroll
             for (int m = 0; m < MT; m++) {
                 const mjt_f32x4 v = acc[m][t];
@@ -344,7 +325,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
             const int q = t * 16 + l16;
             const int r = q / OW_, col = q - r * OW_;
             const int orow = r0 + wpx * TRW_ + r;
-            if (q < TRW_ * OW_ && orow < row_end && (!(DBG & 4) || acc[0][t][0] == 123.456f)) {
+            if (q < TRW_ * OW_ && orow < row_end) {
 #pragma unroll
                 for (int m = 0; m < MT; m++)
 #pragma unroll
@@ -380,10 +361,6 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     }
 #if TAIL_TRW > 0
     if (tail) run_tile(mjt_ic<TAIL_TRW>(), mjt_ic<TAIL_NT>(), mjt_ic<TAIL_LROWS>(), row_begin + NFULL * TR, 0, 0);
-#endif
-#if DBG & 512
-    __syncthreads();
-    if (blockIdx.x == 8) for (int i = tid; i < NWAVES * 256; i += NTHR) ((unsigned long long*)p.a[2])[i] = tsl[i >> 8][i & 255];
 #endif
 }
 

@@ -55,7 +55,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
 
     // ---- MFMA path ----------------------------------------------------------------
     const char* wpx_env = getenv("MJT_CONV_WPX");
-    const int64_t WPX = wpx_env && *wpx_env ? atoi(wpx_env) : 2;
+    const int64_t WPX = wpx_env && atoi(wpx_env) == 1 ? 1 : 2;
     const int64_t max_px = WPX == 1 ? 224 : 112;            // pixels per wave: 16 per accumulator tile
     int64_t TRW = OW <= max_px ? max_px / OW : 0;
     if (TRW > OH) TRW = OH;
@@ -69,7 +69,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t LROWS = lds_rows(TRW);
     // output channels per workgroup: 64 per pair of waves, up to 256
     // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
-    const int64_t MT = getenv("MJT_CONV_MT") ? atoi(getenv("MJT_CONV_MT")) : 4;
+    const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
     const int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
     const bool mfma_ok = x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 64 == 0 &&
                          W % 8 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 144 <= 72 * 1024 &&
@@ -108,9 +108,8 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int64_t TAIL_LROWS = TAIL_TRW ? lds_rows(TAIL_TRW) : 0;
         const char* bq_env = getenv("MJT_CONV_BQ");
         const int BQ = bq_env && *bq_env ? atoi(bq_env) : 3;   // B fragments requested ahead of use
-        const int DBG = getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0;
         std::ostringstream key;
-        key << "mfma|" << (getenv("MJT_CONV_FS") ? getenv("MJT_CONV_FS") : "") << "|" << DBG << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT;
+        key << "mfma|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT;
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
@@ -122,7 +121,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo.str()
                 << "#define MT " << MT << "\n#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
-                << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS << "\n#define FETCH_STEP " << (getenv("MJT_CONV_FS") ? atoi(getenv("MJT_CONV_FS")) : 0) << "\n#define DBG " << DBG << "\n#define BQ_DIST " << BQ << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
+                << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS  << "\n#define BQ_DIST " << BQ << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
                 << "\n";
             src << embedded_source("conv_mfma.h") << "\n";
             k = jit_get(src.str(), name.str());
