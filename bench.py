@@ -297,8 +297,8 @@ MEASURED_TRAFFIC = {
     "C2": 2.0 * 15635.8 * 1024 + 225838.1 * 1024,
     "C3add": 2.0 * 65633.8 * 1024 + 41213.3 * 1024,
     "C3max": 2.0 * 65614.6 * 1024 + 41223.5 * 1024,
-    "C4": 2.0 * 65584.3 * 1024 + 131072.0 * 1024,
-    "C5": 2.0 * 102488.2 * 1024 + 211400.0 * 1024,
+    "C4": 2.0 * 65583.3 * 1024 + 131072.0 * 1024,
+    "C5": 2.0 * 113388.1 * 1024 + 211888.2 * 1024,
 }
 
 WORKLOADS = {
