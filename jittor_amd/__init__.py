@@ -18,10 +18,12 @@ from .core import (Var, array, unary, binary, ternary, broadcast, broadcast_var,
 from .executor import run_sync, stats as executor_stats, flags
 from . import dtypes
 from . import nn
+from .grad import grad
+from .core import no_grad
 
 __all__ = ["Var", "array", "unary", "binary", "ternary", "broadcast", "broadcast_var",
            "reduce", "reindex", "reindex_var", "reindex_reduce", "nn", "sync", "sync_all",
-           "fetch_sync", "MjtError"]
+           "fetch_sync", "grad", "no_grad", "MjtError"]
 
 
 def sync(vars, device_sync=False):

@@ -17,6 +17,20 @@ from . import dtypes as dt
 from ._lib import MjtError
 
 _next_id = [0]
+_grad_enabled = [True]
+
+
+class no_grad:
+    """Vars created inside keep no history (jt.no_grad, python/jittor/__init__.py)."""
+
+    def __enter__(self):
+        self._prev = _grad_enabled[0]
+        _grad_enabled[0] = False
+        return self
+
+    def __exit__(self, *exc):
+        _grad_enabled[0] = self._prev
+        return False
 
 
 def _new_id():
@@ -191,6 +205,10 @@ class Var:
         self._op = op
         if op is not None:
             op.out = self
+        # history for grad(): the producing op and its inputs outlive materialisation (the executor
+        # clears _op / op.inputs of computed vars), like the reference's backward liveness
+        # (python/jittor/src/node.h).  Cleared by stop_grad() and under no_grad().
+        self._history = (op, tuple(op.inputs)) if op is not None and _grad_enabled[0] else None
         self._buf = None         # Buffer once materialised
         self._host = None        # host copy for array leaves (and fused scalars)
         self.is_scalar = False   # NodeFlags::_is_scalar
@@ -342,6 +360,14 @@ class Var:
 
     def ternary(self, x, y):
         return ternary(self, x, y)
+
+    def stop_grad(self):
+        """The var becomes a leaf for grad() (var_holder.h stop_grad)."""
+        self._history = None
+        return self
+
+    def detach(self):
+        return unary_clone(self).stop_grad()
 
     def stop_fuse(self):
         self._stop_fuse = True

@@ -1,0 +1,188 @@
+"""GPU tests of jt.grad on the meta-operator path: the gradients (themselves
+built from reindex / reindex_reduce / reduce / broadcast / element-wise ops)
+against closed-form numpy gradients in float64.  Cases follow the reference's
+own gradient tests: pooling through reindex_reduce
+(python/jittor/test/test_reindex_reduce_op.py:62-77), the meta-op convolution
+(python/jittor/test/test_conv_tuner.py:105-133), reduce ops
+(python/jittor/test/test_reduce_op.py)."""
+import numpy as np
+import pytest
+
+import jittor_amd as jt
+
+pytestmark = pytest.mark.gpu
+
+
+def close(a, b, rtol=1e-4, atol=1e-5):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    assert a.shape == b.shape, (a.shape, b.shape)
+    err = np.abs(a - b).max() if a.size else 0.0
+    assert np.allclose(a, b, rtol=rtol, atol=atol), "max abs err %g" % err
+
+
+def sigmoid(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+def test_grad_fused_chain(gpu):
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((4, 8, 16)).astype(np.float32)
+    s = rng.standard_normal((8, 1)).astype(np.float32)
+    b = rng.standard_normal((1, 16)).astype(np.float32)
+    w = rng.standard_normal((4, 8, 16)).astype(np.float32)
+    vx, vs, vb = jt.array(x), jt.array(s), jt.array(b)
+    f = jt.nn.relu(vx * vs + vb)
+    out = (-f).exp() * vx.sigmoid()
+    loss = (out * jt.array(w)).sum()
+    gx, gs, gb = jt.grad(loss, [vx, vs, vb])
+    X, S, B, W = (a.astype(np.float64) for a in (x, s, b, w))
+    u = X * S + B
+    e = np.exp(-np.maximum(u, 0))
+    sg = sigmoid(X)
+    du = W * e * sg * -1.0 * (u > 0)
+    close(gx.numpy(), du * S + W * e * sg * (1 - sg))
+    close(gs.numpy(), (du * X).sum(axis=(0, 2)).reshape(8, 1))
+    close(gb.numpy(), du.sum(axis=(0, 1)).reshape(1, 16))
+
+
+@pytest.mark.parametrize("op", ["exp", "log", "sqrt", "sin", "cos", "tan", "tanh", "sinh", "cosh", "asin", "acos", "atan",
+                                "asinh", "acosh", "atanh", "sigmoid", "erf", "erfinv", "abs", "negative"])
+def test_grad_unary(gpu, op):
+    rng = np.random.default_rng(1)
+    lo, hi = {"log": (0.5, 3), "sqrt": (0.5, 3), "acosh": (1.5, 3), "asin": (-0.8, 0.8), "acos": (-0.8, 0.8),
+              "atanh": (-0.8, 0.8), "erfinv": (-0.8, 0.8), "tan": (-1, 1)}.get(op, (-2, 2))
+    x = rng.uniform(lo, hi, 257).astype(np.float32)
+    x[np.abs(x) < 0.05] = 0.5
+    v = jt.array(x)
+    g = jt.grad(v.unary(op).sum(), v).numpy()
+    X = x.astype(np.float64)
+    from scipy import special
+    with np.errstate(all="ignore"):
+        ref = _unary_refs(X, special)[op]
+    close(g, ref, rtol=2e-4)
+
+
+def _unary_refs(X, special):
+    return {"exp": np.exp(X), "log": 1 / X, "sqrt": 0.5 / np.sqrt(X), "sin": np.cos(X), "cos": -np.sin(X), "tan": 1 / np.cos(X) ** 2,
+           "tanh": 1 / np.cosh(X) ** 2, "sinh": np.cosh(X), "cosh": np.sinh(X), "asin": 1 / np.sqrt(1 - X * X),
+           "acos": -1 / np.sqrt(1 - X * X), "atan": 1 / (1 + X * X), "asinh": 1 / np.sqrt(X * X + 1),
+           "acosh": 1 / np.sqrt(np.maximum(X * X - 1, 1e-30)), "atanh": 1 / (1 - X * X), "sigmoid": sigmoid(X) * (1 - sigmoid(X)),
+           "erf": 2 / np.sqrt(np.pi) * np.exp(-X * X), "erfinv": np.sqrt(np.pi) / 2 * np.exp(special.erfinv(X) ** 2),
+           "abs": np.sign(X), "negative": -np.ones_like(X)}
+
+
+def test_grad_binary(gpu):
+    rng = np.random.default_rng(2)
+    a = rng.uniform(0.5, 2, (5, 7)).astype(np.float32)
+    b = rng.uniform(0.5, 2, (5, 7)).astype(np.float32)
+    A, B = a.astype(np.float64), b.astype(np.float64)
+    cases = {"add": (1 + 0 * A, 1 + 0 * B), "subtract": (1 + 0 * A, -1 + 0 * B), "multiply": (B, A), "divide": (1 / B, -A / B ** 2),
+             "pow": (B * A ** (B - 1), A ** B * np.log(A)), "maximum": ((A > B) * 1.0, (B >= A) * 1.0),
+             "minimum": ((A < B) * 1.0, (B <= A) * 1.0)}
+    for op, (ga, gb) in cases.items():
+        va, vb = jt.array(a), jt.array(b)
+        da, db = jt.grad(jt.binary(va, vb, op).sum(), [va, vb])
+        close(da.numpy(), ga, rtol=2e-4)
+        close(db.numpy(), gb, rtol=2e-4)
+    # a var used twice accumulates both contributions; an untouched target gets zeros
+    va, vb = jt.array(a), jt.array(b)
+    da, db = jt.grad((va * va + va).sum(), [va, vb])
+    close(da.numpy(), 2 * A + 1)
+    assert not db.numpy().any()
+
+
+def test_grad_reduce_and_broadcast(gpu):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((6, 5, 4)).astype(np.float32)
+    X = x.astype(np.float64)
+    w1 = rng.standard_normal((6, 4)).astype(np.float32)
+    v = jt.array(x)
+    close(jt.grad((v.sum(1) * jt.array(w1)).sum(), v).numpy(), np.repeat(w1[:, None, :], 5, 1))
+    close(jt.grad((v.mean(1) * jt.array(w1)).sum(), v).numpy(), np.repeat(w1[:, None, :], 5, 1) / 5)
+    g = jt.grad((v.max(1) * jt.array(w1)).sum(), v).numpy()
+    ref = (X == X.max(1, keepdims=True)) * w1[:, None, :]
+    close(g, ref)
+    g = jt.grad((v.min([0, 2], keepdims=True)).sum(), v).numpy()
+    close(g, (X == X.min(axis=(0, 2), keepdims=True)) * 1.0)
+    g = jt.grad(v.prod(2).sum(), v).numpy()
+    close(g, X.prod(2, keepdims=True) / X, rtol=1e-3)
+    # broadcast: the gradient sums over the broadcast axes
+    s = rng.standard_normal((5, 1)).astype(np.float32)
+    vs = jt.array(s)
+    close(jt.grad((vs.broadcast([6, 5, 4]) * v).sum(), vs).numpy(), X.sum(axis=(0, 2)).reshape(5, 1))
+
+
+def test_grad_pool_reindex_reduce(gpu):
+    """max / add pooling written with reindex_reduce and with reindex + reduce
+    (test_reindex_reduce_op.py:13-77)."""
+    rng = np.random.default_rng(4)
+    N, C, H, W, k = 2, 3, 8, 8, 2
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    r = rng.standard_normal((N, C, H // k, W // k)).astype(np.float32)
+    X = x.astype(np.float64)
+    blocks = X.reshape(N, C, H // k, k, W // k, k)
+    up = lambda a: np.repeat(np.repeat(a, k, 2), k, 3)
+    for op, ref in (("add", up(r)), ("maximum", (X == up(blocks.max(axis=(3, 5)))) * up(r)),
+                    ("minimum", (X == up(blocks.min(axis=(3, 5)))) * up(r))):
+        v = jt.array(x)
+        y = v.reindex_reduce(op, [N, C, H // k, W // k], ["i0", "i1", "i2/%d" % k, "i3/%d" % k])
+        close(jt.grad((y * jt.array(r)).sum(), v).numpy(), ref)
+        v = jt.array(x)
+        xx = v.reindex([N, C, H // k, W // k, k, k], ["i0", "i1", "i2*%d+i4" % k, "i3*%d+i5" % k])
+        y = xx.reduce(op, [4, 5])
+        close(jt.grad((y * jt.array(r)).sum(), v).numpy(), ref)
+
+
+def test_grad_gather_with_extras(gpu):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(50).astype(np.float32)
+    idx = rng.integers(0, 50, 300).astype(np.int32)
+    r = rng.standard_normal(300).astype(np.float32)
+    v = jt.array(x)
+    y = v.reindex([300], ["@e0(i0)"], extras=[jt.array(idx)])
+    g = jt.grad((y * jt.array(r)).sum(), v).numpy()
+    close(g, np.bincount(idx, weights=r.astype(np.float64), minlength=50))
+    # scatter-add forward: the gradient gathers
+    vals = rng.standard_normal(300).astype(np.float32)
+    vv = jt.array(vals)
+    h = vv.reindex_reduce("add", [50], ["@e0(i0)"], extras=[jt.array(idx)])
+    g = jt.grad((h * jt.array(x)).sum(), vv).numpy()
+    close(g, x.astype(np.float64)[idx])
+
+
+def test_grad_meta_conv(gpu):
+    """Gradients of the meta-op convolution (nn.py:1245-1262) with respect to input and weight,
+    against a direct float64 evaluation (test_conv_tuner.py:105-133 checks the same pair)."""
+    rng = np.random.default_rng(6)
+    N, C, H, W, K, R = 2, 3, 6, 6, 4, 3
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    w = rng.standard_normal((K, C, R, R)).astype(np.float32)
+    r = rng.standard_normal((N, K, H, W)).astype(np.float32)
+    vx, vw = jt.array(x), jt.array(w)
+    y = jt.nn.conv2d(vx, vw, padding=1)
+    gx, gw = jt.grad((y * jt.array(r)).sum(), [vx, vw])
+    X = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (1, 1), (1, 1)))
+    Wt, Rr = w.astype(np.float64), r.astype(np.float64)
+    dX = np.zeros_like(X)
+    dW = np.zeros_like(Wt)
+    for kh in range(R):
+        for kw in range(R):
+            patch = X[:, :, kh:kh + H, kw:kw + W]                       # [N,C,H,W]
+            dW[:, :, kh, kw] = np.einsum("nkhw,nchw->kc", Rr, patch)
+            dX[:, :, kh:kh + H, kw:kw + W] += np.einsum("nkhw,kc->nchw", Rr, Wt[:, :, kh, kw])
+    close(gx.numpy(), dX[:, :, 1:-1, 1:-1], rtol=1e-4, atol=1e-4)
+    close(gw.numpy(), dW, rtol=1e-4, atol=1e-4)
+
+
+def test_grad_stop_grad_and_no_grad(gpu):
+    x = jt.array(np.arange(1, 7, dtype=np.float32))
+    y = (x * 2).stop_grad()
+    z = (y * x).sum()
+    close(jt.grad(z, x).numpy(), 2 * np.arange(1, 7))          # only the direct use of x counts
+    with jt.no_grad():
+        q = x * x
+    assert q._history is None
+    assert not jt.grad(q.sum(), x).numpy().any()
+    with pytest.raises(ValueError):
+        jt.grad(jt.array([1, 2, 3]).sum(), x)

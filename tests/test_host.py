@@ -246,3 +246,34 @@ def test_conv2d_builds_the_meta_op_group():
     r = [i for i in mul.inputs if i._op.kind == "reindex"][0]._op
     assert r.indexes == ["i0", "i2", "i3*1-1+i5*1", "i4*1-1+i6*1"]
     assert jt.nn.conv2d(x, w, stride=2, padding=1).shape == [2, 4, 4, 4]
+
+
+# ---- gradients: graph construction (no execution) -------------------------------------------
+def test_grad_graph_is_built_from_path_ops():
+    """The gradient of a meta-op is again a meta-op of the path
+    (reindex_op.cc:76-80, reindex_reduce_op.cc:45-63, reduce_op.cc:339-362,
+    broadcast_to_op.cc:112-117)."""
+    import jittor_amd as jt
+    from jittor_amd import core
+    x = jt.array(np.zeros((2, 3, 8, 8), np.float32))
+    xx = x.reindex([2, 3, 4, 4, 2, 2], ["i0", "i1", "i2*2+i4", "i3*2+i5"], overflow_conditions=["i2<0"])
+    g = jt.grad(xx.sum(), x)
+    assert isinstance(g._op, core.ReindexReduceOp) and g._op.op == "add" and g.shape == x.shape
+    assert g._op.indexes == xx._history[0].indexes and g._op.overflow_conditions == ["i2<0"]
+    y = x.reindex_reduce("add", [2, 3, 4, 4], ["i0", "i1", "i2/2", "i3/2"])
+    g = jt.grad(y.sum(), x)
+    assert isinstance(g._op, core.ReindexOp) and g.shape == x.shape and g._op.overflow_value == 0
+    g = jt.grad(x.sum([1, 3]).sum(), x)                    # reduce -> broadcast (of the ones seed)
+    assert g.shape == x.shape and isinstance(g._op, core.BroadcastOp)
+    s = jt.array(np.zeros((3, 1, 1), np.float32))
+    g = jt.grad((x * s).sum(), s)                          # broadcast -> reduce add
+    assert g.shape == [3, 1, 1] and isinstance(g._op, core.ReduceOp) and g._op.op == "add"
+    # only float targets and losses; untouched targets get zeros of their shape
+    with pytest.raises(ValueError):
+        jt.grad(x.sum(), jt.array([1, 2]))
+    z = jt.grad(x.sum(), s)
+    assert z.shape == s.shape
+    # history is dropped by stop_grad and under no_grad
+    assert (x * 2).stop_grad()._history is None
+    with jt.no_grad():
+        assert (x * 2)._history is None
