@@ -433,6 +433,11 @@ def _conv_call(xbits, wbits, params, out_dtype="float32", in_dtype="bfloat16"):
     dict(x=(2, 64, 20, 32), w=(128, 64, 3, 3), p=(1, 1, 2, 2, 2, 2)),      # dilation 2
     dict(x=(2, 192, 14, 8), w=(128, 192, 1, 1), p=(1, 1, 0, 0, 1, 1)),     # 1x1, three channel blocks
     dict(x=(1, 64, 9, 40), w=(128, 64, 5, 3), p=(1, 1, 2, 1, 1, 1)),       # 5x3 taps, odd height
+    dict(x=(2, 64, 12, 72), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),       # 72 columns: two staging segments; 64 output channels
+    dict(x=(2, 64, 10, 16), w=(128, 64, 3, 3), p=(1, 1, 0, 0, 1, 1)),      # output width 14: 4-byte store epilogue
+    dict(x=(6, 64, 35, 16), w=(128, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), rpw=35),   # two full tiles + a short tile whose last row is masked
+    dict(x=(5, 64, 30, 16), w=(128, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), rpw=20),   # second row range of an image is cut short
+    dict(x=(3, 128, 24, 24), w=(128, 128, 3, 3), p=(1, 1, 1, 1, 1, 1), rpw=24, out="bfloat16"),   # bfloat16 output, several tiles
 ])
 def test_conv_mfma_matches_oracle(gpu, case):
     from oracle import kernels as K
@@ -440,7 +445,15 @@ def test_conv_mfma_matches_oracle(gpu, case):
     xb = _bf16(rng.standard_normal(case["x"]))
     wb = _bf16(rng.standard_normal(case["w"]) * 0.05)
     sh, sw, ph, pw, dh, dw = case["p"]
-    got, kern = _conv_call(xb, wb, case["p"])
+    if "rpw" in case:
+        os.environ["MJT_CONV_RPW"] = str(case["rpw"])      # rows per workgroup, forced: the heuristic would pick it only for large batches
+    try:
+        got, kern = _conv_call(xb, wb, case["p"])
+        if "out" in case:                                  # narrower output = truncation of the same accumulators
+            got16, kern16 = _conv_call(xb, wb, case["p"], out_dtype=case["out"])
+            assert kern16.startswith("mjt_conv_mfma_bf16") and np.array_equal(got16, O.f32_to_bf16_bits(got))
+    finally:
+        os.environ.pop("MJT_CONV_RPW", None)
     assert kern.startswith("mjt_conv_mfma_bf16"), kern
     if sh == sw and ph == pw and dh == dw:
         ref = K.conv_meta_bf16(xb, wb, sh, ph, dh, 8)
