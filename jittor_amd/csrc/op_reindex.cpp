@@ -291,7 +291,10 @@ void reindex_reduce_impl(const mjt_tensor* y, const mjt_tensor* x, int op, int n
     int64_t xn = numel(x);
     if (xn == 0) return;
     if (plan->plain_e0 && numel(y) > 0 && numel(&ex[0]) == numel(y) && try_scatter_1d(y, x, op, &ex[0])) return;
-    if (op != MJT_OP_VOID) launch_fill_pattern(x->ptr, identity_bits(op, x->dtype), dtype_size(x->dtype), (size_t)xn);
+    // "void" skips the initialisation in the reference (ops/reindex_reduce_op.cc:113-120), which leaves the
+    // elements no update reaches unspecified; here they are zero, so that results do not depend on what the
+    // buffer held before
+    launch_fill_pattern(x->ptr, op == MJT_OP_VOID ? 0 : identity_bits(op, x->dtype), dtype_size(x->dtype), (size_t)xn);
     run_generic(plan, true, op, x, y, 0.0, n_ex, ex);
 }
 

@@ -33,6 +33,116 @@ class ConvUnit:
         self.id = reduce_op.id
 
 
+class ConvBwdDataUnit:
+    """reindex_reduce.add <- multiply <- {broadcast(w), broadcast(dy)}: the gradient of the convolution with
+    respect to its input (the pattern ConvTuner relays to conv_backward_x, conv_tuner.cc:375-397).  For
+    stride 1 it is the forward kernel on dy with the weights flipped and transposed."""
+    kind = "conv_bwd_x"
+    fusable = False
+
+    def __init__(self, root, dy, w, params):
+        self.out = root.out
+        self.inputs = [dy, w]
+        self.params = params
+        self.id = root.id
+
+
+class ConvBwdWeightUnit:
+    """reduce.add over (n, oh, ow) <- multiply <- {reindex(x), broadcast(dy)}: the gradient with respect to
+    the weights (conv_backward_w).  It is the forward kernel with batch and channel axes of x and dy swapped,
+    stride and dilation exchanged."""
+    kind = "conv_bwd_w"
+    fusable = False
+
+    def __init__(self, root, x, dy, params):
+        self.out = root.out
+        self.inputs = [x, dy]
+        self.params = params
+        self.id = root.id
+
+
+def _conv_affine(indexes, xshape, yshape):
+    """Solves ['i0','i2','i3*s-p+i5*d','i4*s-p+i6*d'] for (sh, sw, ph, pw, dh, dw); None if it is not that."""
+    aff = [_affine(s_, xshape, yshape) for s_ in indexes]
+    if len(aff) != 4 or any(a_ is None for a_ in aff):
+        return None
+
+    def only(co, allowed):
+        return all(co[k] == 0 for k in range(10) if k not in allowed)
+    (c0n, con), (c0c, coc), (c0h, coh), (c0w, cow) = aff
+    if c0n or c0c or con[0] != 1 or coc[2] != 1 or not only(con, (0,)) or not only(coc, (2,)):
+        return None
+    if not only(coh, (3, 5)) or not only(cow, (4, 6)):
+        return None
+    sh, dh, sw, dw = coh[3], coh[5], cow[4], cow[6]
+    ph, pw = -c0h, -c0w
+    if min(sh, dh, sw, dw) < 1 or ph < 0 or pw < 0:
+        return None
+    return sh, sw, ph, pw, dh, dw
+
+
+def _lazy_op(v, cls):
+    return v._op if (not v.materialised and isinstance(v._op, cls)) else None
+
+
+def _match_conv_bwd(op):
+    """The two gradient patterns of the meta-op convolution as jt.grad builds them (fp32 / equal dtypes)."""
+    if isinstance(op, ReindexReduceOp) and op.op == "add" and len(op.inputs) == 1 and not op.overflow_conditions:
+        y7 = op.inputs[0]
+        mul = _lazy_op(y7, BinaryOp)
+        if mul is None or mul.op != "multiply" or y7.ndim != 7 or op.out.ndim != 4:
+            return None
+        params = _conv_affine(op.indexes, op.out.shape, y7.shape)
+        if params is None or params[0] != 1 or params[1] != 1:
+            return None                                         # stride 1 only
+        N, K, C, OH, OW, R, S = y7.shape
+        for a, b in (mul.inputs, mul.inputs[::-1]):
+            ba, bb = _lazy_op(a, BroadcastOp), _lazy_op(b, BroadcastOp)
+            if ba is None or bb is None or ba.bcast_mask != 0b0011001 or bb.bcast_mask != 0b1100100:
+                continue
+            w, dy = ba.inputs[0], bb.inputs[0]
+            if list(w.shape) != [K, C, R, S] or list(dy.shape) != [N, K, OH, OW] or w.dtype != dy.dtype:
+                continue
+            if w.dtype not in ("float32", "bfloat16") or op.out.dtype not in ("float32", w.dtype):
+                continue
+            sh, sw, ph, pw, dh, dw = params
+            if dh * (R - 1) - ph < 0 or dw * (S - 1) - pw < 0:
+                continue
+            if list(op.out.shape) != [N, C, OH + dh * (R - 1) - 2 * ph, OW + dw * (S - 1) - 2 * pw]:
+                continue
+            return ConvBwdDataUnit(op, dy, w, params)
+        return None
+    if isinstance(op, ReduceOp) and op.op == "add" and op.reduce_mask == 0b0011001 and op.out.ndim == 4:
+        y7 = op.inputs[0]
+        mul = _lazy_op(y7, BinaryOp)
+        if mul is None or mul.op != "multiply" or y7.ndim != 7:
+            return None
+        N, K, C, OH, OW, R, S = y7.shape
+        if list(op.out.shape) != [K, C, R, S]:
+            return None
+        for a, b in (mul.inputs, mul.inputs[::-1]):
+            ra, bb = _lazy_op(a, ReindexOp), _lazy_op(b, BroadcastOp)
+            if ra is None or bb is None or bb.bcast_mask != 0b1100100 or len(ra.inputs) != 1:
+                continue
+            if ra.overflow_conditions or ra.overflow_value != 0.0:
+                continue
+            x, dy = ra.inputs[0], bb.inputs[0]
+            if x.ndim != 4 or list(dy.shape) != [N, K, OH, OW] or x.dtype != dy.dtype or x.shape[0] != N or x.shape[1] != C:
+                continue
+            if x.dtype not in ("float32", "bfloat16") or op.out.dtype not in ("float32", x.dtype):
+                continue
+            params = _conv_affine(ra.indexes, x.shape, y7.shape)
+            if params is None:
+                continue
+            sh, sw, ph, pw, dh, dw = params
+            H, W = x.shape[2], x.shape[3]
+            # as a convolution of x^T [C,N,H,W] with dy^T [K,N,OH,OW] (stride d, dilation s) the output must be R x S
+            if (H + 2 * ph - sh * (OH - 1) - 1) // dh + 1 != R or (W + 2 * pw - sw * (OW - 1) - 1) // dw + 1 != S:
+                continue
+            return ConvBwdWeightUnit(op, x, dy, params)
+    return None
+
+
 def _pending_ops(targets):
     """Pending producers behind `targets`, in topological order."""
     order, seen = [], set()
@@ -69,15 +179,12 @@ def _match_conv(red, consumers, targets):
         return None
     yy = red.inputs[0]
     extra = set()
-    if (not yy.materialised and isinstance(yy._op, UnaryOp) and yy._op.op == "cast" and yy.dtype == "float32"
-            and yy.id not in targets and len(consumers.get(yy.id, ())) == 1):
+    if not yy.materialised and isinstance(yy._op, UnaryOp) and yy._op.op == "cast" and yy.dtype == "float32":
         # 16-bit inputs: the sum was rewritten to cast -> reduce(float32) -> cast (ops/reduce_op.cc:259-266);
         # fused, the product is an exact float temporary (opt/kernel_ir.cc:958-968), so the cast is a no-op
         extra.add(yy._op.id)
         yy = yy._op.inputs[0]
     if yy.materialised or yy.ndim != 7 or not isinstance(yy._op, BinaryOp) or yy._op.op != "multiply":
-        return None
-    if yy.id in targets or len(consumers.get(yy.id, ())) != 1:
         return None
     a, b = yy._op.inputs
     for xx, ww in ((a, b), (b, a)):
@@ -85,10 +192,6 @@ def _match_conv(red, consumers, targets):
             continue
         ro, bo = xx._op, ww._op
         if not isinstance(ro, ReindexOp) or not isinstance(bo, BroadcastOp):
-            continue
-        if xx.id in targets or ww.id in targets:
-            continue
-        if len(consumers.get(xx.id, ())) != 1 or len(consumers.get(ww.id, ())) != 1:
             continue
         if len(ro.inputs) != 1 or ro.overflow_conditions or ro.overflow_value != 0.0:
             continue
@@ -143,24 +246,36 @@ def _execute(ops, target_ids):
         for u in op.inputs:
             consumers.setdefault(u.id, []).append(op)
 
-    # ---- convolution pattern -------------------------------------------------
-    units = []
-    absorbed = set()
+    # ---- convolution patterns -------------------------------------------------
+    # A matched root op is replaced by a unit that reads the convolution's operands directly.  What the
+    # units no longer read (the 7-d reindex / broadcast / product vars) is dropped by the liveness pass
+    # below unless something else still consumes it.
+    units = {}
     if flags["enable_conv_match"]:
         for op in ops:
+            cu = None
             if isinstance(op, ReduceOp):
                 cu = _match_conv(op, consumers, target_ids)
-                if cu is not None:
-                    absorbed |= cu.absorbed
-                    units.append(cu)
-                    stats["conv_matches"] += 1
-    conv_by_id = {u.id: u for u in units}
-    sched = []
-    for op in ops:
-        if op.id in conv_by_id:
-            sched.append(conv_by_id[op.id])
-        elif op.id not in absorbed:
-            sched.append(op)
+            if cu is None and isinstance(op, (ReduceOp, ReindexReduceOp)):
+                cu = _match_conv_bwd(op)
+            if cu is not None:
+                units[op.id] = cu
+                stats["conv_matches"] += 1
+    nodes = [units.get(op.id, op) for op in ops]
+    produced_by = {node.out.id: node for node in nodes}
+    needed = set()
+    stack = list(target_ids)
+    while stack:
+        node = produced_by.get(stack.pop())
+        if node is None or node.id in needed:
+            continue
+        needed.add(node.id)
+        stack.extend(u.id for u in node.inputs)
+    sched = [node for node in nodes if node.id in needed]
+    consumers = {}
+    for node in sched:
+        for u in node.inputs:
+            consumers.setdefault(u.id, []).append(node)
 
     # ---- stages: an op can share a kernel with its producer only inside a stage ---------
     producer = {}
@@ -269,6 +384,37 @@ def _run_single(op):
         ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
         p = _lib.ConvParams(*op.params)
         _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
+    elif isinstance(op, ConvBwdDataUnit):
+        dy, w = op.inputs
+        sh, sw, ph, pw, dh, dw = op.params
+        K, C, R, S = w.shape
+        with core.no_grad():
+            wt = core.reindex(w, [C, K, R, S], ["i1", "i0", "%d-i2" % (R - 1), "%d-i3" % (S - 1)])
+        _run_single(wt._op)
+        tx, tw = _tensor_of(dy), _tensor_of(wt)
+        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        p = _lib.ConvParams(1, 1, dh * (R - 1) - ph, dw * (S - 1) - pw, dh, dw)
+        _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
+    elif isinstance(op, ConvBwdWeightUnit):
+        x, dy = op.inputs
+        sh, sw, ph, pw, dh, dw = op.params
+        N, C, H, W = x.shape
+        _, K, OH, OW = dy.shape
+        with core.no_grad():
+            xt = core.reindex(x, [C, N, H, W], ["i1", "i0", "i2", "i3"])
+            dyt = core.reindex(dy, [K, N, OH, OW], ["i1", "i0", "i2", "i3"])
+        _run_single(xt._op)
+        _run_single(dyt._op)
+        R, S = out.shape[2], out.shape[3]
+        tmp = Var([C, K, R, S], out.dtype)
+        tx, tw = _tensor_of(xt), _tensor_of(dyt)
+        tt = _lib.tensor(_alloc_out(tmp), tmp.dtype, tmp.shape)
+        p = _lib.ConvParams(dh, dw, ph, pw, sh, sw)              # stride and dilation trade places
+        _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(tt), ctypes.byref(p)))
+        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        idx, none = _lib.c_strings(["i1", "i0", "i2", "i3"]), _lib.c_strings([])
+        ex = (_lib.Tensor * 1)()
+        _lib.check(lib.mjt_reindex(ctypes.byref(tt), ctypes.byref(ty), 4, idx, 0.0, 0, none, 0, ex))
     else:
         raise MjtError(-2, "no kernel for op %r" % (op,))
 

@@ -151,28 +151,58 @@ def test_grad_gather_with_extras(gpu):
     close(g, x.astype(np.float64)[idx])
 
 
-def test_grad_meta_conv(gpu):
-    """Gradients of the meta-op convolution (nn.py:1245-1262) with respect to input and weight,
-    against a direct float64 evaluation (test_conv_tuner.py:105-133 checks the same pair)."""
-    rng = np.random.default_rng(6)
-    N, C, H, W, K, R = 2, 3, 6, 6, 4, 3
-    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
-    w = rng.standard_normal((K, C, R, R)).astype(np.float32)
-    r = rng.standard_normal((N, K, H, W)).astype(np.float32)
-    vx, vw = jt.array(x), jt.array(w)
-    y = jt.nn.conv2d(vx, vw, padding=1)
-    gx, gw = jt.grad((y * jt.array(r)).sum(), [vx, vw])
-    X = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (1, 1), (1, 1)))
+def _conv_grads_ref(x, w, r, stride, pad, dil):
+    N, C, H, W = x.shape
+    K, _, R, S = w.shape
+    OH, OW = r.shape[2], r.shape[3]
+    X = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (pad, pad), (pad, pad)))
     Wt, Rr = w.astype(np.float64), r.astype(np.float64)
-    dX = np.zeros_like(X)
-    dW = np.zeros_like(Wt)
+    dX, dW = np.zeros_like(X), np.zeros_like(Wt)
     for kh in range(R):
-        for kw in range(R):
-            patch = X[:, :, kh:kh + H, kw:kw + W]                       # [N,C,H,W]
-            dW[:, :, kh, kw] = np.einsum("nkhw,nchw->kc", Rr, patch)
-            dX[:, :, kh:kh + H, kw:kw + W] += np.einsum("nkhw,kc->nchw", Rr, Wt[:, :, kh, kw])
-    close(gx.numpy(), dX[:, :, 1:-1, 1:-1], rtol=1e-4, atol=1e-4)
+        for kw in range(S):
+            sl = (slice(None), slice(None), slice(kh * dil, kh * dil + (OH - 1) * stride + 1, stride),
+                  slice(kw * dil, kw * dil + (OW - 1) * stride + 1, stride))
+            dW[:, :, kh, kw] = np.einsum("nkhw,nchw->kc", Rr, X[sl])
+            dX[sl] += np.einsum("nkhw,kc->nchw", Rr, Wt[:, :, kh, kw])
+    return dX[:, :, pad:pad + H, pad:pad + W], dW
+
+
+@pytest.mark.parametrize("case", [
+    dict(x=(2, 3, 6, 6), w=(4, 3, 3, 3), stride=1, pad=1, dil=1, units=3),
+    dict(x=(3, 8, 12, 10), w=(6, 8, 3, 3), stride=1, pad=2, dil=2, units=3),
+    dict(x=(2, 4, 9, 9), w=(5, 4, 3, 3), stride=1, pad=0, dil=1, units=3),
+    dict(x=(2, 4, 11, 11), w=(5, 4, 3, 3), stride=2, pad=1, dil=1, units=2),     # input gradient: generic kernels
+    dict(x=(2, 6, 8, 8), w=(4, 6, 1, 1), stride=1, pad=0, dil=1, units=3),
+])
+def test_grad_meta_conv(gpu, case):
+    """Gradients of the meta-op convolution (nn.py:1245-1262) with respect to input and weight against a
+    direct float64 evaluation (test_conv_tuner.py:105-133 checks the same pair).  Forward, input gradient
+    (stride 1) and weight gradient are each recognised and run as one convolution call, so the
+    7-dimensional intermediates are never computed (the invariant of test_longest_dis_fuse.py:51-66)."""
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal(case["x"]).astype(np.float32)
+    w = rng.standard_normal(case["w"]).astype(np.float32)
+    vx, vw = jt.array(x), jt.array(w)
+    y = jt.nn.conv2d(vx, vw, stride=case["stride"], padding=case["pad"], dilation=case["dil"])
+    r = rng.standard_normal(y.shape).astype(np.float32)
+    gx, gw = jt.grad((y * jt.array(r)).sum(), [vx, vw])
+    before = jt.executor_stats["conv_matches"]
+    jt.sync([y, gx, gw])
+    assert jt.executor_stats["conv_matches"] - before == case["units"]
+    dX, dW = _conv_grads_ref(x, w, r, case["stride"], case["pad"], case["dil"])
+    close(gx.numpy(), dX, rtol=1e-4, atol=1e-4)
     close(gw.numpy(), dW, rtol=1e-4, atol=1e-4)
+    if case["units"] == 3:
+        # nothing of rank 7 was materialised on the way
+        seen, stack = set(), [gx, gw, y]
+        while stack:
+            v = stack.pop()
+            if v.id in seen:
+                continue
+            seen.add(v.id)
+            assert not (v.ndim == 7 and v._buf is not None)
+            if v._history is not None:
+                stack.extend(v._history[1])
 
 
 def test_grad_stop_grad_and_no_grad(gpu):
