@@ -554,3 +554,23 @@ def test_conv_full_size_c5_properties(gpu):
     # linearity in w: conv(x, 2w) == 2 conv(x, w) exactly
     got2, _ = _conv_call(xb[:4], _bf16(2 * O.BF16(wb).to_f32()), (1, 1, 1, 1, 1, 1))
     assert np.array_equal(got2, 2 * got[:4])
+
+
+# ---- 64-bit index mode ------------------------------------------------------------------------------
+def test_index64_mode_beyond_2g_elements(gpu):
+    """A Var with 2^31 or more elements switches index arithmetic to 64 bit
+    (python/jittor/src/op.cc:158-192): reindex, fused element-wise and reduce on a
+    [2^31 + 4096] int8 tensor, checked at the far end and through closed-form sums."""
+    n = (1 << 31) + 4096
+    base = np.arange(251, dtype=np.int8)                       # values 0..250 as int8 (wraps above 127)
+    x = jt.array(base)
+    y = x.reindex([n], ["i0 % 251"])                           # 2 GiB of int8
+    z = y + 1                                                  # fused kernel over >= 2^31 elements (int8 wraps like C)
+    tail = z.reindex([4096], ["i0 + %d" % (1 << 31)]).data
+    idx = (np.arange(4096, dtype=np.int64) + (1 << 31)) % 251
+    assert np.array_equal(tail, (base[idx].astype(np.int16) + 1).astype(np.int8))
+    # reduce: maximum over everything, and a sum of a 0/1 pattern (int32 accumulator would overflow int8)
+    assert int(y.max().data[0]) == int(base.max())
+    ones = (y == 7).int32().sum().data[0]
+    want = n // 251 + (1 if n % 251 > 7 else 0)
+    assert int(ones) == want
