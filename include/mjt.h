@@ -192,6 +192,16 @@ typedef struct {
 
 int mjt_fused_elementwise(const mjt_fused_desc* desc);
 
+/* A fused group that ends in a reduce (executor.cc:555 lets element, broadcast
+ * and reduce ops share a group; fused_op.cc:41-118): `desc` describes the
+ * element-wise part over the shape of the reduce input and has exactly one
+ * output var -- the reduce input, which is never written to memory (its ptr
+ * is ignored).  Every tensor input must have the full shape (bcast_mask 0),
+ * scalars are by value; other groups return MJT_ERR_UNSUPPORTED and run as
+ * mjt_fused_elementwise followed by mjt_reduce.  y, op and reduce_mask as in
+ * mjt_reduce. */
+int mjt_fused_reduce(const mjt_fused_desc* desc, const mjt_tensor* y, int op, uint32_t reduce_mask);
+
 /* ---- meta-op convolution ----------------------------------------------
  * The group reindex + broadcast + multiply + reduce.add that
  * python/jittor/nn.py:1251-1262 builds and opt/tuner/conv_tuner.cc:218-411

@@ -15,6 +15,13 @@
 //   ROW             1: innermost merged axis is reduced; 0: it is kept
 //   UNR             independent loads per lane and step (row kernel)
 //   MJT_LD          mjt_load or mjt_load_nt (streaming input)
+//   NPRO, MJT_PRO_SCALARS, MJT_RD(dst, off)
+//                   element-wise prologue (a fused group whose only consumer is
+//                   this reduce, python/jittor/src/executor.cc:555): NPRO extra
+//                   parameter words, by-value scalars, and the statement that
+//                   fills the pack `dst` with the elements at offset `off` --
+//                   one vector load per prologue input, then the op chain.
+//                   Without a prologue MJT_RD is a plain load from x.
 //
 // The host merges adjacent axes of equal kind, so kept and reduced axes
 // alternate.  Row kernel: G lanes stride over the contiguous reduced run with
@@ -24,11 +31,17 @@
 // When SPLIT is set the partials go to a scratch buffer and a second launch of
 // the same kernel family folds them (two-pass grid reduce).
 
-struct Params { void* a[8 + 6 * 5]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
+#ifndef NPRO
+#define NPRO 0
+#define MJT_PRO_SCALARS
+#define MJT_RD(dst, off) MJT_LD(dst, xp + (off))
+#endif
+struct Params { void* a[8 + 6 * 5 + NPRO]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
 // a[0] x, a[1] y or partials, a[2] O (outputs), a[3] S (splits), a[4] rcount (double bits),
 // a[5] work items per split, a[6] total work items,
 // a[8+0*5..]  kshape   a[8+1*5..] kstride (in x)   a[8+2*5..] kdiv
 // a[8+3*5..]  rshape   a[8+4*5..] rstride (in x)   a[8+5*5..] rdiv
+// a[38..]     prologue inputs (pointers) and scalars
 
 #if USE64
 #define MJT_DIVQ(n, k, tab) ((n) / (index_t)(unsigned long long)p.a[8 + ((tab)-2) * 5 + (k)])
@@ -87,6 +100,8 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const index_t S = (index_t)(unsigned long long)p.a[3];
     const TY rcount = (TY)__longlong_as_double((long long)(unsigned long long)p.a[4]);
     (void)rcount;
+    (void)xp;
+    MJT_PRO_SCALARS
     const unsigned lane = threadIdx.x % G;
     const index_t o = (index_t)blockIdx.x * (256 / G) + threadIdx.x / G;
     const index_t s = blockIdx.y;
@@ -104,7 +119,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
         index_t ro = (NR == 1) ? 0 : it / nL;
         index_t lc = (NR == 1) ? it : it - ro * nL;
         while (it < it_end) {
-            const TX* __restrict__ row = xp + kbase + ((NR == 1) ? 0 : mjt_red_offset<(NR > 1 ? NR - 1 : 1)>(p, ro));
+            const index_t row = kbase + ((NR == 1) ? 0 : mjt_red_offset<(NR > 1 ? NR - 1 : 1)>(p, ro));
             index_t lc_end = nL - lc < it_end - it ? nL : lc + (it_end - it);
             it += lc_end - lc;
             // full steps: every lane in range, UNR independent loads in flight
@@ -112,7 +127,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
             for (; lc + UNR <= lc_end && lc + UNR <= nfull; lc += UNR) {
                 mjt_pack<TX, VEC> v[UNR];
 #pragma unroll
-                for (int u = 0; u < UNR; u++) MJT_LD(v[u], row + ((lc + u) * G + lane) * VEC);
+                for (int u = 0; u < UNR; u++) MJT_RD(v[u], row + ((lc + u) * G + lane) * VEC);
 #pragma unroll
                 for (int u = 0; u < UNR; u++)
 #pragma unroll
@@ -122,7 +137,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
                 index_t l = (lc * G + lane) * VEC;
                 if (l < L) {
                     mjt_pack<TX, VEC> v;
-                    MJT_LD(v, row + l);
+                    MJT_RD(v, row + l);
 #pragma unroll
                     for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v.v[k]));
                 }
@@ -148,6 +163,8 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const index_t O = (index_t)(unsigned long long)p.a[2];
     const TY rcount = (TY)__longlong_as_double((long long)(unsigned long long)p.a[4]);
     (void)rcount;
+    (void)xp;
+    MJT_PRO_SCALARS
     const index_t o = ((index_t)blockIdx.x * 256 + threadIdx.x) * VEC;
     const index_t s = blockIdx.y;
     if (o >= O) return;
@@ -159,12 +176,11 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     TY acc[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; k++) acc[k] = INIT;
-    const TX* __restrict__ col = xp + kbase;
 #pragma unroll 4
     for (; r < r_end; r++) {
         index_t roff = (NR == 1) ? r * (index_t)(unsigned long long)p.a[8 + 4 * 5] : mjt_red_offset<NR>(p, r);
         mjt_pack<TX, VEC> v;
-        MJT_LD(v, col + roff);
+        MJT_RD(v, kbase + roff);
 #pragma unroll
         for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v.v[k]));
     }

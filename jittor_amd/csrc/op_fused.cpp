@@ -24,8 +24,7 @@ std::string vname(int i) { return "v" + std::to_string(i); }
 
 }  // namespace
 
-void fused_impl(const mjt_fused_desc* d) {
-    require_init();
+int64_t fused_validate(const mjt_fused_desc* d, std::vector<int>* inputs_out, bool outputs_need_data) {
     MJT_CHECK(d, "fused: null descriptor");
     MJT_CHECK(d->ndim >= 1 && d->ndim <= MJT_MAX_DIM, "fused: rank " << d->ndim);
     MJT_CHECK(d->n_vars > 0 && d->n_ops > 0 && d->vars && d->ops, "fused: empty group");
@@ -36,9 +35,8 @@ void fused_impl(const mjt_fused_desc* d) {
         total *= d->shape[i];
     }
     const int nv = d->n_vars;
-    // ---- validate the graph ------------------------------------------------
     std::vector<int> defined(nv, 0);
-    std::vector<int> inputs;          // var ids of tensor inputs
+    std::vector<int>& inputs = *inputs_out;          // var ids of tensor inputs
     for (int i = 0; i < nv; i++) {
         const mjt_fused_var& v = d->vars[i];
         dtype_size(v.dtype);
@@ -51,7 +49,7 @@ void fused_impl(const mjt_fused_desc* d) {
         } else if (v.role == MJT_VAR_SCALAR) {
             defined[i] = 1;
         } else if (v.role == MJT_VAR_OUTPUT) {
-            MJT_CHECK(total == 0 || v.ptr, "fused: output var " << i << " has no data");
+            MJT_CHECK(!outputs_need_data || total == 0 || v.ptr, "fused: output var " << i << " has no data");
         }
     }
     for (int k = 0; k < d->n_ops; k++) {
@@ -74,6 +72,47 @@ void fused_impl(const mjt_fused_desc* d) {
         defined[o.out] = 1;
     }
     for (int i = 0; i < nv; i++) MJT_CHECK(defined[i], "fused: var " << i << " is never produced");
+    return total;
+}
+
+// The op chain for one element as C statements: every var i becomes `vI`; intermediates keep the natural
+// type of their expression, outputs take their dtype (and are also written to `outI.v[k]` when
+// store_outputs is set).
+std::string fused_emit_ops(const mjt_fused_desc* d, bool store_outputs) {
+    std::ostringstream body;
+    for (int k = 0; k < d->n_ops; k++) {
+        const mjt_fused_op& o = d->ops[k];
+        const mjt_fused_var& ov = d->vars[o.out];
+        const char* Tz = dtype_cname(ov.dtype);
+        std::string expr;
+        if (o.kind == MJT_FOP_BROADCAST) {
+            expr = vname(o.in[0]);
+        } else if (o.kind == MJT_FOP_UNARY) {
+            expr = std::string("mjt_") + mjt_op_name(o.op) + "<" + Tz + ">(" + vname(o.in[0]) + ")";
+        } else if (o.kind == MJT_FOP_BINARY) {
+            expr = std::string("mjt_") + mjt_op_name(o.op) + "<" + Tz + ">(" + vname(o.in[0]) + ", " + vname(o.in[1]) + ")";
+        } else {
+            expr = std::string("(") + vname(o.in[0]) + " ? (" + Tz + ")(" + vname(o.in[1]) + ") : (" + Tz + ")(" +
+                   vname(o.in[2]) + "))";
+        }
+        // bool results are wrapped in (bool)(...) (type/common_op_type.cc:161); outputs take the
+        // declared dtype, intermediates keep the natural type of the expression
+        if (ov.dtype == MJT_BOOL) expr = "(bool)(" + expr + ")";
+        if (ov.role == MJT_VAR_OUTPUT) {
+            body << "const " << Tz << " " << vname(o.out) << " = (" << Tz << ")(" << expr << "); ";
+            if (store_outputs) body << "out" << o.out << ".v[k] = " << vname(o.out) << "; ";
+        } else {
+            body << "const auto " << vname(o.out) << " = " << expr << "; ";
+        }
+    }
+    return body.str();
+}
+
+void fused_impl(const mjt_fused_desc* d) {
+    require_init();
+    std::vector<int> inputs;          // var ids of tensor inputs
+    const int64_t total = fused_validate(d, &inputs, true);
+    const int nv = d->n_vars;
     if (total == 0) return;
 
     // ---- merge axes: drop extent-1 axes, fuse neighbours on which every input agrees -------
@@ -246,31 +285,7 @@ void fused_impl(const mjt_fused_desc* d) {
             else
                 body << "const " << T << " " << vname(id) << " = in" << id << ".v[k]; ";
         }
-        for (int k = 0; k < d->n_ops; k++) {
-            const mjt_fused_op& o = d->ops[k];
-            const mjt_fused_var& ov = d->vars[o.out];
-            const char* Tz = dtype_cname(ov.dtype);
-            std::string expr;
-            if (o.kind == MJT_FOP_BROADCAST) {
-                expr = vname(o.in[0]);
-            } else if (o.kind == MJT_FOP_UNARY) {
-                expr = std::string("mjt_") + mjt_op_name(o.op) + "<" + Tz + ">(" + vname(o.in[0]) + ")";
-            } else if (o.kind == MJT_FOP_BINARY) {
-                expr = std::string("mjt_") + mjt_op_name(o.op) + "<" + Tz + ">(" + vname(o.in[0]) + ", " + vname(o.in[1]) + ")";
-            } else {
-                expr = std::string("(") + vname(o.in[0]) + " ? (" + Tz + ")(" + vname(o.in[1]) + ") : (" + Tz + ")(" +
-                       vname(o.in[2]) + "))";
-            }
-            // bool results are wrapped in (bool)(...) (type/common_op_type.cc:161); outputs take the
-            // declared dtype, intermediates keep the natural type of the expression
-            if (ov.dtype == MJT_BOOL) expr = "(bool)(" + expr + ")";
-            if (ov.role == MJT_VAR_OUTPUT) {
-                body << "const " << Tz << " " << vname(o.out) << " = (" << Tz << ")(" << expr << "); out" << o.out
-                     << ".v[k] = " << vname(o.out) << "; ";
-            } else {
-                body << "const auto " << vname(o.out) << " = " << expr << "; ";
-            }
-        }
+        body << fused_emit_ops(d, true);
         for (int i = 0; i < nv; i++)
             if (d->vars[i].role == MJT_VAR_OUTPUT)
                 stores << "MJT_ST((" << dtype_cname(d->vars[i].dtype) << "*)p.a[" << p_var[i] << "] + e, out" << i << "); ";

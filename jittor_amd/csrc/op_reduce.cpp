@@ -33,15 +33,24 @@ int env_int(const char* n, int d) {
     return v && *v ? atoi(v) : d;
 }
 
+// element-wise prologue of a reduce: macro text for the kernel, its cache key, its parameter words
+struct Prologue {
+    std::string defs, key;
+    std::vector<uint64_t> args;
+    std::vector<std::pair<const void*, int>> inputs;   // (pointer, element size) of every tensor it loads
+};
+
 struct Variant {
     int tx, ty, op, nk, nr, vec, g, unr, nt;
     bool row, split, use64, second;   // second: folding partials (TX == TY, plain merge)
+    const Prologue* pro;
 };
 
 JitKernel* get_kernel(const Variant& v) {
     std::ostringstream key;
     key << v.tx << "," << v.ty << "," << v.op << "," << v.nk << "," << v.nr << "," << v.vec << "," << v.g << ","
         << v.row << v.split << v.use64 << v.second << "," << v.unr << "," << v.nt;
+    if (v.pro) key << "|" << v.pro->key;
     std::lock_guard<std::mutex> lock(g_mu);
     auto it = g_kernels.find(key.str());
     if (it != g_kernels.end()) return it->second;
@@ -51,6 +60,16 @@ JitKernel* get_kernel(const Variant& v) {
     name << "mjt_reduce_" << (v.row ? "row_" : "col_") << opn << "_" << mjt_dtype_name(v.tx) << "_"
          << mjt_dtype_name(v.ty) << "_k" << v.nk << "r" << v.nr << "v" << v.vec << "g" << v.g
          << (v.split ? "_split" : "") << (v.second ? "_fold" : "") << (v.use64 ? "_i64" : "");
+    if (v.pro) {
+        uint64_t h = 1469598103934665603ull;
+        for (unsigned char ch : v.pro->key) {
+            h ^= ch;
+            h *= 1099511628211ull;
+        }
+        char buf[32];
+        snprintf(buf, sizeof(buf), "_pro%016llx", (unsigned long long)h);
+        name << buf;
+    }
     std::ostringstream src;
     src << "#define ENTRY " << name.str() << "\n";
     src << "#define TX " << dtype_cname(v.tx) << "\n#define TY " << dtype_cname(v.ty) << "\n";
@@ -64,6 +83,7 @@ JitKernel* get_kernel(const Variant& v) {
     else   // (acc + Ty(x) * Ty(rcount)), type/common_op_type.cc:141
         src << "#define COMBINE(a, x) ((a) + TY(x) * TY(rcount))\n";
     src << "#define INIT mjt_init_" << merge_op << "<TY>()\n";
+    if (v.pro) src << v.pro->defs;
     src << embedded_source("prelude.h") << "\n" << embedded_source("reduce.h") << "\n";
     JitKernel* k = jit_get(src.str(), name.str());
     g_kernels.emplace(key.str(), k);
@@ -76,6 +96,17 @@ int pick_vec(int elem_size, int64_t run, const void* p, const void* q, int out_s
     while (vec > 1 && (run % vec != 0 || ((uintptr_t)p % (size_t)(vec * elem_size)) != 0 ||
                        (q && ((uintptr_t)q % (size_t)(vec * out_size)) != 0)))
         vec /= 2;
+    return vec;
+}
+
+// same with a prologue: every tensor it loads must take the vector width
+int pick_vec_pro(const Prologue* pro, int elem_size, int64_t run, const void* p, const void* q, int out_size) {
+    if (!pro) return pick_vec(elem_size, run, p, q, out_size);
+    int widest = 1;
+    for (auto& in : pro->inputs) widest = in.second > widest ? in.second : widest;
+    int vec = pick_vec(widest, run, nullptr, q, out_size);
+    for (auto& in : pro->inputs)
+        while (vec > 1 && (uintptr_t)in.first % (size_t)(vec * in.second)) vec /= 2;
     return vec;
 }
 
@@ -96,10 +127,10 @@ void fill_axes(std::vector<uint64_t>& a, const std::vector<Axis>& kept, const st
 // S > 1) are written to `out` as [O, S] (row) or [S, O] (column).
 void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* out, int64_t O, int64_t S,
             const std::vector<Axis>& kept, const std::vector<Axis>& red, double rcount, bool use64, int vec, int g,
-            int64_t per, int64_t total, bool stream = false) {
+            int64_t per, int64_t total, bool stream = false, const Prologue* pro = nullptr) {
     // inputs larger than the caches are streamed (read once, non-temporal loads)
     Variant v{tx, ty, op, (int)kept.size(), (int)red.size(), vec, g, env_int("MJT_REDUCE_UNR", 8),
-              env_int("MJT_REDUCE_NT", stream ? 1 : 0), row, S > 1, use64, second};
+              env_int("MJT_REDUCE_NT", stream ? 1 : 0), row, S > 1, use64, second, pro};
     JitKernel* k = get_kernel(v);
     std::vector<uint64_t> a(8 + 6 * 5, 0);
     a[0] = bits_of_ptr(x);
@@ -110,6 +141,7 @@ void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* 
     a[5] = (uint64_t)per;
     a[6] = (uint64_t)total;
     fill_axes(a, kept, red);
+    if (pro) a.insert(a.end(), pro->args.begin(), pro->args.end());
     int64_t blocks = row ? (O + (256 / g) - 1) / (256 / g) : ((O / vec) + 255) / 256;
     MJT_CHECK(blocks < (int64_t(1) << 31) && S < 65536, "reduce: launch too large");
     jit_launch(k, (unsigned)blocks, (unsigned)S, 256, 0, a);
@@ -117,9 +149,9 @@ void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* 
 
 }  // namespace
 
-void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask) {
+void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask, const Prologue* pro) {
     require_init();
-    check_tensor(x, "reduce x");
+    if (!pro) check_tensor(x, "reduce x");
     check_tensor(y, "reduce y");
     MJT_CHECK(op >= 0 && op < MJT_OP_COUNT && reducible(op),
               "reduce: op '" << (mjt_op_name(op) ? mjt_op_name(op) : "?") << "' is not an associative binary op");
@@ -168,7 +200,7 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         std::vector<Axis> r1{Axis{xn == 0 ? 0 : 1, 0}};
         std::vector<Axis> k1{Axis{O, 1}};
         launch(false, tx, ty, op, false, x->ptr ? x->ptr : y->ptr, y->ptr, O, 1, k1, r1, rcount, false, 1, 1,
-               r1[0].size, r1[0].size);
+               r1[0].size, r1[0].size, false, xn ? pro : nullptr);
         return;
     }
     bool use64 = xn >= (int64_t(1) << 31);
@@ -178,7 +210,7 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
 
     if (row) {
         int64_t L = red.back().size;
-        int vec = pick_vec(dtype_size(tx), L, x->ptr, nullptr, 0);
+        int vec = pick_vec_pro(pro, dtype_size(tx), L, x->ptr, nullptr, 0);
         for (auto& a : kept)
             if (a.stride % vec) vec = 1;
         for (size_t i = 0; i + 1 < red.size(); i++)
@@ -200,10 +232,10 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         int64_t per = (total + S - 1) / S;
         S = (total + per - 1) / per;
         if (S == 1) {
-            launch(true, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, g, per, total, stream);
+            launch(true, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, g, per, total, stream, pro);
         } else {
             void* part = scratch((size_t)O * S * tsz);
-            launch(true, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, g, per, total, stream);
+            launch(true, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, g, per, total, stream, pro);
             // fold [O, S] along the last axis
             std::vector<Axis> k2{Axis{O, S}}, r2{Axis{S, 1}};
             int vec2 = pick_vec(tsz, S, part, nullptr, 0);
@@ -214,7 +246,7 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         }
     } else {
         int64_t Lk = kept.back().size;
-        int vec = pick_vec(dtype_size(tx), Lk, x->ptr, y->ptr, tsz);
+        int vec = pick_vec_pro(pro, dtype_size(tx), Lk, x->ptr, y->ptr, tsz);
         for (size_t i = 0; i + 1 < kept.size(); i++)
             if (kept[i].stride % vec) vec = 1;
         for (auto& a : red)
@@ -231,10 +263,10 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         int64_t per = (R + S - 1) / S;
         S = (R + per - 1) / per;
         if (S == 1) {
-            launch(false, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, 1, per, R, stream);
+            launch(false, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, 1, per, R, stream, pro);
         } else {
             void* part = scratch((size_t)O * S * tsz);
-            launch(false, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R, stream);
+            launch(false, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R, stream, pro);
             std::vector<Axis> k2{Axis{O, 1}}, r2{Axis{S, O}};
             int vec2 = pick_vec(tsz, O, part, y->ptr, tsz);
             launch(false, ty, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, 1, S, S);
@@ -242,7 +274,79 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
     }
 }
 
+void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask) {
+    reduce_core(x, y, op, reduce_mask, nullptr);
+}
+
+// Reduce whose input is produced element by element from other tensors: the group's single output var
+// is never written to memory.
+void fused_reduce_impl(const mjt_fused_desc* d, const mjt_tensor* y, int op, uint32_t reduce_mask) {
+    require_init();
+    std::vector<int> inputs;
+    fused_validate(d, &inputs, false);
+    int out = -1;
+    for (int i = 0; i < d->n_vars; i++)
+        if (d->vars[i].role == MJT_VAR_OUTPUT) {
+            MJT_CHECK(out < 0, "fused reduce: the group must have exactly one output var (the reduce input)");
+            out = i;
+        }
+    MJT_CHECK(out >= 0, "fused reduce: the group has no output var");
+    for (int id : inputs)
+        if (d->vars[id].bcast_mask)
+            MJT_FAIL(MJT_ERR_UNSUPPORTED, "fused reduce: input var " << id << " is broadcast; only full-shape inputs and scalars");
+    Prologue pro;
+    const int base = 8 + 6 * 5;
+    std::ostringstream scal, loads, elems, key;
+    std::vector<int> slot(d->n_vars, -1);
+    for (int i = 0; i < d->n_vars; i++) {
+        const mjt_fused_var& fv = d->vars[i];
+        const char* T = dtype_cname(fv.dtype);
+        key << fv.role << ":" << fv.dtype << ";";
+        if (fv.role == MJT_VAR_INPUT) {
+            slot[i] = base + (int)pro.args.size();
+            pro.args.push_back(bits_of_ptr(fv.ptr));
+            pro.inputs.emplace_back(fv.ptr, dtype_size(fv.dtype));
+            loads << "mjt_pack<" << T << ", VEC> in" << i << "; MJT_LD(in" << i << ", (const " << T << "*)p.a[" << slot[i]
+                  << "] + o_); ";
+            elems << "const " << T << " v" << i << " = in" << i << ".v[k]; ";
+        } else if (fv.role == MJT_VAR_SCALAR) {
+            slot[i] = base + (int)pro.args.size();
+            if (dtype_is_float(fv.dtype)) {
+                pro.args.push_back(bits_of(fv.fvalue));
+                scal << "const " << T << " v" << i << " = (" << T << ")__longlong_as_double((long long)(unsigned long long)p.a["
+                     << slot[i] << "]); ";
+            } else {
+                pro.args.push_back((uint64_t)fv.ivalue);
+                scal << "const " << T << " v" << i << " = (" << T << ")(long long)(unsigned long long)p.a[" << slot[i] << "]; ";
+            }
+        }
+    }
+    for (int k = 0; k < d->n_ops; k++) {
+        const mjt_fused_op& o = d->ops[k];
+        key << o.kind << ":" << o.op << ":" << o.in[0] << ":" << (o.kind >= MJT_FOP_BINARY ? o.in[1] : -1) << ":"
+            << (o.kind == MJT_FOP_TERNARY ? o.in[2] : -1) << ">" << o.out << ";";
+    }
+    std::ostringstream defs;
+    defs << "#define NPRO " << pro.args.size() << "\n#define MJT_PRO_SCALARS " << scal.str() << "\n"
+         << "#define MJT_RD(dst, off) do { const index_t o_ = (off); " << loads.str()
+         << "_Pragma(\"unroll\") for (int k = 0; k < VEC; k++) { " << elems.str() << fused_emit_ops(d, false) << "(dst).v[k] = (TX)(v"
+         << out << "); } } while (0)\n";
+    pro.defs = defs.str();
+    pro.key = key.str();
+    mjt_tensor x{};                        // the virtual reduce input: dtype of the group's output, shape of the group
+    x.ptr = nullptr;
+    x.dtype = d->vars[out].dtype;
+    x.ndim = d->ndim;
+    for (int i = 0; i < d->ndim; i++) x.shape[i] = d->shape[i];
+    dtype_size(x.dtype);
+    reduce_core(&x, y, op, reduce_mask, &pro);
+}
+
 }  // namespace mjt
+
+extern "C" int mjt_fused_reduce(const mjt_fused_desc* desc, const mjt_tensor* y, int op, uint32_t reduce_mask) {
+    return mjt::guarded([&] { mjt::fused_reduce_impl(desc, y, op, reduce_mask); });
+}
 
 extern "C" int mjt_reduce(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask) {
     return mjt::guarded([&] { mjt::reduce_impl(x, y, op, reduce_mask); });

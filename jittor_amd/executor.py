@@ -16,8 +16,8 @@ from .core import (Var, Buffer, UnaryOp, BinaryOp, TernaryOp, BroadcastOp,
                    ReduceOp, ReindexOp, ReindexReduceOp)
 from ._lib import MjtError
 
-stats = {"launches": 0, "fused_groups": 0, "conv_matches": 0, "syncs": 0}
-flags = {"enable_conv_match": True}
+stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0}
+flags = {"enable_conv_match": True, "enable_reduce_fusion": True}
 
 
 class ConvUnit:
@@ -331,10 +331,34 @@ def _execute(ops, target_ids):
     for op in sched:
         if not op.fusable:
             by_stage_other[stage[op.id]].append(op)
+    # a group whose single result feeds one reduce of the same stage becomes that reduce's prologue: the
+    # result is never written to memory (element, broadcast and reduce ops share a group, executor.cc:555)
+    prologue_of = {}
+    absorbed_groups = set()
+    if flags["enable_reduce_fusion"]:
+        for members in (m for st in by_stage_groups for m in st):
+            ids = {op.id for op in members}
+            outs = [op.out for op in members
+                    if op.out.id in target_ids or any(c.id not in ids for c in consumers.get(op.out.id, ()))]
+            if len(outs) != 1 or outs[0].id in target_ids:
+                continue
+            users = consumers.get(outs[0].id, ())
+            if len(users) != 1 or not isinstance(users[0], ReduceOp) or users[0].id in prologue_of:
+                continue
+            if stage[users[0].id] != stage[members[0].id] or outs[0].shape != members[-1].out.shape:
+                continue
+            prologue_of[users[0].id] = members
+            absorbed_groups.add(id(members))
     for s in range(nstage):
         for members in by_stage_groups[s]:
-            _run_group(members, consumers, target_ids)
+            if id(members) not in absorbed_groups:
+                _run_group(members, consumers, target_ids)
         for op in by_stage_other[s]:
+            members = prologue_of.get(op.id)
+            if members is not None:
+                if _run_group(members, consumers, target_ids, reduce=op):
+                    continue
+                _run_group(members, consumers, target_ids)
             _run_single(op)
     # materialised vars become leaves: the graph behind them can be dropped
     for op in sched:
@@ -419,8 +443,10 @@ def _run_single(op):
         raise MjtError(-2, "no kernel for op %r" % (op,))
 
 
-def _run_group(members, consumers, target_ids):
-    """One launch for a group of element / broadcast ops."""
+def _run_group(members, consumers, target_ids, reduce=None):
+    """One launch for a group of element / broadcast ops.  With `reduce` (the ReduceOp that consumes the
+    group's only result) the group runs as that reduce's prologue; returns False when the library does
+    not take the group in that form (a tensor broadcast inside it), True otherwise."""
     lib = _lib.ensure_init()
     member_ids = {op.id for op in members}
     shape = members[-1].out.shape
@@ -472,7 +498,7 @@ def _run_group(members, consumers, target_ids):
         out = op.out
         used_outside = out.id in target_ids or any(c.id not in member_ids for c in consumers.get(out.id, ()))
         if used_outside:
-            oi = add_var(_lib.VAR_OUTPUT, out.dtype, ptr=_alloc_out(out))
+            oi = add_var(_lib.VAR_OUTPUT, out.dtype, ptr=None if reduce is not None else _alloc_out(out))
             outputs.append(out)
         else:
             oi = add_var(_lib.VAR_INTERMEDIATE, out.dtype)
@@ -491,7 +517,7 @@ def _run_group(members, consumers, target_ids):
         fo.out = oi
         fops.append(fo)
     if not outputs:
-        return
+        return True
     desc = _lib.FusedDesc()
     desc.ndim = len(shape)
     for i, s in enumerate(shape):
@@ -499,6 +525,20 @@ def _run_group(members, consumers, target_ids):
     varr = (_lib.FusedVar * len(fvars))(*fvars)
     oarr = (_lib.FusedOp * len(fops))(*fops)
     desc.n_vars, desc.vars, desc.n_ops, desc.ops = len(fvars), varr, len(fops), oarr
+    if reduce is not None:
+        rout = reduce.out
+        had_buf = rout._buf is not None
+        ty = _lib.tensor(_alloc_out(rout), rout.dtype, rout.shape)
+        rc = lib.mjt_fused_reduce(ctypes.byref(desc), ctypes.byref(ty), _lib.OP_CODE[reduce.op], reduce.reduce_mask)
+        if rc == -2:                                   # MJT_ERR_UNSUPPORTED: run the two kernels instead
+            if not had_buf:
+                rout._buf = None
+            return False
+        _lib.check(rc)
+        stats["launches"] += 1
+        stats["fused_reduces"] += 1
+        return True
     stats["launches"] += 1
     stats["fused_groups"] += 1
     _lib.check(lib.mjt_fused_elementwise(ctypes.byref(desc)))
+    return True

@@ -574,3 +574,51 @@ def test_index64_mode_beyond_2g_elements(gpu):
     ones = (y == 7).int32().sum().data[0]
     want = n // 251 + (1 if n % 251 > 7 else 0)
     assert int(ones) == want
+
+
+# ---- reduce with an element-wise prologue -----------------------------------------------------------
+def test_fused_reduce_prologue(gpu):
+    """A group of element-wise ops whose only result feeds a reduce runs inside the reduce kernel
+    (element, broadcast and reduce ops share a group, python/jittor/src/executor.cc:555); results must
+    equal the two-kernel path and the oracle."""
+    rng = np.random.default_rng(40)
+    x = rng.standard_normal((37, 129)).astype(np.float32)
+    y = rng.standard_normal((37, 129)).astype(np.float32)
+    cases = [
+        (lambda a, b: (a * a).sum(1), lambda X, Y: (X * X).sum(1)),                          # row kernel
+        (lambda a, b: ((a - b) * (a - b)).sum(0), lambda X, Y: ((X - Y) ** 2).sum(0)),       # column kernel
+        (lambda a, b: (a * 2.0 + 1.0).abs().max(), lambda X, Y: np.abs(X * 2 + 1).max(keepdims=True).reshape(1)),   # all axes, scalars by value
+        (lambda a, b: (a > b).int32().sum(1), lambda X, Y: (X > Y).sum(1)),                  # bool -> int32 prologue
+        (lambda a, b: (a * b).mean(1), lambda X, Y: (X * Y).mean(1)),
+        (lambda a, b: a.exp().min(0), lambda X, Y: np.exp(X).min(0)),
+    ]
+    for f, ref in cases:
+        before = dict(jt.executor_stats)
+        got = f(jt.array(x), jt.array(y)).data
+        assert jt.executor_stats["fused_reduces"] == before["fused_reduces"] + 1
+        assert jt.executor_stats["fused_groups"] == before["fused_groups"]          # nothing was materialised on the way
+        want = ref(x.astype(np.float64), y.astype(np.float64))
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-4), (got, want)
+        jt.flags["enable_reduce_fusion"] = False
+        try:
+            two = f(jt.array(x), jt.array(y)).data
+        finally:
+            jt.flags["enable_reduce_fusion"] = True
+        assert np.allclose(got, two, rtol=1e-6, atol=1e-5)
+    # large input: split path (partials + fold) with a prologue; bf16 sum is cast -> reduce -> cast
+    big = rng.standard_normal((4, 1 << 18)).astype(np.float32)
+    got = (jt.array(big) * jt.array(big)).sum().data
+    assert np.allclose(got, (big.astype(np.float64) ** 2).sum(), rtol=1e-5)
+    xb = jt.array(x).bfloat16()
+    before = jt.executor_stats["fused_reduces"]
+    s = xb.sum(1)
+    got = s.data
+    assert jt.executor_stats["fused_reduces"] == before + 1 and s.dtype == "bfloat16"
+    want = O.BF16(O.f32_to_bf16_bits(O.BF16(xb.raw()).to_f32().astype(np.float64).sum(1).astype(np.float32))).to_f32()
+    assert np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max()
+    # a tensor broadcast inside the group is not taken as a prologue: two kernels, same result
+    sc = rng.standard_normal((37, 1)).astype(np.float32)
+    before = dict(jt.executor_stats)
+    got = (jt.array(x) * jt.array(sc)).sum(1).data
+    assert jt.executor_stats["fused_reduces"] == before["fused_reduces"]
+    assert np.allclose(got, (x.astype(np.float64) * sc).sum(1), rtol=1e-5, atol=1e-4)

@@ -277,3 +277,47 @@ def test_grad_graph_is_built_from_path_ops():
     assert (x * 2).stop_grad()._history is None
     with jt.no_grad():
         assert (x * 2)._history is None
+
+
+def test_fused_reduce_descriptor_checks_and_specialisation(compile_only):
+    """mjt_fused_reduce: one output var (the reduce input), full-shape inputs only; the kernel with the
+    prologue compiles for gfx950."""
+    L = compile_only
+    lib = L.load()
+    V, F = L.FusedVar, L.FusedOp
+
+    def desc(mask=0, outputs=1):
+        spec = [(0, "float32", 0x1000, 0), (0, "float32", 0x2000, mask), (3, "float32", None, 0), (1, "float32", None, 0),
+                (2, "float32", None, 0)]
+        if outputs == 2:
+            spec[3] = (2, "float32", None, 0)
+        va = (V * len(spec))()
+        for i, (role, dt_, ptr, m) in enumerate(spec):
+            va[i].role, va[i].dtype, va[i].ptr, va[i].bcast_mask = role, L.DTYPE_CODE[dt_], ptr, m
+        va[2].fvalue = 0.5
+        ops = [(1, "multiply", [0, 1], 3), (1, "add", [3, 2], 4)]
+        oa = (F * len(ops))()
+        for i, (kind, op, ins, out) in enumerate(ops):
+            oa[i].kind, oa[i].op, oa[i].out = kind, L.OP_CODE[op], out
+            for j, u in enumerate(ins):
+                oa[i].inp[j] = u
+        d = L.FusedDesc()
+        d.ndim = 2
+        d.shape[0], d.shape[1] = 64, 256
+        d.n_vars, d.vars, d.n_ops, d.ops = len(spec), va, len(ops), oa
+        return d, (va, oa)
+
+    ty = L.tensor(0x3000, "float32", [64])
+    d, keep = desc()
+    assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty), L.OP_CODE["add"], 0b10) == 0
+    assert "_pro" in L.last_kernel() and L.last_kernel().startswith("mjt_reduce_row_add")
+    ty0 = L.tensor(0x3000, "float32", [256])
+    assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty0), L.OP_CODE["maximum"], 0b01) == 0
+    assert L.last_kernel().startswith("mjt_reduce_col_maximum")
+    d, keep = desc(mask=0b01)                                    # a broadcast tensor input
+    assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty), L.OP_CODE["add"], 0b10) == -2
+    d, keep = desc(outputs=2)
+    assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty), L.OP_CODE["add"], 0b10) == -1
+    d, keep = desc()
+    assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty0), L.OP_CODE["add"], 0b10) == -1    # y has the wrong size
+    assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty), L.OP_CODE["subtract"], 0b10) == -1
