@@ -19,11 +19,14 @@ from .executor import run_sync, stats as executor_stats, flags
 from . import dtypes
 from . import nn
 from .grad import grad
+from . import misc
+from .misc import gather, scatter, pad, pool, permute, transpose, reshape, flip
 from .core import no_grad
 
 __all__ = ["Var", "array", "unary", "binary", "ternary", "broadcast", "broadcast_var",
            "reduce", "reindex", "reindex_var", "reindex_reduce", "nn", "sync", "sync_all",
-           "fetch_sync", "grad", "no_grad", "MjtError"]
+           "fetch_sync", "grad", "no_grad", "gather", "scatter", "pad", "pool", "permute", "transpose", "reshape",
+           "flip", "MjtError"]
 
 
 def sync(vars, device_sync=False):

@@ -1,0 +1,218 @@
+"""Callers of the meta-operator path: the library functions the reference
+writes with reindex / reindex_reduce / reduce, with the same signatures.
+
+gather / scatter (python/jittor/misc.py:1563-1640), pad
+(python/jittor/nn.py:1679-1700), pool (python/jittor/pool.py:200-208, the
+meta-operator branch), transpose / permute, reshape, flip, basic slicing.
+Everything here only builds Var graphs; execution is the path's kernels.
+"""
+import numbers
+
+from . import core
+from .core import Var, reindex, reindex_reduce, ternary, binary, array, broadcast
+
+
+def gather(x, dim, index):
+    """out[i][j][k] = x[index[i][j][k]][j][k] (dim 0), ... (misc.py:1617-1640)."""
+    nd = index.ndim
+    if x.ndim != nd:
+        raise ValueError("gather: index must have the rank of x")
+    dim = dim + nd if dim < 0 else dim
+    args = ",".join("i%d" % i for i in range(nd))
+    idx = ["i%d" % i for i in range(nd)]
+    idx[dim] = "@e0(%s)" % args
+    return reindex(x, index.shape, idx, extras=[index])
+
+
+def scatter(x, dim, index, src, reduce="void"):
+    """x[index[i][j][k]][j][k] = src[i][j][k] (dim 0), ...; reduce 'void' (assign), 'add' or 'multiply'
+    (misc.py:1563-1612).  Built from reindex_reduce: the scattered tensor starts from the op's identity,
+    and for 'void' a count of updates per element selects between it and x."""
+    if reduce not in ("void", "add", "multiply"):
+        raise ValueError("scatter: reduce must be 'void', 'add' or 'multiply'")
+    nd = index.ndim
+    if x.ndim != nd:
+        raise ValueError("scatter: index must have the rank of x")
+    dim = dim + nd if dim < 0 else dim
+    src = core._as_var(src)
+    if src.num == 1 and list(src.shape) != list(index.shape):
+        src = broadcast(src.cast(x.dtype) if src.dtype != x.dtype else src, index.shape)
+    elif list(src.shape) != list(index.shape):
+        src = src[tuple(slice(None, s) for s in index.shape)]
+    if src.dtype != x.dtype:
+        src = src.cast(x.dtype)
+    args = ",".join("i%d" % i for i in range(nd))
+    idx = ["i%d" % i for i in range(nd)]
+    idx[dim] = "@e0(%s)" % args
+    upd = reindex_reduce(src, reduce, x.shape, idx, extras=[index])
+    if reduce == "add":
+        return x + upd
+    if reduce == "multiply":
+        return x * upd
+    one = broadcast(array(1, "int32"), index.shape)
+    hit = reindex_reduce(one, "add", x.shape, idx, extras=[index])
+    return ternary(hit > 0, upd, x)
+
+
+def pad(x, padding, mode="constant", value=0):
+    """padding = (left_last, right_last, left_prev, right_prev, ...) as nn.py:1679-1700."""
+    if mode not in ("constant", "replicate", "reflect", "circular"):
+        raise ValueError("only support constant,replicate,reflect,circular pad")
+    padding = list(padding)
+    if len(padding) % 2 or len(padding) // 2 > x.ndim:
+        raise ValueError("pad: bad padding %r for rank %d" % (padding, x.ndim))
+    left = [0] * (x.ndim - len(padding) // 2) + padding[::2][::-1]
+    right = [0] * (x.ndim - len(padding) // 2) + padding[1::2][::-1]
+    dims, shape = [], []
+    for i, (n, l, r) in enumerate(zip(x.shape, left, right)):
+        shape.append(n + l + r)
+        if mode == "constant":
+            dims.append("i%d-%d" % (i, l))
+        elif mode == "replicate":
+            dims.append("i%d<%d ? 0 : i%d > %d ? %d : i%d-%d" % (i, l, i, n + l - 1, n - 1, i, l))
+        elif mode == "reflect":
+            dims.append("i%d<%d ? %d-i%d : i%d > %d ? %d-i%d : i%d-%d" % (i, l, l, i, i, n + l - 1, 2 * (n - 1) + l, i, i, l))
+        else:
+            dims.append("i%d<%d ? %d+i%d : i%d > %d ? i%d-%d : i%d-%d" % (i, l, n - l, i, i, n + l - 1, i, n + l, i, l))
+    return reindex(x, shape, dims, overflow_value=value)
+
+
+def _pair(v):
+    return (v, v) if isinstance(v, numbers.Integral) else tuple(v)
+
+
+def pool(x, kernel_size, op, padding=0, stride=None):
+    """2-d pooling of an NCHW Var as reindex + reduce (pool.py:200-208): window elements outside the
+    image take the reindex overflow value 0, as in the reference's meta-operator branch."""
+    kh, kw = _pair(kernel_size)
+    sh, sw = _pair(stride if stride else kernel_size)
+    ph, pw = _pair(padding)
+    if op not in ("maximum", "minimum", "mean", "add"):
+        raise ValueError("pool: op %r" % (op,))
+    N, C, H, W = x.shape
+    h = (H + ph * 2 - kh) // sh + 1
+    w = (W + pw * 2 - kw) // sw + 1
+    xx = reindex(x, [N, C, h, w, kh, kw], ["i0", "i1", "i2*%d-%d+i4" % (sh, ph), "i3*%d-%d+i5" % (sw, pw)])
+    return core.reduce(xx, op, [4, 5])
+
+
+def permute(x, *dims):
+    if len(dims) == 1 and isinstance(dims[0], (list, tuple)):
+        dims = tuple(dims[0])
+    if not dims:
+        dims = tuple(range(x.ndim))[::-1]
+    dims = [d + x.ndim if d < 0 else d for d in dims]
+    if sorted(dims) != list(range(x.ndim)):
+        raise ValueError("permute: %r is not a permutation of the axes" % (dims,))
+    idx = [None] * x.ndim
+    for out_axis, in_axis in enumerate(dims):
+        idx[in_axis] = "i%d" % out_axis
+    return reindex(x, [x.shape[d] for d in dims], idx)
+
+
+def transpose(x, *dims):
+    return permute(x, *dims)
+
+
+def flip(x, dim=0):
+    dims = [dim] if isinstance(dim, numbers.Integral) else list(dim)
+    dims = [d + x.ndim if d < 0 else d for d in dims]
+    idx = ["%d-i%d" % (x.shape[i] - 1, i) if i in dims else "i%d" % i for i in range(x.ndim)]
+    return reindex(x, x.shape, idx)
+
+
+def reshape(x, *shape):
+    """Row-major reinterpretation: a reindex through the flat offset (the reference aliases the buffer,
+    python/jittor/src/ops/reshape_op.cc; a copy gives the same values)."""
+    if len(shape) == 1 and isinstance(shape[0], (list, tuple)):
+        shape = tuple(shape[0])
+    shape = list(shape)
+    total = x.num
+    if shape.count(-1) > 1:
+        raise ValueError("reshape: more than one -1")
+    if -1 in shape:
+        known = 1
+        for s in shape:
+            if s != -1:
+                known *= s
+        if known == 0 or total % known:
+            raise ValueError("reshape: cannot infer -1 for %r from %d elements" % (shape, total))
+        shape[shape.index(-1)] = total // known
+    n = 1
+    for s in shape:
+        n *= s
+    if n != total:
+        raise ValueError("reshape: %r has %d elements, the Var has %d" % (shape, n, total))
+    if shape == list(x.shape):
+        return x
+    # flat offset of the output coordinate, then the input coordinate it corresponds to
+    flat, stride = [], 1
+    for i in range(len(shape) - 1, -1, -1):
+        flat.append("i%d*%d" % (i, stride))
+        stride *= shape[i]
+    flat = "(" + "+".join(flat[::-1]) + ")"
+    idx, stride = [], 1
+    for d in range(x.ndim - 1, -1, -1):
+        idx.append("%s/%d%%%d" % (flat, stride, x.shape[d]))
+        stride *= x.shape[d]
+    return reindex(x, shape, idx[::-1])
+
+
+def getitem(x, key):
+    """Basic indexing with integers, slices (positive or negative step), None and Ellipsis, and one
+    integer Var per axis (gather along that axis); one reindex."""
+    if not isinstance(key, tuple):
+        key = (key,)
+    if sum(1 for k in key if k is Ellipsis) > 1:
+        raise IndexError("an index can only have a single ellipsis")
+    n_real = sum(1 for k in key if k is not None and k is not Ellipsis)
+    if n_real > x.ndim:
+        raise IndexError("too many indices for a Var of rank %d" % x.ndim)
+    full = []
+    for k in key:
+        if k is Ellipsis:
+            full.extend([slice(None)] * (x.ndim - n_real))
+        else:
+            full.append(k)
+    full.extend([slice(None)] * (x.ndim - sum(1 for k in full if k is not None)))
+    out_shape, exprs, extras = [], [], []
+    axis = 0
+    var_axes = []
+    for k in full:
+        if k is None:
+            out_shape.append(1)
+            continue
+        n = x.shape[axis]
+        if isinstance(k, numbers.Integral):
+            k = int(k)
+            if k < -n or k >= n:
+                raise IndexError("index %d is out of bounds for axis %d with size %d" % (k, axis, n))
+            exprs.append(str(k + n if k < 0 else k))
+        elif isinstance(k, slice):
+            start, stop, step = k.indices(n)
+            count = len(range(start, stop, step))
+            exprs.append("%d+i%d*(%d)" % (start, len(out_shape), step))
+            out_shape.append(count)
+        elif isinstance(k, Var):
+            if k.ndim != 1 or k.is_float():
+                raise IndexError("only 1-d integer Vars index an axis")
+            exprs.append("@e%d(i%d)" % (len(extras), len(out_shape)))
+            extras.append(k)
+            out_shape.append(k.shape[0])
+            var_axes.append(axis)
+        else:
+            raise IndexError("unsupported index %r" % (k,))
+        axis += 1
+    if not out_shape:
+        out_shape = [1]
+    return reindex(x, out_shape, exprs, extras=extras)
+
+
+Var.gather = gather
+Var.scatter = scatter
+Var.permute = permute
+Var.transpose = transpose
+Var.reshape = reshape
+Var.view = reshape
+Var.flip = flip
+Var.__getitem__ = getitem

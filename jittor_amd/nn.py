@@ -43,3 +43,21 @@ def conv2d(x, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
         b = bias.broadcast(y.shape, [0, 2, 3])
         y = y + b
     return y
+
+
+def pad(x, padding, mode="constant", value=0):
+    from .misc import pad as _pad
+    return _pad(x, padding, mode, value)
+
+
+def pool(x, kernel_size, op, padding=0, stride=None):
+    from .misc import pool as _pool
+    return _pool(x, kernel_size, op, padding, stride)
+
+
+def max_pool2d(x, kernel_size, stride=None, padding=0):
+    return pool(x, kernel_size, "maximum", padding, stride)
+
+
+def avg_pool2d(x, kernel_size, stride=None, padding=0):
+    return pool(x, kernel_size, "mean", padding, stride)

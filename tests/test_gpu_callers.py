@@ -1,0 +1,97 @@
+"""GPU tests of the callers built on the path (gather, scatter, pad, pool,
+permute, reshape, flip, slicing) against numpy, with the examples of the
+reference's docstrings (python/jittor/misc.py:1575-1600,1628-1634) and its
+tests of pooling and padding as cases."""
+import numpy as np
+import pytest
+
+import jittor_amd as jt
+
+pytestmark = pytest.mark.gpu
+
+
+def test_gather_scatter_docstring_examples(gpu):
+    t = jt.array([[1, 2], [3, 4]])
+    assert t.gather(1, jt.array([[0, 0], [1, 0]])).data.tolist() == [[1, 1], [4, 3]]
+    assert t.gather(0, jt.array([[0, 0], [1, 0]])).data.tolist() == [[1, 2], [3, 2]]
+    src = jt.array(np.arange(1, 11, dtype=np.int32).reshape(2, 5))
+    x = jt.zeros((3, 5), "int32").scatter(0, jt.array([[0, 1, 2, 0]]), src)
+    assert x.data.tolist() == [[1, 0, 0, 4, 0], [0, 2, 0, 0, 0], [0, 0, 3, 0, 0]]
+    x = jt.zeros((3, 5), "int32").scatter(1, jt.array([[0, 1, 2], [0, 1, 4]]), src)
+    assert x.data.tolist() == [[1, 2, 3, 0, 0], [6, 7, 0, 0, 8], [0, 0, 0, 0, 0]]
+    full = jt.array(np.full((2, 4), 2.0, np.float32))
+    x = full.scatter(1, jt.array([[2], [3]]), jt.array(1.23), reduce="multiply")
+    assert np.allclose(x.data, [[2, 2, 2.46, 2], [2, 2, 2, 2.46]])
+    x = full.scatter(1, jt.array([[2], [3]]), jt.array(1.23), reduce="add")
+    assert np.allclose(x.data, [[2, 2, 3.23, 2], [2, 2, 2, 3.23]])
+
+
+def test_gather_scatter_random(gpu):
+    rng = np.random.default_rng(50)
+    x = rng.standard_normal((7, 9, 5)).astype(np.float32)
+    for dim in range(3):
+        idx = rng.integers(0, x.shape[dim], (7, 9, 5)).astype(np.int32)
+        assert np.array_equal(jt.array(x).gather(dim, jt.array(idx)).data, np.take_along_axis(x, idx, dim))
+        src = rng.standard_normal((7, 9, 5)).astype(np.float32)
+        want = x.astype(np.float64).copy()
+        np.add.at(want, tuple(idx if d == dim else np.indices(idx.shape)[d] for d in range(3)), src)
+        got = jt.array(x).scatter(dim, jt.array(idx), jt.array(src), reduce="add").data
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("mode", ["constant", "replicate", "reflect", "circular"])
+def test_pad_modes(gpu, mode):
+    rng = np.random.default_rng(51)
+    x = rng.standard_normal((2, 3, 6, 7)).astype(np.float32)
+    padding = (2, 1, 3, 2)                                   # left, right of the last axis, then of the one before
+    got = jt.pad(jt.array(x), padding, mode, 1.5).data
+    widths = ((0, 0), (0, 0), (3, 2), (2, 1))
+    np_mode = {"constant": "constant", "replicate": "edge", "reflect": "reflect", "circular": "wrap"}[mode]
+    want = np.pad(x, widths, np_mode, **({"constant_values": 1.5} if mode == "constant" else {}))
+    assert np.array_equal(got, want)
+
+
+def test_pool_against_numpy(gpu):
+    rng = np.random.default_rng(52)
+    x = rng.standard_normal((2, 3, 12, 10)).astype(np.float32)
+    for k, s, p in [(2, 2, 0), (3, 2, 1), (3, 1, 1)]:
+        H = (12 + 2 * p - k) // s + 1
+        W = (10 + 2 * p - k) // s + 1
+        xp = np.pad(x, ((0, 0), (0, 0), (p, p), (p, p)))     # the reference's meta-operator pooling pads with 0
+        win = np.stack([xp[:, :, i:i + (H - 1) * s + 1:s, j:j + (W - 1) * s + 1:s] for i in range(k) for j in range(k)], -1)
+        for op, f in (("maximum", np.max), ("minimum", np.min), ("mean", np.mean), ("add", np.sum)):
+            got = jt.pool(jt.array(x), k, op, p, s).data
+            assert np.allclose(got, f(win.astype(np.float64), axis=-1), rtol=1e-5, atol=1e-6), (k, s, p, op)
+    # gradient of max pooling: ones at the arg-max of every window
+    v = jt.array(x)
+    g = jt.grad(jt.nn.max_pool2d(v, 2).sum(), v).data
+    blocks = x.reshape(2, 3, 6, 2, 5, 2)
+    want = (blocks == blocks.max(axis=(3, 5), keepdims=True)).reshape(x.shape).astype(np.float32)
+    assert np.array_equal(g, want)
+
+
+def test_layout_ops_and_slicing(gpu):
+    rng = np.random.default_rng(53)
+    x = rng.standard_normal((4, 5, 6, 7)).astype(np.float32)
+    v = jt.array(x)
+    assert np.array_equal(v.permute(0, 2, 3, 1).data, x.transpose(0, 2, 3, 1))
+    assert np.array_equal(v.transpose().data, x.transpose())
+    assert np.array_equal(v.reshape(20, -1).data, x.reshape(20, -1))
+    assert np.array_equal(v.reshape(2, 2, 5, 42).data, x.reshape(2, 2, 5, 42))
+    assert np.array_equal(v.flip([1, 3]).data, x[:, ::-1, :, ::-1])
+    assert np.array_equal(v[1].data, x[1])
+    assert np.array_equal(v[1:3, ::2, -1].data, x[1:3, ::2, -1])
+    assert np.array_equal(v[..., ::-2].data, x[..., ::-2])
+    assert np.array_equal(v[:, None, 2].data, x[:, None, 2])
+    idx = np.array([3, 0, 3, 1], np.int32)
+    assert np.array_equal(v[:, jt.array(idx)].data, x[:, idx])
+    with pytest.raises(IndexError):
+        v[4]
+    with pytest.raises(IndexError):
+        v[0, 0, 0, 0, 0]
+    # gradients flow through the layout ops: d/dx sum(x[1:3] * w) = w placed at the slice
+    w = rng.standard_normal((2, 5, 6, 7)).astype(np.float32)
+    g = jt.grad((v[1:3] * jt.array(w)).sum(), v).data
+    want = np.zeros_like(x)
+    want[1:3] = w
+    assert np.array_equal(g, want)

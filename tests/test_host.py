@@ -321,3 +321,24 @@ def test_fused_reduce_descriptor_checks_and_specialisation(compile_only):
     d, keep = desc()
     assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty0), L.OP_CODE["add"], 0b10) == -1    # y has the wrong size
     assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty), L.OP_CODE["subtract"], 0b10) == -1
+
+
+def test_callers_build_path_graphs():
+    """gather / pad / pool / slicing are one reindex (plus a reduce for pool) with the reference's index
+    strings (misc.py:1617-1640, nn.py:1679-1700, pool.py:200-208)."""
+    import jittor_amd as jt
+    from jittor_amd import core
+    x = jt.array(np.zeros((2, 3, 8, 8), np.float32))
+    g = x.gather(1, jt.array(np.zeros((2, 3, 8, 8), np.int32)))
+    assert isinstance(g._op, core.ReindexOp) and g._op.indexes == ["i0", "@e0(i0,i1,i2,i3)", "i2", "i3"]
+    p = jt.pad(x, (1, 2), "reflect")
+    assert p.shape == [2, 3, 8, 11] and p._op.indexes[3] == "i3<1 ? 1-i3 : i3 > 8 ? 15-i3 : i3-1"
+    y = jt.pool(x, 3, "maximum", 1, 2)
+    assert isinstance(y._op, core.ReduceOp) and y.shape == [2, 3, 4, 4]
+    assert y._history[1][0]._op.indexes == ["i0", "i1", "i2*2-1+i4", "i3*2-1+i5"]
+    s = x[1, :, ::2, 3]
+    assert s.shape == [3, 4] and s._op.indexes == ["1", "0+i0*(1)", "0+i1*(2)", "3"]
+    with pytest.raises(ValueError):
+        x.reshape(5, -1)
+    with pytest.raises(ValueError):
+        jt.pad(x, (1, 2), "mirror")
