@@ -20,13 +20,15 @@ from . import dtypes
 from . import nn
 from .grad import grad
 from . import misc
+from . import profiler
+from .profiler import profile_scope
 from .misc import gather, scatter, pad, pool, permute, transpose, reshape, flip
 from .core import no_grad
 
 __all__ = ["Var", "array", "unary", "binary", "ternary", "broadcast", "broadcast_var",
            "reduce", "reindex", "reindex_var", "reindex_reduce", "nn", "sync", "sync_all",
            "fetch_sync", "grad", "no_grad", "gather", "scatter", "pad", "pool", "permute", "transpose", "reshape",
-           "flip", "MjtError"]
+           "flip", "profile_scope", "MjtError"]
 
 
 def sync(vars, device_sync=False):

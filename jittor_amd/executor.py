@@ -15,6 +15,7 @@ from . import core
 from .core import (Var, Buffer, UnaryOp, BinaryOp, TernaryOp, BroadcastOp,
                    ReduceOp, ReindexOp, ReindexReduceOp)
 from ._lib import MjtError
+from . import profiler as _profiler
 
 stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0}
 flags = {"enable_conv_match": True, "enable_reduce_fusion": True}
@@ -349,17 +350,34 @@ def _execute(ops, target_ids):
                 continue
             prologue_of[users[0].id] = members
             absorbed_groups.add(id(members))
+    def group_io(members, extra_out=None):
+        ids = {op.id for op in members}
+        made = {op.out.id for op in members}
+        ins = {}
+        for op in members:
+            for u in op.inputs:
+                if u.id not in made and not (u._op is None and u._host is not None and u.num == 1):
+                    ins[u.id] = u.nbytes
+        outs = sum(op.out.nbytes for op in members
+                   if extra_out is None and (op.out.id in target_ids or any(c.id not in ids for c in consumers.get(op.out.id, ()))))
+        return sum(ins.values()), outs + (extra_out.nbytes if extra_out is not None else 0)
+
+    def timed(call, kind, io):
+        rec = _profiler.active()
+        return call() if rec is None else rec.run(call, kind, *io())
+
     for s in range(nstage):
         for members in by_stage_groups[s]:
             if id(members) not in absorbed_groups:
-                _run_group(members, consumers, target_ids)
+                timed(lambda: _run_group(members, consumers, target_ids), "fused", lambda: group_io(members))
         for op in by_stage_other[s]:
             members = prologue_of.get(op.id)
             if members is not None:
-                if _run_group(members, consumers, target_ids, reduce=op):
+                if timed(lambda: _run_group(members, consumers, target_ids, reduce=op), "fused+reduce",
+                         lambda: group_io(members, op.out)):
                     continue
-                _run_group(members, consumers, target_ids)
-            _run_single(op)
+                timed(lambda: _run_group(members, consumers, target_ids), "fused", lambda: group_io(members))
+            timed(lambda: _run_single(op), op.kind, lambda: (sum(u.nbytes for u in op.inputs), op.out.nbytes))
     # materialised vars become leaves: the graph behind them can be dropped
     for op in sched:
         if op.out._buf is not None:

@@ -95,3 +95,26 @@ def test_layout_ops_and_slicing(gpu):
     want = np.zeros_like(x)
     want[1:3] = w
     assert np.array_equal(g, want)
+
+
+def test_profile_scope_report(gpu):
+    """jt.profile_scope: rows per kernel with count, times and byte rates (profiler.cc:374-470)."""
+    rng = np.random.default_rng(54)
+    a = jt.array(rng.standard_normal((512, 2048)).astype(np.float32))
+    b = jt.array(rng.standard_normal((512, 2048)).astype(np.float32))
+    jt.sync([a, b])
+    with jt.profile_scope(warmup=1, rerun=4) as report:
+        y = (a * b + 1.0).sum(1)
+        z = a.reindex([512, 2048], ["i0", "2047-i1"])
+        jt.sync([y, z])
+    assert report[0] == ["Name", "FileName", "Count", "TotalTime", "AvgTime", "MinTime", "MaxTime", "Input", "Output", "InOut", "Compute"]
+    rows = {r[0]: r for r in report[2:]}
+    red = [r for n, r in rows.items() if n.startswith("mjt_reduce_row_add")]
+    rei = [r for n, r in rows.items() if n.startswith("mjt_reindex")]
+    assert len(red) == 1 and len(rei) == 1
+    for r in red + rei:
+        assert int(r[2]) == 5 and 0 < float(r[5]) <= float(r[4]) <= float(r[6])       # 1 + rerun launches; min <= avg <= max
+    # byte accounting: external inputs and outputs of the group
+    total_ns = float(red[0][3])
+    assert abs(float(red[0][7]) - 5 * 2 * a.nbytes / (total_ns * 1e-9)) / float(red[0][7]) < 1e-3
+    assert np.allclose(y.data, (a.data.astype(np.float64) * b.data + 1).sum(1), rtol=1e-5, atol=1e-3)
