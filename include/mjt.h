@@ -196,7 +196,9 @@ int mjt_fused_elementwise(const mjt_fused_desc* desc);
  * and reduce ops share a group; fused_op.cc:41-118): `desc` describes the
  * element-wise part over the shape of the reduce input and has exactly one
  * output var -- the reduce input, which is never written to memory (its ptr
- * is ignored).  Every tensor input must have the full shape (bcast_mask 0),
+ * is ignored).  A tensor input has the full shape (bcast_mask 0) or is
+ * broadcast along exactly the reduced axes (bcast_mask == reduce_mask on the
+ * axes of extent > 1: one value per output, e.g. the mean inside a variance);
  * scalars are by value; other groups return MJT_ERR_UNSUPPORTED and run as
  * mjt_fused_elementwise followed by mjt_reduce.  y, op and reduce_mask as in
  * mjt_reduce. */

@@ -21,7 +21,10 @@
 //                   parameter words, by-value scalars, and the statement that
 //                   fills the pack `dst` with the elements at offset `off` --
 //                   one vector load per prologue input, then the op chain.
-//                   Without a prologue MJT_RD is a plain load from x.
+//                   MJT_PRO_PER_OUTPUT loads the prologue inputs that are broadcast
+//                   along exactly the reduced axes (one value per output: the
+//                   mean in a variance, the maximum in a softmax) once, at output
+//                   index `o`.  Without a prologue MJT_RD is a plain load from x.
 //
 // The host merges adjacent axes of equal kind, so kept and reduced axes
 // alternate.  Row kernel: G lanes stride over the contiguous reduced run with
@@ -34,6 +37,7 @@
 #ifndef NPRO
 #define NPRO 0
 #define MJT_PRO_SCALARS
+#define MJT_PRO_PER_OUTPUT
 #define MJT_RD(dst, off) MJT_LD(dst, xp + (off))
 #endif
 struct Params { void* a[8 + 6 * 5 + NPRO]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
@@ -109,6 +113,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 #pragma unroll
     for (int k = 0; k < VEC; k++) acc[k] = INIT;
     if (o < O) {
+        MJT_PRO_PER_OUTPUT
         const index_t kbase = mjt_kept_offset(p, o);
         const index_t L = (index_t)(unsigned long long)p.a[8 + 3 * 5 + (NR - 1)];
         const index_t nL = (L + (G * VEC) - 1) / (G * VEC);
@@ -168,6 +173,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const index_t o = ((index_t)blockIdx.x * 256 + threadIdx.x) * VEC;
     const index_t s = blockIdx.y;
     if (o >= O) return;
+    MJT_PRO_PER_OUTPUT
     const index_t kbase = mjt_kept_offset(p, o);
     const index_t per = (index_t)(unsigned long long)p.a[5];
     const index_t total = (index_t)(unsigned long long)p.a[6];

@@ -291,12 +291,21 @@ void fused_reduce_impl(const mjt_fused_desc* d, const mjt_tensor* y, int op, uin
             out = i;
         }
     MJT_CHECK(out >= 0, "fused reduce: the group has no output var");
-    for (int id : inputs)
-        if (d->vars[id].bcast_mask)
-            MJT_FAIL(MJT_ERR_UNSUPPORTED, "fused reduce: input var " << id << " is broadcast; only full-shape inputs and scalars");
+    // a tensor input is either full-shape or broadcast along exactly the reduced axes (one value per output)
+    uint32_t live_mask = 0, red_live = 0;          // axes of extent > 1; those of them that are reduced
+    for (int a = 0; a < d->ndim; a++)
+        if (d->shape[a] != 1) {
+            live_mask |= 1u << a;
+            if (reduce_mask >> a & 1) red_live |= 1u << a;
+        }
+    for (int id : inputs) {
+        const uint32_t m = d->vars[id].bcast_mask & live_mask;
+        if (m != 0 && m != red_live)
+            MJT_FAIL(MJT_ERR_UNSUPPORTED, "fused reduce: input var " << id << " is broadcast along axes other than the reduced ones");
+    }
     Prologue pro;
     const int base = 8 + 6 * 5;
-    std::ostringstream scal, loads, elems, key;
+    std::ostringstream scal, loads, elems, key, per_out;
     std::vector<int> slot(d->n_vars, -1);
     for (int i = 0; i < d->n_vars; i++) {
         const mjt_fused_var& fv = d->vars[i];
@@ -305,10 +314,18 @@ void fused_reduce_impl(const mjt_fused_desc* d, const mjt_tensor* y, int op, uin
         if (fv.role == MJT_VAR_INPUT) {
             slot[i] = base + (int)pro.args.size();
             pro.args.push_back(bits_of_ptr(fv.ptr));
-            pro.inputs.emplace_back(fv.ptr, dtype_size(fv.dtype));
-            loads << "mjt_pack<" << T << ", VEC> in" << i << "; MJT_LD(in" << i << ", (const " << T << "*)p.a[" << slot[i]
-                  << "] + o_); ";
-            elems << "const " << T << " v" << i << " = in" << i << ".v[k]; ";
+            if ((fv.bcast_mask & live_mask) == 0 || red_live == 0) {
+                pro.inputs.emplace_back(fv.ptr, dtype_size(fv.dtype));
+                loads << "mjt_pack<" << T << ", VEC> in" << i << "; MJT_LD(in" << i << ", (const " << T << "*)p.a[" << slot[i]
+                      << "] + o_); ";
+                elems << "const " << T << " v" << i << " = in" << i << ".v[k]; ";
+            } else {
+                // one value per output: a scalar per lane group in the row kernel, VEC adjacent outputs per lane in
+                // the column kernel (scalar loads there: the outputs' alignment is not part of the vector-width choice)
+                key << "P";
+                per_out << "T_ROWCOL(" << T << ", " << i << ", " << slot[i] << ") ";
+                elems << "const " << T << " v" << i << " = V_ROWCOL(" << i << "); ";
+            }
         } else if (fv.role == MJT_VAR_SCALAR) {
             slot[i] = base + (int)pro.args.size();
             if (dtype_is_float(fv.dtype)) {
@@ -327,6 +344,10 @@ void fused_reduce_impl(const mjt_fused_desc* d, const mjt_tensor* y, int op, uin
             << (o.kind == MJT_FOP_TERNARY ? o.in[2] : -1) << ">" << o.out << ";";
     }
     std::ostringstream defs;
+    defs << "#if ROW\n#define T_ROWCOL(T, i, slot) const T r##i = ((const T*)p.a[slot])[o];\n#define V_ROWCOL(i) r##i\n#else\n"
+         << "#define T_ROWCOL(T, i, slot) T r##i[VEC]; _Pragma(\"unroll\") for (int k = 0; k < VEC; k++) r##i[k] = ((const T*)p.a[slot])[o + k];\n"
+         << "#define V_ROWCOL(i) r##i[k]\n#endif\n"
+         << "#define MJT_PRO_PER_OUTPUT " << per_out.str() << "\n";
     defs << "#define NPRO " << pro.args.size() << "\n#define MJT_PRO_SCALARS " << scal.str() << "\n"
          << "#define MJT_RD(dst, off) do { const index_t o_ = (off); " << loads.str()
          << "_Pragma(\"unroll\") for (int k = 0; k < VEC; k++) { " << elems.str() << fused_emit_ops(d, false) << "(dst).v[k] = (TX)(v"

@@ -616,9 +616,43 @@ def test_fused_reduce_prologue(gpu):
     assert jt.executor_stats["fused_reduces"] == before + 1 and s.dtype == "bfloat16"
     want = O.BF16(O.f32_to_bf16_bits(O.BF16(xb.raw()).to_f32().astype(np.float64).sum(1).astype(np.float32))).to_f32()
     assert np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max()
-    # a tensor broadcast inside the group is not taken as a prologue: two kernels, same result
-    sc = rng.standard_normal((37, 1)).astype(np.float32)
+    # a tensor broadcast along an axis that is kept is not taken as a prologue: two kernels, same result
+    sc = rng.standard_normal((1, x.shape[1])).astype(np.float32)
     before = dict(jt.executor_stats)
     got = (jt.array(x) * jt.array(sc)).sum(1).data
     assert jt.executor_stats["fused_reduces"] == before["fused_reduces"]
     assert np.allclose(got, (x.astype(np.float64) * sc).sum(1), rtol=1e-5, atol=1e-4)
+
+
+def test_fused_reduce_with_per_output_inputs(gpu):
+    """Prologue inputs broadcast along exactly the reduced axes (the mean inside a variance, the maximum
+    inside a softmax) are read once per output: the variance of a
+    normalisation is one launch (the pattern of python/jittor/test/test_new_fused_op.py:24-40)."""
+    rng = np.random.default_rng(41)
+    x = rng.standard_normal((33, 7, 130)).astype(np.float32)
+    X = x.astype(np.float64)
+    for dims in ([2], [0], [1, 2], [0, 2]):
+        v = jt.array(x)
+        before = dict(jt.executor_stats)
+        mean = v.mean(dims, keepdims=True)
+        var = ((v - mean) * (v - mean)).mean(dims, keepdims=True)
+        y = (v - mean) / (var + 1e-5).sqrt()
+        got = y.data
+        assert jt.executor_stats["fused_reduces"] - before["fused_reduces"] == 1          # the variance
+        ax = tuple(dims)
+        want = (X - X.mean(ax, keepdims=True)) / np.sqrt(X.var(ax, keepdims=True) + 1e-5)
+        assert np.allclose(got, want, rtol=1e-4, atol=1e-5), dims
+    # softmax over the last axis
+    v = jt.array(x)
+    m = v.max(2, keepdims=True)
+    e = (v - m).exp()
+    s = e.sum(2, keepdims=True)
+    got = (e / s).data
+    ex = np.exp(X - X.max(2, keepdims=True))
+    assert np.allclose(got, ex / ex.sum(2, keepdims=True), rtol=1e-5, atol=1e-7)
+    # an input broadcast along other axes than the reduced ones stays a separate kernel
+    w = rng.standard_normal((1, 7, 1)).astype(np.float32)
+    before = dict(jt.executor_stats)
+    got = (jt.array(x) * jt.array(w)).sum(2).data
+    assert jt.executor_stats["fused_reduces"] == before["fused_reduces"]
+    assert np.allclose(got, (X * w).sum(2), rtol=1e-5, atol=1e-4)

@@ -280,8 +280,8 @@ def test_grad_graph_is_built_from_path_ops():
 
 
 def test_fused_reduce_descriptor_checks_and_specialisation(compile_only):
-    """mjt_fused_reduce: one output var (the reduce input), full-shape inputs only; the kernel with the
-    prologue compiles for gfx950."""
+    """mjt_fused_reduce: one output var (the reduce input); inputs are full-shape or broadcast along exactly
+    the reduced axes (one value per output); the kernel with the prologue compiles for gfx950."""
     L = compile_only
     lib = L.load()
     V, F = L.FusedVar, L.FusedOp
@@ -314,8 +314,14 @@ def test_fused_reduce_descriptor_checks_and_specialisation(compile_only):
     ty0 = L.tensor(0x3000, "float32", [256])
     assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty0), L.OP_CODE["maximum"], 0b01) == 0
     assert L.last_kernel().startswith("mjt_reduce_col_maximum")
-    d, keep = desc(mask=0b01)                                    # a broadcast tensor input
+    d, keep = desc(mask=0b01)                                    # broadcast along a kept axis
     assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty), L.OP_CODE["add"], 0b10) == -2
+    d, keep = desc(mask=0b10)                                    # one value per output: row and column kernels
+    assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty), L.OP_CODE["add"], 0b10) == 0
+    assert L.last_kernel().startswith("mjt_reduce_row_add") and "_pro" in L.last_kernel()
+    d, keep = desc(mask=0b01)
+    assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty0), L.OP_CODE["add"], 0b01) == 0
+    assert L.last_kernel().startswith("mjt_reduce_col_add")
     d, keep = desc(outputs=2)
     assert lib.mjt_fused_reduce(ctypes.byref(d), ctypes.byref(ty), L.OP_CODE["add"], 0b10) == -1
     d, keep = desc()
