@@ -4,68 +4,94 @@
 // python/jittor/src/ops/reindex_reduce_op.cc:93-131).
 //
 // Scattered global atomics run at about 2e10 updates/s on this chip whatever
-// their scope, and a hot bin serialises them further, so this path uses none
-// on its main route.  The bin axis is cut into buckets of WBINS bins (one
-// bucket fits in LDS):
-//   sample  a strided sample of the indices votes for the bucket that receives
-//           the most updates (the "hot" bucket);
-//   main    every workgroup streams its share of (idx, y): updates of the hot
-//           bucket are applied to a private LDS copy of that bucket, all other
-//           updates are appended to per-(workgroup, bucket) lists in scratch
-//           memory (list cursors are LDS counters); at the end the private
-//           copy and the list lengths are written out;
-//   cold    workgroup (bucket, split) folds the lists of its bucket into a
-//           private LDS copy and writes it out
-//           (the number of workgroups per bucket follows the bucket's population;
-//           entries that did not fit a list -- rare: a second hot region -- sit in
-//           one overflow list that the first workgroup of each bucket scans);
+// their scope, and a hot bin serialises them further, so this path uses none.
+// The bin axis is cut into buckets of WBINS bins (one bucket fits in LDS):
+//   main    every workgroup streams its share of (idx, y) in rounds of
+//           NP*EPT elements.  A sample of its own indices picks the bucket
+//           that receives most of its updates (its "hot" bucket); updates of
+//           that bucket go to a private LDS copy.  All other updates are put
+//           into an LDS staging area (a wave takes its slots of a round with
+//           one LDS atomic), and a few waves that load no input append what
+//           the previous round staged to the workgroup's per-bucket lists in
+//           scratch memory.  At the end the private copy, the list lengths and
+//           the hot bucket's number are written out;
+//   plan    one workgroup sums the list lengths per bucket and lays out the
+//           work of the cold pass;
+//   cold    a fixed number of workgroups walks the work items.  A list item
+//           (bucket, split) folds the lists of its bucket written by main
+//           workgroups split, split + nsplit, ... into a private LDS copy and
+//           writes it out; the number of list items per bucket follows the
+//           bucket's population.  Entries that did not fit a list (rare: a
+//           second hot region) sit in per-workgroup overflow lists that item
+//           (bucket, 0) scans.  A merge item merges a segment of the private
+//           copies of 16 main workgroups that had the same hot bucket;
 //   final   x[bin] = merge of the partial copies of its bucket (plain stores:
 //           x needs no prior fill).
+// Workgroups of one launch share nothing, so no buffer has to be cleared
+// beforehand and no global atomic is issued.
 //
 // Supplied by the host: TX (4-byte element type), TE (index type), WBINS
-// (power of two), LOGW, NBMAX (bound on the bucket count), NTHREADS, NHOT (bins kept in
-// registers), MODE (0 add,
-// 1 maximum, 2 minimum),
+// (power of two), LOGW, NBMAX (power of two >= bucket count, <= NTHREADS),
+// NTHREADS, NFLUSH (threads that only store), EPT (elements per thread and
+// round, multiple of 4), SCAP (entries of each of the two staging areas), MODE (0 add, 1 maximum, 2 minimum), ACC64, COLD_TARGET,
 // IDENT_BITS (bit pattern of the identity).
 
-struct Params { void* a[16]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
+struct Params { void* a[20]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
 // a[0] x          a[1] y           a[2] idx        a[3] n          a[4] bins
-// a[5] control    a[6] per (elements per main workgroup)           a[7] G1 (main workgroups)
-// a[8] NB (buckets)  a[9] CAP (list capacity)  a[10] counts  a[11] lists
-// a[12] partial_main  a[13] partial_cold  a[14] unused  a[15] overflow list
-// control: int[0] hot bucket, unsigned[1] overflow count, unsigned[64 + b] list entries of bucket b
+// a[5] plan (written by the plan kernel)
+// a[6] per (elements per main workgroup)           a[7] G1 (main workgroups)
+// a[8] NB (buckets)  a[9] CAP (list capacity)  a[10] counts[G1][NB]  a[11] lists[NB][G1][CAP]
+// a[12] partial_main[G1][WBINS]  a[13] partial_cold[items][WBINS]  a[14] hotof[G1]
+// a[15] overflow lists[G1][per]   a[16] novf[G1]
 
 struct mjt_pair { int bin; TX val; };
 
+// TA: type partial results are merged in.  TW: type of the private copies in LDS.
+// add: a float LDS add costs 3 cycles per lane on this chip, a double one 0.25 (0.6 with the same-address
+// conflicts of a Zipf head), so float sums are kept in double: faster, and each partial sum is rounded
+// once, when it is written out.
+// maximum / minimum: the copies hold order-preserving integer keys, so one integer LDS atomic serves every
+// sign; NaN updates are dropped (std::max(cur, v) keeps cur when v is NaN).
+#if ACC64
+typedef double TA;
+#else
+typedef TX TA;
+#endif
 #if MODE == 0
-#define LDS_UPDATE(addr, v) atomicAdd((addr), (v))
-#define GLB_UPDATE(addr, v) mjt_atomic_add<TX>((addr), (v))
+typedef TA TW;
 #define MERGE2(a, b) ((a) + (b))
-#elif MODE == 1
-#define LDS_UPDATE(addr, v) mjt_lds_max((addr), (v))
-#define GLB_UPDATE(addr, v) mjt_atomic_maximum<TX>((addr), (v))
+__device__ __forceinline__ TW mjt_win_from(TX v) { return (TW)v; }
+__device__ __forceinline__ TX mjt_win_read(TW w) { return (TX)w; }
+__device__ __forceinline__ void mjt_win_update(TW* a, TX v) { atomicAdd(a, (TW)v); }
+#else
+typedef int TW;
+#if MODE == 1
 #define MERGE2(a, b) (((a) < (b)) ? (b) : (a))
 #else
-#define LDS_UPDATE(addr, v) mjt_lds_min((addr), (v))
-#define GLB_UPDATE(addr, v) mjt_atomic_minimum<TX>((addr), (v))
 #define MERGE2(a, b) (((b) < (a)) ? (b) : (a))
 #endif
-
-// std::max(cur, v) keeps cur when v is NaN: NaN updates are dropped
-__device__ __forceinline__ void mjt_lds_max(float* a, float v) {
-    if (v != v) return;
-    unsigned b = __float_as_uint(v);
-    if (b >> 31) atomicMin((unsigned*)a, b); else atomicMax((int*)a, (int)b);
+__device__ __forceinline__ int mjt_win_from(float v) {
+    const int b = __float_as_int(v);
+    return b ^ ((b >> 31) & 0x7fffffff);
 }
-__device__ __forceinline__ void mjt_lds_min(float* a, float v) {
-    if (v != v) return;
-    unsigned b = __float_as_uint(v);
-    if (b >> 31) atomicMax((unsigned*)a, b); else atomicMin((int*)a, (int)b);
+__device__ __forceinline__ int mjt_win_from(int v) { return v; }
+__device__ __forceinline__ int mjt_win_from(unsigned v) { return (int)(v ^ 0x80000000u); }
+__device__ __forceinline__ void mjt_win_to(int k, float& v) { v = __int_as_float(k ^ ((k >> 31) & 0x7fffffff)); }
+__device__ __forceinline__ void mjt_win_to(int k, int& v) { v = k; }
+__device__ __forceinline__ void mjt_win_to(int k, unsigned& v) { v = (unsigned)k ^ 0x80000000u; }
+__device__ __forceinline__ TX mjt_win_read(TW w) { TX v; mjt_win_to(w, v); return v; }
+__device__ __forceinline__ bool mjt_is_nan(float v) { return v != v; }
+__device__ __forceinline__ bool mjt_is_nan(int) { return false; }
+__device__ __forceinline__ bool mjt_is_nan(unsigned) { return false; }
+__device__ __forceinline__ void mjt_win_update(TW* a, TX v) {
+    if (mjt_is_nan(v)) return;
+#if MODE == 1
+    atomicMax(a, mjt_win_from(v));
+#else
+    atomicMin(a, mjt_win_from(v));
+#endif
 }
-__device__ __forceinline__ void mjt_lds_max(int* a, int v) { atomicMax(a, v); }
-__device__ __forceinline__ void mjt_lds_min(int* a, int v) { atomicMin(a, v); }
-__device__ __forceinline__ void mjt_lds_max(unsigned* a, unsigned v) { atomicMax(a, v); }
-__device__ __forceinline__ void mjt_lds_min(unsigned* a, unsigned v) { atomicMin(a, v); }
+#endif
 
 __device__ __forceinline__ TX mjt_ident() {
     TX t;
@@ -74,341 +100,471 @@ __device__ __forceinline__ TX mjt_ident() {
     return t;
 }
 
-// ---- sample -------------------------------------------------------------------------
-extern "C" __global__ __launch_bounds__(1024) void ENTRY_SAMPLE(Params p) {
-    const TE* __restrict__ ip = (const TE*)p.a[2];
-    const long long n = (long long)(unsigned long long)p.a[3];
-    const long long bins = (long long)(unsigned long long)p.a[4];
-    int* control = (int*)p.a[5];
-    const int NB = (int)(unsigned long long)p.a[8];
-    __shared__ int votes[1024];
-    __shared__ int best_votes, best_slot;
-    const int group = (NB + 1023) / 1024;            // buckets per counter when there are more than 1024
-    votes[threadIdx.x] = 0;
-    if (threadIdx.x == 0) { best_votes = -1; best_slot = 0; }
-    __syncthreads();
-    // 32 runs of 64 consecutive indices spread over the input (a lone workgroup can pull only a few
-    // tens of GB/s, and every isolated 4-byte sample would cost a whole 128-byte line)
-    long long b[2];
-    const long long runs = 32, run_stride = n / runs;
+// Inclusive scan of one 64-bit value per thread over the workgroup (NTHREADS <= 1024): shuffle scan
+// inside each wave, then the wave totals through wsum (16 words of LDS that nobody else touches between
+// two barriers around this call).  Contains one barrier.
+__device__ __forceinline__ unsigned long long mjt_block_scan_value(unsigned long long v, unsigned long long* wsum) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-    for (int k = 0; k < 2; k++) {
-        const long long r = k * 16 + (threadIdx.x >> 6);
-        const long long pos = run_stride >= 64 ? r * run_stride + (threadIdx.x & 63) : (long long)threadIdx.x + k * 1024;
-        b[k] = pos < n ? (long long)ip[pos] : -1;
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long o = __shfl_up(v, off, 64);
+        if (lane >= off) v += o;
     }
-#pragma unroll
-    for (int k = 0; k < 2; k++)
-        if (b[k] >= 0 && b[k] < bins) atomicAdd(&votes[(int)(b[k] >> LOGW) / group], 1);
+    if (lane == 63) wsum[wave] = v;
     __syncthreads();
-    atomicMax(&best_votes, votes[threadIdx.x]);
-    __syncthreads();
-    if (votes[threadIdx.x] == best_votes) atomicMax(&best_slot, (int)threadIdx.x);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        control[0] = best_slot * group;
-        control[1] = 0;
-    }
-    for (int t = threadIdx.x; t < NB; t += 1024) control[64 + t] = 0;
+    unsigned long long base = 0;
+    for (int w = 0; w < wave; w++) base += wsum[w];
+    return v + base;
 }
 
 // ---- main ---------------------------------------------------------------------------
+constexpr int NP = NTHREADS - NFLUSH;                        // threads that load input; the others append to the lists
+
 extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
     const TX* __restrict__ yp = (const TX*)p.a[1];
     const TE* __restrict__ ip = (const TE*)p.a[2];
     const long long n = (long long)(unsigned long long)p.a[3];
     const long long bins = (long long)(unsigned long long)p.a[4];
-    int* control = (int*)p.a[5];
     const long long per = (long long)(unsigned long long)p.a[6];
     const int NB = (int)(unsigned long long)p.a[8];
     const unsigned CAP = (unsigned)(unsigned long long)p.a[9];
     unsigned* __restrict__ counts = (unsigned*)p.a[10];
     mjt_pair* __restrict__ lists = (mjt_pair*)p.a[11];
     TX* __restrict__ pmain = (TX*)p.a[12];
-    mjt_pair* __restrict__ ovf = (mjt_pair*)p.a[15];
-    __shared__ TX win[WBINS];
-    __shared__ unsigned cursor[NBMAX];
-    __shared__ unsigned cand[NTHREADS];
-    __shared__ int hotbin_s[NHOT];
-    const long long hot = control[0];
+    int* __restrict__ hotof = (int*)p.a[14];
+    mjt_pair* __restrict__ ovf = (mjt_pair*)p.a[15] + (size_t)blockIdx.x * per;
+    unsigned* __restrict__ novf = (unsigned*)p.a[16];
+    __shared__ TW win[WBINS];
+    __shared__ mjt_pair staging[2][SCAP];  // updates of a round on their way to the lists, by round parity
+    __shared__ unsigned cursor[NBMAX];     // list lengths (votes during the sample)
+    __shared__ unsigned best, staged[3], ovf_len;        // staged: entries of a round, by round number mod 3
     const TX ident = mjt_ident();
     const long long begin = (long long)blockIdx.x * per;
     const long long end = begin + per < n ? begin + per : n;
     const int lane = threadIdx.x & 63;
 
-    // Phase 0: the NHOT most frequent bins of the hot bucket in the first 4*NTHREADS elements of this
-    // workgroup's share.  Same-address LDS atomics serialise, so these bins are accumulated in
-    // registers instead and folded into the private copy once per wave at the end.
-    unsigned* hist = (unsigned*)win;
-    for (int t = threadIdx.x; t < WBINS; t += NTHREADS) hist[t] = 0;
-    for (int t = threadIdx.x; t < NB; t += NTHREADS) cursor[t] = 0;
+    for (int t = threadIdx.x; t < NBMAX; t += NTHREADS) cursor[t] = 0;
+    for (int t = threadIdx.x; t < WBINS; t += NTHREADS) win[t] = mjt_win_from(ident);
+    if (threadIdx.x == 0) { best = 0; staged[0] = 0; staged[1] = 0; staged[2] = 0; ovf_len = 0; }
     __syncthreads();
-    {
-        const long long i0 = begin + (long long)threadIdx.x * 4;
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const long long b = i0 + k < end ? (long long)ip[i0 + k] : -1;
-            if (b >= 0 && b < bins && (b >> LOGW) == hot) atomicAdd(&hist[b & (WBINS - 1)], 1u);
-        }
+    // the hot bucket: vote of 8 runs of 64 consecutive indices spread over this workgroup's share
+    if (threadIdx.x < 512) {
+        const long long run = threadIdx.x >> 6;
+        const long long pos = begin + run * ((end - begin) >> 3) + (threadIdx.x & 63);
+        const long long b = pos < end ? (long long)ip[pos] : -1;
+        if ((unsigned long long)b < (unsigned long long)bins) atomicAdd(&cursor[(int)(b >> LOGW)], 1u);
     }
     __syncthreads();
-    {
-        unsigned best = 0;                                   // (count << LOGW) | local bin
-        for (int t = threadIdx.x; t < WBINS; t += NTHREADS) {
-            const unsigned c = (hist[t] << LOGW) | (unsigned)t;
-            best = c > best ? c : best;
-        }
-        cand[threadIdx.x] = best;
-    }
+    for (int t = threadIdx.x; t < NB; t += NTHREADS)
+        if (cursor[t]) atomicMax(&best, (cursor[t] << 12) | (unsigned)(4095 - t));   // ties: the lowest bucket
     __syncthreads();
-    if (threadIdx.x < 64) {
-        unsigned mine[NTHREADS / 64];
-#pragma unroll
-        for (int k = 0; k < NTHREADS / 64; k++) mine[k] = cand[k * 64 + lane];
-        for (int r = 0; r < NHOT; r++) {
-            unsigned m = 0;
-#pragma unroll
-            for (int k = 0; k < NTHREADS / 64; k++) m = mine[k] > m ? mine[k] : m;
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) {
-                const unsigned o = (unsigned)__shfl_xor((int)m, off, 64);
-                m = o > m ? o : m;
-            }
-#pragma unroll
-            for (int k = 0; k < NTHREADS / 64; k++) if (mine[k] == m) mine[k] = 0;
-            // at least 1/128 of the sample, else the slot stays unused
-            if (lane == 0) hotbin_s[r] = (m >> LOGW) >= (4 * NTHREADS) / 128 ? (int)(m & (WBINS - 1)) : -1;
-        }
-    }
-    __syncthreads();
-    int hotbin[NHOT];
-    TX hotacc[NHOT];
-#pragma unroll
-    for (int r = 0; r < NHOT; r++) { hotbin[r] = hotbin_s[r]; hotacc[r] = ident; }
-    for (int t = threadIdx.x; t < WBINS; t += NTHREADS) win[t] = ident;
+    const unsigned hot = best ? 4095u - (best & 4095u) : 0u;
+    for (int t = threadIdx.x; t < NBMAX; t += NTHREADS) cursor[t] = 0;
     __syncthreads();
 
-    mjt_pair* __restrict__ mylists = lists + (size_t)blockIdx.x * NB * CAP;
-    auto update = [&](long long b, TX v) {
-        if (b < 0 || b >= bins) return;                      // overflow: skipped
-        const long long bucket = b >> LOGW;
-        const int local = (int)(b & (WBINS - 1));
-        if (bucket == hot) {
-            bool taken = false;
-#pragma unroll
-            for (int r = 0; r < NHOT; r++) {
-                const bool hit = local == hotbin[r];
-#if MODE == 0
-                hotacc[r] = hit ? hotacc[r] + v : hotacc[r];
-#elif MODE == 1
-                hotacc[r] = (hit && hotacc[r] < v) ? v : hotacc[r];     // false for NaN: dropped
-#else
-                hotacc[r] = (hit && v < hotacc[r]) ? v : hotacc[r];
-#endif
-                taken = taken || hit;
-            }
-            if (!taken) { LDS_UPDATE(&win[local], v); }
-        } else {
-            const unsigned pos = atomicAdd(&cursor[bucket], 1u);
-            mjt_pair e;
-            if (pos < CAP) {
-                e.bin = local;
-                e.val = v;
-                mylists[(size_t)bucket * CAP + pos] = e;
-            } else {
-                const unsigned g = atomicAdd((unsigned*)control + 1, 1u);
-                e.bin = (int)b;
-                e.val = v;
-                ovf[g] = e;
-            }
-        }
+    // lists of one bucket are neighbours in memory: the cold item that folds them then touches few pages
+    mjt_pair* __restrict__ mylists = lists + (size_t)blockIdx.x * CAP;
+    const size_t bucket_stride = (size_t)gridDim.x * CAP;
+    // next entry of its bucket's list, or of the overflow list once that is full
+    auto append = [&](mjt_pair e) {
+        const int b = e.bin >> LOGW;
+        const unsigned pos = atomicAdd(&cursor[b], 1u);
+        if (pos < CAP) mylists[(size_t)b * bucket_stride + pos] = e;
+        else ovf[atomicAdd(&ovf_len, 1u)] = e;
     };
-    // per is a multiple of 4*NTHREADS and the bases are 16-byte aligned: full vectors first
-    long long i = begin + (long long)threadIdx.x * 4;
-    for (; i + 3 < end; i += (long long)NTHREADS * 4) {
-        mjt_pack<TX, 4> v;
-        mjt_pack<TE, 4> id;
-        mjt_load_nt(v, yp + i);
-        mjt_load_nt(id, ip + i);
-#pragma unroll
-        for (int k = 0; k < 4; k++) update((long long)id.v[k], v.v[k]);
-    }
-    for (; i < end; i++) update((long long)ip[i], yp[i]);    // ragged tail of the last workgroup
-    // fold the register accumulators: xor-shuffle tree, then one LDS update per wave and bin
-#pragma unroll
-    for (int r = 0; r < NHOT; r++) {
-        TX a = hotacc[r];
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            int ob = __shfl_xor(*reinterpret_cast<int*>(&a), off, 64);
-            const TX o = *reinterpret_cast<TX*>(&ob);
-            a = MERGE2(a, o);
+    // Rounds of NP*EPT elements, one barrier each.  Producers (threads < NP) load input, apply the updates of
+    // the hot bucket to the private copy and put every other update into the staging area of the round's
+    // parity; flushers (the last NFLUSH threads) append what the previous round staged to the lists and load
+    // nothing.  The split matters: memory operations of a wave complete in order, so in a wave that both
+    // loads and stores every wait for loaded data is also a wait for the acknowledgement of earlier stores.
+    const long long end4 = begin + ((end - begin) & ~3ll);
+    constexpr long long STEP = (long long)NP * EPT;
+    const int rounds = 2 * (int)((end4 - begin + 2 * STEP - 1) / (2 * STEP)) + (end4 < end ? 1 : 0);
+    if (threadIdx.x >= NP) {
+        int prev3 = 2, next3 = 1;                             // (r - 1) mod 3, (r + 1) mod 3
+        for (int r = 0; r <= rounds; r++) {
+            if (r > 0) {                                      // drain what round r-1 staged
+                const unsigned total = staged[prev3];
+                const unsigned m = total < SCAP ? total : SCAP;
+                for (unsigned t = threadIdx.x - NP; t < m; t += NFLUSH) append(staging[(r - 1) & 1][t]);
+            }
+            if (threadIdx.x == NP) staged[next3] = 0;         // drained one round ago, used from the next round on
+            prev3 = prev3 == 2 ? 0 : prev3 + 1;
+            next3 = next3 == 2 ? 0 : next3 + 1;
+            __syncthreads();                                  // (r == rounds: matches the producers' closing barrier)
         }
-        if (lane == 0 && hotbin[r] >= 0) { LDS_UPDATE(&win[hotbin[r]], a); }
+    } else {
+        constexpr unsigned SKIP = 0xffffffffu;                // index of an element that takes no part: its bucket is none
+        // one round of a producer over EPT elements; cnt = staged[round number mod 3]
+        auto round = [&](int r, unsigned* cnt, const unsigned (&idx)[EPT], const TX (&val)[EPT]) {
+            // hot bucket: private copy.  Every other element takes a staging slot: the wave counts them with
+            // ballots and takes all its slots of the round with a single LDS atomic.
+            bool cold[EPT];
+            unsigned long long mask[EPT];
+            unsigned before[EPT], total = 0;
+#pragma unroll
+            for (int k = 0; k < EPT; k++) {
+                const unsigned bucket = idx[k] >> LOGW;
+                if (bucket == hot) mjt_win_update(&win[idx[k] & (WBINS - 1)], val[k]);
+                cold[k] = bucket != hot && bucket < (unsigned)NB;
+                mask[k] = __builtin_amdgcn_ballot_w64(cold[k]);
+                before[k] = total;
+                total += (unsigned)__popcll(mask[k]);
+            }
+            unsigned base = 0;
+            if (total) {
+                if (lane == 0) base = atomicAdd(cnt, total);
+                base = (unsigned)__shfl((int)base, 0, 64);
+            }
+#pragma unroll
+            for (int k = 0; k < EPT; k++) {
+                if (cold[k]) {
+                    const unsigned slot = base + before[k] +
+                        __builtin_amdgcn_mbcnt_hi((unsigned)(mask[k] >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask[k], 0u));
+                    mjt_pair e;
+                    e.bin = (int)idx[k];
+                    e.val = val[k];
+                    if (slot < SCAP) staging[r & 1][slot] = e;
+                    else append(e);                          // more than the staging area holds: straight to memory
+                }
+            }
+            __syncthreads();
+        };
+        // The loads of a round are issued two rounds ahead and unconditionally (a load under a branch would
+        // make every later wait a wait for all loads in flight): past the end they re-read the start of the
+        // input and are ignored.
+        mjt_pack<TX, 4> vva[EPT / 4], vvb[EPT / 4];
+        mjt_pack<TE, 4> ida[EPT / 4], idb[EPT / 4];
+        auto fetch = [&](long long r0, mjt_pack<TX, 4> (&vv)[EPT / 4], mjt_pack<TE, 4> (&id)[EPT / 4]) {
+#pragma unroll
+            for (int v = 0; v < EPT / 4; v++) {
+                const long long i = r0 + ((long long)v * NP + threadIdx.x) * 4;
+                const long long ic = i < end4 ? i : 0;
+                mjt_load_nt(vv[v], yp + ic);
+                mjt_load_nt(id[v], ip + ic);
+            }
+        };
+        auto step = [&](int r, unsigned* cnt, long long r0, mjt_pack<TX, 4> (&vv)[EPT / 4], mjt_pack<TE, 4> (&id)[EPT / 4]) {
+            unsigned idx[EPT];
+            TX val[EPT];
+#pragma unroll
+            for (int v = 0; v < EPT / 4; v++) {
+                const long long i = r0 + ((long long)v * NP + threadIdx.x) * 4;
+                const bool present = i < end4;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    bool inside;                              // overflow (index outside [0, bins)): skipped
+                    if constexpr (sizeof(TE) == 4) inside = (unsigned)id[v].v[k] < (unsigned)bins;   // bins < 2^31
+                    else inside = (unsigned long long)id[v].v[k] < (unsigned long long)bins;
+                    idx[v * 4 + k] = (present && inside) ? (unsigned)id[v].v[k] : SKIP;
+                    val[v * 4 + k] = vv[v].v[k];
+                }
+            }
+            fetch(r0 + 2 * STEP, vv, id);
+            round(r, cnt, idx, val);
+        };
+        fetch(begin, vva, ida);
+        fetch(begin + STEP, vvb, idb);
+        int r = 0, r3 = 0;                                    // r3 = r mod 3
+        for (long long r0 = begin; r0 < end4; r0 += 2 * STEP) {
+            step(r++, &staged[r3], r0, vva, ida);
+            r3 = r3 == 2 ? 0 : r3 + 1;
+            step(r++, &staged[r3], r0 + STEP, vvb, idb);      // possibly past the end: a round of skipped elements
+            r3 = r3 == 2 ? 0 : r3 + 1;
+        }
+        if (end4 < end) {                                     // the last 1..3 elements of the input
+            unsigned idx[EPT];
+            TX val[EPT];
+#pragma unroll
+            for (int k = 0; k < EPT; k++) { idx[k] = SKIP; val[k] = ident; }
+            const long long i = end4 + threadIdx.x;
+            if (i < end) {
+                const long long b = (long long)ip[i];
+                idx[0] = (unsigned long long)b < (unsigned long long)bins ? (unsigned)b : SKIP;
+                val[0] = yp[i];
+            }
+            round(r, &staged[r3], idx, val);
+        }
+        __syncthreads();                                      // the flushers have drained the last round
     }
     __syncthreads();
     TX* __restrict__ out = pmain + (size_t)blockIdx.x * WBINS;
     for (int t = threadIdx.x * 4; t < WBINS; t += NTHREADS * 4) {
         mjt_pack<TX, 4> o;
 #pragma unroll
-        for (int k = 0; k < 4; k++) o.v[k] = win[t + k];
+        for (int k = 0; k < 4; k++) o.v[k] = mjt_win_read(win[t + k]);
         mjt_store(out + t, o);
     }
     for (int t = threadIdx.x; t < NB; t += NTHREADS) {
-        const unsigned c = cursor[t] < CAP ? cursor[t] : CAP;
-        counts[(size_t)blockIdx.x * NB + t] = c;
-        if (c) atomicAdd((unsigned*)control + 64 + t, c);     // bucket populations, read by the cold plan
+        const unsigned c = cursor[t];
+        counts[(size_t)blockIdx.x * NB + t] = c < CAP ? c : CAP;
+    }
+    if (threadIdx.x == 0) {
+        hotof[blockIdx.x] = (int)hot;
+        novf[blockIdx.x] = ovf_len;
     }
 }
 
-
-// Work plan of the cold pass, recomputed identically by every workgroup that needs it:
-// bucket b is folded by nsplit[b] workgroups (list entries / COLD_TARGET, at least 1, at most
-// G1), the hot bucket by none; first[b] is the index of its first partial copy.
+// Work plan of the cold pass, computed identically by every cold workgroup.  Bucket b has nsplit[b] list
+// items (list entries / COLD_TARGET, at least 1 when it has entries, at most G1), each producing one
+// partial copy, followed by nmerge[b] * MSEG merge items: the partial copies of MERGE_ROWS main workgroups
+// whose hot bucket it was are merged into one, MSEG items sharing the work by segments of MBINS bins (one
+// compute unit pulls little more than 100 GB/s: an item should not read more than about 100 KB).
+// first[b] is the number of the bucket's first item, pfirst[b] of its first partial copy; first[NBMAX] and
+// pfirst[NBMAX] are the totals.
+constexpr int MERGE_ROWS = 16;
+constexpr int MBINS = WBINS < 2048 ? WBINS : 2048;
+constexpr int MSEG = WBINS / MBINS;
 struct mjt_plan {
     unsigned nsplit[NBMAX];
+    unsigned nmerge[NBMAX];
     unsigned first[NBMAX + 1];
+    unsigned pfirst[NBMAX + 1];
 };
-// In-place inclusive scan of arr[0..n), n <= blockDim.x <= 1024: xor-free shuffle scan inside each
-// wave, then the wave totals.
-__device__ __forceinline__ void mjt_block_scan(unsigned* arr, int n, unsigned* wsum) {
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    unsigned v = t < n ? arr[t] : 0u;
+
+__device__ __forceinline__ void mjt_make_plan(mjt_plan& plan, const unsigned* __restrict__ counts,
+                                              const int* __restrict__ hotof, int G1, int NB, unsigned long long* wsum) {
+    for (int b = threadIdx.x; b < NBMAX; b += NTHREADS) { plan.nsplit[b] = 0; plan.nmerge[b] = 0; }   // populations first
+    __syncthreads();
+    {
+        const int b = threadIdx.x & (NBMAX - 1);
+        unsigned sum = 0;
+        if (b < NB) {                                         // independent loads, several in flight
+            constexpr int RSTEP = NTHREADS / NBMAX;
+            for (int r0 = threadIdx.x / NBMAX; r0 < G1; r0 += 8 * RSTEP) {
+                unsigned c[8];
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const unsigned o = (unsigned)__shfl_up((int)v, off, 64);
-        if (lane >= off) v += o;
+                for (int u = 0; u < 8; u++) c[u] = r0 + u * RSTEP < G1 ? counts[(size_t)(r0 + u * RSTEP) * NB + b] : 0u;
+#pragma unroll
+                for (int u = 0; u < 8; u++) sum += c[u];
+            }
+        }
+        if (sum) atomicAdd(&plan.nsplit[b], sum);
+        for (int j = threadIdx.x; j < G1; j += NTHREADS) atomicAdd(&plan.nmerge[hotof[j]], 1u);
     }
-    if (lane == 63) wsum[wave] = v;
     __syncthreads();
-    unsigned base = 0;
-    for (int w = 0; w < wave; w++) base += wsum[w];
-    if (t < n) arr[t] = v + base;
-    __syncthreads();
-}
-
-__device__ __forceinline__ void mjt_make_plan(mjt_plan& plan, const unsigned* __restrict__ pop, int G1, int NB, int hot,
-                                              unsigned* wsum) {
-    for (int b = threadIdx.x; b < NB; b += blockDim.x) {
-        unsigned k = b == hot ? 0u : (pop[b] + COLD_TARGET - 1) / COLD_TARGET;
-        if (b != hot && k < 1) k = 1;
+    const int b = threadIdx.x;
+    unsigned k = 0, m = 0;
+    if (b < NBMAX) {
+        k = (plan.nsplit[b] + COLD_TARGET - 1) / COLD_TARGET;
         if (k > (unsigned)G1) k = (unsigned)G1;
+        m = (plan.nmerge[b] + MERGE_ROWS - 1) / MERGE_ROWS;
+    }
+    // items in the low word, partial copies in the high word
+    const unsigned long long mine = (unsigned long long)(k + m * MSEG) | ((unsigned long long)(k + m) << 32);
+    const unsigned long long incl = mjt_block_scan_value(mine, wsum);
+    if (b < NBMAX) {
         plan.nsplit[b] = k;
-        plan.first[b + 1] = k;
+        plan.nmerge[b] = m;
+        plan.first[b] = (unsigned)incl - (k + m * MSEG);
+        plan.pfirst[b] = (unsigned)(incl >> 32) - (k + m);
     }
-    if (threadIdx.x == 0) plan.first[0] = 0;
+    if (b == NBMAX - 1) {
+        plan.first[NBMAX] = (unsigned)incl;
+        plan.pfirst[NBMAX] = (unsigned)(incl >> 32);
+    }
     __syncthreads();
-    if (NB <= (int)blockDim.x) {
-        mjt_block_scan(plan.first + 1, NB, wsum);            // first[b + 1] = nsplit[0] + ... + nsplit[b]
-    } else {
-        if (threadIdx.x == 0)
-            for (int b = 0; b < NB; b++) plan.first[b + 1] += plan.first[b];
-        __syncthreads();
-    }
 }
 
-// ---- cold: workgroup (bucket, split) folds the lists of main workgroups split, split+nsplit, ... ----------
+// ---- plan: one workgroup computes the work plan of the cold pass -------------------------------------------
+// layout of the plan in memory, in words: nsplit[NBMAX], nmerge[NBMAX], first[NBMAX + 1], pfirst[NBMAX + 1], any_ovf
+extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_PLAN(Params p) {
+    unsigned* __restrict__ planout = (unsigned*)p.a[5];
+    const int G1 = (int)(unsigned long long)p.a[7];
+    const int NB = (int)(unsigned long long)p.a[8];
+    const unsigned* __restrict__ counts = (const unsigned*)p.a[10];
+    const int* __restrict__ hotof = (const int*)p.a[14];
+    const unsigned* __restrict__ novf = (const unsigned*)p.a[16];
+    __shared__ mjt_plan plan;
+    __shared__ unsigned long long wsum[16];
+    __shared__ unsigned any_ovf;
+    if (threadIdx.x == 0) any_ovf = 0;
+    mjt_make_plan(plan, counts, hotof, G1, NB, wsum);
+    for (int w = threadIdx.x; w < G1; w += NTHREADS)
+        if (novf[w]) any_ovf = 1;
+    __syncthreads();
+    for (int t = threadIdx.x; t < NBMAX; t += NTHREADS) {
+        planout[t] = plan.nsplit[t];
+        planout[NBMAX + t] = plan.nmerge[t];
+    }
+    for (int t = threadIdx.x; t <= NBMAX; t += NTHREADS) {
+        planout[2 * NBMAX + t] = plan.first[t];
+        planout[3 * NBMAX + 1 + t] = plan.pfirst[t];
+    }
+    if (threadIdx.x == 0) planout[4 * NBMAX + 2] = any_ovf;
+}
+
+// ---- cold: folds the lists into partial copies, and the partial copies of main MERGE_ROWS at a time ----------
 extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_COLD(Params p) {
-    const int* control = (const int*)p.a[5];
+    const unsigned* __restrict__ planin = (const unsigned*)p.a[5];
+    const long long per = (long long)(unsigned long long)p.a[6];
     const int G1 = (int)(unsigned long long)p.a[7];
     const int NB = (int)(unsigned long long)p.a[8];
     const unsigned CAP = (unsigned)(unsigned long long)p.a[9];
     const unsigned* __restrict__ counts = (const unsigned*)p.a[10];
     const mjt_pair* __restrict__ lists = (const mjt_pair*)p.a[11];
+    const TX* __restrict__ pmain = (const TX*)p.a[12];
     TX* __restrict__ pcold = (TX*)p.a[13];
+    const int* __restrict__ hotof = (const int*)p.a[14];
     const mjt_pair* __restrict__ ovf = (const mjt_pair*)p.a[15];
-    __shared__ TX win[WBINS];
-    __shared__ unsigned prefix[512];                         // running totals of the list lengths (G1 <= 512)
+    const unsigned* __restrict__ novf = (const unsigned*)p.a[16];
+    // the private copy of a list item, or the rows of a merge item on their way to being combined
+    constexpr size_t WIN_BYTES = sizeof(TW) * WBINS > sizeof(TA) * NTHREADS * 4 ? sizeof(TW) * WBINS : sizeof(TA) * NTHREADS * 4;
+    __shared__ __attribute__((aligned(16))) unsigned char win_bytes[WIN_BYTES];
+    TW* win = (TW*)win_bytes;
     __shared__ mjt_plan plan;
-    __shared__ unsigned wsum[16];
-    const int hot = control[0];
-    mjt_make_plan(plan, (const unsigned*)control + 64, G1, NB, hot, wsum);
-    if (blockIdx.x >= plan.first[NB]) return;
-    int bucket = 0;
-    {
-        int lo = 0, hi = NB - 1;                              // first bucket whose running total exceeds blockIdx.x
-        while (lo < hi) {
-            const int mid = (lo + hi) >> 1;
-            if (plan.first[mid + 1] > blockIdx.x) hi = mid; else lo = mid + 1;
-        }
-        bucket = lo;
+    __shared__ unsigned length[512];                          // lengths of the lists of an item (G1 <= 512)
+    __shared__ int rows[MERGE_ROWS];
+    __shared__ unsigned long long wsum[16];
+    __shared__ unsigned any_ovf, nmatch;
+    for (int t = threadIdx.x; t < NBMAX; t += NTHREADS) {
+        plan.nsplit[t] = planin[t];
+        plan.nmerge[t] = planin[NBMAX + t];
     }
-    const int split = (int)(blockIdx.x - plan.first[bucket]);
-    const int SPLIT = (int)plan.nsplit[bucket];
+    for (int t = threadIdx.x; t <= NBMAX; t += NTHREADS) {
+        plan.first[t] = planin[2 * NBMAX + t];
+        plan.pfirst[t] = planin[3 * NBMAX + 1 + t];
+    }
+    if (threadIdx.x == 0) any_ovf = planin[4 * NBMAX + 2];
+    __syncthreads();
     const TX ident = mjt_ident();
-    for (int t = threadIdx.x; t < WBINS; t += NTHREADS) win[t] = ident;
-    const int nsrc = (G1 - split + SPLIT - 1) / SPLIT;       // lists this workgroup folds
-    for (int t = threadIdx.x; t < nsrc; t += NTHREADS) prefix[t] = counts[(size_t)(split + t * SPLIT) * NB + bucket];
-    __syncthreads();
-    mjt_block_scan(prefix, nsrc, wsum);
-    const unsigned total = nsrc ? prefix[nsrc - 1] : 0;
-    for (unsigned q0 = threadIdx.x; q0 < total; q0 += NTHREADS * 4) {
-        mjt_pair e[4];
-        bool live[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) {                        // four independent reads in flight per lane
-            const unsigned q = q0 + u * NTHREADS;
-            live[u] = q < total;
-            int lo = 0, hi = nsrc - 1;                       // first list whose running total exceeds q
-            while (lo < hi) {
-                const int mid = (lo + hi) >> 1;
-                if (prefix[mid] > q) hi = mid; else lo = mid + 1;
+    for (unsigned item = blockIdx.x; item < plan.first[NBMAX]; item += gridDim.x) {
+        int bucket;
+        {
+            int lo = 0, hi = NBMAX - 1;                       // the last bucket whose first item is <= item: it has items,
+            while (lo < hi) {                                 // buckets without share `first` with their successor
+                const int mid = (lo + hi + 1) >> 1;
+                if (plan.first[mid] <= item) lo = mid; else hi = mid - 1;
             }
-            const unsigned within = q - (lo ? prefix[lo - 1] : 0);
-            if (live[u]) e[u] = lists[((size_t)(split + lo * SPLIT) * NB + bucket) * CAP + within];
+            bucket = lo;
         }
+        const int within = (int)(item - plan.first[bucket]);
+        const int SPLIT = (int)plan.nsplit[bucket];
+        if (within >= SPLIT) {
+            // merge item: segment sgm of the partial copies of main workgroups number g*MERGE_ROWS ... of this bucket
+            const int g = (within - SPLIT) / MSEG, sgm = (within - SPLIT) - g * MSEG;
+            const unsigned match = (int)threadIdx.x < G1 && hotof[threadIdx.x] == bucket ? 1u : 0u;
+            const unsigned incl = (unsigned)mjt_block_scan_value(match, wsum);
+            if (match && (int)(incl - 1) / MERGE_ROWS == g) rows[(incl - 1) % MERGE_ROWS] = threadIdx.x;
+            if (threadIdx.x == NTHREADS - 1) nmatch = incl;
+            __syncthreads();
+            const int nrows = (int)nmatch - g * MERGE_ROWS < MERGE_ROWS ? (int)nmatch - g * MERGE_ROWS : MERGE_ROWS;
+            // MBINS / 4 threads across, the rows dealt to the groups of MBINS / 4 threads; combined through LDS
+            constexpr int ACROSS = MBINS / 4, GROUPS = NTHREADS / ACROSS;
+            const int col = threadIdx.x % ACROSS, grp = threadIdx.x / ACROSS;
+            const int t = sgm * MBINS + col * 4;
+            TA acc[4] = {(TA)ident, (TA)ident, (TA)ident, (TA)ident};
+            // all rows of the thread in flight at once
+            constexpr int RPT = (MERGE_ROWS + GROUPS - 1) / GROUPS;
+            mjt_pack<TX, 4> v[RPT];
 #pragma unroll
-        for (int u = 0; u < 4; u++)
-            if (live[u]) { LDS_UPDATE(&win[e[u].bin], e[u].val); }
-    }
-    // entries that did not fit a list: the first workgroup of the bucket scans the overflow list
-    if (split == 0) {
-        const unsigned novf = ((const unsigned*)control)[1];
-        for (unsigned q = threadIdx.x; q < novf; q += NTHREADS) {
-            const mjt_pair e = ovf[q];
-            if ((e.bin >> LOGW) == bucket) { LDS_UPDATE(&win[e.bin & (WBINS - 1)], e.val); }
+            for (int j = 0; j < RPT; j++) {
+                const int r = grp + j * GROUPS;
+                mjt_load(v[j], pmain + (size_t)rows[r < nrows ? r : 0] * WBINS + t);
+            }
+#pragma unroll
+            for (int j = 0; j < RPT; j++)
+                if (grp + j * GROUPS < nrows) {
+#pragma unroll
+                    for (int k = 0; k < 4; k++) acc[k] = MERGE2(acc[k], (TA)v[j].v[k]);
+                }
+            TA* comb = (TA*)win_bytes;                        // GROUPS x MBINS = NTHREADS * 4 values
+#pragma unroll
+            for (int k = 0; k < 4; k++) comb[grp * MBINS + col * 4 + k] = acc[k];
+            __syncthreads();
+            if (grp == 0) {
+                mjt_pack<TX, 4> o;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    TA r = comb[col * 4 + k];
+                    for (int q = 1; q < GROUPS; q++) r = MERGE2(r, comb[q * MBINS + col * 4 + k]);
+                    o.v[k] = (TX)r;
+                }
+                mjt_store(pcold + (size_t)(plan.pfirst[bucket] + SPLIT + g) * WBINS + t, o);
+            }
+            __syncthreads();
+            continue;
         }
-    }
-    __syncthreads();
-    TX* __restrict__ out = pcold + (size_t)blockIdx.x * WBINS;
-    for (int t = threadIdx.x * 4; t < WBINS; t += NTHREADS * 4) {
-        mjt_pack<TX, 4> o;
+        const int split = within;
+        TX* __restrict__ out = pcold + (size_t)(plan.pfirst[bucket] + split) * WBINS;
+        for (int t = threadIdx.x; t < WBINS; t += NTHREADS) win[t] = mjt_win_from(ident);
+        const int nsrc = (G1 - split + SPLIT - 1) / SPLIT;       // lists this item folds
+        for (int t = threadIdx.x; t < nsrc; t += NTHREADS) length[t] = counts[(size_t)(split + t * SPLIT) * NB + bucket];
+        __syncthreads();
+        // Each wave walks whole lists (no search for the list an entry belongs to), 64 consecutive entries per
+        // load and DEPTH loads in flight; when the item has fewer lists than waves, several waves share a list.
+        {
+            constexpr int WAVES = NTHREADS / 64, DEPTH = 8;
+            const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+            int wpl = 1;                                          // waves per list
+            while (wpl * 2 * nsrc <= WAVES) wpl *= 2;
+            const unsigned first_off = (unsigned)(wave % wpl) * 64u, off_step = (unsigned)wpl * 64u;
+            const int list_step = WAVES / wpl;
+            int li = wave / wpl;
+            unsigned off = first_off;
+            while (li < nsrc) {
+                mjt_pair e[DEPTH];
 #pragma unroll
-        for (int k = 0; k < 4; k++) o.v[k] = win[t + k];
-        mjt_store(out + t, o);
+                for (int d = 0; d < DEPTH; d++) {
+                    e[d].bin = -1;
+                    if (li < nsrc) {
+                        const unsigned c = length[li];
+                        const unsigned q = off + lane;
+                        if (q < c) e[d] = lists[((size_t)bucket * G1 + (split + li * SPLIT)) * CAP + q];
+                        off += off_step;
+                        if (off >= c) { li += list_step; off = first_off; }
+                    }
+                }
+#pragma unroll
+                for (int d = 0; d < DEPTH; d++)
+                    if (e[d].bin >= 0) mjt_win_update(&win[e[d].bin & (WBINS - 1)], e[d].val);
+            }
+        }
+        // entries that did not fit a list: the first item of the bucket scans the overflow lists
+        if (split == 0 && any_ovf) {
+            for (int w = 0; w < G1; w++) {
+                const unsigned c = novf[w];
+                const mjt_pair* __restrict__ l = ovf + (size_t)w * per;
+                for (unsigned q = threadIdx.x; q < c; q += NTHREADS) {
+                    const mjt_pair e = l[q];
+                    if ((e.bin >> LOGW) == bucket) mjt_win_update(&win[e.bin & (WBINS - 1)], e.val);
+                }
+            }
+        }
+        __syncthreads();
+        for (int t = threadIdx.x * 4; t < WBINS; t += NTHREADS * 4) {
+            mjt_pack<TX, 4> o;
+#pragma unroll
+            for (int k = 0; k < 4; k++) o.v[k] = mjt_win_read(win[t + k]);
+            mjt_store(out + t, o);
+        }
+        __syncthreads();
     }
 }
 
 // ---- final: x[bin] = merge of the partial copies of its bucket --------------------------------
-// workgroup = (bucket, segment of 256 bins); 64 lanes x 4 bins across, 4 groups of partials down
+// workgroup = (bucket, segment of 256 bins); 64 lanes x 4 bins across, 4 groups of partial copies down
 extern "C" __global__ __launch_bounds__(256) void ENTRY_FINAL(Params p) {
     TX* __restrict__ xp = (TX*)p.a[0];
     const long long bins = (long long)(unsigned long long)p.a[4];
-    const int* control = (const int*)p.a[5];
-    const int G1 = (int)(unsigned long long)p.a[7];
-    const TX* __restrict__ pmain = (const TX*)p.a[12];
+    const unsigned* __restrict__ planin = (const unsigned*)p.a[5];
     const TX* __restrict__ pcold = (const TX*)p.a[13];
-    const int NB = (int)(unsigned long long)p.a[8];
     constexpr int SEGS = WBINS / 256;
     const int bucket = blockIdx.x / SEGS, seg = blockIdx.x - bucket * SEGS;
-    const bool hot = bucket == control[0];
-    __shared__ mjt_plan plan;
-    __shared__ unsigned wsum[16];
-    if (NB > 1) mjt_make_plan(plan, (const unsigned*)control + 64, G1, NB, control[0], wsum);
-    const TX* __restrict__ src = hot ? pmain : pcold + (size_t)plan.first[bucket] * WBINS;
-    const int P = hot ? G1 : (int)plan.nsplit[bucket];
     const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int t = seg * 256 + lane * 4;
-    const TX ident = mjt_ident();
-    TX acc[4] = {ident, ident, ident, ident};
+    const int P = (int)(planin[bucket] + planin[NBMAX + bucket]);
+    const size_t first = planin[3 * NBMAX + 1 + bucket];
+    const TA ident = (TA)mjt_ident();
+    TA acc[4] = {ident, ident, ident, ident};
 #pragma unroll 8
     for (int j = grp; j < P; j += 4) {
         mjt_pack<TX, 4> v;
-        mjt_load(v, src + (size_t)j * WBINS + t);
+        mjt_load(v, pcold + (first + j) * WBINS + t);
 #pragma unroll
-        for (int k = 0; k < 4; k++) acc[k] = MERGE2(acc[k], v.v[k]);
+        for (int k = 0; k < 4; k++) acc[k] = MERGE2(acc[k], (TA)v.v[k]);
     }
-    __shared__ TX comb[4][256];
+    __shared__ TA comb[4][256];
 #pragma unroll
     for (int k = 0; k < 4; k++) comb[grp][lane * 4 + k] = acc[k];
     __syncthreads();
@@ -416,12 +572,11 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY_FINAL(Params p) {
         const long long b0 = (long long)bucket * WBINS + t;
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            TX r = comb[0][lane * 4 + k];
+            TA r = comb[0][lane * 4 + k];
             r = MERGE2(r, comb[1][lane * 4 + k]);
             r = MERGE2(r, comb[2][lane * 4 + k]);
             r = MERGE2(r, comb[3][lane * 4 + k]);
-            if (b0 + k < bins) xp[b0 + k] = r;
+            if (b0 + k < bins) xp[b0 + k] = (TX)r;
         }
     }
 }
-

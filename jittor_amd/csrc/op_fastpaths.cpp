@@ -135,17 +135,27 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     if (bins >= (int64_t(1) << 31) || n >= (int64_t(1) << 40)) return false;
     if ((uintptr_t)y->ptr % 16 || (uintptr_t)index->ptr % 32 || (uintptr_t)x->ptr % 4) return false;
     Context& c = ctx();
-    int logw = env_int("MJT_SCATTER_LOGW", 14);              // 16384 bins = 64 KB of LDS per private copy
+    int logw = env_int("MJT_SCATTER_LOGW", 14);              // 16384 bins: 64 KB (128 KB for float sums) of LDS per private copy
     while (logw > 8 && (int64_t(1) << (logw - 1)) >= bins) logw--;
     const int64_t W = int64_t(1) << logw;
     const int64_t NB = (bins + W - 1) / W;
-    if (NB > 4096) return false;                              // list cursors live in LDS
+    const int nthreads = 1024;
+    if (NB > 512) return false;                               // per-bucket tables live in LDS, one loading thread per bucket
     int64_t nbmax = 1;
     while (nbmax < NB) nbmax *= 2;
-    const int nthreads = env_int("MJT_SCATTER_THREADS", 1024);
     const int per_cu = env_int("MJT_SCATTER_WG_PER_CU", 1);
-    const int64_t cold_target = env_int("MJT_SCATTER_COLD_TARGET", 8192);   // list entries per cold workgroup
-    const int nhot = env_int("MJT_SCATTER_NHOT", mode == 0 ? 8 : 4);
+    const int64_t cold_target = env_int("MJT_SCATTER_COLD_TARGET", 16384);   // list entries per cold item
+    const int acc64 = mode == 0 && x->dtype == MJT_FLOAT32 && env_int("MJT_SCATTER_ACC64", 1);
+    const int ept = env_int("MJT_SCATTER_EPT", 8);           // elements per thread and round
+    if (ept < 4 || ept % 4 || ept > 32) return false;
+    const int nflush = env_int("MJT_SCATTER_NFLUSH", 256);    // threads of a main workgroup that only append to the lists
+    if (nflush < 64 || nflush % 64 || nflush > 512) return false;
+    // staging entries: what the private copy and the per-bucket table leave of the 160 KB of LDS, in two areas
+    const int64_t lds_left = 160 * 1024 - 1024 - W * (acc64 ? 8 : 4) - nbmax * 4;
+    int64_t scap = lds_left / 16 / 64 * 64;
+    if (scap > 4096) scap = 4096;
+    scap = env_int("MJT_SCATTER_SCAP", (int)scap);
+    if (scap < 64 || scap * 16 > lds_left) return false;
     // identity
     uint32_t ident = 0;
     if (mode) {
@@ -159,31 +169,35 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     const int64_t chunk = (int64_t)nthreads * 4;
     const int64_t per = ((n + G1 - 1) / G1 + chunk - 1) / chunk * chunk;
     G1 = n ? (n + per - 1) / per : 1;
-    // cold workgroups: one per bucket plus population / cold_target (see mjt_make_plan)
-    const int64_t cold_wgs = NB > 1 ? NB + n / cold_target + 1 : 0;
+    // cold items: at most one per bucket plus population / cold_target (see mjt_make_plan)
+    // plus the merge items: one per 16 main workgroups of a bucket
+    const int64_t cold_items = NB + n / cold_target + 1 + G1 / 16 + (NB < G1 ? NB : G1) + 1;
+    int64_t cold_wgs = (int64_t)c.prop.multiProcessorCount * (acc64 ? 1 : 2);
+    if (cold_wgs > cold_items) cold_wgs = cold_items;
     int64_t CAP = NB > 1 ? (4 * per / NB + 63) / 64 * 64 : 64;
     if (CAP < 64) CAP = 64;
     if (CAP > per) CAP = (per + 63) / 64 * 64;
 
     std::ostringstream key;
-    key << "sc1|" << x->dtype << "|" << index->dtype << "|" << mode << "|" << logw << "|" << nbmax << "|" << nthreads << "|" << nhot << "|" << cold_target;
-    static const char* parts[] = {"sample", "main", "cold", "final"};
+    key << "sc1|" << x->dtype << "|" << index->dtype << "|" << mode << "|" << logw << "|" << nbmax << "|" << nthreads << "|" << nflush << "|" << ept
+        << "|" << scap << "|" << cold_target << "|" << acc64;
+    static const char* parts[] = {"main", "plan", "cold", "final"};
     JitKernel* ks[4];
     bool have = true;
     for (int i = 0; i < 4; i++) have = (ks[i] = cached(key.str() + "|" + parts[i])) != nullptr && have;
     if (!have) {
         std::ostringstream name;
         name << "mjt_scatter1d_" << mjt_op_name(op) << "_" << mjt_dtype_name(x->dtype) << "_" << mjt_dtype_name(index->dtype)
-             << "_w" << W << "_b" << nbmax << "_t" << nthreads;
+             << "_w" << W << "_b" << nbmax << "_e" << ept << "_s" << scap;
         std::ostringstream src;
-        src << "#define ENTRY_SAMPLE " << name.str() << "_sample\n#define ENTRY_MAIN " << name.str() << "_main\n#define ENTRY_COLD "
+        src << "#define ENTRY_MAIN " << name.str() << "_main\n#define ENTRY_PLAN " << name.str() << "_plan\n#define ENTRY_COLD "
             << name.str() << "_cold\n#define ENTRY_FINAL " << name.str() << "_final\n#define COLD_TARGET " << cold_target
             << "u\n#define TX " << dtype_cname(x->dtype) << "\n#define TE " << dtype_cname(index->dtype) << "\n#define WBINS "
             << W << "\n#define LOGW " << logw << "\n#define NBMAX " << nbmax << "\n#define NTHREADS " << nthreads
-            << "\n#define NHOT " << nhot << "\n#define MODE " << mode << "\n#define IDENT_BITS " << ident << "u\n";
-        src << embedded_source("prelude.h") << "\n" << embedded_source("atomics.h") << "\n" << embedded_source("scatter1d.h")
-            << "\n";
-        JitKernel* first = jit_get(src.str(), name.str() + "_sample");
+            << "\n#define NFLUSH " << nflush << "\n#define EPT " << ept << "\n#define SCAP " << scap << "\n#define ACC64 " << acc64
+            << "\n#define MODE " << mode << "\n#define IDENT_BITS " << ident << "u\n";
+        src << embedded_source("prelude.h") << "\n" << embedded_source("scatter1d.h") << "\n";
+        JitKernel* first = jit_get(src.str(), name.str() + "_main");
         for (int i = 0; i < 4; i++) {
             JitKernel* k = i == 0 ? first : new JitKernel();
             if (i) {
@@ -197,20 +211,23 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     }
     // scratch layout
     auto align = [](size_t v) { return (v + 255) / 256 * 256; };
-    const size_t off_counts = 32768;                          // control block: 64 words + one word per bucket
+    const size_t off_hotof = align((size_t)(4 * nbmax + 3) * 4);          // after the plan
+    const size_t off_novf = off_hotof + align((size_t)G1 * 4);
+    const size_t off_counts = off_novf + align((size_t)G1 * 4);
     const size_t off_pmain = off_counts + align((size_t)G1 * NB * 4);
     const size_t off_pcold = off_pmain + align((size_t)G1 * W * 4);
-    const size_t off_lists = off_pcold + align((size_t)cold_wgs * W * 4);
+    const size_t off_lists = off_pcold + align((size_t)cold_items * W * 4);
     const size_t off_ovf = off_lists + align(NB > 1 ? (size_t)G1 * NB * CAP * 8 : 0);
-    const size_t total = off_ovf + align(NB > 1 ? (size_t)n * 8 : 0);
+    const size_t total = off_ovf + align(NB > 1 ? (size_t)G1 * per * 8 : 0);
     char* base = (char*)scratch(total);
     std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), bits_of_ptr(index->ptr), (uint64_t)n, (uint64_t)bins,
                             bits_of_ptr(base), (uint64_t)per, (uint64_t)G1, (uint64_t)NB, (uint64_t)CAP,
                             bits_of_ptr(base + off_counts), bits_of_ptr(base + off_lists), bits_of_ptr(base + off_pmain),
-                            bits_of_ptr(base + off_pcold), 0, bits_of_ptr(base + off_ovf)};
-    jit_launch(ks[0], 1, 1, 1024, 0, a);
-    jit_launch(ks[1], (unsigned)G1, 1, (unsigned)nthreads, 0, a);
-    if (NB > 1) jit_launch(ks[2], (unsigned)cold_wgs, 1, (unsigned)nthreads, 0, a);
+                            bits_of_ptr(base + off_pcold), bits_of_ptr(base + off_hotof), bits_of_ptr(base + off_ovf),
+                            bits_of_ptr(base + off_novf), 0, 0, 0};
+    jit_launch(ks[0], (unsigned)G1, 1, (unsigned)nthreads, 0, a);
+    jit_launch(ks[1], 1, 1, (unsigned)nthreads, 0, a);
+    jit_launch(ks[2], (unsigned)cold_wgs, 1, (unsigned)nthreads, 0, a);
     jit_launch(ks[3], (unsigned)(NB * (W / 256)), 1, 256, 0, a);
     return true;
 }

@@ -242,6 +242,43 @@ def test_scatter_1d_fast_path(gpu, n, bins):
     assert np.array_equal(got, np.bincount(idx[ok], minlength=bins).astype(np.int32))
 
 
+def _scatter_check(v, idx, bins, ops=("add", "maximum", "minimum")):
+    ok = (idx >= 0) & (idx < bins)
+    jv, ji = jt.array(v), jt.array(idx, "int64" if idx.dtype == np.int64 else "int32")
+    for op in ops:
+        got = jv.reindex_reduce(op, [bins], ["@e0(i0)"], extras=[ji]).data
+        assert L.last_kernel().startswith("mjt_scatter1d_" + op), L.last_kernel()
+        if op == "add":
+            ref = np.bincount(idx[ok], weights=v[ok].astype(np.float64), minlength=bins)
+            assert np.allclose(got, ref, rtol=1e-4, atol=1e-6), op
+        else:
+            ref = np.full(bins, np.finfo(np.float32).min if op == "maximum" else np.finfo(np.float32).max, np.float32)
+            (np.maximum if op == "maximum" else np.minimum).at(ref, idx[ok], v[ok])
+            assert np.array_equal(got, ref), op
+
+
+def test_scatter_1d_index_distributions(gpu):
+    """The routes of the 1-d scatter besides the Zipf head: no hot bucket at all (every update is listed, the
+    staging areas overflow), two hot regions (lists overflow into the overflow lists), sorted indices (every
+    workgroup has its own hot bucket), a single value, a ragged tail, indices far outside the bins."""
+    rng = np.random.default_rng(17)
+    n, bins = 1 << 21, 1 << 20
+    v = (rng.random(n, dtype=np.float32) - 0.25).astype(np.float32)            # both signs
+    _scatter_check(v, rng.integers(0, bins, n).astype(np.int32), bins)                       # uniform over 64 buckets
+    two = np.where(rng.random(n) < 0.5, rng.integers(0, 9000, n), rng.integers(500000, 509000, n)).astype(np.int32)
+    _scatter_check(v, two, bins)                                                             # two hot regions
+    _scatter_check(v, np.sort(rng.integers(0, bins, n)).astype(np.int32), bins)              # sorted
+    _scatter_check(v, np.full(n, 777777, np.int32), bins, ops=("add", "maximum"))            # one bin takes everything
+    far = rng.integers(-(1 << 40), 1 << 40, 100003).astype(np.int64)                         # mostly out of range
+    far[::3] = rng.integers(0, bins, far[::3].size)
+    _scatter_check(v[:100003], far, bins)
+    for m in (1, 2, 3, 6, 4097):                                                             # tails and tiny inputs
+        _scatter_check(v[:m], rng.integers(0, 50, m).astype(np.int32), 50)
+    big = 9_000_000                                                                          # more than 512 buckets: generic kernel
+    got = jt.array(v[:4096]).reindex_reduce("add", [big], ["@e0(i0)"], extras=[jt.array(rng.integers(0, big, 4096).astype(np.int32))]).data
+    assert not L.last_kernel().startswith("mjt_scatter1d_") and abs(got.sum() - v[:4096].astype(np.float64).sum()) < 1e-2
+
+
 def _zipf_indices(n, bins):
     w = np.arange(1, bins + 1, dtype=np.float64) ** -1.1
     cdf = np.cumsum(w) / w.sum()
