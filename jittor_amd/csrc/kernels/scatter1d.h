@@ -136,7 +136,7 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
     unsigned* __restrict__ novf = (unsigned*)p.a[16];
     __shared__ TW win[WBINS];
     __shared__ mjt_pair staging[2][SCAP];  // updates of a round on their way to the lists, by round parity
-    __shared__ unsigned cursor[NBMAX];     // list lengths (votes during the sample)
+    __shared__ unsigned cursor[NBMAX + 1]; // list lengths (votes during the sample); the last one is a dummy
     __shared__ unsigned best, staged[3], ovf_len;        // staged: entries of a round, by round number mod 3
     const TX ident = mjt_ident();
     const long long begin = (long long)blockIdx.x * per;
@@ -186,7 +186,29 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
             if (r > 0) {                                      // drain what round r-1 staged
                 const unsigned total = staged[prev3];
                 const unsigned m = total < SCAP ? total : SCAP;
-                for (unsigned t = threadIdx.x - NP; t < m; t += NFLUSH) append(staging[(r - 1) & 1][t]);
+                // FDEPTH entries per thread at a time: their LDS reads, their list cursors and their stores each
+                // go out back to back (one entry at a time would cost two LDS round trips per entry in a row)
+                constexpr int FDEPTH = 4;
+                for (unsigned t0 = threadIdx.x - NP; t0 < m; t0 += NFLUSH * FDEPTH) {
+                    mjt_pair e[FDEPTH];
+                    unsigned pos[FDEPTH];
+#pragma unroll
+                    for (int u = 0; u < FDEPTH; u++) {
+                        const unsigned t = t0 + u * NFLUSH;
+                        e[u] = staging[(r - 1) & 1][t < m ? t : 0];
+                        if (t >= m) e[u].bin = NBMAX << LOGW;    // a cursor of its own that nobody reads
+                    }
+#pragma unroll
+                    for (int u = 0; u < FDEPTH; u++) pos[u] = atomicAdd(&cursor[e[u].bin >> LOGW], 1u);
+#pragma unroll
+                    for (int u = 0; u < FDEPTH; u++) {
+                        const int b = e[u].bin >> LOGW;
+                        if (b < NBMAX) {
+                            if (pos[u] < CAP) mylists[(size_t)b * bucket_stride + pos[u]] = e[u];
+                            else ovf[atomicAdd(&ovf_len, 1u)] = e[u];
+                        }
+                    }
+                }
             }
             if (threadIdx.x == NP) staged[next3] = 0;         // drained one round ago, used from the next round on
             prev3 = prev3 == 2 ? 0 : prev3 + 1;

@@ -151,7 +151,7 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     const int nflush = env_int("MJT_SCATTER_NFLUSH", 256);    // threads of a main workgroup that only append to the lists
     if (nflush < 64 || nflush % 64 || nflush > 512) return false;
     // staging entries: what the private copy and the per-bucket table leave of the 160 KB of LDS, in two areas
-    const int64_t lds_left = 160 * 1024 - 1024 - W * (acc64 ? 8 : 4) - nbmax * 4;
+    const int64_t lds_left = 160 * 1024 - 1024 - W * (acc64 ? 8 : 4) - (nbmax + 1) * 4;
     int64_t scap = lds_left / 16 / 64 * 64;
     if (scap > 4096) scap = 4096;
     scap = env_int("MJT_SCATTER_SCAP", (int)scap);
