@@ -174,7 +174,7 @@ def wl_c3(L, lib, steps, warmup, with_cpu, op):
     out = {"workload": "C3 ReindexReduceOp scatter-%s, 2^24 fp32 values into 2^20 bins, int32 Zipf(1.1) indices" % op,
            "kernel": L.last_kernel(), "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
            "roofline": roofline("hbm", work, ms),
-           "note": "a step = identity fill of the bins + window sampling pass + scatter kernel"}
+           "note": "a step = the four launches of the 1-d scatter (main, plan, cold, final); the bins need no prior fill"}
     dev.release()
     if with_cpu:
         t1 = cpu_time(lambda: K.scatter_1d(v, idx, bins, op))
