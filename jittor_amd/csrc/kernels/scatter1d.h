@@ -34,6 +34,7 @@
 // (power of two), LOGW, NBMAX (power of two >= bucket count, <= NTHREADS),
 // NTHREADS, NFLUSH (threads that only store), EPT (elements per thread and
 // round, multiple of 4), SCAP (entries of each of the two staging areas), MODE (0 add, 1 maximum, 2 minimum), ACC64, COLD_TARGET,
+// EXACT_BINS (the bin count is a multiple of WBINS),
 // IDENT_BITS (bit pattern of the identity).
 
 struct Params { void* a[20]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
@@ -118,6 +119,7 @@ __device__ __forceinline__ unsigned long long mjt_block_scan_value(unsigned long
 }
 
 // ---- main ---------------------------------------------------------------------------
+template <bool V> struct mjt_flag { static constexpr bool value = V; };
 constexpr int NP = NTHREADS - NFLUSH;                        // threads that load input; the others append to the lists
 
 extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
@@ -147,20 +149,7 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
     for (int t = threadIdx.x; t < WBINS; t += NTHREADS) win[t] = mjt_win_from(ident);
     if (threadIdx.x == 0) { best = 0; staged[0] = 0; staged[1] = 0; staged[2] = 0; ovf_len = 0; }
     __syncthreads();
-    // the hot bucket: vote of 8 runs of 64 consecutive indices spread over this workgroup's share
-    if (threadIdx.x < 512) {
-        const long long run = threadIdx.x >> 6;
-        const long long pos = begin + run * ((end - begin) >> 3) + (threadIdx.x & 63);
-        const long long b = pos < end ? (long long)ip[pos] : -1;
-        if ((unsigned long long)b < (unsigned long long)bins) atomicAdd(&cursor[(int)(b >> LOGW)], 1u);
-    }
-    __syncthreads();
-    for (int t = threadIdx.x; t < NB; t += NTHREADS)
-        if (cursor[t]) atomicMax(&best, (cursor[t] << 12) | (unsigned)(4095 - t));   // ties: the lowest bucket
-    __syncthreads();
-    const unsigned hot = best ? 4095u - (best & 4095u) : 0u;
-    for (int t = threadIdx.x; t < NBMAX; t += NTHREADS) cursor[t] = 0;
-    __syncthreads();
+    unsigned hot = 0;                                         // the hot bucket, voted below (used by the producers only)
 
     // lists of one bucket are neighbours in memory: the cold item that folds them then touches few pages
     mjt_pair* __restrict__ mylists = lists + (size_t)blockIdx.x * CAP;
@@ -181,6 +170,9 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
     constexpr long long STEP = (long long)NP * EPT;
     const int rounds = 2 * (int)((end4 - begin + 2 * STEP - 1) / (2 * STEP)) + (end4 < end ? 1 : 0);
     if (threadIdx.x >= NP) {
+        __syncthreads();                                      // the three barriers of the producers' vote
+        __syncthreads();
+        __syncthreads();
         int prev3 = 2, next3 = 1;                             // (r - 1) mod 3, (r + 1) mod 3
         for (int r = 0; r <= rounds; r++) {
             if (r > 0) {                                      // drain what round r-1 staged
@@ -266,18 +258,23 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
                 mjt_load_nt(id[v], ip + ic);
             }
         };
-        auto step = [&](int r, unsigned* cnt, long long r0, mjt_pack<TX, 4> (&vv)[EPT / 4], mjt_pack<TE, 4> (&id)[EPT / 4]) {
+        // FULL: every vector of the round lies inside the share (no per-vector test)
+        auto step = [&](auto full, int r, unsigned* cnt, long long r0, mjt_pack<TX, 4> (&vv)[EPT / 4], mjt_pack<TE, 4> (&id)[EPT / 4]) {
+            constexpr bool FULL = decltype(full)::value;
             unsigned idx[EPT];
             TX val[EPT];
 #pragma unroll
             for (int v = 0; v < EPT / 4; v++) {
                 const long long i = r0 + ((long long)v * NP + threadIdx.x) * 4;
-                const bool present = i < end4;
+                const bool present = FULL || i < end4;
 #pragma unroll
                 for (int k = 0; k < 4; k++) {
-                    bool inside;                              // overflow (index outside [0, bins)): skipped
-                    if constexpr (sizeof(TE) == 4) inside = (unsigned)id[v].v[k] < (unsigned)bins;   // bins < 2^31
-                    else inside = (unsigned long long)id[v].v[k] < (unsigned long long)bins;
+                    // overflow (index outside [0, bins)): skipped.  When the bins fill their buckets exactly and the
+                    // index has 32 bits, an index outside the bins is an index outside the buckets: the test
+                    // against the bucket count in `round` covers it.
+                    bool inside = true;
+                    if constexpr (sizeof(TE) != 4) inside = (unsigned long long)id[v].v[k] < (unsigned long long)bins;
+                    else if constexpr (!EXACT_BINS) inside = (unsigned)id[v].v[k] < (unsigned)bins;   // bins < 2^31
                     idx[v * 4 + k] = (present && inside) ? (unsigned)id[v].v[k] : SKIP;
                     val[v * 4 + k] = vv[v].v[k];
                 }
@@ -287,11 +284,33 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
         };
         fetch(begin, vva, ida);
         fetch(begin + STEP, vvb, idb);
+        // The hot bucket: a vote among 256 indices of the first round (already on their way: no extra memory
+        // round trip before the stream starts).
+        if (threadIdx.x < 256 && begin + (long long)threadIdx.x * 4 < end4) {
+            bool inside;
+            if constexpr (sizeof(TE) == 4) inside = (unsigned)ida[0].v[0] < (unsigned)bins;
+            else inside = (unsigned long long)ida[0].v[0] < (unsigned long long)bins;
+            if (inside) atomicAdd(&cursor[(unsigned)ida[0].v[0] >> LOGW], 1u);
+        }
+        __syncthreads();
+        for (int t = threadIdx.x; t < NB; t += NP)
+            if (cursor[t]) atomicMax(&best, (cursor[t] << 12) | (unsigned)(4095 - t));   // ties: the lowest bucket
+        __syncthreads();
+        hot = best ? 4095u - (best & 4095u) : 0u;
+        for (int t = threadIdx.x; t < NBMAX; t += NP) cursor[t] = 0;
+        __syncthreads();
         int r = 0, r3 = 0;                                    // r3 = r mod 3
-        for (long long r0 = begin; r0 < end4; r0 += 2 * STEP) {
-            step(r++, &staged[r3], r0, vva, ida);
+        long long r0 = begin;
+        for (; r0 + 2 * STEP <= end4; r0 += 2 * STEP) {       // pairs of whole rounds
+            step(mjt_flag<true>(), r++, &staged[r3], r0, vva, ida);
             r3 = r3 == 2 ? 0 : r3 + 1;
-            step(r++, &staged[r3], r0 + STEP, vvb, idb);      // possibly past the end: a round of skipped elements
+            step(mjt_flag<true>(), r++, &staged[r3], r0 + STEP, vvb, idb);
+            r3 = r3 == 2 ? 0 : r3 + 1;
+        }
+        for (; r0 < end4; r0 += 2 * STEP) {                   // the ragged end
+            step(mjt_flag<false>(), r++, &staged[r3], r0, vva, ida);
+            r3 = r3 == 2 ? 0 : r3 + 1;
+            step(mjt_flag<false>(), r++, &staged[r3], r0 + STEP, vvb, idb);   // possibly past the end: a round of skipped elements
             r3 = r3 == 2 ? 0 : r3 + 1;
         }
         if (end4 < end) {                                     // the last 1..3 elements of the input

@@ -180,7 +180,7 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
 
     std::ostringstream key;
     key << "sc1|" << x->dtype << "|" << index->dtype << "|" << mode << "|" << logw << "|" << nbmax << "|" << nthreads << "|" << nflush << "|" << ept
-        << "|" << scap << "|" << cold_target << "|" << acc64;
+        << "|" << scap << "|" << cold_target << "|" << acc64 << "|" << (bins % W == 0);
     static const char* parts[] = {"main", "plan", "cold", "final"};
     JitKernel* ks[4];
     bool have = true;
@@ -194,7 +194,7 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
             << name.str() << "_cold\n#define ENTRY_FINAL " << name.str() << "_final\n#define COLD_TARGET " << cold_target
             << "u\n#define TX " << dtype_cname(x->dtype) << "\n#define TE " << dtype_cname(index->dtype) << "\n#define WBINS "
             << W << "\n#define LOGW " << logw << "\n#define NBMAX " << nbmax << "\n#define NTHREADS " << nthreads
-            << "\n#define NFLUSH " << nflush << "\n#define EPT " << ept << "\n#define SCAP " << scap << "\n#define ACC64 " << acc64
+            << "\n#define EXACT_BINS " << (bins % W == 0 ? 1 : 0) << "\n#define NFLUSH " << nflush << "\n#define EPT " << ept << "\n#define SCAP " << scap << "\n#define ACC64 " << acc64
             << "\n#define MODE " << mode << "\n#define IDENT_BITS " << ident << "u\n";
         src << embedded_source("prelude.h") << "\n" << embedded_source("scatter1d.h") << "\n";
         JitKernel* first = jit_get(src.str(), name.str() + "_main");
