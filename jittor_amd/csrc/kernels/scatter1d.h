@@ -372,12 +372,12 @@ __device__ __forceinline__ void mjt_make_plan(mjt_plan& plan, const unsigned* __
         unsigned sum = 0;
         if (b < NB) {                                         // independent loads, several in flight
             constexpr int RSTEP = NTHREADS / NBMAX;
-            for (int r0 = threadIdx.x / NBMAX; r0 < G1; r0 += 8 * RSTEP) {
-                unsigned c[8];
+            for (int r0 = threadIdx.x / NBMAX; r0 < G1; r0 += 16 * RSTEP) {
+                unsigned c[16];
 #pragma unroll
-                for (int u = 0; u < 8; u++) c[u] = r0 + u * RSTEP < G1 ? counts[(size_t)(r0 + u * RSTEP) * NB + b] : 0u;
+                for (int u = 0; u < 16; u++) c[u] = r0 + u * RSTEP < G1 ? counts[(size_t)(r0 + u * RSTEP) * NB + b] : 0u;
 #pragma unroll
-                for (int u = 0; u < 8; u++) sum += c[u];
+                for (int u = 0; u < 16; u++) sum += c[u];
             }
         }
         if (sum) atomicAdd(&plan.nsplit[b], sum);
