@@ -17,8 +17,8 @@ from .core import (Var, Buffer, UnaryOp, BinaryOp, TernaryOp, BroadcastOp,
 from ._lib import MjtError
 from . import profiler as _profiler
 
-stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0}
-flags = {"enable_conv_match": True, "enable_reduce_fusion": True}
+stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0}
+flags = {"enable_conv_match": True, "enable_reduce_fusion": True, "enable_broadcast_sink": True}
 
 
 class ConvUnit:
@@ -278,6 +278,83 @@ def _execute(ops, target_ids):
         for u in node.inputs:
             consumers.setdefault(u.id, []).append(node)
 
+    # ---- element ops whose result is only ever broadcast move behind the broadcast ------------
+    # broadcast(f(a, b)) == f(broadcast(a), broadcast(b)): the small op then runs inside the kernel of the
+    # broadcast's consumers (recomputed per element) instead of as a launch of its own, as the reference's
+    # fuser does with cheap shared producers (executor.cc:466-474; test_new_fused_op.py:24-40: a
+    # normalisation is three kernels).  pre[b.id] = the ops to evaluate at b's output shape, in order;
+    # leaves[b.id] = the vars they read through b's broadcast mask.
+    pre, leaves = {}, {}
+    if flags["enable_broadcast_sink"]:
+        producer0 = {node.out.id: node for node in sched}
+        sinkable = {}
+        for node in reversed(sched):
+            users = consumers.get(node.out.id, ())
+            const = isinstance(node, BroadcastOp) and node.inputs[0]._op is None and node.inputs[0]._host is not None \
+                and node.inputs[0].num == 1                  # a number spread over a small shape stays a number
+            ok = (const or isinstance(node, (UnaryOp, BinaryOp, TernaryOp))) and node.out.id not in target_ids and users \
+                and node.out._buf is None and not getattr(node.out, "_stop_fuse", False)
+            if ok:
+                for c in users:
+                    if not (isinstance(c, BroadcastOp) or (sinkable.get(c.id) and c.out.shape == node.out.shape)):
+                        ok = False
+                        break
+            if ok:
+                for u in node.inputs:
+                    if not (u.shape == node.out.shape or (u._op is None and u._host is not None and u.num == 1)):
+                        ok = False
+                        break
+            sinkable[node.id] = bool(ok)
+        for node in sched:
+            if not isinstance(node, BroadcastOp):
+                continue
+            p = producer0.get(node.inputs[0].id)
+            if p is None or not sinkable.get(p.id):
+                continue
+            chain, seen, lv = [], set(), []
+
+            def visit(op):
+                if op.id in seen:
+                    return
+                seen.add(op.id)
+                for u in op.inputs:
+                    q = producer0.get(u.id)
+                    if q is not None and sinkable.get(q.id):
+                        visit(q)
+                    elif not any(u is w for w in lv):
+                        lv.append(u)
+                chain.append(op)
+
+            visit(p)
+            if len(chain) <= 32:
+                pre[node.id], leaves[node.id] = chain, lv
+        # a sunk op runs on its own only if some broadcast could not take its chain
+        taken = set()
+        for bid, chain in pre.items():
+            taken.update(op.id for op in chain)
+        left = {node.id for node in sched if isinstance(node, BroadcastOp) and node.id not in pre}
+        keep_ids = set()
+        stack = [producer0[node.inputs[0].id] for node in sched
+                 if node.id in left and node.inputs[0].id in producer0 and producer0[node.inputs[0].id].id in taken]
+        while stack:
+            op = stack.pop()
+            if op.id in keep_ids:
+                continue
+            keep_ids.add(op.id)
+            stack.extend(producer0[u.id] for u in op.inputs if u.id in producer0 and producer0[u.id].id in taken)
+        dropped = taken - keep_ids
+        if dropped:
+            stats["sunk_ops"] += len(dropped)
+            sched = [node for node in sched if node.id not in dropped]
+
+    def ins(op):
+        return leaves.get(op.id, op.inputs)
+
+    consumers = {}
+    for node in sched:
+        for u in ins(node):
+            consumers.setdefault(u.id, []).append(node)
+
     # ---- stages: an op can share a kernel with its producer only inside a stage ---------
     producer = {}
     for op in sched:
@@ -285,7 +362,7 @@ def _execute(ops, target_ids):
     stage = {}
     for op in sched:
         s = 0
-        for u in op.inputs:
+        for u in ins(op):
             p = producer.get(u.id)
             if p is None:
                 continue
@@ -298,6 +375,20 @@ def _execute(ops, target_ids):
                 step = 1
             s = max(s, stage[p.id] + step)
         stage[op.id] = s
+    # An element or broadcast op whose consumers all run in later stages waits for them: it then shares their
+    # kernel instead of writing its result to memory first (`(x - mean) / std`: the subtraction could run as
+    # soon as the mean is known, but belongs in the kernel of the division, which has to wait for std).
+    for op in reversed(sched):
+        if not op.fusable or op.out.id in target_ids or op.out._buf is not None:
+            continue
+        latest = None
+        for c in consumers.get(op.out.id, ()):
+            lim = stage[c.id]
+            if isinstance(c, BroadcastOp) or getattr(op.out, "_stop_fuse", False) or (c.fusable and c.out.shape != op.out.shape):
+                lim -= 1                                      # the consumer reads this result from memory
+            latest = lim if latest is None else min(latest, lim)
+        if latest is not None and latest > stage[op.id]:
+            stage[op.id] = latest
 
     # ---- union element ops into groups ---------------------------------------------
     parent = {}
@@ -353,14 +444,14 @@ def _execute(ops, target_ids):
     def group_io(members, extra_out=None):
         ids = {op.id for op in members}
         made = {op.out.id for op in members}
-        ins = {}
+        read = {}
         for op in members:
-            for u in op.inputs:
+            for u in ins(op):
                 if u.id not in made and not (u._op is None and u._host is not None and u.num == 1):
-                    ins[u.id] = u.nbytes
+                    read[u.id] = u.nbytes
         outs = sum(op.out.nbytes for op in members
                    if extra_out is None and (op.out.id in target_ids or any(c.id not in ids for c in consumers.get(op.out.id, ()))))
-        return sum(ins.values()), outs + (extra_out.nbytes if extra_out is not None else 0)
+        return sum(read.values()), outs + (extra_out.nbytes if extra_out is not None else 0)
 
     def timed(call, kind, io):
         rec = _profiler.active()
@@ -369,14 +460,14 @@ def _execute(ops, target_ids):
     for s in range(nstage):
         for members in by_stage_groups[s]:
             if id(members) not in absorbed_groups:
-                timed(lambda: _run_group(members, consumers, target_ids), "fused", lambda: group_io(members))
+                timed(lambda: _run_group(members, consumers, target_ids, pre=pre), "fused", lambda: group_io(members))
         for op in by_stage_other[s]:
             members = prologue_of.get(op.id)
             if members is not None:
-                if timed(lambda: _run_group(members, consumers, target_ids, reduce=op), "fused+reduce",
+                if timed(lambda: _run_group(members, consumers, target_ids, reduce=op, pre=pre), "fused+reduce",
                          lambda: group_io(members, op.out)):
                     continue
-                timed(lambda: _run_group(members, consumers, target_ids), "fused", lambda: group_io(members))
+                timed(lambda: _run_group(members, consumers, target_ids, pre=pre), "fused", lambda: group_io(members))
             timed(lambda: _run_single(op), op.kind, lambda: (sum(u.nbytes for u in op.inputs), op.out.nbytes))
     # materialised vars become leaves: the graph behind them can be dropped
     for op in sched:
@@ -461,7 +552,7 @@ def _run_single(op):
         raise MjtError(-2, "no kernel for op %r" % (op,))
 
 
-def _run_group(members, consumers, target_ids, reduce=None):
+def _run_group(members, consumers, target_ids, reduce=None, pre=None):
     """One launch for a group of element / broadcast ops.  With `reduce` (the ReduceOp that consumes the
     group's only result) the group runs as that reduce's prologue; returns False when the library does
     not take the group in that form (a tensor broadcast inside it), True otherwise."""
@@ -499,10 +590,36 @@ def _run_group(members, consumers, target_ids, reduce=None):
         index[key] = i
         return i
 
+    def add_op(op, ins, oi):
+        fo = _lib.FusedOp()
+        if isinstance(op, UnaryOp):
+            fo.kind, fo.op = _lib.FOP_UNARY, _lib.OP_CODE[op.op]
+        elif isinstance(op, BinaryOp):
+            fo.kind, fo.op = _lib.FOP_BINARY, _lib.OP_CODE[op.op]
+        elif isinstance(op, TernaryOp):
+            fo.kind, fo.op = _lib.FOP_TERNARY, 0
+        else:
+            fo.kind, fo.op = _lib.FOP_BROADCAST, 0
+        for j, v in enumerate(ins):
+            fo.inp[j] = v
+        fo.out = oi
+        fops.append(fo)
+        return oi
+
     outputs = []
     for op in members:
         ins = []
-        if isinstance(op, BroadcastOp):
+        if isinstance(op, BroadcastOp) and pre and op.id in pre:
+            # the element ops in front of this broadcast, evaluated per element of its output: what they read
+            # is loaded through the broadcast's mask
+            full = (1 << len(shape)) - 1
+            mask = op.bcast_mask & full
+            local = {}
+            for q in pre[op.id]:
+                qin = [local[u.id] if u.id in local else external(u, mask) for u in q.inputs]
+                local[q.out.id] = add_op(q, qin, add_var(_lib.VAR_INTERMEDIATE, q.out.dtype))
+            ins.append(local[op.inputs[0].id])
+        elif isinstance(op, BroadcastOp):
             u = op.inputs[0]
             full = (1 << len(shape)) - 1
             ins.append(external(u, op.bcast_mask & full))
@@ -521,19 +638,7 @@ def _run_group(members, consumers, target_ids, reduce=None):
         else:
             oi = add_var(_lib.VAR_INTERMEDIATE, out.dtype)
         index[(out.id, 0)] = oi
-        fo = _lib.FusedOp()
-        if isinstance(op, UnaryOp):
-            fo.kind, fo.op = _lib.FOP_UNARY, _lib.OP_CODE[op.op]
-        elif isinstance(op, BinaryOp):
-            fo.kind, fo.op = _lib.FOP_BINARY, _lib.OP_CODE[op.op]
-        elif isinstance(op, TernaryOp):
-            fo.kind, fo.op = _lib.FOP_TERNARY, 0
-        else:
-            fo.kind, fo.op = _lib.FOP_BROADCAST, 0
-        for j, v in enumerate(ins):
-            fo.inp[j] = v
-        fo.out = oi
-        fops.append(fo)
+        add_op(op, ins, oi)
     if not outputs:
         return True
     desc = _lib.FusedDesc()

@@ -676,6 +676,8 @@ def test_fused_reduce_with_per_output_inputs(gpu):
         y = (v - mean) / (var + 1e-5).sqrt()
         got = y.data
         assert jt.executor_stats["fused_reduces"] - before["fused_reduces"] == 1          # the variance
+        # mean, variance, and one kernel for the rest: + eps and sqrt run behind their broadcast
+        assert jt.executor_stats["launches"] - before["launches"] == 3
         ax = tuple(dims)
         want = (X - X.mean(ax, keepdims=True)) / np.sqrt(X.var(ax, keepdims=True) + 1e-5)
         assert np.allclose(got, want, rtol=1e-4, atol=1e-5), dims
@@ -687,6 +689,21 @@ def test_fused_reduce_with_per_output_inputs(gpu):
     got = (e / s).data
     ex = np.exp(X - X.max(2, keepdims=True))
     assert np.allclose(got, ex / ex.sum(2, keepdims=True), rtol=1e-5, atol=1e-7)
+    # the same chain with the broadcast sink switched off gives the same values from more launches
+    jt.flags["enable_broadcast_sink"] = False
+    try:
+        v = jt.array(x)
+        before = dict(jt.executor_stats)
+        mean = v.mean([2], keepdims=True)
+        var = ((v - mean) * (v - mean)).mean([2], keepdims=True)
+        ref = ((v - mean) / (var + 1e-5).sqrt()).data
+        assert jt.executor_stats["launches"] - before["launches"] > 3
+    finally:
+        jt.flags["enable_broadcast_sink"] = True
+    v = jt.array(x)
+    mean = v.mean([2], keepdims=True)
+    var = ((v - mean) * (v - mean)).mean([2], keepdims=True)
+    assert np.allclose(((v - mean) / (var + 1e-5).sqrt()).data, ref, rtol=1e-6, atol=1e-6)
     # an input broadcast along other axes than the reduced ones stays a separate kernel
     w = rng.standard_normal((1, 7, 1)).astype(np.float32)
     before = dict(jt.executor_stats)

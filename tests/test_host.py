@@ -348,3 +348,50 @@ def test_callers_build_path_graphs():
         x.reshape(5, -1)
     with pytest.raises(ValueError):
         jt.pad(x, (1, 2), "mirror")
+
+
+def test_executor_partitions_a_normalisation_into_three_kernels(monkeypatch):
+    """mean, variance (reduce with the subtraction and the square as prologue) and one element-wise kernel:
+    `+ eps` and `sqrt` act on the small variance and are evaluated behind their broadcast, and the
+    subtraction waits for the division's stage (python/jittor/test/test_new_fused_op.py:24-40 counts the same
+    three kernels).  The launches are replaced by recorders: no device is needed."""
+    import jittor_amd as jt
+    from jittor_amd import executor
+    log = []
+
+    def run_group(members, consumers, target_ids, reduce=None, pre=None):
+        ids = {m.id for m in members}
+        log.append(("group", [getattr(m, "op", m.kind) for m in members], reduce is not None,
+                    sorted(getattr(q, "op", q.kind) for m in members for q in (pre or {}).get(m.id, ()))))
+        if reduce is not None:
+            reduce.out._buf = object()
+        for m in members:
+            if m.out.id in target_ids or any(c.id not in ids for c in consumers.get(m.out.id, ())):
+                m.out._buf = object()
+        return True
+
+    def run_single(op):
+        log.append(("single", getattr(op, "op", op.kind)))
+        op.out._buf = object()
+
+    monkeypatch.setattr(executor, "_run_group", run_group)
+    monkeypatch.setattr(executor, "_run_single", run_single)
+    v = jt.array(np.zeros((33, 7, 130), np.float32))
+    v._buf = object()
+    mean = v.mean([2], keepdims=True)
+    var = ((v - mean) * (v - mean)).mean([2], keepdims=True)
+    y = (v - mean) / (var + 1e-5).sqrt()
+    executor._execute(executor._pending_ops([y]), {y.id})
+    assert log[0] == ("single", "mean")
+    assert log[1][0] == "group" and log[1][2] and log[1][1].count("subtract") == 2 and "multiply" in log[1][1]
+    assert log[2][0] == "group" and not log[2][2] and log[2][1][-1] == "divide" and "subtract" in log[2][1]
+    assert log[2][3] == ["add", "broadcast", "sqrt"] and len(log) == 3
+    # both rules can be switched off
+    log.clear()
+    monkeypatch.setitem(executor.flags, "enable_broadcast_sink", False)
+    v2 = jt.array(np.zeros((4, 6), np.float32))
+    v2._buf = object()
+    s = v2.sum([1], keepdims=True)
+    z = v2 / (s + 1.0)
+    executor._execute(executor._pending_ops([z]), {z.id})
+    assert [e[0] for e in log] == ["single", "group", "group"]      # sum, s + 1, division
