@@ -121,3 +121,62 @@ def test_random_fused_chains(gpu):
         want = refs[-1]
         assert got.shape == want.shape, (case, shape)
         assert np.allclose(got, want, rtol=3e-5, atol=1e-6, equal_nan=True), (case, shape, np.abs(got - want).max())
+
+
+def test_random_graphs_of_element_reduce_and_broadcast_ops(gpu):
+    """Random DAGs mixing element-wise ops, reduces with keepdims and the broadcasts that bring their results
+    back to the full shape (normalisation-like chains), several results fetched at once: what the executor
+    makes of them -- prologues, ops evaluated behind a broadcast, ops delayed to their consumers' stage -- must
+    not change any value.  Checked against the same DAG evaluated by numpy in float64."""
+    rng = np.random.default_rng(3000)
+    before = dict(jt.executor_stats)
+    unary = {"negative": np.negative, "abs": np.abs, "exp": lambda a: np.exp(np.clip(a, -20, 3)), "sigmoid": None,
+             "sqrt": lambda a: np.sqrt(np.abs(a))}
+    for case in range(60):
+        rank = int(rng.integers(2, 4))
+        shape = [int(rng.choice([2, 3, 5, 8, 17, 32, 65])) for _ in range(rank)]
+        pairs = []                                                        # (Var, float64 array)
+        for _ in range(int(rng.integers(1, 4))):
+            a = rng.uniform(-1.5, 1.5, shape).astype(np.float32)
+            pairs.append((jt.array(a), a.astype(np.float64)))
+
+        def pick(full_only=False):
+            cand = [p for p in pairs if not full_only or list(p[1].shape) == shape]
+            return cand[int(rng.integers(len(cand)))]
+
+        for step in range(int(rng.integers(4, 14))):
+            r = rng.random()
+            if r < 0.3:
+                name = list(unary)[int(rng.integers(len(unary)))]
+                v, a = pick()
+                if name == "sigmoid":
+                    pairs.append((jt.unary(v, "sigmoid"), 1.0 / (1.0 + np.exp(-a))))
+                elif name == "exp":
+                    pairs.append((jt.unary(v.minimum(3.0).maximum(-20.0), "exp"), unary[name](a)))
+                elif name == "sqrt":
+                    pairs.append((jt.unary(jt.unary(v, "abs"), "sqrt"), unary[name](a)))
+                else:
+                    pairs.append((jt.unary(v, name), unary[name](a)))
+            elif r < 0.65:
+                (v, a), (w, b) = pick(), pick()
+                op = ["add", "subtract", "multiply", "maximum"][int(rng.integers(4))]
+                f = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "maximum": np.maximum}[op]
+                pairs.append((jt.binary(v, w, op), f(a, b)))
+            elif r < 0.8:
+                v, a = pick()
+                k = float(rng.uniform(0.5, 2.0))
+                pairs.append((v * k + 0.25, a * np.float32(k) + 0.25))
+            else:
+                v, a = pick(full_only=True)
+                dims = sorted(set(int(d) for d in rng.integers(0, rank, int(rng.integers(1, rank)))))
+                op = ["add", "maximum", "mean"][int(rng.integers(3))]
+                f = {"add": np.sum, "maximum": np.max, "mean": np.mean}[op]
+                pairs.append((v.reduce(op, dims, True), f(a, axis=tuple(dims), keepdims=True)))
+        nout = int(rng.integers(1, 4))
+        chosen = [pairs[-1 - i] for i in range(min(nout, len(pairs)))]
+        got = jt.fetch_sync([v for v, _ in chosen])
+        for g, (_, want) in zip(got, chosen):
+            assert list(g.shape) == list(want.shape), (case, g.shape, want.shape)
+            scale = max(1.0, float(np.abs(want).max()))
+            assert np.allclose(g, want, rtol=2e-4, atol=2e-4 * scale), (case, float(np.abs(g - want).max()), scale)
+    assert jt.executor_stats["sunk_ops"] > before["sunk_ops"] and jt.executor_stats["fused_reduces"] > before["fused_reduces"]
