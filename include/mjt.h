@@ -219,6 +219,18 @@ typedef struct {
 int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y,
                     const mjt_conv_params* p);
 
+/* ---- matrix product ---------------------------------------------------
+ * c[n,k] = op(a) * op(b) for 2-d float operands of one dtype, op = transpose
+ * when the flag is set: the call the reference relays the pattern
+ * broadcast * broadcast -> reduce.add to (opt/tuner/matmul_tuner.cc:16-104 ->
+ * cublas_matmul, extern/cuda/cublas/ops/cublas_matmul_op.cc:27-56,118-126).
+ * c has the inputs' dtype, or float32 for 16-bit inputs; the accumulator is
+ * float32 (float64 for float64).  The product itself is rocBLAS' gemm_ex,
+ * loaded on first use: MJT_ERR_UNSUPPORTED when the library is absent, and
+ * mjt_matmul_available() tells beforehand (1 / 0). */
+int mjt_matmul(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, int trans_a, int trans_b);
+int mjt_matmul_available(void);
+
 /* ---- index-expression helper ------------------------------------------
  * Parses one index expression (the language of opt/expr.h:38-143 restricted
  * to what ops/reindex_op.h:58-68 allows) and, when it is affine in i0..i9

@@ -17,8 +17,8 @@ from .core import (Var, Buffer, UnaryOp, BinaryOp, TernaryOp, BroadcastOp,
 from ._lib import MjtError
 from . import profiler as _profiler
 
-stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0}
-flags = {"enable_conv_match": True, "enable_reduce_fusion": True, "enable_broadcast_sink": True}
+stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0, "matmul_matches": 0}
+flags = {"enable_conv_match": True, "enable_reduce_fusion": True, "enable_broadcast_sink": True, "enable_matmul_match": True}
 
 
 class ConvUnit:
@@ -31,6 +31,19 @@ class ConvUnit:
         self.inputs = [x, w]
         self.params = params
         self.absorbed = absorbed
+        self.id = reduce_op.id
+
+
+class MatmulUnit:
+    """broadcast * broadcast -> reduce.add over 2-d operands matched as one matrix product
+    (opt/tuner/matmul_tuner.cc:16-104)."""
+    kind = "matmul"
+    fusable = False
+
+    def __init__(self, reduce_op, a, b, trans_a, trans_b):
+        self.out = reduce_op.out
+        self.inputs = [a, b]
+        self.trans = (trans_a, trans_b)
         self.id = reduce_op.id
 
 
@@ -228,6 +241,38 @@ def _match_conv(red, consumers, targets):
     return None
 
 
+_matmul_ok = []
+
+
+def _match_matmul(red):
+    """reduce.add <- multiply <- {broadcast(xx), broadcast(yy)}, xx and yy 2-d, the product 3-d: the three
+    layouts the reference relays to its matmul op (matmul_tuner.cc:33-83), either operand order."""
+    if red.op != "add" or red.reduce_mask not in (0b001, 0b010, 0b100):
+        return None
+    yy = red.inputs[0]
+    if not yy.materialised and isinstance(yy._op, UnaryOp) and yy._op.op == "cast" and yy.dtype == "float32":
+        yy = yy._op.inputs[0]                                 # 16-bit inputs: cast -> reduce(float32) -> cast
+    if yy.materialised or yy.ndim != 3 or not isinstance(yy._op, BinaryOp) or yy._op.op != "multiply":
+        return None
+    a, b = yy._op.inputs
+    if a.materialised or b.materialised or not isinstance(a._op, BroadcastOp) or not isinstance(b._op, BroadcastOp):
+        return None
+    xa, xb = a._op.inputs[0], b._op.inputs[0]
+    if xa.ndim != 2 or xb.ndim != 2 or xa.dtype != xb.dtype or not xa.is_float():
+        return None
+    if red.out.dtype != xa.dtype and not (red.out.dtype == "float32" and xa.dtype in ("float16", "bfloat16")):
+        return None
+    table = {(0b010, 0b100, 0b001): (False, False), (0b001, 0b100, 0b010): (True, False), (0b100, 0b010, 0b001): (False, True)}
+    for (p, q, pm, qm) in ((xa, xb, a._op.bcast_mask, b._op.bcast_mask), (xb, xa, b._op.bcast_mask, a._op.bcast_mask)):
+        t = table.get((red.reduce_mask, pm, qm))
+        if t is None:
+            continue
+        if not _matmul_ok:
+            _matmul_ok.append(bool(_lib.load().mjt_matmul_available()))
+        return MatmulUnit(red, p, q, t[0], t[1]) if _matmul_ok[0] else None
+    return None
+
+
 def run_sync(targets, device_sync=False):
     targets = [t for t in targets if isinstance(t, Var)]
     stats["syncs"] += 1
@@ -262,6 +307,11 @@ def _execute(ops, target_ids):
             if cu is not None:
                 units[op.id] = cu
                 stats["conv_matches"] += 1
+            elif isinstance(op, ReduceOp) and flags["enable_matmul_match"]:
+                cu = _match_matmul(op)
+                if cu is not None:
+                    units[op.id] = cu
+                    stats["matmul_matches"] += 1
     nodes = [units.get(op.id, op) for op in ops]
     produced_by = {node.out.id: node for node in nodes}
     needed = set()
@@ -517,6 +567,13 @@ def _run_single(op):
         ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
         p = _lib.ConvParams(*op.params)
         _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
+    elif isinstance(op, MatmulUnit):
+        a, b = op.inputs
+        n = a.shape[1] if op.trans[0] else a.shape[0]
+        k = b.shape[0] if op.trans[1] else b.shape[1]
+        ta, tb = _tensor_of(a), _tensor_of(b)
+        tc = _lib.tensor(_alloc_out(out), out.dtype, [n, k])   # a kept reduced axis of extent 1 changes nothing in memory
+        _lib.check(lib.mjt_matmul(ctypes.byref(ta), ctypes.byref(tb), ctypes.byref(tc), int(op.trans[0]), int(op.trans[1])))
     elif isinstance(op, ConvBwdDataUnit):
         dy, w = op.inputs
         sh, sw, ph, pw, dh, dw = op.params

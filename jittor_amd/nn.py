@@ -61,3 +61,65 @@ def max_pool2d(x, kernel_size, stride=None, padding=0):
 
 def avg_pool2d(x, kernel_size, stride=None, padding=0):
     return pool(x, kernel_size, "mean", padding, stride)
+
+
+def matmul_transpose(a, b):
+    """a * b^T as broadcast, multiply, sum (python/jittor/nn.py:28-43); the executor recognises the group as
+    a matrix product (opt/tuner/matmul_tuner.cc:16-104)."""
+    a, b = core._as_var(a), core._as_var(b)
+    assert a.shape[-1] == b.shape[-1], (a.shape, b.shape)
+    if a.ndim != 2:
+        from . import misc
+        aa = misc.reshape(a, [-1, a.shape[-1]])
+        cc = matmul_transpose(aa, b)
+        return misc.reshape(cc, list(a.shape[:-1]) + [-1])
+    assert a.ndim == 2 and b.ndim == 2
+    shape = list(a.shape)[:-1] + list(b.shape)
+    a = core.broadcast(a, shape, [len(shape) - 2])
+    b = core.broadcast(b, shape)
+    return core.reduce(core.binary(a, b, "multiply"), "add", [len(shape) - 1])
+
+
+def matmul(a, b):
+    """Matrix product with the reference's shape rules (python/jittor/nn.py:83-159): vectors, matrices and
+    leading batch dimensions that broadcast, all through broadcast, multiply and sum."""
+    from . import misc
+    a, b = core._as_var(a), core._as_var(b)
+    len_a, len_b = a.ndim, b.ndim
+    if len_b == 1:
+        return core.reduce(core.binary(a, b, "multiply"), "add", [-1])           # a: [n, m], b: [m] -> [n]
+    if len_a == 1:
+        return core.reduce(core.binary(core.broadcast_var(a, b, [-1]), b, "multiply"), "add", [0])   # [n] x [n, k] -> [k]
+    len_c = max(len_a, len_b)
+    (n, m), (m_, k) = a.shape[-2:], b.shape[-2:]
+    assert m == m_, "dimension not match, a.shape:%s, b.shape:%s" % (a.shape, b.shape)
+    if len_b == 2 and len_a > 2:
+        cc = matmul(misc.reshape(a, [-1, m]), b)
+        return misc.reshape(cc, list(a.shape[:-1]) + [k])
+    shape = []
+    for i in range(len_c - 2):
+        ai, bi = len_a - (len_c - i), len_b - (len_c - i)
+        an = a.shape[ai] if ai >= 0 else 1
+        bn = b.shape[bi] if bi >= 0 else 1
+        if an != 1 and bn != 1:
+            assert an == bn, "dimension not match, a.shape:%s, b.shape:%s" % (a.shape, b.shape)
+        shape.append(max(an, bn))
+    shape.extend([n, m, k])
+    a = core.broadcast(a, shape, [-1])
+    b = core.broadcast(b, shape, [-3])
+    return core.reduce(core.binary(a, b, "multiply"), "add", [-2])
+
+
+def bmm(a, b):
+    """[batch, n, m] x [batch, m, k] (python/jittor/nn.py:57-80)."""
+    assert a.ndim >= 3 and a.ndim == b.ndim
+    return matmul(a, b)
+
+
+def linear(x, weight, bias=None):
+    """x * weight^T + bias (python/jittor/nn.py: linear)."""
+    y = matmul_transpose(x, weight)
+    return y if bias is None else core.binary(y, bias, "add")
+
+
+core.Var.matmul = core.Var.__matmul__ = matmul

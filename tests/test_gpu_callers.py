@@ -6,6 +6,8 @@ import numpy as np
 import pytest
 
 import jittor_amd as jt
+from jittor_amd import _lib as L
+from oracle import oracle as O
 
 pytestmark = pytest.mark.gpu
 
@@ -118,3 +120,59 @@ def test_profile_scope_report(gpu):
     total_ns = float(red[0][3])
     assert abs(float(red[0][7]) - 5 * 2 * a.nbytes / (total_ns * 1e-9)) / float(red[0][7]) < 1e-3
     assert np.allclose(y.data, (a.data.astype(np.float64) * b.data + 1).sum(1), rtol=1e-5, atol=1e-3)
+
+
+def test_matmul_forms_and_relay(gpu):
+    """jt.matmul / nn.matmul_transpose / nn.linear build broadcast * broadcast -> sum; 2-d products are
+    recognised (the three layouts of opt/tuner/matmul_tuner.cc:33-83) and run as one library GEMM, batched
+    and vector forms run on the generic kernels.  Values against numpy in float64."""
+    from jittor_amd import nn
+    rng = np.random.default_rng(50)
+    a = rng.standard_normal((70, 129)).astype(np.float32)
+    b = rng.standard_normal((129, 45)).astype(np.float32)
+    w = rng.standard_normal((45, 129)).astype(np.float32)
+    A, B, W = a.astype(np.float64), b.astype(np.float64), w.astype(np.float64)
+
+    def close(got, want, tol=1e-4):
+        return np.allclose(got, want, rtol=tol, atol=tol * np.abs(want).max())
+
+    before = dict(jt.executor_stats)
+    assert close(jt.matmul(jt.array(a), jt.array(b)).data, A @ B)
+    assert L.last_kernel() == "rocblas_gemm_ex"
+    assert close(nn.matmul_transpose(jt.array(a), jt.array(w)).data, A @ W.T)
+    assert close((jt.array(a) @ jt.array(b)).data, A @ B)
+    # the transposed-first layout appears in gradients: sum over axis 0 of [m, n, k]
+    at = jt.array(a.T.copy())
+    tn = (at.broadcast([129, 70, 45], [2]) * jt.array(b).broadcast([129, 70, 45], [1])).sum(0)
+    assert close(tn.data, A @ B)
+    assert jt.executor_stats["matmul_matches"] - before["matmul_matches"] == 4
+    # bfloat16 operands: float32 accumulation, result narrowed by the cast that follows the sum
+    ab, bb = jt.array(a).bfloat16(), jt.array(b).bfloat16()
+    got = jt.matmul(ab, bb)
+    assert got.dtype == "bfloat16"
+    want = O.BF16(ab.raw()).to_f32().astype(np.float64) @ O.BF16(bb.raw()).to_f32().astype(np.float64)
+    assert close(got.float32().data, want, 1e-2)
+    # the flag switches the relay off: same values from the generic path
+    jt.flags["enable_matmul_match"] = False
+    try:
+        assert close(jt.matmul(jt.array(a), jt.array(b)).data, A @ B)
+        assert L.last_kernel() != "rocblas_gemm_ex"
+    finally:
+        jt.flags["enable_matmul_match"] = True
+    # shape rules (python/jittor/nn.py:83-159)
+    x = rng.standard_normal((2, 3, 70, 129)).astype(np.float32)
+    assert close(jt.matmul(jt.array(x), jt.array(b)).data, x.astype(np.float64) @ B)
+    b3 = rng.standard_normal((3, 129, 45)).astype(np.float32)
+    assert close(jt.matmul(jt.array(x), jt.array(b3)).data, x.astype(np.float64) @ b3.astype(np.float64))
+    v = rng.standard_normal(129).astype(np.float32)
+    assert close(jt.matmul(jt.array(a), jt.array(v)).data, A @ v.astype(np.float64))
+    assert close(jt.matmul(jt.array(v), jt.array(b)).data, v.astype(np.float64) @ B)
+    bias = rng.standard_normal(45).astype(np.float32)
+    assert close(nn.linear(jt.array(x), jt.array(w), jt.array(bias)).data, x.astype(np.float64) @ W.T + bias)
+    # gradients of a product are products again (both are matched)
+    ja, jb = jt.array(a), jt.array(b)
+    before = dict(jt.executor_stats)
+    loss = (jt.matmul(ja, jb) * jt.array(np.ones((70, 45), np.float32))).sum()
+    da, db = jt.grad(loss, [ja, jb])
+    assert close(da.data, np.ones((70, 45)) @ B.T) and close(db.data, A.T @ np.ones((70, 45)))
+    assert jt.executor_stats["matmul_matches"] - before["matmul_matches"] >= 2

@@ -395,3 +395,22 @@ def test_executor_partitions_a_normalisation_into_three_kernels(monkeypatch):
     z = v2 / (s + 1.0)
     executor._execute(executor._pending_ops([z]), {z.id})
     assert [e[0] for e in log] == ["single", "group", "group"]      # sum, s + 1, division
+
+
+def test_matmul_entry_checks(compile_only):
+    """mjt_matmul validates like the reference's relay op (cublas_matmul_op.cc:34-52): 2-d float operands of one
+    dtype, matching inner extents, result [n, k]."""
+    L = compile_only
+    lib = L.load()
+    t = lambda dt, shape: L.tensor(0x1000, dt, shape)
+    call = lambda a, b, c, ta=0, tb=0: lib.mjt_matmul(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c), ta, tb)
+    assert call(t("float32", [4, 8]), t("float32", [8, 5]), t("float32", [4, 5])) == 0
+    assert call(t("float32", [8, 4]), t("float32", [8, 5]), t("float32", [4, 5]), 1, 0) == 0
+    assert call(t("float32", [4, 8]), t("float32", [5, 8]), t("float32", [4, 5]), 0, 1) == 0
+    assert call(t("bfloat16", [4, 8]), t("bfloat16", [8, 5]), t("float32", [4, 5])) == 0
+    assert call(t("float32", [4, 8]), t("float32", [7, 5]), t("float32", [4, 5])) == -1
+    assert call(t("float32", [4, 8]), t("float32", [8, 5]), t("float32", [5, 4])) == -1
+    assert call(t("float32", [4, 8]), t("float16", [8, 5]), t("float32", [4, 5])) == -1
+    assert call(t("int32", [4, 8]), t("int32", [8, 5]), t("int32", [4, 5])) == -1
+    assert call(t("float32", [4, 8, 1]), t("float32", [8, 5]), t("float32", [4, 5])) == -1
+    assert lib.mjt_matmul_available() in (0, 1)
