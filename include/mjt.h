@@ -224,6 +224,8 @@ int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* 
  * when the flag is set: the call the reference relays the pattern
  * broadcast * broadcast -> reduce.add to (opt/tuner/matmul_tuner.cc:16-104 ->
  * cublas_matmul, extern/cuda/cublas/ops/cublas_matmul_op.cc:27-56,118-126).
+ * With more than two dims the leading extents must be equal on a, b and c and
+ * count as a batch of products (cublas_batched_matmul_op.cc:63-85,113-166).
  * c has the inputs' dtype, or float32 for 16-bit inputs; the accumulator is
  * float32 (float64 for float64).  The product itself is rocBLAS' gemm_ex,
  * loaded on first use: MJT_ERR_UNSUPPORTED when the library is absent, and

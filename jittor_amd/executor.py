@@ -245,26 +245,36 @@ _matmul_ok = []
 
 
 def _match_matmul(red):
-    """reduce.add <- multiply <- {broadcast(xx), broadcast(yy)}, xx and yy 2-d, the product 3-d: the three
-    layouts the reference relays to its matmul op (matmul_tuner.cc:33-83), either operand order."""
-    if red.op != "add" or red.reduce_mask not in (0b001, 0b010, 0b100):
-        return None
+    """reduce.add <- multiply <- {broadcast(xx), broadcast(yy)}: the three layouts the reference relays to its
+    matmul op (matmul_tuner.cc:33-83), either operand order.  xx and yy are 2-d and the product 3-d, or all
+    carry the same leading batch extents (the batched product nn.matmul hands to cublas_batched_matmul,
+    python/jittor/nn.py:127-131)."""
     yy = red.inputs[0]
+    if red.op != "add":
+        return None
     if not yy.materialised and isinstance(yy._op, UnaryOp) and yy._op.op == "cast" and yy.dtype == "float32":
         yy = yy._op.inputs[0]                                 # 16-bit inputs: cast -> reduce(float32) -> cast
-    if yy.materialised or yy.ndim != 3 or not isinstance(yy._op, BinaryOp) or yy._op.op != "multiply":
+    nd = yy.ndim
+    if yy.materialised or nd < 3 or not isinstance(yy._op, BinaryOp) or yy._op.op != "multiply":
+        return None
+    nb = nd - 3                                               # leading batch axes
+    rm = red.reduce_mask >> nb
+    if red.reduce_mask & ((1 << nb) - 1) or rm not in (0b001, 0b010, 0b100):
         return None
     a, b = yy._op.inputs
     if a.materialised or b.materialised or not isinstance(a._op, BroadcastOp) or not isinstance(b._op, BroadcastOp):
         return None
     xa, xb = a._op.inputs[0], b._op.inputs[0]
-    if xa.ndim != 2 or xb.ndim != 2 or xa.dtype != xb.dtype or not xa.is_float():
+    am, bm = a._op.bcast_mask, b._op.bcast_mask
+    if xa.ndim != nb + 2 or xb.ndim != nb + 2 or xa.dtype != xb.dtype or not xa.is_float():
         return None
+    if (am | bm) & ((1 << nb) - 1) or xa.shape[:nb] != yy.shape[:nb] or xb.shape[:nb] != yy.shape[:nb]:
+        return None                                           # a batch axis that is broadcast: not a plain batched product
     if red.out.dtype != xa.dtype and not (red.out.dtype == "float32" and xa.dtype in ("float16", "bfloat16")):
         return None
     table = {(0b010, 0b100, 0b001): (False, False), (0b001, 0b100, 0b010): (True, False), (0b100, 0b010, 0b001): (False, True)}
-    for (p, q, pm, qm) in ((xa, xb, a._op.bcast_mask, b._op.bcast_mask), (xb, xa, b._op.bcast_mask, a._op.bcast_mask)):
-        t = table.get((red.reduce_mask, pm, qm))
+    for (p, q, pm, qm) in ((xa, xb, am >> nb, bm >> nb), (xb, xa, bm >> nb, am >> nb)):
+        t = table.get((rm, pm, qm))
         if t is None:
             continue
         if not _matmul_ok:
@@ -569,10 +579,11 @@ def _run_single(op):
         _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
     elif isinstance(op, MatmulUnit):
         a, b = op.inputs
-        n = a.shape[1] if op.trans[0] else a.shape[0]
-        k = b.shape[0] if op.trans[1] else b.shape[1]
+        n = a.shape[-1] if op.trans[0] else a.shape[-2]
+        k = b.shape[-2] if op.trans[1] else b.shape[-1]
         ta, tb = _tensor_of(a), _tensor_of(b)
-        tc = _lib.tensor(_alloc_out(out), out.dtype, [n, k])   # a kept reduced axis of extent 1 changes nothing in memory
+        # a kept reduced axis of extent 1 changes nothing in memory
+        tc = _lib.tensor(_alloc_out(out), out.dtype, list(a.shape[:-2]) + [n, k])
         _lib.check(lib.mjt_matmul(ctypes.byref(ta), ctypes.byref(tb), ctypes.byref(tc), int(op.trans[0]), int(op.trans[1])))
     elif isinstance(op, ConvBwdDataUnit):
         dy, w = op.inputs

@@ -164,6 +164,16 @@ def test_matmul_forms_and_relay(gpu):
     assert close(jt.matmul(jt.array(x), jt.array(b)).data, x.astype(np.float64) @ B)
     b3 = rng.standard_normal((3, 129, 45)).astype(np.float32)
     assert close(jt.matmul(jt.array(x), jt.array(b3)).data, x.astype(np.float64) @ b3.astype(np.float64))
+    assert L.last_kernel() != "rocblas_gemm_strided_batched_ex"       # a broadcast batch axis: generic kernels
+    b4 = rng.standard_normal((2, 3, 129, 45)).astype(np.float32)       # equal batch extents: one strided batched GEMM
+    jx, jb4 = jt.array(x), jt.array(b4)
+    y4 = jt.matmul(jx, jb4)
+    assert close(y4.data, x.astype(np.float64) @ b4.astype(np.float64))
+    assert L.last_kernel() == "rocblas_gemm_strided_batched_ex"
+    gx, gb = jt.grad((y4 * y4).sum(), [jx, jb4])
+    Y = x.astype(np.float64) @ b4.astype(np.float64)
+    assert close(gx.data, 2 * Y @ np.swapaxes(b4.astype(np.float64), -1, -2), 1e-3)
+    assert close(gb.data, np.swapaxes(x.astype(np.float64), -1, -2) @ (2 * Y), 1e-3)
     v = rng.standard_normal(129).astype(np.float32)
     assert close(jt.matmul(jt.array(a), jt.array(v)).data, A @ v.astype(np.float64))
     assert close(jt.matmul(jt.array(v), jt.array(b)).data, v.astype(np.float64) @ B)

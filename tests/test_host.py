@@ -413,4 +413,6 @@ def test_matmul_entry_checks(compile_only):
     assert call(t("float32", [4, 8]), t("float16", [8, 5]), t("float32", [4, 5])) == -1
     assert call(t("int32", [4, 8]), t("int32", [8, 5]), t("int32", [4, 5])) == -1
     assert call(t("float32", [4, 8, 1]), t("float32", [8, 5]), t("float32", [4, 5])) == -1
+    assert call(t("float32", [3, 4, 8]), t("float32", [3, 8, 5]), t("float32", [3, 4, 5])) == 0       # equal batch extents
+    assert call(t("float32", [3, 4, 8]), t("float32", [2, 8, 5]), t("float32", [3, 4, 5])) == -1
     assert lib.mjt_matmul_available() in (0, 1)
