@@ -467,6 +467,8 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_COLD(Params p) {
         plan.pfirst[t] = planin[3 * NBMAX + 1 + t];
     }
     if (threadIdx.x == 0) any_ovf = planin[4 * NBMAX + 2];
+    // fetched together with the plan: a merge item then has one memory round trip less in front of its rows
+    const int my_hot = (int)threadIdx.x < G1 ? hotof[threadIdx.x] : -1;
     __syncthreads();
     const TX ident = mjt_ident();
     for (unsigned item = blockIdx.x; item < plan.first[NBMAX]; item += gridDim.x) {
@@ -484,7 +486,7 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_COLD(Params p) {
         if (within >= SPLIT) {
             // merge item: segment sgm of the partial copies of main workgroups number g*MERGE_ROWS ... of this bucket
             const int g = (within - SPLIT) / MSEG, sgm = (within - SPLIT) - g * MSEG;
-            const unsigned match = (int)threadIdx.x < G1 && hotof[threadIdx.x] == bucket ? 1u : 0u;
+            const unsigned match = my_hot == bucket ? 1u : 0u;
             const unsigned incl = (unsigned)mjt_block_scan_value(match, wsum);
             if (match && (int)(incl - 1) / MERGE_ROWS == g) rows[(incl - 1) % MERGE_ROWS] = threadIdx.x;
             if (threadIdx.x == NTHREADS - 1) nmatch = incl;
