@@ -24,7 +24,7 @@
 //           bucket's population.  Entries that did not fit a list (rare: a
 //           second hot region) sit in per-workgroup overflow lists that item
 //           (bucket, 0) scans.  A merge item merges a segment of the private
-//           copies of 16 main workgroups that had the same hot bucket;
+//           copies of 32 main workgroups that had the same hot bucket;
 //   final   x[bin] = merge of the partial copies of its bucket (plain stores:
 //           x needs no prior fill).
 // Workgroups of one launch share nothing, so no buffer has to be cleared
@@ -353,7 +353,7 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
 // compute unit pulls little more than 100 GB/s: an item should not read more than about 100 KB).
 // first[b] is the number of the bucket's first item, pfirst[b] of its first partial copy; first[NBMAX] and
 // pfirst[NBMAX] are the totals.
-constexpr int MERGE_ROWS = 16;
+constexpr int MERGE_ROWS = 32;
 constexpr int MBINS = WBINS < 2048 ? WBINS : 2048;
 constexpr int MSEG = WBINS / MBINS;
 struct mjt_plan {

@@ -170,7 +170,7 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     const int64_t per = ((n + G1 - 1) / G1 + chunk - 1) / chunk * chunk;
     G1 = n ? (n + per - 1) / per : 1;
     // cold items: at most one per bucket plus population / cold_target (see mjt_make_plan)
-    // plus the merge items: one per 16 main workgroups of a bucket
+    // plus the partial copies of the merge items: at most one per 16 main workgroups of a bucket and one per bucket
     const int64_t cold_items = NB + n / cold_target + 1 + G1 / 16 + (NB < G1 ? NB : G1) + 1;
     int64_t cold_wgs = (int64_t)c.prop.multiProcessorCount * (acc64 ? 1 : 2);
     if (cold_wgs > cold_items) cold_wgs = cold_items;
