@@ -144,7 +144,7 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     int64_t nbmax = 1;
     while (nbmax < NB) nbmax *= 2;
     const int per_cu = env_int("MJT_SCATTER_WG_PER_CU", 1);
-    const int64_t cold_target = env_int("MJT_SCATTER_COLD_TARGET", 16384);   // list entries per cold item
+    const int64_t cold_target = env_int("MJT_SCATTER_COLD_TARGET", 24576);   // list entries per cold item
     const int acc64 = mode == 0 && x->dtype == MJT_FLOAT32 && env_int("MJT_SCATTER_ACC64", 1);
     const int ept = env_int("MJT_SCATTER_EPT", 8);           // elements per thread and round
     if (ept < 4 || ept % 4 || ept > 32) return false;
