@@ -99,8 +99,36 @@ def _lazy_op(v, cls):
     return v._op if (not v.materialised and isinstance(v._op, cls)) else None
 
 
+_FLOAT_RANK = {"float16": 1, "bfloat16": 1, "float32": 2, "float64": 3}
+
+
+def _lazy_broadcast(v):
+    """The BroadcastOp behind v and the var it spreads, looking through float casts that change nothing:
+    cast(broadcast(cast(s))) with only wider float types in between and v.dtype == s.dtype, which is what
+    the gradient of a 16-bit convolution puts between dy and the product (the sum runs in float32,
+    ops/reduce_op.cc:259-266).  Returns (op, source) or (None, None)."""
+    chain = [v.dtype]
+    u = v
+    while not u.materialised and isinstance(u._op, UnaryOp) and u._op.op == "cast":
+        u = u._op.inputs[0]
+        chain.append(u.dtype)
+    bo = _lazy_op(u, BroadcastOp)
+    if bo is None:
+        return None, None
+    src = bo.inputs[0]
+    while not src.materialised and isinstance(src._op, UnaryOp) and src._op.op == "cast":
+        src = src._op.inputs[0]
+        chain.append(src.dtype)
+    if len(chain) > 1:
+        r0 = _FLOAT_RANK.get(src.dtype)
+        if r0 is None or src.dtype != v.dtype or any(_FLOAT_RANK.get(d, 0) < r0 or (_FLOAT_RANK.get(d) == r0 and d != src.dtype)
+                                                     for d in chain):
+            return None, None
+    return bo, src
+
+
 def _match_conv_bwd(op):
-    """The two gradient patterns of the meta-op convolution as jt.grad builds them (fp32 / equal dtypes)."""
+    """The two gradient patterns of the meta-op convolution as jt.grad builds them."""
     if isinstance(op, ReindexReduceOp) and op.op == "add" and len(op.inputs) == 1 and not op.overflow_conditions:
         y7 = op.inputs[0]
         mul = _lazy_op(y7, BinaryOp)
@@ -111,10 +139,9 @@ def _match_conv_bwd(op):
             return None                                         # stride 1 only
         N, K, C, OH, OW, R, S = y7.shape
         for a, b in (mul.inputs, mul.inputs[::-1]):
-            ba, bb = _lazy_op(a, BroadcastOp), _lazy_op(b, BroadcastOp)
+            (ba, w), (bb, dy) = _lazy_broadcast(a), _lazy_broadcast(b)
             if ba is None or bb is None or ba.bcast_mask != 0b0011001 or bb.bcast_mask != 0b1100100:
                 continue
-            w, dy = ba.inputs[0], bb.inputs[0]
             if list(w.shape) != [K, C, R, S] or list(dy.shape) != [N, K, OH, OW] or w.dtype != dy.dtype:
                 continue
             if w.dtype not in ("float32", "bfloat16") or op.out.dtype not in ("float32", w.dtype):
@@ -128,6 +155,8 @@ def _match_conv_bwd(op):
         return None
     if isinstance(op, ReduceOp) and op.op == "add" and op.reduce_mask == 0b0011001 and op.out.ndim == 4:
         y7 = op.inputs[0]
+        if not y7.materialised and isinstance(y7._op, UnaryOp) and y7._op.op == "cast" and y7.dtype == "float32":
+            y7 = y7._op.inputs[0]                             # 16-bit product summed in float32
         mul = _lazy_op(y7, BinaryOp)
         if mul is None or mul.op != "multiply" or y7.ndim != 7:
             return None
@@ -135,12 +164,12 @@ def _match_conv_bwd(op):
         if list(op.out.shape) != [K, C, R, S]:
             return None
         for a, b in (mul.inputs, mul.inputs[::-1]):
-            ra, bb = _lazy_op(a, ReindexOp), _lazy_op(b, BroadcastOp)
+            ra, (bb, dy) = _lazy_op(a, ReindexOp), _lazy_broadcast(b)
             if ra is None or bb is None or bb.bcast_mask != 0b1100100 or len(ra.inputs) != 1:
                 continue
             if ra.overflow_conditions or ra.overflow_value != 0.0:
                 continue
-            x, dy = ra.inputs[0], bb.inputs[0]
+            x = ra.inputs[0]
             if x.ndim != 4 or list(dy.shape) != [N, K, OH, OW] or x.dtype != dy.dtype or x.shape[0] != N or x.shape[1] != C:
                 continue
             if x.dtype not in ("float32", "bfloat16") or op.out.dtype not in ("float32", x.dtype):
@@ -601,12 +630,48 @@ def _run_single(op):
         sh, sw, ph, pw, dh, dw = op.params
         N, C, H, W = x.shape
         _, K, OH, OW = dy.shape
+        R, S = out.shape[2], out.shape[3]
+        if not _matmul_ok:
+            _matmul_ok.append(bool(lib.mjt_matmul_available()))
+        if _matmul_ok[0] and flags["enable_matmul_match"]:
+            # dw[k, (c,r,s)] = sum over images of dy[n] [K, P] times cols[n]^T, cols[n] = the shifted input planes
+            # [(c,r,s), P] (P = OH*OW, the innermost axis of both): one reindex per chunk of images, one
+            # batched GEMM per chunk, one sum over the images.
+            esz = _lib.DTYPE_SIZE[x.dtype]
+            P, CRS = OH * OW, C * R * S
+            chunk = max(1, min(N, (1 << 30) // max(1, CRS * P * esz)))
+            pdt = "float32" if x.dtype in ("float16", "bfloat16") else x.dtype
+            cols = Var([chunk, C, R, S, OH, OW], x.dtype)
+            part = Var([N, K, CRS], pdt)
+            cols_ptr, part_ptr = _alloc_out(cols), _alloc_out(part)
+            idx = _lib.c_strings(["i0", "i1", "i4*%d-%d+i2*%d" % (sh, ph, dh), "i5*%d-%d+i3*%d" % (sw, pw, dw)])
+            none, ex = _lib.c_strings([]), (_lib.Tensor * 1)()
+            psz = _lib.DTYPE_SIZE[pdt]
+            for n0 in range(0, N, chunk):
+                nb = min(chunk, N - n0)
+                tx = _lib.tensor(x._device_ptr() + n0 * C * H * W * esz, x.dtype, [nb, C, H, W])
+                tc = _lib.tensor(cols_ptr, x.dtype, [nb, C, R, S, OH, OW])
+                _lib.check(lib.mjt_reindex(ctypes.byref(tx), ctypes.byref(tc), 4, idx, 0.0, 0, none, 0, ex))
+                ta = _lib.tensor(dy._device_ptr() + n0 * K * P * esz, dy.dtype, [nb, K, P])
+                tb = _lib.tensor(cols_ptr, x.dtype, [nb, CRS, P])
+                tp = _lib.tensor(part_ptr + n0 * K * CRS * psz, pdt, [nb, K, CRS])
+                _lib.check(lib.mjt_matmul(ctypes.byref(ta), ctypes.byref(tb), ctypes.byref(tp), 0, 1))
+                stats["launches"] += 2
+            acc = out if out.dtype == pdt else Var([K, C, R, S], pdt)
+            tpart = _lib.tensor(part_ptr, pdt, [N, K * CRS])
+            tacc = _lib.tensor(_alloc_out(acc), pdt, [K * CRS])
+            _lib.check(lib.mjt_reduce(ctypes.byref(tpart), ctypes.byref(tacc), _lib.OP_CODE["add"], 0b01))
+            if acc is not out:                                 # narrow the float32 sum to the weights' dtype
+                with core.no_grad():
+                    narrowed = core.unary(acc, out.dtype)
+                _run_group([narrowed._op], {}, {narrowed.id})
+                out._buf = narrowed._buf
+            return
         with core.no_grad():
             xt = core.reindex(x, [C, N, H, W], ["i1", "i0", "i2", "i3"])
             dyt = core.reindex(dy, [K, N, OH, OW], ["i1", "i0", "i2", "i3"])
         _run_single(xt._op)
         _run_single(dyt._op)
-        R, S = out.shape[2], out.shape[3]
         tmp = Var([C, K, R, S], out.dtype)
         tx, tw = _tensor_of(xt), _tensor_of(dyt)
         tt = _lib.tensor(_alloc_out(tmp), tmp.dtype, tmp.shape)

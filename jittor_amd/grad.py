@@ -116,6 +116,9 @@ def _op_grad(op, inputs, out, dout, index):
     if isinstance(op, BroadcastOp):                     # ops/broadcast_to_op.cc:112-117
         if op.bcast_mask == 0:
             return dout
+        if dout.dtype in ("float16", "bfloat16"):          # the constructor's 16-bit rewrite (ops/reduce_op.cc:259-266)
+            r = core._reduce_mask(unary(dout, "float32"), "add", op.bcast_mask, op.keepdims_mask)
+            return unary(r, dout.dtype)
         return core._reduce_mask(dout, "add", op.bcast_mask, op.keepdims_mask)
     if isinstance(op, ReduceOp):                        # ops/reduce_op.cc:339-362
         bc = lambda v: core._broadcast_mask(v, x.shape, op.reduce_mask, op.keepdims_mask)

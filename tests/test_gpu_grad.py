@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 import jittor_amd as jt
+from oracle import oracle as O
 
 pytestmark = pytest.mark.gpu
 
@@ -203,6 +204,40 @@ def test_grad_meta_conv(gpu, case):
             assert not (v.ndim == 7 and v._buf is not None)
             if v._history is not None:
                 stack.extend(v._history[1])
+
+
+def test_grad_meta_conv_bfloat16(gpu):
+    """The same three units for bfloat16 operands: the float32 casts that the 16-bit sum puts between dy and
+    the products (ops/reduce_op.cc:259-266) are looked through, the MFMA kernel runs forward and input
+    gradient, the weight gradient is a batched GEMM over shifted input planes; gradients keep the dtype of
+    their variable."""
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((2, 64, 16, 16)).astype(np.float32)
+    w = (rng.standard_normal((64, 64, 3, 3)) * 0.05).astype(np.float32)
+    vx, vw = jt.array(x).bfloat16(), jt.array(w).bfloat16()
+    jt.sync([vx, vw])
+    xb = O.BF16(vx.raw()).to_f32()
+    wb = O.BF16(vw.raw()).to_f32()
+    y = jt.nn.conv2d(vx, vw, padding=1)
+    r = (rng.integers(-2, 3, y.shape) * 0.5).astype(np.float32)            # exact in bfloat16
+    gx, gw = jt.grad((y * jt.array(r).bfloat16()).sum(), [vx, vw])
+    assert gx.dtype == "bfloat16" and gw.dtype == "bfloat16"
+    before = jt.executor_stats["conv_matches"]
+    jt.sync([y, gx, gw])
+    assert jt.executor_stats["conv_matches"] - before == 3
+    dX, dW = _conv_grads_ref(xb, wb, r, 1, 1, 1)
+    tol = 2.0 ** -7                                                         # results are rounded to bfloat16
+    assert np.abs(gx.float32().numpy() - dX).max() <= tol * np.abs(dX).max()
+    assert np.abs(gw.float32().numpy() - dW).max() <= tol * np.abs(dW).max()
+    seen, stack = set(), [gx, gw, y]
+    while stack:
+        v = stack.pop()
+        if v.id in seen:
+            continue
+        seen.add(v.id)
+        assert not (v.ndim == 7 and v._buf is not None)
+        if v._history is not None:
+            stack.extend(v._history[1])
 
 
 def test_grad_stop_grad_and_no_grad(gpu):
