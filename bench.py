@@ -295,12 +295,12 @@ def wl_copy(L, lib, steps, warmup, with_cpu):
 # Summaries: profiles/hbm_traffic_all_workloads.txt
 MEASURED_TRAFFIC = {
     "C1": 2.0 * 65557.6 * 1024 + 64.0 * 1024,
-    "C2": 2.0 * 15635.8 * 1024 + 225838.1 * 1024,
-    "C3add": 2.0 * 65650.4 * 1024 + 41041.1 * 1024,
-    "C3max": 2.0 * 65650.3 * 1024 + 41335.3 * 1024,
-    "C4": 2.0 * 65583.3 * 1024 + 131072.0 * 1024,
-    "C5": 2.0 * 113396.9 * 1024 + 212053.2 * 1024,
-    "C5bf16out": 2.0 * 112137.5 * 1024 + 113048.5 * 1024,
+    "C2": 2.0 * 15636.0 * 1024 + 225834.9 * 1024,
+    "C3add": 2.0 * 65692.8 * 1024 + 41163.5 * 1024,
+    "C3max": 2.0 * 65695.2 * 1024 + 41701.9 * 1024,
+    "C4": 2.0 * 65583.9 * 1024 + 131072.0 * 1024,
+    "C5": 2.0 * 113421.8 * 1024 + 211875.7 * 1024,
+    "C5bf16out": 2.0 * 112180.0 * 1024 + 112985.8 * 1024,
 }
 
 WORKLOADS = {
