@@ -219,6 +219,14 @@ typedef struct {
 int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y,
                     const mjt_conv_params* p);
 
+/* The grouped form (python/jittor/nn.py:1272-1294: reindex(x) * reindex(w) ->
+ * reindex_reduce.add, the group count handed to the tuner as compile option
+ * "G"): x [N, groups*Cg, H, W], w [K, Cg, R, S], y [N, K, OH, OW]; output
+ * channel k reads the Cg input channels of group k / (K / groups).
+ * groups == 1 is mjt_conv2d_meta. */
+int mjt_conv2d_meta_grouped(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y,
+                            const mjt_conv_params* p, int groups);
+
 /* ---- matrix product ---------------------------------------------------
  * c[n,k] = op(a) * op(b) for 2-d float operands of one dtype, op = transpose
  * when the flag is set: the call the reference relays the pattern

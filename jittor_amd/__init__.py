@@ -162,18 +162,23 @@ def ternary_out_hint(cond, x, y):
 
 
 def histc(input, bins, min=0.0, max=0.0):
-    """python/jittor/misc.py:2212-2235: scatter-add of ones by bin index.
-    `input` is a 1-d Var."""
-    if input.ndim != 1:
-        raise ValueError("histc expects a 1-d Var")
+    """Histogram of an N-d Var with `bins` equal bins over [min, max] (python/jittor/misc.py:2212-2235): a
+    scatter-add of ones by bin index floor((x - min) / ((max - min) / bins)).  Values outside [min, max] are
+    not counted and values equal to max go to the last bin, as there; the reference selects the values in
+    range with a boolean mask first, here they keep their place and get an index outside [0, bins), which
+    reindex_reduce drops."""
+    if bins <= 0:
+        raise RuntimeError("bins must be > 0, but got %s" % bins)
+    flat = input.reshape([input.num]) if input.ndim != 1 else input
     if min == 0 and max == 0:
-        lo, hi = input.min().item(), input.max().item()
+        lo, hi = flat.min().item(), flat.max().item()
     else:
         lo, hi = min, max
-    assert lo <= hi
-    if hi - lo < 1e-5:
-        hi, lo = hi + 1e-5, lo - 1e-5
-    pos = (input - lo) * (bins / (hi - lo))
-    idx = unary(pos, "floor_int").minimum(bins - 1)
-    one = ones(input.shape, "float32")
+    assert lo < hi
+    bin_length = (hi - lo) / bins
+    idx = unary((flat - lo) / bin_length, "floor_int")
+    inside = binary(flat >= lo, flat < hi, "logical_and")
+    idx = ternary(inside, idx, ternary(flat == hi, broadcast(array(bins - 1, "int32"), idx.shape),
+                                       broadcast(array(-1, "int32"), idx.shape)))
+    one = ones(flat.shape, "float32")
     return reindex_reduce(one, "add", [bins], ["@e0(i0)"], extras=[idx])

@@ -2,7 +2,9 @@
 // cover: one lane per output element, the reference's loop order (c, kh, kw)
 // with float products and a float32 accumulator
 // (python/jittor/nn.py:1251-1262, python/jittor/src/ops/reduce_op.cc:374-399).
-// Supplied by the host: TIN (element type of x and w), TOUT, and the geometry.
+// With G_ > 1 the channels fall into G_ groups: output channel ko belongs to group ko / (K_ / G_) and
+// sees the C_ input channels of that group only (python/jittor/nn.py:1272-1294); x has C_ * G_ channels.
+// Supplied by the host: TIN (element type of x and w), TOUT, G_ and the geometry (C_ = channels per group).
 
 struct Params { void* a[4]; };   // 8-byte words; typed as pointers so loads/stores use the global address space   // x, w, y, number of outputs
 
@@ -17,13 +19,14 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const int oh = (int)((o / OW_) % OH_);
     const int ko = (int)((o / ((long long)OW_ * OH_)) % K_);
     const long long n = o / ((long long)OW_ * OH_ * K_);
+    const int cbase = (ko / (K_ / G_)) * C_;          // first input channel of ko's group
     float acc = 0.0f;
     for (int c = 0; c < C_; c++)
         for (int kh = 0; kh < R_; kh++)
             for (int kw = 0; kw < S_; kw++) {
                 const int ih = oh * SH - PH + kh * DH, iw = ow * SW - PW + kw * DW;
                 const bool ov = ih < 0 || ih >= H_ || iw < 0 || iw >= W_;
-                const float xv = ov ? 0.0f : (float)xp[((n * C_ + c) * H_ + ih) * W_ + iw];
+                const float xv = ov ? 0.0f : (float)xp[((n * (C_ * G_) + cbase + c) * H_ + ih) * W_ + iw];
                 const float wv = (float)wp[(((long long)ko * C_ + c) * R_ + kh) * S_ + kw];
                 acc = acc + xv * wv;
             }

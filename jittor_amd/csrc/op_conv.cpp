@@ -23,7 +23,7 @@ void* g_wpack = nullptr;
 size_t g_wpack_bytes = 0;
 }  // namespace
 
-void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p) {
+void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p, int64_t G) {
     require_init();
     check_tensor(x, "conv x");
     check_tensor(w, "conv w");
@@ -33,9 +33,12 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     MJT_CHECK(x->dtype == w->dtype && (x->dtype == MJT_BFLOAT16 || x->dtype == MJT_FLOAT32),
               "conv: x and w must both be bfloat16 or float32");
     MJT_CHECK(y->dtype == MJT_FLOAT32 || y->dtype == x->dtype, "conv: y must be float32 or the input dtype");
-    const int64_t N = x->shape[0], C = x->shape[1], H = x->shape[2], W = x->shape[3];
+    MJT_CHECK(G >= 1, "conv: groups must be >= 1, got " << G);
+    // C is the number of channels one output channel sees: all of x's, or those of its group
+    const int64_t N = x->shape[0], C = w->shape[1], H = x->shape[2], W = x->shape[3];
     const int64_t K = w->shape[0], R = w->shape[2], S = w->shape[3];
-    MJT_CHECK(w->shape[1] == C, "conv: weight channels " << w->shape[1] << " != input channels " << C);
+    MJT_CHECK(x->shape[1] == C * G, "conv: weight channels " << C << " x " << G << " group(s) != input channels " << x->shape[1]);
+    MJT_CHECK(K % G == 0, "conv: " << K << " output channels do not divide into " << G << " groups");
     MJT_CHECK(p->stride_h >= 1 && p->stride_w >= 1 && p->dil_h >= 1 && p->dil_w >= 1 && p->pad_h >= 0 && p->pad_w >= 0,
               "conv: bad stride / padding / dilation");
     const int64_t OH = (H + 2 * p->pad_h - p->dil_h * (R - 1) - 1) / p->stride_h + 1;
@@ -71,7 +74,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
     const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
     const int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
-    const bool mfma_ok = x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 64 == 0 &&
+    const bool mfma_ok = G == 1 && x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 64 == 0 &&
                          W % 8 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 144 <= 72 * 1024 &&
                          (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49;
     if (mfma_ok) {
@@ -156,16 +159,17 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
 
     // ---- direct path ----------------------------------------------------------------
     std::ostringstream key;
-    key << "direct|" << geo.str() << x->dtype << "|" << y->dtype;
+    key << "direct|" << geo.str() << x->dtype << "|" << y->dtype << "|" << G;
     JitKernel* k = cached(key.str());
     if (!k) {
         std::ostringstream name;
         name << "mjt_conv_direct_" << mjt_dtype_name(x->dtype) << "_" << mjt_dtype_name(y->dtype) << "_c" << C << "_k" << K
              << "_" << H << "x" << W << "_r" << R << "x" << S << "_s" << p->stride_h << "x" << p->stride_w << "_p" << p->pad_h
              << "x" << p->pad_w << "_d" << p->dil_h << "x" << p->dil_w;
+        if (G > 1) name << "_g" << G;
         std::ostringstream src;
         src << "#define ENTRY " << name.str() << "\n#define TIN " << dtype_cname(x->dtype) << "\n#define TOUT "
-            << dtype_cname(y->dtype) << "\n" << geo.str();
+            << dtype_cname(y->dtype) << "\n#define G_ " << G << "\n" << geo.str();
         src << embedded_source("prelude.h") << "\n" << embedded_source("conv_direct.h") << "\n";
         k = jit_get(src.str(), name.str());
         remember(key.str(), k);
@@ -180,5 +184,10 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
 }  // namespace mjt
 
 extern "C" int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p) {
-    return mjt::guarded([&] { mjt::conv_impl(x, w, y, p); });
+    return mjt::guarded([&] { mjt::conv_impl(x, w, y, p, 1); });
+}
+
+extern "C" int mjt_conv2d_meta_grouped(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p,
+                                       int groups) {
+    return mjt::guarded([&] { mjt::conv_impl(x, w, y, p, groups); });
 }

@@ -26,11 +26,12 @@ class ConvUnit:
     kind = "conv"
     fusable = False
 
-    def __init__(self, reduce_op, x, w, params, absorbed):
+    def __init__(self, reduce_op, x, w, params, absorbed, groups=1):
         self.out = reduce_op.out
         self.inputs = [x, w]
         self.params = params
         self.absorbed = absorbed
+        self.groups = groups
         self.id = reduce_op.id
 
 
@@ -270,6 +271,57 @@ def _match_conv(red, consumers, targets):
     return None
 
 
+def _match_conv_grouped(op):
+    """reindex_reduce.add <- multiply <- {reindex(x), reindex(w)} over the 8-d product
+    [N, G, K/G, C/G, OH, OW, R, S]: the grouped convolution as python/jittor/nn.py:1272-1294 writes it."""
+    if op.op != "add" or len(op.inputs) != 1 or op.overflow_conditions or op.out.ndim != 4:
+        return None
+    yy = op.inputs[0]
+    mul = _lazy_op(yy, BinaryOp)
+    if mul is None or mul.op != "multiply" or yy.ndim != 8:
+        return None
+    N, G, KG, CG, OH, OW, R, S = yy.shape
+    if list(op.out.shape) != [N, G * KG, OH, OW]:
+        return None
+
+    def is_sum(aff, terms, c0=0):
+        """aff == c0 + sum(coef * i_k for k, coef in terms)"""
+        return aff is not None and aff[0] == c0 and all(aff[1][k] == dict(terms).get(k, 0) for k in range(10))
+    out_aff = [_affine(e, op.out.shape, yy.shape) for e in op.indexes]
+    if len(out_aff) != 4 or not (is_sum(out_aff[0], [(0, 1)]) and is_sum(out_aff[1], [(1, KG), (2, 1)])
+                                 and is_sum(out_aff[2], [(4, 1)]) and is_sum(out_aff[3], [(5, 1)])):
+        return None
+    for a, b in (mul.inputs, mul.inputs[::-1]):
+        rx, rw = _lazy_op(a, ReindexOp), _lazy_op(b, ReindexOp)
+        if rx is None or rw is None or len(rx.inputs) != 1 or len(rw.inputs) != 1:
+            continue
+        if rx.overflow_conditions or rw.overflow_conditions or rx.overflow_value != 0.0:
+            continue
+        x, w = rx.inputs[0], rw.inputs[0]
+        if x.ndim != 4 or list(w.shape) != [G * KG, CG, R, S] or x.shape[0] != N or x.shape[1] != G * CG:
+            continue
+        if x.dtype != w.dtype or x.dtype not in ("float32", "bfloat16") or op.out.dtype not in ("float32", x.dtype):
+            continue
+        wa = [_affine(e, w.shape, yy.shape) for e in rw.indexes]
+        if len(wa) != 4 or not (is_sum(wa[0], [(1, KG), (2, 1)]) and is_sum(wa[1], [(3, 1)])
+                                and is_sum(wa[2], [(6, 1)]) and is_sum(wa[3], [(7, 1)])):
+            continue
+        xa = [_affine(e, x.shape, yy.shape) for e in rx.indexes]
+        if len(xa) != 4 or any(a_ is None for a_ in xa) or not (is_sum(xa[0], [(0, 1)]) and is_sum(xa[1], [(1, CG), (3, 1)])):
+            continue
+        (c0h, coh), (c0w, cow) = xa[2], xa[3]
+        if any(coh[k] for k in range(10) if k not in (4, 6)) or any(cow[k] for k in range(10) if k not in (5, 7)):
+            continue
+        sh, dh, sw, dw, ph, pw = coh[4], coh[6], cow[5], cow[7], -c0h, -c0w
+        if min(sh, dh, sw, dw) < 1 or ph < 0 or pw < 0:
+            continue
+        H, W = x.shape[2], x.shape[3]
+        if OH != (H + 2 * ph - dh * (R - 1) - 1) // sh + 1 or OW != (W + 2 * pw - dw * (S - 1) - 1) // sw + 1:
+            continue
+        return ConvUnit(op, x, w, (sh, sw, ph, pw, dh, dw), {op.id, mul.id, rx.id, rw.id}, groups=G)
+    return None
+
+
 _matmul_ok = []
 
 
@@ -343,6 +395,8 @@ def _execute(ops, target_ids):
                 cu = _match_conv(op, consumers, target_ids)
             if cu is None and isinstance(op, (ReduceOp, ReindexReduceOp)):
                 cu = _match_conv_bwd(op)
+            if cu is None and isinstance(op, ReindexReduceOp):
+                cu = _match_conv_grouped(op)
             if cu is not None:
                 units[op.id] = cu
                 stats["conv_matches"] += 1
@@ -605,7 +659,11 @@ def _run_single(op):
         tx, tw = _tensor_of(x), _tensor_of(w)
         ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
         p = _lib.ConvParams(*op.params)
-        _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
+        if op.groups > 1:
+            _lib.check(lib.mjt_conv2d_meta_grouped(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p),
+                                                   op.groups))
+        else:
+            _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
     elif isinstance(op, MatmulUnit):
         a, b = op.inputs
         n = a.shape[-1] if op.trans[0] else a.shape[-2]

@@ -20,16 +20,34 @@ def _pair(v):
 
 def conv2d(x, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
     """The meta-op convolution: reindex + broadcast + multiply + sum over
-    (C, Kh, Kw) (python/jittor/nn.py:1245-1269, groups == 1).  The executor
-    recognises the group and runs it as one MFMA kernel."""
-    if groups != 1:
-        raise NotImplementedError("conv2d: groups > 1 is outside the meta-op convolution path")
+    (C, Kh, Kw) (python/jittor/nn.py:1245-1269, groups == 1), or with groups > 1
+    reindex(x) * reindex(w) -> reindex_reduce.add over an 8-d product
+    (python/jittor/nn.py:1272-1294).  The executor recognises either group of ops
+    and runs it as one kernel."""
     padding, stride, dilation = _pair(padding), _pair(stride), _pair(dilation)
     N, C, H, W = x.shape
     K = weight.shape[0]
     Kh, Kw = weight.shape[-2:]
     oh = (H + padding[0] * 2 - Kh * dilation[0] + dilation[0] - 1) // stride[0] + 1
     ow = (W + padding[1] * 2 - Kw * dilation[1] + dilation[1] - 1) // stride[1] + 1
+    if groups != 1:
+        G, CpG = groups, C // groups
+        if groups < 1 or C % G or K % G or weight.shape[1] != CpG:
+            raise ValueError("conv2d: %d input and %d output channels with weight %s do not form %d groups"
+                             % (C, K, list(weight.shape), groups))
+        oc = K
+        xx = x.reindex([N, G, oc // G, CpG, oh, ow, Kh, Kw], [
+            "i0",
+            "i1*%d+i3" % CpG,
+            "i4*%d-%d+i6*%d" % (stride[0], padding[0], dilation[0]),
+            "i5*%d-%d+i7*%d" % (stride[1], padding[1], dilation[1]),
+        ])
+        ww = weight.reindex([N, G, oc // G, CpG, oh, ow, Kh, Kw], ["i1*%d+i2" % (oc // G), "i3", "i6", "i7"])
+        yy = xx * ww
+        y = yy.reindex_reduce("add", [N, oc, oh, ow], ["i0", "i1*%d+i2" % (oc // G), "i4", "i5"])
+        if bias is not None:
+            y = y + bias.broadcast(y.shape, [0, 2, 3])
+        return y
     xx = x.reindex([N, K, C, oh, ow, Kh, Kw], [
         "i0",
         "i2",

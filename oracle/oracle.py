@@ -878,3 +878,24 @@ def conv_meta(x, w, stride=1, padding=0, dilation=1):
     ww = broadcast_to(wf, xx.shape, [0, 3, 4])
     yy = binary(xx, ww, "multiply")
     return reduce(yy, "add", [2, 5, 6])
+
+
+def conv_meta_grouped(x, w, groups, stride=1, padding=0, dilation=1):
+    """The grouped form, python/jittor/nn.py:1272-1294: x [N,G*Cg,H,W], w [K,Cg,R,S];
+    reindex(x) * reindex(w) over [N,G,K/G,Cg,OH,OW,R,S], then reindex_reduce.add into
+    [N,K,OH,OW] (a sequential float32 sum in the loop order of the 8-d product)."""
+    xf = x.to_f32() if isinstance(x, BF16) else np.asarray(x, dtype=np.float32)
+    wf = w.to_f32() if isinstance(w, BF16) else np.asarray(w, dtype=np.float32)
+    N, C, H, W = xf.shape
+    K, CpG, R, S = wf.shape
+    G = groups
+    assert C == CpG * G and K % G == 0
+    oh = (H + padding * 2 - R * dilation + dilation - 1) // stride + 1
+    ow = (W + padding * 2 - S * dilation + dilation - 1) // stride + 1
+    shape = [N, G, K // G, CpG, oh, ow, R, S]
+    xx = reindex(xf, shape, ["i0", "i1*%d+i3" % CpG, "i4*%d-%d+i6*%d" % (stride, padding, dilation),
+                             "i5*%d-%d+i7*%d" % (stride, padding, dilation)])
+    ww = reindex(wf, shape, ["i1*%d+i2" % (K // G), "i3", "i6", "i7"])
+    yy = binary(xx, ww, "multiply")
+    return reindex_reduce(yy, "add", [N, K, oh, ow], ["i0", "i1*%d+i2" % (K // G), "i4", "i5"])
+

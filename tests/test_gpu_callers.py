@@ -186,3 +186,21 @@ def test_matmul_forms_and_relay(gpu):
     da, db = jt.grad(loss, [ja, jb])
     assert close(da.data, np.ones((70, 45)) @ B.T) and close(db.data, A.T @ np.ones((70, 45)))
     assert jt.executor_stats["matmul_matches"] - before["matmul_matches"] >= 2
+
+
+def test_histc_ranges(gpu):
+    """jt.histc (python/jittor/misc.py:2212-2235): values outside [min, max] are not counted, a value equal
+    to max lands in the last bin, N-d inputs are flattened; with min == max == 0 the range is the data's."""
+    rng = np.random.default_rng(77)
+    x = (rng.integers(-4, 40, (37, 50)) / 8.0 + 1.0 / 16).astype(np.float32)      # well inside the bins
+    x[3, :5] = 4.0                                                                # == max
+    h = jt.histc(jt.array(x), 8, 0.0, 4.0).data
+    want = np.histogram(x, 8, (0.0, 4.0))[0].astype(np.float32)
+    assert h.dtype == np.float32 and np.array_equal(h, want)
+    assert h.sum() < x.size                                                       # some values were outside
+    y = rng.integers(0, 16, 1000).astype(np.float32)                              # default range [0, 15]: 15 equal bins
+    h = jt.histc(jt.array(y), 15).data
+    want = np.bincount(np.minimum(y.astype(np.int64), 14), minlength=15).astype(np.float32)
+    assert np.array_equal(h, want)
+    with pytest.raises(RuntimeError):
+        jt.histc(jt.array(y), 0)

@@ -251,3 +251,21 @@ def test_grad_stop_grad_and_no_grad(gpu):
     assert not jt.grad(q.sum(), x).numpy().any()
     with pytest.raises(ValueError):
         jt.grad(jt.array([1, 2, 3]).sum(), x)
+
+
+def test_grad_grouped_conv(gpu):
+    """Gradients of the grouped convolution (nn.py:1272-1294): each group is an independent convolution, so the
+    gradients of its channel slices are those of the plain convolution (float64 closed form per group)."""
+    rng = np.random.default_rng(9)
+    G, cg, kg = 3, 2, 2
+    x = rng.standard_normal((2, G * cg, 7, 6)).astype(np.float32)
+    w = rng.standard_normal((G * kg, cg, 3, 3)).astype(np.float32)
+    vx, vw = jt.array(x), jt.array(w)
+    y = jt.nn.conv2d(vx, vw, padding=1, groups=G)
+    r = rng.standard_normal(y.shape).astype(np.float32)
+    gx, gw = jt.grad((y * jt.array(r)).sum(), [vx, vw])
+    jt.sync([gx, gw])
+    for g in range(G):
+        dX, dW = _conv_grads_ref(x[:, g * cg:(g + 1) * cg], w[g * kg:(g + 1) * kg], r[:, g * kg:(g + 1) * kg], 1, 1, 1)
+        close(gx.numpy()[:, g * cg:(g + 1) * cg], dX, rtol=1e-4, atol=1e-4)
+        close(gw.numpy()[g * kg:(g + 1) * kg], dW, rtol=1e-4, atol=1e-4)

@@ -3,6 +3,7 @@ against the CPU oracle on the same seeded inputs.  Bar: bit-exact for reindex
 and integer work; 1e-5 relative for fp32 reduce / element-wise; 1e-4 relative
 for atomic scatter-add.  Full-size benchmark shapes are checked through
 closed forms and size-independent properties."""
+import ctypes
 import json
 import os
 
@@ -532,6 +533,42 @@ def test_conv_direct_small_shapes_and_fp32(gpu):
         assert np.allclose(got, O.conv_meta(x, w, st, pd, dl), rtol=1e-5, atol=1e-5)
         got, _ = _conv_call(_bf16(x), _bf16(w), (st, st, pd, pd, dl, dl))
         assert np.allclose(got, O.conv_meta(O.BF16(_bf16(x)), O.BF16(_bf16(w)), st, pd, dl), rtol=1e-5, atol=1e-5)
+
+
+def test_conv_grouped_entry_and_front_end(gpu):
+    """Grouped convolution (python/jittor/nn.py:1272-1294): the C entry point against the oracle's 8-d
+    restatement, then nn.conv2d(groups=G) matched by the executor (one kernel, nothing of rank 8 in memory)
+    and, with the matcher off, through the generic reindex / reindex_reduce kernels."""
+    rng = np.random.default_rng(23)
+    for xs, ws, G, st, pd, dl in [((2, 6, 9, 8), (4, 3, 3, 3), 2, 1, 1, 1), ((1, 8, 10, 10), (8, 1, 3, 3), 8, 2, 1, 1),
+                                  ((2, 6, 7, 9), (9, 2, 3, 3), 3, 1, 2, 2)]:
+        x = rng.standard_normal(xs).astype(np.float32)
+        w = rng.standard_normal(ws).astype(np.float32)
+        want = O.conv_meta_grouped(x, w, G, st, pd, dl)
+        lib = L.load()
+        vx, vw, vy = jt.from_storage(x, "float32"), jt.from_storage(w, "float32"), jt.zeros(list(want.shape), "float32")
+        tx, tw = L.tensor(vx.raw_ptr(), "float32", vx.shape), L.tensor(vw.raw_ptr(), "float32", vw.shape)
+        ty = L.tensor(vy.raw_ptr(), "float32", vy.shape)
+        p = L.ConvParams(st, st, pd, pd, dl, dl)
+        L.check(lib.mjt_conv2d_meta_grouped(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p), G))
+        assert L.last_kernel().endswith("_g%d" % G)
+        assert np.allclose(L.d2h(vy.raw_ptr(), vy.shape, np.float32), want, rtol=1e-5, atol=1e-5)
+        before = jt.executor_stats["conv_matches"]
+        v = jt.nn.conv2d(jt.array(x), jt.array(w), stride=st, padding=pd, dilation=dl, groups=G)
+        got = v.data
+        assert jt.executor_stats["conv_matches"] == before + 1 and L.last_kernel().endswith("_g%d" % G)
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+        jt.flags["enable_conv_match"] = False
+        try:
+            got = jt.nn.conv2d(jt.array(x), jt.array(w), stride=st, padding=pd, dilation=dl, groups=G).data
+        finally:
+            jt.flags["enable_conv_match"] = True
+        assert np.allclose(got, want, rtol=1e-4, atol=1e-4)          # scatter-add: order differs
+    # wrong group count: an error, not a fault
+    rc = lib.mjt_conv2d_meta_grouped(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p), 2)
+    assert rc < 0 and "group" in lib.mjt_last_error().decode()
+    with pytest.raises(ValueError):
+        jt.nn.conv2d(jt.array(x), jt.array(w), groups=4)
 
 
 def test_conv_front_end_pattern_match(gpu):

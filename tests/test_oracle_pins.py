@@ -290,6 +290,22 @@ def test_conv_meta_vs_float64(stride, pad, dil):
     assert np.allclose(y, _conv_f64(x, w, stride, pad, dil), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("groups,stride,pad,dil", [(2, 1, 1, 1), (4, 2, 1, 1), (3, 1, 2, 2)])
+def test_conv_meta_grouped_is_one_convolution_per_group(groups, stride, pad, dil):
+    """A grouped convolution is `groups` independent convolutions over channel slices: the 8-d
+    restatement against the float64 convolution of each slice (a wrong group stride in either
+    reindex, or in the scatter back, mixes slices and fails this)."""
+    cg, kg = 2, 3
+    x = rng.standard_normal((2, groups * cg, 7, 6)).astype(np.float32)
+    w = rng.standard_normal((groups * kg, cg, 3, 3)).astype(np.float32)
+    y = O.conv_meta_grouped(x, w, groups, stride, pad, dil)
+    for g in range(groups):
+        want = _conv_f64(x[:, g * cg:(g + 1) * cg], w[g * kg:(g + 1) * kg], stride, pad, dil)
+        assert np.allclose(y[:, g * kg:(g + 1) * kg], want, rtol=1e-5, atol=1e-5)
+    one = O.conv_meta_grouped(x[:, :cg], w[:kg], 1, stride, pad, dil)                # one group = the plain form
+    assert np.allclose(one, O.conv_meta(x[:, :cg], w[:kg], stride, pad, dil), rtol=1e-6, atol=1e-6)
+
+
 def test_conv_meta_one_hot_kernel_is_a_shift():
     x = O.BF16(O.f32_to_bf16_bits(rng.standard_normal((1, 2, 6, 6)).astype(np.float32)))
     w = np.zeros((2, 2, 3, 3), np.float32)
