@@ -15,7 +15,8 @@ from . import _lib
 from ._lib import MjtError, init, shutdown, sync as _device_sync, device_info
 from .core import (Var, array, unary, binary, ternary, broadcast, broadcast_var,
                    reduce, reindex, reindex_var, reindex_reduce, make_number, from_storage)
-from .executor import run_sync, stats as executor_stats, flags
+from .executor import run_sync, stats as executor_stats
+from .flags import flags, flag_scope
 from . import dtypes
 from . import nn
 from .grad import grad

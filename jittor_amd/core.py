@@ -111,6 +111,7 @@ class Op:
         self.inputs = list(inputs)
         self.id = _new_id()
         self.out = None
+        self.amp = dt.amp_reg & 63          # the register at creation; its gradient is built under it (op.cc:38, grad.cc:48-55)
 
     def __repr__(self):
         return "%s#%d" % (self.kind, self.id)
@@ -460,6 +461,12 @@ def array(data, dtype=None):
     v._host = host.reshape(v.shape)
     if v.num == 1:
         v.is_scalar = True
+    if dt.amp_reg & dt.AMP_ARRAY_PREFER and v.num != 1 and dt.is_float(name):
+        # array-like ops follow the preference too (python/jittor/__init__.py:402-411)
+        if dt.amp_reg & dt.AMP_PREFER32:
+            return v if name == "float32" else unary(v, "float32")
+        if dt.amp_reg & dt.AMP_PREFER16:
+            return v if name == "float16" else unary(v, "float16")
     return v
 
 
@@ -655,10 +662,6 @@ def reduce(x, op, dims=(), keepdims=False):
         raise ValueError("unknown reduce op %r" % (op,))
     if op not in dt.REDUCE_OPS:
         raise ValueError("reduce op %r is not associative; not supported on the device" % (op,))
-    if x.dtype in ("float16", "bfloat16") and op in ("mean", "add"):
-        # improve 16-bit float precision: cast -> reduce -> cast (reduce_op.cc:259-266)
-        r = reduce(unary(x, "float32"), op, dims, keepdims)
-        return unary(r, x.dtype)
     if isinstance(dims, numbers.Integral):
         dims = (dims,)
     dims = list(dims)
@@ -678,6 +681,9 @@ def reduce(x, op, dims=(), keepdims=False):
 
 
 def _reduce_mask(x, op, rmask, kmask):
+    if not dt.amp_reg & dt.AMP_REDUCE16_DIRECT and x.dtype in ("float16", "bfloat16") and op in ("mean", "add"):
+        # improve 16-bit float precision: cast -> reduce -> cast (reduce_op.cc:259-266, 295-302)
+        return unary(_reduce_mask(unary(x, "float32"), op, rmask, kmask), x.dtype)
     ys = []
     for i in range(x.ndim):
         if rmask >> i & 1:

@@ -4,14 +4,16 @@
 //
 // Specialised at run time through these macros:
 //   TX, TY          element types of x and y
+//   TACC            accumulator type: TY, or float when TY is a 16-bit float type (the sum is
+//                   rounded to TY once, at the store)
 //   index_t         int or long long
 //   NK, NR          number of merged kept / reduced axes (each 0..5, NR >= 1)
 //   VEC             elements per vector load
 //   G               lanes that cooperate on one output (row kernel), power of 2 <= 64
 //   SPLIT           1: several workgroup rows share one output and write partials
-//   COMBINE(a, x)   first-level update, a is TY, x is TX
-//   MERGE(a, b)     update between two partial results, both TY
-//   INIT            identity, TY
+//   COMBINE(a, x)   first-level update, a is TACC, x is TX
+//   MERGE(a, b)     update between two partial results, both TACC
+//   INIT            identity, TACC
 //   ROW             1: innermost merged axis is reduced; 0: it is kept
 //   UNR             independent loads per lane and step (row kernel)
 //   MJT_LD          mjt_load or mjt_load_nt (streaming input)
@@ -102,14 +104,14 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     TY* __restrict__ yp = (TY*)p.a[1];
     const index_t O = (index_t)(unsigned long long)p.a[2];
     const index_t S = (index_t)(unsigned long long)p.a[3];
-    const TY rcount = (TY)__longlong_as_double((long long)(unsigned long long)p.a[4]);
+    const TACC rcount = (TACC)__longlong_as_double((long long)(unsigned long long)p.a[4]);
     (void)rcount;
     (void)xp;
     MJT_PRO_SCALARS
     const unsigned lane = threadIdx.x % G;
     const index_t o = (index_t)blockIdx.x * (256 / G) + threadIdx.x / G;
     const index_t s = blockIdx.y;
-    TY acc[VEC];
+    TACC acc[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; k++) acc[k] = INIT;
     if (o < O) {
@@ -136,7 +138,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 #pragma unroll
                 for (int u = 0; u < UNR; u++)
 #pragma unroll
-                    for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v[u].v[k]));
+                    for (int k = 0; k < VEC; k++) acc[k] = (TACC)(COMBINE(acc[k], v[u].v[k]));
             }
             for (; lc < lc_end; lc++) {
                 index_t l = (lc * G + lane) * VEC;
@@ -144,29 +146,29 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
                     mjt_pack<TX, VEC> v;
                     MJT_RD(v, row + l);
 #pragma unroll
-                    for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v.v[k]));
+                    for (int k = 0; k < VEC; k++) acc[k] = (TACC)(COMBINE(acc[k], v.v[k]));
                 }
             }
             lc = 0;
             ro++;
         }
     }
-    TY r = acc[0];
+    TACC r = acc[0];
 #pragma unroll
-    for (int k = 1; k < VEC; k++) r = (TY)(MERGE(r, acc[k]));
+    for (int k = 1; k < VEC; k++) r = (TACC)(MERGE(r, acc[k]));
 #pragma unroll
     for (int off = G / 2; off > 0; off >>= 1) {
-        TY other = mjt_shfl_xor_any(r, off);
-        r = (TY)(MERGE(r, other));
+        TACC other = mjt_shfl_xor_any(r, off);
+        r = (TACC)(MERGE(r, other));
     }
-    if (lane == 0 && o < O) yp[SPLIT ? o * S + s : o] = r;
+    if (lane == 0 && o < O) yp[SPLIT ? o * S + s : o] = (TY)r;
 }
 #else
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const TX* __restrict__ xp = (const TX*)p.a[0];
     TY* __restrict__ yp = (TY*)p.a[1];
     const index_t O = (index_t)(unsigned long long)p.a[2];
-    const TY rcount = (TY)__longlong_as_double((long long)(unsigned long long)p.a[4]);
+    const TACC rcount = (TACC)__longlong_as_double((long long)(unsigned long long)p.a[4]);
     (void)rcount;
     (void)xp;
     MJT_PRO_SCALARS
@@ -179,7 +181,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const index_t total = (index_t)(unsigned long long)p.a[6];
     index_t r = s * per;
     const index_t r_end = r + per < total ? r + per : total;
-    TY acc[VEC];
+    TACC acc[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; k++) acc[k] = INIT;
 #pragma unroll 4
@@ -188,11 +190,11 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
         mjt_pack<TX, VEC> v;
         MJT_RD(v, kbase + roff);
 #pragma unroll
-        for (int k = 0; k < VEC; k++) acc[k] = (TY)(COMBINE(acc[k], v.v[k]));
+        for (int k = 0; k < VEC; k++) acc[k] = (TACC)(COMBINE(acc[k], v.v[k]));
     }
     mjt_pack<TY, VEC> out;
 #pragma unroll
-    for (int k = 0; k < VEC; k++) out.v[k] = acc[k];
+    for (int k = 0; k < VEC; k++) out.v[k] = (TY)acc[k];
     mjt_store(yp + (SPLIT ? s * O : 0) + o, out);
 }
 #endif

@@ -40,6 +40,9 @@ struct Prologue {
     std::vector<std::pair<const void*, int>> inputs;   // (pointer, element size) of every tensor it loads
 };
 
+// 16-bit float results are accumulated in float32 and rounded once, at the store
+int acc_dtype(int ty) { return ty == MJT_FLOAT16 || ty == MJT_BFLOAT16 ? MJT_FLOAT32 : ty; }
+
 struct Variant {
     int tx, ty, op, nk, nr, vec, g, unr, nt;
     bool row, split, use64, second;   // second: folding partials (TX == TY, plain merge)
@@ -72,17 +75,17 @@ JitKernel* get_kernel(const Variant& v) {
     }
     std::ostringstream src;
     src << "#define ENTRY " << name.str() << "\n";
-    src << "#define TX " << dtype_cname(v.tx) << "\n#define TY " << dtype_cname(v.ty) << "\n";
+    src << "#define TX " << dtype_cname(v.tx) << "\n#define TY " << dtype_cname(v.ty) << "\n#define TACC " << dtype_cname(acc_dtype(v.ty)) << "\n";
     src << "#define index_t " << (v.use64 ? "long long" : "int") << "\n#define USE64 " << (v.use64 ? 1 : 0) << "\n";
     src << "#define NK " << v.nk << "\n#define NR " << v.nr << "\n#define VEC " << v.vec << "\n#define G " << v.g
         << "\n#define SPLIT " << (v.split ? 1 : 0) << "\n#define ROW " << (v.row ? 1 : 0) << "\n";
     src << "#define UNR " << v.unr << "\n#define MJT_LD " << (v.nt ? "mjt_load_nt" : "mjt_load") << "\n";
-    src << "#define MERGE(a, b) mjt_" << merge_op << "<TY>((a), (b))\n";
+    src << "#define MERGE(a, b) mjt_" << merge_op << "<TACC>((a), (b))\n";
     if (v.second || v.op != MJT_OP_MEAN)
-        src << "#define COMBINE(a, x) mjt_" << (v.second ? merge_op : std::string(opn)) << "<TY>((a), (x))\n";
+        src << "#define COMBINE(a, x) mjt_" << (v.second ? merge_op : std::string(opn)) << "<TACC>((a), (x))\n";
     else   // (acc + Ty(x) * Ty(rcount)), type/common_op_type.cc:141
-        src << "#define COMBINE(a, x) ((a) + TY(x) * TY(rcount))\n";
-    src << "#define INIT mjt_init_" << merge_op << "<TY>()\n";
+        src << "#define COMBINE(a, x) ((a) + TACC(x) * TACC(rcount))\n";
+    src << "#define INIT mjt_init_" << merge_op << "<TACC>()\n";
     if (v.pro) src << v.pro->defs;
     src << embedded_source("prelude.h") << "\n" << embedded_source("reduce.h") << "\n";
     JitKernel* k = jit_get(src.str(), name.str());
@@ -157,7 +160,7 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
               "reduce: op '" << (mjt_op_name(op) ? mjt_op_name(op) : "?") << "' is not an associative binary op");
     MJT_CHECK(reduce_mask != 0 && (reduce_mask >> x->ndim) == 0, "reduce: reduce_mask " << reduce_mask
                                                                                        << " does not fit rank " << x->ndim);
-    MJT_CHECK(dtype_size(y->dtype) >= 1 && y->dtype != MJT_FLOAT16 && y->dtype != MJT_BFLOAT16 && y->dtype != MJT_BOOL,
+    MJT_CHECK(dtype_size(y->dtype) >= 1 && y->dtype != MJT_BOOL,
               "reduce: accumulator dtype " << mjt_dtype_name(y->dtype) << " is not supported");
     int64_t xn = numel(x), O = 1;
     for (int d = 0; d < x->ndim; d++)
@@ -192,7 +195,9 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
     for (auto& a : red) R *= a.size;
     double rcount = xn ? (double)O / (double)xn : 0.0;
     int tx = x->dtype, ty = y->dtype;
+    const int ta = acc_dtype(ty);              // type of the partials of a split reduction
     int tsz = dtype_size(ty);
+    const int asz = dtype_size(ta);
 
     if (xn == 0 || red.empty()) {
         // nothing to fold (empty reduced axis -> identity; extent-1 reduced axes -> copy with conversion):
@@ -234,15 +239,15 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         if (S == 1) {
             launch(true, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, g, per, total, stream, pro);
         } else {
-            void* part = scratch((size_t)O * S * tsz);
-            launch(true, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, g, per, total, stream, pro);
+            void* part = scratch((size_t)O * S * asz);
+            launch(true, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, g, per, total, stream, pro);
             // fold [O, S] along the last axis
             std::vector<Axis> k2{Axis{O, S}}, r2{Axis{S, 1}};
-            int vec2 = pick_vec(tsz, S, part, nullptr, 0);
+            int vec2 = pick_vec(asz, S, part, nullptr, 0);
             int g2 = 64;
             while (g2 > 1 && (int64_t)(g2 / 2) * vec2 >= S) g2 /= 2;
             int64_t nL2 = (S + (int64_t)g2 * vec2 - 1) / ((int64_t)g2 * vec2);
-            launch(true, ty, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, g2, nL2, nL2);
+            launch(true, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, g2, nL2, nL2);
         }
     } else {
         int64_t Lk = kept.back().size;
@@ -265,11 +270,11 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         if (S == 1) {
             launch(false, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, 1, per, R, stream, pro);
         } else {
-            void* part = scratch((size_t)O * S * tsz);
-            launch(false, tx, ty, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R, stream, pro);
+            void* part = scratch((size_t)O * S * asz);
+            launch(false, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R, stream, pro);
             std::vector<Axis> k2{Axis{O, 1}}, r2{Axis{S, O}};
-            int vec2 = pick_vec(tsz, O, part, y->ptr, tsz);
-            launch(false, ty, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, 1, S, S);
+            int vec2 = pick_vec(asz, O, part, y->ptr, tsz);
+            launch(false, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, 1, S, S);
         }
     }
 }

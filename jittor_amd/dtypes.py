@@ -1,7 +1,8 @@
 """dtype vocabulary and inference rules of the meta-operator path.
 
-Restates python/jittor/src/misc/nano_string.h:205-277 (with amp_reg == 0) and
-the op classes of python/jittor/src/misc/nano_string.cc:45-160.
+Restates python/jittor/src/misc/nano_string.h:199-277, including the
+mixed-precision control register amp_reg (python/jittor/src/var.cc:28,65-71),
+and the op classes of python/jittor/src/misc/nano_string.cc:45-160.
 """
 import numpy as np
 
@@ -20,6 +21,24 @@ REDUCE_OPS = ["add", "multiply", "maximum", "minimum", "logical_and",
               "bitwise_xor", "mean"]
 
 
+# amp_reg bits (nano_string.h:199-203; bit 32: ops/reduce_op.cc:260)
+AMP_PREFER32 = 1
+AMP_PREFER16 = 2
+AMP_KEEP_REDUCE = 4
+AMP_KEEP_WHITE = 8
+AMP_ARRAY_PREFER = 16
+AMP_REDUCE16_DIRECT = 32      # a 16-bit add / mean is not rewritten to cast -> reduce(float32) -> cast
+amp_reg = 0
+
+
+def amp_reg_of_level(level):
+    """auto_mixed_precision_level -> amp_reg (var.cc:65-71)."""
+    if level <= 2:
+        return 0
+    return {3: AMP_KEEP_REDUCE | AMP_KEEP_WHITE, 4: AMP_PREFER16, 5: AMP_PREFER16 | AMP_ARRAY_PREFER,
+            6: AMP_PREFER16 | AMP_ARRAY_PREFER | AMP_KEEP_REDUCE | AMP_KEEP_WHITE}.get(level, amp_reg)
+
+
 def dsize_(name):
     return {1: 0, 2: 1, 4: 2, 8: 3}[DTYPE_SIZE[name]]
 
@@ -32,8 +51,13 @@ def is_int(name):
     return name in ("int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64")
 
 
-def float_dtype(d, has_bf16=False):
+def float_dtype(d, has_scalar=False, has_bf16=False):
     """nano_string.h:205-215."""
+    if not has_scalar:
+        if amp_reg & AMP_PREFER32:
+            return "float32"
+        if amp_reg & AMP_PREFER16:
+            return "bfloat16" if has_bf16 else "float16"
     if d == 3:
         return "float64"
     if d == 2:
@@ -54,7 +78,7 @@ def dtype_infer(x, y, xscalar=False, yscalar=False):
     if yscalar:
         d = dsize_(x)
     if is_float(x) or is_float(y):
-        return float_dtype(d, "bfloat16" in (x, y))
+        return float_dtype(d, xscalar or yscalar, "bfloat16" in (x, y))
     return int_dtype(d)
 
 
@@ -69,9 +93,9 @@ def binary_dtype_infer(op, x, y, xscalar=False, yscalar=False):
         d = dsize_(x)
     fl = op not in INT_OPS and (is_float(x) or is_float(y) or op in FLOAT_OPS)
     if fl:
-        if op in WHITE_OPS:
+        if op in WHITE_OPS and not amp_reg & AMP_KEEP_WHITE:
             return "float64" if d == 3 else "float32"
-        return float_dtype(d, "bfloat16" in (x, y))
+        return float_dtype(d, xscalar or yscalar, "bfloat16" in (x, y))
     if x == "bool" and y == "bool":
         return "bool"
     return int_dtype(d)
@@ -83,9 +107,9 @@ def unary_dtype_infer(op, x):
         return "bool"
     d = dsize_(x)
     if op in FLOAT_OPS:
-        if op in WHITE_OPS:
+        if op in WHITE_OPS and not amp_reg & AMP_KEEP_WHITE:
             return "float64" if d == 3 else "float32"
-        return float_dtype(d, x == "bfloat16")
+        return float_dtype(d, False, x == "bfloat16")
     if op in INT_OPS:
         return int_dtype(d)
     return x
@@ -96,6 +120,8 @@ def reduce_dtype_infer(op, x):
     if x == "bool":
         return "int32"
     if is_float(x) or op in FLOAT_OPS:
+        if amp_reg & AMP_KEEP_REDUCE:
+            return float_dtype(dsize_(x), False, x == "bfloat16")
         return "float64" if dsize_(x) == 3 else "float32"
     return x
 

@@ -16,9 +16,9 @@ from .core import (Var, Buffer, UnaryOp, BinaryOp, TernaryOp, BroadcastOp,
                    ReduceOp, ReindexOp, ReindexReduceOp)
 from ._lib import MjtError
 from . import profiler as _profiler
+from .flags import flags
 
 stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0, "matmul_matches": 0}
-flags = {"enable_conv_match": True, "enable_reduce_fusion": True, "enable_broadcast_sink": True, "enable_matmul_match": True}
 
 
 class ConvUnit:

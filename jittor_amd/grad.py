@@ -12,6 +12,7 @@ gradients, contributions of several consumers are added, a target the loss
 does not depend on gets zeros.
 """
 from . import core
+from . import dtypes as dt
 from .core import (Var, UnaryOp, BinaryOp, TernaryOp, BroadcastOp, ReduceOp, ReindexOp, ReindexReduceOp,
                    unary, binary, ternary, make_number, reindex, reindex_reduce, array)
 from . import _lib
@@ -116,9 +117,6 @@ def _op_grad(op, inputs, out, dout, index):
     if isinstance(op, BroadcastOp):                     # ops/broadcast_to_op.cc:112-117
         if op.bcast_mask == 0:
             return dout
-        if dout.dtype in ("float16", "bfloat16"):          # the constructor's 16-bit rewrite (ops/reduce_op.cc:259-266)
-            r = core._reduce_mask(unary(dout, "float32"), "add", op.bcast_mask, op.keepdims_mask)
-            return unary(r, dout.dtype)
         return core._reduce_mask(dout, "add", op.bcast_mask, op.keepdims_mask)
     if isinstance(op, ReduceOp):                        # ops/reduce_op.cc:339-362
         bc = lambda v: core._broadcast_mask(v, x.shape, op.reduce_mask, op.keepdims_mask)
@@ -194,7 +192,12 @@ def grad(loss, targets, retain_graph=True):
         for i, u in enumerate(inputs):
             if u.id not in dep or not u.is_float():
                 continue
-            du = _op_grad(op, inputs, v, g, i)
+            saved = dt.amp_reg                                  # an op's gradient is built under the register
+            dt.amp_reg |= getattr(op, "amp", 0)                 # the op was created with (grad.cc:48-55)
+            try:
+                du = _op_grad(op, inputs, v, g, i)
+            finally:
+                dt.amp_reg = saved
             if du is None:
                 continue
             if du.shape != u.shape:

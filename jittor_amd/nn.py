@@ -2,6 +2,7 @@
 with meta-operators exactly as the reference writes them
 (python/jittor/nn.py:166-183 and :1245-1269)."""
 from . import core
+from .flags import flags, flag_scope
 
 
 def relu(x):
@@ -48,15 +49,17 @@ def conv2d(x, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
         if bias is not None:
             y = y + bias.broadcast(y.shape, [0, 2, 3])
         return y
-    xx = x.reindex([N, K, C, oh, ow, Kh, Kw], [
-        "i0",
-        "i2",
-        "i3*%d-%d+i5*%d" % (stride[0], padding[0], dilation[0]),
-        "i4*%d-%d+i6*%d" % (stride[1], padding[1], dilation[1]),
-    ])
-    ww = weight.broadcast(xx.shape, [0, 3, 4])
-    yy = xx * ww
-    y = yy.sum([2, 5, 6])
+    # 16-bit operands: the sum keeps their type and is not routed through float32 casts (amp_reg | 36, nn.py:1250)
+    with flag_scope(amp_reg=flags.amp_reg | 36):
+        xx = x.reindex([N, K, C, oh, ow, Kh, Kw], [
+            "i0",
+            "i2",
+            "i3*%d-%d+i5*%d" % (stride[0], padding[0], dilation[0]),
+            "i4*%d-%d+i6*%d" % (stride[1], padding[1], dilation[1]),
+        ])
+        ww = weight.broadcast(xx.shape, [0, 3, 4])
+        yy = xx * ww
+        y = yy.sum([2, 5, 6])
     if bias is not None:
         b = bias.broadcast(y.shape, [0, 2, 3])
         y = y + b

@@ -579,7 +579,7 @@ def test_conv_front_end_pattern_match(gpu):
     y = jt.nn.conv2d(x, w, padding=1)              # reindex + broadcast + multiply + sum, bf16 output
     got = y.data
     assert jt.executor_stats["conv_matches"] == before["conv_matches"] + 1
-    assert y.dtype == "bfloat16" and L.last_kernel().startswith("mjt_fused_")     # trailing cast of the fp32 sum
+    assert y.dtype == "bfloat16" and L.last_kernel().endswith("_obf16")           # the sum keeps 16 bit (amp_reg | 36, nn.py:1250)
     from oracle import kernels as K
     acc = K.conv_meta_bf16(x.raw(), w.raw(), 1, 1, 1, 8)
     want = O.BF16(O.f32_to_bf16_bits(acc)).to_f32()
@@ -648,6 +648,30 @@ def test_index64_mode_beyond_2g_elements(gpu):
     ones = (y == 7).int32().sum().data[0]
     want = n // 251 + (1 if n % 251 > 7 else 0)
     assert int(ones) == want
+
+
+def test_reduce_with_16_bit_results(gpu):
+    """With amp_reg's keep_reduce a 16-bit float reduce keeps its type (nano_string.h:268-277), and with bit 32
+    add / mean are not routed through float32 casts (ops/reduce_op.cc:260): the kernel accumulates in float32
+    and rounds once.  Against the float32 reduce of the same values rounded the same way; row, column,
+    split and whole-tensor shapes."""
+    rng = np.random.default_rng(41)
+    for shape, dims in [((37, 129), [1]), ((37, 129), [0]), ((4, 70000), [1]), ((30000, 8), [0]), ((64, 96), [])]:
+        host = rng.uniform(-1, 1, shape).astype(np.float32)
+        for dtype in ("bfloat16", "float16"):
+            a = jt.array(host).cast(dtype)
+            exact = a.float32().data                                     # the 16-bit values
+            with jt.flag_scope(amp_reg=4 + 32):
+                got = {op: a.reduce(op, dims) for op in ("add", "maximum", "mean")}
+                assert all(v.dtype == dtype and v._op.kind == "reduce" for v in got.values())
+                jt.sync(list(got.values()))
+            want = {"add": O.reduce(exact, "add", dims), "maximum": O.reduce(exact, "maximum", dims),
+                    "mean": O.reduce(exact, "mean", dims)}
+            ulp = 2.0 ** -8 if dtype == "bfloat16" else 2.0 ** -11
+            assert np.array_equal(got["maximum"].float32().data, want["maximum"])          # exact
+            for op in ("add", "mean"):
+                g, w = got[op].float32().data, want[op]
+                assert np.all(np.abs(g - w) <= 2 * ulp * np.abs(w) + 1e-4), (shape, dims, dtype, op)
 
 
 # ---- reduce with an element-wise prologue -----------------------------------------------------------

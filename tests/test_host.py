@@ -223,6 +223,53 @@ def test_dtype_rules_of_the_front_end():
     assert i.int32() is i                                      # unary_op.cc:867-870 forwards
 
 
+def test_amp_reg_controls_dtype_inference():
+    """The mixed-precision register (nano_string.h:199-277, var.cc:65-71), with the cases the reference checks
+    in test/test_fp16.py:208-300: reduce keeps 16 bit only with keep_reduce, white-list ops only with
+    keep_white, prefer16 / prefer32 steer float results unless an operand is a scalar, array-like ops follow
+    with array_prefer, and conv2d builds its sum under amp_reg | 36 (nn.py:1250)."""
+    a = jt.array(np.ones((3, 4), np.float32)).float16()
+    assert jt.flags.amp_reg == 0
+    for reg in (0, 1, 2):
+        with jt.flag_scope(amp_reg=reg):
+            assert a.maximum(a).max().dtype == "float32"                  # reduce_dtype_infer
+            assert (a ** a).dtype == "float32"                            # white list
+    with jt.flag_scope(amp_reg=2 + 4):
+        assert a.sum().dtype == "float16" and a.max().dtype == "float16"  # test_fp16.py:248-252
+    with jt.flag_scope(amp_reg=4):
+        s = a.sum()
+        assert s.dtype == "float16" and s._op.kind == "unary"             # still cast -> reduce(float32) -> cast
+        assert a.max().dtype == "float16" and a.max()._op.kind == "reduce"
+    with jt.flag_scope(amp_reg=4 + 32):
+        s = a.sum()
+        assert s.dtype == "float16" and s._op.kind == "reduce" and s._op.amp == 36
+    with jt.flag_scope(amp_reg=2 + 8):
+        assert (a ** a).dtype == "float16" and a.exp().dtype == "float16"
+    with jt.flag_scope(amp_reg=1):
+        assert a.sqrt().dtype == "float32" and (a + a).dtype == "float32"
+        assert (a * 2.0).dtype == "float16"                               # a scalar operand does not count
+    f = jt.array(np.ones((3, 4), np.float32))
+    with jt.flag_scope(amp_reg=2):
+        assert (f + f).dtype == "float16" and f.sqrt().dtype == "float16"
+    assert jt.array([1.0, 2.0]).dtype == "float32"
+    with jt.flag_scope(amp_reg=2 + 16):
+        assert jt.array([1.0, 2.0]).dtype == "float16" and jt.array([1.0]).dtype == "float32"
+    with jt.flag_scope(amp_level=3):                                      # test_fp16.py:293-299
+        assert jt.flags.amp_reg == 12
+        assert a.sum().dtype == "float16" and a.mean().dtype == "float16"
+        assert a.log().dtype == "float16" and a.exp().dtype == "float16"
+    assert jt.flags.amp_reg == 0 and jt.flags.auto_mixed_precision_level == 0
+    # conv2d: 16-bit operands give a 16-bit sum without casts; the gradient inherits the register
+    x, w = jt.zeros([2, 3, 8, 8]).bfloat16(), jt.zeros([4, 3, 3, 3]).bfloat16()
+    y = jt.nn.conv2d(x, w, padding=1)
+    assert y.dtype == "bfloat16" and y._op.kind == "reduce" and y._op.amp & 36 == 36
+    gw = jt.grad(y.sum(), w)
+    assert gw.dtype == "bfloat16" and gw._op.kind == "reduce" and gw._op.reduce_mask == 0b0011001
+    assert jt.flags.amp_reg == 0
+    with pytest.raises(KeyError):
+        jt.flags["no_such_flag"] = 1
+
+
 def test_reindex_constructor_checks():
     x = jt.zeros([10, 10])
     with pytest.raises(ValueError):
