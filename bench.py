@@ -275,6 +275,30 @@ def wl_c5(L, lib, steps, warmup, with_cpu, out_dtype="float32"):
     return out
 
 
+def wl_c5_wgrad(L, lib, steps, warmup, with_cpu):
+    """The weight gradient of the C5 convolution (the backward-w pattern of the same group): not one of the
+    five configurations, run with --only C5wgrad."""
+    from jittor_amd.dtypes import f32_to_bf16_bits
+    xs, ws, ys = (64, 256, 56, 56), (256, 256, 3, 3), (64, 256, 56, 56)
+    flops = 236760072192
+    dev = Dev(L)
+    xb = f32_to_bf16_bits(np.random.default_rng(0).standard_normal(xs).astype(np.float32))
+    db = f32_to_bf16_bits(np.random.default_rng(2).standard_normal(ys).astype(np.float32))
+    p = L.ConvParams(1, 1, 1, 1, 1, 1)
+    calls = []
+    for s in range(2):
+        tx = L.tensor(dev.put(xb), "bfloat16", xs)
+        td = L.tensor(dev.put(db), "bfloat16", ys)
+        tw = L.tensor(dev.empty(int(np.prod(ws)) * 4), "float32", ws)
+        calls.append(lambda tx=tx, td=td, tw=tw: L.check(lib.mjt_conv2d_meta_wgrad(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p))))
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out = {"workload": "C5 weight gradient, x bf16 [64,256,56,56], dy bf16 [64,256,56,56] -> dw fp32 [256,256,3,3]",
+           "kernel": L.last_kernel(), "dtype": "bf16", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+           "roofline": roofline("mfma", flops, ms), "note": "a step = MFMA kernel over slices of images + reduce over the slices"}
+    dev.release()
+    return out
+
+
 def wl_copy(L, lib, steps, warmup, with_cpu):
     """The library's device copy kernel on 256 MiB: the known-size launch that
     calibrates the FETCH_SIZE / WRITE_SIZE counters (not part of the default run)."""
@@ -311,6 +335,7 @@ WORKLOADS = {
     "C4": wl_c4,
     "C5": wl_c5,
     "C5bf16out": lambda L, lib, steps, warmup, with_cpu: wl_c5(L, lib, steps, warmup, False, out_dtype="bfloat16"),
+    "C5wgrad": wl_c5_wgrad,
     "COPY": wl_copy,
 }
 DEFAULT = ["C1", "C2", "C3add", "C3max", "C4", "C5", "C5bf16out"]

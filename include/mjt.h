@@ -227,6 +227,19 @@ int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* 
 int mjt_conv2d_meta_grouped(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y,
                             const mjt_conv_params* p, int groups);
 
+/* Weight gradient of the same convolution (the pattern
+ * reindex(x) * broadcast(dy) -> reduce.add over (n, oh, ow) that jt.grad builds;
+ * opt/tuner/conv_tuner.cc:375-397 relays it to a backward-w library op,
+ * extern/cuda/cudnn/ops/cudnn_conv_backward_w_op.cc):
+ *   dw[k,c,r,s] = sum_{n,oh,ow} dy[n,k,oh,ow] * x[n,c,oh*sh-ph+r*dh,ow*sw-pw+s*dw]
+ * x [N,C,H,W] and dy [N,K,OH,OW] bfloat16, dw [K,C,R,S] float32 or bfloat16
+ * (float32 accumulation, rounded once).  One MFMA kernel plus a reduce over
+ * slices of images; shapes it does not cover (horizontal stride > 1, more
+ * than 9 taps, left padding > 1, K % 64 != 0, ...) return MJT_ERR_UNSUPPORTED
+ * and are the caller's to run through mjt_matmul or mjt_conv2d_meta. */
+int mjt_conv2d_meta_wgrad(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw,
+                          const mjt_conv_params* p);
+
 /* ---- matrix product ---------------------------------------------------
  * c[n,k] = op(a) * op(b) for 2-d float operands of one dtype, op = transpose
  * when the flag is set: the call the reference relays the pattern

@@ -21,6 +21,8 @@ void remember(const std::string& key, JitKernel* k) {
 }
 void* g_wpack = nullptr;
 size_t g_wpack_bytes = 0;
+void* g_wgrad_part = nullptr;      // per-slice partial weight gradients (its own buffer: the reduce that folds them uses the arena)
+size_t g_wgrad_bytes = 0;
 }  // namespace
 
 void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p, int64_t G) {
@@ -181,7 +183,102 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     jit_launch(k, (unsigned)blocks, 1, 256, 0, a);
 }
 
+// Weight gradient: dw[k,c,r,s] = sum_{n,oh,ow} dy[n,k,oh,ow] * x[n,c,oh*sh-ph+r*dh,ow*sw-pw+s*dw].
+void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw, const mjt_conv_params* p) {
+    require_init();
+    check_tensor(x, "conv wgrad x");
+    check_tensor(dy, "conv wgrad dy");
+    check_tensor(dw, "conv wgrad dw");
+    MJT_CHECK(p, "conv wgrad: null parameters");
+    MJT_CHECK(x->ndim == 4 && dy->ndim == 4 && dw->ndim == 4, "conv wgrad: x, dy and dw must have rank 4");
+    MJT_CHECK(p->stride_h >= 1 && p->stride_w >= 1 && p->dil_h >= 1 && p->dil_w >= 1 && p->pad_h >= 0 && p->pad_w >= 0,
+              "conv wgrad: bad stride / padding / dilation");
+    const int64_t N = x->shape[0], C = x->shape[1], H = x->shape[2], W = x->shape[3];
+    const int64_t K = dy->shape[1], OH = dy->shape[2], OW = dy->shape[3];
+    const int64_t R = dw->shape[2], S = dw->shape[3];
+    MJT_CHECK(dy->shape[0] == N, "conv wgrad: dy has " << dy->shape[0] << " images, x " << N);
+    MJT_CHECK(dw->shape[0] == K && dw->shape[1] == C, "conv wgrad: dw shape " << shape_str(dw) << " != [" << K << "," << C << ",R,S]");
+    MJT_CHECK(OH == (H + 2 * p->pad_h - p->dil_h * (R - 1) - 1) / p->stride_h + 1 &&
+                  OW == (W + 2 * p->pad_w - p->dil_w * (S - 1) - 1) / p->stride_w + 1,
+              "conv wgrad: dy shape " << shape_str(dy) << " does not follow from x " << shape_str(x) << " and the " << R << "x" << S
+                                      << " kernel");
+    if (numel(dw) == 0) return;
+    // what the MFMA kernel covers; anything else is for the caller's general path
+    const int64_t KG = K % 256 == 0 ? 4 : K % 128 == 0 ? 2 : 1;
+    const int64_t CTW = 8 / KG;
+    const bool ok = x->dtype == MJT_BFLOAT16 && dy->dtype == MJT_BFLOAT16 && (dw->dtype == MJT_FLOAT32 || dw->dtype == MJT_BFLOAT16) &&
+                    p->stride_w == 1 && p->pad_w <= 1 && K % 64 == 0 && C % (16 * CTW) == 0 && R * S <= 9 && OW % 8 == 0 &&
+                    W % 2 == 0 && N >= 1 && numel(x) * 2 < (int64_t(1) << 31) && numel(dy) * 2 < (int64_t(1) << 31) &&
+                    ((OW + 31) / 32) * S <= 64 && (uintptr_t)x->ptr % 4 == 0 && (uintptr_t)dy->ptr % 16 == 0 &&
+                    !getenv("MJT_NO_FASTPATH");
+    if (!ok)
+        MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: only bfloat16 operands with horizontal stride 1, left padding <= 1, at most 9 taps, "
+                                      "K % 64 == 0, C % " << 16 * CTW << " == 0, OW % 8 == 0 and tensors below 2 GB run on the MFMA kernel");
+    Context& c = ctx();
+    const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
+    const int64_t blocks_per_slice = (K / (64 * KG)) * (C / (16 * CTW));
+    // slices of whole images: enough workgroups for every compute unit, at most one image per slice
+    int64_t slices = (cus + blocks_per_slice - 1) / blocks_per_slice;
+    if (slices > N) slices = N;
+    if (slices < 1) slices = 1;
+    int64_t ips = (N + slices - 1) / slices;
+    if (const char* e = getenv("MJT_WGRAD_IPS"))             // images per slice, for experiments
+        if (atoi(e) >= 1) ips = atoi(e) < N ? atoi(e) : N;
+    slices = (N + ips - 1) / ips;
+
+    std::ostringstream key;
+    key << "wgrad|" << C << "|" << H << "|" << W << "|" << K << "|" << R << "|" << S << "|" << OH << "|" << OW << "|" << p->stride_h << "|"
+        << p->pad_h << "|" << p->pad_w << "|" << p->dil_h << "|" << p->dil_w << "|" << KG;
+    JitKernel* k = cached(key.str());
+    if (!k) {
+        std::ostringstream name;
+        name << "mjt_conv_wgrad_mfma_bf16_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s" << p->stride_h
+             << "x1_p" << p->pad_h << "x" << p->pad_w << "_d" << p->dil_h << "x" << p->dil_w;
+        std::ostringstream src;
+        src << "#define ENTRY " << name.str() << "\n#define C_ " << C << "\n#define H_ " << H << "\n#define W_ " << W << "\n#define K_ " << K
+            << "\n#define R_ " << R << "\n#define S_ " << S << "\n#define OH_ " << OH << "\n#define OW_ " << OW << "\n#define SH "
+            << p->stride_h << "\n#define PH " << p->pad_h << "\n#define PW " << p->pad_w << "\n#define DH " << p->dil_h << "\n#define DW "
+            << p->dil_w << "\n#define KG " << KG << "\n";
+        src << embedded_source("conv_wgrad_mfma.h") << "\n";
+        k = jit_get(src.str(), name.str());
+        remember(key.str(), k);
+    }
+    const size_t pbytes = (size_t)slices * (size_t)numel(dw) * 4;
+    if (!c.dry_run && pbytes > g_wgrad_bytes) {
+        if (g_wgrad_part) {
+            HIP_CHECK(hipStreamSynchronize(c.stream));
+            HIP_CHECK(hipFree(g_wgrad_part));
+            g_wgrad_part = nullptr;
+            g_wgrad_bytes = 0;
+        }
+        HIP_CHECK(hipMalloc(&g_wgrad_part, pbytes));
+        g_wgrad_bytes = pbytes;
+    }
+    void* part = c.dry_run ? (void*)(uintptr_t)0x1000 : g_wgrad_part;
+    std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(dy->ptr), bits_of_ptr(part), (uint64_t)N, (uint64_t)ips, 0};
+    jit_launch(k, (unsigned)((slices + 7) / 8 * 8 * blocks_per_slice), 1, 512, 0, a);
+    // fold the slices: [slices, K*C*R*S] summed over axis 0, rounded once if dw is bfloat16
+    mjt_tensor tp, td;
+    memset(&tp, 0, sizeof(tp));
+    memset(&td, 0, sizeof(td));
+    tp.ptr = part;
+    tp.dtype = MJT_FLOAT32;
+    tp.ndim = 2;
+    tp.shape[0] = slices;
+    tp.shape[1] = numel(dw);
+    td.ptr = dw->ptr;
+    td.dtype = dw->dtype;
+    td.ndim = 1;
+    td.shape[0] = numel(dw);
+    if (mjt_reduce(&tp, &td, MJT_OP_ADD, 0b01) != MJT_OK) MJT_FAIL(MJT_ERR_DEVICE, "conv wgrad: folding the partial sums failed: " << mjt_last_error());
+    set_last_kernel(k->name.c_str());
+}
+
 }  // namespace mjt
+
+extern "C" int mjt_conv2d_meta_wgrad(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw, const mjt_conv_params* p) {
+    return mjt::guarded([&] { mjt::conv_wgrad_impl(x, dy, dw, p); });
+}
 
 extern "C" int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p) {
     return mjt::guarded([&] { mjt::conv_impl(x, w, y, p, 1); });

@@ -18,7 +18,8 @@ from ._lib import MjtError
 from . import profiler as _profiler
 from .flags import flags
 
-stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0, "matmul_matches": 0}
+stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0, "matmul_matches": 0,
+         "wgrad_kernel": 0}
 
 
 class ConvUnit:
@@ -689,6 +690,17 @@ def _run_single(op):
         N, C, H, W = x.shape
         _, K, OH, OW = dy.shape
         R, S = out.shape[2], out.shape[3]
+        if x.dtype == "bfloat16" and flags["enable_conv_wgrad_kernel"]:
+            # the MFMA kernel; shapes it does not cover come back as unsupported and take the paths below
+            tx, td = _tensor_of(x), _tensor_of(dy)
+            tw = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+            p = _lib.ConvParams(sh, sw, ph, pw, dh, dw)
+            rc = lib.mjt_conv2d_meta_wgrad(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p))
+            if rc == 0:
+                stats["wgrad_kernel"] += 1
+                return
+            if rc != _lib.ERR_UNSUPPORTED:
+                _lib.check(rc)
         if not _matmul_ok:
             _matmul_ok.append(bool(lib.mjt_matmul_available()))
         if _matmul_ok[0] and flags["enable_matmul_match"]:

@@ -899,3 +899,20 @@ def conv_meta_grouped(x, w, groups, stride=1, padding=0, dilation=1):
     yy = binary(xx, ww, "multiply")
     return reindex_reduce(yy, "add", [N, K, oh, ow], ["i0", "i1*%d+i2" % (K // G), "i4", "i5"])
 
+
+def conv_meta_wgrad(x, dy, R, S, stride=1, padding=0, dilation=1):
+    """Gradient of conv_meta with respect to w for an output gradient dy, as jt.grad builds it from
+    the op rules: the sum's gradient is a broadcast of dy over (c, kh, kw) (ops/reduce_op.cc:339-362),
+    the product's is dy times the other factor, the broadcast's is a sum over its axes (n, oh, ow)
+    (ops/broadcast_to_op.cc:112-117).  x [N,C,H,W], dy [N,K,OH,OW] (float32 arrays or BF16); returns the
+    float32 accumulator dw [K,C,R,S]."""
+    xf = x.to_f32() if isinstance(x, BF16) else np.asarray(x, dtype=np.float32)
+    df = dy.to_f32() if isinstance(dy, BF16) else np.asarray(dy, dtype=np.float32)
+    N, C, H, W = xf.shape
+    _, K, oh, ow = df.shape
+    xx = reindex(xf, [N, K, C, oh, ow, R, S],
+                 ["i0", "i2", "i3*%d-%d+i5*%d" % (stride, padding, dilation),
+                  "i4*%d-%d+i6*%d" % (stride, padding, dilation)])
+    dd = broadcast_to(df, xx.shape, [2, 5, 6])
+    return reduce(binary(xx, dd, "multiply"), "add", [0, 3, 4])
+

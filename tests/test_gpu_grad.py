@@ -206,14 +206,15 @@ def test_grad_meta_conv(gpu, case):
                 stack.extend(v._history[1])
 
 
-def test_grad_meta_conv_bfloat16(gpu):
-    """The same three units for bfloat16 operands: the float32 casts that the 16-bit sum puts between dy and
-    the products (ops/reduce_op.cc:259-266) are looked through, the MFMA kernel runs forward and input
-    gradient, the weight gradient is a batched GEMM over shifted input planes; gradients keep the dtype of
-    their variable."""
+@pytest.mark.parametrize("xs,ws,wgrad_kernel", [((2, 64, 16, 16), (64, 64, 3, 3), 0), ((2, 128, 8, 16), (64, 128, 3, 3), 1)])
+def test_grad_meta_conv_bfloat16(gpu, xs, ws, wgrad_kernel):
+    """The same three units for bfloat16 operands (conv2d builds them under amp_reg | 36, so the sums keep
+    16 bit without casts): the MFMA kernel runs forward and input gradient; the weight gradient runs on its
+    own MFMA kernel where that applies (second case) and as a batched GEMM over shifted input planes
+    otherwise (first case: 64 input channels); gradients keep the dtype of their variable."""
     rng = np.random.default_rng(8)
-    x = rng.standard_normal((2, 64, 16, 16)).astype(np.float32)
-    w = (rng.standard_normal((64, 64, 3, 3)) * 0.05).astype(np.float32)
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal(ws) * 0.05).astype(np.float32)
     vx, vw = jt.array(x).bfloat16(), jt.array(w).bfloat16()
     jt.sync([vx, vw])
     xb = O.BF16(vx.raw()).to_f32()
@@ -222,9 +223,10 @@ def test_grad_meta_conv_bfloat16(gpu):
     r = (rng.integers(-2, 3, y.shape) * 0.5).astype(np.float32)            # exact in bfloat16
     gx, gw = jt.grad((y * jt.array(r).bfloat16()).sum(), [vx, vw])
     assert gx.dtype == "bfloat16" and gw.dtype == "bfloat16"
-    before = jt.executor_stats["conv_matches"]
+    before, before_k = jt.executor_stats["conv_matches"], jt.executor_stats["wgrad_kernel"]
     jt.sync([y, gx, gw])
     assert jt.executor_stats["conv_matches"] - before == 3
+    assert jt.executor_stats["wgrad_kernel"] - before_k == wgrad_kernel
     dX, dW = _conv_grads_ref(xb, wb, r, 1, 1, 1)
     tol = 2.0 ** -7                                                         # results are rounded to bfloat16
     assert np.abs(gx.float32().numpy() - dX).max() <= tol * np.abs(dX).max()

@@ -571,6 +571,71 @@ def test_conv_grouped_entry_and_front_end(gpu):
         jt.nn.conv2d(jt.array(x), jt.array(w), groups=4)
 
 
+def _wgrad_call(xbits, dybits, R, S, params, out_dtype="float32"):
+    x, dy = jt.from_storage(xbits, "bfloat16"), jt.from_storage(dybits, "bfloat16")
+    dw = jt.zeros([dybits.shape[1], xbits.shape[1], R, S], out_dtype)
+    tx, td = L.tensor(x.raw_ptr(), "bfloat16", x.shape), L.tensor(dy.raw_ptr(), "bfloat16", dy.shape)
+    tw = L.tensor(dw.raw_ptr(), out_dtype, dw.shape)
+    p = L.ConvParams(*params)
+    rc = L.load().mjt_conv2d_meta_wgrad(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p))
+    if rc != 0:
+        return rc, None
+    return 0, L.d2h(dw.raw_ptr(), dw.shape, L.NP_STORAGE[out_dtype])
+
+
+@pytest.mark.parametrize("case", [
+    dict(x=(2, 128, 6, 8), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),        # one partial chunk per row, rows in pairs
+    dict(x=(1, 128, 1, 8), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),        # a single row: the last fragments end at the tensor's end
+    dict(x=(3, 32, 7, 40), k=256, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),       # four channel groups; chunks of 32 + 8 columns; odd height
+    dict(x=(2, 64, 9, 18), k=128, rs=(3, 3), p=(1, 1, 1, 1, 2, 2)),       # dilation 2: every column shift odd
+    dict(x=(2, 128, 6, 10), k=64, rs=(3, 3), p=(1, 1, 0, 0, 1, 1)),       # no padding: shifts 0, 1, 2
+    dict(x=(2, 128, 4, 8), k=64, rs=(1, 1), p=(1, 1, 0, 0, 1, 1)),        # 1x1
+    dict(x=(2, 128, 9, 8), k=64, rs=(3, 3), p=(2, 1, 1, 1, 1, 1)),        # vertical stride 2
+    dict(x=(5, 128, 5, 72), k=64, rs=(2, 3), p=(1, 1, 0, 1, 1, 1), ips=2),   # three chunks (odd), 2x3 taps, two images per slice, the last slice one
+    dict(x=(2, 32, 6, 16), k=256, rs=(3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16"),
+])
+def test_conv_wgrad_mfma_matches_oracle(gpu, case, monkeypatch):
+    """The weight gradient kernel through the C entry point against the oracle's restatement of the
+    gradient graph (float32 accumulator; the kernel sums in another order: 1e-4 of the largest value)."""
+    rng = np.random.default_rng(31)
+    N, C, H, W = case["x"]
+    K, (R, S) = case["k"], case["rs"]
+    sh, sw, ph, pw, dh, dw_ = case["p"]
+    OH = (H + 2 * ph - dh * (R - 1) - 1) // sh + 1
+    OW = (W + 2 * pw - dw_ * (S - 1) - 1) // sw + 1
+    xb = _bf16(rng.standard_normal((N, C, H, W)))
+    db = _bf16(rng.standard_normal((N, K, OH, OW)))
+    out = case.get("out", "float32")
+    if "ips" in case:
+        monkeypatch.setenv("MJT_WGRAD_IPS", str(case["ips"]))
+    rc, got = _wgrad_call(xb, db, R, S, case["p"], out)
+    assert rc == 0 and L.last_kernel().startswith("mjt_conv_wgrad_mfma_bf16")
+    xf, df = O.BF16(xb).to_f32().astype(np.float64), O.BF16(db).to_f32().astype(np.float64)
+    xp = np.pad(xf, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+    want = np.zeros((K, C, R, S))
+    for r in range(R):
+        for s in range(S):
+            patch = xp[:, :, r * dh:r * dh + (OH - 1) * sh + 1:sh, s * dw_:s * dw_ + (OW - 1) * sw + 1:sw]
+            want[:, :, r, s] = np.einsum("nkhw,nchw->kc", df, patch)
+    if out == "bfloat16":
+        got = O.BF16(got).to_f32()
+        assert np.abs(got - want).max() <= 2.0 ** -7 * np.abs(want).max()
+    else:
+        assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+    if N * K * C * OH * OW * R * S <= 4e7 and sh == sw and ph == pw and dh == dw_:
+        ref = O.conv_meta_wgrad(O.BF16(xb), O.BF16(db), R, S, sh, ph, dh)     # the reference's own summation order
+        assert np.abs(got - ref).max() <= (1e-4 if out == "float32" else 2.0 ** -7) * np.abs(ref).max()
+
+
+def test_conv_wgrad_entry_rejects_what_the_kernel_does_not_cover(gpu):
+    rng = np.random.default_rng(32)
+    xb, db = _bf16(rng.standard_normal((1, 128, 9, 9))), _bf16(rng.standard_normal((1, 64, 5, 5)))
+    rc, _ = _wgrad_call(xb, db, 3, 3, (2, 2, 1, 1, 1, 1))                       # horizontal stride 2
+    assert rc == -2 and "stride" in L.load().mjt_last_error().decode()
+    rc, _ = _wgrad_call(xb, _bf16(rng.standard_normal((1, 64, 9, 8))), 3, 3, (1, 1, 1, 1, 1, 1))   # dy does not follow from x
+    assert rc == -1 and "does not follow" in L.load().mjt_last_error().decode()
+
+
 def test_conv_front_end_pattern_match(gpu):
     rng = np.random.default_rng(22)
     x = jt.array(rng.standard_normal((2, 64, 14, 16)).astype(np.float32)).bfloat16()

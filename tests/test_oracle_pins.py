@@ -306,6 +306,27 @@ def test_conv_meta_grouped_is_one_convolution_per_group(groups, stride, pad, dil
     assert np.allclose(one, O.conv_meta(x[:, :cg], w[:kg], stride, pad, dil), rtol=1e-6, atol=1e-6)
 
 
+def test_conv_meta_wgrad_against_finite_differences_of_the_forward():
+    """dw is linear in dy and the convolution is linear in w, so <conv(x, w), dy> = <w, dw> for every w
+    (a transposed or shifted tap, or a wrong reduced axis, breaks the identity), and dw equals the float64
+    correlation of dy with the shifted input planes."""
+    for stride, pad, dil in [(1, 1, 1), (2, 1, 1), (1, 2, 2), (1, 0, 1)]:
+        x = rng.standard_normal((2, 3, 9, 8)).astype(np.float32)
+        w = rng.standard_normal((4, 3, 3, 3)).astype(np.float32)
+        y = _conv_f64(x, w, stride, pad, dil)
+        dy = rng.standard_normal(y.shape).astype(np.float32)
+        dw = O.conv_meta_wgrad(x, dy, 3, 3, stride, pad, dil)
+        assert dw.shape == w.shape and dw.dtype == np.float32
+        assert np.isclose((y * dy).sum(), (w.astype(np.float64) * dw).sum(), rtol=1e-5)
+        xp = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+        oh, ow = dy.shape[2:]
+        for r in range(3):
+            for s_ in range(3):
+                patch = xp[:, :, r * dil:r * dil + (oh - 1) * stride + 1:stride, s_ * dil:s_ * dil + (ow - 1) * stride + 1:stride]
+                want = np.einsum("nkhw,nchw->kc", dy.astype(np.float64), patch)
+                assert np.allclose(dw[:, :, r, s_], want, rtol=1e-4, atol=1e-4)
+
+
 def test_conv_meta_one_hot_kernel_is_a_shift():
     x = O.BF16(O.f32_to_bf16_bits(rng.standard_normal((1, 2, 6, 6)).astype(np.float32)))
     w = np.zeros((2, 2, 3, 3), np.float32)
