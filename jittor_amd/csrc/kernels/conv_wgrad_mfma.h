@@ -18,14 +18,16 @@
 // R_*S_ of x, 4*R_*S_ MFMAs per wave.  In that lane order neighbouring lanes read different rows
 // (a cache line per lane), so a fragment is fetched in row order instead -- lane i takes 16 bytes of
 // row i / 4, piece i % 4, four neighbouring lanes one 64-byte run -- by a load that writes straight
-// into a wave-private 1 KB slot of LDS (no registers, no barrier), and read back from there in
-// fragment order.  A fragment of x whose column shift is odd starts in the middle of a dword: it
+// into a 1 KB slot of LDS (no registers), and read back from there in fragment order.  The slots of
+// a step are shared: the waves of one channel group read the same dy fragments, the waves of one
+// channel tile the same x fragments, so each is fetched once per workgroup (the loads are dealt
+// out to the 8 waves) and a barrier per step separates filling from reading.  A fragment of x whose column shift is odd starts in the middle of a dword: it
 // comes as the four dwords above its first element plus the dword below, shifted down by 16 bits
 // (every load is dword-aligned).  Columns outside the image (and the columns of a last, partial
-// chunk) are cleared with lane masks kept in LDS; rows and images outside read zeros through the
+// chunk) are cleared with lane masks; rows and images outside read zeros through the
 // range check of the buffer loads (the whole offset travels in the lane offset, which is what the
-// hardware checks).  While the MFMAs of a step run, the loads of the next step fill the slots the
-// step's fragments were just read from.
+// hardware checks).  While the MFMAs of a step run, the loads of the next step fill a second set
+// of slots (when two sets fit into LDS; otherwise the same set, after a second barrier).
 //
 // A workgroup owns 64*KG output channels x 16*8/KG input channels x all taps, over the images
 // [slice*ips, slice*ips+ips): the partial sums of the slices go to partial[slice][k][c][r][s]
@@ -50,12 +52,15 @@ template <int I, int N, class F> __device__ __forceinline__ void mjt_static_for(
     }
 }
 __device__ constexpr int mjt_col_shift(int s) { return s * DW - PW; }      // input column - output column of tap column s
+// does chunk ch with tap column s reach outside the row (of dy or of x)?
+__device__ constexpr bool mjt_edge(int ch, int s) {
+    return ch * 32 + mjt_col_shift(s) < 0 || ch * 32 + 31 + mjt_col_shift(s) >= W_ || ch * 32 + 31 >= OW_;
+}
 
 extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     const int n_img = (int)(unsigned long long)p.a[3];
     const int ips = (int)(unsigned long long)p.a[4];
     float* __restrict__ partial = (float*)p.a[2];
-    __shared__ mjt_u32x4v masks[NCHUNK * S_][64];
 
     constexpr int KBLOCKS = K_ / (64 * KG), CBLOCKS = C_ / (16 * CTW);
     // the workgroups of one slice read the same dy: they are 8 apart, so that they land on the same XCD
@@ -75,24 +80,26 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     const int k0 = (kblock * KG + kg) * 64, c0 = (cblock * CTW + ct) * 16;
     const int l16 = lane & 15, lg = lane >> 4;
 
-    // which of a lane's 8 elements lie inside the image, per (chunk, tap column): 16 bits per element pair
-    for (int idx = wave; idx < NCHUNK * S_; idx += 8) {
-        const int ch = idx / S_, s = idx - ch * S_;
-        const int off = s * DW - PW;
-        mjt_u32x4v m;
+    // Which of a lane's 8 elements lie inside the image, per (chunk, tap column): 16 bits per element pair.  Only the
+    // combinations that touch an edge of the row are ever applied (the first chunk with a negative shift, the last
+    // chunk), the others are never materialised.
+    mjt_u32x4v masks[NCHUNK * S_];
+    mjt_static_for<0, NCHUNK * S_>([&](auto ic) {
+        constexpr int idx = decltype(ic)::v, ch = idx / S_, s = idx % S_;
+        if constexpr (mjt_edge(ch, s)) {
+            constexpr int off = mjt_col_shift(s);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            unsigned v = 0;
+            for (int j = 0; j < 4; j++) {
+                unsigned v = 0;
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const int ow = ch * 32 + lg * 8 + 2 * j + h, iw = ow + off;
-                if (ow < OW_ && iw >= 0 && iw < W_) v |= h ? 0xffff0000u : 0x0000ffffu;
+                for (int h = 0; h < 2; h++) {
+                    const int ow = ch * 32 + lg * 8 + 2 * j + h, iw = ow + off;
+                    if (ow < OW_ && iw >= 0 && iw < W_) v |= h ? 0xffff0000u : 0x0000ffffu;
+                }
+                masks[idx][j] = v;
             }
-            m[j] = v;
         }
-        masks[idx][lane] = m;
-    }
-    __syncthreads();
+    });
 
     // buffer descriptors over the whole tensors; every offset is a lane offset, so the range check sees all of it
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.a[0], 0, n_img * (C_ * H_ * W_ * 2), 0x00020000);
@@ -101,11 +108,15 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     const int frow = lane >> 2, fpiece = lane & 3;
     const unsigned a_lane = (unsigned)((frow * OH_ * OW_ + fpiece * 8) * 2);
     const unsigned b_lane = (unsigned)((frow * H_ * W_ + fpiece * 8) * 2);
-    // a wave's slots: 4 fragments of dy, TAPS of x (1 KB each, lane i at byte 16 i), TAPS dwords-below (256 B each)
-    constexpr int SLOT_B = 4 * 1024, SLOT_X = SLOT_B + TAPS * 1024, WAVE_LDS = SLOT_X + TAPS * 256;
-    __shared__ __attribute__((aligned(16))) unsigned char stage[8 * WAVE_LDS];
+    // Staging area of a step, shared by the workgroup: 4 KG fragments of dy (its KG channel groups), CTW * TAPS of x
+    // (its CTW channel tiles; 1 KB each, lane i of the fetch at byte 16 i) and as many dwords-below (256 B each).
+    // Three of them when they fit (the loads of a step are then requested two steps ahead: memory latency under
+    // load is longer than one step), else two, else one.
+    constexpr int NA = 4 * KG, NB = CTW * TAPS;
+    constexpr int AREA_B = NA * 1024, AREA_X = AREA_B + NB * 1024, AREA = AREA_X + NB * 256;
+    constexpr int NBUF = 3 * AREA <= 150 * 1024 ? 3 : 2 * AREA <= 150 * 1024 ? 2 : 1;
+    __shared__ __attribute__((aligned(16))) unsigned char stage[NBUF * AREA];
     typedef __attribute__((address_space(3))) void* mjt_lds_ptr;
-    unsigned char* const mine = stage + wave * WAVE_LDS;
     // fragment order: lane (l16, lg) wants row l16, piece lg
     const int rd = (l16 * 4 + lg) * 16;
 
@@ -115,57 +126,88 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
 #pragma unroll
         for (int t = 0; t < TAPS; t++) acc[m][t] = (mjt_f32x4)(0.0f);
 
-    // bit 31 set in an offset puts it beyond every buffer (the tensors are smaller than 2 GB): the load delivers zeros
-    auto fetch = [&](int img, int oh, int ch) {
-        {
-            const bool ok = img < img_end && oh < OH_;
-            const unsigned base = ok ? (unsigned)((((img * K_ + k0) * OH_ + oh) * OW_ + ch * 32) * 2) : 0u;
-            const unsigned flag = (ok ? 0u : INVALID) | (ch * 32 + fpiece * 8 < OW_ ? 0u : INVALID);
+    // The loads of one step, dealt to the waves (item it to wave it % 8): NA fragments of dy, NB of x, NB dwords-below
+    // (only for odd column shifts).  Bit 31 set in an offset puts it beyond every buffer (the tensors are smaller than
+    // 2 GB): the load delivers zeros.
+    auto fetch = [&](unsigned char* area, int img, int oh, int ch) -> int {
+        int issued = 0;                                                  // by this wave
+        const bool img_ok = img < img_end && oh < OH_;
 #pragma unroll
-            for (int m = 0; m < 4; m++)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(y_rsrc, (mjt_lds_ptr)(mine + m * 1024), 16,
-                                                         (int)((a_lane + base + (unsigned)(m * 16 * OH_ * OW_ * 2)) | flag), 0, 0, 0);
-        }
-        mjt_static_for<0, R_>([&](auto rc) {
-            constexpr int r = decltype(rc)::v;
-            const int ih = oh * SH - PH + r * DH;
-            const bool ok = img < img_end && oh < OH_ && ih >= 0 && ih < H_;
-            const unsigned base = ok ? (unsigned)((((img * C_ + c0) * H_ + ih) * W_ + ch * 32) * 2) : 0u;
-            const unsigned flag = ok ? 0u : INVALID;
-            mjt_static_for<0, S_>([&](auto sc) {
-                constexpr int s = decltype(sc)::v;
-                constexpr int off = mjt_col_shift(s);                    // >= -1: the host admits no wider left padding
-                constexpr int t = r * S_ + s;
-                if constexpr (off & 1) {
-                    // elements off+1 .. off+8 as four dwords, and the dword below them (elements off-1, off); at the very
-                    // start of the tensor that dword lies in front of it: its offset wraps, out of range, zeros
-                    const unsigned o = b_lane + base + (unsigned)((off + 1) * 2);
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(mine + SLOT_B + t * 1024), 16, (int)(o | flag), 0, 0, 0);
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(mine + SLOT_X + t * 256), 4, (int)((o - 4u) | flag), 0, 0, 0);
-                } else {
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(mine + SLOT_B + t * 1024), 16,
-                                                             (int)((b_lane + base + (unsigned)(off * 2)) | flag), 0, 0, 0);
+        for (int it0 = 0; it0 < NA + 2 * NB; it0 += 8) {
+            const int it = it0 + wave;
+            if (it < NA) {
+                const int kk = (kblock * KG + it / 4) * 64 + (it & 3) * 16;
+                const unsigned base = img_ok ? (unsigned)((((img * K_ + kk) * OH_ + oh) * OW_ + ch * 32) * 2) : 0u;
+                const unsigned flag = (img_ok ? 0u : INVALID) | (ch * 32 + fpiece * 8 < OW_ ? 0u : INVALID);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(y_rsrc, (mjt_lds_ptr)(area + it * 1024), 16, (int)((a_lane + base) | flag), 0, 0, 0);
+                issued++;
+            } else if (it < NA + 2 * NB) {
+                const bool below = it >= NA + NB;
+                const int j = it - NA - (below ? NB : 0);
+                const int tile = j / TAPS, t = j - tile * TAPS;
+                const int r = t / S_, sx = t - r * S_;
+                const int off = sx * DW - PW;                            // >= -1: the host admits no wider left padding
+                const int ih = oh * SH - PH + r * DH;
+                const bool ok = img_ok && ih >= 0 && ih < H_;
+                const int cc = (cblock * CTW + tile) * 16;
+                const unsigned base = ok ? (unsigned)((((img * C_ + cc) * H_ + ih) * W_ + ch * 32) * 2) : 0u;
+                const unsigned flag = ok ? 0u : INVALID;
+                // an odd shift: elements off+1 .. off+8 as four dwords, and the dword below them (elements off-1, off); at
+                // the very start of the tensor that dword lies in front of it: its offset wraps, out of range, zeros
+                const unsigned o = b_lane + base + (unsigned)((off + (off & 1)) * 2);
+                if (!below) {
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + AREA_B + j * 1024), 16, (int)(o | flag), 0, 0, 0);
+                    issued++;
+                } else if (off & 1) {
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + AREA_X + j * 256), 4, (int)((o - 4u) | flag), 0, 0, 0);
+                    issued++;
                 }
-            });
-        });
+            }
+        }
+        return issued;
+    };
+    // wait until at most n of this wave's loads are outstanding (they complete in order)
+    auto wait_loads = [&](int n) {
+        switch (n) {
+        case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+        case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+        case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+        case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+        case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+        case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        }
     };
 
-    // One step: read the fragments of (img, oh, CH) that the loads have put into the slots, request those of the
-    // next step into the same slots, and run the MFMAs.
+    // One step: the fragments of (img, oh, CH) are in area `cur` once every wave's loads have arrived; request those of
+    // the step NBUF - 1 ahead (nimg, noh, nch) into the area that was read last (with a single area: into the same,
+    // after everybody has read it), run the MFMAs.
+    int cur = 0, newest = 0;                                             // newest: loads of this wave's latest request
     auto step = [&](auto ch_c, const int nimg, const int noh, const int nch) {
         constexpr int CH = decltype(ch_c)::v;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 // the slots are filled
+        unsigned char* const area = stage + cur * AREA;
+        wait_loads(NBUF == 3 ? newest : 0);                              // this wave's loads for this step have arrived
+        __syncthreads();                                                 // ... everybody's; and the area read last is free
+        if constexpr (NBUF >= 2) newest = fetch(stage + (cur == 0 ? NBUF - 1 : cur - 1) * AREA, nimg, noh, nch);
         mjt_u32x4v afrag[4], bq[TAPS];
         unsigned bx[TAPS];
+        const unsigned char* const my_a = area + kg * 4096 + rd;
+        const unsigned char* const my_b = area + AREA_B + ct * (TAPS * 1024) + rd;
+        const unsigned char* const my_x = area + AREA_X + ct * (TAPS * 256) + (rd >> 2);
 #pragma unroll
-        for (int m = 0; m < 4; m++) afrag[m] = *(const mjt_u32x4v*)(mine + m * 1024 + rd);
+        for (int m = 0; m < 4; m++) afrag[m] = *(const mjt_u32x4v*)(my_a + m * 1024);
         mjt_static_for<0, TAPS>([&](auto tc) {
             constexpr int t = decltype(tc)::v;
-            bq[t] = *(const mjt_u32x4v*)(mine + SLOT_B + t * 1024 + rd);
-            if constexpr (mjt_col_shift(t % S_) & 1) bx[t] = *(const unsigned*)(mine + SLOT_X + t * 256 + (rd >> 2));
+            bq[t] = *(const mjt_u32x4v*)(my_b + t * 1024);
+            if constexpr (mjt_col_shift(t % S_) & 1) bx[t] = *(const unsigned*)(my_x + t * 256);
         });
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");               // ... and read: they may be overwritten
-        fetch(nimg, noh, nch);
+        if constexpr (NBUF == 1) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");           // read by this wave
+            __syncthreads();                                             // ... by everybody: the area may be refilled
+            fetch(area, nimg, noh, nch);
+        }
         mjt_static_for<0, TAPS>([&](auto tc) {
             constexpr int t = decltype(tc)::v;
             constexpr int s = t % S_;
@@ -177,28 +219,41 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
                 v[2] = __builtin_amdgcn_alignbit(d[2], d[1], 16);
                 v[3] = __builtin_amdgcn_alignbit(d[3], d[2], 16);
             }
-            v &= masks[CH * S_ + s][lane];
+            if constexpr (mjt_edge(CH, s)) v &= masks[CH * S_ + s];
             const mjt_bf16x8 b = __builtin_bit_cast(mjt_bf16x8, v);
 #pragma unroll
             for (int m = 0; m < 4; m++)
                 acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mjt_bf16x8, afrag[m]), b, acc[m][t], 0, 0, 0);
         });
+        if constexpr (NBUF >= 2) cur = cur + 1 == NBUF ? 0 : cur + 1;
     };
 
-    // steps in order: images of the slice, rows, chunks
-    fetch(img_begin, 0, 0);
+    // steps in order: images of the slice, rows, chunks; (img, oh, ch) advanced by `ahead` steps
+    constexpr int AHEAD = NBUF == 1 ? 1 : NBUF - 1;
+    auto advance = [&](int& img, int& oh, int& ch, int ahead) {
+        ch += ahead;
+        while (ch >= NCHUNK) {
+            ch -= NCHUNK;
+            if (++oh >= OH_) { oh = 0; img++; }
+        }
+    };
+    fetch(stage, img_begin, 0, 0);
+    if constexpr (NBUF == 3) {
+        int i1 = img_begin, o1 = 0, c1 = 0;
+        advance(i1, o1, c1, 1);
+        newest = fetch(stage + AREA, i1, o1, c1);
+    }
     for (int img = img_begin; img < img_end; img++) {
 #pragma unroll 1
         for (int oh = 0; oh < OH_; oh++) {
-            const bool wrap = oh + 1 >= OH_;
-            const int after_img = wrap ? img + 1 : img, after_oh = wrap ? 0 : oh + 1;
             mjt_static_for<0, NCHUNK>([&](auto cc) {
-                constexpr int ch = decltype(cc)::v;
-                constexpr bool last = ch + 1 == NCHUNK;
-                step(cc, last ? after_img : img, last ? after_oh : oh, last ? 0 : ch + 1);
+                int ni = img, no = oh, nc = decltype(cc)::v;
+                advance(ni, no, nc, AHEAD);                              // beyond the slice: img_end, read as zeros
+                step(cc, ni, no, nc);
             });
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                     // nothing may arrive in LDS after the wave has ended
 
     // lane holds D[k = 4*lg + i][c = l16] of each (channel tile m, tap)
     const size_t KC = (size_t)K_ * C_;
