@@ -33,7 +33,7 @@
 //     before the MFMAs of the current one and written to the other buffer after
 //     them (one barrier per channel block);
 //   * A fragments come straight from the re-packed weights
-//     Wp[tap][c/64][k-step][ko][32 c] (1 KB contiguous per fragment, L2
+//     Wp[tap][c/64][k-step][ko/16][lane][8 c] (1 KB per fragment in lane order, L2
 //     resident) and are loaded one step before the MFMAs that use them.
 // Padding columns are zeroed once; rows outside the image are written as zeros.
 
@@ -198,8 +198,10 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
         }
     };
 
-    // A fragments: Wp[step][ko][32 c], step = (tap * NCB + cb) * 2 + ks; 16 rows x 64 B per fragment
-    const unsigned a_lane_off = (unsigned)(((wko * (16 * MT) + l16) * 32 + lg * 8) * 2);   // bytes
+    // A fragments: Wp[step][ko / 16][lane][8 c], step = (tap * NCB + cb) * 2 + ks: a fragment is 1 KB in lane order
+    // (lane = lg * 16 + l16 holds channels lg*8.. of row l16), so that a wave's load is one linear run of 8 cache
+    // lines; in [ko][32 c] order the 16 lanes the address unit takes together would touch 8 lines each time
+    const unsigned a_lane_off = (unsigned)(wko * MT * 1024 + lane * 16);   // bytes
     const __amdgpu_buffer_rsrc_t w_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(wp + (size_t)kpart * KO_WG * 32), 0, (R_ * S_ * C_ * K_ - kpart * KO_WG * 32) * 2, 0x00020000);
     auto load_a = [&](mjt_bf16x8 (&a)[MT], int cb, int s) {
@@ -364,15 +366,16 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
 #endif
 }
 
-// Weight re-pack: w[ko][c][kh][kw] -> Wp[tap][c/64][k-step][ko][32 c]
+// Weight re-pack: w[ko][c][kh][kw] -> Wp[tap][c/64][k-step][ko/16][lg][l16][8 c] (c = 32 k-step + 8 lg + ..)
 extern "C" __global__ __launch_bounds__(256) void ENTRY_PACK(Params p) {
     const unsigned short* __restrict__ w = (const unsigned short*)p.a[0];
     unsigned short* __restrict__ wp = (unsigned short*)p.a[1];
     const int total = K_ * C_ * R_ * S_;
     for (int o = blockIdx.x * 256 + threadIdx.x; o < total; o += gridDim.x * 256) {
-        int c32 = o & 31;
-        int rest = o >> 5;
-        int ko = rest % K_; rest /= K_;
+        int c8 = o & 7, l16 = (o >> 3) & 15, lg = (o >> 7) & 3;
+        int rest = o >> 9;
+        int ko = (rest % (K_ / 16)) * 16 + l16; rest /= K_ / 16;
+        int c32 = lg * 8 + c8;
         int ks = rest & 1; rest >>= 1;
         int cb = rest % NCB;
         int tap = rest / NCB;
