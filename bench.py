@@ -318,13 +318,13 @@ def wl_copy(L, lib, steps, warmup, with_cpu):
 # (FETCH_SIZE reads 131082 KiB for 262144 KiB fetched: factor 2.0; WRITE_SIZE reads 262144 KiB: factor 1.0).
 # Summaries: profiles/hbm_traffic_all_workloads.txt
 MEASURED_TRAFFIC = {
-    "C1": 2.0 * 65557.6 * 1024 + 64.0 * 1024,
-    "C2": 2.0 * 15636.0 * 1024 + 225834.9 * 1024,
-    "C3add": 2.0 * 65692.8 * 1024 + 41163.5 * 1024,
-    "C3max": 2.0 * 65695.2 * 1024 + 41701.9 * 1024,
-    "C4": 2.0 * 65583.9 * 1024 + 131072.0 * 1024,
-    "C5": 2.0 * 113421.8 * 1024 + 211875.7 * 1024,
-    "C5bf16out": 2.0 * 112180.0 * 1024 + 112985.8 * 1024,
+    "C1": 2.0 * 65557.8 * 1024 + 64.0 * 1024,
+    "C2": 2.0 * 15635.9 * 1024 + 225837.2 * 1024,
+    "C3add": 2.0 * 65692.9 * 1024 + 41115.1 * 1024,
+    "C3max": 2.0 * 65695.3 * 1024 + 41680.2 * 1024,
+    "C4": 2.0 * 65583.5 * 1024 + 131072.1 * 1024,
+    "C5": 2.0 * 113356.3 * 1024 + 212386.9 * 1024,
+    "C5bf16out": 2.0 * 112129.9 * 1024 + 112603.7 * 1024,
 }
 
 WORKLOADS = {
