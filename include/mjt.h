@@ -235,7 +235,7 @@ int mjt_conv2d_meta_grouped(const mjt_tensor* x, const mjt_tensor* w, const mjt_
  * x [N,C,H,W] and dy [N,K,OH,OW] bfloat16, dw [K,C,R,S] float32 or bfloat16
  * (float32 accumulation, rounded once).  One MFMA kernel plus a reduce over
  * slices of images; shapes it does not cover (horizontal stride > 1, more
- * than 9 taps, left padding > 1, K % 64 != 0, ...) return MJT_ERR_UNSUPPORTED
+ * than 9 taps, left padding > 2, K % 64 != 0, ...) return MJT_ERR_UNSUPPORTED
  * and are the caller's to run through mjt_matmul or mjt_conv2d_meta. */
 int mjt_conv2d_meta_wgrad(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw,
                           const mjt_conv_params* p);

@@ -108,14 +108,19 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     const int frow = lane >> 2, fpiece = lane & 3;
     const unsigned a_lane = (unsigned)((frow * OH_ * OW_ + fpiece * 8) * 2);
     const unsigned b_lane = (unsigned)((frow * H_ * W_ + fpiece * 8) * 2);
-    // Staging area of a step, shared by the workgroup: 4 KG fragments of dy (its KG channel groups), CTW * TAPS of x
-    // (its CTW channel tiles; 1 KB each, lane i of the fetch at byte 16 i) and as many dwords-below (256 B each).
-    // Three of them when they fit (the loads of a step are then requested two steps ahead: memory latency under
+    // Staging area of a step, shared by the workgroup: 4 KG fragments of dy (its KG channel groups; 1 KB each, lane i of
+    // the fetch at byte 16 i) and, for each of its CTW channel tiles and each tap row, the 32 columns of the chunk of that
+    // input row (1 KB, same order) plus the 4 columns after and the 2 before (16 B per channel: dwords right0, right1,
+    // left, unused), from which the fragments of all tap columns are cut.
+    // Three areas when they fit (the loads of a step are then requested two steps ahead: memory latency under
     // load is longer than one step), else two, else one.
-    constexpr int NA = 4 * KG, NB = CTW * TAPS;
+    constexpr int NA = 4 * KG, NB = CTW * R_;
     constexpr int AREA_B = NA * 1024, AREA_X = AREA_B + NB * 1024, AREA = AREA_X + NB * 256;
-    constexpr int NBUF = 3 * AREA <= 150 * 1024 ? 3 : 2 * AREA <= 150 * 1024 ? 2 : 1;
-    __shared__ __attribute__((aligned(16))) unsigned char stage[NBUF * AREA];
+    // A unit is what lies between two barriers: a whole row of chunks when three units of that size fit, else a chunk.
+    constexpr int UNIT = NCHUNK <= 2 && 3 * NCHUNK * AREA <= 150 * 1024 ? NCHUNK : 1;
+    constexpr int UAREA = UNIT * AREA;
+    constexpr int NBUF = 3 * UAREA <= 150 * 1024 ? 3 : 2 * UAREA <= 150 * 1024 ? 2 : 1;
+    __shared__ __attribute__((aligned(16))) unsigned char stage[NBUF * UAREA];
     typedef __attribute__((address_space(3))) void* mjt_lds_ptr;
     // fragment order: lane (l16, lg) wants row l16, piece lg
     const int rd = (l16 * 4 + lg) * 16;
@@ -126,9 +131,12 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
 #pragma unroll
         for (int t = 0; t < TAPS; t++) acc[m][t] = (mjt_f32x4)(0.0f);
 
-    // The loads of one step, dealt to the waves (item it to wave it % 8): NA fragments of dy, NB of x, NB dwords-below
-    // (only for odd column shifts).  Bit 31 set in an offset puts it beyond every buffer (the tensors are smaller than
-    // 2 GB): the load delivers zeros.
+    // The loads of one step, dealt to the waves (item it to wave it % 8): NA fragments of dy, NB row chunks of x, NB
+    // sets of edge dwords.  Bit 31 set in an offset puts it beyond every buffer (the tensors are smaller than 2 GB): the
+    // load delivers zeros.
+    // edge dwords: lane i fetches for channel i / 4 one of the two dwords right of the chunk (i % 4 = 0, 1) or the dword
+    // left of it (i % 4 = 2); 16 B per channel: right0, right1, left, unused
+    const unsigned e_lane = (unsigned)(frow * H_ * W_ * 2) + (fpiece == 2 ? (unsigned)-4 : (unsigned)(64 + 4 * fpiece));
     auto fetch = [&](unsigned char* area, int img, int oh, int ch) -> int {
         int issued = 0;                                                  // by this wave
         const bool img_ok = img < img_end && oh < OH_;
@@ -142,26 +150,22 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(y_rsrc, (mjt_lds_ptr)(area + it * 1024), 16, (int)((a_lane + base) | flag), 0, 0, 0);
                 issued++;
             } else if (it < NA + 2 * NB) {
-                const bool below = it >= NA + NB;
-                const int j = it - NA - (below ? NB : 0);
-                const int tile = j / TAPS, t = j - tile * TAPS;
-                const int r = t / S_, sx = t - r * S_;
-                const int off = sx * DW - PW;                            // >= -1: the host admits no wider left padding
+                const bool edge = it >= NA + NB;
+                const int j = it - NA - (edge ? NB : 0);
+                const int tile = j / R_, r = j - tile * R_;
                 const int ih = oh * SH - PH + r * DH;
                 const bool ok = img_ok && ih >= 0 && ih < H_;
                 const int cc = (cblock * CTW + tile) * 16;
                 const unsigned base = ok ? (unsigned)((((img * C_ + cc) * H_ + ih) * W_ + ch * 32) * 2) : 0u;
-                const unsigned flag = ok ? 0u : INVALID;
-                // an odd shift: elements off+1 .. off+8 as four dwords, and the dword below them (elements off-1, off); at
-                // the very start of the tensor that dword lies in front of it: its offset wraps, out of range, zeros
-                const unsigned o = b_lane + base + (unsigned)((off + (off & 1)) * 2);
-                if (!below) {
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + AREA_B + j * 1024), 16, (int)(o | flag), 0, 0, 0);
-                    issued++;
-                } else if (off & 1) {
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + AREA_X + j * 256), 4, (int)((o - 4u) | flag), 0, 0, 0);
-                    issued++;
+                if (!edge) {
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + AREA_B + j * 1024), 16,
+                                                             (int)((b_lane + base) | (ok ? 0u : INVALID)), 0, 0, 0);
+                } else {
+                    // at the very start of the tensor the left dword lies in front of it: its offset wraps, out of range, zeros
+                    const unsigned flag = (ok ? 0u : INVALID) | (fpiece == 3 ? INVALID : 0u);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + AREA_X + j * 256), 4, (int)((e_lane + base) | flag), 0, 0, 0);
                 }
+                issued++;
             }
         }
         return issued;
@@ -177,31 +181,54 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
         case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
         case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
         case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
+        case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+        case 11: asm volatile("s_waitcnt vmcnt(11)" ::: "memory"); break;
+        case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+        case 13: asm volatile("s_waitcnt vmcnt(13)" ::: "memory"); break;
+        case 14: asm volatile("s_waitcnt vmcnt(14)" ::: "memory"); break;
         default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
         }
     };
 
-    // One step: the fragments of (img, oh, CH) are in area `cur` once every wave's loads have arrived; request those of
-    // the step NBUF - 1 ahead (nimg, noh, nch) into the area that was read last (with a single area: into the same,
-    // after everybody has read it), run the MFMAs.
+    // the loads of a unit: its chunks ch0 .. ch0 + UNIT - 1 of row (img, oh), one area each
+    auto fetch_unit = [&](unsigned char* uarea, int img, int oh, int ch0) -> int {
+        int issued = 0;
+#pragma unroll
+        for (int u = 0; u < UNIT; u++) issued += fetch(uarea + u * AREA, img, oh, ch0 + u);
+        return issued;
+    };
+    // One unit: its fragments are in unit area `cur` once every wave's loads have arrived; request those of the unit
+    // NBUF - 1 ahead (nimg, noh, nch) into the area that was read last (with a single area: into the same, after
+    // everybody has read it), run the MFMAs chunk by chunk.
     int cur = 0, newest = 0;                                             // newest: loads of this wave's latest request
-    auto step = [&](auto ch_c, const int nimg, const int noh, const int nch) {
-        constexpr int CH = decltype(ch_c)::v;
-        unsigned char* const area = stage + cur * AREA;
-        wait_loads(NBUF == 3 ? newest : 0);                              // this wave's loads for this step have arrived
+    auto unit = [&](auto ch_c, const int nimg, const int noh, const int nch) {
+        constexpr int CH0 = decltype(ch_c)::v;
+        unsigned char* const uarea = stage + cur * UAREA;
+        wait_loads(NBUF == 3 ? newest : 0);                              // this wave's loads for this unit have arrived
         __syncthreads();                                                 // ... everybody's; and the area read last is free
-        if constexpr (NBUF >= 2) newest = fetch(stage + (cur == 0 ? NBUF - 1 : cur - 1) * AREA, nimg, noh, nch);
-        mjt_u32x4v afrag[4], bq[TAPS];
-        unsigned bx[TAPS];
+        if constexpr (NBUF >= 2) newest = fetch_unit(stage + (cur == 0 ? NBUF - 1 : cur - 1) * UAREA, nimg, noh, nch);
+        mjt_static_for<0, UNIT>([&](auto uc) {
+        constexpr int CH = CH0 + decltype(uc)::v;
+        unsigned char* const area = uarea + decltype(uc)::v * AREA;
+        mjt_u32x4v afrag[4], bd[R_];                                     // per tap row: columns 8 lg .. 8 lg + 7 of the chunk
+        unsigned bp[R_];                                                 // ... the two columns before them
+        unsigned long long bn[R_];                                       // ... the four after them
         const unsigned char* const my_a = area + kg * 4096 + rd;
-        const unsigned char* const my_b = area + AREA_B + ct * (TAPS * 1024) + rd;
-        const unsigned char* const my_x = area + AREA_X + ct * (TAPS * 256) + (rd >> 2);
+        const unsigned char* const my_b = area + AREA_B + ct * (R_ * 1024);
+        const unsigned char* const my_x = area + AREA_X + ct * (R_ * 256);
+        // a lane's neighbours are in the previous / next piece of the row, or among the edge dwords (pieces of the rows of
+        // a tile are 1 KB apart per tap row, their edge dwords 256 B)
+        const unsigned char* const prev0 = lg > 0 ? my_b + rd - 4 : my_x + l16 * 16 + 8;
+        const unsigned char* const next0 = lg < 3 ? my_b + rd + 16 : my_x + l16 * 16;
+        const int prev_step = lg > 0 ? 1024 : 256, next_step = lg < 3 ? 1024 : 256;
 #pragma unroll
         for (int m = 0; m < 4; m++) afrag[m] = *(const mjt_u32x4v*)(my_a + m * 1024);
-        mjt_static_for<0, TAPS>([&](auto tc) {
-            constexpr int t = decltype(tc)::v;
-            bq[t] = *(const mjt_u32x4v*)(my_b + t * 1024);
-            if constexpr (mjt_col_shift(t % S_) & 1) bx[t] = *(const unsigned*)(my_x + t * 256);
+        mjt_static_for<0, R_>([&](auto rc) {
+            constexpr int r = decltype(rc)::v;
+            bd[r] = *(const mjt_u32x4v*)(my_b + r * 1024 + rd);
+            bp[r] = *(const unsigned*)(prev0 + r * prev_step);
+            bn[r] = *(const unsigned long long*)(next0 + r * next_step);
         });
         if constexpr (NBUF == 1) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");           // read by this wave
@@ -210,14 +237,18 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
         }
         mjt_static_for<0, TAPS>([&](auto tc) {
             constexpr int t = decltype(tc)::v;
-            constexpr int s = t % S_;
-            mjt_u32x4v v = bq[t];
-            if constexpr (mjt_col_shift(s) & 1) {                        // (below, d0, d1, d2, d3) shifted down by one element
-                const mjt_u32x4v d = v;
-                v[0] = __builtin_amdgcn_alignbit(d[0], bx[t], 16);
-                v[1] = __builtin_amdgcn_alignbit(d[1], d[0], 16);
-                v[2] = __builtin_amdgcn_alignbit(d[2], d[1], 16);
-                v[3] = __builtin_amdgcn_alignbit(d[3], d[2], 16);
+            constexpr int r = t / S_, s = t % S_;
+            constexpr int off = mjt_col_shift(s);                        // -2 .. 4: the host admits nothing else
+            // the seven dwords around the lane's columns: elements 8 lg - 2 .. 8 lg + 11
+            const unsigned w[7] = {bp[r], bd[r][0], bd[r][1], bd[r][2], bd[r][3], (unsigned)bn[r], (unsigned)(bn[r] >> 32)};
+            constexpr int first = (off + 2) >> 1;                        // dword of element 8 lg + off
+            mjt_u32x4v v;
+            if constexpr (off & 1) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] = __builtin_amdgcn_alignbit(w[first + j + 1], w[first + j], 16);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] = w[first + j];
             }
             if constexpr (mjt_edge(CH, s)) v &= masks[CH * S_ + s];
             const mjt_bf16x8 b = __builtin_bit_cast(mjt_bf16x8, v);
@@ -225,31 +256,33 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
             for (int m = 0; m < 4; m++)
                 acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mjt_bf16x8, afrag[m]), b, acc[m][t], 0, 0, 0);
         });
+        });
         if constexpr (NBUF >= 2) cur = cur + 1 == NBUF ? 0 : cur + 1;
     };
 
-    // steps in order: images of the slice, rows, chunks; (img, oh, ch) advanced by `ahead` steps
+    // units in order: images of the slice, rows, chunks; (img, oh, ch) advanced by `ahead` units
     constexpr int AHEAD = NBUF == 1 ? 1 : NBUF - 1;
     auto advance = [&](int& img, int& oh, int& ch, int ahead) {
-        ch += ahead;
+        ch += ahead * UNIT;
         while (ch >= NCHUNK) {
             ch -= NCHUNK;
             if (++oh >= OH_) { oh = 0; img++; }
         }
     };
-    fetch(stage, img_begin, 0, 0);
+    fetch_unit(stage, img_begin, 0, 0);
     if constexpr (NBUF == 3) {
         int i1 = img_begin, o1 = 0, c1 = 0;
         advance(i1, o1, c1, 1);
-        newest = fetch(stage + AREA, i1, o1, c1);
+        newest = fetch_unit(stage + UAREA, i1, o1, c1);
     }
     for (int img = img_begin; img < img_end; img++) {
 #pragma unroll 1
         for (int oh = 0; oh < OH_; oh++) {
-            mjt_static_for<0, NCHUNK>([&](auto cc) {
-                int ni = img, no = oh, nc = decltype(cc)::v;
+            mjt_static_for<0, NCHUNK / UNIT>([&](auto cc) {
+                constexpr int ch0 = decltype(cc)::v * UNIT;
+                int ni = img, no = oh, nc = ch0;
                 advance(ni, no, nc, AHEAD);                              // beyond the slice: img_end, read as zeros
-                step(cc, ni, no, nc);
+                unit(mjt_ic<ch0>(), ni, no, nc);
             });
         }
     }

@@ -207,12 +207,12 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
     const int64_t KG = K % 256 == 0 ? 4 : K % 128 == 0 ? 2 : 1;
     const int64_t CTW = 8 / KG;
     const bool ok = x->dtype == MJT_BFLOAT16 && dy->dtype == MJT_BFLOAT16 && (dw->dtype == MJT_FLOAT32 || dw->dtype == MJT_BFLOAT16) &&
-                    p->stride_w == 1 && p->pad_w <= 1 && K % 64 == 0 && C % (16 * CTW) == 0 && R * S <= 9 && OW % 8 == 0 &&
+                    p->stride_w == 1 && p->pad_w <= 2 && (S - 1) * p->dil_w - p->pad_w <= 4 && K % 64 == 0 && C % (16 * CTW) == 0 && R * S <= 9 && OW % 8 == 0 &&
                     W % 2 == 0 && N >= 1 && numel(x) * 2 < (int64_t(1) << 31) && numel(dy) * 2 < (int64_t(1) << 31) &&
-                    ((OW + 31) / 32) * S <= 64 && (uintptr_t)x->ptr % 4 == 0 && (uintptr_t)dy->ptr % 16 == 0 &&
+                    (uintptr_t)x->ptr % 4 == 0 && (uintptr_t)dy->ptr % 16 == 0 &&
                     !getenv("MJT_NO_FASTPATH");
     if (!ok)
-        MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: only bfloat16 operands with horizontal stride 1, left padding <= 1, at most 9 taps, "
+        MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: only bfloat16 operands with horizontal stride 1, column shifts of the taps within -2 .. 4, at most 9 taps, "
                                       "K % 64 == 0, C % " << 16 * CTW << " == 0, OW % 8 == 0 and tensors below 2 GB run on the MFMA kernel");
     Context& c = ctx();
     const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;

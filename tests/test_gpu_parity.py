@@ -592,6 +592,9 @@ def _wgrad_call(xbits, dybits, R, S, params, out_dtype="float32"):
     dict(x=(2, 128, 4, 8), k=64, rs=(1, 1), p=(1, 1, 0, 0, 1, 1)),        # 1x1
     dict(x=(2, 128, 9, 8), k=64, rs=(3, 3), p=(2, 1, 1, 1, 1, 1)),        # vertical stride 2
     dict(x=(5, 128, 5, 72), k=64, rs=(2, 3), p=(1, 1, 0, 1, 1, 1), ips=2),   # three chunks (odd), 2x3 taps, two images per slice, the last slice one
+    dict(x=(2, 128, 5, 16), k=64, rs=(1, 5), p=(1, 1, 0, 2, 1, 1)),       # 1x5 taps, padding 2: shifts -2 .. 2
+    dict(x=(2, 128, 8, 16), k=64, rs=(3, 3), p=(1, 1, 2, 2, 2, 2)),       # dilation 2, padding 2: shifts -2, 0, 2
+    dict(x=(2, 128, 6, 12), k=64, rs=(2, 3), p=(1, 1, 0, 0, 1, 2)),       # horizontal dilation 2, no padding: shifts 0, 2, 4
     dict(x=(2, 32, 6, 16), k=256, rs=(3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16"),
 ])
 def test_conv_wgrad_mfma_matches_oracle(gpu, case, monkeypatch):
