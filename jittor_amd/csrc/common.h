@@ -68,6 +68,9 @@ Context& ctx();
 void require_init();
 void require_device();
 void* scratch(size_t bytes);      // grows the scratch arena when needed
+// mjt_shutdown runs these first, while the stream and the kernel modules still exist: whatever a file keeps
+// beyond a call (kernel look-up tables, device buffers, library handles) is dropped there
+void at_shutdown(void (*fn)());
 
 // ---- dtype helpers ---------------------------------------------------------
 int dtype_size(int dtype);

@@ -23,6 +23,19 @@ void* g_wpack = nullptr;
 size_t g_wpack_bytes = 0;
 void* g_wgrad_part = nullptr;      // per-slice partial weight gradients (its own buffer: the reduce that folds them uses the arena)
 size_t g_wgrad_bytes = 0;
+void forget() {
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (auto& kv : g_kernels)
+        if (kv.first.size() > 5 && kv.first.compare(kv.first.size() - 5, 5, "|pack") == 0) delete kv.second;   // shares its module with the main kernel
+    g_kernels.clear();                                  // the kernels themselves belong to the run-time compiler's cache
+    if (!ctx().dry_run) {
+        if (g_wpack) (void)hipFree(g_wpack);
+        if (g_wgrad_part) (void)hipFree(g_wgrad_part);
+    }
+    g_wpack = g_wgrad_part = nullptr;
+    g_wpack_bytes = g_wgrad_bytes = 0;
+}
+const bool g_registered = (at_shutdown(&forget), true);
 }  // namespace
 
 void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p, int64_t G) {

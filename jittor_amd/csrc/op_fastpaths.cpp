@@ -12,6 +12,11 @@ namespace mjt {
 namespace {
 std::mutex g_mu;
 std::unordered_map<std::string, JitKernel*> g_kernels;
+void forget() {   // the kernels belong to the run-time compiler's cache, which mjt_shutdown empties
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_kernels.clear();
+}
+const bool g_registered = (at_shutdown(&forget), true);
 
 JitKernel* cached(const std::string& key) {
     std::lock_guard<std::mutex> lock(g_mu);

@@ -11,6 +11,11 @@ namespace {
 
 std::mutex g_mu;
 std::unordered_map<std::string, JitKernel*> g_kernels;
+void forget() {   // the kernels belong to the run-time compiler's cache, which mjt_shutdown empties
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_kernels.clear();
+}
+const bool g_registered = (at_shutdown(&forget), true);
 
 bool is_unary_op(int op) { return op >= MJT_OP_ABS && op <= MJT_OP_SIGMOID; }
 bool is_binary_op(int op) { return op >= MJT_OP_POW && op <= MJT_OP_MEAN; }

@@ -94,10 +94,10 @@ void matmul_impl(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, 
     if (!blas_load()) MJT_FAIL(MJT_ERR_UNSUPPORTED, "matmul: rocBLAS is not available");
     {
         std::lock_guard<std::mutex> lock(g_mu);
-        if (!g_blas.handle) {
-            if (g_blas.create(&g_blas.handle) != rocblas_status_success) MJT_FAIL(MJT_ERR_DEVICE, "matmul: rocblas_create_handle failed");
-            if (g_blas.set_stream(g_blas.handle, ctxt.stream) != rocblas_status_success) MJT_FAIL(MJT_ERR_DEVICE, "matmul: rocblas_set_stream failed");
-        }
+        if (!g_blas.handle && g_blas.create(&g_blas.handle) != rocblas_status_success)
+            MJT_FAIL(MJT_ERR_DEVICE, "matmul: rocblas_create_handle failed");
+        // every call: the library's stream changes when it is shut down and bound again
+        if (g_blas.set_stream(g_blas.handle, ctxt.stream) != rocblas_status_success) MJT_FAIL(MJT_ERR_DEVICE, "matmul: rocblas_set_stream failed");
     }
     // Row-major c[n,k] = a * b is column-major c^T[k,n] = b^T * a^T: the operands trade places and keep
     // their own transposition flags (cublas_matmul_op.cc:118-126).

@@ -16,6 +16,11 @@ struct Axis {
 
 std::mutex g_mu;
 std::unordered_map<std::string, JitKernel*> g_kernels;
+void forget() {   // the kernels belong to the run-time compiler's cache, which mjt_shutdown empties
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_kernels.clear();
+}
+const bool g_registered = (at_shutdown(&forget), true);
 
 bool reducible(int op) {
     switch (op) {

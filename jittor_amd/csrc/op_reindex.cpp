@@ -31,6 +31,11 @@ struct Plan {
 
 std::mutex g_mu;
 std::unordered_map<std::string, std::unique_ptr<Plan>> g_plans;
+void forget() {   // plans hold kernels of the run-time compiler's cache, which mjt_shutdown empties
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_plans.clear();
+}
+const bool g_registered = (at_shutdown(&forget), true);
 
 std::string plan_key(bool scatter, int op, const mjt_tensor* x, const mjt_tensor* y, int n_idx, const char* const* idx,
                      int n_ofc, const char* const* ofc, int n_ex, const mjt_tensor* ex) {

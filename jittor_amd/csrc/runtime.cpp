@@ -38,6 +38,12 @@ void require_device() {
     if (g_ctx.dry_run) MJT_FAIL(MJT_ERR_NOT_INIT, "compile-only mode (mjt_init(-1)) has no device");
 }
 
+static std::vector<void (*)()>& shutdown_hooks() {
+    static std::vector<void (*)()> hooks;      // built on first use: registration runs during static initialisation
+    return hooks;
+}
+void at_shutdown(void (*fn)()) { shutdown_hooks().push_back(fn); }
+
 void* scratch(size_t bytes) {
     Context& c = ctx();
     if (c.dry_run) return (void*)(uintptr_t)0x1000;
@@ -268,6 +274,7 @@ void mjt_shutdown(void) {
     Context& c = ctx();
     if (!c.ready) return;
     if (!c.dry_run) (void)hipStreamSynchronize(c.stream);
+    for (auto fn : shutdown_hooks()) fn();
     {
         std::lock_guard<std::mutex> lock(g_jit_mutex);
         for (auto& kv : g_jit_cache) {

@@ -839,3 +839,22 @@ def test_fused_reduce_with_per_output_inputs(gpu):
     got = (jt.array(x) * jt.array(w)).sum(2).data
     assert jt.executor_stats["fused_reduces"] == before["fused_reduces"]
     assert np.allclose(got, (X * w).sum(2), rtol=1e-5, atol=1e-4)
+
+
+def test_zz_shutdown_and_rebind_on_the_device(gpu):
+    """mjt_shutdown followed by mjt_init: kernels, scratch buffers and the packed-weight buffer are rebuilt, results
+    stay the same (buffers the caller allocated survive: they are the caller's)."""
+    rng = np.random.default_rng(50)
+    x = rng.standard_normal((300, 257)).astype(np.float32)
+    xb, wb = _bf16(rng.standard_normal((2, 64, 16, 16))), _bf16(rng.standard_normal((128, 64, 3, 3)) * 0.1)
+    a = jt.array(x)
+    s1 = a.sum(1).data
+    y1, _ = _conv_call(xb, wb, (1, 1, 1, 1, 1, 1))
+    lib = L.load()
+    lib.mjt_shutdown()
+    L._device = None
+    L.init(0)
+    s2 = a.sum(1).data                                       # `a` was allocated before the shutdown
+    y2, kern = _conv_call(xb, wb, (1, 1, 1, 1, 1, 1))
+    assert kern.startswith("mjt_conv_mfma_bf16") and np.array_equal(s1, s2) and np.array_equal(y1, y2)
+    assert np.allclose(s2, x.sum(1), rtol=1e-5, atol=1e-4)

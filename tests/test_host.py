@@ -463,3 +463,34 @@ def test_matmul_entry_checks(compile_only):
     assert call(t("float32", [3, 4, 8]), t("float32", [3, 8, 5]), t("float32", [3, 4, 5])) == 0       # equal batch extents
     assert call(t("float32", [3, 4, 8]), t("float32", [2, 8, 5]), t("float32", [3, 4, 5])) == -1
     assert lib.mjt_matmul_available() in (0, 1)
+
+
+def test_shutdown_forgets_kernels_and_rebinding_compiles_again(compile_only, monkeypatch):
+    """mjt_shutdown unloads every kernel module; the per-op look-up tables must not keep pointers to them: the same
+    calls after binding again have to find (compile or load) their kernels anew."""
+    lib = L.load()
+    P = 0x100000
+    monkeypatch.setenv("MJT_NO_DISK_CACHE", "1")            # count real compilations
+    lib.mjt_shutdown()                                       # start from empty tables whatever ran before
+    L._device = None
+    L.init(-1)
+
+    def calls():
+        x, y = L.tensor(P, "float32", (64, 128)), L.tensor(P, "float32", (64,))
+        assert lib.mjt_reduce(ctypes.byref(x), ctypes.byref(y), L.OP_CODE["add"], 2) == 0
+        xb, w = L.tensor(P, "bfloat16", (2, 64, 16, 16)), L.tensor(P, "bfloat16", (64, 64, 3, 3))
+        yb, p = L.tensor(P, "float32", (2, 64, 16, 16)), L.ConvParams(1, 1, 1, 1, 1, 1)
+        assert lib.mjt_conv2d_meta(ctypes.byref(xb), ctypes.byref(w), ctypes.byref(yb), ctypes.byref(p)) == 0
+        assert L.last_kernel().startswith("mjt_conv_mfma_bf16")
+        z = L.tensor(P, "float32", (128, 64))
+        assert lib.mjt_reindex(ctypes.byref(x), ctypes.byref(z), 2, L.c_strings(["i1", "i0"]), 0.0, 0, L.c_strings([]), 0, None) == 0
+        return L.jit_stats()
+
+    before = L.jit_stats()[0]
+    first = calls()[0]
+    assert first >= before + 3                               # reduce, convolution (+ its repack), transpose
+    assert calls()[0] == first                               # second time: everything from the look-up tables
+    lib.mjt_shutdown()
+    L._device = None
+    L.init(-1)
+    assert calls()[0] >= first + 3                           # compiled again, not taken from a stale table
