@@ -21,17 +21,17 @@
 // whatever the row count, and the stores of one tile and the loads of the next
 // overlap the MFMAs.  Within a tile wave (wko, wpx) owns 64 channels x TRW rows =
 // 4 x NT accumulator tiles.  Channels are consumed 64 at a time:
-//   * the input rows the tile touches are staged through LDS as
-//     [row][col][64 c] (channel innermost) so that a B fragment is one 16-byte
-//     LDS read per lane.  The NCHW -> channel-innermost transpose happens in the
-//     LDS write: a lane loads 8 columns of one channel, swaps halves with its
-//     neighbour lane so that it owns two channels x four columns, packs the two
-//     channels of a column into one dword, and the dwords of a wave fill whole
-//     128-byte rows; positions are padded to 144 bytes, which makes the address
-//     of a fragment linear in the tap.  The tile is double buffered across
-//     channel blocks and across tiles: the loads of the next block are issued
-//     before the MFMAs of the current one and written to the other buffer after
-//     them (one barrier per channel block);
+//   * the input rows the tile touches are staged through LDS as 8 planes
+//     [8 c][row][col][8 c] (one per group of 8 channels, channels innermost) so
+//     that a B fragment is one 16-byte LDS read per lane.  The NCHW ->
+//     channel-innermost transpose happens on the way: a lane loads 8 columns of
+//     one channel, the 8 lanes of a column group exchange among themselves until
+//     each owns one column for the 8 channels, and writes 16 bytes: a wave fills
+//     a linear 1 KB run of a plane.  The address of a fragment is linear in the
+//     tap and the k-step.  The tile is double buffered across channel blocks and
+//     across tiles: the loads of the next block are issued before the MFMAs of
+//     the current one and written to the other buffer after them (one barrier
+//     per channel block);
 //   * A fragments come straight from the re-packed weights
 //     Wp[tap][c/64][k-step][ko/16][lane][8 c] (1 KB per fragment in lane order, L2
 //     resident) and are loaded one step before the MFMAs that use them.
@@ -53,16 +53,17 @@ struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as p
 #define NCB (C_ / CB)
 #define GROUPS (W_ / 8)                 // groups of 8 columns
 #define SEGS ((GROUPS + 7) / 8)         // segments of 64 columns
-#define TILE_ELEMS (LROWS * LCOLS * PSTRIDE)
+#define TILE_ELEMS (LROWS * LCOLS * 64)
 
-// LDS tile: position (row, col) holds its 64 channels in 128 bytes followed by 16 bytes of padding.
-// With a 144-byte stride, 8 neighbouring positions read by 8 lanes (one 16-byte chunk each) fall on 8
-// different groups of 4 banks, so fragment reads are conflict-free, and the address of a fragment is
-// linear in the tap: it folds into the immediate offset of the LDS read.
-#define PSTRIDE 72
+// LDS tile: 8 planes, one per group of 8 channels, each [row][col][8 c] (16 bytes per position).  The 16 lanes
+// that read a fragment together (16 neighbouring pixels, one channel group) then touch one 256-byte run, which
+// the LDS serves at its full rate (a position stride of 64 bytes or more halves it, whatever the banks), the
+// address of a fragment stays linear in the tap (it folds into the immediate offset of the read), and the
+// transposed tile is written as linear 1 KB runs.
+#define PLANE_ELEMS (LROWS * LCOLS * 8)
 __device__ __forceinline__ int mjt_lds_off(int pos, int chunk) {
     // element offset (in bf16) of 16-byte chunk `chunk` (0..7) of position `pos`
-    return pos * PSTRIDE + (chunk << 3);
+    return chunk * PLANE_ELEMS + (pos << 3);
 }
 
 template <int V> struct mjt_ic { static constexpr int v = V; };
@@ -72,9 +73,9 @@ template <int I, int N, class F> __device__ __forceinline__ void mjt_static_for(
         mjt_static_for<I + 1, N>(f);
     }
 }
-// byte offset inside the LDS tile of step s = (tap, k-step): row/column shift of the tap, 64 bytes per k-step
+// byte offset inside the LDS tile of step s = (tap, k-step): row/column shift of the tap, 4 planes per k-step
 __device__ constexpr int mjt_frag_off(int s) {
-    return ((((s >> 1) / S_) * DH * LCOLS + ((s >> 1) % S_) * DW) * PSTRIDE + (s & 1) * 32) * 2;
+    return ((((s >> 1) / S_) * DH * LCOLS + ((s >> 1) % S_) * DW) * 8 + (s & 1) * 4 * PLANE_ELEMS) * 2;
 }
 // value of lane ^ 1, ^ 2, ^ 4 through data-parallel-primitive moves (quad permutes; ^ 4 is a mirror
 // of each group of 8 lanes followed by a reversal inside each quad)
@@ -192,7 +193,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
             f[2] = __builtin_amdgcn_perm(s1, c2, sel_a);
             f[3] = __builtin_amdgcn_perm(s1, c3, sel_b);
             if (lr < lrows && seg * 8 + sg < GROUPS) {       // rows outside the image carry zeros
-                unsigned short* dst = &xs[buf][0] + mjt_lds_off(lr * LCOLS + PW + seg * 64, cg) + lane * PSTRIDE;
+                unsigned short* dst = &xs[buf][0] + mjt_lds_off(lr * LCOLS + PW + seg * 64 + lane, cg);
                 *(mjt_u32x4v*)dst = f;
             }
         }

@@ -82,7 +82,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t LCOLS = (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1 > W + 2 * p->pad_w
                               ? (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1
                               : W + 2 * p->pad_w;
-    while (TRW > 1 && lds_rows(TRW) * LCOLS * 144 > 72 * 1024) TRW--;   // two buffers of this size live in LDS
+    while (TRW > 1 && lds_rows(TRW) * LCOLS * 128 > 72 * 1024) TRW--;   // two buffers of this size live in LDS
     const int64_t NT = TRW ? (TRW * OW + 15) / 16 : 0;
     const int64_t LROWS = lds_rows(TRW);
     // output channels per workgroup: 64 per pair of waves, up to 256
@@ -90,7 +90,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
     const int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
     const bool mfma_ok = G == 1 && x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 64 == 0 &&
-                         W % 8 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 144 <= 72 * 1024 &&
+                         W % 8 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 128 <= 72 * 1024 &&
+                         // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
+                         ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + 4 * LROWS * LCOLS * 16 < 65536 &&
                          (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49;
     if (mfma_ok) {
         const int64_t items = LROWS * ((W / 8 + 7) / 8) * 8;     // (row, 64 columns, 8 channels); a wave moves one item per load
