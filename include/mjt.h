@@ -209,9 +209,10 @@ int mjt_fused_reduce(const mjt_fused_desc* desc, const mjt_tensor* y, int op, ui
  * python/jittor/nn.py:1251-1262 builds and opt/tuner/conv_tuner.cc:218-411
  * recognises; the parameters are the ones the matcher solves for
  * (conv_tuner.cc:333-356).  x [N,C,H,W], w [K,C,R,S], y [N,K,OH,OW].
- * x and w are bfloat16 or float32 (same dtype); y is float32 (the
+ * x and w are bfloat16, float16 or float32 (same dtype); y is float32 (the
  * accumulator) or x's dtype (narrowed by truncation for bfloat16,
- * type/fp16_compute.h:238-241).  Out-of-range taps contribute 0. */
+ * type/fp16_compute.h:238-241, by rounding to nearest even for float16,
+ * :147-198).  Out-of-range taps contribute 0. */
 typedef struct {
     int32_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
 } mjt_conv_params;
@@ -232,7 +233,7 @@ int mjt_conv2d_meta_grouped(const mjt_tensor* x, const mjt_tensor* w, const mjt_
  * opt/tuner/conv_tuner.cc:375-397 relays it to a backward-w library op,
  * extern/cuda/cudnn/ops/cudnn_conv_backward_w_op.cc):
  *   dw[k,c,r,s] = sum_{n,oh,ow} dy[n,k,oh,ow] * x[n,c,oh*sh-ph+r*dh,ow*sw-pw+s*dw]
- * x [N,C,H,W] and dy [N,K,OH,OW] bfloat16, dw [K,C,R,S] float32 or bfloat16
+ * x [N,C,H,W] and dy [N,K,OH,OW] bfloat16 or float16, dw [K,C,R,S] float32 or their dtype
  * (float32 accumulation, rounded once).  One MFMA kernel plus a reduce over
  * slices of images; shapes it does not cover (horizontal stride > 1, more
  * than 9 taps, left padding > 2, K % 64 != 0, ...) return MJT_ERR_UNSUPPORTED

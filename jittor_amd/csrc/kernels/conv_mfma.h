@@ -3,7 +3,7 @@
 // (reference: python/jittor/nn.py:1251-1262; recognised by
 // python/jittor/src/opt/tuner/conv_tuner.cc:218-411) as an implicit GEMM
 //   Y[n][ko][p] = sum_{kh,kw,c} Wp[kh,kw][ko][c] * X[n][c][oh*SH-PH+kh*DH][ow*SW-PW+kw*DW]
-// with bfloat16 operands, exact products and float32 accumulation
+// with bfloat16 (or float16) operands, exact products and float32 accumulation
 // (opt/kernel_ir.cc:958-968, ops/reduce_op.cc:259-266).  Taps outside the image
 // contribute 0 (overflow value 0 times w).
 //
@@ -12,7 +12,7 @@
 // groups per workgroup), TRW / NT / LROWS (output rows per wave, 16-pixel tiles per
 // wave and input rows in LDS of a full tile), RPW (output rows a workgroup owns),
 // NFULL full tiles followed, when TAIL_TRW > 0, by one shorter tile (TAIL_TRW,
-// TAIL_NT, TAIL_LROWS), LCOLS, ITEMS_PER_WAVE, Y_BF16.
+// TAIL_NT, TAIL_LROWS), LCOLS, ITEMS_PER_WAVE, Y_BF16 (16-bit output in the operand type), IN_F16.
 //
 // Mapping.  v_mfma_f32_16x16x32_bf16 computes D[16 ko][16 px] += A[16 ko][32 c] *
 // B[32 c][16 px].  A workgroup of WPX*WKO waves owns 64*WKO output channels x RPW
@@ -37,7 +37,26 @@
 //     resident) and are loaded one step before the MFMAs that use them.
 // Padding columns are zeroed once; rows outside the image are written as zeros.
 
+// operands: bfloat16, or with IN_F16 float16 (same kernel: only the MFMA and the narrowing of a 16-bit result differ)
+#if IN_F16
+typedef _Float16 mjt_bf16x8 __attribute__((ext_vector_type(8)));
+#define MJT_MFMA __builtin_amdgcn_mfma_f32_16x16x32_f16
+// float16 <- float rounds to nearest even (type/fp16_compute.h:147-198)
+__device__ __forceinline__ unsigned mjt_narrow2(float lo, float hi) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 v;
+    v[0] = (_Float16)lo;
+    v[1] = (_Float16)hi;
+    return __builtin_bit_cast(unsigned, v);
+}
+#else
 typedef __bf16 mjt_bf16x8 __attribute__((ext_vector_type(8)));
+#define MJT_MFMA __builtin_amdgcn_mfma_f32_16x16x32_bf16
+// bfloat16 <- float keeps the upper 16 bits (type/fp16_compute.h:238-241)
+__device__ __forceinline__ unsigned mjt_narrow2(float lo, float hi) {
+    return (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
+}
+#endif
 typedef float mjt_f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned mjt_u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
@@ -269,7 +288,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
                     const mjt_bf16x8 b = __builtin_bit_cast(mjt_bf16x8, bq[f % (BQ_DIST + 1)]);
 #pragma unroll
                     for (int m = 0; m < MT; m++)
-                        acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[st & 1][m], b, acc[m][t], 0, 0, 0);
+                        acc[m][t] = MJT_MFMA(ring[st & 1][m], b, acc[m][t], 0, 0, 0);
                 });
             });
             if (more || next_lrows) {
@@ -313,8 +332,8 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
                     const size_t o = (((size_t)n * K_ + ko) * OH_ + orow) * OW_ + col;
 #if Y_BF16
                     mjt_u32x2 pk;
-                    pk[0] = (__float_as_uint(y4[0]) >> 16) | (__float_as_uint(y4[1]) & 0xffff0000u);
-                    pk[1] = (__float_as_uint(y4[2]) >> 16) | (__float_as_uint(y4[3]) & 0xffff0000u);
+                    pk[0] = mjt_narrow2(y4[0], y4[1]);
+                    pk[1] = mjt_narrow2(y4[2], y4[3]);
                     *(mjt_u32x2*)((unsigned short*)p.a[2] + o) = pk;
 #else
                     *(mjt_f32x4*)((float*)p.a[2] + o) = y4;
@@ -336,7 +355,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
                         const int ko = ko_base + m * 16 + lg * 4 + i;
                         const size_t o = (((size_t)n * K_ + ko) * OH_ + orow) * OW_ + col;
 #if Y_BF16
-                        ((unsigned short*)p.a[2])[o] = (unsigned short)(__float_as_uint(acc[m][t][i]) >> 16);
+                        ((unsigned short*)p.a[2])[o] = (unsigned short)mjt_narrow2(acc[m][t][i], 0.0f);
 #else
                         ((float*)p.a[2])[o] = acc[m][t][i];
 #endif

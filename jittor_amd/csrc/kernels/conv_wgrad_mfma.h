@@ -4,7 +4,7 @@
 // ops/reduce_op.cc:339-362, ops/broadcast_to_op.cc:112-117; recognised by
 // opt/tuner/conv_tuner.cc:375-397 and relayed there to a backward-w library call):
 //   dW[k][c][r][s] = sum_{n,oh,ow} dy[n][k][oh][ow] * x[n][c][oh*SH-PH+r*DH][ow-PW+s*DW]
-// for bfloat16 operands with exact products and float32 accumulation; taps outside the image
+// for bfloat16 (or, with IN_F16, float16) operands with exact products and float32 accumulation; taps outside the image
 // contribute 0.  Horizontal stride 1 only (consecutive output columns read consecutive input
 // columns), everything else is baked in by the host: C_, H_, W_, K_, R_, S_, OH_, OW_, SH, PH, PW, DH,
 // DW, KG (groups of 64 output channels per workgroup: 1, 2 or 4; the 8 waves of a workgroup are KG
@@ -33,7 +33,13 @@
 // [slice*ips, slice*ips+ips): the partial sums of the slices go to partial[slice][k][c][r][s]
 // (float32) and are added up by a reduce launch.
 
+#if IN_F16
+typedef _Float16 mjt_bf16x8 __attribute__((ext_vector_type(8)));
+#define MJT_MFMA __builtin_amdgcn_mfma_f32_16x16x32_f16
+#else
 typedef __bf16 mjt_bf16x8 __attribute__((ext_vector_type(8)));
+#define MJT_MFMA __builtin_amdgcn_mfma_f32_16x16x32_bf16
+#endif
 typedef float mjt_f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
 
@@ -254,7 +260,7 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
             const mjt_bf16x8 b = __builtin_bit_cast(mjt_bf16x8, v);
 #pragma unroll
             for (int m = 0; m < 4; m++)
-                acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mjt_bf16x8, afrag[m]), b, acc[m][t], 0, 0, 0);
+                acc[m][t] = MJT_MFMA(__builtin_bit_cast(mjt_bf16x8, afrag[m]), b, acc[m][t], 0, 0, 0);
         });
         });
         if constexpr (NBUF >= 2) cur = cur + 1 == NBUF ? 0 : cur + 1;

@@ -45,8 +45,8 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     check_tensor(y, "conv y");
     MJT_CHECK(p, "conv: null parameters");
     MJT_CHECK(x->ndim == 4 && w->ndim == 4 && y->ndim == 4, "conv: x, w and y must have rank 4");
-    MJT_CHECK(x->dtype == w->dtype && (x->dtype == MJT_BFLOAT16 || x->dtype == MJT_FLOAT32),
-              "conv: x and w must both be bfloat16 or float32");
+    MJT_CHECK(x->dtype == w->dtype && (x->dtype == MJT_BFLOAT16 || x->dtype == MJT_FLOAT16 || x->dtype == MJT_FLOAT32),
+              "conv: x and w must both be bfloat16, float16 or float32");
     MJT_CHECK(y->dtype == MJT_FLOAT32 || y->dtype == x->dtype, "conv: y must be float32 or the input dtype");
     MJT_CHECK(G >= 1, "conv: groups must be >= 1, got " << G);
     // C is the number of channels one output channel sees: all of x's, or those of its group
@@ -89,7 +89,8 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
     const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
     const int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
-    const bool mfma_ok = G == 1 && x->dtype == MJT_BFLOAT16 && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 64 == 0 &&
+    const bool half = x->dtype == MJT_FLOAT16;
+    const bool mfma_ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && C % 64 == 0 && K % 64 == 0 &&
                          W % 8 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 128 <= 72 * 1024 &&
                          // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
                          ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + 4 * LROWS * LCOLS * 16 < 65536 &&
@@ -129,19 +130,19 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const char* bq_env = getenv("MJT_CONV_BQ");
         const int BQ = bq_env && *bq_env ? atoi(bq_env) : 3;   // B fragments requested ahead of use
         std::ostringstream key;
-        key << "mfma|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype == MJT_BFLOAT16) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT;
+        key << "mfma|" << half << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT;
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
             std::ostringstream name;
-            name << "mjt_conv_mfma_bf16_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s"
+            name << "mjt_conv_mfma_" << (half ? "f16" : "bf16") << "_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s"
                  << p->stride_h << "x" << p->stride_w << "_p" << p->pad_h << "x" << p->pad_w << "_d" << p->dil_h << "x"
-                 << p->dil_w << "_rows" << RPW << (y->dtype == MJT_BFLOAT16 ? "_obf16" : "_of32");
+                 << p->dil_w << "_rows" << RPW << (y->dtype == MJT_FLOAT32 ? "_of32" : half ? "_of16" : "_obf16");
             std::ostringstream src;
             src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo.str()
                 << "#define MT " << MT << "\n#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
-                << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS  << "\n#define BQ_DIST " << BQ << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype == MJT_BFLOAT16 ? 1 : 0)
+                << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS  << "\n#define BQ_DIST " << BQ << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype != MJT_FLOAT32 ? 1 : 0) << "\n#define IN_F16 " << (half ? 1 : 0)
                 << "\n";
             src << embedded_source("conv_mfma.h") << "\n";
             k = jit_get(src.str(), name.str());
@@ -221,13 +222,14 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
     // what the MFMA kernel covers; anything else is for the caller's general path
     const int64_t KG = K % 256 == 0 ? 4 : K % 128 == 0 ? 2 : 1;
     const int64_t CTW = 8 / KG;
-    const bool ok = x->dtype == MJT_BFLOAT16 && dy->dtype == MJT_BFLOAT16 && (dw->dtype == MJT_FLOAT32 || dw->dtype == MJT_BFLOAT16) &&
+    const bool half = x->dtype == MJT_FLOAT16;
+    const bool ok = (x->dtype == MJT_BFLOAT16 || half) && dy->dtype == x->dtype && (dw->dtype == MJT_FLOAT32 || dw->dtype == x->dtype) &&
                     p->stride_w == 1 && p->pad_w <= 2 && (S - 1) * p->dil_w - p->pad_w <= 4 && K % 64 == 0 && C % (16 * CTW) == 0 && R * S <= 9 && OW % 8 == 0 &&
                     W % 2 == 0 && N >= 1 && numel(x) * 2 < (int64_t(1) << 31) && numel(dy) * 2 < (int64_t(1) << 31) &&
                     (uintptr_t)x->ptr % 4 == 0 && (uintptr_t)dy->ptr % 16 == 0 &&
                     !getenv("MJT_NO_FASTPATH");
     if (!ok)
-        MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: only bfloat16 operands with horizontal stride 1, column shifts of the taps within -2 .. 4, at most 9 taps, "
+        MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: only bfloat16 or float16 operands with horizontal stride 1, column shifts of the taps within -2 .. 4, at most 9 taps, "
                                       "K % 64 == 0, C % " << 16 * CTW << " == 0, OW % 8 == 0 and tensors below 2 GB run on the MFMA kernel");
     Context& c = ctx();
     const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
@@ -243,17 +245,17 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
 
     std::ostringstream key;
     key << "wgrad|" << C << "|" << H << "|" << W << "|" << K << "|" << R << "|" << S << "|" << OH << "|" << OW << "|" << p->stride_h << "|"
-        << p->pad_h << "|" << p->pad_w << "|" << p->dil_h << "|" << p->dil_w << "|" << KG;
+        << p->pad_h << "|" << p->pad_w << "|" << p->dil_h << "|" << p->dil_w << "|" << KG << "|" << half;
     JitKernel* k = cached(key.str());
     if (!k) {
         std::ostringstream name;
-        name << "mjt_conv_wgrad_mfma_bf16_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s" << p->stride_h
+        name << "mjt_conv_wgrad_mfma_" << (half ? "f16" : "bf16") << "_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s" << p->stride_h
              << "x1_p" << p->pad_h << "x" << p->pad_w << "_d" << p->dil_h << "x" << p->dil_w;
         std::ostringstream src;
         src << "#define ENTRY " << name.str() << "\n#define C_ " << C << "\n#define H_ " << H << "\n#define W_ " << W << "\n#define K_ " << K
             << "\n#define R_ " << R << "\n#define S_ " << S << "\n#define OH_ " << OH << "\n#define OW_ " << OW << "\n#define SH "
             << p->stride_h << "\n#define PH " << p->pad_h << "\n#define PW " << p->pad_w << "\n#define DH " << p->dil_h << "\n#define DW "
-            << p->dil_w << "\n#define KG " << KG << "\n";
+            << p->dil_w << "\n#define KG " << KG << "\n#define IN_F16 " << (half ? 1 : 0) << "\n";
         src << embedded_source("conv_wgrad_mfma.h") << "\n";
         k = jit_get(src.str(), name.str());
         remember(key.str(), k);

@@ -146,7 +146,7 @@ def _match_conv_bwd(op):
                 continue
             if list(w.shape) != [K, C, R, S] or list(dy.shape) != [N, K, OH, OW] or w.dtype != dy.dtype:
                 continue
-            if w.dtype not in ("float32", "bfloat16") or op.out.dtype not in ("float32", w.dtype):
+            if w.dtype not in ("float32", "bfloat16", "float16") or op.out.dtype not in ("float32", w.dtype):
                 continue
             sh, sw, ph, pw, dh, dw = params
             if dh * (R - 1) - ph < 0 or dw * (S - 1) - pw < 0:
@@ -174,7 +174,7 @@ def _match_conv_bwd(op):
             x = ra.inputs[0]
             if x.ndim != 4 or list(dy.shape) != [N, K, OH, OW] or x.dtype != dy.dtype or x.shape[0] != N or x.shape[1] != C:
                 continue
-            if x.dtype not in ("float32", "bfloat16") or op.out.dtype not in ("float32", x.dtype):
+            if x.dtype not in ("float32", "bfloat16", "float16") or op.out.dtype not in ("float32", x.dtype):
                 continue
             params = _conv_affine(ra.indexes, x.shape, y7.shape)
             if params is None:
@@ -243,7 +243,7 @@ def _match_conv(red, consumers, targets):
         x, w = ro.inputs[0], bo.inputs[0]
         if x.ndim != 4 or w.ndim != 4 or bo.bcast_mask != 0b0011001:
             continue
-        if x.dtype != w.dtype or x.dtype not in ("float32", "bfloat16"):
+        if x.dtype != w.dtype or x.dtype not in ("float32", "bfloat16", "float16"):
             continue
         N, K, C, OH, OW, R, S = xx.shape
         if list(w.shape) != [K, C, R, S] or x.shape[0] != N or x.shape[1] != C:
@@ -301,7 +301,7 @@ def _match_conv_grouped(op):
         x, w = rx.inputs[0], rw.inputs[0]
         if x.ndim != 4 or list(w.shape) != [G * KG, CG, R, S] or x.shape[0] != N or x.shape[1] != G * CG:
             continue
-        if x.dtype != w.dtype or x.dtype not in ("float32", "bfloat16") or op.out.dtype not in ("float32", x.dtype):
+        if x.dtype != w.dtype or x.dtype not in ("float32", "bfloat16", "float16") or op.out.dtype not in ("float32", x.dtype):
             continue
         wa = [_affine(e, w.shape, yy.shape) for e in rw.indexes]
         if len(wa) != 4 or not (is_sum(wa[0], [(1, KG), (2, 1)]) and is_sum(wa[1], [(3, 1)])
@@ -690,7 +690,7 @@ def _run_single(op):
         N, C, H, W = x.shape
         _, K, OH, OW = dy.shape
         R, S = out.shape[2], out.shape[3]
-        if x.dtype == "bfloat16" and flags["enable_conv_wgrad_kernel"]:
+        if x.dtype in ("bfloat16", "float16") and flags["enable_conv_wgrad_kernel"]:
             # the MFMA kernel; shapes it does not cover come back as unsupported and take the paths below
             tx, td = _tensor_of(x), _tensor_of(dy)
             tw = _lib.tensor(_alloc_out(out), out.dtype, out.shape)

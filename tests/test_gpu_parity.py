@@ -571,10 +571,10 @@ def test_conv_grouped_entry_and_front_end(gpu):
         jt.nn.conv2d(jt.array(x), jt.array(w), groups=4)
 
 
-def _wgrad_call(xbits, dybits, R, S, params, out_dtype="float32"):
-    x, dy = jt.from_storage(xbits, "bfloat16"), jt.from_storage(dybits, "bfloat16")
+def _wgrad_call(xbits, dybits, R, S, params, out_dtype="float32", in_dtype="bfloat16"):
+    x, dy = jt.from_storage(xbits, in_dtype), jt.from_storage(dybits, in_dtype)
     dw = jt.zeros([dybits.shape[1], xbits.shape[1], R, S], out_dtype)
-    tx, td = L.tensor(x.raw_ptr(), "bfloat16", x.shape), L.tensor(dy.raw_ptr(), "bfloat16", dy.shape)
+    tx, td = L.tensor(x.raw_ptr(), in_dtype, x.shape), L.tensor(dy.raw_ptr(), in_dtype, dy.shape)
     tw = L.tensor(dw.raw_ptr(), out_dtype, dw.shape)
     p = L.ConvParams(*params)
     rc = L.load().mjt_conv2d_meta_wgrad(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p))
@@ -637,6 +637,43 @@ def test_conv_wgrad_entry_rejects_what_the_kernel_does_not_cover(gpu):
     assert rc == -2 and "stride" in L.load().mjt_last_error().decode()
     rc, _ = _wgrad_call(xb, _bf16(rng.standard_normal((1, 64, 9, 8))), 3, 3, (1, 1, 1, 1, 1, 1))   # dy does not follow from x
     assert rc == -1 and "does not follow" in L.load().mjt_last_error().decode()
+
+
+def test_conv_float16_operands(gpu):
+    """float16 operands take the same kernels as bfloat16 (the f16 MFMA; a float16 result is rounded to nearest
+    even, type/fp16_compute.h:147-198): forward on the MFMA and the direct kernel, weight gradient, and the three
+    units through the front end with float16 gradients."""
+    rng = np.random.default_rng(33)
+    x = rng.standard_normal((2, 64, 12, 16)).astype(np.float16)
+    w = (rng.standard_normal((128, 64, 3, 3)) * 0.1).astype(np.float16)
+    want = O.conv_meta(x.astype(np.float32), w.astype(np.float32), 1, 1, 1)
+    got, kern = _conv_call(x, w, (1, 1, 1, 1, 1, 1), in_dtype="float16")
+    assert kern.startswith("mjt_conv_mfma_f16") and np.allclose(got, want, rtol=1e-5, atol=1e-5)
+    got16, kern = _conv_call(x, w, (1, 1, 1, 1, 1, 1), out_dtype="float16", in_dtype="float16")
+    assert kern.endswith("_of16") and got16.dtype == np.float16
+    assert np.all(np.abs(got16.astype(np.float32) - want) <= 2.0 ** -10 * np.abs(want) + 1e-5)   # rounding + summation order
+    xs, ws = rng.standard_normal((2, 3, 9, 8)).astype(np.float16), rng.standard_normal((4, 3, 3, 3)).astype(np.float16)
+    got, kern = _conv_call(xs, ws, (1, 1, 1, 1, 1, 1), in_dtype="float16")
+    assert kern.startswith("mjt_conv_direct_float16")
+    assert np.allclose(got, O.conv_meta(xs.astype(np.float32), ws.astype(np.float32), 1, 1, 1), rtol=1e-5, atol=1e-5)
+    # weight gradient
+    xg, dy = rng.standard_normal((2, 128, 6, 8)).astype(np.float16), rng.standard_normal((2, 64, 6, 8)).astype(np.float16)
+    rc, dw = _wgrad_call(xg, dy, 3, 3, (1, 1, 1, 1, 1, 1), in_dtype="float16")
+    assert rc == 0 and L.last_kernel().startswith("mjt_conv_wgrad_mfma_f16")
+    ref = O.conv_meta_wgrad(xg.astype(np.float32), dy.astype(np.float32), 3, 3, 1, 1, 1)
+    assert np.abs(dw - ref).max() <= 1e-4 * np.abs(ref).max()
+    # front end
+    vx, vw = jt.array(x), jt.array(w)
+    assert vx.dtype == "float16"
+    y = jt.nn.conv2d(vx, vw, padding=1)
+    r = (rng.integers(-2, 3, y.shape) * 0.5).astype(np.float16)
+    gx, gw = jt.grad((y * jt.array(r)).sum(), [vx, vw])
+    before = jt.executor_stats["conv_matches"]
+    jt.sync([y, gx, gw])
+    assert jt.executor_stats["conv_matches"] - before == 3 and (y.dtype, gx.dtype, gw.dtype) == ("float16",) * 3
+    assert np.abs(y.float32().data - want).max() <= 2.0 ** -10 * np.abs(want).max()
+    ref_gw = O.conv_meta_wgrad(x.astype(np.float32), r.astype(np.float32), 3, 3, 1, 1, 1)
+    assert np.abs(gw.float32().data - ref_gw).max() <= 2.0 ** -9 * np.abs(ref_gw).max()
 
 
 def test_conv_front_end_pattern_match(gpu):
