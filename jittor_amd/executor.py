@@ -117,15 +117,24 @@ def _lazy_broadcast(v):
     bo = _lazy_op(u, BroadcastOp)
     if bo is None:
         return None, None
-    src = bo.inputs[0]
-    while not src.materialised and isinstance(src._op, UnaryOp) and src._op.op == "cast":
+    # behind the broadcast: go down through casts as far as they change nothing, i.e. to the deepest var of v's dtype
+    # with only wider float types on the way (a var of v's dtype that is itself a narrowing cast stays what it is)
+    def widening_only(types, r0):
+        return all(_FLOAT_RANK.get(d, 0) > r0 or d == v.dtype for d in types)
+    r0 = _FLOAT_RANK.get(v.dtype)
+    src, best, below = bo.inputs[0], None, []
+    while True:
+        below.append(src.dtype)
+        if src.dtype == v.dtype and r0 is not None and widening_only(chain + below, r0):
+            best = src
+        if src.materialised or not isinstance(src._op, UnaryOp) or src._op.op != "cast":
+            break
         src = src._op.inputs[0]
-        chain.append(src.dtype)
-    if len(chain) > 1:
-        r0 = _FLOAT_RANK.get(src.dtype)
-        if r0 is None or src.dtype != v.dtype or any(_FLOAT_RANK.get(d, 0) < r0 or (_FLOAT_RANK.get(d) == r0 and d != src.dtype)
-                                                     for d in chain):
-            return None, None
+    if best is None:
+        if len(chain) == 1 and bo.inputs[0].dtype == v.dtype:
+            return bo, bo.inputs[0]                      # no casts at all (any dtype)
+        return None, None
+    src = best
     return bo, src
 
 

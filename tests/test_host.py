@@ -494,3 +494,20 @@ def test_shutdown_forgets_kernels_and_rebinding_compiles_again(compile_only, mon
     L._device = None
     L.init(-1)
     assert calls()[0] >= first + 3                           # compiled again, not taken from a stale table
+
+
+def test_conv_gradient_patterns_match_for_common_losses():
+    """The two backward patterns are recognised whatever stands between the convolution and the loss: the loss may
+    be the output itself (jt.grad seeds ones, test_conv_tuner.py:105-133), its sum or mean (for 16-bit outputs these
+    put float32 casts around dy: the narrowing cast of dy stays, the identity casts are looked through) or a product."""
+    from jittor_amd import executor as E
+    for dtype in ("float32", "float16", "bfloat16"):
+        x, w = jt.zeros([2, 3, 8, 8]).cast(dtype), jt.zeros([4, 3, 3, 3]).cast(dtype)
+        y = jt.nn.conv2d(x, w, padding=1)
+        r = jt.zeros(y.shape).cast(dtype)
+        for loss in (y, y.sum(), y.mean(), (y * r).sum(), (y * y).sum()):
+            gx, gw = jt.grad(loss, [x, w])
+            ux, uw = E._match_conv_bwd(gx._op), E._match_conv_bwd(gw._op)
+            assert isinstance(ux, E.ConvBwdDataUnit) and isinstance(uw, E.ConvBwdWeightUnit), (dtype, loss)
+            assert ux.inputs[0].dtype == dtype and list(ux.inputs[0].shape) == [2, 4, 8, 8]
+            assert uw.inputs[1].dtype == dtype and gx.dtype == dtype and gw.dtype == dtype
