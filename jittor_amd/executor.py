@@ -146,8 +146,8 @@ def _match_conv_bwd(op):
         if mul is None or mul.op != "multiply" or y7.ndim != 7 or op.out.ndim != 4:
             return None
         params = _conv_affine(op.indexes, op.out.shape, y7.shape)
-        if params is None or params[0] != 1 or params[1] != 1:
-            return None                                         # stride 1 only
+        if params is None:
+            return None
         N, K, C, OH, OW, R, S = y7.shape
         for a, b in (mul.inputs, mul.inputs[::-1]):
             (ba, w), (bb, dy) = _lazy_broadcast(a), _lazy_broadcast(b)
@@ -160,7 +160,9 @@ def _match_conv_bwd(op):
             sh, sw, ph, pw, dh, dw = params
             if dh * (R - 1) - ph < 0 or dw * (S - 1) - pw < 0:
                 continue
-            if list(op.out.shape) != [N, C, OH + dh * (R - 1) - 2 * ph, OW + dw * (S - 1) - 2 * pw]:
+            H, W = op.out.shape[2], op.out.shape[3]
+            if list(op.out.shape[:2]) != [N, C] or OH != (H + 2 * ph - dh * (R - 1) - 1) // sh + 1 \
+                    or OW != (W + 2 * pw - dw * (S - 1) - 1) // sw + 1:
                 continue
             return ConvBwdDataUnit(op, dy, w, params)
         return None
@@ -190,8 +192,8 @@ def _match_conv_bwd(op):
                 continue
             sh, sw, ph, pw, dh, dw = params
             H, W = x.shape[2], x.shape[3]
-            # as a convolution of x^T [C,N,H,W] with dy^T [K,N,OH,OW] (stride d, dilation s) the output must be R x S
-            if (H + 2 * ph - sh * (OH - 1) - 1) // dh + 1 != R or (W + 2 * pw - sw * (OW - 1) - 1) // dw + 1 != S:
+            # dy must be the output gradient of that convolution of x
+            if OH != (H + 2 * ph - dh * (R - 1) - 1) // sh + 1 or OW != (W + 2 * pw - dw * (S - 1) - 1) // sw + 1:
                 continue
             return ConvBwdWeightUnit(op, x, dy, params)
     return None
@@ -689,6 +691,14 @@ def _run_single(op):
         with core.no_grad():
             wt = core.reindex(w, [C, K, R, S], ["i1", "i0", "%d-i2" % (R - 1), "%d-i3" % (S - 1)])
         _run_single(wt._op)
+        if sh != 1 or sw != 1:
+            # a strided convolution's input gradient is the stride-1 one of dy with sh-1 (sw-1) zeros between its rows
+            # (columns) and zeros up to the size that makes the result H x W: one reindex, out of range reads 0
+            H, W = out.shape[2], out.shape[3]
+            with core.no_grad():
+                dy = core.reindex(dy, [dy.shape[0], K, H + 2 * ph - dh * (R - 1), W + 2 * pw - dw * (S - 1)],
+                                  ["i0", "i1", "i2/%d" % sh, "i3/%d" % sw], 0.0, ["i2%%%d!=0" % sh, "i3%%%d!=0" % sw])
+            _run_single(dy._op)
         tx, tw = _tensor_of(dy), _tensor_of(wt)
         ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
         p = _lib.ConvParams(1, 1, dh * (R - 1) - ph, dw * (S - 1) - pw, dh, dw)
@@ -751,7 +761,9 @@ def _run_single(op):
             dyt = core.reindex(dy, [K, N, OH, OW], ["i1", "i0", "i2", "i3"])
         _run_single(xt._op)
         _run_single(dyt._op)
-        tmp = Var([C, K, R, S], out.dtype)
+        # as a convolution of x^T [C,N,H,W] with dy^T [K,N,OH,OW] (stride d, dilation s); rows and columns of x that
+        # the stride never reaches make its output larger than R x S: the reindex below keeps the first R x S taps
+        tmp = Var([C, K, (H + 2 * ph - sh * (OH - 1) - 1) // dh + 1, (W + 2 * pw - sw * (OW - 1) - 1) // dw + 1], out.dtype)
         tx, tw = _tensor_of(xt), _tensor_of(dyt)
         tt = _lib.tensor(_alloc_out(tmp), tmp.dtype, tmp.shape)
         p = _lib.ConvParams(dh, dw, ph, pw, sh, sw)              # stride and dilation trade places

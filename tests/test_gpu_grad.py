@@ -172,7 +172,9 @@ def _conv_grads_ref(x, w, r, stride, pad, dil):
     dict(x=(2, 3, 6, 6), w=(4, 3, 3, 3), stride=1, pad=1, dil=1, units=3),
     dict(x=(3, 8, 12, 10), w=(6, 8, 3, 3), stride=1, pad=2, dil=2, units=3),
     dict(x=(2, 4, 9, 9), w=(5, 4, 3, 3), stride=1, pad=0, dil=1, units=3),
-    dict(x=(2, 4, 11, 11), w=(5, 4, 3, 3), stride=2, pad=1, dil=1, units=2),     # input gradient: generic kernels
+    dict(x=(2, 4, 11, 11), w=(5, 4, 3, 3), stride=2, pad=1, dil=1, units=3),     # strided: input gradient over zero-spaced dy
+    dict(x=(2, 4, 12, 10), w=(5, 4, 3, 3), stride=2, pad=1, dil=1, units=3),     # ... rows and columns the stride never reaches
+    dict(x=(1, 3, 13, 13), w=(2, 3, 3, 3), stride=3, pad=0, dil=2, units=3),     # stride 3, dilation 2
     dict(x=(2, 6, 8, 8), w=(4, 6, 1, 1), stride=1, pad=0, dil=1, units=3),
 ])
 def test_grad_meta_conv(gpu, case):
