@@ -319,12 +319,12 @@ def wl_copy(L, lib, steps, warmup, with_cpu):
 # Summaries: profiles/hbm_traffic_all_workloads.txt
 MEASURED_TRAFFIC = {
     "C1": 2.0 * 65557.8 * 1024 + 64.0 * 1024,
-    "C2": 2.0 * 15635.9 * 1024 + 225837.2 * 1024,
+    "C2": 2.0 * 15636.1 * 1024 + 225806.5 * 1024,
     "C3add": 2.0 * 65692.9 * 1024 + 41115.1 * 1024,
     "C3max": 2.0 * 65695.3 * 1024 + 41680.2 * 1024,
-    "C4": 2.0 * 65583.5 * 1024 + 131072.1 * 1024,
-    "C5": 2.0 * 113356.3 * 1024 + 212386.9 * 1024,
-    "C5bf16out": 2.0 * 112129.9 * 1024 + 112603.7 * 1024,
+    "C4": 2.0 * 65582.8 * 1024 + 131072.0 * 1024,
+    "C5": 2.0 * 113405.4 * 1024 + 211332.1 * 1024,
+    "C5bf16out": 2.0 * 112114.2 * 1024 + 112616.1 * 1024,
 }
 
 WORKLOADS = {
