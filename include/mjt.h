@@ -145,6 +145,21 @@ int mjt_reindex_reduce(const mjt_tensor* y, const mjt_tensor* x, int op,
                        int n_overflow_conditions, const char* const* overflow_conditions,
                        int n_extras, const mjt_tensor* extras);
 
+/* ReindexOp fused with the ReduceOp that consumes it: z = reduce(reindex(x,
+ * yshape, indexes, overflow_value, overflow_conditions, extras), op) over the
+ * last n_reduced axes of the reindex result, which is never written (the
+ * reference fuses a reindex -- a broadcast-type op -- with its consumer,
+ * executor.cc:555; this is the pooling group of python/jittor/pool.py:200-208).
+ * yshape gives the shape of the reindex result (its pointer is not used);
+ * z holds the kept axes, accumulation in z's dtype (float32 for 16-bit float
+ * results, rounded once) from the identity of op; op is add, mean, maximum,
+ * minimum or multiply. */
+int mjt_reindex_then_reduce(const mjt_tensor* x, const mjt_tensor* yshape, const mjt_tensor* z,
+                            int op, int n_reduced,
+                            int n_indexes, const char* const* indexes, double overflow_value,
+                            int n_overflow_conditions, const char* const* overflow_conditions,
+                            int n_extras, const mjt_tensor* extras);
+
 /* ---- fused element-wise group: fused_op.h:29-60 -----------------------
  * One kernel for a group of broadcast / unary / binary / ternary ops
  * (ops/broadcast_to_op.cc:177-194, ops/unary_op.cc:1021-1027,

@@ -19,6 +19,35 @@
 
 struct Params { void* a[NPARAM]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
 
+#if REDUCE_TAIL
+// Gather fused with the reduce that consumes it (the reference fuses a reindex with its consumer: it is a
+// broadcast-type op, executor.cc:555; the pooling group of python/jittor/pool.py:200-208): the loop space y is never
+// written.  One lane per output: it walks the RTAIL elements of y's last axes that fold into it, gathers each and
+// combines them in TACC.  Extra constants: TZ, TACC, COMBINE(a, x), INIT; a[1] is z, a[2] its element count,
+// P_RTAIL / P_RCOUNT the parameter words of the tail length and of 1 / tail length (mean).
+extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
+    const TX* __restrict__ xp = (const TX*)p.a[0];
+    TZ* __restrict__ zp = (TZ*)p.a[1];
+    const TX ovalue_ = (TX)__longlong_as_double((long long)(unsigned long long)p.a[3]);
+    const index_t nout = (index_t)(unsigned long long)p.a[2];
+    const index_t rtail = (index_t)(unsigned long long)p.a[P_RTAIL];
+    const TACC rcount = (TACC)__longlong_as_double((long long)(unsigned long long)p.a[P_RCOUNT]);
+    (void)rcount;
+    MJT_RX_SETUP
+    const index_t o = (index_t)blockIdx.x * 256 + threadIdx.x;
+    if (o >= nout) return;
+    TACC acc = INIT;
+    for (index_t r = 0; r < rtail; r++) {
+        const index_t e = o * rtail + r;
+        MJT_RX_DECODE
+        const index_t MJT_RX_LASTVAR = ilast_;
+        MJT_RX_INDEX
+        const TX v = ov_ ? ovalue_ : xp[xid];
+        acc = (TACC)(COMBINE(acc, v));
+    }
+    zp[o] = (TZ)acc;
+}
+#else
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 #if SCATTER
     TX* __restrict__ xp = (TX*)p.a[0];
@@ -52,3 +81,4 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     mjt_store(yp + e, yv);
 #endif
 }
+#endif

@@ -98,8 +98,9 @@ int pick_vec(int elem_size, int64_t last, const void* p) {
 }
 
 // Specialises (once per plan and variant) and launches the generic kernel.
+// With z: the gather is fused with a reduce (rop) over y's last nred axes; y then only gives the loop shape.
 void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mjt_tensor* y, double overflow_value,
-                 int n_ex, const mjt_tensor* ex) {
+                 int n_ex, const mjt_tensor* ex, const mjt_tensor* z = nullptr, int rop = 0, int nred = 0) {
     // the loop runs over y (gather output / scatter input)
     const int LD = y->ndim, XD = x->ndim;
     int64_t yn = numel(y), xn = numel(x);
@@ -107,11 +108,14 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
     int64_t biggest = std::max(xn, yn);
     for (int i = 0; i < n_ex; i++) biggest = std::max(biggest, numel(&ex[i]));
     bool use64 = biggest >= (int64_t(1) << 31);   // index_t rule of op.cc:158-192
-    int vec = pick_vec(dtype_size(x->dtype), y->shape[LD - 1], y->ptr);
+    int vec = z ? 1 : pick_vec(dtype_size(x->dtype), y->shape[LD - 1], y->ptr);
+    int64_t rtail = 1;
+    for (int i = LD - nred; z && i < LD; i++) rtail *= y->shape[i];
 
     // parameter block: a[0] x, a[1] y, a[2] nvec, a[3] overflow value,
     // then yshape[LD], ydiv[LD], xshape[XD], per extra: pointer, shape[rank]
-    std::vector<uint64_t> args{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), (uint64_t)(yn / vec), bits_of(overflow_value)};
+    std::vector<uint64_t> args{bits_of_ptr(x->ptr), bits_of_ptr(z ? z->ptr : y->ptr), (uint64_t)(z ? yn / rtail : yn / vec),
+                               bits_of(overflow_value)};
     int p_ys = (int)args.size();
     for (int i = 0; i < LD; i++) args.push_back((uint64_t)y->shape[i]);
     int p_yd = (int)args.size();
@@ -125,7 +129,14 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
         for (int i = 0; i < ex[k].ndim; i++) args.push_back((uint64_t)ex[k].shape[i]);
     }
 
+    int p_tail = 0;
+    if (z) {
+        p_tail = (int)args.size();
+        args.push_back((uint64_t)rtail);
+        args.push_back(bits_of(rtail ? 1.0 / (double)rtail : 0.0));
+    }
     std::string vkey = std::to_string(vec) + (use64 ? "L" : "I");
+    if (z) vkey += "|R" + std::to_string(rop) + "," + std::to_string(z->dtype) + "," + std::to_string(nred);
     JitKernel* kern = nullptr;
     {
         std::lock_guard<std::mutex> lock(g_mu);
@@ -185,13 +196,25 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
         frag << "#define MJT_RX_DECODE " << dec.str() << "\n";
         frag << "#define MJT_RX_INDEX " << index.str() << "\n";
         if (scatter) frag << "#define ATOMIC_UPDATE(addr, v) mjt_atomic_" << mjt_op_name(op) << "<TX>((addr), (v))\n";
+        frag << "#define REDUCE_TAIL " << (z ? 1 : 0) << "\n";
+        if (z) {
+            // accumulator as in the reduce kernels: z's type, float for 16-bit float results
+            const int ta = z->dtype == MJT_FLOAT16 || z->dtype == MJT_BFLOAT16 ? MJT_FLOAT32 : z->dtype;
+            const std::string opn = rop == MJT_OP_MEAN ? "add" : mjt_op_name(rop);
+            frag << "#define TZ " << dtype_cname(z->dtype) << "\n#define TACC " << dtype_cname(ta) << "\n#define P_RTAIL " << p_tail
+                 << "\n#define P_RCOUNT " << p_tail + 1 << "\n#define INIT mjt_init_" << opn << "<TACC>()\n";
+            if (rop == MJT_OP_MEAN) frag << "#define COMBINE(a, x) ((a) + TACC(x) * TACC(rcount))\n";
+            else frag << "#define COMBINE(a, x) mjt_" << opn << "<TACC>((a), (x))\n";
+        }
         uint64_t h = 1469598103934665603ull;
         for (unsigned char ch : frag.str()) {
             h ^= ch;
             h *= 1099511628211ull;
         }
         char name[96];
-        snprintf(name, sizeof(name), "mjt_%s_%016llx", scatter ? (std::string("reindex_reduce_") + mjt_op_name(op)).c_str() : "reindex",
+        snprintf(name, sizeof(name), "mjt_%s_%016llx",
+                 scatter ? (std::string("reindex_reduce_") + mjt_op_name(op)).c_str()
+                         : z ? (std::string("reindex_then_") + mjt_op_name(rop)).c_str() : "reindex",
                  (unsigned long long)h);
         std::string src = std::string("#define ENTRY ") + name + "\n" + frag.str() + embedded_source("prelude.h") + "\n" +
                           (scatter ? std::string(embedded_source("atomics.h")) + "\n" : std::string()) +
@@ -200,7 +223,7 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
         std::lock_guard<std::mutex> lock(g_mu);
         plan->kernels.emplace(vkey, kern);
     }
-    int64_t nvec = yn / vec;
+    int64_t nvec = z ? yn / rtail : yn / vec;
     int64_t blocks = (nvec + 255) / 256;
     MJT_CHECK(blocks < (int64_t(1) << 31), "reindex: launch too large");
     jit_launch(kern, (unsigned)blocks, 1, 256, 0, args);
@@ -277,6 +300,38 @@ void reindex_impl(const mjt_tensor* x, const mjt_tensor* y, int n_idx, const cha
     run_generic(plan, false, 0, x, y, overflow_value, n_ex, ex);
 }
 
+// reduce(reindex(x), rop) over the last nred axes of the reindex result, whose shape yshape gives (its pointer is unused)
+void reindex_then_reduce_impl(const mjt_tensor* x, const mjt_tensor* yshape, const mjt_tensor* z, int rop, int nred, int n_idx,
+                              const char* const* idx, double overflow_value, int n_ofc, const char* const* ofc, int n_ex,
+                              const mjt_tensor* ex) {
+    require_init();
+    check_tensor(x, "reindex_then_reduce x");
+    check_tensor(z, "reindex_then_reduce z");
+    check_extras(n_ex, ex);
+    MJT_CHECK(yshape && yshape->ndim >= 1 && yshape->ndim <= MJT_MAX_DIM, "reindex_then_reduce: bad loop shape");
+    MJT_CHECK(n_idx == x->ndim, "Number of x's shape and indexes should be the same. (x rank " << x->ndim << ", " << n_idx << " indexes)");
+    MJT_CHECK(n_idx == 0 || idx, "null indexes");
+    MJT_CHECK(n_ofc >= 0 && (n_ofc == 0 || ofc), "null overflow conditions");
+    MJT_CHECK(nred >= 1 && nred <= yshape->ndim, "reindex_then_reduce: " << nred << " reduced axes of " << yshape->ndim);
+    MJT_CHECK(rop == MJT_OP_ADD || rop == MJT_OP_MEAN || rop == MJT_OP_MAXIMUM || rop == MJT_OP_MINIMUM || rop == MJT_OP_MULTIPLY,
+              "reindex_then_reduce: op must be add, mean, maximum, minimum or multiply");
+    MJT_CHECK(z->dtype != MJT_BOOL, "reindex_then_reduce: accumulator dtype bool is not supported");
+    int64_t kept = 1;
+    for (int i = 0; i < yshape->ndim - nred; i++) kept *= yshape->shape[i];
+    MJT_CHECK(numel(z) == kept, "reindex_then_reduce: z has " << numel(z) << " elements, the kept axes give " << kept);
+    if (kept == 0) return;
+    if (numel(yshape) == 0) {                         // nothing folds into z: every element is the identity
+        launch_fill_pattern(z->ptr, identity_bits(rop == MJT_OP_MEAN ? MJT_OP_ADD : rop, z->dtype), dtype_size(z->dtype), (size_t)kept);
+        return;
+    }
+    mjt_tensor y = *yshape;
+    y.dtype = x->dtype;
+    y.ptr = z->ptr;                                   // never dereferenced: only its shape is used
+    std::string key = plan_key(false, 0, x, &y, n_idx, idx, n_ofc, ofc, n_ex, ex);
+    Plan* plan = get_plan(key, x, &y, y.ndim, n_idx, idx, n_ofc, ofc, n_ex, ex);
+    run_generic(plan, false, 0, x, &y, overflow_value, n_ex, ex, z, rop, nred);
+}
+
 void reindex_reduce_impl(const mjt_tensor* y, const mjt_tensor* x, int op, int n_idx, const char* const* idx, int n_ofc,
                          const char* const* ofc, int n_ex, const mjt_tensor* ex) {
     require_init();
@@ -311,6 +366,16 @@ extern "C" int mjt_reindex(const mjt_tensor* x, const mjt_tensor* y, int n_index
     return mjt::guarded([&] {
         mjt::reindex_impl(x, y, n_indexes, indexes, overflow_value, n_overflow_conditions, overflow_conditions, n_extras,
                           extras);
+    });
+}
+
+extern "C" int mjt_reindex_then_reduce(const mjt_tensor* x, const mjt_tensor* yshape, const mjt_tensor* z, int op, int n_reduced,
+                                       int n_indexes, const char* const* indexes, double overflow_value,
+                                       int n_overflow_conditions, const char* const* overflow_conditions, int n_extras,
+                                       const mjt_tensor* extras) {
+    return mjt::guarded([&] {
+        mjt::reindex_then_reduce_impl(x, yshape, z, op, n_reduced, n_indexes, indexes, overflow_value, n_overflow_conditions,
+                                      overflow_conditions, n_extras, extras);
     });
 }
 

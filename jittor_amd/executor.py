@@ -19,7 +19,7 @@ from . import profiler as _profiler
 from .flags import flags
 
 stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0, "matmul_matches": 0,
-         "wgrad_kernel": 0}
+         "wgrad_kernel": 0, "gather_reduces": 0}
 
 
 class ConvUnit:
@@ -33,6 +33,22 @@ class ConvUnit:
         self.params = params
         self.absorbed = absorbed
         self.groups = groups
+        self.id = reduce_op.id
+
+
+class GatherReduceUnit:
+    """reindex -> reduce over the last axes of its result, run as one kernel that never writes the reindex result
+    (the reference fuses a reindex with its consumer, executor.cc:555; pooling, pool.py:200-208)."""
+    kind = "gather_reduce"
+    fusable = False
+
+    def __init__(self, reduce_op, reindex_op, nred, absorbed):
+        self.out = reduce_op.out
+        self.inputs = list(reindex_op.inputs)
+        self.reindex = reindex_op
+        self.op = reduce_op.op
+        self.nred = nred
+        self.absorbed = absorbed
         self.id = reduce_op.id
 
 
@@ -334,6 +350,28 @@ def _match_conv_grouped(op):
     return None
 
 
+def _match_gather_reduce(red, consumers, target_ids):
+    """reduce(op) over the trailing axes of a reindex result nobody else reads."""
+    if red.op not in ("add", "mean", "maximum", "minimum", "multiply"):
+        return None
+    xx, absorbed = red.inputs[0], {red.id}
+    if not xx.materialised and isinstance(xx._op, UnaryOp) and xx._op.op == "cast" and xx.dtype == "float32" \
+            and xx._op.inputs[0].dtype in ("float16", "bfloat16"):
+        # a 16-bit sum or mean was rewritten to cast -> reduce(float32) -> cast: the kernel accumulates in float32 anyway
+        if xx.id in target_ids or len(consumers.get(xx.id, ())) != 1:
+            return None
+        absorbed.add(xx._op.id)
+        xx = xx._op.inputs[0]
+    ro = _lazy_op(xx, ReindexOp)
+    if ro is None or xx.id in target_ids or len(consumers.get(xx.id, ())) != 1 or getattr(xx, "_stop_fuse", False):
+        return None
+    nd, nred = xx.ndim, bin(red.reduce_mask).count("1")
+    if nred < 1 or red.reduce_mask != ((1 << nred) - 1) << (nd - nred) or red.out.dtype == "bool":
+        return None
+    absorbed.add(ro.id)
+    return GatherReduceUnit(red, ro, nred, absorbed)
+
+
 _matmul_ok = []
 
 
@@ -417,6 +455,11 @@ def _execute(ops, target_ids):
                 if cu is not None:
                     units[op.id] = cu
                     stats["matmul_matches"] += 1
+            if cu is None and isinstance(op, ReduceOp) and flags["enable_gather_reduce"]:
+                cu = _match_gather_reduce(op, consumers, target_ids)
+                if cu is not None:
+                    units[op.id] = cu
+                    stats["gather_reduces"] += 1
     nodes = [units.get(op.id, op) for op in ops]
     produced_by = {node.out.id: node for node in nodes}
     needed = set()
@@ -676,6 +719,17 @@ def _run_single(op):
                                                    op.groups))
         else:
             _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
+    elif isinstance(op, GatherReduceUnit):
+        ro = op.reindex
+        x, extras = ro.inputs[0], ro.inputs[1:]
+        tx = _tensor_of(x)
+        ts = _lib.tensor(0, x.dtype, ro.out.shape)                       # the reindex result: its shape only
+        tz = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        ex = (_lib.Tensor * max(1, len(extras)))(*[_tensor_of(e) for e in extras])
+        _lib.check(lib.mjt_reindex_then_reduce(ctypes.byref(tx), ctypes.byref(ts), ctypes.byref(tz), _lib.OP_CODE[op.op], op.nred,
+                                               len(ro.indexes), _lib.c_strings(ro.indexes), ro.overflow_value,
+                                               len(ro.overflow_conditions), _lib.c_strings(ro.overflow_conditions),
+                                               len(extras), ex))
     elif isinstance(op, MatmulUnit):
         a, b = op.inputs
         n = a.shape[-1] if op.trans[0] else a.shape[-2]

@@ -895,3 +895,60 @@ def test_zz_shutdown_and_rebind_on_the_device(gpu):
     y2, kern = _conv_call(xb, wb, (1, 1, 1, 1, 1, 1))
     assert kern.startswith("mjt_conv_mfma_bf16") and np.array_equal(s1, s2) and np.array_equal(y1, y2)
     assert np.allclose(s2, x.sum(1), rtol=1e-5, atol=1e-4)
+
+
+def test_gather_fused_with_reduce(gpu):
+    """mjt_reindex_then_reduce: a reindex whose only consumer is a reduce over its last axes runs as one kernel
+    (pooling, pool.py:200-208).  Through the C entry point against the oracle's reindex + reduce, then the
+    front end: same results as the two-kernel path, no rank-6 tensor in memory."""
+    rng = np.random.default_rng(60)
+    lib = L.load()
+    x = rng.standard_normal((2, 3, 9, 10)).astype(np.float32)
+    none, noex = L.c_strings([]), (L.Tensor * 1)()
+    for op, shape, idx, ov, nred in [
+            ("maximum", [2, 3, 4, 5, 3, 2], ["i0", "i1", "i2*2-1+i4", "i3*2-0+i5"], -1e30, 2),
+            ("mean", [2, 3, 4, 5, 3, 2], ["i0", "i1", "i2*2-1+i4", "i3*2-0+i5"], 0.0, 2),
+            ("add", [2, 9, 10, 3], ["i0", "i3", "i1", "i2"], 0.0, 1),                      # sum over channels, moved last
+            ("minimum", [7, 2, 3, 9, 10], ["i1", "i2", "(i3+i0)%9", "i4"], 5.0, 4),        # keeps only the first axis
+            ("multiply", [4, 2, 3, 3, 3], ["i1", "i2", "i0+i3", "i4*5"], 1.0, 2)]:
+        want = O.reduce(O.reindex(x, shape, idx, ov), op, list(range(len(shape) - nred, len(shape))))
+        vx, vz = jt.from_storage(x, "float32"), jt.zeros(list(want.shape), "float32")
+        tx, ts = L.tensor(vx.raw_ptr(), "float32", vx.shape), L.tensor(0, "float32", shape)
+        tz = L.tensor(vz.raw_ptr(), "float32", vz.shape)
+        L.check(lib.mjt_reindex_then_reduce(ctypes.byref(tx), ctypes.byref(ts), ctypes.byref(tz), L.OP_CODE[op], nred, len(idx),
+                                            L.c_strings(idx), ov, 0, none, 0, noex))
+        assert L.last_kernel().startswith("mjt_reindex_then_" + op)
+        got = L.d2h(vz.raw_ptr(), vz.shape, np.float32)
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-6), (op, shape)
+    # integers with an overflow condition and an extra (a gather by an index tensor, then a sum): bit-exact
+    xi = rng.integers(-50, 50, (6, 20)).astype(np.int32)
+    e0 = rng.integers(0, 20, (6, 5, 4)).astype(np.int32)
+    shape, idx, ofc = [6, 5, 4], ["i0", "@e0(i0,i1,i2)"], ["i2>2"]
+    want = O.reduce(O.reindex(xi, shape, idx, 7, ofc, [e0]), "add", [1, 2])
+    got = jt.array(xi).reindex(shape, idx, 7, ofc, [jt.array(e0)]).sum([1, 2])
+    before = jt.executor_stats["gather_reduces"]
+    assert np.array_equal(got.data, want) and jt.executor_stats["gather_reduces"] == before + 1
+    # pooling through the front end, float32 and bfloat16 (the 16-bit mean's float32 casts are part of the group)
+    xp = rng.standard_normal((3, 5, 11, 12)).astype(np.float32)
+    for dtype in ("float32", "bfloat16"):
+        for op in ("maximum", "mean"):
+            v = jt.array(xp).cast(dtype)
+            jt.sync([v])
+            before, l0 = jt.executor_stats["gather_reduces"], jt.executor_stats["launches"]
+            y = jt.pool(v, 3, op, 1, 2)
+            jt.sync([y])
+            l1 = jt.executor_stats["launches"]
+            fused = y.float32().data
+            assert jt.executor_stats["gather_reduces"] == before + 1 and y.dtype == ("float32" if op == "maximum" or dtype == "float32" else dtype)
+            jt.flags["enable_gather_reduce"] = False
+            try:
+                l2 = jt.executor_stats["launches"]
+                yp = jt.pool(v, 3, op, 1, 2)
+                jt.sync([yp])
+                assert jt.executor_stats["launches"] - l2 > l1 - l0            # the window tensor costs a launch of its own
+                plain = yp.float32().data
+            finally:
+                jt.flags["enable_gather_reduce"] = True
+            # a 16-bit mean is rounded after a float32 sum whose order differs between the two paths
+            tol = 1e-5 if dtype == "float32" else 2.0 ** -7
+            assert np.array_equal(fused, plain) if op == "maximum" else np.allclose(fused, plain, rtol=tol, atol=tol * 1e-1)
