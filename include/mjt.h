@@ -169,7 +169,10 @@ int mjt_reindex_then_reduce(const mjt_tensor* x, const mjt_tensor* yshape, const
  * ops[] is FusedOp::ops in topological order. */
 typedef enum {
     MJT_VAR_INPUT = 0, MJT_VAR_INTERMEDIATE = 1, MJT_VAR_OUTPUT = 2,
-    MJT_VAR_SCALAR = 3
+    MJT_VAR_SCALAR = 3,
+    /* mjt_fused_reindex_reduce only: a tensor of the scatter target's shape read through the scatter's own index
+     * program (the reindex of the forward pass, recomputed instead of stored) */
+    MJT_VAR_GATHERED = 4
 } mjt_var_role;
 
 typedef struct {
@@ -218,6 +221,20 @@ int mjt_fused_elementwise(const mjt_fused_desc* desc);
  * mjt_fused_elementwise followed by mjt_reduce.  y, op and reduce_mask as in
  * mjt_reduce. */
 int mjt_fused_reduce(const mjt_fused_desc* desc, const mjt_tensor* y, int op, uint32_t reduce_mask);
+
+/* A fused group that ends in a ReindexReduceOp (element, broadcast, reindex and
+ * reduce-type ops share a group in the reference, executor.cc:555; this is the
+ * gradient of pooling, python/jittor/pool.py:200-208 differentiated): `desc`
+ * describes the element-wise part over the shape of the scatter's input y and
+ * has exactly one output var -- that input, never written to memory.  Tensor
+ * inputs have y's shape or are broadcast along the axes of their bcast_mask;
+ * MJT_VAR_GATHERED inputs have x's shape and are read at the element the
+ * scatter's index program points to.  x, op and the index program as in
+ * mjt_reindex_reduce (x's dtype is the output var's). */
+int mjt_fused_reindex_reduce(const mjt_fused_desc* desc, const mjt_tensor* x, int op,
+                             int n_indexes, const char* const* indexes,
+                             int n_overflow_conditions, const char* const* overflow_conditions,
+                             int n_extras, const mjt_tensor* extras);
 
 /* ---- meta-op convolution ----------------------------------------------
  * The group reindex + broadcast + multiply + reduce.add that

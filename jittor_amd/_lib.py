@@ -37,7 +37,7 @@ OP_CODE = {n: i for i, n in enumerate(OPS)}
 BINARY_OPS = OPS[:24]
 UNARY_OPS = OPS[24:53]
 
-VAR_INPUT, VAR_INTERMEDIATE, VAR_OUTPUT, VAR_SCALAR = 0, 1, 2, 3
+VAR_INPUT, VAR_INTERMEDIATE, VAR_OUTPUT, VAR_SCALAR, VAR_GATHERED = 0, 1, 2, 3, 4
 FOP_UNARY, FOP_BINARY, FOP_TERNARY, FOP_BROADCAST = 0, 1, 2, 3
 ERR_INVALID, ERR_UNSUPPORTED, ERR_COMPILE, ERR_DEVICE, ERR_NOT_INIT = -1, -2, -3, -4, -5     # mjt_status
 
@@ -91,7 +91,7 @@ EXPORTS = ["mjt_init", "mjt_shutdown", "mjt_last_error", "mjt_get_device_info",
            "mjt_alloc", "mjt_free", "mjt_h2d", "mjt_d2h", "mjt_d2d", "mjt_fill_u32",
            "mjt_sync", "mjt_event_create", "mjt_event_record", "mjt_event_elapsed_ms",
            "mjt_event_destroy", "mjt_reduce", "mjt_reindex", "mjt_reindex_reduce",
-           "mjt_fused_elementwise", "mjt_fused_reduce", "mjt_conv2d_meta", "mjt_conv2d_meta_grouped", "mjt_conv2d_meta_wgrad", "mjt_reindex_then_reduce", "mjt_matmul", "mjt_matmul_available",
+           "mjt_fused_elementwise", "mjt_fused_reduce", "mjt_conv2d_meta", "mjt_conv2d_meta_grouped", "mjt_conv2d_meta_wgrad", "mjt_reindex_then_reduce", "mjt_fused_reindex_reduce", "mjt_matmul", "mjt_matmul_available",
            "mjt_expr_affine",
            "mjt_jit_stats", "mjt_last_kernel"]
 
@@ -133,6 +133,8 @@ def load():
     lib.mjt_reindex_then_reduce.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.c_int,
                                             ctypes.c_int, ctypes.c_int, strs, ctypes.c_double, ctypes.c_int, strs, ctypes.c_int,
                                             ctypes.POINTER(Tensor)]
+    lib.mjt_fused_reindex_reduce.argtypes = [ctypes.POINTER(FusedDesc), ctypes.POINTER(Tensor), ctypes.c_int, ctypes.c_int, strs,
+                                             ctypes.c_int, strs, ctypes.c_int, ctypes.POINTER(Tensor)]
     lib.mjt_fused_elementwise.argtypes = [ctypes.POINTER(FusedDesc)]
     lib.mjt_fused_reduce.argtypes = [ctypes.POINTER(FusedDesc), ctypes.POINTER(Tensor), ctypes.c_int, ctypes.c_uint32]
     lib.mjt_conv2d_meta.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.POINTER(Tensor),

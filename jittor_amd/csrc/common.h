@@ -102,7 +102,8 @@ void jit_launch(JitKernel* k, unsigned grid_x, unsigned grid_y, unsigned block, 
 const char* embedded_source(const char* name);
 
 // shared by the fused element-wise group and the reduce with an element-wise prologue (op_fused.cpp)
-int64_t fused_validate(const mjt_fused_desc* d, std::vector<int>* inputs, bool outputs_need_data);   // returns the element count
+int64_t fused_validate(const mjt_fused_desc* d, std::vector<int>* inputs, bool outputs_need_data,
+                       bool allow_gathered = false);   // returns the element count
 std::string fused_emit_ops(const mjt_fused_desc* d, bool store_outputs);
 
 // plan cache: per entry point, a string key maps to a prepared plan object

@@ -12,6 +12,9 @@
 //   MJT_RX_LASTVAR  name of the innermost coordinate (iN)
 //   MJT_RX_INDEX    per element: xid0.., flat xid, bool ov_
 //   ATOMIC_UPDATE(addr, v)   scatter only
+//   SC_PROLOGUE, MJT_SC_SCALARS, MJT_SC_VALUE   scatter with an element-wise prologue: by-value scalars, and the
+//                   statements that compute the scattered value `val_` of element e_ (coordinates i0..) from the
+//                   group's inputs
 //
 // The loop runs over y: the output of a gather, the input of a scatter.  Each
 // lane owns VEC adjacent elements of y's innermost axis so that y moves as
@@ -64,14 +67,26 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const index_t e = j * VEC;
     MJT_RX_DECODE
     mjt_pack<TX, VEC> yv;
-#if SCATTER
+#if SCATTER && SC_PROLOGUE
+    MJT_SC_SCALARS
+    (void)yp;
+#elif SCATTER
     mjt_load(yv, yp + e);
 #endif
 #pragma unroll
     for (int k = 0; k < VEC; k++) {
         const index_t MJT_RX_LASTVAR = ilast_ + k;
         MJT_RX_INDEX
-#if SCATTER
+#if SCATTER && SC_PROLOGUE
+        // the scattered value is computed here from the group's inputs (MJT_SC_VALUE leaves it in val_): only for
+        // elements that land somewhere, so a gathered input is always read inside its tensor
+        if (!ov_) {
+            const index_t e_ = e + k;
+            (void)e_;
+            MJT_SC_VALUE
+            ATOMIC_UPDATE(xp + xid, val_);
+        }
+#elif SCATTER
         if (!ov_) { ATOMIC_UPDATE(xp + xid, yv.v[k]); }
 #else
         if (ov_) yv.v[k] = ovalue_; else yv.v[k] = xp[xid];

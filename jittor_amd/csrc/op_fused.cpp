@@ -29,7 +29,7 @@ std::string vname(int i) { return "v" + std::to_string(i); }
 
 }  // namespace
 
-int64_t fused_validate(const mjt_fused_desc* d, std::vector<int>* inputs_out, bool outputs_need_data) {
+int64_t fused_validate(const mjt_fused_desc* d, std::vector<int>* inputs_out, bool outputs_need_data, bool allow_gathered) {
     MJT_CHECK(d, "fused: null descriptor");
     MJT_CHECK(d->ndim >= 1 && d->ndim <= MJT_MAX_DIM, "fused: rank " << d->ndim);
     MJT_CHECK(d->n_vars > 0 && d->n_ops > 0 && d->vars && d->ops, "fused: empty group");
@@ -45,7 +45,12 @@ int64_t fused_validate(const mjt_fused_desc* d, std::vector<int>* inputs_out, bo
     for (int i = 0; i < nv; i++) {
         const mjt_fused_var& v = d->vars[i];
         dtype_size(v.dtype);
-        MJT_CHECK(v.role >= MJT_VAR_INPUT && v.role <= MJT_VAR_SCALAR, "fused: var " << i << " has role " << v.role);
+        MJT_CHECK(v.role >= MJT_VAR_INPUT && v.role <= (allow_gathered ? MJT_VAR_GATHERED : MJT_VAR_SCALAR),
+                  "fused: var " << i << " has role " << v.role);
+        if (v.role == MJT_VAR_GATHERED) {
+            MJT_CHECK(total == 0 || v.ptr, "fused: gathered var " << i << " has no data");
+            defined[i] = 1;
+        }
         if (v.role == MJT_VAR_INPUT) {
             MJT_CHECK(total == 0 || v.ptr, "fused: input var " << i << " has no data");
             MJT_CHECK((v.bcast_mask >> d->ndim) == 0, "fused: bcast_mask of var " << i << " exceeds the rank");

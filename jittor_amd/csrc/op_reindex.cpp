@@ -9,6 +9,7 @@
 // kernels (sliding-window gather, one-axis scatter with LDS-privatised bins)
 // and otherwise uses the generic kernel with the expressions pasted in.
 #include "common.h"
+#include <functional>
 #include "expr.h"
 #include <mutex>
 #include <unordered_map>
@@ -98,9 +99,19 @@ int pick_vec(int elem_size, int64_t last, const void* p) {
 }
 
 // Specialises (once per plan and variant) and launches the generic kernel.
+// An element-wise prologue of a scatter: the parameter words it needs, a key, and the macro definitions
+// (SC_PROLOGUE 1, MJT_SC_SCALARS, MJT_SC_VALUE) given the index of its first parameter word.
+struct ScatterPrologue {
+    std::vector<uint64_t> args;
+    std::string key;
+    std::function<std::string(int)> defs;
+};
+
 // With z: the gather is fused with a reduce (rop) over y's last nred axes; y then only gives the loop shape.
+// With sp (scatter only): y's values are computed by the prologue, y gives the loop shape and dtype.
 void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mjt_tensor* y, double overflow_value,
-                 int n_ex, const mjt_tensor* ex, const mjt_tensor* z = nullptr, int rop = 0, int nred = 0) {
+                 int n_ex, const mjt_tensor* ex, const mjt_tensor* z = nullptr, int rop = 0, int nred = 0,
+                 const ScatterPrologue* sp = nullptr) {
     // the loop runs over y (gather output / scatter input)
     const int LD = y->ndim, XD = x->ndim;
     int64_t yn = numel(y), xn = numel(x);
@@ -108,7 +119,7 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
     int64_t biggest = std::max(xn, yn);
     for (int i = 0; i < n_ex; i++) biggest = std::max(biggest, numel(&ex[i]));
     bool use64 = biggest >= (int64_t(1) << 31);   // index_t rule of op.cc:158-192
-    int vec = z ? 1 : pick_vec(dtype_size(x->dtype), y->shape[LD - 1], y->ptr);
+    int vec = z || sp ? 1 : pick_vec(dtype_size(x->dtype), y->shape[LD - 1], y->ptr);
     int64_t rtail = 1;
     for (int i = LD - nred; z && i < LD; i++) rtail *= y->shape[i];
 
@@ -135,7 +146,13 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
         args.push_back((uint64_t)rtail);
         args.push_back(bits_of(rtail ? 1.0 / (double)rtail : 0.0));
     }
+    int p_sp = 0;
+    if (sp) {
+        p_sp = (int)args.size();
+        args.insert(args.end(), sp->args.begin(), sp->args.end());
+    }
     std::string vkey = std::to_string(vec) + (use64 ? "L" : "I");
+    if (sp) vkey += "|P" + sp->key;
     if (z) vkey += "|R" + std::to_string(rop) + "," + std::to_string(z->dtype) + "," + std::to_string(nred);
     JitKernel* kern = nullptr;
     {
@@ -197,6 +214,8 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
         frag << "#define MJT_RX_INDEX " << index.str() << "\n";
         if (scatter) frag << "#define ATOMIC_UPDATE(addr, v) mjt_atomic_" << mjt_op_name(op) << "<TX>((addr), (v))\n";
         frag << "#define REDUCE_TAIL " << (z ? 1 : 0) << "\n";
+        if (sp) frag << sp->defs(p_sp);
+        else frag << "#define SC_PROLOGUE 0\n";
         if (z) {
             // accumulator as in the reduce kernels: z's type, float for 16-bit float results
             const int ta = z->dtype == MJT_FLOAT16 || z->dtype == MJT_BFLOAT16 ? MJT_FLOAT32 : z->dtype;
@@ -332,6 +351,96 @@ void reindex_then_reduce_impl(const mjt_tensor* x, const mjt_tensor* yshape, con
     run_generic(plan, false, 0, x, &y, overflow_value, n_ex, ex, z, rop, nred);
 }
 
+// reindex_reduce whose input is computed by an element-wise group (desc: the group over y's shape, one output var)
+void fused_reindex_reduce_impl(const mjt_fused_desc* d, const mjt_tensor* x, int op, int n_idx, const char* const* idx, int n_ofc,
+                               const char* const* ofc, int n_ex, const mjt_tensor* ex) {
+    require_init();
+    check_tensor(x, "fused reindex_reduce x");
+    check_extras(n_ex, ex);
+    std::vector<int> inputs;
+    fused_validate(d, &inputs, false, true);
+    int out = -1;
+    for (int i = 0; i < d->n_vars; i++)
+        if (d->vars[i].role == MJT_VAR_OUTPUT) {
+            MJT_CHECK(out < 0, "fused reindex_reduce: the group must have exactly one output var (the scattered values)");
+            out = i;
+        }
+    MJT_CHECK(out >= 0, "fused reindex_reduce: the group has no output var");
+    MJT_CHECK((op >= MJT_OP_POW && op < MJT_OP_MEAN) || op == MJT_OP_VOID,
+              "reindex_reduce: op must be a binary op other than mean, or void");
+    MJT_CHECK(n_idx == x->ndim, "Number of shape and indexes should be the same. (shape rank " << x->ndim << ", " << n_idx << " indexes)");
+    MJT_CHECK(n_idx == 0 || idx, "null indexes");
+    MJT_CHECK(n_ofc >= 0 && (n_ofc == 0 || ofc), "null overflow conditions");
+    MJT_CHECK(d->vars[out].dtype == x->dtype, "fused reindex_reduce: x dtype must equal the group's output dtype");
+    mjt_tensor y{};                                   // the virtual scatter input
+    y.ptr = x->ptr;                                   // never dereferenced
+    y.dtype = x->dtype;
+    y.ndim = d->ndim;
+    for (int i = 0; i < d->ndim; i++) y.shape[i] = d->shape[i];
+    std::string key = plan_key(true, op, x, &y, n_idx, idx, n_ofc, ofc, n_ex, ex);
+    Plan* plan = get_plan(key, x, &y, y.ndim, n_idx, idx, n_ofc, ofc, n_ex, ex);
+    const int64_t xn = numel(x);
+    if (xn == 0) return;
+    launch_fill_pattern(x->ptr, op == MJT_OP_VOID ? 0 : identity_bits(op, x->dtype), dtype_size(x->dtype), (size_t)xn);
+    if (numel(&y) == 0) return;
+
+    ScatterPrologue sp;
+    std::ostringstream key2;
+    std::vector<int> slot(d->n_vars, -1);
+    for (int i = 0; i < d->n_vars; i++) {
+        const mjt_fused_var& fv = d->vars[i];
+        key2 << fv.role << ":" << fv.dtype << ":" << fv.bcast_mask << ";";
+        if (fv.role == MJT_VAR_INPUT || fv.role == MJT_VAR_GATHERED) {
+            slot[i] = (int)sp.args.size();
+            sp.args.push_back(bits_of_ptr(fv.ptr));
+        } else if (fv.role == MJT_VAR_SCALAR) {
+            slot[i] = (int)sp.args.size();
+            sp.args.push_back(dtype_is_float(fv.dtype) ? bits_of(fv.fvalue) : (uint64_t)fv.ivalue);
+        }
+    }
+    for (int k = 0; k < d->n_ops; k++) {
+        const mjt_fused_op& o = d->ops[k];
+        key2 << o.kind << ":" << o.op << ":" << o.in[0] << ":" << (o.kind >= MJT_FOP_BINARY ? o.in[1] : -1) << ":"
+             << (o.kind == MJT_FOP_TERNARY ? o.in[2] : -1) << ">" << o.out << ";";
+    }
+    sp.key = key2.str();
+    sp.defs = [d, slot, out](int base) {
+        std::ostringstream scal, val;
+        for (int i = 0; i < d->n_vars; i++) {
+            const mjt_fused_var& fv = d->vars[i];
+            const char* T = dtype_cname(fv.dtype);
+            if (fv.role == MJT_VAR_SCALAR) {
+                if (dtype_is_float(fv.dtype))
+                    scal << "const " << T << " v" << i << " = (" << T << ")__longlong_as_double((long long)(unsigned long long)p.a["
+                         << base + slot[i] << "]); ";
+                else
+                    scal << "const " << T << " v" << i << " = (" << T << ")(long long)(unsigned long long)p.a[" << base + slot[i] << "]; ";
+            } else if (fv.role == MJT_VAR_GATHERED) {
+                val << "const " << T << " v" << i << " = ((const " << T << "*)p.a[" << base + slot[i] << "])[xid]; ";
+            } else if (fv.role == MJT_VAR_INPUT) {
+                // offset inside a tensor that has extent 1 along the axes of its mask: Horner over the other axes
+                std::string off = "(index_t)0";
+                bool full = true;
+                for (int a = 0; a < d->ndim; a++)
+                    if ((fv.bcast_mask >> a & 1) && d->shape[a] != 1) full = false;
+                if (full) {
+                    off = "e_";
+                } else {
+                    for (int a = 0; a < d->ndim; a++)
+                        if (!(fv.bcast_mask >> a & 1) && d->shape[a] != 1)
+                            off = "(" + off + " * yshape" + std::to_string(a) + " + i" + std::to_string(a) + ")";
+                }
+                val << "const " << T << " v" << i << " = ((const " << T << "*)p.a[" << base + slot[i] << "])[" << off << "]; ";
+            }
+        }
+        std::ostringstream defs;
+        defs << "#define SC_PROLOGUE 1\n#define MJT_SC_SCALARS " << scal.str() << "\n#define MJT_SC_VALUE " << val.str()
+             << fused_emit_ops(d, false) << "const TX val_ = (TX)(v" << out << ");\n";
+        return defs.str();
+    };
+    run_generic(plan, true, op, x, &y, 0.0, n_ex, ex, nullptr, 0, 0, &sp);
+}
+
 void reindex_reduce_impl(const mjt_tensor* y, const mjt_tensor* x, int op, int n_idx, const char* const* idx, int n_ofc,
                          const char* const* ofc, int n_ex, const mjt_tensor* ex) {
     require_init();
@@ -376,6 +485,14 @@ extern "C" int mjt_reindex_then_reduce(const mjt_tensor* x, const mjt_tensor* ys
     return mjt::guarded([&] {
         mjt::reindex_then_reduce_impl(x, yshape, z, op, n_reduced, n_indexes, indexes, overflow_value, n_overflow_conditions,
                                       overflow_conditions, n_extras, extras);
+    });
+}
+
+extern "C" int mjt_fused_reindex_reduce(const mjt_fused_desc* desc, const mjt_tensor* x, int op, int n_indexes,
+                                        const char* const* indexes, int n_overflow_conditions,
+                                        const char* const* overflow_conditions, int n_extras, const mjt_tensor* extras) {
+    return mjt::guarded([&] {
+        mjt::fused_reindex_reduce_impl(desc, x, op, n_indexes, indexes, n_overflow_conditions, overflow_conditions, n_extras, extras);
     });
 }
 

@@ -19,7 +19,7 @@ from . import profiler as _profiler
 from .flags import flags
 
 stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0, "matmul_matches": 0,
-         "wgrad_kernel": 0, "gather_reduces": 0}
+         "wgrad_kernel": 0, "gather_reduces": 0, "fused_scatters": 0}
 
 
 class ConvUnit:
@@ -351,19 +351,21 @@ def _match_conv_grouped(op):
 
 
 def _match_gather_reduce(red, consumers, target_ids):
-    """reduce(op) over the trailing axes of a reindex result nobody else reads."""
+    """reduce(op) over the trailing axes of a reindex result."""
     if red.op not in ("add", "mean", "maximum", "minimum", "multiply"):
         return None
     xx, absorbed = red.inputs[0], {red.id}
     if not xx.materialised and isinstance(xx._op, UnaryOp) and xx._op.op == "cast" and xx.dtype == "float32" \
             and xx._op.inputs[0].dtype in ("float16", "bfloat16"):
         # a 16-bit sum or mean was rewritten to cast -> reduce(float32) -> cast: the kernel accumulates in float32 anyway
-        if xx.id in target_ids or len(consumers.get(xx.id, ())) != 1:
+        if xx.id in target_ids:
             return None
         absorbed.add(xx._op.id)
         xx = xx._op.inputs[0]
     ro = _lazy_op(xx, ReindexOp)
-    if ro is None or xx.id in target_ids or len(consumers.get(xx.id, ())) != 1 or getattr(xx, "_stop_fuse", False):
+    # other readers of the reindex result do not matter: the unit reads the reindex's own input, and the reindex
+    # itself still runs if somebody needs its result in memory
+    if ro is None or xx.id in target_ids or getattr(xx, "_stop_fuse", False):
         return None
     nd, nred = xx.ndim, bin(red.reduce_mask).count("1")
     if nred < 1 or red.reduce_mask != ((1 << nred) - 1) << (nd - nred) or red.out.dtype == "bool":
@@ -639,6 +641,40 @@ def _execute(ops, target_ids):
                 continue
             prologue_of[users[0].id] = members
             absorbed_groups.add(id(members))
+    # a group whose single result is what one reindex_reduce of the same stage scatters becomes that scatter's
+    # prologue; a reindex with the scatter's own index program whose result only the group reads (the forward
+    # pass's window tensor in a pooling gradient) is read through that program instead of being computed
+    scatter_of, absorbed_nodes = {}, set()
+    if flags["enable_scatter_fusion"]:
+        for members in (m for st in by_stage_groups for m in st):
+            if id(members) in absorbed_groups:
+                continue
+            ids = {op.id for op in members}
+            outs = [op.out for op in members
+                    if op.out.id in target_ids or any(c.id not in ids for c in consumers.get(op.out.id, ()))]
+            if len(outs) != 1 or outs[0].id in target_ids:
+                continue
+            users = consumers.get(outs[0].id, ())
+            if len(users) != 1 or not isinstance(users[0], ReindexReduceOp) or users[0].id in scatter_of:
+                continue
+            rr = users[0]
+            if stage[rr.id] != stage[members[0].id] or outs[0].shape != members[-1].out.shape or rr.inputs[0].id != outs[0].id \
+                    or any(e.id == outs[0].id for e in rr.inputs[1:]):
+                continue
+            gathered = {}
+            for op in members:
+                for u in op.inputs:
+                    p = producer.get(u.id)
+                    if isinstance(p, ReindexOp) and p.id not in ids and u._buf is None and u.id not in target_ids \
+                            and p.indexes == rr.indexes and p.overflow_conditions == rr.overflow_conditions \
+                            and [e.id for e in p.inputs[1:]] == [e.id for e in rr.inputs[1:]] \
+                            and list(p.inputs[0].shape) == list(rr.out.shape) and not isinstance(op, BroadcastOp) \
+                            and all(c.id in ids for c in consumers.get(u.id, ())):
+                        gathered[u.id] = p
+            scatter_of[rr.id] = (members, gathered)
+            absorbed_groups.add(id(members))
+            absorbed_nodes.update(p.id for p in gathered.values())
+
     def group_io(members, extra_out=None):
         ids = {op.id for op in members}
         made = {op.out.id for op in members}
@@ -660,6 +696,16 @@ def _execute(ops, target_ids):
             if id(members) not in absorbed_groups:
                 timed(lambda: _run_group(members, consumers, target_ids, pre=pre), "fused", lambda: group_io(members))
         for op in by_stage_other[s]:
+            if op.id in absorbed_nodes:
+                continue
+            sc = scatter_of.get(op.id)
+            if sc is not None:
+                if timed(lambda: _run_group(sc[0], consumers, target_ids, scatter=op, gathered=sc[1], pre=pre), "fused+scatter",
+                         lambda: group_io(sc[0], op.out)):
+                    continue
+                for p in sc[1].values():                       # not taken in that form: the plain sequence
+                    timed(lambda: _run_single(p), p.kind, lambda: (sum(u.nbytes for u in p.inputs), p.out.nbytes))
+                timed(lambda: _run_group(sc[0], consumers, target_ids, pre=pre), "fused", lambda: group_io(sc[0]))
             members = prologue_of.get(op.id)
             if members is not None:
                 if timed(lambda: _run_group(members, consumers, target_ids, reduce=op, pre=pre), "fused+reduce",
@@ -830,7 +876,7 @@ def _run_single(op):
         raise MjtError(-2, "no kernel for op %r" % (op,))
 
 
-def _run_group(members, consumers, target_ids, reduce=None, pre=None):
+def _run_group(members, consumers, target_ids, reduce=None, pre=None, scatter=None, gathered=None):
     """One launch for a group of element / broadcast ops.  With `reduce` (the ReduceOp that consumes the
     group's only result) the group runs as that reduce's prologue; returns False when the library does
     not take the group in that form (a tensor broadcast inside it), True otherwise."""
@@ -852,6 +898,10 @@ def _run_group(members, consumers, target_ids, reduce=None, pre=None):
         key = (u.id, mask)
         if key in index:
             return index[key]
+        if gathered and u.id in gathered:
+            i = add_var(_lib.VAR_GATHERED, u.dtype, ptr=gathered[u.id].inputs[0]._device_ptr())
+            index[key] = i
+            return i
         if u._op is None and u._host is not None and u.num == 1:
             # one-element host array: by-value kernel argument (ops/array_op.cc:56-60)
             h = u._host.reshape(-1)[0]
@@ -911,7 +961,7 @@ def _run_group(members, consumers, target_ids, reduce=None, pre=None):
         out = op.out
         used_outside = out.id in target_ids or any(c.id not in member_ids for c in consumers.get(out.id, ()))
         if used_outside:
-            oi = add_var(_lib.VAR_OUTPUT, out.dtype, ptr=None if reduce is not None else _alloc_out(out))
+            oi = add_var(_lib.VAR_OUTPUT, out.dtype, ptr=None if reduce is not None or scatter is not None else _alloc_out(out))
             outputs.append(out)
         else:
             oi = add_var(_lib.VAR_INTERMEDIATE, out.dtype)
@@ -926,6 +976,22 @@ def _run_group(members, consumers, target_ids, reduce=None, pre=None):
     varr = (_lib.FusedVar * len(fvars))(*fvars)
     oarr = (_lib.FusedOp * len(fops))(*fops)
     desc.n_vars, desc.vars, desc.n_ops, desc.ops = len(fvars), varr, len(fops), oarr
+    if scatter is not None:
+        rout, extras = scatter.out, scatter.inputs[1:]
+        had_buf = rout._buf is not None
+        tx = _lib.tensor(_alloc_out(rout), rout.dtype, rout.shape)
+        ex = (_lib.Tensor * max(1, len(extras)))(*[_tensor_of(e) for e in extras])
+        rc = lib.mjt_fused_reindex_reduce(ctypes.byref(desc), ctypes.byref(tx), _lib.OP_CODE[scatter.op], len(scatter.indexes),
+                                          _lib.c_strings(scatter.indexes), len(scatter.overflow_conditions),
+                                          _lib.c_strings(scatter.overflow_conditions), len(extras), ex)
+        if rc == _lib.ERR_UNSUPPORTED:
+            if not had_buf:
+                rout._buf = None
+            return False
+        _lib.check(rc)
+        stats["launches"] += 1
+        stats["fused_scatters"] += 1
+        return True
     if reduce is not None:
         rout = reduce.out
         had_buf = rout._buf is not None

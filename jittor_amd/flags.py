@@ -46,7 +46,7 @@ class Flags(dict):
 
 flags = Flags()
 for _name, _value in (("enable_conv_match", True), ("enable_reduce_fusion", True), ("enable_broadcast_sink", True),
-                      ("enable_matmul_match", True), ("enable_conv_wgrad_kernel", True), ("enable_gather_reduce", True), ("auto_mixed_precision_level", 0)):
+                      ("enable_matmul_match", True), ("enable_conv_wgrad_kernel", True), ("enable_gather_reduce", True), ("enable_scatter_fusion", True), ("auto_mixed_precision_level", 0)):
     dict.__setitem__(flags, _name, _value)
 
 

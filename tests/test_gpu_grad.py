@@ -273,3 +273,45 @@ def test_grad_grouped_conv(gpu):
         dX, dW = _conv_grads_ref(x[:, g * cg:(g + 1) * cg], w[g * kg:(g + 1) * kg], r[:, g * kg:(g + 1) * kg], 1, 1, 1)
         close(gx.numpy()[:, g * cg:(g + 1) * cg], dX, rtol=1e-4, atol=1e-4)
         close(gw.numpy()[g * kg:(g + 1) * kg], dW, rtol=1e-4, atol=1e-4)
+
+
+def test_pooling_forward_and_backward_keep_rank_six_out_of_memory(gpu):
+    """Pooling and its gradient run without the rank-6 window tensors ever being written (the invariant of
+    test_longest_dis_fuse.py:51-66): forward = reindex fused with its reduce, backward = the element-wise group
+    (equal / ternary over the window tensor, recomputed through the scatter's index program) fused into the
+    scatter.  Values against the plain path and closed forms."""
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((2, 3, 9, 10)).astype(np.float32)
+    for op in ("maximum", "mean"):
+        results = {}
+        for fused in (True, False):
+            jt.flags["enable_gather_reduce"] = jt.flags["enable_scatter_fusion"] = fused
+            try:
+                vx = jt.array(x)
+                y = jt.pool(vx, 3, op, 1, 2)
+                r = jt.array(rng.standard_normal(y.shape).astype(np.float32)) if "r" not in results else results["r"]
+                results["r"] = r
+                g = jt.grad((y * r).sum(), vx)
+                before = dict(jt.executor_stats)
+                jt.sync([y, g])
+                results[fused] = (y.numpy(), g.numpy())
+                if fused:
+                    assert jt.executor_stats["fused_scatters"] == before["fused_scatters"] + 1
+                    seen, stack = set(), [y, g]
+                    while stack:                                       # nothing of rank 6 has memory
+                        v = stack.pop()
+                        if v.id in seen:
+                            continue
+                        seen.add(v.id)
+                        assert not (v.ndim == 6 and v._buf is not None)
+                        if v._history is not None:
+                            stack.extend(v._history[1])
+            finally:
+                jt.flags["enable_gather_reduce"] = jt.flags["enable_scatter_fusion"] = True
+        close(results[True][0], results[False][0], rtol=1e-6, atol=1e-6)
+        close(results[True][1], results[False][1], rtol=1e-5, atol=1e-6)
+    # mean pooling without padding: every input element gets r / 9 from each window that covers it
+    xs = rng.standard_normal((1, 2, 6, 6)).astype(np.float32)
+    vx = jt.array(xs)
+    g = jt.grad(jt.pool(vx, 3, "mean", 0, 3).sum(), vx)
+    close(g.numpy(), np.full(xs.shape, 1.0 / 9, np.float32))

@@ -952,3 +952,46 @@ def test_gather_fused_with_reduce(gpu):
             # a 16-bit mean is rounded after a float32 sum whose order differs between the two paths
             tol = 1e-5 if dtype == "float32" else 2.0 ** -7
             assert np.array_equal(fused, plain) if op == "maximum" else np.allclose(fused, plain, rtol=tol, atol=tol * 1e-1)
+
+
+def test_scatter_with_element_wise_prologue(gpu):
+    """mjt_fused_reindex_reduce through the C entry point: the scattered values are computed in the kernel from a
+    full-shape tensor, a tensor broadcast along the window axes, a scalar, and a tensor read through the scatter's
+    own index program; against the oracle's reindex / element-wise / reindex_reduce chain."""
+    rng = np.random.default_rng(61)
+    lib = L.load()
+    xshape, yshape = [2, 3, 8, 9], [2, 3, 4, 4, 3, 3]
+    idx = ["i0", "i1", "i2*2-1+i4", "i3*2-0+i5"]
+    src = rng.standard_normal(xshape).astype(np.float32)          # read through the index program
+    full = rng.standard_normal(yshape).astype(np.float32)
+    small = rng.standard_normal(yshape[:4] + [1, 1]).astype(np.float32)
+    # value = (gathered(src) * full + small) * 0.5
+    want_y = (O.reindex(src, yshape, idx, 0.0) * full + small) * np.float32(0.5)
+    want = O.reindex_reduce(want_y.astype(np.float32), "add", xshape, idx)
+    vs, vf, vm, vx = jt.from_storage(src, "float32"), jt.from_storage(full, "float32"), jt.from_storage(small, "float32"), jt.zeros(xshape)
+    V, F = L.FusedVar, L.FusedOp
+    spec = [(L.VAR_GATHERED, vs.raw_ptr(), 0, 0.0), (L.VAR_INPUT, vf.raw_ptr(), 0, 0.0), (L.VAR_INPUT, vm.raw_ptr(), 0b110000, 0.0),
+            (L.VAR_SCALAR, None, 0, 0.5), (L.VAR_INTERMEDIATE, None, 0, 0.0), (L.VAR_INTERMEDIATE, None, 0, 0.0),
+            (L.VAR_OUTPUT, None, 0, 0.0)]
+    va = (V * len(spec))()
+    for i, (role, ptr, mask, f) in enumerate(spec):
+        va[i].role, va[i].dtype, va[i].ptr, va[i].bcast_mask, va[i].fvalue = role, L.DTYPE_CODE["float32"], ptr, mask, f
+    ops = [("multiply", [0, 1], 4), ("add", [4, 2], 5), ("multiply", [5, 3], 6)]
+    oa = (F * len(ops))()
+    for i, (name, ins, out) in enumerate(ops):
+        oa[i].kind, oa[i].op, oa[i].out = L.FOP_BINARY, L.OP_CODE[name], out
+        for j, v in enumerate(ins):
+            oa[i].inp[j] = v
+    d = L.FusedDesc()
+    d.ndim = len(yshape)
+    for i, s_ in enumerate(yshape):
+        d.shape[i] = s_
+    d.n_vars, d.vars, d.n_ops, d.ops = len(spec), va, len(ops), oa
+    tx = L.tensor(vx.raw_ptr(), "float32", xshape)
+    L.check(lib.mjt_fused_reindex_reduce(ctypes.byref(d), ctypes.byref(tx), L.OP_CODE["add"], 4, L.c_strings(idx), 0, L.c_strings([]),
+                                         0, (L.Tensor * 1)()))
+    assert L.last_kernel().startswith("mjt_reindex_reduce_add_")
+    got = L.d2h(vx.raw_ptr(), xshape, np.float32)
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-5)
+    # a gathered var is refused where it has no meaning
+    assert lib.mjt_fused_elementwise(ctypes.byref(d)) < 0 and "role" in lib.mjt_last_error().decode()
