@@ -370,6 +370,11 @@ def _match_gather_reduce(red, consumers, target_ids):
     nd, nred = xx.ndim, bin(red.reduce_mask).count("1")
     if nred < 1 or red.reduce_mask != ((1 << nred) - 1) << (nd - nred) or red.out.dtype == "bool":
         return None
+    tail = 1
+    for n in xx.shape[nd - nred:]:
+        tail *= n
+    if tail > 128:
+        return None            # one lane walks the folded elements: beyond a pooling window the two-kernel path is faster
     absorbed.add(ro.id)
     return GatherReduceUnit(red, ro, nred, absorbed)
 
