@@ -315,3 +315,47 @@ def test_pooling_forward_and_backward_keep_rank_six_out_of_memory(gpu):
     vx = jt.array(xs)
     g = jt.grad(jt.pool(vx, 3, "mean", 0, 3).sum(), vx)
     close(g.numpy(), np.full(xs.shape, 1.0 / 9, np.float32))
+
+
+def test_small_cnn_step_with_and_without_the_executor_rewrites(gpu):
+    """One training step of a small CNN (conv, relu, max pool, strided conv, global mean, linear, softmax
+    cross-entropy): loss and all gradients with every executor rewrite on (convolution units, weight-gradient
+    kernel, matrix products, reduce prologues, broadcast sinking, gather-reduce, scatter prologue) against the same
+    graph run op by op through the generic kernels."""
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal((4, 8, 12, 12)).astype(np.float32)
+    w1 = (rng.standard_normal((16, 8, 3, 3)) * 0.2).astype(np.float32)
+    w2 = (rng.standard_normal((16, 16, 3, 3)) * 0.2).astype(np.float32)
+    wl, bl = (rng.standard_normal((5, 16)) * 0.3).astype(np.float32), rng.standard_normal(5).astype(np.float32)
+    onehot = np.eye(5, dtype=np.float32)[rng.integers(0, 5, 4)]
+    names = ["enable_conv_match", "enable_reduce_fusion", "enable_broadcast_sink", "enable_matmul_match", "enable_conv_wgrad_kernel",
+             "enable_gather_reduce", "enable_scatter_fusion"]
+
+    def step():
+        vx, v1, v2, vl, vb = (jt.array(a) for a in (x, w1, w2, wl, bl))
+        h = jt.nn.relu(jt.nn.conv2d(vx, v1, padding=1))
+        h = jt.nn.max_pool2d(h, 3, 2, 1)
+        h = jt.nn.relu(jt.nn.conv2d(h, v2, stride=2, padding=1))
+        f = h.mean([2, 3])
+        logits = jt.nn.linear(f, vl, vb)
+        m = logits.max([1], keepdims=True)
+        e = jt.unary(logits - m, "exp")
+        logp = logits - m - jt.unary(e.sum([1], keepdims=True), "log")
+        loss = (logp * jt.array(onehot)).sum() * (-1.0 / 4)
+        grads = jt.grad(loss, [vx, v1, v2, vl, vb])
+        jt.sync([loss] + grads)
+        return [loss.numpy()] + [g.numpy() for g in grads]
+
+    fast = step()
+    saved = {n: jt.flags[n] for n in names}
+    try:
+        for n in names:
+            jt.flags[n] = False
+        plain = step()
+    finally:
+        for n, v in saved.items():
+            jt.flags[n] = v
+    for a, b in zip(fast, plain):
+        assert a.shape == b.shape
+        close(a, b, rtol=2e-4, atol=2e-5)
+    assert np.isfinite(fast[0]).all() and float(fast[0][0]) > 0
