@@ -273,6 +273,19 @@ int mjt_conv2d_meta_grouped(const mjt_tensor* x, const mjt_tensor* w, const mjt_
 int mjt_conv2d_meta_wgrad(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw,
                           const mjt_conv_params* p);
 
+/* The same gradient for any geometry and for grouped convolutions
+ * (python/jittor/nn.py:1272-1294: x has `groups` groups of dw->shape[1] channels,
+ * dy `groups` groups of K / groups; the reference's tuner relays the grouped
+ * pattern to the same backward-w library op with a group count,
+ * opt/tuner/conv_tuner.cc:375-397):
+ *   dw[k,c,r,s] = sum_{n,oh,ow} dy[n,k,oh,ow] * x[n,(k/(K/groups))*C+c,oh*sh-ph+r*dh,ow*sw-pw+s*dw]
+ * float32, bfloat16 or float16 operands (float32 products and sums, rounded
+ * once).  With groups == 1 shapes the MFMA kernel covers run on it; everything
+ * else runs on a direct kernel (one workgroup per output channel x up to four
+ * input channels x slice of images, sums kept in registers). */
+int mjt_conv2d_meta_wgrad_grouped(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw,
+                                  const mjt_conv_params* p, int groups);
+
 /* ---- matrix product ---------------------------------------------------
  * c[n,k] = op(a) * op(b) for 2-d float operands of one dtype, op = transpose
  * when the flag is set: the call the reference relays the pattern

@@ -199,8 +199,100 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     jit_launch(k, (unsigned)blocks, 1, 256, 0, a);
 }
 
+// The buffer of per-slice partial weight gradients, grown to `bytes`.
+static void* wgrad_partials(size_t bytes) {
+    Context& c = ctx();
+    if (c.dry_run) return (void*)(uintptr_t)0x1000;
+    if (bytes > g_wgrad_bytes) {
+        if (g_wgrad_part) {
+            HIP_CHECK(hipStreamSynchronize(c.stream));
+            HIP_CHECK(hipFree(g_wgrad_part));
+            g_wgrad_part = nullptr;
+            g_wgrad_bytes = 0;
+        }
+        HIP_CHECK(hipMalloc(&g_wgrad_part, bytes));
+        g_wgrad_bytes = bytes;
+    }
+    return g_wgrad_part;
+}
+
+// [slices, numel(dw)] float partial sums summed over axis 0 into dw, rounded once if dw is a 16-bit type.
+static void fold_wgrad_slices(void* part, int64_t slices, const mjt_tensor* dw) {
+    mjt_tensor tp, td;
+    memset(&tp, 0, sizeof(tp));
+    memset(&td, 0, sizeof(td));
+    tp.ptr = part;
+    tp.dtype = MJT_FLOAT32;
+    tp.ndim = 2;
+    tp.shape[0] = slices;
+    tp.shape[1] = numel(dw);
+    td.ptr = dw->ptr;
+    td.dtype = dw->dtype;
+    td.ndim = 1;
+    td.shape[0] = numel(dw);
+    if (mjt_reduce(&tp, &td, MJT_OP_ADD, 0b01) != MJT_OK) MJT_FAIL(MJT_ERR_DEVICE, "conv wgrad: folding the partial sums failed: " << mjt_last_error());
+}
+
+// The direct weight-gradient kernel (kernels/conv_wgrad_direct.h): any groups, any geometry, float32 / bfloat16 / float16.
+static void conv_wgrad_direct(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw, const mjt_conv_params* p, int64_t G) {
+    const int64_t N = x->shape[0], C = x->shape[1] / G, H = x->shape[2], W = x->shape[3];
+    const int64_t K = dy->shape[1], OH = dy->shape[2], OW = dy->shape[3], R = dw->shape[2], S = dw->shape[3];
+    const bool flt = x->dtype == MJT_FLOAT32 || x->dtype == MJT_BFLOAT16 || x->dtype == MJT_FLOAT16;
+    if (!flt || dy->dtype != x->dtype || !(dw->dtype == MJT_FLOAT32 || dw->dtype == x->dtype))
+        MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: x and dy must share one of float32 / bfloat16 / float16 and dw be of that type or float32");
+    MJT_CHECK(H * W < (int64_t(1) << 31) && OH * OW < (int64_t(1) << 31), "conv wgrad: image too large");
+    if (N == 0 || OH * OW == 0) {                                // a sum over nothing: zeros, written by the reduce kernel
+        fold_wgrad_slices(wgrad_partials(4), 0, dw);
+        return;
+    }
+    const int64_t taps = R * S;
+    const int64_t TCH = taps <= 49 ? taps : 32;
+    int64_t CT = taps <= 49 ? 40 / taps : 1;
+    if (CT > 4) CT = 4;
+    if (CT > C) CT = C;
+    if (CT < 1) CT = 1;
+    const int64_t per_slice = K * ((C + CT - 1) / CT) * ((taps + TCH - 1) / TCH);
+    Context& c = ctx();
+    const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
+    // slices of whole images: about four workgroups per compute unit, at least a thousand positions per slice
+    int64_t slices = (4 * cus + per_slice - 1) / per_slice;
+    if (slices > N * OH * OW / 1024) slices = N * OH * OW / 1024;
+    if (slices > N) slices = N;
+    if (slices < 1) slices = 1;
+    const int64_t ips = (N + slices - 1) / slices;
+    slices = (N + ips - 1) / ips;
+    MJT_CHECK(slices * per_slice < (int64_t(1) << 31), "conv wgrad: launch too large");
+
+    std::ostringstream key;
+    key << "wgrad_direct|" << x->dtype << "|" << C << "|" << H << "|" << W << "|" << K << "|" << R << "|" << S << "|" << OH << "|" << OW << "|"
+        << p->stride_h << "|" << p->stride_w << "|" << p->pad_h << "|" << p->pad_w << "|" << p->dil_h << "|" << p->dil_w << "|" << G << "|" << CT;
+    JitKernel* k = cached(key.str());
+    if (!k) {
+        std::ostringstream name;
+        name << "mjt_conv_wgrad_direct_" << mjt_dtype_name(x->dtype) << "_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s"
+             << p->stride_h << "x" << p->stride_w << "_p" << p->pad_h << "x" << p->pad_w << "_d" << p->dil_h << "x" << p->dil_w << "_g" << G;
+        std::ostringstream src;
+        src << "#define ENTRY " << name.str() << "\n#define TIN " << dtype_cname(x->dtype) << "\n#define C_ " << C << "\n#define H_ " << H
+            << "\n#define W_ " << W << "\n#define K_ " << K << "\n#define R_ " << R << "\n#define S_ " << S << "\n#define OH_ " << OH
+            << "\n#define OW_ " << OW << "\n#define SH " << p->stride_h << "\n#define SW " << p->stride_w << "\n#define PH " << p->pad_h
+            << "\n#define PW " << p->pad_w << "\n#define DH " << p->dil_h << "\n#define DW " << p->dil_w << "\n#define G_ " << G
+            << "\n#define CT " << CT << "\n#define TCH " << TCH << "\n";
+        src << embedded_source("prelude.h") << "\n" << embedded_source("conv_wgrad_direct.h") << "\n";
+        k = jit_get(src.str(), name.str());
+        remember(key.str(), k);
+    }
+    const bool in_place = slices == 1 && dw->dtype == MJT_FLOAT32;       // one slice of float sums is the result
+    void* part = in_place ? dw->ptr : wgrad_partials((size_t)slices * (size_t)numel(dw) * 4);
+    std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(dy->ptr), bits_of_ptr(part), (uint64_t)N, (uint64_t)ips, 0};
+    jit_launch(k, (unsigned)(slices * per_slice), 1, 256, 0, a);
+    if (!in_place) fold_wgrad_slices(part, slices, dw);
+    set_last_kernel(k->name.c_str());
+}
+
 // Weight gradient: dw[k,c,r,s] = sum_{n,oh,ow} dy[n,k,oh,ow] * x[n,c,oh*sh-ph+r*dh,ow*sw-pw+s*dw].
-void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw, const mjt_conv_params* p) {
+// With `any_shape` (the grouped entry point) what the MFMA kernel does not cover runs on the direct kernel instead of
+// being handed back; G > 1: x has G groups of dw->shape[1] channels, dy G groups of K / G (python/jittor/nn.py:1272-1294).
+void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw, const mjt_conv_params* p, int64_t G, bool any_shape) {
     require_init();
     check_tensor(x, "conv wgrad x");
     check_tensor(dy, "conv wgrad dy");
@@ -209,9 +301,12 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
     MJT_CHECK(x->ndim == 4 && dy->ndim == 4 && dw->ndim == 4, "conv wgrad: x, dy and dw must have rank 4");
     MJT_CHECK(p->stride_h >= 1 && p->stride_w >= 1 && p->dil_h >= 1 && p->dil_w >= 1 && p->pad_h >= 0 && p->pad_w >= 0,
               "conv wgrad: bad stride / padding / dilation");
-    const int64_t N = x->shape[0], C = x->shape[1], H = x->shape[2], W = x->shape[3];
+    MJT_CHECK(G >= 1, "conv wgrad: groups must be positive");
+    const int64_t N = x->shape[0], H = x->shape[2], W = x->shape[3];
     const int64_t K = dy->shape[1], OH = dy->shape[2], OW = dy->shape[3];
     const int64_t R = dw->shape[2], S = dw->shape[3];
+    MJT_CHECK(x->shape[1] % G == 0 && K % G == 0, "conv wgrad: " << x->shape[1] << " input and " << K << " output channels do not split into " << G << " groups");
+    const int64_t C = x->shape[1] / G;                           // input channels per group
     MJT_CHECK(dy->shape[0] == N, "conv wgrad: dy has " << dy->shape[0] << " images, x " << N);
     MJT_CHECK(dw->shape[0] == K && dw->shape[1] == C, "conv wgrad: dw shape " << shape_str(dw) << " != [" << K << "," << C << ",R,S]");
     MJT_CHECK(OH == (H + 2 * p->pad_h - p->dil_h * (R - 1) - 1) / p->stride_h + 1 &&
@@ -223,11 +318,15 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
     const int64_t KG = K % 256 == 0 ? 4 : K % 128 == 0 ? 2 : 1;
     const int64_t CTW = 8 / KG;
     const bool half = x->dtype == MJT_FLOAT16;
-    const bool ok = (x->dtype == MJT_BFLOAT16 || half) && dy->dtype == x->dtype && (dw->dtype == MJT_FLOAT32 || dw->dtype == x->dtype) &&
+    const bool ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && dy->dtype == x->dtype && (dw->dtype == MJT_FLOAT32 || dw->dtype == x->dtype) &&
                     p->stride_w == 1 && p->pad_w <= 2 && (S - 1) * p->dil_w - p->pad_w <= 4 && K % 64 == 0 && C % (16 * CTW) == 0 && R * S <= 9 && OW % 8 == 0 &&
                     W % 2 == 0 && N >= 1 && numel(x) * 2 < (int64_t(1) << 31) && numel(dy) * 2 < (int64_t(1) << 31) &&
                     (uintptr_t)x->ptr % 4 == 0 && (uintptr_t)dy->ptr % 16 == 0 &&
                     !getenv("MJT_NO_FASTPATH");
+    if (!ok && any_shape) {
+        conv_wgrad_direct(x, dy, dw, p, G);
+        return;
+    }
     if (!ok)
         MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: only bfloat16 or float16 operands with horizontal stride 1, column shifts of the taps within -2 .. 4, at most 9 taps, "
                                       "K % 64 == 0, C % " << 16 * CTW << " == 0, OW % 8 == 0 and tensors below 2 GB run on the MFMA kernel");
@@ -260,41 +359,22 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
         k = jit_get(src.str(), name.str());
         remember(key.str(), k);
     }
-    const size_t pbytes = (size_t)slices * (size_t)numel(dw) * 4;
-    if (!c.dry_run && pbytes > g_wgrad_bytes) {
-        if (g_wgrad_part) {
-            HIP_CHECK(hipStreamSynchronize(c.stream));
-            HIP_CHECK(hipFree(g_wgrad_part));
-            g_wgrad_part = nullptr;
-            g_wgrad_bytes = 0;
-        }
-        HIP_CHECK(hipMalloc(&g_wgrad_part, pbytes));
-        g_wgrad_bytes = pbytes;
-    }
-    void* part = c.dry_run ? (void*)(uintptr_t)0x1000 : g_wgrad_part;
+    void* part = wgrad_partials((size_t)slices * (size_t)numel(dw) * 4);
     std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(dy->ptr), bits_of_ptr(part), (uint64_t)N, (uint64_t)ips, 0};
     jit_launch(k, (unsigned)((slices + 7) / 8 * 8 * blocks_per_slice), 1, 512, 0, a);
-    // fold the slices: [slices, K*C*R*S] summed over axis 0, rounded once if dw is bfloat16
-    mjt_tensor tp, td;
-    memset(&tp, 0, sizeof(tp));
-    memset(&td, 0, sizeof(td));
-    tp.ptr = part;
-    tp.dtype = MJT_FLOAT32;
-    tp.ndim = 2;
-    tp.shape[0] = slices;
-    tp.shape[1] = numel(dw);
-    td.ptr = dw->ptr;
-    td.dtype = dw->dtype;
-    td.ndim = 1;
-    td.shape[0] = numel(dw);
-    if (mjt_reduce(&tp, &td, MJT_OP_ADD, 0b01) != MJT_OK) MJT_FAIL(MJT_ERR_DEVICE, "conv wgrad: folding the partial sums failed: " << mjt_last_error());
+    fold_wgrad_slices(part, slices, dw);
     set_last_kernel(k->name.c_str());
 }
 
 }  // namespace mjt
 
 extern "C" int mjt_conv2d_meta_wgrad(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw, const mjt_conv_params* p) {
-    return mjt::guarded([&] { mjt::conv_wgrad_impl(x, dy, dw, p); });
+    return mjt::guarded([&] { mjt::conv_wgrad_impl(x, dy, dw, p, 1, false); });
+}
+
+extern "C" int mjt_conv2d_meta_wgrad_grouped(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw, const mjt_conv_params* p,
+                                             int groups) {
+    return mjt::guarded([&] { mjt::conv_wgrad_impl(x, dy, dw, p, groups, true); });
 }
 
 extern "C" int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p) {

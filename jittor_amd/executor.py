@@ -72,10 +72,11 @@ class ConvBwdDataUnit:
     kind = "conv_bwd_x"
     fusable = False
 
-    def __init__(self, root, dy, w, params):
+    def __init__(self, root, dy, w, params, groups=1):
         self.out = root.out
         self.inputs = [dy, w]
         self.params = params
+        self.groups = groups
         self.id = root.id
 
 
@@ -86,10 +87,11 @@ class ConvBwdWeightUnit:
     kind = "conv_bwd_w"
     fusable = False
 
-    def __init__(self, root, x, dy, params):
+    def __init__(self, root, x, dy, params, groups=1):
         self.out = root.out
         self.inputs = [x, dy]
         self.params = params
+        self.groups = groups
         self.id = root.id
 
 
@@ -300,8 +302,12 @@ def _match_conv(red, consumers, targets):
 
 
 def _match_conv_grouped(op):
-    """reindex_reduce.add <- multiply <- {reindex(x), reindex(w)} over the 8-d product
-    [N, G, K/G, C/G, OH, OW, R, S]: the grouped convolution as python/jittor/nn.py:1272-1294 writes it."""
+    """The grouped convolution as python/jittor/nn.py:1272-1294 writes it and its two gradients as jt.grad builds
+    them, all over the 8-d product [N, G, K/G, C/G, OH, OW, R, S]:
+        reindex_reduce.add <- multiply <- {reindex(a), reindex(b)}
+    Each of x, w and y (or dy) has its own index pattern into that product; the one that is scattered into names the
+    result (y: forward, x: input gradient, w: weight gradient), the other two are the gathered factors
+    (the reference's tuner recognises the same three, opt/tuner/conv_tuner.cc:375-397)."""
     if op.op != "add" or len(op.inputs) != 1 or op.overflow_conditions or op.out.ndim != 4:
         return None
     yy = op.inputs[0]
@@ -309,45 +315,61 @@ def _match_conv_grouped(op):
     if mul is None or mul.op != "multiply" or yy.ndim != 8:
         return None
     N, G, KG, CG, OH, OW, R, S = yy.shape
-    if list(op.out.shape) != [N, G * KG, OH, OW]:
-        return None
 
     def is_sum(aff, terms, c0=0):
         """aff == c0 + sum(coef * i_k for k, coef in terms)"""
         return aff is not None and aff[0] == c0 and all(aff[1][k] == dict(terms).get(k, 0) for k in range(10))
-    out_aff = [_affine(e, op.out.shape, yy.shape) for e in op.indexes]
-    if len(out_aff) != 4 or not (is_sum(out_aff[0], [(0, 1)]) and is_sum(out_aff[1], [(1, KG), (2, 1)])
-                                 and is_sum(out_aff[2], [(4, 1)]) and is_sum(out_aff[3], [(5, 1)])):
+
+    def role_of(exprs, vshape):
+        """('y', None), ('w', None), ('x', params) or None for the index list of a var of shape vshape."""
+        aff = [_affine(e, vshape, yy.shape) for e in exprs]
+        if len(aff) != 4 or any(a_ is None for a_ in aff):
+            return None
+        if list(vshape) == [N, G * KG, OH, OW] and is_sum(aff[0], [(0, 1)]) and is_sum(aff[1], [(1, KG), (2, 1)]) \
+                and is_sum(aff[2], [(4, 1)]) and is_sum(aff[3], [(5, 1)]):
+            return "y", None
+        if list(vshape) == [G * KG, CG, R, S] and is_sum(aff[0], [(1, KG), (2, 1)]) and is_sum(aff[1], [(3, 1)]) \
+                and is_sum(aff[2], [(6, 1)]) and is_sum(aff[3], [(7, 1)]):
+            return "w", None
+        if vshape[0] == N and vshape[1] == G * CG and is_sum(aff[0], [(0, 1)]) and is_sum(aff[1], [(1, CG), (3, 1)]):
+            (c0h, coh), (c0w, cow) = aff[2], aff[3]
+            if any(coh[k] for k in range(10) if k not in (4, 6)) or any(cow[k] for k in range(10) if k not in (5, 7)):
+                return None
+            sh, dh, sw, dw, ph, pw = coh[4], coh[6], cow[5], cow[7], -c0h, -c0w
+            if min(sh, dh, sw, dw) < 1 or ph < 0 or pw < 0:
+                return None
+            H, W = vshape[2], vshape[3]
+            if OH != (H + 2 * ph - dh * (R - 1) - 1) // sh + 1 or OW != (W + 2 * pw - dw * (S - 1) - 1) // sw + 1:
+                return None
+            return "x", (sh, sw, ph, pw, dh, dw)
         return None
-    for a, b in (mul.inputs, mul.inputs[::-1]):
-        rx, rw = _lazy_op(a, ReindexOp), _lazy_op(b, ReindexOp)
-        if rx is None or rw is None or len(rx.inputs) != 1 or len(rw.inputs) != 1:
-            continue
-        if rx.overflow_conditions or rw.overflow_conditions or rx.overflow_value != 0.0:
-            continue
-        x, w = rx.inputs[0], rw.inputs[0]
-        if x.ndim != 4 or list(w.shape) != [G * KG, CG, R, S] or x.shape[0] != N or x.shape[1] != G * CG:
-            continue
-        if x.dtype != w.dtype or x.dtype not in ("float32", "bfloat16", "float16") or op.out.dtype not in ("float32", x.dtype):
-            continue
-        wa = [_affine(e, w.shape, yy.shape) for e in rw.indexes]
-        if len(wa) != 4 or not (is_sum(wa[0], [(1, KG), (2, 1)]) and is_sum(wa[1], [(3, 1)])
-                                and is_sum(wa[2], [(6, 1)]) and is_sum(wa[3], [(7, 1)])):
-            continue
-        xa = [_affine(e, x.shape, yy.shape) for e in rx.indexes]
-        if len(xa) != 4 or any(a_ is None for a_ in xa) or not (is_sum(xa[0], [(0, 1)]) and is_sum(xa[1], [(1, CG), (3, 1)])):
-            continue
-        (c0h, coh), (c0w, cow) = xa[2], xa[3]
-        if any(coh[k] for k in range(10) if k not in (4, 6)) or any(cow[k] for k in range(10) if k not in (5, 7)):
-            continue
-        sh, dh, sw, dw, ph, pw = coh[4], coh[6], cow[5], cow[7], -c0h, -c0w
-        if min(sh, dh, sw, dw) < 1 or ph < 0 or pw < 0:
-            continue
-        H, W = x.shape[2], x.shape[3]
-        if OH != (H + 2 * ph - dh * (R - 1) - 1) // sh + 1 or OW != (W + 2 * pw - dw * (S - 1) - 1) // sw + 1:
-            continue
-        return ConvUnit(op, x, w, (sh, sw, ph, pw, dh, dw), {op.id, mul.id, rx.id, rw.id}, groups=G)
-    return None
+
+    target = role_of(op.indexes, op.out.shape)
+    if target is None:
+        return None
+    found = {target[0]: (op.out, target[1])}
+    ids = {op.id, mul.id}
+    for v in mul.inputs:
+        ro = _lazy_op(v, ReindexOp)
+        if ro is None or len(ro.inputs) != 1 or ro.overflow_conditions:
+            return None
+        role = role_of(ro.indexes, ro.inputs[0].shape)
+        if role is None or role[0] in found or (role[0] == "x" and ro.overflow_value != 0.0):
+            return None
+        found[role[0]] = (ro.inputs[0], role[1])
+        ids.add(ro.id)
+    (x, params), (w, _), (y, _) = found["x"], found["w"], found["y"]
+    a, b = (v for r_, (v, _) in found.items() if r_ != target[0])
+    if a.dtype != b.dtype or a.dtype not in ("float32", "bfloat16", "float16") or op.out.dtype not in ("float32", a.dtype):
+        return None
+    if target[0] == "y":
+        return ConvUnit(op, x, w, params, ids, groups=G)
+    if target[0] == "x":
+        sh, sw, ph, pw, dh, dw = params
+        if dh * (R - 1) - ph < 0 or dw * (S - 1) - pw < 0:
+            return None
+        return ConvBwdDataUnit(op, y, w, params, groups=G)
+    return ConvBwdWeightUnit(op, x, y, params, groups=G)
 
 
 def _match_gather_reduce(red, consumers, target_ids):
@@ -793,8 +815,14 @@ def _run_single(op):
         dy, w = op.inputs
         sh, sw, ph, pw, dh, dw = op.params
         K, C, R, S = w.shape
+        G = op.groups
         with core.no_grad():
-            wt = core.reindex(w, [C, K, R, S], ["i1", "i0", "%d-i2" % (R - 1), "%d-i3" % (S - 1)])
+            if G > 1:
+                # w [G*Kg, Cg, R, S] -> [G*Cg, Kg, R, S]: transposed within each group, taps flipped
+                kg = K // G
+                wt = core.reindex(w, [G * C, kg, R, S], ["i0/%d*%d+i1" % (C, kg), "i0%%%d" % C, "%d-i2" % (R - 1), "%d-i3" % (S - 1)])
+            else:
+                wt = core.reindex(w, [C, K, R, S], ["i1", "i0", "%d-i2" % (R - 1), "%d-i3" % (S - 1)])
         _run_single(wt._op)
         if sh != 1 or sw != 1:
             # a strided convolution's input gradient is the stride-1 one of dy with sh-1 (sw-1) zeros between its rows
@@ -807,7 +835,16 @@ def _run_single(op):
         tx, tw = _tensor_of(dy), _tensor_of(wt)
         ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
         p = _lib.ConvParams(1, 1, dh * (R - 1) - ph, dw * (S - 1) - pw, dh, dw)
-        _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
+        if G > 1:
+            _lib.check(lib.mjt_conv2d_meta_grouped(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p), G))
+        else:
+            _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p)))
+    elif isinstance(op, ConvBwdWeightUnit) and op.groups > 1:
+        x, dy = op.inputs
+        tx, td = _tensor_of(x), _tensor_of(dy)
+        tw = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        p = _lib.ConvParams(*op.params)
+        _lib.check(lib.mjt_conv2d_meta_wgrad_grouped(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p), op.groups))
     elif isinstance(op, ConvBwdWeightUnit):
         x, dy = op.inputs
         sh, sw, ph, pw, dh, dw = op.params

@@ -900,6 +900,34 @@ def conv_meta_grouped(x, w, groups, stride=1, padding=0, dilation=1):
     return reindex_reduce(yy, "add", [N, K, oh, ow], ["i0", "i1*%d+i2" % (K // G), "i4", "i5"])
 
 
+def conv_meta_grouped_grads(x, w, dy, groups, stride=1, padding=0, dilation=1):
+    """Gradients of conv_meta_grouped with respect to x and w for an output gradient dy, as jt.grad builds
+    them over the same 8-d product: the scatter-add's gradient is a reindex of dy with the scatter's indexes
+    (ops/reindex_reduce_op.cc:45-63), the product's is that times the other factor, and each reindex's
+    gradient is a scatter-add with the reindex's own indexes, out-of-range ones dropped
+    (ops/reindex_op.cc:76-80).  stride / padding / dilation: a number or a (vertical, horizontal) pair.
+    Returns float32 (dx [N,G*Cg,H,W], dw [K,Cg,R,S])."""
+    xf = x.to_f32() if isinstance(x, BF16) else np.asarray(x, dtype=np.float32)
+    wf = w.to_f32() if isinstance(w, BF16) else np.asarray(w, dtype=np.float32)
+    df = dy.to_f32() if isinstance(dy, BF16) else np.asarray(dy, dtype=np.float32)
+    N, C, H, W = xf.shape
+    K, CpG, R, S = wf.shape
+    G = groups
+    assert C == CpG * G and K % G == 0
+    (sh, sw), (ph, pw), (dh, dw_) = [v if isinstance(v, (tuple, list)) else (v, v) for v in (stride, padding, dilation)]
+    oh = (H + ph * 2 - R * dh + dh - 1) // sh + 1
+    ow = (W + pw * 2 - S * dw_ + dw_ - 1) // sw + 1
+    assert list(df.shape) == [N, K, oh, ow]
+    shape = [N, G, K // G, CpG, oh, ow, R, S]
+    xi = ["i0", "i1*%d+i3" % CpG, "i4*%d-%d+i6*%d" % (sh, ph, dh), "i5*%d-%d+i7*%d" % (sw, pw, dw_)]
+    wi = ["i1*%d+i2" % (K // G), "i3", "i6", "i7"]
+    yi = ["i0", "i1*%d+i2" % (K // G), "i4", "i5"]
+    xx, ww, dd = reindex(xf, shape, xi), reindex(wf, shape, wi), reindex(df, shape, yi)
+    dx = reindex_reduce(binary(dd, ww, "multiply"), "add", [N, C, H, W], xi)
+    dw = reindex_reduce(binary(dd, xx, "multiply"), "add", [K, CpG, R, S], wi)
+    return dx, dw
+
+
 def conv_meta_wgrad(x, dy, R, S, stride=1, padding=0, dilation=1):
     """Gradient of conv_meta with respect to w for an output gradient dy, as jt.grad builds it from
     the op rules: the sum's gradient is a broadcast of dy over (c, kh, kw) (ops/reduce_op.cc:339-362),

@@ -275,6 +275,54 @@ def test_grad_grouped_conv(gpu):
         close(gw.numpy()[g * kg:(g + 1) * kg], dW, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("dtype,G,cg,kg,kw", [
+    ("float32", 8, 1, 1, dict(padding=1)),                       # depthwise
+    ("float32", 2, 3, 2, dict(stride=2, padding=1)),
+    ("float32", 3, 2, 3, dict(padding=2, dilation=2)),
+    ("bfloat16", 4, 2, 2, dict(padding=1)),
+    ("float16", 2, 2, 3, dict(stride=(2, 1), padding=(0, 1))),
+])
+def test_grad_grouped_conv_runs_as_convolutions(gpu, dtype, G, cg, kg, kw):
+    """Forward and both gradients of a grouped convolution are recognised over the 8-d product and run as
+    convolution kernels (the weight gradient on the direct kernel, the input gradient as the grouped forward kernel
+    on dy with the weights transposed per group and flipped); the 8-d tensors are never written.  Values against
+    the plain execution of the same graph (which sums in the same float type but another order) and, for float32,
+    the oracle's gradient graph."""
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal((3, G * cg, 9, 8)).astype(np.float32)
+    w = (rng.standard_normal((G * kg, cg, 3, 3)) * 0.3).astype(np.float32)
+    results = {}
+    for matched in (True, False):
+        jt.flags["enable_conv_match"] = matched
+        try:
+            vx, vw = jt.array(x).cast(dtype), jt.array(w).cast(dtype)
+            y = jt.nn.conv2d(vx, vw, groups=G, **kw)
+            if "r" not in results:
+                results["r"] = rng.standard_normal(y.shape).astype(np.float32)
+            gx, gw = jt.grad((y * jt.array(results["r"]).cast(dtype)).sum(), [vx, vw])
+            before = dict(jt.executor_stats)
+            jt.sync([y, gx, gw])
+            if matched:
+                assert jt.executor_stats["conv_matches"] == before["conv_matches"] + 3
+            results[matched] = [np.asarray(v.numpy(), dtype=np.float32) for v in (y, gx, gw)]
+        finally:
+            jt.flags["enable_conv_match"] = True
+    # the plain path sums 16-bit products in 16 bits (bfloat16 truncates every partial sum: a few hundred terms lose
+    # tens of percent), the kernels in float32: only float32 results are comparable between the two
+    for a, b in zip(results[True], results[False]):
+        assert a.shape == b.shape
+        if dtype == "float32":
+            assert np.abs(a - b).max() <= 1e-4 * np.abs(b).max()
+    # against the oracle's gradient graph on the same (narrowed) operands: one rounding of a float32 sum
+    def stored(a):
+        return np.asarray(jt.array(a).cast(dtype).numpy(), dtype=np.float32)
+    dx, dw = O.conv_meta_grouped_grads(stored(x), stored(w), stored(results["r"]), G, kw.get("stride", 1), kw.get("padding", 0),
+                                       kw.get("dilation", 1))
+    tol = {"float32": 1e-4, "float16": 2.0 ** -9, "bfloat16": 2.0 ** -7}[dtype]
+    assert np.abs(results[True][1] - dx).max() <= tol * np.abs(dx).max()
+    assert np.abs(results[True][2] - dw).max() <= tol * np.abs(dw).max()
+
+
 def test_pooling_forward_and_backward_keep_rank_six_out_of_memory(gpu):
     """Pooling and its gradient run without the rank-6 window tensors ever being written (the invariant of
     test_longest_dis_fuse.py:51-66): forward = reindex fused with its reduce, backward = the element-wise group

@@ -630,6 +630,77 @@ def test_conv_wgrad_mfma_matches_oracle(gpu, case, monkeypatch):
         assert np.abs(got - ref).max() <= (1e-4 if out == "float32" else 2.0 ** -7) * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("case", [
+    dict(dt="float32", x=(2, 6, 9, 8), k=6, g=6, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),          # depthwise
+    dict(dt="float32", x=(3, 12, 8, 9), k=4, g=2, rs=(3, 3), p=(2, 1, 1, 0, 1, 2)),         # 6 channels per group: a tile of 4 and a tile of 2
+    dict(dt="bfloat16", x=(2, 8, 10, 7), k=8, g=4, rs=(3, 3), p=(2, 2, 1, 1, 1, 1)),        # stride 2
+    dict(dt="float16", x=(2, 4, 9, 9), k=6, g=2, rs=(2, 3), p=(1, 1, 2, 2, 2, 2), out="float16"),
+    dict(dt="float32", x=(1, 2, 12, 12), k=2, g=2, rs=(9, 9), p=(1, 1, 4, 4, 1, 1)),        # 81 taps: three chunks of 32, the last short
+    dict(dt="float32", x=(8, 4, 16, 16), k=4, g=4, rs=(1, 1), p=(1, 1, 0, 0, 1, 1)),        # 1x1; several slices of images, folded by the reduce
+    dict(dt="bfloat16", x=(9, 6, 17, 16), k=6, g=3, rs=(3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16"),   # slices with a short last one, 16-bit result
+    dict(dt="float32", x=(2, 3, 7, 6), k=5, g=1, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),          # one group, float32: the direct kernel
+    dict(dt="bfloat16", x=(2, 128, 6, 8), k=64, g=1, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),      # one group the MFMA kernel covers
+    dict(dt="float32", x=(2, 4, 5, 5), k=4, g=2, rs=(3, 3), p=(1, 1, 0, 0, 1, 1), empty=True),
+])
+def test_conv_wgrad_grouped_matches_oracle(gpu, case):
+    """mjt_conv2d_meta_wgrad_grouped against the oracle's restatement of the gradient graph of the grouped
+    convolution (scatter-add over the 8-d product) and a float64 closed form per group; the kernel sums in another
+    order: 1e-4 of the largest value, 2^-7 for a 16-bit result."""
+    rng = np.random.default_rng(33)
+    dt, (N, C, H, W), K, G, (R, S) = case["dt"], case["x"], case["k"], case["g"], case["rs"]
+    sh, sw, ph, pw, dh, dw_ = case["p"]
+    if case.get("empty"):
+        N = 0
+    OH = (H + 2 * ph - dh * (R - 1) - 1) // sh + 1
+    OW = (W + 2 * pw - dw_ * (S - 1) - 1) // sw + 1
+    narrow = {"float32": lambda a: a.astype(np.float32), "bfloat16": _bf16, "float16": lambda a: a.astype(np.float16)}[dt]
+    widen = {"float32": lambda a: a, "bfloat16": lambda a: O.BF16(a).to_f32(), "float16": lambda a: a.astype(np.float32)}
+    xb, db = narrow(rng.standard_normal((N, C, H, W))), narrow(rng.standard_normal((N, K, OH, OW)))
+    out = case.get("out", "float32")
+    x, dy = jt.from_storage(xb, dt), jt.from_storage(db, dt)
+    dw = jt.zeros([K, C // G, R, S], out) + 7.0                       # stale values must be overwritten, not added to
+    jt.sync([dw], True)
+    tx, td, tw = L.tensor(x.raw_ptr(), dt, x.shape), L.tensor(dy.raw_ptr(), dt, dy.shape), L.tensor(dw.raw_ptr(), out, dw.shape)
+    p = L.ConvParams(*case["p"])
+    L.check(L.load().mjt_conv2d_meta_wgrad_grouped(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p), G))
+    mfma = G == 1 and dt == "bfloat16"
+    if N:
+        assert L.last_kernel().startswith("mjt_conv_wgrad_mfma" if mfma else "mjt_conv_wgrad_direct_" + dt), L.last_kernel()
+    got = widen[out](L.d2h(dw.raw_ptr(), dw.shape, L.NP_STORAGE[out]))
+    xf, df = widen[dt](xb).astype(np.float64), widen[dt](db).astype(np.float64)
+    xp = np.pad(xf, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+    cg, kg = C // G, K // G
+    want = np.zeros((K, cg, R, S))
+    for g in range(G):
+        for r in range(R):
+            for s in range(S):
+                patch = xp[:, g * cg:(g + 1) * cg, r * dh:r * dh + (OH - 1) * sh + 1:sh, s * dw_:s * dw_ + (OW - 1) * sw + 1:sw]
+                want[g * kg:(g + 1) * kg, :, r, s] = np.einsum("nkhw,nchw->kc", df[:, g * kg:(g + 1) * kg], patch)
+    tol = 1e-4 if out == "float32" else 2.0 ** -7
+    assert np.abs(got - want).max() <= tol * max(np.abs(want).max(), 1e-30)
+    if N and sh == sw and ph == pw and dh == dw_ and N * K * cg * OH * OW * R * S <= 2e7:
+        w0 = np.zeros((K, cg, R, S), np.float32)
+        _, ref = O.conv_meta_grouped_grads(widen[dt](xb), w0, widen[dt](db), G, sh, ph, dh)   # the reference's own summation order
+        assert np.abs(got - ref).max() <= tol * np.abs(ref).max()
+
+
+def test_conv_wgrad_grouped_entry_errors(gpu):
+    rng = np.random.default_rng(34)
+    x, dy = jt.array(rng.standard_normal((1, 6, 5, 5)).astype(np.float32)), jt.array(rng.standard_normal((1, 4, 5, 5)).astype(np.float32))
+    dw = jt.zeros([4, 3, 3, 3])
+    jt.sync([x, dy, dw], True)
+    tx, td, tw = (L.tensor(v.raw_ptr(), "float32", v.shape) for v in (x, dy, dw))
+    p = L.ConvParams(1, 1, 1, 1, 1, 1)
+    lib = L.load()
+    assert lib.mjt_conv2d_meta_wgrad_grouped(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p), 4) == -1
+    assert "groups" in lib.mjt_last_error().decode()
+    assert lib.mjt_conv2d_meta_wgrad_grouped(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p), 0) == -1
+    tw2 = L.tensor(dw.raw_ptr(), "float32", [4, 2, 3, 3])
+    assert lib.mjt_conv2d_meta_wgrad_grouped(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw2), ctypes.byref(p), 2) == -1
+    ti = L.tensor(x.raw_ptr(), "int32", x.shape)
+    assert lib.mjt_conv2d_meta_wgrad_grouped(ctypes.byref(ti), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p), 2) == -2
+
+
 def test_conv_wgrad_entry_rejects_what_the_kernel_does_not_cover(gpu):
     rng = np.random.default_rng(32)
     xb, db = _bf16(rng.standard_normal((1, 128, 9, 9))), _bf16(rng.standard_normal((1, 64, 5, 5)))

@@ -511,3 +511,28 @@ def test_conv_gradient_patterns_match_for_common_losses():
             assert isinstance(ux, E.ConvBwdDataUnit) and isinstance(uw, E.ConvBwdWeightUnit), (dtype, loss)
             assert ux.inputs[0].dtype == dtype and list(ux.inputs[0].shape) == [2, 4, 8, 8]
             assert uw.inputs[1].dtype == dtype and gx.dtype == dtype and gw.dtype == dtype
+
+
+def test_grouped_conv_and_its_gradients_are_matched_by_role():
+    """Over the grouped form's 8-d product each of x, w and y has its own index pattern; the scattered-into one names
+    the unit.  Forward, input gradient and weight gradient of a grouped and of a depthwise convolution are recognised,
+    with the geometry read back from the x pattern."""
+    from jittor_amd import executor as E
+    for dtype in ("float32", "bfloat16"):
+        for groups, cin, cout, kw in ((2, 4, 6, dict(padding=1)), (4, 4, 4, dict(stride=2, padding=1)), (3, 6, 3, dict(padding=2, dilation=2))):
+            x, w = jt.zeros([2, cin, 9, 8]).cast(dtype), jt.zeros([cout, cin // groups, 3, 3]).cast(dtype)
+            y = jt.nn.conv2d(x, w, groups=groups, **kw)
+            r = jt.zeros(y.shape).cast(dtype)
+            fwd = E._match_conv_grouped(y._op)
+            assert isinstance(fwd, E.ConvUnit) and fwd.groups == groups and fwd.inputs[0] is x and fwd.inputs[1] is w
+            gx, gw = jt.grad((y * r).sum(), [x, w])
+            ux, uw = E._match_conv_grouped(gx._op), E._match_conv_grouped(gw._op)
+            assert isinstance(ux, E.ConvBwdDataUnit) and isinstance(uw, E.ConvBwdWeightUnit), (dtype, groups)
+            assert ux.groups == groups and uw.groups == groups and ux.params == fwd.params and uw.params == fwd.params
+            assert ux.inputs[1] is w and uw.inputs[0] is x
+            assert list(ux.inputs[0].shape) == list(y.shape) and ux.inputs[0] is uw.inputs[1]
+            assert gx.dtype == dtype and gw.dtype == dtype
+    # an 8-d scatter-add that is none of the three stays what it is
+    a = jt.zeros([2, 2, 3, 2, 4, 4, 3, 3])
+    z = (a * a).reindex_reduce("add", [2, 6, 4, 4], ["i0", "i1*3+i2", "i5", "i4"])
+    assert E._match_conv_grouped(z._op) is None

@@ -327,6 +327,40 @@ def test_conv_meta_wgrad_against_finite_differences_of_the_forward():
                 assert np.allclose(dw[:, :, r, s_], want, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("groups,stride,pad,dil", [(2, 1, 1, 1), (3, 2, 1, 1), (4, 1, 2, 2), (2, 2, 0, 1)])
+def test_conv_meta_grouped_grads_are_the_adjoints_of_the_forward(groups, stride, pad, dil):
+    """The grouped convolution is linear in x and in w, so <conv(x, w), dy> = <x, dx> = <w, dw> with the pinned
+    forward on the left (a wrong group stride, a flipped tap or a dropped padding row breaks one of them), and
+    each group's slices equal the float64 gradients of that group's plain convolution."""
+    cg, kg = 2, 3
+    x = rng.standard_normal((2, groups * cg, 8, 7)).astype(np.float32)
+    w = rng.standard_normal((groups * kg, cg, 3, 3)).astype(np.float32)
+    y = O.conv_meta_grouped(x, w, groups, stride, pad, dil).astype(np.float64)
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    dx, dw = O.conv_meta_grouped_grads(x, w, dy, groups, stride, pad, dil)
+    assert dx.shape == x.shape and dw.shape == w.shape and dx.dtype == np.float32 and dw.dtype == np.float32
+    inner = (y * dy).sum()
+    assert np.isclose(inner, (x.astype(np.float64) * dx).sum(), rtol=1e-4)
+    assert np.isclose(inner, (w.astype(np.float64) * dw).sum(), rtol=1e-4)
+    oh, ow = dy.shape[2:]
+    for g in range(groups):
+        xs, ds = x[:, g * cg:(g + 1) * cg].astype(np.float64), dy[:, g * kg:(g + 1) * kg].astype(np.float64)
+        xp = np.pad(xs, ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+        dxp = np.zeros_like(xp)
+        for r in range(3):
+            for s_ in range(3):
+                rows = slice(r * dil, r * dil + (oh - 1) * stride + 1, stride)
+                cols = slice(s_ * dil, s_ * dil + (ow - 1) * stride + 1, stride)
+                want = np.einsum("nkhw,nchw->kc", ds, xp[:, :, rows, cols])
+                assert np.allclose(dw[g * kg:(g + 1) * kg, :, r, s_], want, rtol=1e-4, atol=1e-4)
+                dxp[:, :, rows, cols] += np.einsum("nkhw,kc->nchw", ds, w[g * kg:(g + 1) * kg, :, r, s_].astype(np.float64))
+        want_dx = dxp[:, :, pad:pad + x.shape[2], pad:pad + x.shape[3]]
+        assert np.allclose(dx[:, g * cg:(g + 1) * cg], want_dx, rtol=1e-4, atol=1e-4)
+    if groups == 2 and stride == 1:                      # one group: the plain weight gradient
+        _, dw1 = O.conv_meta_grouped_grads(x[:, :cg], w[:kg], dy[:, :kg], 1, stride, pad, dil)
+        assert np.allclose(dw1, O.conv_meta_wgrad(x[:, :cg], dy[:, :kg], 3, 3, stride, pad, dil), rtol=1e-5, atol=1e-5)
+
+
 def test_conv_meta_one_hot_kernel_is_a_shift():
     x = O.BF16(O.f32_to_bf16_bits(rng.standard_normal((1, 2, 6, 6)).astype(np.float32)))
     w = np.zeros((2, 2, 3, 3), np.float32)
