@@ -9,6 +9,7 @@ Nothing executes until a Var is synchronised (lazy_execution,
 var_holder.cc:25-33); execution is in executor.py.
 """
 import numbers
+import weakref
 
 import numpy as np
 
@@ -110,8 +111,20 @@ class Op:
     def __init__(self, inputs):
         self.inputs = list(inputs)
         self.id = _new_id()
-        self.out = None
+        self._out_ref = None
         self.amp = dt.amp_reg & 63          # the register at creation; its gradient is built under it (op.cc:38, grad.cc:48-55)
+
+    # The result is held weakly: a Var owns its producing op (and through it the inputs), never the other way round, so
+    # a Var nobody refers to any more is released at once together with its buffer, without waiting for the cycle collector
+    # (an op is only ever reached through its result or through a consumer of its result).
+    @property
+    def out(self):
+        ref = self._out_ref
+        return ref() if ref is not None else None
+
+    @out.setter
+    def out(self, v):
+        self._out_ref = weakref.ref(v) if v is not None else None
 
     def __repr__(self):
         return "%s#%d" % (self.kind, self.id)

@@ -23,6 +23,9 @@ void* g_wpack = nullptr;
 size_t g_wpack_bytes = 0;
 void* g_wgrad_part = nullptr;      // per-slice partial weight gradients (its own buffer: the reduce that folds them uses the arena)
 size_t g_wgrad_bytes = 0;
+void* g_conv_scratch[2] = {nullptr, nullptr};   // column matrices of a chunk of images; float32 copy of a bfloat16 result
+size_t g_conv_scratch_bytes[2] = {0, 0};
+
 void forget() {
     std::lock_guard<std::mutex> lock(g_mu);
     for (auto& kv : g_kernels)
@@ -31,12 +34,34 @@ void forget() {
     if (!ctx().dry_run) {
         if (g_wpack) (void)hipFree(g_wpack);
         if (g_wgrad_part) (void)hipFree(g_wgrad_part);
+        for (void* b : g_conv_scratch)
+            if (b) (void)hipFree(b);
     }
-    g_wpack = g_wgrad_part = nullptr;
-    g_wpack_bytes = g_wgrad_bytes = 0;
+    g_wpack = g_wgrad_part = g_conv_scratch[0] = g_conv_scratch[1] = nullptr;
+    g_wpack_bytes = g_wgrad_bytes = g_conv_scratch_bytes[0] = g_conv_scratch_bytes[1] = 0;
 }
 const bool g_registered = (at_shutdown(&forget), true);
+
+// One of the two growing buffers of the GEMM path.
+void* conv_scratch(int which, size_t bytes) {
+    Context& c = ctx();
+    if (c.dry_run) return (void*)(uintptr_t)0x1000;
+    if (bytes > g_conv_scratch_bytes[which]) {
+        if (g_conv_scratch[which]) {
+            HIP_CHECK(hipStreamSynchronize(c.stream));
+            HIP_CHECK(hipFree(g_conv_scratch[which]));
+            g_conv_scratch[which] = nullptr;
+            g_conv_scratch_bytes[which] = 0;
+        }
+        HIP_CHECK(hipMalloc(&g_conv_scratch[which], bytes));
+        g_conv_scratch_bytes[which] = bytes;
+    }
+    return g_conv_scratch[which];
+}
 }  // namespace
+
+void matmul_impl(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, int trans_a, int trans_b, bool share_a);
+bool matmul_available();
 
 void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p, int64_t G) {
     require_init();
@@ -172,6 +197,57 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         MJT_CHECK(blocks < (int64_t(1) << 31), "conv: launch too large");
         std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(g_wpack), bits_of_ptr(y->ptr), (uint64_t)N};
         jit_launch(k, (unsigned)blocks, 1, (unsigned)(64 * WPX * WKO), 0, a);
+        return;
+    }
+
+    // ---- column matrices + library GEMM -----------------------------------------------
+    // What the MFMA kernel does not take (float32, widths that are no multiple of 8, strides) and is large enough to
+    // matter: y[n] [K, P] = w [K, C*R*S] x cols[n] [C*R*S, P], cols = the shifted input planes written by one reindex per
+    // chunk of images (a 1x1 convolution of stride 1 without padding reads x itself).  A bfloat16 result goes through
+    // a float32 copy so that it is narrowed the way every other kernel narrows it (by truncation), not rounded by the library.
+    const int64_t P = OH * OW, CRS = C * R * S;
+    if (G == 1 && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_GEMM") && (double)N * K * P * CRS >= (double)(1 << 22) &&
+        P < (int64_t(1) << 31) && CRS < (int64_t(1) << 31) && matmul_available()) {
+        const int64_t esz = dtype_size(x->dtype);
+        const bool plain = R == 1 && S == 1 && p->stride_h == 1 && p->stride_w == 1 && p->pad_h == 0 && p->pad_w == 0;
+        const bool via_f32 = y->dtype == MJT_BFLOAT16;
+        int64_t chunk = (int64_t(1) << 30) / (CRS * P * esz);
+        if (const char* e = getenv("MJT_CONV_GEMM_CHUNK"))      // images per chunk, for tests of the chunk loop
+            if (atoi(e) >= 1) chunk = atoi(e);
+        if (chunk < 1) chunk = 1;
+        if (chunk > N) chunk = N;
+        void* cols = plain ? nullptr : conv_scratch(0, (size_t)(chunk * CRS * P * esz));
+        void* ytmp = via_f32 ? conv_scratch(1, (size_t)(chunk * K * P * 4)) : nullptr;
+        std::string sh = "i4*" + std::to_string(p->stride_h) + "-" + std::to_string(p->pad_h) + "+i2*" + std::to_string(p->dil_h);
+        std::string sw = "i5*" + std::to_string(p->stride_w) + "-" + std::to_string(p->pad_w) + "+i3*" + std::to_string(p->dil_w);
+        const char* idx[4] = {"i0", "i1", sh.c_str(), sw.c_str()};
+        auto view = [](void* ptr, int dtype, std::initializer_list<int64_t> shape) {
+            mjt_tensor t;
+            memset(&t, 0, sizeof(t));
+            t.ptr = ptr;
+            t.dtype = dtype;
+            for (int64_t e : shape) t.shape[t.ndim++] = e;
+            return t;
+        };
+        for (int64_t n0 = 0; n0 < N; n0 += chunk) {
+            const int64_t nb = N - n0 < chunk ? N - n0 : chunk;
+            char* xn = (char*)x->ptr + n0 * C * H * W * esz;
+            if (!plain) {
+                mjt_tensor tx = view(xn, x->dtype, {nb, C, H, W}), tc = view(cols, x->dtype, {nb, C, R, S, OH, OW});
+                if (mjt_reindex(&tx, &tc, 4, idx, 0.0, 0, nullptr, 0, nullptr) != MJT_OK)
+                    MJT_FAIL(MJT_ERR_DEVICE, "conv: writing the column matrices failed: " << mjt_last_error());
+            }
+            char* yn = (char*)y->ptr + n0 * K * P * dtype_size(y->dtype);
+            mjt_tensor ta = view(w->ptr, w->dtype, {nb, K, CRS}), tb = view(plain ? (void*)xn : cols, x->dtype, {nb, CRS, P});
+            mjt_tensor tc = view(via_f32 ? ytmp : (void*)yn, via_f32 ? MJT_FLOAT32 : y->dtype, {nb, K, P});
+            matmul_impl(&ta, &tb, &tc, 0, 0, true);
+            if (via_f32) {
+                mjt_tensor ts = view(ytmp, MJT_FLOAT32, {1, nb * K * P}), td = view(yn, y->dtype, {nb * K * P});
+                if (mjt_reduce(&ts, &td, MJT_OP_ADD, 0b01) != MJT_OK)
+                    MJT_FAIL(MJT_ERR_DEVICE, "conv: narrowing the result failed: " << mjt_last_error());
+            }
+        }
+        set_last_kernel(plain ? "conv_as_gemm" : "conv_as_reindex_gemm");
         return;
     }
 

@@ -58,7 +58,9 @@ rocblas_datatype blas_type(int dtype) {
 }
 }  // namespace
 
-void matmul_impl(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, int trans_a, int trans_b) {
+// With `share_a` every matrix of the batch is multiplied by the first matrix of a (batch stride 0: the weights of a
+// convolution against the column matrices of a chunk of images).
+void matmul_impl(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, int trans_a, int trans_b, bool share_a) {
     require_init();
     MJT_CHECK(a && b && c, "matmul: null tensor");
     // the relay's own checks (cublas_matmul_op.cc:34-52)
@@ -118,7 +120,7 @@ void matmul_impl(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, 
     else
         st = g_blas.gemm_batched(g_blas.handle, opb, opa, (rocblas_int)k, (rocblas_int)n, (rocblas_int)m, alpha, b->ptr,
                                  blas_type(b->dtype), ldb, (rocblas_stride)(m * k), a->ptr, blas_type(a->dtype), lda,
-                                 (rocblas_stride)(n * m), beta, c->ptr, blas_type(c->dtype), (rocblas_int)k,
+                                 (rocblas_stride)(share_a ? 0 : n * m), beta, c->ptr, blas_type(c->dtype), (rocblas_int)k,
                                  (rocblas_stride)(n * k), c->ptr, blas_type(c->dtype), (rocblas_int)k, (rocblas_stride)(n * k),
                                  (rocblas_int)batch, tc, rocblas_gemm_algo_standard, 0, 0);
     if (st != rocblas_status_success) MJT_FAIL(MJT_ERR_DEVICE, "matmul: rocBLAS returned " << (int)st);
@@ -128,8 +130,12 @@ void matmul_impl(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, 
 }  // namespace mjt
 
 extern "C" int mjt_matmul(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, int trans_a, int trans_b) {
-    return mjt::guarded([&] { mjt::matmul_impl(a, b, c, trans_a, trans_b); });
+    return mjt::guarded([&] { mjt::matmul_impl(a, b, c, trans_a, trans_b, false); });
 }
+
+namespace mjt {
+bool matmul_available() { return blas_load(); }
+}  // namespace mjt
 
 extern "C" int mjt_matmul_available(void) {
     return mjt::blas_load() ? 1 : 0;

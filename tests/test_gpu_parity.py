@@ -535,6 +535,52 @@ def test_conv_direct_small_shapes_and_fp32(gpu):
         assert np.allclose(got, O.conv_meta(O.BF16(_bf16(x)), O.BF16(_bf16(w)), st, pd, dl), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("case", [
+    dict(dt="float32", x=(4, 32, 28, 28), w=(48, 32, 3, 3), p=(1, 1, 1, 1, 1, 1)),
+    dict(dt="float32", x=(3, 16, 30, 27), w=(48, 16, 3, 2), p=(2, 1, 1, 0, 1, 2), chunk=2),       # chunks of 2 + 1 images
+    dict(dt="bfloat16", x=(2, 64, 28, 28), w=(128, 64, 3, 3), p=(2, 2, 1, 1, 1, 1), out="bfloat16"),   # width no multiple of 8
+    dict(dt="bfloat16", x=(2, 64, 14, 14), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),
+    dict(dt="float16", x=(4, 64, 14, 14), w=(96, 64, 1, 1), p=(1, 1, 0, 0, 1, 1), out="float16", plain=True),
+    dict(dt="float32", x=(5, 40, 16, 16), w=(96, 40, 1, 1), p=(1, 1, 0, 0, 1, 1), plain=True, chunk=2),
+])
+def test_conv_as_reindex_and_library_gemm(gpu, case, monkeypatch):
+    """Shapes the MFMA kernel does not take and that are large enough to matter run as column matrices (one reindex)
+    times the weights (library GEMM, float32 accumulation): against a float64 closed form and, for float32, the
+    oracle's own summation order; a bfloat16 result is truncated like everywhere else, a float16 one rounded."""
+    rng = np.random.default_rng(41)
+    dt = case["dt"]
+    sh, sw, ph, pw, dh, dw_ = case["p"]
+    narrow = {"float32": lambda a: a.astype(np.float32), "bfloat16": _bf16, "float16": lambda a: a.astype(np.float16)}[dt]
+    widen = {"float32": lambda a: a, "bfloat16": lambda a: O.BF16(a).to_f32(), "float16": lambda a: a.astype(np.float32)}
+    xb, wb = narrow(rng.standard_normal(case["x"])), narrow(rng.standard_normal(case["w"]) * 0.1)
+    out = case.get("out", "float32")
+    if "chunk" in case:
+        monkeypatch.setenv("MJT_CONV_GEMM_CHUNK", str(case["chunk"]))
+    got, kern = _conv_call(xb, wb, case["p"], out_dtype=out, in_dtype=dt)
+    assert kern == ("conv_as_gemm" if case.get("plain") else "conv_as_reindex_gemm"), kern
+    got = widen[out](got)
+    xf, wf = widen[dt](xb).astype(np.float64), widen[dt](wb).astype(np.float64)
+    K, _, R, S = wf.shape
+    oh, ow = got.shape[2:]
+    xp = np.pad(xf, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+    ref = np.zeros(got.shape)
+    for r in range(R):
+        for s in range(S):
+            patch = xp[:, :, r * dh:r * dh + (oh - 1) * sh + 1:sh, s * dw_:s * dw_ + (ow - 1) * sw + 1:sw]
+            ref += np.einsum("nchw,kc->nkhw", patch, wf[:, :, r, s])
+    tol = {"float32": 1e-4, "bfloat16": 2.0 ** -7, "float16": 2.0 ** -10}[out]
+    assert np.abs(got - ref).max() <= tol * np.abs(ref).max()
+    if out == "bfloat16":                                    # truncated, never rounded up in magnitude
+        assert np.all(np.abs(got) <= np.abs(ref) + 1e-5 * np.abs(ref).max())
+    if dt == "float32" and sh == sw and ph == pw and dh == dw_:
+        assert np.abs(got - O.conv_meta(xb, wb, sh, ph, dh)).max() <= 1e-4 * np.abs(ref).max()
+    # the same call with the library path off: the direct kernel, same values to the same bound
+    monkeypatch.setenv("MJT_CONV_NO_GEMM", "1")
+    got2, kern2 = _conv_call(xb, wb, case["p"], out_dtype=out, in_dtype=dt)
+    assert kern2.startswith("mjt_conv_direct")
+    assert np.abs(widen[out](got2) - ref).max() <= tol * np.abs(ref).max()
+
+
 def test_conv_grouped_entry_and_front_end(gpu):
     """Grouped convolution (python/jittor/nn.py:1272-1294): the C entry point against the oracle's 8-d
     restatement, then nn.conv2d(groups=G) matched by the executor (one kernel, nothing of rank 8 in memory)
