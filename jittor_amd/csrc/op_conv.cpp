@@ -252,8 +252,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     }
 
     // ---- direct path ----------------------------------------------------------------
+    const bool idx32 = numel(x) < (int64_t(1) << 31) && numel(y) < (int64_t(1) << 31) - 256 && numel(w) < (int64_t(1) << 31);
     std::ostringstream key;
-    key << "direct|" << geo.str() << x->dtype << "|" << y->dtype << "|" << G;
+    key << "direct|" << geo.str() << x->dtype << "|" << y->dtype << "|" << G << "|" << idx32;
     JitKernel* k = cached(key.str());
     if (!k) {
         std::ostringstream name;
@@ -261,9 +262,11 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
              << "_" << H << "x" << W << "_r" << R << "x" << S << "_s" << p->stride_h << "x" << p->stride_w << "_p" << p->pad_h
              << "x" << p->pad_w << "_d" << p->dil_h << "x" << p->dil_w;
         if (G > 1) name << "_g" << G;
+        if (!idx32) name << "_i64";
         std::ostringstream src;
         src << "#define ENTRY " << name.str() << "\n#define TIN " << dtype_cname(x->dtype) << "\n#define TOUT "
-            << dtype_cname(y->dtype) << "\n#define G_ " << G << "\n" << geo.str();
+            << dtype_cname(y->dtype) << "\n#define G_ " << G << "\n#define IDX " << (idx32 ? "int" : "long long")
+            << "\n" << geo.str();
         src << embedded_source("prelude.h") << "\n" << embedded_source("conv_direct.h") << "\n";
         k = jit_get(src.str(), name.str());
         remember(key.str(), k);
