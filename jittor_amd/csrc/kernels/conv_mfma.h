@@ -70,7 +70,7 @@ struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as p
 #define TR (WPX * TRW)
 #define SPLITS ((OH_ + RPW - 1) / RPW)      // row ranges per image
 #define NCB (C_ / CB)
-#define GROUPS (W_ / 8)                 // groups of 8 columns
+#define GROUPS ((W_ + 7) / 8)           // groups of 8 columns; the last one may reach past the row: what it reads there is never written
 #define SEGS ((GROUPS + 7) / 8)         // segments of 64 columns
 #define TILE_ELEMS (LROWS * LCOLS * 64)
 
@@ -211,7 +211,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
             f[1] = __builtin_amdgcn_perm(s0, c1, sel_b);
             f[2] = __builtin_amdgcn_perm(s1, c2, sel_a);
             f[3] = __builtin_amdgcn_perm(s1, c3, sel_b);
-            if (lr < lrows && seg * 8 + sg < GROUPS) {       // rows outside the image carry zeros
+            if (lr < lrows && seg * 64 + lane < W_) {        // rows outside the image carry zeros; columns past the row end are not the row's
                 unsigned short* dst = &xs[buf][0] + mjt_lds_off(lr * LCOLS + PW + seg * 64 + lane, cg);
                 *(mjt_u32x4v*)dst = f;
             }

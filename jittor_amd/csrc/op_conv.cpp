@@ -116,12 +116,12 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
     const bool half = x->dtype == MJT_FLOAT16;
     const bool mfma_ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % 64 == 0 && K % 64 == 0 &&
-                         W % 8 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 128 <= 72 * 1024 &&
+                         W % 2 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 128 <= 72 * 1024 &&
                          // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
                          ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + 4 * LROWS * LCOLS * 16 < 65536 &&
                          (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49;
     if (mfma_ok) {
-        const int64_t items = LROWS * ((W / 8 + 7) / 8) * 8;     // (row, 64 columns, 8 channels); a wave moves one item per load
+        const int64_t items = LROWS * (((W + 7) / 8 + 7) / 8) * 8;     // (row, 64 columns, 8 channels); a wave moves one item per load
         const int64_t items_per_wave = (items + WPX * WKO - 1) / (WPX * WKO);
         // Rows per workgroup: a workgroup walks RPW output rows as NFULL tiles of TR rows plus one
         // shorter tile.  Pick the RPW that minimises (rounds of workgroups over the compute units) x

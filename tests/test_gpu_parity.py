@@ -476,6 +476,11 @@ def _conv_call(xbits, wbits, params, out_dtype="float32", in_dtype="bfloat16"):
     dict(x=(6, 64, 35, 16), w=(128, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), rpw=35),   # two full tiles + a short tile whose last row is masked
     dict(x=(5, 64, 30, 16), w=(128, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), rpw=20),   # second row range of an image is cut short
     dict(x=(3, 128, 24, 24), w=(128, 128, 3, 3), p=(1, 1, 1, 1, 1, 1), rpw=24, out="bfloat16"),   # bfloat16 output, several tiles
+    dict(x=(3, 64, 28, 28), w=(128, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16"),   # width 28: the last group of 8 columns is half a group, rows 8-byte aligned
+    dict(x=(2, 128, 14, 14), w=(64, 128, 3, 3), p=(1, 1, 1, 1, 1, 1)),      # width 14: 4-byte store epilogue too
+    dict(x=(2, 64, 28, 28), w=(64, 64, 3, 3), p=(2, 2, 1, 1, 1, 1)),        # width 28, stride 2: output width 14
+    dict(x=(2, 64, 9, 12), w=(64, 64, 1, 1), p=(1, 1, 0, 0, 1, 1)),         # width 12, 1x1: the last image row ends at the tensor's end
+    dict(x=(1, 64, 11, 70), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),        # 70 columns: a second staging segment of 6
 ])
 def test_conv_mfma_matches_oracle(gpu, case):
     from oracle import kernels as K
@@ -538,8 +543,8 @@ def test_conv_direct_small_shapes_and_fp32(gpu):
 @pytest.mark.parametrize("case", [
     dict(dt="float32", x=(4, 32, 28, 28), w=(48, 32, 3, 3), p=(1, 1, 1, 1, 1, 1)),
     dict(dt="float32", x=(3, 16, 30, 27), w=(48, 16, 3, 2), p=(2, 1, 1, 0, 1, 2), chunk=2),       # chunks of 2 + 1 images
-    dict(dt="bfloat16", x=(2, 64, 28, 28), w=(128, 64, 3, 3), p=(2, 2, 1, 1, 1, 1), out="bfloat16"),   # width no multiple of 8
-    dict(dt="bfloat16", x=(2, 64, 14, 14), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),
+    dict(dt="bfloat16", x=(2, 64, 27, 27), w=(128, 64, 3, 3), p=(2, 2, 1, 1, 1, 1), out="bfloat16"),   # odd width
+    dict(dt="bfloat16", x=(2, 48, 14, 14), w=(64, 48, 3, 3), p=(1, 1, 1, 1, 1, 1)),                     # channels no multiple of 64
     dict(dt="float16", x=(4, 64, 14, 14), w=(96, 64, 1, 1), p=(1, 1, 0, 0, 1, 1), out="float16", plain=True),
     dict(dt="float32", x=(5, 40, 16, 16), w=(96, 40, 1, 1), p=(1, 1, 0, 0, 1, 1), plain=True, chunk=2),
 ])
