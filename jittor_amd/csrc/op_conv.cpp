@@ -113,7 +113,17 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     // output channels per workgroup: 64 per pair of waves, up to 256
     // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
     const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
-    const int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
+    int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
+    {
+        // fewer output channels per workgroup while the grid would leave compute units idle (small maps, small batches):
+        // the same input tile is then staged by more workgroups, which the L2 absorbs
+        const int64_t cus0 = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
+        const int64_t tile_rows = WPX * (TRW > 0 ? TRW : 1);
+        const int64_t min_ranges = N * ((OH + tile_rows - 1) / tile_rows);
+        while (WKO > 1 && 2 * min_ranges * (K / (16 * MT * WKO)) <= cus0) WKO /= 2;     // only while at most half of them would work
+        if (const char* e = getenv("MJT_CONV_WKO"))
+            if (atoi(e) >= 1 && atoi(e) <= WKO * 4 && K % (16 * MT * atoi(e)) == 0 && (atoi(e) & (atoi(e) - 1)) == 0 && atoi(e) <= 256 / (16 * MT)) WKO = atoi(e);
+    }
     const bool half = x->dtype == MJT_FLOAT16;
     const bool mfma_ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % 64 == 0 && K % 64 == 0 &&
                          W % 2 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 128 <= 72 * 1024 &&
