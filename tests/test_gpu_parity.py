@@ -481,6 +481,8 @@ def _conv_call(xbits, wbits, params, out_dtype="float32", in_dtype="bfloat16"):
     dict(x=(2, 64, 28, 28), w=(64, 64, 3, 3), p=(2, 2, 1, 1, 1, 1)),        # width 28, stride 2: output width 14
     dict(x=(2, 64, 9, 12), w=(64, 64, 1, 1), p=(1, 1, 0, 0, 1, 1)),         # width 12, 1x1: the last image row ends at the tensor's end
     dict(x=(1, 64, 11, 70), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),        # 70 columns: a second staging segment of 6
+    dict(x=(3, 64, 6, 6), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),          # rows shorter than one group of 8 columns
+    dict(x=(2, 64, 5, 2), w=(64, 64, 1, 1), p=(1, 1, 0, 0, 1, 1)),          # two columns: a load spans four rows
 ])
 def test_conv_mfma_matches_oracle(gpu, case):
     from oracle import kernels as K
