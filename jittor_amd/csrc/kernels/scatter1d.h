@@ -456,8 +456,10 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_COLD(Params p) {
     __shared__ mjt_plan plan;
     __shared__ unsigned length[512];                          // lengths of the lists of an item (G1 <= 512)
     __shared__ int rows[MERGE_ROWS];
+    __shared__ unsigned novf_s[512];                          // entries of each main workgroup's overflow list
     __shared__ unsigned long long wsum[16];
     __shared__ unsigned any_ovf, nmatch;
+    for (int t = threadIdx.x; t < G1; t += NTHREADS) novf_s[t] = novf[t];
     for (int t = threadIdx.x; t < NBMAX; t += NTHREADS) {
         plan.nsplit[t] = planin[t];
         plan.nmerge[t] = planin[NBMAX + t];
@@ -566,7 +568,7 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_COLD(Params p) {
         // entries that did not fit a list: the first item of the bucket scans the overflow lists
         if (split == 0 && any_ovf) {
             for (int w = 0; w < G1; w++) {
-                const unsigned c = novf[w];
+                const unsigned c = novf_s[w];                 // (from LDS: a load from memory per workgroup would be a chain of round trips)
                 const mjt_pair* __restrict__ l = ovf + (size_t)w * per;
                 for (unsigned q = threadIdx.x; q < c; q += NTHREADS) {
                     const mjt_pair e = l[q];

@@ -129,7 +129,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                          W % 2 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 128 <= 72 * 1024 &&
                          // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
                          ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + 4 * LROWS * LCOLS * 16 < 65536 &&
-                         (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49;
+                         (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49 &&
+                         // byte offsets inside one image and inside the weights are 32-bit in the kernel
+                         C * H * W * 2 < (int64_t(1) << 31) && K * OH * OW * 4 < (int64_t(1) << 31) && numel(w) * 2 < (int64_t(1) << 31);
     if (mfma_ok) {
         const int64_t items = LROWS * (((W + 7) / 8 + 7) / 8) * 8;     // (row, 64 columns, 8 channels); a wave moves one item per load
         const int64_t items_per_wave = (items + WPX * WKO - 1) / (WPX * WKO);

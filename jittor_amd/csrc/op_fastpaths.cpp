@@ -91,6 +91,19 @@ bool try_window_gather(const mjt_tensor* x, const mjt_tensor* y, const std::vect
     const int64_t tiles = (OH + TH - 1) / TH;
     if (planes * tiles >= (int64_t(1) << 31)) return false;
 
+    // overflow value as raw bits of Tx(overflow_value); dtypes without an encoding here take the generic kernel
+    // (decided before a kernel is compiled for them)
+    uint64_t ovbits = 0;
+    switch (x->dtype) {
+        case MJT_FLOAT32: { float f = (float)overflow_value; uint32_t u; memcpy(&u, &f, 4); ovbits = u; break; }
+        case MJT_FLOAT64: ovbits = bits_of(overflow_value); break;
+        case MJT_BFLOAT16: { float f = (float)overflow_value; uint32_t u; memcpy(&u, &f, 4); ovbits = u >> 16; break; }
+        case MJT_FLOAT16: return false;
+        case MJT_INT32: case MJT_INT64: case MJT_INT16: ovbits = (uint64_t)(int64_t)overflow_value; break;
+        case MJT_UINT32: case MJT_UINT64: case MJT_UINT16: ovbits = (uint64_t)overflow_value; break;
+        default: return false;
+    }
+    if (esz < 8) ovbits &= (1ull << (8 * esz)) - 1;
     std::ostringstream key;
     key << "win|" << esz << "|" << vec << "|" << H << "," << W << "," << OH << "," << OW << "," << KH << "," << KW << ","
         << SH << "," << SW << "," << DH << "," << DW << "," << CH << "," << CW << "," << TH << "," << wthreads;
@@ -109,18 +122,6 @@ bool try_window_gather(const mjt_tensor* x, const mjt_tensor* y, const std::vect
         k = jit_get(src.str(), name.str());
         remember(key.str(), k);
     }
-    // overflow value as raw bits of Tx(overflow_value)
-    uint64_t ovbits = 0;
-    switch (x->dtype) {
-        case MJT_FLOAT32: { float f = (float)overflow_value; uint32_t u; memcpy(&u, &f, 4); ovbits = u; break; }
-        case MJT_FLOAT64: ovbits = bits_of(overflow_value); break;
-        case MJT_BFLOAT16: { float f = (float)overflow_value; uint32_t u; memcpy(&u, &f, 4); ovbits = u >> 16; break; }
-        case MJT_FLOAT16: return false;
-        case MJT_INT32: case MJT_INT64: case MJT_INT16: ovbits = (uint64_t)(int64_t)overflow_value; break;
-        case MJT_UINT32: case MJT_UINT64: case MJT_UINT16: ovbits = (uint64_t)overflow_value; break;
-        default: return false;
-    }
-    if (esz < 8) ovbits &= (1ull << (8 * esz)) - 1;
     std::vector<uint64_t> args{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), ovbits, (uint64_t)planes};
     jit_launch(k, (unsigned)(planes * tiles), 1, (unsigned)wthreads, 0, args);
     return true;
@@ -137,7 +138,7 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     if (index->dtype != MJT_INT32 && index->dtype != MJT_INT64) return false;
     if (x->ndim != 1 || y->ndim != 1) return false;
     const int64_t n = numel(y), bins = numel(x);
-    if (bins >= (int64_t(1) << 31) || n >= (int64_t(1) << 40)) return false;
+    if (bins >= (int64_t(1) << 31) || n >= (int64_t(1) << 36)) return false;
     if ((uintptr_t)y->ptr % 16 || (uintptr_t)index->ptr % 32 || (uintptr_t)x->ptr % 4) return false;
     Context& c = ctx();
     int logw = env_int("MJT_SCATTER_LOGW", 14);              // 16384 bins: 64 KB (128 KB for float sums) of LDS per private copy
@@ -179,8 +180,10 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     const int64_t cold_items = NB + n / cold_target + 1 + G1 / 16 + (NB < G1 ? NB : G1) + 1;
     int64_t cold_wgs = (int64_t)c.prop.multiProcessorCount * (acc64 ? 1 : 2);
     if (cold_wgs > cold_items) cold_wgs = cold_items;
-    int64_t CAP = NB > 1 ? (4 * per / NB + 63) / 64 * 64 : 64;
-    if (CAP < 64) CAP = 64;
+    // A list holds four times its share of a uniformly spread input, plus 512 bytes: all workgroups append to
+    // the lists of one bucket at about the same position, and lists that lie a power of two apart (32 KB for
+    // 2^24 elements into 2^20 bins) put those appends into the same memory channels (main pass 40 instead of 44 us).
+    int64_t CAP = NB > 1 ? (4 * per / NB + 63) / 64 * 64 + 64 : 64;
     if (CAP > per) CAP = (per + 63) / 64 * 64;
 
     std::ostringstream key;
@@ -224,7 +227,16 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     const size_t off_lists = off_pcold + align((size_t)cold_items * W * 4);
     const size_t off_ovf = off_lists + align(NB > 1 ? (size_t)G1 * NB * CAP * 8 : 0);
     const size_t total = off_ovf + align(NB > 1 ? (size_t)G1 * per * 8 : 0);
-    char* base = (char*)scratch(total);
+    // about 40 bytes of scratch per input element: when that is more than a sixteenth of the device's memory, or
+    // the arena cannot grow, the generic kernel (global atomics, no scratch) takes the call
+    if (!c.dry_run && total > c.prop.totalGlobalMem / 16) return false;
+    char* base;
+    try {
+        base = (char*)scratch(total);
+    } catch (const Error&) {
+        (void)hipGetLastError();
+        return false;
+    }
     std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), bits_of_ptr(index->ptr), (uint64_t)n, (uint64_t)bins,
                             bits_of_ptr(base), (uint64_t)per, (uint64_t)G1, (uint64_t)NB, (uint64_t)CAP,
                             bits_of_ptr(base + off_counts), bits_of_ptr(base + off_lists), bits_of_ptr(base + off_pmain),

@@ -209,7 +209,7 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         // run the column kernel over a reduced axis of extent R (0 or 1)
         std::vector<Axis> r1{Axis{xn == 0 ? 0 : 1, 0}};
         std::vector<Axis> k1{Axis{O, 1}};
-        launch(false, tx, ty, op, false, x->ptr ? x->ptr : y->ptr, y->ptr, O, 1, k1, r1, rcount, false, 1, 1,
+        launch(false, tx, ty, op, false, x->ptr ? x->ptr : y->ptr, y->ptr, O, 1, k1, r1, rcount, O >= (int64_t(1) << 31), 1, 1,
                r1[0].size, r1[0].size, false, xn ? pro : nullptr);
         return;
     }

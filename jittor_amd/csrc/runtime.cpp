@@ -176,6 +176,16 @@ static std::vector<char> compile_source(const std::string& source, const std::st
     return code;
 }
 
+// Writes a code object under its final name only when every byte reached the file.
+static void store_code(const std::string& path, const std::vector<char>& code) {
+    std::string tmp = path + "." + std::to_string((long)getpid());
+    std::ofstream f(tmp, std::ios::binary);
+    f.write(code.data(), (std::streamsize)code.size());
+    f.close();
+    if (f.good()) rename(tmp.c_str(), path.c_str());
+    else unlink(tmp.c_str());
+}
+
 JitKernel* jit_get(const std::string& source, const std::string& entry) {
     require_init();
     std::lock_guard<std::mutex> lock(g_jit_mutex);
@@ -201,21 +211,32 @@ JitKernel* jit_get(const std::string& source, const std::string& entry) {
         std::ofstream f(std::string(dump) + "/" + entry + ".hip");
         f << source;
     }
+    const bool from_disk = !code.empty();
     if (code.empty()) {
         code = compile_source(source, entry + ".hip");
         g_jit_compiled++;
         if (use_disk) {
-            std::string tmp = path + "." + std::to_string((long)getpid());
-            std::ofstream f(tmp, std::ios::binary);
-            f.write(code.data(), (std::streamsize)code.size());
-            f.close();
-            rename(tmp.c_str(), path.c_str());
+            store_code(path, code);
         }
     }
     JitKernel* k = new JitKernel();
     k->name = entry;
     if (!ctx().dry_run) {
-        HIP_CHECK(hipModuleLoadData(&k->module, code.data()));
+        hipError_t e = hipModuleLoadData(&k->module, code.data());
+        if (e != hipSuccess && from_disk) {
+            // a cached file that does not load (truncated by a full disk, written by another build): drop it,
+            // build from source and try once more
+            (void)hipGetLastError();
+            unlink(path.c_str());
+            code = compile_source(source, entry + ".hip");
+            g_jit_compiled++;
+            store_code(path, code);
+            e = hipModuleLoadData(&k->module, code.data());
+        }
+        if (e != hipSuccess) {
+            delete k;
+            MJT_FAIL(MJT_ERR_DEVICE, "hipModuleLoadData(" << entry << "): " << hipGetErrorString(e));
+        }
         HIP_CHECK(hipModuleGetFunction(&k->fn, k->module, entry.c_str()));
     }
     g_jit_cache.emplace(source, k);
