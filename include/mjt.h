@@ -31,7 +31,8 @@ typedef enum {
     MJT_ERR_UNSUPPORTED = -2,
     MJT_ERR_COMPILE = -3,   /* runtime kernel specialisation failed */
     MJT_ERR_DEVICE = -4,    /* HIP runtime error */
-    MJT_ERR_NOT_INIT = -5
+    MJT_ERR_NOT_INIT = -5,
+    MJT_ERR_NOT_READY = -6  /* an allocation-free entry point would have to build or load a kernel */
 } mjt_status;
 
 /* dtype codes: order of misc/nano_string.h:17-31 */
@@ -119,6 +120,24 @@ int mjt_event_destroy(void* ev);
  * in y->dtype starting from the identity init_OP
  * (type/common_op_type.cc:116-117,142-151: lowest()/max() for max/min). */
 int mjt_reduce(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask);
+
+/* mjt_reduce for callers that may not allocate device memory (code under HIP
+ * graph capture, serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, same kernels and the same
+ * results as mjt_reduce; the partial results of a two-pass reduction go to a
+ * fixed array in device memory (MJT_STATIC_SCRATCH_BYTES per device, held
+ * until the process ends) instead of the growing scratch arena.  The call
+ * allocates nothing: a reduction whose partial results need more than the
+ * array holds fails with MJT_ERR_UNSUPPORTED, and one whose kernels are not
+ * loaded yet with MJT_ERR_NOT_READY (run mjt_reduce once with a descriptor
+ * of the same dtypes, op, mask and shape beforehand, outside the region that
+ * may not allocate: building and loading a kernel allocates).  All calls on a
+ * device share the array: calls that overlap in time on one device race;
+ * calls queued on the library's stream do not overlap.  Nothing in the array
+ * has to be cleared between calls (every partial result is written before
+ * it is read). */
+#define MJT_STATIC_SCRATCH_BYTES (4u << 20)
+int mjt_reduce_static(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask);
 
 /* ---- ReindexOp: ops/reindex_op.cc:111-139 -----------------------------
  * y[i..] = overflow ? Tx(overflow_value) : x[idx_0(i..), ..., idx_{XDIM-1}(i..)]

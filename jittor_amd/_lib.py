@@ -90,7 +90,7 @@ EXPORTS = ["mjt_init", "mjt_shutdown", "mjt_last_error", "mjt_get_device_info",
            "mjt_dtype_name", "mjt_op_name", "mjt_dtype_from_name", "mjt_op_from_name",
            "mjt_alloc", "mjt_free", "mjt_h2d", "mjt_d2h", "mjt_d2d", "mjt_fill_u32",
            "mjt_sync", "mjt_event_create", "mjt_event_record", "mjt_event_elapsed_ms",
-           "mjt_event_destroy", "mjt_reduce", "mjt_reindex", "mjt_reindex_reduce",
+           "mjt_event_destroy", "mjt_reduce", "mjt_reduce_static", "mjt_reindex", "mjt_reindex_reduce",
            "mjt_fused_elementwise", "mjt_fused_reduce", "mjt_conv2d_meta", "mjt_conv2d_meta_grouped", "mjt_conv2d_meta_wgrad", "mjt_conv2d_meta_wgrad_grouped",
            "mjt_reindex_then_reduce", "mjt_fused_reindex_reduce", "mjt_matmul", "mjt_matmul_available",
            "mjt_expr_affine",
@@ -125,6 +125,7 @@ def load():
     lib.mjt_event_elapsed_ms.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]
     lib.mjt_event_destroy.argtypes = [ctypes.c_void_p]
     lib.mjt_reduce.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.c_int, ctypes.c_uint32]
+    lib.mjt_reduce_static.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.c_int, ctypes.c_uint32]
     strs = ctypes.POINTER(ctypes.c_char_p)
     lib.mjt_reindex.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.c_int, strs,
                                 ctypes.c_double, ctypes.c_int, strs, ctypes.c_int, ctypes.POINTER(Tensor)]

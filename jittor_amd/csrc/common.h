@@ -94,6 +94,10 @@ struct JitKernel {
 // Compiles `source` (which must define extern "C" __global__ `entry`) for the
 // current device, or returns the cached kernel for an identical source.
 JitKernel* jit_get(const std::string& source, const std::string& entry);
+// The cached kernel for `source`, or nullptr: never compiles, never loads.
+JitKernel* jit_lookup(const std::string& source);
+// per-device set-up of the fixed scratch array behind mjt_reduce_static (op_reduce.cpp); called by mjt_init
+void reduce_static_setup(int device);
 // Launch with a parameter block of 8-byte words.
 void jit_launch(JitKernel* k, unsigned grid_x, unsigned grid_y, unsigned block, unsigned shmem,
                 const std::vector<uint64_t>& args);

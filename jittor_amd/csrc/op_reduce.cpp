@@ -48,13 +48,21 @@ struct Prologue {
 // 16-bit float results are accumulated in float32 and rounded once, at the store
 int acc_dtype(int ty) { return ty == MJT_FLOAT16 || ty == MJT_BFLOAT16 ? MJT_FLOAT32 : ty; }
 
+// The fixed scratch array behind mjt_reduce_static.  In host code the array's name is only a handle: its device
+// address is looked up once per device (every device holds its own copy at its own address) and that pointer is
+// what kernels get.
+static __device__ __align__(256) __attribute__((used)) unsigned char g_static_scratch[MJT_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+void* g_static_ptr[kMaxDevices] = {};
+
 struct Variant {
     int tx, ty, op, nk, nr, vec, g, unr, nt;
     bool row, split, use64, second;   // second: folding partials (TX == TY, plain merge)
     const Prologue* pro;
 };
 
-JitKernel* get_kernel(const Variant& v) {
+// may_build == false: only a kernel that is already loaded is returned (no compiler, no module load)
+JitKernel* get_kernel(const Variant& v, bool may_build = true) {
     std::ostringstream key;
     key << v.tx << "," << v.ty << "," << v.op << "," << v.nk << "," << v.nr << "," << v.vec << "," << v.g << ","
         << v.row << v.split << v.use64 << v.second << "," << v.unr << "," << v.nt;
@@ -93,7 +101,10 @@ JitKernel* get_kernel(const Variant& v) {
     src << "#define INIT mjt_init_" << merge_op << "<TACC>()\n";
     if (v.pro) src << v.pro->defs;
     src << embedded_source("prelude.h") << "\n" << embedded_source("reduce.h") << "\n";
-    JitKernel* k = jit_get(src.str(), name.str());
+    JitKernel* k = may_build ? jit_get(src.str(), name.str()) : jit_lookup(src.str());
+    if (!k)
+        throw Error{MJT_ERR_NOT_READY, "reduce: kernel " + name.str() + " is not loaded yet and this entry point may not build it: "
+                                       "call mjt_reduce once with a descriptor of the same kind first"};
     g_kernels.emplace(key.str(), k);
     return k;
 }
@@ -135,11 +146,11 @@ void fill_axes(std::vector<uint64_t>& a, const std::vector<Axis>& kept, const st
 // S > 1) are written to `out` as [O, S] (row) or [S, O] (column).
 void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* out, int64_t O, int64_t S,
             const std::vector<Axis>& kept, const std::vector<Axis>& red, double rcount, bool use64, int vec, int g,
-            int64_t per, int64_t total, bool stream = false, const Prologue* pro = nullptr) {
+            int64_t per, int64_t total, bool stream = false, const Prologue* pro = nullptr, bool may_build = true) {
     // inputs larger than the caches are streamed (read once, non-temporal loads)
     Variant v{tx, ty, op, (int)kept.size(), (int)red.size(), vec, g, env_int("MJT_REDUCE_UNR", 8),
               env_int("MJT_REDUCE_NT", stream ? 1 : 0), row, S > 1, use64, second, pro};
-    JitKernel* k = get_kernel(v);
+    JitKernel* k = get_kernel(v, may_build);
     std::vector<uint64_t> a(8 + 6 * 5, 0);
     a[0] = bits_of_ptr(x);
     a[1] = bits_of_ptr(out);
@@ -157,8 +168,22 @@ void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* 
 
 }  // namespace
 
-void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask, const Prologue* pro) {
+// fixed_scratch: the allocation-free variant (partials in the fixed array, only kernels that are already loaded)
+void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask, const Prologue* pro,
+                 bool fixed_scratch = false) {
     require_init();
+    const bool mb = !fixed_scratch;
+    auto partials = [&](size_t bytes) -> void* {
+        if (!fixed_scratch) return scratch(bytes);
+        Context& cc = ctx();
+        if (bytes > MJT_STATIC_SCRATCH_BYTES)
+            MJT_FAIL(MJT_ERR_UNSUPPORTED, "mjt_reduce_static: this reduction is split into " << bytes << " bytes of partial results; "
+                                          "the fixed scratch array holds " << MJT_STATIC_SCRATCH_BYTES << " (use mjt_reduce)");
+        if (cc.dry_run) return (void*)(uintptr_t)0x1000;
+        void* ptr = cc.device >= 0 && cc.device < kMaxDevices ? g_static_ptr[cc.device] : nullptr;
+        if (!ptr) MJT_FAIL(MJT_ERR_NOT_INIT, "mjt_reduce_static: the fixed scratch array was not set up on device " << cc.device);
+        return ptr;
+    };
     if (!pro) check_tensor(x, "reduce x");
     check_tensor(y, "reduce y");
     MJT_CHECK(op >= 0 && op < MJT_OP_COUNT && reducible(op),
@@ -210,7 +235,7 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         std::vector<Axis> r1{Axis{xn == 0 ? 0 : 1, 0}};
         std::vector<Axis> k1{Axis{O, 1}};
         launch(false, tx, ty, op, false, x->ptr ? x->ptr : y->ptr, y->ptr, O, 1, k1, r1, rcount, O >= (int64_t(1) << 31), 1, 1,
-               r1[0].size, r1[0].size, false, xn ? pro : nullptr);
+               r1[0].size, r1[0].size, false, xn ? pro : nullptr, mb);
         return;
     }
     bool use64 = xn >= (int64_t(1) << 31);
@@ -242,17 +267,17 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         int64_t per = (total + S - 1) / S;
         S = (total + per - 1) / per;
         if (S == 1) {
-            launch(true, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, g, per, total, stream, pro);
+            launch(true, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, g, per, total, stream, pro, mb);
         } else {
-            void* part = scratch((size_t)O * S * asz);
-            launch(true, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, g, per, total, stream, pro);
+            void* part = partials((size_t)O * S * asz);
+            launch(true, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, g, per, total, stream, pro, mb);
             // fold [O, S] along the last axis
             std::vector<Axis> k2{Axis{O, S}}, r2{Axis{S, 1}};
             int vec2 = pick_vec(asz, S, part, nullptr, 0);
             int g2 = 64;
             while (g2 > 1 && (int64_t)(g2 / 2) * vec2 >= S) g2 /= 2;
             int64_t nL2 = (S + (int64_t)g2 * vec2 - 1) / ((int64_t)g2 * vec2);
-            launch(true, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, g2, nL2, nL2);
+            launch(true, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, g2, nL2, nL2, false, nullptr, mb);
         }
     } else {
         int64_t Lk = kept.back().size;
@@ -273,19 +298,29 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         int64_t per = (R + S - 1) / S;
         S = (R + per - 1) / per;
         if (S == 1) {
-            launch(false, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, 1, per, R, stream, pro);
+            launch(false, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, 1, per, R, stream, pro, mb);
         } else {
-            void* part = scratch((size_t)O * S * asz);
-            launch(false, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R, stream, pro);
+            void* part = partials((size_t)O * S * asz);
+            launch(false, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R, stream, pro, mb);
             std::vector<Axis> k2{Axis{O, 1}}, r2{Axis{S, O}};
             int vec2 = pick_vec(asz, O, part, y->ptr, tsz);
-            launch(false, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, 1, S, S);
+            launch(false, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, 1, S, S, false, nullptr, mb);
         }
     }
 }
 
 void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask) {
     reduce_core(x, y, op, reduce_mask, nullptr);
+}
+
+// Looks up where this device keeps the fixed scratch array.  Runs once per device, with that device current
+// (mjt_init calls it after hipSetDevice).
+void reduce_static_setup(int device) {
+    MJT_CHECK(device >= 0 && device < kMaxDevices, "device " << device << " is outside the table of fixed scratch arrays");
+    if (g_static_ptr[device]) return;
+    void* ptr = nullptr;
+    HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch)));
+    g_static_ptr[device] = ptr;
 }
 
 // Reduce whose input is produced element by element from other tensors: the group's single output var
@@ -377,6 +412,10 @@ void fused_reduce_impl(const mjt_fused_desc* d, const mjt_tensor* y, int op, uin
 
 extern "C" int mjt_fused_reduce(const mjt_fused_desc* desc, const mjt_tensor* y, int op, uint32_t reduce_mask) {
     return mjt::guarded([&] { mjt::fused_reduce_impl(desc, y, op, reduce_mask); });
+}
+
+extern "C" int mjt_reduce_static(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask) {
+    return mjt::guarded([&] { mjt::reduce_core(x, y, op, reduce_mask, nullptr, true); });
 }
 
 extern "C" int mjt_reduce(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t reduce_mask) {

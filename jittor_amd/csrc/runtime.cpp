@@ -243,6 +243,12 @@ JitKernel* jit_get(const std::string& source, const std::string& entry) {
     return k;
 }
 
+JitKernel* jit_lookup(const std::string& source) {
+    std::lock_guard<std::mutex> lock(g_jit_mutex);
+    auto it = g_jit_cache.find(source);
+    return it == g_jit_cache.end() ? nullptr : it->second;
+}
+
 void jit_launch(JitKernel* k, unsigned grid_x, unsigned grid_y, unsigned block, unsigned shmem,
                 const std::vector<uint64_t>& args) {
     size_t size = args.size() * sizeof(uint64_t);
@@ -286,6 +292,7 @@ int mjt_init(int device) {
         MJT_CHECK(strncmp(c.prop.gcnArchName, "gfx950", 6) == 0,
                   "mjt_init: this library is built for gfx950 only; device is " << c.prop.gcnArchName);
         HIP_CHECK(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
+        reduce_static_setup(device);
         c.device = device;
         c.ready = true;
     });
