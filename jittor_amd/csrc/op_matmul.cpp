@@ -1,62 +1,127 @@
-// Plain matrix product behind the reference's matmul relay.
+// Matrix product behind the reference's matmul relay.
 //
 // The reference recognises broadcast * broadcast -> reduce.add over 2-d
 // operands (opt/tuner/matmul_tuner.cc:16-104) and relays it to a library GEMM:
 // cublas_matmul(a, b, trans_a, trans_b) on the GPU
-// (extern/cuda/cublas/ops/cublas_matmul_op.cc:27-56, one GemmEx call with the
-// row-major operands swapped, :118-126).  The counterpart here is rocBLAS'
-// gemm_ex, opened on first use so that a process that never multiplies matrices
-// never loads the library.  Float accumulation for every input type.
+// (extern/cuda/cublas/ops/cublas_matmul_op.cc:27-56, batched form
+// cublas_batched_matmul_op.cc:63-85).  Here the product runs on the library's
+// own kernels: kernels/gemm_mfma.h (MFMA, LDS-tiled; bfloat16, float16 and
+// float32 operands whose rows are 16-byte aligned) and kernels/gemm_plain.h
+// (everything else, float64 included).  Float accumulation for every input
+// type (double for float64).
 #include "common.h"
-#include <dlfcn.h>
+#include <cmath>
 #include <mutex>
-#include <rocblas/rocblas.h>
+#include <unordered_map>
 
 namespace mjt {
 
 void launch_fill_pattern(void* dst, uint64_t pattern, int elem_size, size_t n);
 
 namespace {
-struct Blas {
-    void* so = nullptr;
-    rocblas_handle handle = nullptr;
-    decltype(&rocblas_create_handle) create = nullptr;
-    decltype(&rocblas_set_stream) set_stream = nullptr;
-    decltype(&rocblas_gemm_ex) gemm_ex = nullptr;
-    decltype(&rocblas_gemm_strided_batched_ex) gemm_batched = nullptr;
-    bool tried = false;
-};
-Blas g_blas;
 std::mutex g_mu;
-
-bool blas_load() {
+std::unordered_map<std::string, JitKernel*> g_kernels;
+void forget() {   // the kernels belong to the run-time compiler's cache, which mjt_shutdown empties
     std::lock_guard<std::mutex> lock(g_mu);
-    if (g_blas.tried) return g_blas.gemm_ex != nullptr;
-    g_blas.tried = true;
-    const char* names[] = {"librocblas.so.5", "librocblas.so", "/opt/rocm/lib/librocblas.so"};
-    for (const char* n : names) {
-        g_blas.so = dlopen(n, RTLD_NOW | RTLD_LOCAL);
-        if (g_blas.so) break;
-    }
-    if (!g_blas.so) return false;
-    g_blas.create = (decltype(g_blas.create))dlsym(g_blas.so, "rocblas_create_handle");
-    g_blas.set_stream = (decltype(g_blas.set_stream))dlsym(g_blas.so, "rocblas_set_stream");
-    auto gemm = (decltype(g_blas.gemm_ex))dlsym(g_blas.so, "rocblas_gemm_ex");
-    g_blas.gemm_batched = (decltype(g_blas.gemm_batched))dlsym(g_blas.so, "rocblas_gemm_strided_batched_ex");
-    if (!g_blas.create || !g_blas.set_stream || !gemm || !g_blas.gemm_batched) return false;
-    g_blas.gemm_ex = gemm;
-    return true;
+    g_kernels.clear();
 }
+const bool g_registered = (at_shutdown(&forget), true);
 
-rocblas_datatype blas_type(int dtype) {
-    switch (dtype) {
-        case MJT_FLOAT32: return rocblas_datatype_f32_r;
-        case MJT_FLOAT64: return rocblas_datatype_f64_r;
-        case MJT_FLOAT16: return rocblas_datatype_f16_r;
-        default: return rocblas_datatype_bf16_r;
-    }
+JitKernel* cached(const std::string& key) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_kernels.find(key);
+    return it == g_kernels.end() ? nullptr : it->second;
+}
+void remember(const std::string& key, JitKernel* k) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_kernels.emplace(key, k);
+}
+int env_int(const char* name, int dflt) {
+    const char* v = getenv(name);
+    return v && *v ? atoi(v) : dflt;
 }
 }  // namespace
+
+// One strided-batched product C[b] = A'[b] * B'[b] over plain pointers: M x K times K x N, leading dimensions and
+// batch strides in elements (a batch stride of 0 shares the operand).  a_kcont / b_kcont: the operand's memory has
+// k innermost (a as given, b transposed).
+void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                 int64_t lda, int64_t ldb, int64_t ldc, int64_t sa, int64_t sb, int64_t sc, int64_t batch, bool a_kcont,
+                 bool b_kcont) {
+    Context& c = ctx();
+    const int esz = dtype_size(in_dtype);
+    const bool mfma_type = in_dtype == MJT_BFLOAT16 || in_dtype == MJT_FLOAT16 || in_dtype == MJT_FLOAT32;
+    const bool out_ok = out_dtype == MJT_FLOAT32 || (out_dtype == in_dtype && esz == 2);
+    auto al16 = [&](const void* p, int64_t ld, int64_t stride) {
+        return (uintptr_t)p % 16 == 0 && (ld * esz) % 16 == 0 && (stride * esz) % 16 == 0;
+    };
+    const bool fast = mfma_type && out_ok && !getenv("MJT_GEMM_PLAIN") && al16(A, lda, sa) && al16(B, ldb, sb) &&
+                      M < (int64_t(1) << 31) && N < (int64_t(1) << 31) && K < (int64_t(1) << 31) && batch < 65536;
+    std::vector<uint64_t> args{bits_of_ptr(A), bits_of_ptr(B), bits_of_ptr(C), (uint64_t)M, (uint64_t)N, (uint64_t)K,
+                               (uint64_t)lda, (uint64_t)ldb, (uint64_t)ldc, (uint64_t)sa, (uint64_t)sb, (uint64_t)sc};
+    if (fast) {
+        // Tile: the largest of 64 MI x 64 NI (MI, NI in 1, 2, 4) that still gives every compute unit work and wastes
+        // little on the edges; larger tiles read each operand element less often.
+        const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
+        int best_mi = 1, best_ni = 1;
+        double best = -1.0;
+        for (int mi = 4; mi >= 1; mi /= 2)
+            for (int ni = 4; ni >= 1; ni /= 2) {
+                const int64_t tm = (M + 64 * mi - 1) / (64 * mi), tn = (N + 64 * ni - 1) / (64 * ni);
+                const double tiles = (double)tm * tn * batch;
+                const double edge = ((double)M * N) / ((double)tm * 64 * mi * tn * 64 * ni);
+                const double waves = std::ceil(tiles / cus);
+                const double util = tiles / (waves * cus);
+                const double reuse = 1.0 / (1.0 / (64.0 * mi) + 1.0 / (64.0 * ni)) / 128.0;   // 1 for 256 x 256
+                const double score = edge * util * (0.55 + 0.45 * reuse);
+                if (score > best) { best = score; best_mi = mi; best_ni = ni; }
+            }
+        int MI = env_int("MJT_GEMM_MI", best_mi), NI = env_int("MJT_GEMM_NI", best_ni);
+        if ((MI != 1 && MI != 2 && MI != 4) || (NI != 1 && NI != 2 && NI != 4)) { MI = best_mi; NI = best_ni; }
+        const int in = in_dtype == MJT_BFLOAT16 ? 0 : in_dtype == MJT_FLOAT16 ? 1 : 2;
+        const int out = out_dtype == MJT_BFLOAT16 ? 0 : out_dtype == MJT_FLOAT16 ? 1 : 2;
+        std::ostringstream key;
+        key << "gemm|" << in << out << MI << NI << a_kcont << b_kcont;
+        JitKernel* k = cached(key.str());
+        if (!k) {
+            std::ostringstream name;
+            name << "mjt_gemm_mfma_" << mjt_dtype_name(in_dtype) << "_" << mjt_dtype_name(out_dtype) << "_" << 64 * MI << "x" << 64 * NI
+                 << (a_kcont ? "_n" : "_t") << (b_kcont ? "t" : "n");
+            std::ostringstream src;
+            src << "#define ENTRY " << name.str() << "\n#define IN " << in << "\n#define OUT " << out << "\n#define MI " << MI
+                << "\n#define NI " << NI << "\n#define A_KCONT " << (a_kcont ? 1 : 0) << "\n#define B_KCONT " << (b_kcont ? 1 : 0) << "\n";
+            src << embedded_source("gemm_mfma.h") << "\n";
+            k = jit_get(src.str(), name.str());
+            remember(key.str(), k);
+        }
+        const int64_t tiles = ((M + 64 * MI - 1) / (64 * MI)) * ((N + 64 * NI - 1) / (64 * NI));
+        const int64_t grid = (tiles + 7) / 8 * 8;
+        MJT_CHECK(grid < (int64_t(1) << 31), "matmul: launch too large");
+        jit_launch(k, (unsigned)grid, (unsigned)batch, 256, 0, args);
+        return;
+    }
+    std::ostringstream key;
+    key << "gemmp|" << in_dtype << "|" << out_dtype << a_kcont << b_kcont;
+    JitKernel* k = cached(key.str());
+    if (!k) {
+        std::ostringstream name;
+        name << "mjt_gemm_plain_" << mjt_dtype_name(in_dtype) << "_" << mjt_dtype_name(out_dtype) << (a_kcont ? "_n" : "_t") << (b_kcont ? "t" : "n");
+        std::ostringstream src;
+        src << "#define ENTRY " << name.str() << "\n#define TIN " << dtype_cname(in_dtype) << "\n#define TOUT " << dtype_cname(out_dtype)
+            << "\n#define TACC " << (in_dtype == MJT_FLOAT64 ? "double" : "float") << "\n#define A_KCONT " << (a_kcont ? 1 : 0)
+            << "\n#define B_KCONT " << (b_kcont ? 1 : 0) << "\n";
+        src << embedded_source("prelude.h") << "\n" << embedded_source("gemm_plain.h") << "\n";
+        k = jit_get(src.str(), name.str());
+        remember(key.str(), k);
+    }
+    MJT_CHECK(batch < 65536 && (M + 63) / 64 < 65536, "matmul: launch too large");
+    set_last_kernel(k->name.c_str());
+    if (c.dry_run) return;
+    size_t size = args.size() * sizeof(uint64_t);
+    void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, (void*)args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+    HIP_CHECK(hipModuleLaunchKernel(k->fn, (unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)batch, 256, 1, 1, 0, c.stream,
+                                    nullptr, config));
+}
 
 // With `share_a` every matrix of the batch is multiplied by the first matrix of a (batch stride 0: the weights of a
 // convolution against the column matrices of a chunk of images).
@@ -87,44 +152,21 @@ void matmul_impl(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, 
     if (batch == 0) return;
     if (n == 0 || k == 0) return;
     Context& ctxt = ctx();
-    if (ctxt.dry_run) return;
-    MJT_CHECK(a->ptr && b->ptr && c->ptr, "matmul: null data");
+    if (!ctxt.dry_run) MJT_CHECK(a->ptr && b->ptr && c->ptr, "matmul: null data");
     if (m == 0) {                                             // an empty sum
-        launch_fill_pattern(c->ptr, 0, dtype_size(c->dtype), (size_t)batch * n * k);
+        if (!ctxt.dry_run) launch_fill_pattern(c->ptr, 0, dtype_size(c->dtype), (size_t)batch * n * k);
         return;
     }
-    if (!blas_load()) MJT_FAIL(MJT_ERR_UNSUPPORTED, "matmul: rocBLAS is not available");
-    {
-        std::lock_guard<std::mutex> lock(g_mu);
-        if (!g_blas.handle && g_blas.create(&g_blas.handle) != rocblas_status_success)
-            MJT_FAIL(MJT_ERR_DEVICE, "matmul: rocblas_create_handle failed");
-        // every call: the library's stream changes when it is shut down and bound again
-        if (g_blas.set_stream(g_blas.handle, ctxt.stream) != rocblas_status_success) MJT_FAIL(MJT_ERR_DEVICE, "matmul: rocblas_set_stream failed");
+    // c[n,k] = a'[n,m] * b'[m,k]: rows n, columns k, sum over m
+    const int64_t lda = a->shape[nd - 1], ldb = b->shape[nd - 1];
+    const int64_t per_launch = 65535;                         // the batch rides on a grid axis
+    for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
+        const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
+        const char* pa = (const char*)a->ptr + (share_a ? 0 : b0 * n * m * dtype_size(a->dtype));
+        const char* pb = (const char*)b->ptr + b0 * m * k * dtype_size(b->dtype);
+        char* pc = (char*)c->ptr + b0 * n * k * dtype_size(c->dtype);
+        gemm_launch(a->dtype, c->dtype, pa, pb, pc, n, k, m, lda, ldb, k, share_a ? 0 : n * m, m * k, n * k, nb, !trans_a, trans_b != 0);
     }
-    // Row-major c[n,k] = a * b is column-major c^T[k,n] = b^T * a^T: the operands trade places and keep
-    // their own transposition flags (cublas_matmul_op.cc:118-126).
-    const float alpha_f = 1.0f, beta_f = 0.0f;
-    const double alpha_d = 1.0, beta_d = 0.0;
-    const bool f64 = a->dtype == MJT_FLOAT64;
-    const void* alpha = f64 ? (const void*)&alpha_d : (const void*)&alpha_f;
-    const void* beta = f64 ? (const void*)&beta_d : (const void*)&beta_f;
-    const rocblas_operation opb = trans_b ? rocblas_operation_transpose : rocblas_operation_none;
-    const rocblas_operation opa = trans_a ? rocblas_operation_transpose : rocblas_operation_none;
-    const rocblas_int ldb = (rocblas_int)(trans_b ? m : k), lda = (rocblas_int)(trans_a ? n : m);
-    const rocblas_datatype tc = f64 ? rocblas_datatype_f64_r : rocblas_datatype_f32_r;
-    rocblas_status st;
-    if (batch == 1)
-        st = g_blas.gemm_ex(g_blas.handle, opb, opa, (rocblas_int)k, (rocblas_int)n, (rocblas_int)m, alpha, b->ptr,
-                            blas_type(b->dtype), ldb, a->ptr, blas_type(a->dtype), lda, beta, c->ptr, blas_type(c->dtype),
-                            (rocblas_int)k, c->ptr, blas_type(c->dtype), (rocblas_int)k, tc, rocblas_gemm_algo_standard, 0, 0);
-    else
-        st = g_blas.gemm_batched(g_blas.handle, opb, opa, (rocblas_int)k, (rocblas_int)n, (rocblas_int)m, alpha, b->ptr,
-                                 blas_type(b->dtype), ldb, (rocblas_stride)(m * k), a->ptr, blas_type(a->dtype), lda,
-                                 (rocblas_stride)(share_a ? 0 : n * m), beta, c->ptr, blas_type(c->dtype), (rocblas_int)k,
-                                 (rocblas_stride)(n * k), c->ptr, blas_type(c->dtype), (rocblas_int)k, (rocblas_stride)(n * k),
-                                 (rocblas_int)batch, tc, rocblas_gemm_algo_standard, 0, 0);
-    if (st != rocblas_status_success) MJT_FAIL(MJT_ERR_DEVICE, "matmul: rocBLAS returned " << (int)st);
-    set_last_kernel(batch == 1 ? "rocblas_gemm_ex" : "rocblas_gemm_strided_batched_ex");
 }
 
 }  // namespace mjt
@@ -134,9 +176,7 @@ extern "C" int mjt_matmul(const mjt_tensor* a, const mjt_tensor* b, const mjt_te
 }
 
 namespace mjt {
-bool matmul_available() { return blas_load(); }
+bool matmul_available() { return true; }
 }  // namespace mjt
 
-extern "C" int mjt_matmul_available(void) {
-    return mjt::blas_load() ? 1 : 0;
-}
+extern "C" int mjt_matmul_available(void) { return 1; }
