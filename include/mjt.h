@@ -313,9 +313,11 @@ int mjt_conv2d_meta_wgrad_grouped(const mjt_tensor* x, const mjt_tensor* dy, con
  * With more than two dims the leading extents must be equal on a, b and c and
  * count as a batch of products (cublas_batched_matmul_op.cc:63-85,113-166).
  * c has the inputs' dtype, or float32 for 16-bit inputs; the accumulator is
- * float32 (float64 for float64).  The product itself is rocBLAS' gemm_ex,
- * loaded on first use: MJT_ERR_UNSUPPORTED when the library is absent, and
- * mjt_matmul_available() tells beforehand (1 / 0). */
+ * float32 (float64 for float64).  The product runs on the library's own
+ * kernels: an LDS-tiled MFMA kernel for bfloat16 / float16 / float32 operands
+ * whose rows are multiples of 16 bytes, a plain kernel for the rest (float64,
+ * unaligned rows).  mjt_matmul_available() is kept for callers written
+ * against an earlier build that relayed to a vendor library: it returns 1. */
 int mjt_matmul(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, int trans_a, int trans_b);
 int mjt_matmul_available(void);
 

@@ -62,6 +62,9 @@ void* conv_scratch(int which, size_t bytes) {
 
 void matmul_impl(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, int trans_a, int trans_b, bool share_a);
 bool matmul_available();
+void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                 int64_t lda, int64_t ldb, int64_t ldc, int64_t sa, int64_t sb, int64_t sc, int64_t batch, bool a_kcont,
+                 bool b_kcont);
 
 void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p, int64_t G) {
     require_init();
@@ -212,27 +215,24 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         return;
     }
 
-    // ---- column matrices + library GEMM -----------------------------------------------
-    // What the MFMA kernel does not take (float32, widths that are no multiple of 8, strides) and is large enough to
-    // matter: y[n] [K, P] = w [K, C*R*S] x cols[n] [C*R*S, P], cols = the shifted input planes written by one reindex per
-    // chunk of images (a 1x1 convolution of stride 1 without padding reads x itself).  A bfloat16 result goes through
-    // a float32 copy so that it is narrowed the way every other kernel narrows it (by truncation), not rounded by the library.
+    // ---- column matrices x weights on the GEMM kernel -----------------------------------
+    // What the MFMA convolution kernel does not take (float32, odd widths, channel counts that are no multiple of 64,
+    // tiles that do not fit) and is large enough to matter: y[n] [K, P] = w [K, C*R*S] x cols[n] [C*R*S, P], cols = the
+    // shifted input planes written by one reindex per chunk of images (a 1x1 convolution of stride 1 without padding
+    // reads x itself), the product on kernels/gemm_mfma.h with the weights shared across the batch.  Rows of cols are
+    // padded to a multiple of 16 bytes when the pixel count is not one (the GEMM kernel's fast path wants aligned rows).
     const int64_t P = OH * OW, CRS = C * R * S;
     if (G == 1 && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_GEMM") && (double)N * K * P * CRS >= (double)(1 << 22) &&
         P < (int64_t(1) << 31) && CRS < (int64_t(1) << 31) && matmul_available()) {
         const int64_t esz = dtype_size(x->dtype);
-        const bool plain = R == 1 && S == 1 && p->stride_h == 1 && p->stride_w == 1 && p->pad_h == 0 && p->pad_w == 0;
-        const bool via_f32 = y->dtype == MJT_BFLOAT16;
-        int64_t chunk = (int64_t(1) << 30) / (CRS * P * esz);
+        const int64_t Ppad = (P * esz + 15) / 16 * 16 / esz;
+        const bool plain = R == 1 && S == 1 && p->stride_h == 1 && p->stride_w == 1 && p->pad_h == 0 && p->pad_w == 0 && Ppad == P;
+        int64_t chunk = (int64_t(1) << 30) / (CRS * Ppad * esz);
         if (const char* e = getenv("MJT_CONV_GEMM_CHUNK"))      // images per chunk, for tests of the chunk loop
             if (atoi(e) >= 1) chunk = atoi(e);
         if (chunk < 1) chunk = 1;
         if (chunk > N) chunk = N;
-        void* cols = plain ? nullptr : conv_scratch(0, (size_t)(chunk * CRS * P * esz));
-        void* ytmp = via_f32 ? conv_scratch(1, (size_t)(chunk * K * P * 4)) : nullptr;
-        std::string sh = "i4*" + std::to_string(p->stride_h) + "-" + std::to_string(p->pad_h) + "+i2*" + std::to_string(p->dil_h);
-        std::string sw = "i5*" + std::to_string(p->stride_w) + "-" + std::to_string(p->pad_w) + "+i3*" + std::to_string(p->dil_w);
-        const char* idx[4] = {"i0", "i1", sh.c_str(), sw.c_str()};
+        void* cols = plain ? nullptr : conv_scratch(0, (size_t)(chunk * CRS * Ppad * esz));
         auto view = [](void* ptr, int dtype, std::initializer_list<int64_t> shape) {
             mjt_tensor t;
             memset(&t, 0, sizeof(t));
@@ -241,23 +241,31 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             for (int64_t e : shape) t.shape[t.ndim++] = e;
             return t;
         };
+        // index strings of the column matrices: [n, c, kh, kw, oh, ow] when a row needs no padding (the window
+        // pattern of the reindex fast path), else [n, c, kh, kw, pixel] with the pixel split by division and
+        // remainder and the padding marked as overflow
+        std::string sh, sw, over;
+        if (Ppad == P) {
+            sh = "i4*" + std::to_string(p->stride_h) + "-" + std::to_string(p->pad_h) + "+i2*" + std::to_string(p->dil_h);
+            sw = "i5*" + std::to_string(p->stride_w) + "-" + std::to_string(p->pad_w) + "+i3*" + std::to_string(p->dil_w);
+        } else {
+            sh = "i4/" + std::to_string(OW) + "*" + std::to_string(p->stride_h) + "-" + std::to_string(p->pad_h) + "+i2*" + std::to_string(p->dil_h);
+            sw = "i4%" + std::to_string(OW) + "*" + std::to_string(p->stride_w) + "-" + std::to_string(p->pad_w) + "+i3*" + std::to_string(p->dil_w);
+            over = "i4>=" + std::to_string(P);
+        }
+        const char* idx[4] = {"i0", "i1", sh.c_str(), sw.c_str()};
+        const char* ovc[1] = {over.c_str()};
         for (int64_t n0 = 0; n0 < N; n0 += chunk) {
             const int64_t nb = N - n0 < chunk ? N - n0 : chunk;
             char* xn = (char*)x->ptr + n0 * C * H * W * esz;
             if (!plain) {
-                mjt_tensor tx = view(xn, x->dtype, {nb, C, H, W}), tc = view(cols, x->dtype, {nb, C, R, S, OH, OW});
-                if (mjt_reindex(&tx, &tc, 4, idx, 0.0, 0, nullptr, 0, nullptr) != MJT_OK)
+                mjt_tensor tx = view(xn, x->dtype, {nb, C, H, W});
+                mjt_tensor tc = Ppad == P ? view(cols, x->dtype, {nb, C, R, S, OH, OW}) : view(cols, x->dtype, {nb, C, R, S, Ppad});
+                if (mjt_reindex(&tx, &tc, 4, idx, 0.0, Ppad == P ? 0 : 1, ovc, 0, nullptr) != MJT_OK)
                     MJT_FAIL(MJT_ERR_DEVICE, "conv: writing the column matrices failed: " << mjt_last_error());
             }
             char* yn = (char*)y->ptr + n0 * K * P * dtype_size(y->dtype);
-            mjt_tensor ta = view(w->ptr, w->dtype, {nb, K, CRS}), tb = view(plain ? (void*)xn : cols, x->dtype, {nb, CRS, P});
-            mjt_tensor tc = view(via_f32 ? ytmp : (void*)yn, via_f32 ? MJT_FLOAT32 : y->dtype, {nb, K, P});
-            matmul_impl(&ta, &tb, &tc, 0, 0, true);
-            if (via_f32) {
-                mjt_tensor ts = view(ytmp, MJT_FLOAT32, {1, nb * K * P}), td = view(yn, y->dtype, {nb * K * P});
-                if (mjt_reduce(&ts, &td, MJT_OP_ADD, 0b01) != MJT_OK)
-                    MJT_FAIL(MJT_ERR_DEVICE, "conv: narrowing the result failed: " << mjt_last_error());
-            }
+            gemm_launch(x->dtype, y->dtype, w->ptr, plain ? (void*)xn : cols, yn, K, P, CRS, CRS, Ppad, P, 0, CRS * Ppad, K * P, nb, true, false);
         }
         set_last_kernel(plain ? "conv_as_gemm" : "conv_as_reindex_gemm");
         return;

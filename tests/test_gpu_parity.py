@@ -547,12 +547,15 @@ def test_conv_direct_small_shapes_and_fp32(gpu):
     dict(dt="float32", x=(3, 16, 30, 27), w=(48, 16, 3, 2), p=(2, 1, 1, 0, 1, 2), chunk=2),       # chunks of 2 + 1 images
     dict(dt="bfloat16", x=(2, 64, 27, 27), w=(128, 64, 3, 3), p=(2, 2, 1, 1, 1, 1), out="bfloat16"),   # odd width
     dict(dt="bfloat16", x=(2, 48, 14, 14), w=(64, 48, 3, 3), p=(1, 1, 1, 1, 1, 1)),                     # channels no multiple of 64
-    dict(dt="float16", x=(4, 64, 14, 14), w=(96, 64, 1, 1), p=(1, 1, 0, 0, 1, 1), out="float16", plain=True),
+    dict(dt="float16", x=(4, 64, 14, 14), w=(96, 64, 1, 1), p=(1, 1, 0, 0, 1, 1), out="float16"),   # 196 pixels: rows of 392 bytes are padded
+    dict(dt="float16", x=(4, 64, 16, 16), w=(96, 64, 1, 1), p=(1, 1, 0, 0, 1, 1), out="float16", plain=True),
+    dict(dt="float32", x=(12, 24, 7, 7), w=(40, 24, 3, 3), p=(1, 1, 1, 1, 1, 1)),                      # 49 pixels: padded rows, k ends inside a stage
+    dict(dt="bfloat16", x=(3, 72, 9, 11), w=(40, 72, 3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16"),
     dict(dt="float32", x=(5, 40, 16, 16), w=(96, 40, 1, 1), p=(1, 1, 0, 0, 1, 1), plain=True, chunk=2),
 ])
-def test_conv_as_reindex_and_library_gemm(gpu, case, monkeypatch):
+def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
     """Shapes the MFMA kernel does not take and that are large enough to matter run as column matrices (one reindex)
-    times the weights (library GEMM, float32 accumulation): against a float64 closed form and, for float32, the
+    times the weights (the GEMM kernel, float32 accumulation): against a float64 closed form and, for float32, the
     oracle's own summation order; a bfloat16 result is truncated like everywhere else, a float16 one rounded."""
     rng = np.random.default_rng(41)
     dt = case["dt"]
@@ -581,7 +584,7 @@ def test_conv_as_reindex_and_library_gemm(gpu, case, monkeypatch):
         assert np.all(np.abs(got) <= np.abs(ref) + 1e-5 * np.abs(ref).max())
     if dt == "float32" and sh == sw and ph == pw and dh == dw_:
         assert np.abs(got - O.conv_meta(xb, wb, sh, ph, dh)).max() <= 1e-4 * np.abs(ref).max()
-    # the same call with the library path off: the direct kernel, same values to the same bound
+    # the same call with that path off: the direct kernel, same values to the same bound
     monkeypatch.setenv("MJT_CONV_NO_GEMM", "1")
     got2, kern2 = _conv_call(xb, wb, case["p"], out_dtype=out, in_dtype=dt)
     assert kern2.startswith("mjt_conv_direct")
