@@ -4,16 +4,22 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only C2]
 
 A step is one pass of one workload's hot path (one C-ABI call = one kernel, or
-a fill + kernel pair for the scatter) over synthetic input that is already
-resident in HBM.  The headline line is BASELINE.json's configs[1] (C2, the
-im2col reindex); the other configurations are reported inside the same JSON
-line under "workloads".  Each workload rotates over several buffer sets whose
-total size exceeds the 256 MB memory-side cache, so the rates are HBM rates.
+the launches of the scatter) over synthetic input that is already resident in
+HBM.  The headline line is BASELINE.json's configs[1] (C2, the im2col reindex);
+every configuration is reported inside the same JSON line under "workloads",
+and its fraction of the roofline beside the headline under "fractions" with
+the number of configurations that meet north_star's targets ("targets_met").
+Each workload rotates over buffer sets whose inputs alone exceed the 256 MB
+memory-side cache, so the rates are HBM rates.  A block of exactly --steps
+launches is timed between two HIP events; blocks are repeated until 0.2 s of
+device time per workload and the median block is reported with min and max.
 
 For every workload the line carries
-  roofline     algorithmic bytes (or flops) per launch / average launch time,
-               timed with HIP events on the library's stream, against the
-               published peak (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s)
+  roofline     algorithmic bytes (or flops) per launch / launch time of the
+               median block, timed with HIP events on the library's stream,
+               against the published peak (HBM 8 TB/s, dense bf16 MFMA
+               2.5 PFLOP/s); "traffic" = HBM bytes per launch from counter
+               runs, reported only while the kernel is the one profiled
   cpu_baseline the CPU restatement of the reference's kernel
                (oracle/oracle_kernels.cc) timed on this box's host cores.
 """
@@ -64,22 +70,40 @@ class Dev:
         self.ptrs = []
 
 
+MIN_DEVICE_SECONDS = 0.2      # a workload's blocks of `steps` launches are repeated until this much device time
+MAX_BLOCKS = 400
+LAST_SPREAD = {}
+
+
 def time_calls(L, calls, steps, warmup):
     """calls: list of zero-argument launch functions used round-robin.
-    Returns (average device ms per step, wall ms per step)."""
+    A block = exactly `steps` launches between two HIP events on the library's stream.  Blocks are repeated
+    until MIN_DEVICE_SECONDS of device time have passed (at least 3 blocks), so the figure is a sustained rate
+    and not one burst.  Returns (median device ms per step over the blocks, wall ms per step of the median
+    block); min / max / block count of the last call are left in LAST_SPREAD."""
     n = len(calls)
     for i in range(warmup):
         calls[i % n]()
     L.sync()
-    e0, e1 = L.Event(), L.Event()
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        calls[i % n]()
-    e1.record()
-    L.sync()
-    t1 = time.perf_counter()
-    return e1.elapsed_ms_since(e0) / steps, (t1 - t0) * 1e3 / steps
+    dev_ms, wall_ms = [], []
+    k = 0
+    while len(dev_ms) < 3 or (sum(dev_ms) * steps * 1e-3 < MIN_DEVICE_SECONDS and len(dev_ms) < MAX_BLOCKS):
+        e0, e1 = L.Event(), L.Event()
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(steps):
+            calls[(k + i) % n]()
+        e1.record()
+        L.sync()
+        t1 = time.perf_counter()
+        k += steps
+        dev_ms.append(e1.elapsed_ms_since(e0) / steps)
+        wall_ms.append((t1 - t0) * 1e3 / steps)
+    order = np.argsort(dev_ms)
+    mid = int(order[len(order) // 2])
+    LAST_SPREAD.clear()
+    LAST_SPREAD.update({"blocks": len(dev_ms), "kernel_ms_min": round(float(min(dev_ms)), 5), "kernel_ms_max": round(float(max(dev_ms)), 5)})
+    return float(dev_ms[mid]), float(wall_ms[mid])
 
 
 def roofline(bound, work, ms, traffic=None):
@@ -117,7 +141,7 @@ def wl_c1(L, lib, steps, warmup, with_cpu):
         calls.append(lambda tx=tx, ty=ty: L.check(lib.mjt_reduce(ctypes.byref(tx), ctypes.byref(ty), L.OP_CODE["add"], 0b10)))
     ms, wall = time_calls(L, calls, steps, warmup)
     out = {"workload": "C1 ReduceOp sum axis 1, fp32 [8192,4096]", "kernel": L.last_kernel(), "dtype": "f32",
-           "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5), "roofline": roofline("hbm", work, ms)}
+           "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5), "roofline": roofline("hbm", work, ms), **LAST_SPREAD}
     dev.release()
     if with_cpu:
         t1 = cpu_time(lambda: K.reduce_sum_axis1(x, 1))
@@ -136,14 +160,15 @@ def wl_c2(L, lib, steps, warmup, with_cpu):
     x = np.random.default_rng(0).standard_normal(xs).astype(np.float32)
     idx, e = L.c_strings(["i0", "i1", "i2+i4-1", "i3+i5-1"]), L.c_strings([])
     calls = []
-    for s in range(3):
+    sets = CACHE_BYTES // x.nbytes + 2                  # the inputs alone exceed the 256 MB memory-side cache
+    for s in range(sets):
         tx = L.tensor(dev.put(x), "float32", xs)
         ty = L.tensor(dev.empty(int(np.prod(ys)) * 4), "float32", ys)
         calls.append(lambda tx=tx, ty=ty: L.check(lib.mjt_reindex(ctypes.byref(tx), ctypes.byref(ty), 4, idx, 0.0, 0, e, 0, None)))
     ms, wall = time_calls(L, calls, steps, warmup)
     out = {"workload": "C2 ReindexOp im2col gather, fp32 [32,64,56,56] -> [32,64,56,56,3,3], 3x3 stride 1 pad 1",
            "kernel": L.last_kernel(), "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
-           "roofline": roofline("hbm", work, ms)}
+           "roofline": roofline("hbm", work, ms), **LAST_SPREAD}
     dev.release()
     if with_cpu:
         buf = np.empty(ys, np.float32)
@@ -173,7 +198,7 @@ def wl_c3(L, lib, steps, warmup, with_cpu, op):
     ms, wall = time_calls(L, calls, steps, warmup)
     out = {"workload": "C3 ReindexReduceOp scatter-%s, 2^24 fp32 values into 2^20 bins, int32 Zipf(1.1) indices" % op,
            "kernel": L.last_kernel(), "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
-           "roofline": roofline("hbm", work, ms),
+           "roofline": roofline("hbm", work, ms), **LAST_SPREAD,
            "note": "a step = the four launches of the 1-d scatter (main, plan, cold, final); the bins need no prior fill"}
     dev.release()
     if with_cpu:
@@ -227,7 +252,7 @@ def wl_c4(L, lib, steps, warmup, with_cpu):
     ms, wall = time_calls(L, calls, steps, warmup)
     out = {"workload": "C4 fused exp(-relu(x*scale+bias))*sigmoid(x), x fp32 [64,512,1024], scale [512,1], bias [1,1024]",
            "kernel": L.last_kernel(), "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
-           "roofline": roofline("hbm", work, ms)}
+           "roofline": roofline("hbm", work, ms), **LAST_SPREAD}
     dev.release()
     if with_cpu:
         sub = x[:8]                                    # 1/8 of the batch axis, scaled
@@ -261,17 +286,20 @@ def wl_c5(L, lib, steps, warmup, with_cpu, out_dtype="float32"):
     out = {"workload": "C5 meta-op conv, x bf16 [64,256,56,56], w bf16 [256,256,3,3], 3x3 s1 p1, fp32 accumulate, %s output"
                        % ("fp32" if out_dtype == "float32" else "bf16 (the dtype the reference's Var graph gives the result)"),
            "kernel": L.last_kernel(), "dtype": "bf16", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
-           "roofline": roofline("mfma", flops, ms), "note": "a step = weight repack + convolution kernel"}
+           "roofline": roofline("mfma", flops, ms), **LAST_SPREAD, "note": "a step = weight repack + convolution kernel"}
     dev.release()
     if with_cpu:
         nt = K.max_threads()
         sub = xb[:1, :, :14, :]                      # one image, 14 of 56 rows: 1/256 of the MACs (edge rows differ slightly)
-        t0 = time.perf_counter()
-        K.conv_meta_bf16(sub, wb, 1, 1, 1, nt)
-        tn = time.perf_counter() - t0
         sub_flops = 2.0 * 1 * 256 * 14 * 56 * 256 * 9
-        out["cpu_baseline"] = {"value": round(sub_flops / tn / 1e12, 5), "unit": "TFLOP/s", "cores": nt, "kind": "port",
-                               "sample": "x[:1,:,:14,:] (1 image, 14 rows), all cores, one run"}
+        tn = cpu_time(lambda: K.conv_meta_bf16(sub, wb, 1, 1, 1, nt), repeat=3)
+        one = xb[:1, :, :4, :]                       # 4 rows for the single-thread figure (the reference's default): 1/896 of the MACs
+        one_flops = 2.0 * 1 * 256 * 4 * 56 * 256 * 9
+        t1 = cpu_time(lambda: K.conv_meta_bf16(one, wb, 1, 1, 1, 1), repeat=3)
+        out["cpu_baseline"] = {"value": round(one_flops / t1 / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                               "sample": "x[:1,:,:4,:] (1 image, 4 of 56 rows: 1/896 of the work), one thread, median of 3",
+                               "all_cores": {"value": round(sub_flops / tn / 1e12, 5), "cores": nt,
+                                             "sample": "x[:1,:,:14,:] (1/256 of the work), median of 3"}}
     return out
 
 
@@ -294,7 +322,7 @@ def wl_c5_wgrad(L, lib, steps, warmup, with_cpu):
     ms, wall = time_calls(L, calls, steps, warmup)
     out = {"workload": "C5 weight gradient, x bf16 [64,256,56,56], dy bf16 [64,256,56,56] -> dw fp32 [256,256,3,3]",
            "kernel": L.last_kernel(), "dtype": "bf16", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
-           "roofline": roofline("mfma", flops, ms), "note": "a step = MFMA kernel over slices of images + reduce over the slices"}
+           "roofline": roofline("mfma", flops, ms), **LAST_SPREAD, "note": "a step = MFMA kernel over slices of images + reduce over the slices"}
     dev.release()
     return out
 
@@ -310,22 +338,52 @@ def wl_copy(L, lib, steps, warmup, with_cpu):
     dev.release()
     return {"workload": "COPY device copy of 268435456 bytes (reads 268435456 B, writes 268435456 B)",
             "kernel": L.last_kernel(), "dtype": "u8", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
-            "roofline": roofline("hbm", 2 * n, ms)}
+            "roofline": roofline("hbm", 2 * n, ms), **LAST_SPREAD}
 
 
-# HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# HBM bytes per launch of the workload's kernels, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # runs of this file (KiB per dispatch), each scaled by what the same counter reads for the COPY workload
 # (FETCH_SIZE reads 131082 KiB for 262144 KiB fetched: factor 2.0; WRITE_SIZE reads 262144 KiB: factor 1.0).
-# Summaries: profiles/hbm_traffic_all_workloads.txt
+# Each entry names the kernel it was measured on: when the kernel that ran is another one (a new tiling, another
+# code path) the figure is not reported rather than passed on stale.
+TRAFFIC_SOURCE = "profiles/hbm_traffic_all_workloads.txt"
 MEASURED_TRAFFIC = {
-    "C1": 2.0 * 65557.8 * 1024 + 64.0 * 1024,
-    "C2": 2.0 * 15636.1 * 1024 + 225806.5 * 1024,
-    "C3add": 2.0 * 65692.9 * 1024 + 41115.1 * 1024,
-    "C3max": 2.0 * 65695.3 * 1024 + 41680.2 * 1024,
-    "C4": 2.0 * 65582.8 * 1024 + 131072.0 * 1024,
-    "C5": 2.0 * 113405.4 * 1024 + 211332.1 * 1024,
-    "C5bf16out": 2.0 * 112114.2 * 1024 + 112616.1 * 1024,
+    "C1": ("mjt_reduce_row_add_float32_float32_k1r1v4g64", 2.0 * 65557.8 * 1024 + 64.0 * 1024),
+    "C2": ("mjt_window_gather_b4_56x56_k3x3_s1x1_d1x1_o56x56_t8", 2.0 * 15636.1 * 1024 + 225806.5 * 1024),
+    "C3add": ("mjt_scatter1d_add_float32_int32_w16384_b64_e8_s1920_final", 2.0 * 65692.9 * 1024 + 41115.1 * 1024),
+    "C3max": ("mjt_scatter1d_maximum_float32_int32_w16384_b64_e8_s4096_final", 2.0 * 65695.3 * 1024 + 41680.2 * 1024),
+    "C4": ("mjt_fused_11ops_524174662d216c32", 2.0 * 65582.8 * 1024 + 131072.0 * 1024),
+    "C5": ("mjt_conv_mfma_bf16_c256_k256_56x56_r3x3_s1x1_p1x1_d1x1_rows14_of32", 2.0 * 113405.4 * 1024 + 211332.1 * 1024),
+    "C5bf16out": ("mjt_conv_mfma_bf16_c256_k256_56x56_r3x3_s1x1_p1x1_d1x1_rows14_obf16", 2.0 * 112114.2 * 1024 + 112616.1 * 1024),
 }
+
+
+def measured_traffic(name, kernel):
+    entry = MEASURED_TRAFFIC.get(name)
+    return int(entry[1]) if entry and entry[0] == kernel else None
+
+
+def wl_gemm(L, lib, steps, warmup, with_cpu, trans_b=1):
+    """The matrix product the matmul pattern runs on (kernels/gemm_mfma.h): 4096^3 in bfloat16, a @ b^T (the layout
+    of nn.linear) or a @ b.  Not one of the five configurations: run with --only GEMM or GEMMnn."""
+    n = 4096
+    flops = 2.0 * n * n * n
+    dev = Dev(L)
+    from jittor_amd.dtypes import f32_to_bf16_bits
+    rng = np.random.default_rng(0)
+    calls = []
+    for s in range(3):
+        a = f32_to_bf16_bits(rng.standard_normal((n, n)).astype(np.float32))
+        ta, tb = L.tensor(dev.put(a), "bfloat16", (n, n)), L.tensor(dev.put(a.T.copy()), "bfloat16", (n, n))
+        tc = L.tensor(dev.empty(n * n * 2), "bfloat16", (n, n))
+        calls.append(lambda ta=ta, tb=tb, tc=tc: L.check(lib.mjt_matmul(ctypes.byref(ta), ctypes.byref(tb), ctypes.byref(tc), 0, trans_b)))
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out = {"workload": "GEMM bf16 4096 x 4096 x 4096, a @ b%s, fp32 accumulate, bf16 result" % ("^T" if trans_b else ""),
+           "kernel": L.last_kernel(), "dtype": "bf16", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+           "roofline": roofline("mfma", flops, ms), **LAST_SPREAD}
+    dev.release()
+    return out
+
 
 WORKLOADS = {
     "C1": wl_c1,
@@ -336,6 +394,8 @@ WORKLOADS = {
     "C5": wl_c5,
     "C5bf16out": lambda L, lib, steps, warmup, with_cpu: wl_c5(L, lib, steps, warmup, False, out_dtype="bfloat16"),
     "C5wgrad": wl_c5_wgrad,
+    "GEMM": wl_gemm,
+    "GEMMnn": lambda *a: wl_gemm(*a, trans_b=0),
     "COPY": wl_copy,
 }
 DEFAULT = ["C1", "C2", "C3add", "C3max", "C4", "C5", "C5bf16out"]
@@ -361,12 +421,22 @@ def main():
     for name in only:
         try:
             results[name] = WORKLOADS[name](L, lib, args.steps, args.warmup, not args.no_cpu)
-            if name in MEASURED_TRAFFIC and "roofline" in results[name]:
-                results[name]["roofline"]["traffic"] = int(MEASURED_TRAFFIC[name])
+            if "roofline" in results[name]:
+                results[name]["roofline"]["traffic"] = measured_traffic(name, results[name].get("kernel", ""))
+                if results[name]["roofline"]["traffic"] is not None:
+                    results[name]["roofline"]["traffic_source"] = TRAFFIC_SOURCE
         except L.MjtError as err:
             results[name] = {"error": str(err)}
         print("[bench] %s: %s" % (name, json.dumps(results[name])), file=sys.stderr, flush=True)
     head = results.get("C2") or next(iter(results.values()))
+    # every configuration's fraction of its roofline beside the headline, against north_star's targets
+    # (0.70 of peak HBM bandwidth for C1-C4, 0.50 of peak MFMA throughput for C5)
+    targets = {"C1": 0.70, "C2": 0.70, "C3add": 0.70, "C3max": 0.70, "C4": 0.70, "C5": 0.50}
+    fractions = {k: results[k]["roofline"]["frac"] for k in targets if k in results and "roofline" in results[k]}
+    by_config = {}
+    for k, f in fractions.items():
+        by_config.setdefault(k[:2], []).append(f >= targets[k])
+    met = sum(1 for v in by_config.values() if all(v))
     line = {
         "metric": "achieved HBM GB/s (% peak) for reduce/reindex/fused ops; conv TFLOP/s",
         "value": head.get("roofline", {}).get("achieved"),
@@ -375,9 +445,13 @@ def main():
         "ms_per_step": head.get("ms_per_step"),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": head.get("dtype", "f32"), "data": "synthetic",
-        "config": {"workload": head.get("workload"), "buffer_sets": "rotating, > 256 MB in total"},
+        "config": {"workload": head.get("workload"), "buffer_sets": "rotating; the inputs alone exceed the 256 MB memory-side cache"},
         "roofline": head.get("roofline"),
         "cpu_baseline": head.get("cpu_baseline"),
+        "fractions": fractions,
+        "targets": targets,
+        "targets_met": "%d/%d" % (met, len(by_config)),
+        "timing": "median over blocks of `steps` launches, repeated until %.1f s of device time per workload" % MIN_DEVICE_SECONDS,
         "device": {"arch": di.arch.decode(), "compute_units": di.compute_units, "clock_khz": di.clock_khz,
                    "mem_clock_khz": di.mem_clock_khz, "mem_bus_bits": di.mem_bus_bits},
         "workloads": results,

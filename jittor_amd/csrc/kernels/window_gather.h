@@ -8,56 +8,132 @@
 // DW, CH, CW, TH (output rows per workgroup), LH x LW (LDS tile), ESZ-byte
 // elements moved as raw bits (TB), VEC elements per store.
 //
-// One workgroup owns TH output rows of one plane.  It stages the input rows
-// they touch in LDS once (out-of-range cells hold the overflow value, so no
-// bounds test is left in the inner loop), then writes its part of y, which is
-// one contiguous run of TH*OW*KH*KW elements, as 16-byte vectors: lane l owns
-// vectors l, l+256, ... of that run and finds (row, ow, kh, kw) of each
-// element by constant division.
+// A workgroup owns TPW consecutive tiles of one plane, a tile being TH output rows.  Per tile it stages the
+// input rows they touch in LDS (out-of-range cells hold the overflow value, so no bounds test is left in the
+// inner loop), then writes its part of y, which is one contiguous run of TH*OW*KH*KW elements, as 16-byte
+// vectors: lane l owns vectors l, l+WTHREADS, ... of that run and finds (row, ow, kh, kw) of each element by
+// constant division.  The input of the next tile is loaded into registers before the current tile is stored and
+// written to the other LDS buffer after: the read latency hides behind the stores.  Loads and stores are
+// unconditional instructions with clamped addresses or masked lanes, and the store loop has a constant trip
+// count: memory operations of a wave complete in order, and the wait for the prefetched input may leave exactly
+// the stores issued after it outstanding only if their number is known.
 
 struct Params { void* a[4]; };   // 8-byte words; typed as pointers so loads/stores use the global address space   // x, y, overflow bits, number of planes
+
+// Element and vector moves through buffer descriptors: an offset past the end of the descriptor's range reads
+// zeros and drops a store, which is how lanes without work stay out of the way without a branch.
+typedef unsigned mjt_wu32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned mjt_wu32x4 __attribute__((ext_vector_type(4)));
+template <int BYTES> struct mjt_win_io;
+template <> struct mjt_win_io<2> {
+    typedef unsigned short raw;
+    static __device__ __forceinline__ raw load(__amdgpu_buffer_rsrc_t r, unsigned off) { return __builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, 0); }
+    static __device__ __forceinline__ void store(raw v, __amdgpu_buffer_rsrc_t r, unsigned off) { __builtin_amdgcn_raw_buffer_store_b16(v, r, (int)off, 0, 2); }
+};
+template <> struct mjt_win_io<4> {
+    typedef unsigned raw;
+    static __device__ __forceinline__ raw load(__amdgpu_buffer_rsrc_t r, unsigned off) { return __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0); }
+    static __device__ __forceinline__ void store(raw v, __amdgpu_buffer_rsrc_t r, unsigned off) { __builtin_amdgcn_raw_buffer_store_b32(v, r, (int)off, 0, 2); }
+};
+template <> struct mjt_win_io<8> {
+    typedef mjt_wu32x2 raw;
+    static __device__ __forceinline__ raw load(__amdgpu_buffer_rsrc_t r, unsigned off) { return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0); }
+    static __device__ __forceinline__ void store(raw v, __amdgpu_buffer_rsrc_t r, unsigned off) { __builtin_amdgcn_raw_buffer_store_b64(v, r, (int)off, 0, 2); }
+};
+template <> struct mjt_win_io<16> {
+    typedef mjt_wu32x4 raw;
+    static __device__ __forceinline__ void store(raw v, __amdgpu_buffer_rsrc_t r, unsigned off) { __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)off, 0, 2); }
+};
+__device__ __forceinline__ TB mjt_win_load(__amdgpu_buffer_rsrc_t r, unsigned off) {
+    return __builtin_bit_cast(TB, mjt_win_io<sizeof(TB)>::load(r, off));
+}
+__device__ __forceinline__ void mjt_win_store(__amdgpu_buffer_rsrc_t r, unsigned off, const mjt_pack<TB, VEC>& v) {
+    typedef mjt_win_io<sizeof(TB) * VEC> io;
+    io::store(__builtin_bit_cast(typename io::raw, v), r, off);
+}
 
 extern "C" __global__ __launch_bounds__(WTHREADS) void ENTRY(Params p) {
     const TB* __restrict__ xp = (const TB*)p.a[0];
     TB* __restrict__ yp = (TB*)p.a[1];
     const TB ov = (TB)(unsigned long long)p.a[2];
-    __shared__ TB tile[LH * LW];
+    __shared__ TB tile[2][LH * LW];
     constexpr int TILES = (OH + TH - 1) / TH;
-    const unsigned plane = blockIdx.x / TILES;
-    const int oh0 = (int)(blockIdx.x % TILES) * TH;
-    const int rows = (OH - oh0) < TH ? (OH - oh0) : TH;
-    const int ih0 = oh0 * SH + CH;          // input row of LDS row 0
-    const TB* __restrict__ xplane = xp + (size_t)plane * (H * W);
-    for (int t = threadIdx.x; t < LH * LW; t += WTHREADS) {
-        const int lr = t / LW, lc = t - lr * LW;
-        const int ih = ih0 + lr, iw = CW + lc;
-        TB v = ov;
-        if (ih >= 0 && ih < H && iw >= 0 && iw < W) v = xplane[ih * W + iw];
-        tile[t] = v;
-    }
-    __syncthreads();
+    constexpr int PARTS = (TILES + TPW - 1) / TPW;          // workgroups per plane
+    const unsigned plane = blockIdx.x / PARTS;
+    const int first = (int)(blockIdx.x % PARTS) * TPW;
+    const int last = first + TPW < TILES ? first + TPW : TILES;
     constexpr int KK = KH * KW;
     constexpr int ROWLEN = OW * KK;
-    const int nvec = rows * ROWLEN / VEC;
-    TB* __restrict__ yrun = yp + ((size_t)plane * OH + oh0) * ROWLEN;
-    for (int q = threadIdx.x; q < nvec; q += WTHREADS) {
-        const int t0 = q * VEC;
-        int r = t0 / ROWLEN;
-        int rem = t0 - r * ROWLEN;
-        int ow = rem / KK;
-        int kk = rem - ow * KK;
-        int kh = kk / KW;
-        int kw = kk - kh * KW;
-        mjt_pack<TB, VEC> out;
+    constexpr unsigned OUTSIDE = 0x80000000u;               // beyond every plane (the host keeps planes below 2 GB)
+    const __amdgpu_buffer_rsrc_t xr =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(xp + (size_t)plane * (H * W)), 0, (int)(H * W * sizeof(TB)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t yr =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(yp + (size_t)plane * OH * ROWLEN), 0, (int)(OH * ROWLEN * sizeof(TB)), 0x00020000);
+    constexpr int NLOAD = (LH * LW + WTHREADS - 1) / WTHREADS;
+    TB pre[NLOAD];
+    // whether element i of this lane's share of tile t lies inside the input, and its byte offset there
+    auto cell = [&](int t, int i, unsigned& off) -> bool {
+        const int e = threadIdx.x + i * WTHREADS;
+        const int lr = e / LW, lc = e - lr * LW;
+        const int ih = t * TH * SH + CH + lr, iw = CW + lc;
+        off = (unsigned)((ih * W + iw) * sizeof(TB));
+        return e < LH * LW && ih >= 0 && ih < H && iw >= 0 && iw < W;
+    };
+    auto fetch = [&](int t) {                               // issues the loads; nothing here looks at a loaded value
 #pragma unroll
-        for (int k = 0; k < VEC; k++) {
-            out.v[k] = tile[(r * SH + kh * DH) * LW + ow * SW + kw * DW];
-            // advance to the next element of the run
-            kw++;
-            if (kw == KW) { kw = 0; kh++; }
-            if (kh == KH) { kh = 0; ow++; }
-            if (ow == OW) { ow = 0; r++; }
+        for (int i = 0; i < NLOAD; i++) {
+            unsigned off;
+            const bool inside = cell(t, i, off);
+            pre[i] = mjt_win_load(xr, inside ? off : OUTSIDE);
         }
-        mjt_store_nt(yrun + t0, out);
+    };
+    auto commit = [&](int t, int buf) {
+#pragma unroll
+        for (int i = 0; i < NLOAD; i++) {
+            unsigned off;
+            const bool inside = cell(t, i, off);
+            if (threadIdx.x + i * WTHREADS < LH * LW) tile[buf][threadIdx.x + i * WTHREADS] = inside ? pre[i] : ov;
+        }
+    };
+    constexpr int NV = (TH * ROWLEN / VEC + WTHREADS - 1) / WTHREADS;    // vectors per lane of a full tile
+    fetch(first);
+    commit(first, first & 1);
+    __syncthreads();
+#pragma unroll 1
+    for (int t = first; t < last; t++) {
+        if (t + 1 < last) fetch(t + 1);                     // (uniform)
+        const int oh0 = t * TH;
+        const int rows = (OH - oh0) < TH ? (OH - oh0) : TH;
+        const int nvec = rows * ROWLEN / VEC;
+        const unsigned run0 = (unsigned)(oh0 * ROWLEN * sizeof(TB));
+        const TB* __restrict__ cur = tile[t & 1];
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int q = threadIdx.x + j * WTHREADS;
+            const int qc = q < nvec ? q : 0;                // lanes past the end recompute vector 0 and store nowhere
+            const int t0 = qc * VEC;
+            int r = t0 / ROWLEN;
+            int rem = t0 - r * ROWLEN;
+            int ow = rem / KK;
+            int kk = rem - ow * KK;
+            int kh = kk / KW;
+            int kw = kk - kh * KW;
+            mjt_pack<TB, VEC> out;
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                out.v[k] = cur[(r * SH + kh * DH) * LW + ow * SW + kw * DW];
+                // advance to the next element of the run
+                kw++;
+                if (kw == KW) { kw = 0; kh++; }
+                if (kh == KH) { kh = 0; ow++; }
+                if (ow == OW) { ow = 0; r++; }
+            }
+            mjt_win_store(yr, q < nvec ? run0 + (unsigned)(t0 * sizeof(TB)) : OUTSIDE, out);
+        }
+        if (t + 1 < last) {
+            commit(t + 1, (t + 1) & 1);
+            // LDS traffic only: a full fence would also wait for the stores of this tile to be acknowledged
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+        }
     }
 }

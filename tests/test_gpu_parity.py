@@ -280,6 +280,22 @@ def test_scatter_1d_index_distributions(gpu):
     assert not L.last_kernel().startswith("mjt_scatter1d_") and abs(got.sum() - v[:4096].astype(np.float64).sum()) < 1e-2
 
 
+def test_window_gather_several_tiles_per_workgroup(gpu, monkeypatch):
+    """MJT_WINDOW_TPW > 1: a workgroup walks several tiles of a plane and loads the next tile's input while it
+    stores the current one; same bits as the oracle, also when the last workgroup of a plane has fewer tiles."""
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((3, 5, 41, 23)).astype(np.float32)
+    idx = ["i0", "i1", "i2*2+i4-1", "i3+i5-2"]
+    shape = [3, 5, 21, 24, 3, 4]
+    want = O.reindex(x, shape, idx, -7.0)
+    for tpw, th in ((3, 4), (2, 8), (50, 1)):
+        monkeypatch.setenv("MJT_WINDOW_TPW", str(tpw))
+        monkeypatch.setenv("MJT_WINDOW_TH", str(th))
+        got = jt.array(x).reindex(shape, idx, -7.0).data
+        assert L.last_kernel().startswith("mjt_window_gather") and L.last_kernel().endswith("x%d" % min(tpw, -(-21 // th))), L.last_kernel()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (tpw, th)
+
+
 def _zipf_indices(n, bins):
     w = np.arange(1, bins + 1, dtype=np.float64) ** -1.1
     cdf = np.cumsum(w) / w.sum()

@@ -371,3 +371,73 @@ def test_conv_meta_one_hot_kernel_is_a_shift():
     ref0 = np.zeros((6, 6), np.float32)
     ref0[1:, :5] = xf[0, 0, :5, 1:]
     assert np.array_equal(y[0, 0], ref0) and np.array_equal(y[0, 1], xf[0, 1])
+
+
+# ---- the index-expression evaluator: every operator of python/jittor/src/opt/expr.cc:16-52 ---------------------
+_EXPR_VARS = {"a": 7, "b": -3, "i0": 5, "i1": 12}
+# literal known answers (C semantics: division truncates towards zero, the remainder takes the dividend's sign,
+# comparisons and logical operators give 0 / 1, << binds tighter than <, ?: is right-associative)
+_EXPR_KNOWN = [
+    ("10+2*6", 22), ("100 * 2 + 12", 212), ("100 * ( 2 + 12 )", 1400), ("100*(2+12)/14", 100), ("-1", -1), ("- 1", -1),
+    ("a", 7), ("a+b", 4), ("-1 +a *b", -22),                          # python/jittor/test/test_op_compiler.py:33-46
+    ("a/b", -2), ("a%b", 1), ("b/2", -1), ("b%2", -1), ("(-a)%4", -3), ("-a/2", -3),
+    ("1+2*3<<1", 14), ("1<<2+1", 8), ("a<b", 0), ("a>b", 1), ("a<=7", 1), ("a>=8", 0), ("a==7", 1), ("a!=b", 1),
+    ("a<b?a:b", -3), ("a>b?(b<0?1:2):3", 1), ("0?1:0?2:3", 3), ("1?1:0?2:3", 1),
+    ("a>=7&&b<0", 1), ("a==8||b", 1), ("0||0", 0), ("!a", 0), ("!0", 1), ("~a", -8), ("a&b", 5), ("a|b", -1), ("a^b", -6),
+    ("a<<2", 28), ("a>>1", 3), ("b>>1", -2), ("a&3|8", 11), ("a|2&1", 7), ("a^1&3", 6), ("1|2^3&4", 3),
+    ("i0*3+i1%5-2", 15), ("i1/i0*i0+i1%i0", 12), ("0x1f+0b101", 36), ("2-3-4", -5), ("100/10/5", 2), ("1<2==1", 1),
+    ("int(2.7)", 2), ("int(-2.7)", -2), ("int(float(a)/2)", 3), ("int(float(a)/2*2)", 7), ("bool(a)+bool(0)", 1),
+]
+
+
+def test_expression_evaluator_known_answers():
+    env = {k: np.int64(v) for k, v in _EXPR_VARS.items()}
+    for text, want in _EXPR_KNOWN:
+        got = O.eval_expr(O.parse_expr(text), env, [])
+        assert int(np.asarray(got)) == want, (text, got, want)
+    assert float(np.asarray(O.eval_expr(O.parse_expr("float(a)/2"), env, []))) == 3.5
+    for bad in ("*****", "a//b", "a+", "(a", "a b"):                  # test_op_compiler.py:47; loop_var_analyze_pass.cc:298-309
+        with pytest.raises(ValueError):
+            O.eval_expr(O.parse_expr(bad), env, [])
+
+
+def test_expression_evaluator_against_the_c_compiler(tmp_path):
+    """The expressions are C: compiled as C (gcc, 64-bit integers) they must give what the oracle's evaluator
+    gives.  An independent evaluator for precedence, associativity, truncating division and the 0 / 1 results."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    rng = np.random.default_rng(12)
+    ops2 = ["+", "-", "*", "/", "%", "<<", ">>", "<", "<=", ">", ">=", "==", "!=", "&", "|", "^", "&&", "||"]
+    texts = [t for t, _ in _EXPR_KNOWN if "int(" not in t and "float(" not in t and "bool(" not in t]
+    names = list(_EXPR_VARS)
+    for _ in range(200):                                              # random three-operator expressions without parentheses
+        t = names[rng.integers(4)]
+        for _k in range(3):
+            op = ops2[rng.integers(len(ops2))]
+            rhs = names[rng.integers(4)] if rng.random() < 0.6 else str(int(rng.integers(1, 6)))
+            if op in ("<<", ">>"):
+                rhs = str(int(rng.integers(0, 4)))
+            if op in ("/", "%"):
+                rhs = str(int(rng.integers(1, 6)))                    # no division by zero or by a negative shift count
+            t = "%s%s%s" % (t, op, rhs)
+        if "<<" in t and "b<<" in t:
+            continue                                                  # shifting a negative value left is undefined in C
+        texts.append(t)
+    for _ in range(40):
+        texts.append("%s%s%s?%s:%s" % (names[rng.integers(4)], ops2[rng.integers(7, 13)], names[rng.integers(4)],
+                                       texts[rng.integers(len(texts))], texts[rng.integers(len(texts))]))
+    src = ["#include <stdio.h>", "int main(void) {"]
+    src += ["  long long %s = %d;" % kv for kv in _EXPR_VARS.items()]
+    src += ['  printf("%%lld\\n", (long long)(%s));' % t for t in texts]
+    src += ["  return 0;", "}"]
+    c = tmp_path / "e.c"
+    c.write_text("\n".join(src))
+    subprocess.check_call(["gcc", "-O0", "-w", "-o", str(tmp_path / "e"), str(c)])
+    want = [int(v) for v in subprocess.check_output([str(tmp_path / "e")]).split()]
+    env = {k: np.int64(v) for k, v in _EXPR_VARS.items()}
+    assert len(want) == len(texts)
+    for t, w in zip(texts, want):
+        got = int(np.asarray(O.eval_expr(O.parse_expr(t), env, [])))
+        assert got == w, (t, got, w)
