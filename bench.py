@@ -278,7 +278,7 @@ def wl_c5(L, lib, steps, warmup, with_cpu, out_dtype="float32"):
     p = L.ConvParams(1, 1, 1, 1, 1, 1)
     calls = []
     tw = L.tensor(dev.put(wb), "bfloat16", ws)
-    for s in range(2):
+    for s in range(3):                               # 3 x 103 MB of input: more than the memory-side cache holds
         tx = L.tensor(dev.put(xb), "bfloat16", xs)
         ty = L.tensor(dev.empty(int(np.prod(ys)) * 4), out_dtype, ys)
         calls.append(lambda tx=tx, ty=ty: L.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p))))

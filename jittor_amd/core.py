@@ -110,6 +110,10 @@ class Op:
 
     def __init__(self, inputs):
         self.inputs = list(inputs)
+        for v in self.inputs:              # who reads a Var: Var.assign moves them to the old value
+            if v._consumers is None:
+                v._consumers = weakref.WeakSet()
+            v._consumers.add(self)
         self.id = _new_id()
         self._out_ref = None
         self.amp = dt.amp_reg & 63          # the register at creation; its gradient is built under it (op.cc:38, grad.cc:48-55)
@@ -228,6 +232,7 @@ class Var:
         self.is_scalar = False   # NodeFlags::_is_scalar
         self.id = _new_id()
         self._name = None
+        self._consumers = None   # ops that take this Var as an input (weakly)
 
     # ---- properties ----
     @property
@@ -374,6 +379,45 @@ class Var:
 
     def ternary(self, x, y):
         return ternary(self, x, y)
+
+    def _split_off_value(self):
+        """Moves this Var's present value to a new Var and hands every op that reads this Var over to it: the
+        object is then free to be rebound without changing what was built from its old value (in the reference
+        the Python object is a holder and ops refer to the node behind it, python/jittor/src/var_holder.h:37-60)."""
+        old = Var.__new__(Var)
+        old.__dict__.update(self.__dict__)           # the old value keeps its id: ids grow along the data flow (grad() orders by them)
+        self.id = _new_id()
+        old._consumers = self._consumers
+        self._consumers = None
+        self._op = self._history = self._buf = self._host = None     # nothing left here until assign() fills it
+        if old._op is not None:
+            old._op.out = old
+        for op in list(old._consumers or ()):
+            op.inputs = [old if v is self else v for v in op.inputs]
+            out = op.out
+            if out is not None and out._history is not None:
+                out._history = (out._history[0], tuple(old if v is self else v for v in out._history[1]))
+        return old
+
+    def assign(self, other):
+        """This Var becomes `other` (shape, dtype and value), as VarHolder::assign rebinds a holder
+        (python/jittor/src/var_holder.cc).  Ops built from the old value keep reading the old value."""
+        other = _as_var(other)
+        if other is self:
+            return self
+        if self._op is not None or self._buf is not None or self._host is not None:
+            self._split_off_value()
+        name = self._name
+        src = other._split_off_value()                 # `other` stays valid: it now reads this Var (and has a new id)
+        self.__dict__.update(src.__dict__)             # with the id of the value taken over
+        self._name = name
+        if self._op is not None:
+            self._op.out = self
+        alias = ReindexOp(self, ["i%d" % i for i in range(len(self.shape))], 0, [], [])
+        other._op, other._buf, other._host = alias, None, None
+        alias.out = other
+        other._history = (alias, (self,)) if _grad_enabled[0] else None
+        return self
 
     def stop_grad(self):
         """The var becomes a leaf for grad() (var_holder.h stop_grad)."""

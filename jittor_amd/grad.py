@@ -139,8 +139,8 @@ def _op_grad(op, inputs, out, dout, index):
         if index:
             return None
         back = lambda v: reindex(v, x.shape, op.indexes, 0, op.overflow_conditions, inputs[1:])
-        if op.op == "add":
-            return back(dout)
+        if op.op in ("add", "void"):                    # void (plain assignment, setitem_op.cc: the gradient of the value is the
+            return back(dout)                           # gradient read back where it was written)
         if op.op == "multiply":
             return binary(back(binary(dout, out, "multiply")), x, "divide")
         if op.op in ("maximum", "minimum"):

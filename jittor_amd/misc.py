@@ -158,9 +158,11 @@ def reshape(x, *shape):
     return reindex(x, shape, idx[::-1])
 
 
-def getitem(x, key):
-    """Basic indexing with integers, slices (positive or negative step), None and Ellipsis, and one
-    integer Var per axis (gather along that axis); one reindex."""
+def _parse_key(x, key):
+    """Splits an index into, per axis of x, what selects it: returns (out_shape, exprs, extras) where exprs[d] is
+    the index expression of axis d of x in terms of the coordinates of the selection."""
+    if isinstance(key, Var) and key.dtype == "bool":
+        raise IndexError("a boolean mask selects a data-dependent number of elements: use ternary(mask, a, b)")
     if not isinstance(key, tuple):
         key = (key,)
     if sum(1 for k in key if k is Ellipsis) > 1:
@@ -203,9 +205,40 @@ def getitem(x, key):
         else:
             raise IndexError("unsupported index %r" % (k,))
         axis += 1
+    return out_shape, exprs, extras
+
+
+def getitem(x, key):
+    """Basic indexing with integers, slices (positive or negative step), None and Ellipsis, and one
+    integer Var per axis (gather along that axis); one reindex (python/jittor/src/ops/getitem_op.cc)."""
+    out_shape, exprs, extras = _parse_key(x, key)
     if not out_shape:
         out_shape = [1]
     return reindex(x, out_shape, exprs, extras=extras)
+
+
+def setitem(x, key, value):
+    """x[key] = value (python/jittor/src/ops/setitem_op.cc): the same keys as getitem.  The value, broadcast to
+    the selection, is scattered into a tensor of x's shape (reindex_reduce 'void' with the selection's index
+    expressions), a scatter of ones marks the cells that were written, and a ternary takes the new value there
+    and x elsewhere (the construction of misc.scatter); x is rebound to the result.  With an index Var that holds
+    duplicates, which of the values lands is undefined, as in the reference."""
+    out_shape, exprs, extras = _parse_key(x, key)
+    if not out_shape:
+        out_shape = [1]
+    value = core._as_var(value)
+    if value.dtype != x.dtype:
+        value = value.cast(x.dtype)
+    vs = list(value.shape)
+    if len(vs) > len(out_shape) and all(s == 1 for s in vs[:len(vs) - len(out_shape)]):
+        value = reshape(value, vs[len(vs) - len(out_shape):])
+    if list(value.shape) != out_shape:
+        value = broadcast(value, out_shape)
+    upd = reindex_reduce(value, "void", x.shape, exprs, extras=extras)
+    one = broadcast(array(1, "int32"), out_shape)
+    hit = reindex_reduce(one, "add", x.shape, exprs, extras=extras)
+    old = x._split_off_value()                          # the ternary reads the old value, x is rebound to its result
+    return x.assign(ternary(hit > 0, upd, old))
 
 
 Var.gather = gather
@@ -216,3 +249,5 @@ Var.reshape = reshape
 Var.view = reshape
 Var.flip = flip
 Var.__getitem__ = getitem
+Var.__setitem__ = lambda self, key, value: (setitem(self, key, value), None)[1]
+Var.setitem = setitem

@@ -1,6 +1,8 @@
 """Callers that define the patterns of the path: relu and conv2d expressed
 with meta-operators exactly as the reference writes them
 (python/jittor/nn.py:166-183 and :1245-1269)."""
+import numpy as np
+
 from . import core
 from .flags import flags, flag_scope
 
@@ -117,15 +119,11 @@ def matmul(a, b):
     if len_b == 2 and len_a > 2:
         cc = matmul(misc.reshape(a, [-1, m]), b)
         return misc.reshape(cc, list(a.shape[:-1]) + [k])
-    shape = []
-    for i in range(len_c - 2):
-        ai, bi = len_a - (len_c - i), len_b - (len_c - i)
-        an = a.shape[ai] if ai >= 0 else 1
-        bn = b.shape[bi] if bi >= 0 else 1
-        if an != 1 and bn != 1:
-            assert an == bn, "dimension not match, a.shape:%s, b.shape:%s" % (a.shape, b.shape)
-        shape.append(max(an, bn))
-    shape.extend([n, m, k])
+    # the leading axes broadcast against each other like any element-wise pair
+    try:
+        shape = list(np.broadcast_shapes(tuple(a.shape[:-2]), tuple(b.shape[:-2]))) + [n, m, k]
+    except ValueError:
+        raise AssertionError("dimension not match, a.shape:%s, b.shape:%s" % (a.shape, b.shape))
     a = core.broadcast(a, shape, [-1])
     b = core.broadcast(b, shape, [-3])
     return core.reduce(core.binary(a, b, "multiply"), "add", [-2])

@@ -204,3 +204,58 @@ def test_histc_ranges(gpu):
     assert np.array_equal(h, want)
     with pytest.raises(RuntimeError):
         jt.histc(jt.array(y), 0)
+
+
+def test_setitem_and_assign(gpu):
+    """x[key] = value (python/jittor/src/ops/setitem_op.cc) for the keys getitem takes, against numpy; ops built
+    from the old value keep the old value (lazy graph), gradients flow through the written and the kept part."""
+    rng = np.random.default_rng(61)
+    a = rng.standard_normal((6, 7, 5)).astype(np.float32)
+    cases = [
+        (np.s_[2], 1.5), (np.s_[1:4], rng.standard_normal((3, 7, 5)).astype(np.float32)),
+        (np.s_[:, ::2, 1], rng.standard_normal((6, 4)).astype(np.float32)), (np.s_[..., -1], 0.0),
+        (np.s_[::-2, 3:, :], rng.standard_normal((7 - 3, 5)).astype(np.float32)),          # broadcast along the first axis
+        (np.s_[5, 6, 4], 9.0), (np.s_[:, None, 2, :], rng.standard_normal((6, 1, 5)).astype(np.float32)),
+    ]
+    for key, val in cases:
+        want = a.copy()
+        want[key] = val
+        x = jt.array(a)
+        y_before = x * 2                                         # built before the write, evaluated after it
+        x[key] = jt.array(val) if isinstance(val, np.ndarray) else val
+        assert np.array_equal(x.data, want), key
+        assert np.array_equal(y_before.data, a * 2), key
+    # one integer Var per axis (distinct positions)
+    idx = np.array([4, 0, 2], np.int32)
+    v = rng.standard_normal((3, 7, 5)).astype(np.float32)
+    x = jt.array(a)
+    x[jt.array(idx)] = jt.array(v)
+    want = a.copy()
+    want[idx] = v
+    assert np.array_equal(x.data, want)
+    # integer data, and a chain of writes
+    b = np.arange(24, dtype=np.int32).reshape(4, 6)
+    x = jt.array(b)
+    x[1:3, ::3] = -1
+    x[0] = x[3] + 100
+    want = b.copy()
+    want[1:3, ::3] = -1
+    want[0] = want[3] + 100
+    assert np.array_equal(x.data, want)
+    # gradients: d/dx of sum(w * x') where x' = x with a slice replaced by 3 * v
+    xv, vv = jt.array(a), jt.array(v[0, :3])
+    w = rng.standard_normal(a.shape).astype(np.float32)
+    x2 = xv * 1.0
+    x2[2, 1:4] = vv * 3
+    loss = (x2 * jt.array(w)).sum()
+    gx, gv = jt.grad(loss, [xv, vv])
+    wx = w.copy()
+    wx[2, 1:4] = 0
+    assert np.allclose(gx.data, wx) and np.allclose(gv.data, 3 * w[2, 1:4])
+    # assign: the object takes another Var's value; what was built from the old value keeps it
+    p, q = jt.array(a), jt.array(a[::-1].copy())
+    s_old = p + 1
+    p.assign(q * 2)
+    assert np.array_equal(p.data, a[::-1] * 2) and np.array_equal(s_old.data, a + 1)
+    with pytest.raises(IndexError):
+        jt.array(a)[jt.array(a > 0)]

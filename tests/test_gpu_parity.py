@@ -520,21 +520,24 @@ def test_conv_mfma_matches_oracle(gpu, case):
         ref = K.conv_meta_bf16(xb, wb, sh, ph, dh, 8)
     else:
         ref = None
+    xf, wf = O.BF16(xb).to_f32().astype(np.float64), O.BF16(wb).to_f32().astype(np.float64)
+    R, S = wf.shape[2], wf.shape[3]
+    oh, ow = got.shape[2], got.shape[3]
+    xp = np.pad(xf, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+    ref64, terms = np.zeros(got.shape), np.zeros(got.shape)      # the float64 result and the sum of |x * w| per output
+    for r in range(R):
+        for s in range(S):
+            patch = xp[:, :, r * dh:r * dh + (oh - 1) * sh + 1:sh, s * dw:s * dw + (ow - 1) * sw + 1:sw]
+            ref64 += np.einsum("nchw,kc->nkhw", patch, wf[:, :, r, s])
+            terms += np.einsum("nchw,kc->nkhw", np.abs(patch), np.abs(wf[:, :, r, s]))
     if ref is None:
-        xf, wf = O.BF16(xb).to_f32().astype(np.float64), O.BF16(wb).to_f32().astype(np.float64)
-        N, C, H, W = xf.shape
-        Kc, _, R, S = wf.shape
-        oh, ow = got.shape[2], got.shape[3]
-        xp = np.pad(xf, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
-        ref = np.zeros(got.shape)
-        for r in range(R):
-            for s in range(S):
-                patch = xp[:, :, r * dh:r * dh + (oh - 1) * sh + 1:sh, s * dw:s * dw + (ow - 1) * sw + 1:sw]
-                ref += np.einsum("nchw,kc->nkhw", patch, wf[:, :, r, s])
-    # fp32 accumulation in a different order than the reference's (c, kh, kw) loop: 1e-4 relative to the
-    # magnitude of the accumulated terms
+        ref = ref64
+    # fp32 accumulation in a different order than the reference's (c, kh, kw) loop: every element within 1e-4 of
+    # the sum of the magnitudes of its terms, against the float64 result and against the oracle's own fp32 loop
+    bound = 1e-4 * terms + 1e-30
+    assert (np.abs(got - ref64) <= bound).all(), float((np.abs(got - ref64) / bound).max())
+    assert (np.abs(got - ref) <= 2 * bound).all(), float((np.abs(got - ref) / bound).max())
     scale = np.abs(ref).max()
-    assert np.abs(got - ref).max() <= 1e-4 * scale, (np.abs(got - ref).max(), scale)
     # the direct kernel follows the reference's loop order exactly
     os.environ["MJT_NO_FASTPATH"] = "1"
     try:
@@ -865,6 +868,15 @@ def test_conv_full_size_c5_properties(gpu):
         err = max(err, abs(ref - got[n, k, h, w_]))
         mag = max(mag, float(np.abs(patch * wf[k]).sum()))
     assert err <= 1e-4 * mag, (err, mag)
+    # two whole images (the first and the last, all 256 output channels) against the float64 product of the
+    # weights with the image's column matrix, every element held to 1e-4 of the sum of its |x * w| terms
+    wm = wf.reshape(256, 256 * 9)
+    for n in (0, 63):
+        win = np.lib.stride_tricks.sliding_window_view(xp[n].astype(np.float64), (3, 3), axis=(1, 2))   # [c, oh, ow, kh, kw]
+        cols = win.transpose(0, 3, 4, 1, 2).reshape(256 * 9, 56 * 56)
+        want = (wm @ cols).reshape(256, 56, 56)
+        bound = 1e-4 * (np.abs(wm) @ np.abs(cols)).reshape(256, 56, 56)
+        assert (np.abs(got[n] - want) <= bound).all(), (n, float(np.abs(got[n] - want).max()))
     # padding taps contribute exactly 0 and a one-hot kernel is a shift (bit-exact)
     w1 = np.zeros(ws, np.float32)
     for k in range(256):
