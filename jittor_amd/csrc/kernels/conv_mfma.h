@@ -41,6 +41,7 @@
 #if IN_F16
 typedef _Float16 mjt_bf16x8 __attribute__((ext_vector_type(8)));
 #define MJT_MFMA __builtin_amdgcn_mfma_f32_16x16x32_f16
+#define MJT_MFMA_ASM "v_mfma_f32_16x16x32_f16"
 // float16 <- float rounds to nearest even (type/fp16_compute.h:147-198)
 __device__ __forceinline__ unsigned mjt_narrow2(float lo, float hi) {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
@@ -52,6 +53,7 @@ __device__ __forceinline__ unsigned mjt_narrow2(float lo, float hi) {
 #else
 typedef __bf16 mjt_bf16x8 __attribute__((ext_vector_type(8)));
 #define MJT_MFMA __builtin_amdgcn_mfma_f32_16x16x32_bf16
+#define MJT_MFMA_ASM "v_mfma_f32_16x16x32_bf16"
 // bfloat16 <- float keeps the upper 16 bits (type/fp16_compute.h:238-241)
 __device__ __forceinline__ unsigned mjt_narrow2(float lo, float hi) {
     return (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
@@ -105,19 +107,32 @@ __device__ __forceinline__ float mjt_xor2f(float v) { return __uint_as_float(mjt
 __device__ __forceinline__ unsigned mjt_xor4(unsigned v) {
     return (unsigned)__builtin_amdgcn_mov_dpp(__builtin_amdgcn_mov_dpp((int)v, 0x141, 0xf, 0xf, true), 0x1B, 0xf, 0xf, true);
 }
+// The MFMAs of the main loop are spelled out like its LDS reads and waits: between those the compiler would
+// otherwise move them freely (it sees no latency in the reads), and the order below is the schedule.  The
+// compiler takes a spelled-out MFMA for finished the moment it is issued and keeps none of the cycles the
+// hardware wants between an MFMA and an instruction that touches its registers.  The accumulators therefore live
+// in the accumulation registers for the whole loop, where nothing but these MFMAs touches them (the loop has no
+// use for them, and no copies are made to feed an MFMA); before and after the loop they are tied to points
+// behind explicit idle cycles.
+__device__ __forceinline__ void mjt_mfma(mjt_f32x4& c, const mjt_u32x4v& a, const mjt_u32x4v& b) {
+    asm volatile(MJT_MFMA_ASM " %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mjt_keep(const mjt_u32x4v& x) { asm volatile("" : : "v"(x)); }     // x is in its registers up to here
+__device__ __forceinline__ void mjt_pin(mjt_f32x4& x) { asm volatile("" : "+a"(x)); }             // what reads x later comes after this point
 template <int OFF> __device__ __forceinline__ void mjt_ds_read(mjt_u32x4v& dst, unsigned addr) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
 }
 // wait until at most N LDS operations issued after the one that fills x are outstanding (LDS returns in order)
 template <int N> __device__ __forceinline__ void mjt_lds_wait(mjt_u32x4v& x) {
-    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N < 15 ? N : 15));   // the counter has four bits
 }
 
-extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
+extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu(WPS, WPS))) void ENTRY(Params p) {
     const unsigned short* __restrict__ xp = (const unsigned short*)p.a[0];
     const unsigned short* __restrict__ wp = (const unsigned short*)p.a[1];
     const int n_img = (int)(unsigned long long)p.a[3];
     __shared__ __attribute__((aligned(16))) unsigned short xs[2][TILE_ELEMS];
+    __shared__ __attribute__((aligned(16))) unsigned short as_ring[4 * KO_WG * 32 + (KO_WG / 16 / (NWAVES >= 2 ? NWAVES / 2 : 1)) * 512];   // ring of weight slabs and a spare piece, see below
 
     // range id: the channel groups of one row range are 8 workgroups apart, so
     // they land on the same XCD (workgroups go round-robin over 8 XCDs) and
@@ -157,89 +172,177 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const unsigned sel_t = b0 ? 0x05040100u : 0x07060302u;
     const unsigned sel_a = b0 ? 0x03020504u : 0x05040100u;
     const unsigned sel_b = b0 ? 0x03020706u : 0x07060100u;
-    mjt_u32x4v stage[ITEMS_PER_WAVE];
+    // Roles.  Vector memory operations of a wave complete in order, so a wave that waits for weights it asked
+    // for after a slow load (input rows from HBM) waits for that load too.  The two kinds of load are therefore
+    // issued by different waves: the first half of the waves ("loaders") bring the weights in, the second
+    // half ("stagers") the input rows; with a single wave it does both.
+    constexpr int A_WAVES = NWAVES >= 2 ? NWAVES / 2 : 1;
+    constexpr int X_WAVES = NWAVES >= 2 ? NWAVES / 2 : 1;
+    const bool loader = wave < A_WAVES;
+    const bool stager = wave >= NWAVES - X_WAVES;
+    const int stager_id = wave - (NWAVES - X_WAVES);
+    constexpr int ITEMS = LROWS * SEGS * 8;                       // of a full tile
+    constexpr int IPW = (ITEMS + X_WAVES - 1) / X_WAVES;          // items of one stager per channel block
+    // A stager asks for item k of its share at the start of step fetch_step(k) and writes it to LDS at the end
+    // of step fetch_step(k) + SD - 1: SD steps for the row to arrive from HBM, SG items per step, SQ registers.
+    constexpr int STEPS = 2 * R_ * S_;            // steps per channel block (even)
+    // When the steps of a block are too few for that (more than SGMAX items per step), the items of a step go in
+    // rounds of at most SGMAX instead, each written as soon as it has arrived, the last one at the end of the step.
+    constexpr int SGMAX = 8;
+    constexpr int SD0 = STEPS < STAGE_DEPTH ? STEPS : STAGE_DEPTH;
+    constexpr bool BULK = (IPW + (STEPS - SD0 + 1) - 1) / (STEPS - SD0 + 1) > SGMAX;
+    constexpr int SD = BULK ? 1 : SD0;
+    constexpr int SG = (IPW + (STEPS - SD + 1) - 1) / (STEPS - SD + 1);
+    constexpr int RPS = BULK ? (SG + SGMAX - 1) / SGMAX : 1;      // rounds per step
+    constexpr int RS = (SG + RPS - 1) / RPS;                      // items per round
+    constexpr int SQ = BULK ? RS : SG * SD < IPW ? SG * SD : IPW;
+    mjt_u32x4v stage[SQ];
     // buffer descriptors (base, size in bytes): addresses are a scalar offset plus a 32-bit lane offset,
     // so no per-item 64-bit address lives in vector registers
     const __amdgpu_buffer_rsrc_t x_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(xp + (size_t)n * C_ * H_ * W_), 0, C_ * H_ * W_ * 2, 0x00020000);
     const unsigned x_lane_off = (unsigned)sr * (H_ * W_ * 2);
-    auto item_of = [&](int it, int& lr, int& seg, int& cg) {
-        const int item = wave * ITEMS_PER_WAVE + it;
+    const unsigned as_spare = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned short*)&as_ring[0] + 4 * KO_WG * 64;
+    auto item_of = [&](int item, int& lr, int& seg, int& cg) {
         cg = item & 7;
         const int rest = item >> 3;
         lr = rest / SEGS;
         seg = rest - lr * SEGS;
     };
-    // The loads are unconditional (rows outside the image and idle lanes read a clamped address and
-    // are zeroed or skipped when written): a load under a branch would make every later wait for a
-    // weight fragment wait for all staging loads as well.
-    auto fetch = [&](int r0, int lrows, int cb) {            // input rows of the tile whose first output row is r0
+    // The loads are unconditional instructions (rows outside the image and idle lanes read a clamped address and
+    // are zeroed or skipped when written; a wave whose role this is not reads beyond the descriptor's range, which
+    // costs no memory traffic): around a load under a branch the compiler no longer knows how many loads are under
+    // way and makes every later wait a wait for all of them.
+    auto fetch_item = [&](bool live, int r0, int lrows, int cb, int item) -> mjt_u32x4v {   // of the tile whose first output row is r0
         const int ir0 = r0 * SH - PH;
-#pragma unroll
-        for (int it = 0; it < ITEMS_PER_WAVE; it++) {
-            int lr, seg, cg;
-            item_of(it, lr, seg, cg);
-            int ir = ir0 + (lr < lrows ? lr : lrows - 1);
-            ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
-            const int soff = (((cb * CB + cg * 8) * H_ + ir) * W_) * 2;     // uniform: channel group and row inside the image
-            int grp = seg * 8 + sg;
-            grp = grp < GROUPS ? grp : GROUPS - 1;
-            stage[it] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)(x_lane_off + (unsigned)grp * 16), soff, 0);
-        }
+        int lr, seg, cg;
+        item_of(item, lr, seg, cg);
+        int ir = ir0 + (lr < lrows ? lr : lrows - 1);
+        ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
+        const int soff = __builtin_amdgcn_readfirstlane((((cb * CB + cg * 8) * H_ + ir) * W_) * 2);     // uniform: channel group and row inside the image
+        int grp = seg * 8 + sg;
+        grp = grp < GROUPS ? grp : GROUPS - 1;
+#if DBG & 4
+        return (mjt_u32x4v)((unsigned)soff);
+#else
+        return __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)((live ? x_lane_off : 0x80000000u) + (unsigned)grp * 16), soff, 0);
+#endif
     };
-    auto commit = [&](int r0, int lrows, int buf) {
-        const int ir0 = r0 * SH - PH;
-#pragma unroll
-        for (int it = 0; it < ITEMS_PER_WAVE; it++) {
-            int lr, seg, cg;
-            item_of(it, lr, seg, cg);
-            mjt_u32x4v d = stage[it];                        // d[k] = columns 2k (low half), 2k+1 (high half) of channel r
+    // Writing an item to LDS, in four stages that work in place on its four registers (the main loop spreads them
+    // between its MFMAs): three exchanges, then the write.
+    auto commit_stage = [&](auto sc, bool live, mjt_u32x4v& d, int r0, int lrows, int buf, int item, int limit) {
+        constexpr int stg = decltype(sc)::v;
+        int lr, seg, cg;
+        item_of(item, lr, seg, cg);
+        if constexpr (stg == 0) {
+            // d[k] = columns 2k (low half), 2k+1 (high half) of channel r
+            const int ir0 = r0 * SH - PH;
             if (ir0 + lr < 0 || ir0 + lr >= H_) d = (mjt_u32x4v)(0u);   // uniform: a row outside the image
             // lane ^ 4: keep one half of the columns, get the same half from the channel 4 away
             const unsigned g0 = mjt_xor4(b2 ? d[0] : d[2]), g1 = mjt_xor4(b2 ? d[1] : d[3]);
             const unsigned a0 = b2 ? g0 : d[0], a1 = b2 ? g1 : d[1];      // channel r & 3:       column pairs 0, 1 of the half
             const unsigned a2 = b2 ? d[2] : g0, a3 = b2 ? d[3] : g1;      // channel (r & 3) + 4
+            d[0] = a0; d[1] = a1; d[2] = a2; d[3] = a3;
+        } else if constexpr (stg == 1) {
             // lane ^ 2: keep one column pair, get it from the channel 2 away
-            const unsigned h0 = mjt_xor2(b1 ? a0 : a1), h1 = mjt_xor2(b1 ? a2 : a3);
-            const unsigned c0 = b1 ? h0 : a0, c1 = b1 ? a1 : h0;          // channels q, q+2 (q = r & 1), one column pair
-            const unsigned c2 = b1 ? h1 : a2, c3 = b1 ? a3 : h1;          // channels q+4, q+6
+            const unsigned h0 = mjt_xor2(b1 ? d[0] : d[1]), h1 = mjt_xor2(b1 ? d[2] : d[3]);
+            const unsigned c0 = b1 ? h0 : d[0], c1 = b1 ? d[1] : h0;      // channels q, q+2 (q = r & 1), one column pair
+            const unsigned c2 = b1 ? h1 : d[2], c3 = b1 ? d[3] : h1;      // channels q+4, q+6
+            d[0] = c0; d[1] = c1; d[2] = c2; d[3] = c3;
+        } else if constexpr (stg == 2) {
             // lane ^ 1: keep one column, get it from the neighbouring channels (two 16-bit values per
             // move; byte permutes with per-lane selectors keep this free of branches)
-            const unsigned s0 = mjt_xor1(__builtin_amdgcn_perm(c1, c0, sel_t)), s1 = mjt_xor1(__builtin_amdgcn_perm(c3, c2, sel_t));
+            const unsigned s0 = mjt_xor1(__builtin_amdgcn_perm(d[1], d[0], sel_t)), s1 = mjt_xor1(__builtin_amdgcn_perm(d[3], d[2], sel_t));
             mjt_u32x4v f;                                    // channels (0,1) (2,3) (4,5) (6,7) of column 8g + r
-            f[0] = __builtin_amdgcn_perm(s0, c0, sel_a);
-            f[1] = __builtin_amdgcn_perm(s0, c1, sel_b);
-            f[2] = __builtin_amdgcn_perm(s1, c2, sel_a);
-            f[3] = __builtin_amdgcn_perm(s1, c3, sel_b);
-            if (lr < lrows && seg * 64 + lane < W_) {        // rows outside the image carry zeros; columns past the row end are not the row's
-                unsigned short* dst = &xs[buf][0] + mjt_lds_off(lr * LCOLS + PW + seg * 64 + lane, cg);
-                *(mjt_u32x4v*)dst = f;
-            }
+            f[0] = __builtin_amdgcn_perm(s0, d[0], sel_a);
+            f[1] = __builtin_amdgcn_perm(s0, d[1], sel_b);
+            f[2] = __builtin_amdgcn_perm(s1, d[2], sel_a);
+            f[3] = __builtin_amdgcn_perm(s1, d[3], sel_b);
+            d = f;
+        } else {
+            // rows outside the image carry zeros; columns past the row end are not the row's; what is not to be written
+            // goes to the spare piece of LDS.  The write is spelled out: a compiler-made LDS access after the copies
+            // into the slab ring would wait for all of those first.
+            const bool wr = live && item < limit && lr < lrows && seg * 64 + lane < W_;
+            const unsigned dst = wr ? xs_base + (unsigned)(buf * TILE_ELEMS + mjt_lds_off(lr * LCOLS + PW + seg * 64 + lane, cg)) * 2
+                                    : as_spare + (unsigned)lane * 16;
+            asm volatile("ds_write_b128 %0, %1" : : "v"(dst), "v"(d) : "memory");
         }
+    };
+    auto commit_item = [&](bool live, mjt_u32x4v d, int r0, int lrows, int buf, int item, int limit) {
+        mjt_static_for<0, 4>([&](auto sc) { commit_stage(sc, live, d, r0, lrows, buf, item, limit); });
     };
 
     // A fragments: Wp[step][ko / 16][lane][8 c], step = (tap * NCB + cb) * 2 + ks: a fragment is 1 KB in lane order
-    // (lane = lg * 16 + l16 holds channels lg*8.. of row l16), so that a wave's load is one linear run of 8 cache
-    // lines; in [ko][32 c] order the 16 lanes the address unit takes together would touch 8 lines each time
-    const unsigned a_lane_off = (unsigned)(wko * MT * 1024 + lane * 16);   // bytes
+    // (lane = lg * 16 + l16 holds channels lg*8.. of row l16).  The fragments of one step for the workgroup's
+    // output channels (a slab: KO_WG / 16 KB, contiguous in Wp) go through a ring of NS slabs in LDS: the
+    // loaders copy slab g + 3 straight from memory into LDS (no registers) while step g runs; every wave
+    // reads its own MT fragments of slab g + 1 into registers during step g.  One barrier per step hands a
+    // landed slab over and frees the oldest one.
+    constexpr int NS = 4;
+    constexpr int SLAB = KO_WG * 64;              // bytes
+    constexpr int FPL = (KO_WG / 16) / A_WAVES;   // fragments a loader moves per slab
+    const unsigned as_base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned short*)&as_ring[0];
+    const unsigned a_rd_base = as_base + (unsigned)(wko * MT * 1024 + lane * 16);
     const __amdgpu_buffer_rsrc_t w_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(wp + (size_t)kpart * KO_WG * 32), 0, (R_ * S_ * C_ * K_ - kpart * KO_WG * 32) * 2, 0x00020000);
-    auto load_a = [&](mjt_bf16x8 (&a)[MT], int cb, int s) {
-        const int tap = s >> 1, ks = s & 1;
-        const int soff = ((tap * NCB + cb) * 2 + ks) * (K_ * 32 * 2);   // uniform
-#pragma unroll
-        for (int m = 0; m < MT; m++)
-            a[m] = __builtin_bit_cast(mjt_bf16x8, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)a_lane_off + (m & 3) * 1024, soff + (m >> 2) * 4096, 0));
+    auto slab_load = [&](int cb, int st, int slot) {          // all arguments uniform
+        const int tap = st >> 1, ks = st & 1;
+        const int soff = ((tap * NCB + cb) * 2 + ks) * (K_ * 64) + (loader ? wave * (FPL * 1024) : 0);
+        // the other waves issue the same instructions, out of range (zeros, no traffic) into a spare piece of LDS
+        __attribute__((address_space(3))) unsigned short* dst =
+            (__attribute__((address_space(3))) unsigned short*)&as_ring[0] + (loader ? slot * SLAB + wave * (FPL * 1024) : NS * SLAB) / 2;
+        const unsigned voff = (loader ? 0u : 0x80000000u) + (unsigned)lane * 16;
+        mjt_static_for<0, FPL>([&](auto fc) {
+            constexpr int f = decltype(fc)::v;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (__attribute__((address_space(3))) void*)(dst + (f >> 2) * 2048), 16, (int)voff,
+                                                     soff + (f >> 2) * 4096, (f & 3) * 1024, 0);
+        });
+    };
+    // (channel block, step) k steps after (cb, st); the sequence wraps after the last block: every tile uses the same weights
+    auto slab_ahead = [&](int cb, int st, int k, int& cb2, int& st2) {
+        st2 = st + k;
+        cb2 = cb;
+        while (st2 >= STEPS) {
+            st2 -= STEPS;
+            cb2 = cb2 + 1 < NCB ? cb2 + 1 : 0;
+        }
+    };
+    // End of a step: the slab asked for in the previous step has landed.  Only the FPL most recent loads of
+    // a loader may still be under way: normally the slab it has just asked for.  The loads of input rows that a
+    // loader issues are of the idle kind (out of range, they return at once); wherever the compiler places them,
+    // they can only make this wait stricter.
+    auto step_sync = [&]() {
+#if !(DBG & 32)
+        if (loader) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(FPL) : "memory");
+        asm volatile("s_barrier" : : : "memory");
+#endif
     };
 
-    constexpr int STEPS = 2 * R_ * S_;            // steps per channel block (even)
-    mjt_bf16x8 ring[2][MT];                       // weights of the next step are in flight during a step
+#if DBG & 8
+    unsigned long long* ts_out = (unsigned long long*)((float*)p.a[2] + (size_t)n_img * K_ * OH_ * OW_) + ((size_t)blockIdx.x * NWAVES + wave) * 64;
+    const __amdgpu_buffer_rsrc_t ts_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)ts_out, 0, 512, 0x00020000);
+    int ts_n = 2;
+    {
+        mjt_u32x2 hw;
+        hw[0] = __builtin_amdgcn_s_getreg(63492); hw[1] = 0;
+        __builtin_amdgcn_raw_buffer_store_b64(hw, ts_rsrc, lane == 0 ? 0 : 0x80000000, 0, 0);
+        hw[0] = __builtin_amdgcn_s_getreg((31 << 11) | 20);
+        __builtin_amdgcn_raw_buffer_store_b64(hw, ts_rsrc, lane == 0 ? 8 : 0x80000000, 0, 0);
+    }
+#define STAMP() do { unsigned long long t_ = __builtin_amdgcn_s_memrealtime(); mjt_u32x2 v_; v_[0] = (unsigned)t_; v_[1] = (unsigned)(t_ >> 32); \
+        __builtin_amdgcn_raw_buffer_store_b64(v_, ts_rsrc, lane == 0 ? ts_n * 8 : 0x80000000, 0, 0); ts_n++; } while (0)
+#else
+#define STAMP() do {} while (0)
+#endif
     int buf = 0;                                  // LDS buffer that holds the current channel block
+    int g = 0;                                    // steps done so far, modulo NS: slab of the current step is in slot g
 
     // One tile: TRW_ output rows per wave starting at r0, NT_ accumulator tiles per wave, LR_ input rows
-    // in LDS.  On entry its first channel block is in xs[buf] and its first A fragments are in ring[0];
-    // when another tile follows (next_lrows > 0) its first block and fragments are prepared the same way.
-    auto run_tile = [&](auto trw_c, auto nt_c, auto lr_c, const int r0, const int next_r0, const int next_lrows) {
+    // in LDS.  On entry its first channel block is in xs[buf], its first A fragments are in ring[0] and the
+    // slabs of its first three steps are in the ring or under way; when another tile follows
+    // (next_lrows > 0) its first block is prepared the same way.
+    auto run_tile = [&](auto trw_c, auto nt_c, auto lr_c, const int r0, const int row_lim, const int next_r0, const int next_lrows) {
         constexpr int TRW_ = decltype(trw_c)::v, NT_ = decltype(nt_c)::v, LR_ = decltype(lr_c)::v;
         // per-lane pixel of each of the NT_ tiles
         unsigned baddr[NT_];                                 // LDS byte address of the fragment at tap (0,0), k-step 0, in the current buffer
@@ -255,45 +358,124 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
         for (int m = 0; m < MT; m++)
 #pragma unroll
             for (int t = 0; t < NT_; t++) acc[m][t] = (mjt_f32x4)(0.0f);
+        // the zeros are written here, not next to the first MFMA that reads them: between a plain write of a register
+        // and a spelled-out MFMA that reads it the compiler leaves none of the cycles the hardware asks for
+        mjt_static_for<0, MT * NT_>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / NT_][decltype(ic)::v % NT_]); });
+        asm volatile("s_nop 7" : : : "memory");
 
-        // Main loop.  Per channel block the STEPS x NT_ B fragments form one stream; fragment f is
-        // requested BQ_DIST fragments before the four MFMAs that use it (a ring of BQ_DIST + 1
-        // registers), so the LDS latency hides behind 4 * BQ_DIST MFMAs of this wave.  The reads and
-        // the waits for them are written out so that this order is what runs: tap and k-step are
-        // compile-time here and fold into the offset field of the read.
-        constexpr int NF = STEPS * NT_;
-        mjt_u32x4v bq[BQ_DIST + 1];
+        // Main loop.  A step multiplies MT A fragments with NT_ B fragments.  It runs fragment by fragment of A
+        // (MT passes of NT_ MFMAs on independent accumulators): the A fragment of the next pass is read during a
+        // pass, and in the last pass each B register is refilled with the next step's fragment right after
+        // its last use, so that every LDS read has at least a pass of MFMAs to arrive.  The reads and the
+        // waits for them are written out so that this order is what runs (tap and k-step are compile-time here
+        // and fold into the offset field of the read).  LDS operations of a wave complete in order; a wait names
+        // how many of those issued later may still be under way.
+        constexpr auto writes_in = [](int st) {                  // input rows written to LDS at the end of step st
+            int n = 0;
+            for (int k = 0; k < IPW; k++) n += (k / SG + SD - 1 == st) ? 1 : 0;
+            return n;
+        };
+        // item i of round r of step st, or -1
+        constexpr auto bulk_item = [](int st, int r, int i) {
+            const int k = st * SG + r * RS + i;
+            return (r * RS + i < SG && k < IPW) ? k : -1;
+        };
+        mjt_u32x4v bfr[NT_];
+        mjt_u32x4v afr[3];                                   // A fragments of this pass and the next two
+        constexpr int PASSES = STEPS * MT;
+        STAMP();
 #pragma unroll 1
         for (int cb = 0; cb < NCB; cb++) {
             const bool more = cb + 1 < NCB;
-            mjt_static_for<0, BQ_DIST>([&](auto fc) {
-                constexpr int f = decltype(fc)::v;
-                mjt_ds_read<mjt_frag_off(f / NT_)>(bq[f % (BQ_DIST + 1)], baddr[f % NT_]);
-            });
+            const bool feed = more || next_lrows;                // somebody needs another block of input rows
+            const int f_r0 = more ? r0 : next_r0, f_lrows = more ? LR_ : next_lrows, f_cb = more ? cb + 1 : 0;
+            const int my_first = stager_id * IPW, my_limit = (stager_id + 1) * IPW < ITEMS ? (stager_id + 1) * IPW : ITEMS;
+            // nothing is under way here
+            mjt_ds_read<0>(afr[0], a_rd_base + (unsigned)((g & (NS - 1)) * SLAB));
+            mjt_ds_read<1024>(afr[1], a_rd_base + (unsigned)((g & (NS - 1)) * SLAB));
+            mjt_static_for<0, NT_>([&](auto tc) { mjt_ds_read<mjt_frag_off(0)>(bfr[decltype(tc)::v], baddr[decltype(tc)::v]); });
             mjt_static_for<0, STEPS>([&](auto sc) {
                 constexpr int st = decltype(sc)::v;
-                if (st + 1 < STEPS) load_a(ring[(st + 1) & 1], cb, st + 1);
-                else if (more) load_a(ring[0], cb + 1, 0);
-                else if (next_lrows) load_a(ring[0], 0, 0);
-                if (st == 0) {                                   // in flight during this block's MFMAs; after the weight loads,
-                    if (more) fetch(r0, LR_, cb + 1);            // so that the wait for those does not include these
-                    else if (next_lrows) fetch(next_r0, next_lrows, 0);
-                }
-                mjt_static_for<0, NT_>([&](auto tc) {
-                    constexpr int t = decltype(tc)::v;
-                    constexpr int f = st * NT_ + t;
-                    if constexpr (f + BQ_DIST < NF)
-                        mjt_ds_read<mjt_frag_off((f + BQ_DIST) / NT_)>(bq[(f + BQ_DIST) % (BQ_DIST + 1)], baddr[(f + BQ_DIST) % NT_]);
-                    mjt_lds_wait<(NF - 1 - f < BQ_DIST ? NF - 1 - f : BQ_DIST)>(bq[f % (BQ_DIST + 1)]);
-                    const mjt_bf16x8 b = __builtin_bit_cast(mjt_bf16x8, bq[f % (BQ_DIST + 1)]);
-#pragma unroll
-                    for (int m = 0; m < MT; m++)
-                        acc[m][t] = MJT_MFMA(ring[st & 1][m], b, acc[m][t], 0, 0, 0);
+                // what a step does besides its MFMAs goes between them, where it costs no MFMA time: the loads right after
+                // the first one, the stages of writing input rows to LDS after MFMA number stage_at(0..3) of the step
+                auto issue_loads = [&]() {
+                    if constexpr (!BULK) {
+                        mjt_static_for<0, IPW>([&](auto kc) {
+                            constexpr int k = decltype(kc)::v;
+                            if constexpr (k / SG == st) stage[k % SQ] = fetch_item(stager && feed, f_r0, f_lrows, f_cb, my_first + k);
+                        });
+                    } else {
+                        mjt_static_for<0, RPS>([&](auto rc) {
+                            constexpr int r = decltype(rc)::v;
+                            mjt_static_for<0, RS>([&](auto ic) {
+                                constexpr int k = bulk_item(st, r, decltype(ic)::v);
+                                if constexpr (k >= 0) stage[decltype(ic)::v] = fetch_item(stager && feed, f_r0, f_lrows, f_cb, my_first + k);
+                            });
+                            if constexpr (r + 1 < RPS)
+                                mjt_static_for<0, RS>([&](auto ic) {
+                                    constexpr int k = bulk_item(st, r, decltype(ic)::v);
+                                    if constexpr (k >= 0) commit_item(stager && feed, stage[decltype(ic)::v], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);
+                                });
+                        });
+                    }
+#if !(DBG & 16)
+                    int cb3, st3;
+                    slab_ahead(cb, st, NS - 1, cb3, st3);
+                    slab_load(cb3, st3, (g + st + NS - 1) & (NS - 1));
+#endif
+                };
+                constexpr auto stage_at = [](int sg) { return NT_ + (sg * (MT - 2) * NT_) / 4; };
+                auto commit_stages = [&](auto ic) {          // ic: MFMAs of this step issued so far
+                    constexpr int i = decltype(ic)::v;
+                    mjt_static_for<0, 4>([&](auto sc) {
+                        if constexpr (stage_at(decltype(sc)::v) == i) {
+                            if constexpr (!BULK) {
+                                mjt_static_for<0, IPW>([&](auto kc) {
+                                    constexpr int k = decltype(kc)::v;
+                                    if constexpr (k / SG + SD - 1 == st)
+                                        commit_stage(sc, stager && feed, stage[k % SQ], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);   // the other buffer: nobody reads it now
+                                });
+                            } else {
+                                mjt_static_for<0, RS>([&](auto jc) {
+                                    constexpr int k = bulk_item(st, RPS - 1, decltype(jc)::v);
+                                    if constexpr (k >= 0) commit_stage(sc, stager && feed, stage[decltype(jc)::v], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);
+                                });
+                            }
+                        }
+                    });
+                };
+                const unsigned a_cur = a_rd_base + (unsigned)(((g + st) & (NS - 1)) * SLAB);
+                const unsigned a_nxt = a_rd_base + (unsigned)(((g + st + 1) & (NS - 1)) * SLAB);
+                mjt_static_for<0, MT>([&](auto mc) {
+                    constexpr int m = decltype(mc)::v;
+                    constexpr int P = st * MT + m;                           // pass number in the block; its fragment sits in afr[P % 3]
+#if !(DBG & 128)
+                    if constexpr (P + 2 < PASSES) {                          // the fragment two passes ahead: of this step or the next
+                        if constexpr (m + 2 < MT) mjt_ds_read<(m + 2) * 1024>(afr[(P + 2) % 3], a_cur);
+                        else mjt_ds_read<(m + 2 - MT) * 1024>(afr[(P + 2) % 3], a_nxt);
+                    }
+#endif
+                    mjt_static_for<0, NT_>([&](auto tc) {
+                        constexpr int t = decltype(tc)::v;
+                        // the rows written in this step are written before its last pass: no LDS write follows the B reads
+                        // B fragment t was asked for before the reads of the rest of its step and of the A fragment two passes
+                        // ahead (the A fragment of this pass is older than all of those); behind an A fragment come those of
+                        // the next two passes
+                        if constexpr (m == 0) mjt_lds_wait<(BULK ? 0 : NT_ - 1 - t + (P + 2 < PASSES ? 1 : 0))>(bfr[t]);
+                        else if constexpr (t == 0) mjt_lds_wait<(P + 1 < PASSES ? 1 : 0) + (P + 2 < PASSES ? 1 : 0)>(afr[P % 3]);
+                        mjt_mfma(acc[m][t], afr[P % 3], bfr[t]);
+#if !(DBG & 64)
+                        if constexpr (m + 1 == MT && st + 1 < STEPS) mjt_ds_read<mjt_frag_off(st + 1)>(bfr[t], baddr[t]);
+#endif
+                        if constexpr (m == 0 && t == 0) issue_loads();
+                        commit_stages(mjt_ic<m * NT_ + t + 1>());
+                    });
                 });
+                if (st + 1 == STEPS) asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");   // the rows written for the next block
+                step_sync();
             });
-            if (more || next_lrows) {
-                commit(more ? r0 : next_r0, more ? LR_ : next_lrows, buf ^ 1);        // the other buffer: nobody reads it now
-                __syncthreads();
+            g = (g + STEPS) & (NS - 1);
+            if (feed) {
                 buf ^= 1;
 #pragma unroll
                 for (int t = 0; t < NT_; t++) baddr[t] += buf ? (unsigned)(TILE_ELEMS * 2) : (unsigned)(-(TILE_ELEMS * 2));
@@ -301,6 +483,16 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
         }
 
         // epilogue: lane holds D[ko = 4*(lane/16)+i][px = lane%16] of each tile
+        // The compiler takes a spelled-out MFMA for finished the moment it is issued.  Give the last ones the
+        // time to read their operands and write their results, and tie the registers to a point behind that:
+        // the operands stay allocated up to here, and nothing reads an accumulator before.
+        asm volatile("s_nop 15\n\ts_nop 15" : : : "memory");
+        mjt_keep(afr[0]);
+        mjt_keep(afr[1]);
+        mjt_keep(afr[2]);
+        mjt_static_for<0, NT_>([&](auto tc) { mjt_keep(bfr[decltype(tc)::v]); });
+        mjt_static_for<0, MT * NT_>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / NT_][decltype(ic)::v % NT_]); });
+        STAMP();
 #if OW_ % 4 == 0
         // The four lanes of a quad (4 pixels x 4 channels) transpose among themselves, after which lane j
         // of the quad owns channel 4*(lane/16)+j for the quad's 4 consecutive pixels: one 16-byte (or
@@ -312,7 +504,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
             const int q0 = t * 16 + (l16 & ~3);
             const int r = q0 / OW_, col = q0 - r * OW_;
             const int orow = r0 + wpx * TRW_ + r;
-            const bool ok = q0 < TRW_ * OW_ && orow < row_end;
+            const bool ok = q0 < TRW_ * OW_ && orow < row_lim;
 #pragma unroll
             for (int m = 0; m < MT; m++) {
                 const mjt_f32x4 v = acc[m][t];
@@ -327,9 +519,18 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
                 y4[1] = b1 ? h1 : a1;
                 y4[2] = b1 ? a2 : h0;
                 y4[3] = b1 ? a3 : h1;
+#if (DBG & 3) == 2
+                if (y4[0] == 123.456f) ((float*)p.a[2])[0] = y4[1] + y4[2] + y4[3];
+                if (false) {
+#else
                 if (ok) {
+#endif
                     const int ko = ko_base + m * 16 + lg * 4 + qj;
+#if (DBG & 3) == 1
+                    const size_t o = ((size_t)blockIdx.x * NWAVES + wave) * (MT * NT * 256) + (size_t)((t * MT + m) * 256 + lane * 4);
+#else
                     const size_t o = (((size_t)n * K_ + ko) * OH_ + orow) * OW_ + col;
+#endif
 #if Y_BF16
                     mjt_u32x2 pk;
                     pk[0] = mjt_narrow2(y4[0], y4[1]);
@@ -347,7 +548,7 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
             const int q = t * 16 + l16;
             const int r = q / OW_, col = q - r * OW_;
             const int orow = r0 + wpx * TRW_ + r;
-            if (q < TRW_ * OW_ && orow < row_end) {
+            if (q < TRW_ * OW_ && orow < row_lim) {
 #pragma unroll
                 for (int m = 0; m < MT; m++)
 #pragma unroll
@@ -365,25 +566,64 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
 #endif
     };
 
-    // tiles of this workgroup: full tiles while they start inside the row range, then the short one
+    STAMP();
+    // tiles of this workgroup: full tiles while they start inside the row range, then the short one.  With
+    // TAIL_FIRST every other workgroup of a compute unit walks the short tile first instead: the two then reach
+    // the ends of their tiles, where a workgroup only stores, at different times, and the MFMAs of one cover
+    // the stores of the other.
     int nfull = (row_end - row_begin + TR - 1) / TR;
     if (nfull > NFULL) nfull = NFULL;
     const bool tail = TAIL_TRW > 0 && row_begin + NFULL * TR < row_end;
-    const int first_lrows = nfull ? LROWS : TAIL_LROWS;
-
-    load_a(ring[0], 0, 0);
-    fetch(row_begin, first_lrows, 0);
-    __syncthreads();                              // zero fill done
-    commit(row_begin, first_lrows, 0);
-    __syncthreads();
-    for (int s = 0; s < nfull; s++) {
-        const int r0 = row_begin + s * TR;
-        const int next_lrows = s + 1 < nfull ? LROWS : tail ? TAIL_LROWS : 0;
-        run_tile(mjt_ic<TRW>(), mjt_ic<NT>(), mjt_ic<LROWS>(), r0, r0 + TR, next_lrows);
-    }
-#if TAIL_TRW > 0
-    if (tail) run_tile(mjt_ic<TAIL_TRW>(), mjt_ic<TAIL_NT>(), mjt_ic<TAIL_LROWS>(), row_begin + NFULL * TR, 0, 0);
+#if TAIL_FIRST && TAIL_TRW > 0
+    constexpr int REM = RPW - NFULL * TR;          // rows of the short tile
+    const bool tail_first = tail && row_begin + RPW <= OH_ && ((j / SLOT_STRIDE) & 1);
+#else
+    constexpr int REM = 0;
+    const bool tail_first = false;
 #endif
+    const int first_lrows = tail_first ? TAIL_LROWS : nfull ? LROWS : TAIL_LROWS;
+    const int ntiles = nfull + (tail ? 1 : 0);
+    const int tail_at = tail ? (tail_first ? 0 : nfull) : -1;
+    const int full_base = row_begin + (tail_first ? REM : 0);
+
+    // the slabs of the first three steps, the first block of input rows (every wave takes a share here), the
+    // fragments of the first step
+    mjt_static_for<0, NS - 1>([&](auto kc) {
+        int cb0, st0;
+        slab_ahead(0, 0, decltype(kc)::v, cb0, st0);
+        slab_load(cb0, st0, decltype(kc)::v);
+    });
+    __syncthreads();                              // zero fill done
+    {
+        constexpr int PQ0 = (ITEMS + NWAVES - 1) / NWAVES;     // no accumulators yet: registers to spare
+        constexpr int PQ = PQ0 < 16 ? PQ0 : 16;
+        mjt_u32x4v pre[PQ];
+#pragma unroll 1
+        for (int first = wave * PQ; first < ITEMS; first += NWAVES * PQ) {
+#pragma unroll
+            for (int k = 0; k < PQ; k++) pre[k] = fetch_item(true, row_begin, first_lrows, 0, first + k);
+#pragma unroll
+            for (int k = 0; k < PQ; k++) commit_item(true, pre[k], row_begin, first_lrows, 0, first + k, ITEMS);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");   // the slabs
+    __syncthreads();
+#pragma unroll 1
+    for (int i = 0; i < ntiles; i++) {
+        const int next_lrows = i + 1 >= ntiles ? 0 : i + 1 == tail_at ? TAIL_LROWS : LROWS;
+        const int s = tail_first ? i - 1 : i;    // index among the full tiles
+#if TAIL_TRW > 0
+        if (i == tail_at) {
+            const int r0 = tail_first ? row_begin : row_begin + NFULL * TR;
+            run_tile(mjt_ic<TAIL_TRW>(), mjt_ic<TAIL_NT>(), mjt_ic<TAIL_LROWS>(), r0, tail_first ? row_begin + REM : row_end, full_base, next_lrows);
+            continue;
+        }
+#endif
+        const int r0 = full_base + s * TR;
+        run_tile(mjt_ic<TRW>(), mjt_ic<NT>(), mjt_ic<LROWS>(), r0, row_end, i + 1 == tail_at ? row_begin + NFULL * TR : r0 + TR, next_lrows);
+    }
+    STAMP();
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");   // slabs asked for past the last step
 }
 
 // Weight re-pack: w[ko][c][kh][kw] -> Wp[tap][c/64][k-step][ko/16][lg][l16][8 c] (c = 32 k-step + 8 lg + ..)

@@ -102,7 +102,15 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     // ---- MFMA path ----------------------------------------------------------------
     const char* wpx_env = getenv("MJT_CONV_WPX");
     const int64_t WPX = wpx_env && atoi(wpx_env) == 1 ? 1 : 2;
-    const int64_t max_px = WPX == 1 ? 224 : 112;            // pixels per wave: 16 per accumulator tile
+    const char* pxw_env = getenv("MJT_CONV_PXW");
+    const int64_t max_px = pxw_env && (atoi(pxw_env) == 112 || atoi(pxw_env) == 224) ? atoi(pxw_env) : WPX == 1 ? 224 : 112;   // pixels per wave: 16 per accumulator tile
+    const int64_t WPS = max_px == 224 ? 1 : 2;              // waves per SIMD the register budget is set for
+    // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
+    const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
+    int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
+    // LDS: two buffers of input rows and a ring of four weight slabs (64 bytes per output channel of the workgroup each)
+    const int64_t lds_total = 160 * 1024;
+    const int64_t tile_limit = (lds_total - 4 * 64 * 16 * MT * WKO) / 2;
     int64_t TRW = OW <= max_px ? max_px / OW : 0;
     if (TRW > OH) TRW = OH;
     while (TRW > 1 && WPX * TRW > OH && (OH % (WPX * TRW)) != 0 && (WPX * (TRW - 1)) >= OH) TRW--;
@@ -110,13 +118,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t LCOLS = (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1 > W + 2 * p->pad_w
                               ? (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1
                               : W + 2 * p->pad_w;
-    while (TRW > 1 && lds_rows(TRW) * LCOLS * 128 > 72 * 1024) TRW--;   // two buffers of this size live in LDS
+    while (TRW > 1 && lds_rows(TRW) * LCOLS * 128 > tile_limit) TRW--;
     const int64_t NT = TRW ? (TRW * OW + 15) / 16 : 0;
     const int64_t LROWS = lds_rows(TRW);
-    // output channels per workgroup: 64 per pair of waves, up to 256
-    // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
-    const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
-    int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
     {
         // fewer output channels per workgroup while the grid would leave compute units idle (small maps, small batches):
         // the same input tile is then staged by more workgroups, which the L2 absorbs
@@ -129,7 +133,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     }
     const bool half = x->dtype == MJT_FLOAT16;
     const bool mfma_ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % 64 == 0 && K % 64 == 0 &&
-                         W % 2 == 0 && TRW >= 1 && NT <= (WPX == 1 ? 14 : 7) && LROWS * LCOLS * 128 <= 72 * 1024 &&
+                         W % 2 == 0 && TRW >= 1 && NT <= max_px / 16 && LROWS * LCOLS * 128 <= tile_limit &&
                          // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
                          ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + 4 * LROWS * LCOLS * 16 < 65536 &&
                          (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49 &&
@@ -170,7 +174,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const char* bq_env = getenv("MJT_CONV_BQ");
         const int BQ = bq_env && *bq_env ? atoi(bq_env) : 3;   // B fragments requested ahead of use
         std::ostringstream key;
-        key << "mfma|" << half << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT;
+        const bool tail_first = getenv("MJT_CONV_TAIL_FIRST") && atoi(getenv("MJT_CONV_TAIL_FIRST")) && TAIL_TRW > 0 && (RPW - NFULL * TR) % WPX == 0;
+        const int64_t slot_stride = getenv("MJT_CONV_SLOT_STRIDE") ? atoi(getenv("MJT_CONV_SLOT_STRIDE")) : cus / 8 > 0 ? cus / 8 : 1;
+        key << "mfma|" << half << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT << "|" << WPS << "|" << tail_first << "|" << slot_stride << "|" << (getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0) << "|" << (getenv("MJT_CONV_SD") ? atoi(getenv("MJT_CONV_SD")) : 4);
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
@@ -183,7 +189,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                 << "#define MT " << MT << "\n#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
                 << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS  << "\n#define BQ_DIST " << BQ << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype != MJT_FLOAT32 ? 1 : 0) << "\n#define IN_F16 " << (half ? 1 : 0)
-                << "\n";
+                << "\n#define WPS " << WPS << "\n#define TAIL_FIRST " << (tail_first ? 1 : 0) << "\n#define STAGE_DEPTH " << (getenv("MJT_CONV_SD") ? atoi(getenv("MJT_CONV_SD")) : 4) << "\n#define SLOT_STRIDE " << slot_stride << "\n#define DBG " << (getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0) << "\n";
             src << embedded_source("conv_mfma.h") << "\n";
             k = jit_get(src.str(), name.str());
             kp = new JitKernel();
