@@ -65,7 +65,7 @@ typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
 
 struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as pointers: global address space)
 
-#define CB 64
+#define KSTEPS (CB / 32)                    // MFMA k-steps per tap in a channel block of CB (32 or 64) channels
 #define KO_WG (16 * MT * WKO)
 #define NWAVES (WPX * WKO)
 #define NTHR (64 * NWAVES)
@@ -74,7 +74,7 @@ struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as p
 #define NCB (C_ / CB)
 #define GROUPS ((W_ + 7) / 8)           // groups of 8 columns; the last one may reach past the row: what it reads there is never written
 #define SEGS ((GROUPS + 7) / 8)         // segments of 64 columns
-#define TILE_ELEMS (LROWS * LCOLS * 64)
+#define TILE_ELEMS (LROWS * LCOLS * CB)
 
 // LDS tile: 8 planes, one per group of 8 channels, each [row][col][8 c] (16 bytes per position).  The 16 lanes
 // that read a fragment together (16 neighbouring pixels, one channel group) then touch one 256-byte run, which
@@ -96,7 +96,7 @@ template <int I, int N, class F> __device__ __forceinline__ void mjt_static_for(
 }
 // byte offset inside the LDS tile of step s = (tap, k-step): row/column shift of the tap, 4 planes per k-step
 __device__ constexpr int mjt_frag_off(int s) {
-    return ((((s >> 1) / S_) * DH * LCOLS + ((s >> 1) % S_) * DW) * 8 + (s & 1) * 4 * PLANE_ELEMS) * 2;
+    return ((((s / KSTEPS) / S_) * DH * LCOLS + ((s / KSTEPS) % S_) * DW) * 8 + (s % KSTEPS) * 4 * PLANE_ELEMS) * 2;
 }
 // value of lane ^ 1, ^ 2, ^ 4 through data-parallel-primitive moves (quad permutes; ^ 4 is a mirror
 // of each group of 8 lanes followed by a reversal inside each quad)
@@ -132,7 +132,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     const unsigned short* __restrict__ wp = (const unsigned short*)p.a[1];
     const int n_img = (int)(unsigned long long)p.a[3];
     __shared__ __attribute__((aligned(16))) unsigned short xs[2][TILE_ELEMS];
-    __shared__ __attribute__((aligned(16))) unsigned short as_ring[4 * KO_WG * 32 + (KO_WG / 16 / (NWAVES >= 2 ? NWAVES / 2 : 1)) * 512];   // ring of weight slabs and a spare piece, see below
+    __shared__ __attribute__((aligned(16))) unsigned short as_ring[NS * KO_WG * 32 + 4096];   // ring of weight slabs and a spare piece, see below
 
     // range id: the channel groups of one row range are 8 workgroups apart, so
     // they land on the same XCD (workgroups go round-robin over 8 XCDs) and
@@ -176,16 +176,22 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // for after a slow load (input rows from HBM) waits for that load too.  The two kinds of load are therefore
     // issued by different waves: the first half of the waves ("loaders") bring the weights in, the second
     // half ("stagers") the input rows; with a single wave it does both.
+#if ROLES
     constexpr int A_WAVES = NWAVES >= 2 ? NWAVES / 2 : 1;
     constexpr int X_WAVES = NWAVES >= 2 ? NWAVES / 2 : 1;
     const bool loader = wave < A_WAVES;
     const bool stager = wave >= NWAVES - X_WAVES;
     const int stager_id = wave - (NWAVES - X_WAVES);
-    constexpr int ITEMS = LROWS * SEGS * 8;                       // of a full tile
+#else
+    constexpr int A_WAVES = NWAVES, X_WAVES = NWAVES;
+    constexpr bool loader = true, stager = true;
+    const int stager_id = wave;
+#endif
+    constexpr int ITEMS = LROWS * SEGS * (CB / 8);                       // of a full tile
     constexpr int IPW = (ITEMS + X_WAVES - 1) / X_WAVES;          // items of one stager per channel block
     // A stager asks for item k of its share at the start of step fetch_step(k) and writes it to LDS at the end
     // of step fetch_step(k) + SD - 1: SD steps for the row to arrive from HBM, SG items per step, SQ registers.
-    constexpr int STEPS = 2 * R_ * S_;            // steps per channel block (even)
+    constexpr int STEPS = KSTEPS * R_ * S_;       // steps per channel block
     // When the steps of a block are too few for that (more than SGMAX items per step), the items of a step go in
     // rounds of at most SGMAX instead, each written as soon as it has arrived, the last one at the end of the step.
     constexpr int SGMAX = 8;
@@ -202,10 +208,10 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     const __amdgpu_buffer_rsrc_t x_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(xp + (size_t)n * C_ * H_ * W_), 0, C_ * H_ * W_ * 2, 0x00020000);
     const unsigned x_lane_off = (unsigned)sr * (H_ * W_ * 2);
-    const unsigned as_spare = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned short*)&as_ring[0] + 4 * KO_WG * 64;
+    const unsigned as_spare = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned short*)&as_ring[0] + NS * KO_WG * 64;
     auto item_of = [&](int item, int& lr, int& seg, int& cg) {
-        cg = item & 7;
-        const int rest = item >> 3;
+        cg = item % (CB / 8);
+        const int rest = item / (CB / 8);
         lr = rest / SEGS;
         seg = rest - lr * SEGS;
     };
@@ -230,6 +236,33 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     };
     // Writing an item to LDS, in four stages that work in place on its four registers (the main loop spreads them
     // between its MFMAs): three exchanges, then the write.
+    // The same load spelled out, for the main loop: every vector memory operation there is, and so the number of them
+    // issued between two points is known and the waits can name exactly the loads that may still be under way.
+    mjt_u32x4v x_desc;
+    {
+        const unsigned long long base = (unsigned long long)(xp + (size_t)n * C_ * H_ * W_);
+        x_desc[0] = __builtin_amdgcn_readfirstlane((unsigned)base);
+        x_desc[1] = __builtin_amdgcn_readfirstlane((unsigned)(base >> 32) & 0xffffu);
+        x_desc[2] = C_ * H_ * W_ * 2;
+        x_desc[3] = 0x00020000;
+    }
+    auto fetch_item_fixed = [&](mjt_u32x4v& dst, bool live, int r0, int lrows, int cb, int item) {
+        const int ir0 = r0 * SH - PH;
+        int lr, seg, cg;
+        item_of(item, lr, seg, cg);
+        int ir = ir0 + (lr < lrows ? lr : lrows - 1);
+        ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
+        const int soff = __builtin_amdgcn_readfirstlane((((cb * CB + cg * 8) * H_ + ir) * W_) * 2);
+        int grp = seg * 8 + sg;
+        grp = grp < GROUPS ? grp : GROUPS - 1;
+        const unsigned voff = (live ? x_lane_off : 0x80000000u) + (unsigned)grp * 16;
+#if DBG & 4
+        dst = (mjt_u32x4v)(voff);
+        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=v"(dst[0]) : "v"(0x80000000u), "s"(x_desc), "s"(soff) : "memory");
+#else
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(dst) : "v"(voff), "s"(x_desc), "s"(soff) : "memory");
+#endif
+    };
     auto commit_stage = [&](auto sc, bool live, mjt_u32x4v& d, int r0, int lrows, int buf, int item, int limit) {
         constexpr int stg = decltype(sc)::v;
         int lr, seg, cg;
@@ -279,7 +312,6 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // loaders copy slab g + 3 straight from memory into LDS (no registers) while step g runs; every wave
     // reads its own MT fragments of slab g + 1 into registers during step g.  One barrier per step hands a
     // landed slab over and frees the oldest one.
-    constexpr int NS = 4;
     constexpr int SLAB = KO_WG * 64;              // bytes
     constexpr int FPL = (KO_WG / 16) / A_WAVES;   // fragments a loader moves per slab
     const unsigned as_base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned short*)&as_ring[0];
@@ -287,8 +319,8 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     const __amdgpu_buffer_rsrc_t w_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(wp + (size_t)kpart * KO_WG * 32), 0, (R_ * S_ * C_ * K_ - kpart * KO_WG * 32) * 2, 0x00020000);
     auto slab_load = [&](int cb, int st, int slot) {          // all arguments uniform
-        const int tap = st >> 1, ks = st & 1;
-        const int soff = ((tap * NCB + cb) * 2 + ks) * (K_ * 64) + (loader ? wave * (FPL * 1024) : 0);
+        const int tap = st / KSTEPS, ks = st % KSTEPS;
+        const int soff = ((tap * NCB + cb) * KSTEPS + ks) * (K_ * 64) + (loader ? wave * (FPL * 1024) : 0);
         // the other waves issue the same instructions, out of range (zeros, no traffic) into a spare piece of LDS
         __attribute__((address_space(3))) unsigned short* dst =
             (__attribute__((address_space(3))) unsigned short*)&as_ring[0] + (loader ? slot * SLAB + wave * (FPL * 1024) : NS * SLAB) / 2;
@@ -308,13 +340,12 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
             cb2 = cb2 + 1 < NCB ? cb2 + 1 : 0;
         }
     };
-    // End of a step: the slab asked for in the previous step has landed.  Only the FPL most recent loads of
-    // a loader may still be under way: normally the slab it has just asked for.  The loads of input rows that a
-    // loader issues are of the idle kind (out of range, they return at once); wherever the compiler places them,
-    // they can only make this wait stricter.
-    auto step_sync = [&]() {
+    // End of step g: slab g + 2 has landed (the next step reads its first fragments).  What was asked for later may
+    // still be under way: the loads of the last NS - 3 steps, slabs and input rows alike (all of them are spelled out
+    // in the loop, so their number is known).
+    auto step_sync = [&](auto nc) {                  // nc: loads issued in the last NS - 3 steps, this one included
 #if !(DBG & 32)
-        if (loader) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(FPL) : "memory");
+        if (loader) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(decltype(nc)::v < 63 ? decltype(nc)::v : 63) : "memory");
         asm volatile("s_barrier" : : : "memory");
 #endif
     };
@@ -375,6 +406,18 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
             for (int k = 0; k < IPW; k++) n += (k / SG + SD - 1 == st) ? 1 : 0;
             return n;
         };
+        // input-row loads a wave issues in step s of a block (s may run past the block's ends: every block has the same schedule)
+        constexpr auto loads_in = [](int s) {
+            const int st = ((s % STEPS) + STEPS) % STEPS;
+            int n = 0;
+            for (int k = 0; k < IPW; k++) n += (k / SG == st) ? 1 : 0;
+            return n;
+        };
+        constexpr auto loads_between = [=](int s0, int s1) {      // in steps s0 .. s1 - 1
+            int n = 0;
+            for (int s = s0; s < s1; s++) n += loads_in(s);
+            return n;
+        };
         // item i of round r of step st, or -1
         constexpr auto bulk_item = [](int st, int r, int i) {
             const int k = st * SG + r * RS + i;
@@ -391,8 +434,8 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
             const int f_r0 = more ? r0 : next_r0, f_lrows = more ? LR_ : next_lrows, f_cb = more ? cb + 1 : 0;
             const int my_first = stager_id * IPW, my_limit = (stager_id + 1) * IPW < ITEMS ? (stager_id + 1) * IPW : ITEMS;
             // nothing is under way here
-            mjt_ds_read<0>(afr[0], a_rd_base + (unsigned)((g & (NS - 1)) * SLAB));
-            mjt_ds_read<1024>(afr[1], a_rd_base + (unsigned)((g & (NS - 1)) * SLAB));
+            mjt_ds_read<0>(afr[0], a_rd_base + (unsigned)((g % NS) * SLAB));
+            mjt_ds_read<1024>(afr[1], a_rd_base + (unsigned)((g % NS) * SLAB));
             mjt_static_for<0, NT_>([&](auto tc) { mjt_ds_read<mjt_frag_off(0)>(bfr[decltype(tc)::v], baddr[decltype(tc)::v]); });
             mjt_static_for<0, STEPS>([&](auto sc) {
                 constexpr int st = decltype(sc)::v;
@@ -402,7 +445,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                     if constexpr (!BULK) {
                         mjt_static_for<0, IPW>([&](auto kc) {
                             constexpr int k = decltype(kc)::v;
-                            if constexpr (k / SG == st) stage[k % SQ] = fetch_item(stager && feed, f_r0, f_lrows, f_cb, my_first + k);
+                            if constexpr (k / SG == st) fetch_item_fixed(stage[k % SQ], stager && feed, f_r0, f_lrows, f_cb, my_first + k);
                         });
                     } else {
                         mjt_static_for<0, RPS>([&](auto rc) {
@@ -421,7 +464,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
 #if !(DBG & 16)
                     int cb3, st3;
                     slab_ahead(cb, st, NS - 1, cb3, st3);
-                    slab_load(cb3, st3, (g + st + NS - 1) & (NS - 1));
+                    slab_load(cb3, st3, (g + st + NS - 1) % NS);
 #endif
                 };
                 constexpr auto stage_at = [](int sg) { return NT_ + (sg * (MT - 2) * NT_) / 4; };
@@ -432,8 +475,15 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                             if constexpr (!BULK) {
                                 mjt_static_for<0, IPW>([&](auto kc) {
                                     constexpr int k = decltype(kc)::v;
-                                    if constexpr (k / SG + SD - 1 == st)
+                                    if constexpr (k / SG + SD - 1 == st) {
+                                        // loads issued after that of item k: the rest of its step (input rows come first in a step, then
+                                        // the slab), then SD - 1 whole steps
+                                        if constexpr (decltype(sc)::v == 0) {
+                                            constexpr int after = (loads_in(k / SG) - 1 - k % SG) + FPL + (SD - 1) * FPL + loads_between(k / SG + 1, k / SG + SD);
+                                            asm volatile("s_waitcnt vmcnt(%1)" : "+v"(stage[k % SQ]) : "n"(after < 63 ? after : 63));
+                                        }
                                         commit_stage(sc, stager && feed, stage[k % SQ], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);   // the other buffer: nobody reads it now
+                                    }
                                 });
                             } else {
                                 mjt_static_for<0, RS>([&](auto jc) {
@@ -444,8 +494,11 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                         }
                     });
                 };
-                const unsigned a_cur = a_rd_base + (unsigned)(((g + st) & (NS - 1)) * SLAB);
-                const unsigned a_nxt = a_rd_base + (unsigned)(((g + st + 1) & (NS - 1)) * SLAB);
+                const unsigned a_cur = a_rd_base + (unsigned)(((g + st) % NS) * SLAB);
+                const unsigned a_nxt = a_rd_base + (unsigned)(((g + st + 1) % NS) * SLAB);
+#if DBG & 256
+                if constexpr (st >= 4 && st < 10) STAMP();
+#endif
                 mjt_static_for<0, MT>([&](auto mc) {
                     constexpr int m = decltype(mc)::v;
                     constexpr int P = st * MT + m;                           // pass number in the block; its fragment sits in afr[P % 3]
@@ -470,11 +523,14 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                         if constexpr (m == 0 && t == 0) issue_loads();
                         commit_stages(mjt_ic<m * NT_ + t + 1>());
                     });
+#if DBG & 256
+                    if constexpr (st >= 4 && st < 10) STAMP();
+#endif
                 });
                 if (st + 1 == STEPS) asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");   // the rows written for the next block
-                step_sync();
+                step_sync(mjt_ic<(BULK ? 0 : (NS - 3) * FPL + loads_between(st - (NS - 4), st + 1))>());
             });
-            g = (g + STEPS) & (NS - 1);
+            g = (g + STEPS) % NS;
             if (feed) {
                 buf ^= 1;
 #pragma unroll
@@ -537,7 +593,11 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                     pk[1] = mjt_narrow2(y4[2], y4[3]);
                     *(mjt_u32x2*)((unsigned short*)p.a[2] + o) = pk;
 #else
+#if STORE_NT
+                    __builtin_nontemporal_store(y4, (mjt_f32x4*)((float*)p.a[2] + o));
+#else
                     *(mjt_f32x4*)((float*)p.a[2] + o) = y4;
+#endif
 #endif
                 }
             }
@@ -636,7 +696,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY_PACK(Params p) {
         int rest = o >> 9;
         int ko = (rest % (K_ / 16)) * 16 + l16; rest /= K_ / 16;
         int c32 = lg * 8 + c8;
-        int ks = rest & 1; rest >>= 1;
+        int ks = rest % KSTEPS; rest /= KSTEPS;
         int cb = rest % NCB;
         int tap = rest / NCB;
         int c = cb * CB + ks * 32 + c32;

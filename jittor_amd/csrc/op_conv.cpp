@@ -108,9 +108,13 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
     const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
     int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
-    // LDS: two buffers of input rows and a ring of four weight slabs (64 bytes per output channel of the workgroup each)
+    // LDS: two buffers of input rows (one block of CB channels each), a ring of NS weight slabs (64 bytes per output
+    // channel of the workgroup each) and a spare piece the size of a loader's share of a slab.  Blocks of 32 channels
+    // leave room for a deeper ring, which is what hides the latency of the slabs; the ring needs three slabs at least.
     const int64_t lds_total = 160 * 1024;
-    const int64_t tile_limit = (lds_total - 4 * 64 * 16 * MT * WKO) / 2;
+    const int64_t CBLK = getenv("MJT_CONV_CB") && atoi(getenv("MJT_CONV_CB")) == 64 ? 64 : 32;
+    const int64_t slab0 = 64 * 16 * MT * WKO, spare0 = 8 * 1024;
+    const int64_t tile_limit = (lds_total - 4 * slab0 - spare0) / 2;         // leaves room for four slabs of the widest workgroup
     int64_t TRW = OW <= max_px ? max_px / OW : 0;
     if (TRW > OH) TRW = OH;
     while (TRW > 1 && WPX * TRW > OH && (OH % (WPX * TRW)) != 0 && (WPX * (TRW - 1)) >= OH) TRW--;
@@ -118,7 +122,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t LCOLS = (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1 > W + 2 * p->pad_w
                               ? (OW - 1) * p->stride_w + (S - 1) * p->dil_w + 1
                               : W + 2 * p->pad_w;
-    while (TRW > 1 && lds_rows(TRW) * LCOLS * 128 > tile_limit) TRW--;
+    while (TRW > 1 && lds_rows(TRW) * LCOLS * CBLK * 2 > tile_limit) TRW--;
     const int64_t NT = TRW ? (TRW * OW + 15) / 16 : 0;
     const int64_t LROWS = lds_rows(TRW);
     {
@@ -133,9 +137,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     }
     const bool half = x->dtype == MJT_FLOAT16;
     const bool mfma_ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % 64 == 0 && K % 64 == 0 &&
-                         W % 2 == 0 && TRW >= 1 && NT <= max_px / 16 && LROWS * LCOLS * 128 <= tile_limit &&
+                         W % 2 == 0 && TRW >= 1 && NT <= max_px / 16 && LROWS * LCOLS * CBLK * 2 <= tile_limit &&
                          // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
-                         ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + 4 * LROWS * LCOLS * 16 < 65536 &&
+                         ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + (CBLK == 64 ? 4 * LROWS * LCOLS * 16 : 0) < 65536 &&
                          (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49 &&
                          // byte offsets inside one image and inside the weights are 32-bit in the kernel
                          C * H * W * 2 < (int64_t(1) << 31) && K * OH * OW * 4 < (int64_t(1) << 31) && numel(w) * 2 < (int64_t(1) << 31);
@@ -174,9 +178,16 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const char* bq_env = getenv("MJT_CONV_BQ");
         const int BQ = bq_env && *bq_env ? atoi(bq_env) : 3;   // B fragments requested ahead of use
         std::ostringstream key;
+        const int64_t slab = 64 * 16 * MT * WKO;
+        const int64_t spare = 8 * 1024;
+        int64_t NSLAB = (lds_total - 2 * LROWS * LCOLS * CBLK * 2 - spare) / slab;
+        if (NSLAB > 8) NSLAB = 8;
+        if (const char* e = getenv("MJT_CONV_NS"))
+            if (atoi(e) >= 3 && atoi(e) <= NSLAB) NSLAB = atoi(e);
+        MJT_CHECK(NSLAB >= 3, "conv: internal: no room for the weight ring");
         const bool tail_first = getenv("MJT_CONV_TAIL_FIRST") && atoi(getenv("MJT_CONV_TAIL_FIRST")) && TAIL_TRW > 0 && (RPW - NFULL * TR) % WPX == 0;
         const int64_t slot_stride = getenv("MJT_CONV_SLOT_STRIDE") ? atoi(getenv("MJT_CONV_SLOT_STRIDE")) : cus / 8 > 0 ? cus / 8 : 1;
-        key << "mfma|" << half << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT << "|" << WPS << "|" << tail_first << "|" << slot_stride << "|" << (getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0) << "|" << (getenv("MJT_CONV_SD") ? atoi(getenv("MJT_CONV_SD")) : 4);
+        key << "mfma|" << half << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT << "|" << WPS << "|" << tail_first << "|" << slot_stride << "|" << (getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0) << "|" << (getenv("MJT_CONV_SD") ? atoi(getenv("MJT_CONV_SD")) : 4) << "|" << (getenv("MJT_CONV_NT") ? atoi(getenv("MJT_CONV_NT")) : 0) << "|" << CBLK << "|" << NSLAB << "|" << (getenv("MJT_CONV_ROLES") ? atoi(getenv("MJT_CONV_ROLES")) : 0);
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
@@ -189,7 +200,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                 << "#define MT " << MT << "\n#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
                 << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS  << "\n#define BQ_DIST " << BQ << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype != MJT_FLOAT32 ? 1 : 0) << "\n#define IN_F16 " << (half ? 1 : 0)
-                << "\n#define WPS " << WPS << "\n#define TAIL_FIRST " << (tail_first ? 1 : 0) << "\n#define STAGE_DEPTH " << (getenv("MJT_CONV_SD") ? atoi(getenv("MJT_CONV_SD")) : 4) << "\n#define SLOT_STRIDE " << slot_stride << "\n#define DBG " << (getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0) << "\n";
+                << "\n#define WPS " << WPS << "\n#define TAIL_FIRST " << (tail_first ? 1 : 0) << "\n#define ROLES " << (getenv("MJT_CONV_ROLES") ? atoi(getenv("MJT_CONV_ROLES")) : 0) << "\n#define CB " << CBLK << "\n#define NS " << NSLAB << "\n#define STORE_NT " << (getenv("MJT_CONV_NT") ? atoi(getenv("MJT_CONV_NT")) : 0) << "\n#define STAGE_DEPTH " << (getenv("MJT_CONV_SD") ? atoi(getenv("MJT_CONV_SD")) : 4) << "\n#define SLOT_STRIDE " << slot_stride << "\n#define DBG " << (getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0) << "\n";
             src << embedded_source("conv_mfma.h") << "\n";
             k = jit_get(src.str(), name.str());
             kp = new JitKernel();
