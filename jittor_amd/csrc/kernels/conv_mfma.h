@@ -8,33 +8,37 @@
 // contribute 0 (overflow value 0 times w).
 //
 // All geometry is baked in by the host: C_, H_, W_, K_, R_, S_, OH_, OW_, SH, SW,
-// PH, PW, DH, DW, WKO (groups of 64 output channels per workgroup), WPX (row
+// PH, PW, DH, DW, WKO (groups of 16*MT output channels per workgroup), WPX (row
 // groups per workgroup), TRW / NT / LROWS (output rows per wave, 16-pixel tiles per
 // wave and input rows in LDS of a full tile), RPW (output rows a workgroup owns),
 // NFULL full tiles followed, when TAIL_TRW > 0, by one shorter tile (TAIL_TRW,
-// TAIL_NT, TAIL_LROWS), LCOLS, ITEMS_PER_WAVE, Y_BF16 (16-bit output in the operand type), IN_F16.
+// TAIL_NT, TAIL_LROWS), LCOLS, CB (channels per block: 32 or 64), NS (slabs in the
+// weight ring), STAGE_DEPTH, WPS (waves per SIMD the register budget is for),
+// Y_BF16 (16-bit output in the operand type), IN_F16.
 //
 // Mapping.  v_mfma_f32_16x16x32_bf16 computes D[16 ko][16 px] += A[16 ko][32 c] *
-// B[32 c][16 px].  A workgroup of WPX*WKO waves owns 64*WKO output channels x RPW
+// B[32 c][16 px].  A workgroup of WPX*WKO waves owns 16*MT*WKO output channels x RPW
 // consecutive output rows of one image and walks them tile by tile (WPX*TRW rows
 // each), so that the number of workgroups can match the number of compute units
-// whatever the row count, and the stores of one tile and the loads of the next
-// overlap the MFMAs.  Within a tile wave (wko, wpx) owns 64 channels x TRW rows =
-// 4 x NT accumulator tiles.  Channels are consumed 64 at a time:
-//   * the input rows the tile touches are staged through LDS as 8 planes
-//     [8 c][row][col][8 c] (one per group of 8 channels, channels innermost) so
+// whatever the row count.  Within a tile wave (wko, wpx) owns 16*MT channels x TRW
+// rows = MT x NT accumulator tiles.  Channels are consumed CB at a time, a block
+// being CB/32 steps per tap; both operands of a step come from LDS:
+//   * the input rows the tile touches are staged through LDS as CB/8 planes
+//     [row][col][8 c] (one per group of 8 channels, channels innermost) so
 //     that a B fragment is one 16-byte LDS read per lane.  The NCHW ->
 //     channel-innermost transpose happens on the way: a lane loads 8 columns of
 //     one channel, the 8 lanes of a column group exchange among themselves until
 //     each owns one column for the 8 channels, and writes 16 bytes: a wave fills
 //     a linear 1 KB run of a plane.  The address of a fragment is linear in the
 //     tap and the k-step.  The tile is double buffered across channel blocks and
-//     across tiles: the loads of the next block are issued before the MFMAs of
-//     the current one and written to the other buffer after them (one barrier
-//     per channel block);
-//   * A fragments come straight from the re-packed weights
-//     Wp[tap][c/64][k-step][ko/16][lane][8 c] (1 KB per fragment in lane order, L2
-//     resident) and are loaded one step before the MFMAs that use them.
+//     across tiles: the rows of the next block are asked for during the first
+//     steps of a block and written to the other buffer a few steps later;
+//   * the weights are re-packed as Wp[tap][c/32][ko/16][lane][8 c] (1 KB per A
+//     fragment in lane order, L2 resident).  The fragments of one step for the
+//     workgroup's channels, a slab, are contiguous there; slabs are copied
+//     straight into a ring in LDS several steps ahead of their use (no registers
+//     on the way), and every wave reads its MT fragments from the ring.
+// One barrier per step hands over the slab that has landed and frees the oldest.
 // Padding columns are zeroed once; rows outside the image are written as zeros.
 
 // operands: bfloat16, or with IN_F16 float16 (same kernel: only the MFMA and the narrowing of a 16-bit result differ)
@@ -132,7 +136,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     const unsigned short* __restrict__ wp = (const unsigned short*)p.a[1];
     const int n_img = (int)(unsigned long long)p.a[3];
     __shared__ __attribute__((aligned(16))) unsigned short xs[2][TILE_ELEMS];
-    __shared__ __attribute__((aligned(16))) unsigned short as_ring[NS * KO_WG * 32 + 4096];   // ring of weight slabs and a spare piece, see below
+    __shared__ __attribute__((aligned(16))) unsigned short as_ring[NS * KO_WG * 32 + 512];   // ring of weight slabs and a spare KB, see below
 
     // range id: the channel groups of one row range are 8 workgroups apart, so
     // they land on the same XCD (workgroups go round-robin over 8 XCDs) and
@@ -172,24 +176,12 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     const unsigned sel_t = b0 ? 0x05040100u : 0x07060302u;
     const unsigned sel_a = b0 ? 0x03020504u : 0x05040100u;
     const unsigned sel_b = b0 ? 0x03020706u : 0x07060100u;
-    // Roles.  Vector memory operations of a wave complete in order, so a wave that waits for weights it asked
-    // for after a slow load (input rows from HBM) waits for that load too.  The two kinds of load are therefore
-    // issued by different waves: the first half of the waves ("loaders") bring the weights in, the second
-    // half ("stagers") the input rows; with a single wave it does both.
-#if ROLES
-    constexpr int A_WAVES = NWAVES >= 2 ? NWAVES / 2 : 1;
-    constexpr int X_WAVES = NWAVES >= 2 ? NWAVES / 2 : 1;
-    const bool loader = wave < A_WAVES;
-    const bool stager = wave >= NWAVES - X_WAVES;
-    const int stager_id = wave - (NWAVES - X_WAVES);
-#else
-    constexpr int A_WAVES = NWAVES, X_WAVES = NWAVES;
-    constexpr bool loader = true, stager = true;
-    const int stager_id = wave;
-#endif
+    // Every wave moves its share of the input rows of a block and of every weight slab.  Vector memory
+    // operations of a wave complete in order: the ring is deep enough that the wait for a slab, which also waits
+    // for every older load, never asks for an input row earlier than the row is needed itself.
     constexpr int ITEMS = LROWS * SEGS * (CB / 8);                       // of a full tile
-    constexpr int IPW = (ITEMS + X_WAVES - 1) / X_WAVES;          // items of one stager per channel block
-    // A stager asks for item k of its share at the start of step fetch_step(k) and writes it to LDS at the end
+    constexpr int IPW = (ITEMS + NWAVES - 1) / NWAVES;            // items of one wave per channel block
+    // A wave asks for item k of its share at the start of step fetch_step(k) and writes it to LDS at the end
     // of step fetch_step(k) + SD - 1: SD steps for the row to arrive from HBM, SG items per step, SQ registers.
     constexpr int STEPS = KSTEPS * R_ * S_;       // steps per channel block
     // When the steps of a block are too few for that (more than SGMAX items per step), the items of a step go in
@@ -228,11 +220,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         const int soff = __builtin_amdgcn_readfirstlane((((cb * CB + cg * 8) * H_ + ir) * W_) * 2);     // uniform: channel group and row inside the image
         int grp = seg * 8 + sg;
         grp = grp < GROUPS ? grp : GROUPS - 1;
-#if DBG & 4
-        return (mjt_u32x4v)((unsigned)soff);
-#else
         return __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)((live ? x_lane_off : 0x80000000u) + (unsigned)grp * 16), soff, 0);
-#endif
     };
     // Writing an item to LDS, in four stages that work in place on its four registers (the main loop spreads them
     // between its MFMAs): three exchanges, then the write.
@@ -256,12 +244,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         int grp = seg * 8 + sg;
         grp = grp < GROUPS ? grp : GROUPS - 1;
         const unsigned voff = (live ? x_lane_off : 0x80000000u) + (unsigned)grp * 16;
-#if DBG & 4
-        dst = (mjt_u32x4v)(voff);
-        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=v"(dst[0]) : "v"(0x80000000u), "s"(x_desc), "s"(soff) : "memory");
-#else
         asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(dst) : "v"(voff), "s"(x_desc), "s"(soff) : "memory");
-#endif
     };
     auto commit_stage = [&](auto sc, bool live, mjt_u32x4v& d, int r0, int lrows, int buf, int item, int limit) {
         constexpr int stg = decltype(sc)::v;
@@ -306,25 +289,24 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         mjt_static_for<0, 4>([&](auto sc) { commit_stage(sc, live, d, r0, lrows, buf, item, limit); });
     };
 
-    // A fragments: Wp[step][ko / 16][lane][8 c], step = (tap * NCB + cb) * 2 + ks: a fragment is 1 KB in lane order
+    // A fragments: Wp[step][ko / 16][lane][8 c], step = (tap * NCB + cb) * KSTEPS + ks: a fragment is 1 KB in lane order
     // (lane = lg * 16 + l16 holds channels lg*8.. of row l16).  The fragments of one step for the workgroup's
-    // output channels (a slab: KO_WG / 16 KB, contiguous in Wp) go through a ring of NS slabs in LDS: the
-    // loaders copy slab g + 3 straight from memory into LDS (no registers) while step g runs; every wave
-    // reads its own MT fragments of slab g + 1 into registers during step g.  One barrier per step hands a
-    // landed slab over and frees the oldest one.
+    // output channels (a slab: KO_WG / 16 KB, contiguous in Wp) go through a ring of NS slabs in LDS: while step g
+    // runs the waves copy slab g + NS - 1 straight from memory into LDS (no registers); every wave reads its own
+    // MT fragments from the ring two passes ahead of the MFMAs.  One barrier per step hands a landed slab over and
+    // frees the oldest one.
     constexpr int SLAB = KO_WG * 64;              // bytes
-    constexpr int FPL = (KO_WG / 16) / A_WAVES;   // fragments a loader moves per slab
+    constexpr int FPL = (KO_WG / 16) / NWAVES;    // fragments a wave moves per slab
     const unsigned as_base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned short*)&as_ring[0];
     const unsigned a_rd_base = as_base + (unsigned)(wko * MT * 1024 + lane * 16);
     const __amdgpu_buffer_rsrc_t w_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(wp + (size_t)kpart * KO_WG * 32), 0, (R_ * S_ * C_ * K_ - kpart * KO_WG * 32) * 2, 0x00020000);
     auto slab_load = [&](int cb, int st, int slot) {          // all arguments uniform
         const int tap = st / KSTEPS, ks = st % KSTEPS;
-        const int soff = ((tap * NCB + cb) * KSTEPS + ks) * (K_ * 64) + (loader ? wave * (FPL * 1024) : 0);
-        // the other waves issue the same instructions, out of range (zeros, no traffic) into a spare piece of LDS
+        const int soff = ((tap * NCB + cb) * KSTEPS + ks) * (K_ * 64) + wave * (FPL * 1024);
         __attribute__((address_space(3))) unsigned short* dst =
-            (__attribute__((address_space(3))) unsigned short*)&as_ring[0] + (loader ? slot * SLAB + wave * (FPL * 1024) : NS * SLAB) / 2;
-        const unsigned voff = (loader ? 0u : 0x80000000u) + (unsigned)lane * 16;
+            (__attribute__((address_space(3))) unsigned short*)&as_ring[0] + (slot * SLAB + wave * (FPL * 1024)) / 2;
+        const unsigned voff = (unsigned)lane * 16;
         mjt_static_for<0, FPL>([&](auto fc) {
             constexpr int f = decltype(fc)::v;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (__attribute__((address_space(3))) void*)(dst + (f >> 2) * 2048), 16, (int)voff,
@@ -344,28 +326,10 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // still be under way: the loads of the last NS - 3 steps, slabs and input rows alike (all of them are spelled out
     // in the loop, so their number is known).
     auto step_sync = [&](auto nc) {                  // nc: loads issued in the last NS - 3 steps, this one included
-#if !(DBG & 32)
-        if (loader) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(decltype(nc)::v < 63 ? decltype(nc)::v : 63) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(decltype(nc)::v < 63 ? decltype(nc)::v : 63) : "memory");
         asm volatile("s_barrier" : : : "memory");
-#endif
     };
 
-#if DBG & 8
-    unsigned long long* ts_out = (unsigned long long*)((float*)p.a[2] + (size_t)n_img * K_ * OH_ * OW_) + ((size_t)blockIdx.x * NWAVES + wave) * 64;
-    const __amdgpu_buffer_rsrc_t ts_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)ts_out, 0, 512, 0x00020000);
-    int ts_n = 2;
-    {
-        mjt_u32x2 hw;
-        hw[0] = __builtin_amdgcn_s_getreg(63492); hw[1] = 0;
-        __builtin_amdgcn_raw_buffer_store_b64(hw, ts_rsrc, lane == 0 ? 0 : 0x80000000, 0, 0);
-        hw[0] = __builtin_amdgcn_s_getreg((31 << 11) | 20);
-        __builtin_amdgcn_raw_buffer_store_b64(hw, ts_rsrc, lane == 0 ? 8 : 0x80000000, 0, 0);
-    }
-#define STAMP() do { unsigned long long t_ = __builtin_amdgcn_s_memrealtime(); mjt_u32x2 v_; v_[0] = (unsigned)t_; v_[1] = (unsigned)(t_ >> 32); \
-        __builtin_amdgcn_raw_buffer_store_b64(v_, ts_rsrc, lane == 0 ? ts_n * 8 : 0x80000000, 0, 0); ts_n++; } while (0)
-#else
-#define STAMP() do {} while (0)
-#endif
     int buf = 0;                                  // LDS buffer that holds the current channel block
     int g = 0;                                    // steps done so far, modulo NS: slab of the current step is in slot g
 
@@ -426,13 +390,12 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         mjt_u32x4v bfr[NT_];
         mjt_u32x4v afr[3];                                   // A fragments of this pass and the next two
         constexpr int PASSES = STEPS * MT;
-        STAMP();
 #pragma unroll 1
         for (int cb = 0; cb < NCB; cb++) {
             const bool more = cb + 1 < NCB;
             const bool feed = more || next_lrows;                // somebody needs another block of input rows
             const int f_r0 = more ? r0 : next_r0, f_lrows = more ? LR_ : next_lrows, f_cb = more ? cb + 1 : 0;
-            const int my_first = stager_id * IPW, my_limit = (stager_id + 1) * IPW < ITEMS ? (stager_id + 1) * IPW : ITEMS;
+            const int my_first = wave * IPW, my_limit = (wave + 1) * IPW < ITEMS ? (wave + 1) * IPW : ITEMS;
             // nothing is under way here
             mjt_ds_read<0>(afr[0], a_rd_base + (unsigned)((g % NS) * SLAB));
             mjt_ds_read<1024>(afr[1], a_rd_base + (unsigned)((g % NS) * SLAB));
@@ -445,27 +408,25 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                     if constexpr (!BULK) {
                         mjt_static_for<0, IPW>([&](auto kc) {
                             constexpr int k = decltype(kc)::v;
-                            if constexpr (k / SG == st) fetch_item_fixed(stage[k % SQ], stager && feed, f_r0, f_lrows, f_cb, my_first + k);
+                            if constexpr (k / SG == st) fetch_item_fixed(stage[k % SQ], feed, f_r0, f_lrows, f_cb, my_first + k);
                         });
                     } else {
                         mjt_static_for<0, RPS>([&](auto rc) {
                             constexpr int r = decltype(rc)::v;
                             mjt_static_for<0, RS>([&](auto ic) {
                                 constexpr int k = bulk_item(st, r, decltype(ic)::v);
-                                if constexpr (k >= 0) stage[decltype(ic)::v] = fetch_item(stager && feed, f_r0, f_lrows, f_cb, my_first + k);
+                                if constexpr (k >= 0) stage[decltype(ic)::v] = fetch_item(feed, f_r0, f_lrows, f_cb, my_first + k);
                             });
                             if constexpr (r + 1 < RPS)
                                 mjt_static_for<0, RS>([&](auto ic) {
                                     constexpr int k = bulk_item(st, r, decltype(ic)::v);
-                                    if constexpr (k >= 0) commit_item(stager && feed, stage[decltype(ic)::v], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);
+                                    if constexpr (k >= 0) commit_item(feed, stage[decltype(ic)::v], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);
                                 });
                         });
                     }
-#if !(DBG & 16)
                     int cb3, st3;
                     slab_ahead(cb, st, NS - 1, cb3, st3);
                     slab_load(cb3, st3, (g + st + NS - 1) % NS);
-#endif
                 };
                 constexpr auto stage_at = [](int sg) { return NT_ + (sg * (MT - 2) * NT_) / 4; };
                 auto commit_stages = [&](auto ic) {          // ic: MFMAs of this step issued so far
@@ -482,13 +443,13 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                                             constexpr int after = (loads_in(k / SG) - 1 - k % SG) + FPL + (SD - 1) * FPL + loads_between(k / SG + 1, k / SG + SD);
                                             asm volatile("s_waitcnt vmcnt(%1)" : "+v"(stage[k % SQ]) : "n"(after < 63 ? after : 63));
                                         }
-                                        commit_stage(sc, stager && feed, stage[k % SQ], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);   // the other buffer: nobody reads it now
+                                        commit_stage(sc, feed, stage[k % SQ], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);   // the other buffer: nobody reads it now
                                     }
                                 });
                             } else {
                                 mjt_static_for<0, RS>([&](auto jc) {
                                     constexpr int k = bulk_item(st, RPS - 1, decltype(jc)::v);
-                                    if constexpr (k >= 0) commit_stage(sc, stager && feed, stage[decltype(jc)::v], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);
+                                    if constexpr (k >= 0) commit_stage(sc, feed, stage[decltype(jc)::v], f_r0, f_lrows, buf ^ 1, my_first + k, my_limit);
                                 });
                             }
                         }
@@ -496,18 +457,13 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                 };
                 const unsigned a_cur = a_rd_base + (unsigned)(((g + st) % NS) * SLAB);
                 const unsigned a_nxt = a_rd_base + (unsigned)(((g + st + 1) % NS) * SLAB);
-#if DBG & 256
-                if constexpr (st >= 4 && st < 10) STAMP();
-#endif
                 mjt_static_for<0, MT>([&](auto mc) {
                     constexpr int m = decltype(mc)::v;
                     constexpr int P = st * MT + m;                           // pass number in the block; its fragment sits in afr[P % 3]
-#if !(DBG & 128)
                     if constexpr (P + 2 < PASSES) {                          // the fragment two passes ahead: of this step or the next
                         if constexpr (m + 2 < MT) mjt_ds_read<(m + 2) * 1024>(afr[(P + 2) % 3], a_cur);
                         else mjt_ds_read<(m + 2 - MT) * 1024>(afr[(P + 2) % 3], a_nxt);
                     }
-#endif
                     mjt_static_for<0, NT_>([&](auto tc) {
                         constexpr int t = decltype(tc)::v;
                         // the rows written in this step are written before its last pass: no LDS write follows the B reads
@@ -517,15 +473,10 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                         if constexpr (m == 0) mjt_lds_wait<(BULK ? 0 : NT_ - 1 - t + (P + 2 < PASSES ? 1 : 0))>(bfr[t]);
                         else if constexpr (t == 0) mjt_lds_wait<(P + 1 < PASSES ? 1 : 0) + (P + 2 < PASSES ? 1 : 0)>(afr[P % 3]);
                         mjt_mfma(acc[m][t], afr[P % 3], bfr[t]);
-#if !(DBG & 64)
                         if constexpr (m + 1 == MT && st + 1 < STEPS) mjt_ds_read<mjt_frag_off(st + 1)>(bfr[t], baddr[t]);
-#endif
                         if constexpr (m == 0 && t == 0) issue_loads();
                         commit_stages(mjt_ic<m * NT_ + t + 1>());
                     });
-#if DBG & 256
-                    if constexpr (st >= 4 && st < 10) STAMP();
-#endif
                 });
                 if (st + 1 == STEPS) asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");   // the rows written for the next block
                 step_sync(mjt_ic<(BULK ? 0 : (NS - 3) * FPL + loads_between(st - (NS - 4), st + 1))>());
@@ -548,7 +499,6 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         mjt_keep(afr[2]);
         mjt_static_for<0, NT_>([&](auto tc) { mjt_keep(bfr[decltype(tc)::v]); });
         mjt_static_for<0, MT * NT_>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / NT_][decltype(ic)::v % NT_]); });
-        STAMP();
 #if OW_ % 4 == 0
         // The four lanes of a quad (4 pixels x 4 channels) transpose among themselves, after which lane j
         // of the quad owns channel 4*(lane/16)+j for the quad's 4 consecutive pixels: one 16-byte (or
@@ -575,29 +525,16 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                 y4[1] = b1 ? h1 : a1;
                 y4[2] = b1 ? a2 : h0;
                 y4[3] = b1 ? a3 : h1;
-#if (DBG & 3) == 2
-                if (y4[0] == 123.456f) ((float*)p.a[2])[0] = y4[1] + y4[2] + y4[3];
-                if (false) {
-#else
                 if (ok) {
-#endif
                     const int ko = ko_base + m * 16 + lg * 4 + qj;
-#if (DBG & 3) == 1
-                    const size_t o = ((size_t)blockIdx.x * NWAVES + wave) * (MT * NT * 256) + (size_t)((t * MT + m) * 256 + lane * 4);
-#else
                     const size_t o = (((size_t)n * K_ + ko) * OH_ + orow) * OW_ + col;
-#endif
 #if Y_BF16
                     mjt_u32x2 pk;
                     pk[0] = mjt_narrow2(y4[0], y4[1]);
                     pk[1] = mjt_narrow2(y4[2], y4[3]);
                     *(mjt_u32x2*)((unsigned short*)p.a[2] + o) = pk;
 #else
-#if STORE_NT
-                    __builtin_nontemporal_store(y4, (mjt_f32x4*)((float*)p.a[2] + o));
-#else
                     *(mjt_f32x4*)((float*)p.a[2] + o) = y4;
-#endif
 #endif
                 }
             }
@@ -625,29 +562,14 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         }
 #endif
     };
-
-    STAMP();
-    // tiles of this workgroup: full tiles while they start inside the row range, then the short one.  With
-    // TAIL_FIRST every other workgroup of a compute unit walks the short tile first instead: the two then reach
-    // the ends of their tiles, where a workgroup only stores, at different times, and the MFMAs of one cover
-    // the stores of the other.
+    // tiles of this workgroup: full tiles while they start inside the row range, then the short one
     int nfull = (row_end - row_begin + TR - 1) / TR;
     if (nfull > NFULL) nfull = NFULL;
     const bool tail = TAIL_TRW > 0 && row_begin + NFULL * TR < row_end;
-#if TAIL_FIRST && TAIL_TRW > 0
-    constexpr int REM = RPW - NFULL * TR;          // rows of the short tile
-    const bool tail_first = tail && row_begin + RPW <= OH_ && ((j / SLOT_STRIDE) & 1);
-#else
-    constexpr int REM = 0;
-    const bool tail_first = false;
-#endif
-    const int first_lrows = tail_first ? TAIL_LROWS : nfull ? LROWS : TAIL_LROWS;
+    const int first_lrows = nfull ? LROWS : TAIL_LROWS;
     const int ntiles = nfull + (tail ? 1 : 0);
-    const int tail_at = tail ? (tail_first ? 0 : nfull) : -1;
-    const int full_base = row_begin + (tail_first ? REM : 0);
 
-    // the slabs of the first three steps, the first block of input rows (every wave takes a share here), the
-    // fragments of the first step
+    // the slabs of the first NS - 1 steps and the first block of input rows (every wave takes a share)
     mjt_static_for<0, NS - 1>([&](auto kc) {
         int cb0, st0;
         slab_ahead(0, 0, decltype(kc)::v, cb0, st0);
@@ -670,23 +592,20 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     __syncthreads();
 #pragma unroll 1
     for (int i = 0; i < ntiles; i++) {
-        const int next_lrows = i + 1 >= ntiles ? 0 : i + 1 == tail_at ? TAIL_LROWS : LROWS;
-        const int s = tail_first ? i - 1 : i;    // index among the full tiles
+        const int next_lrows = i + 1 >= ntiles ? 0 : i + 1 == nfull ? TAIL_LROWS : LROWS;
+        const int r0 = row_begin + i * TR;
 #if TAIL_TRW > 0
-        if (i == tail_at) {
-            const int r0 = tail_first ? row_begin : row_begin + NFULL * TR;
-            run_tile(mjt_ic<TAIL_TRW>(), mjt_ic<TAIL_NT>(), mjt_ic<TAIL_LROWS>(), r0, tail_first ? row_begin + REM : row_end, full_base, next_lrows);
+        if (i == nfull) {
+            run_tile(mjt_ic<TAIL_TRW>(), mjt_ic<TAIL_NT>(), mjt_ic<TAIL_LROWS>(), r0, row_end, 0, 0);
             continue;
         }
 #endif
-        const int r0 = full_base + s * TR;
-        run_tile(mjt_ic<TRW>(), mjt_ic<NT>(), mjt_ic<LROWS>(), r0, row_end, i + 1 == tail_at ? row_begin + NFULL * TR : r0 + TR, next_lrows);
+        run_tile(mjt_ic<TRW>(), mjt_ic<NT>(), mjt_ic<LROWS>(), r0, row_end, r0 + TR, next_lrows);
     }
-    STAMP();
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");   // slabs asked for past the last step
 }
 
-// Weight re-pack: w[ko][c][kh][kw] -> Wp[tap][c/64][k-step][ko/16][lg][l16][8 c] (c = 32 k-step + 8 lg + ..)
+// Weight re-pack: w[ko][c][kh][kw] -> Wp[tap][c/CB][k-step][ko/16][lg][l16][8 c] (c = CB block + 32 k-step + 8 lg + ..)
 extern "C" __global__ __launch_bounds__(256) void ENTRY_PACK(Params p) {
     const unsigned short* __restrict__ w = (const unsigned short*)p.a[0];
     unsigned short* __restrict__ wp = (unsigned short*)p.a[1];

@@ -102,18 +102,17 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     // ---- MFMA path ----------------------------------------------------------------
     const char* wpx_env = getenv("MJT_CONV_WPX");
     const int64_t WPX = wpx_env && atoi(wpx_env) == 1 ? 1 : 2;
-    const char* pxw_env = getenv("MJT_CONV_PXW");
-    const int64_t max_px = pxw_env && (atoi(pxw_env) == 112 || atoi(pxw_env) == 224) ? atoi(pxw_env) : WPX == 1 ? 224 : 112;   // pixels per wave: 16 per accumulator tile
+    const int64_t max_px = WPX == 1 ? 224 : 112;            // pixels per wave: 16 per accumulator tile
     const int64_t WPS = max_px == 224 ? 1 : 2;              // waves per SIMD the register budget is set for
     // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
     const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
     int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
     // LDS: two buffers of input rows (one block of CB channels each), a ring of NS weight slabs (64 bytes per output
-    // channel of the workgroup each) and a spare piece the size of a loader's share of a slab.  Blocks of 32 channels
+    // channel of the workgroup each) and a spare KB that takes the writes of idle lanes.  Blocks of 32 channels
     // leave room for a deeper ring, which is what hides the latency of the slabs; the ring needs three slabs at least.
     const int64_t lds_total = 160 * 1024;
     const int64_t CBLK = getenv("MJT_CONV_CB") && atoi(getenv("MJT_CONV_CB")) == 64 ? 64 : 32;
-    const int64_t slab0 = 64 * 16 * MT * WKO, spare0 = 8 * 1024;
+    const int64_t slab0 = 64 * 16 * MT * WKO, spare0 = 1024;
     const int64_t tile_limit = (lds_total - 4 * slab0 - spare0) / 2;         // leaves room for four slabs of the widest workgroup
     int64_t TRW = OW <= max_px ? max_px / OW : 0;
     if (TRW > OH) TRW = OH;
@@ -136,7 +135,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             if (atoi(e) >= 1 && atoi(e) <= WKO * 4 && K % (16 * MT * atoi(e)) == 0 && (atoi(e) & (atoi(e) - 1)) == 0 && atoi(e) <= 256 / (16 * MT)) WKO = atoi(e);
     }
     const bool half = x->dtype == MJT_FLOAT16;
-    const bool mfma_ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % 64 == 0 && K % 64 == 0 &&
+    const bool mfma_ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % CBLK == 0 && K % 64 == 0 &&
                          W % 2 == 0 && TRW >= 1 && NT <= max_px / 16 && LROWS * LCOLS * CBLK * 2 <= tile_limit &&
                          // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
                          ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + (CBLK == 64 ? 4 * LROWS * LCOLS * 16 : 0) < 65536 &&
@@ -144,8 +143,6 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                          // byte offsets inside one image and inside the weights are 32-bit in the kernel
                          C * H * W * 2 < (int64_t(1) << 31) && K * OH * OW * 4 < (int64_t(1) << 31) && numel(w) * 2 < (int64_t(1) << 31);
     if (mfma_ok) {
-        const int64_t items = LROWS * (((W + 7) / 8 + 7) / 8) * 8;     // (row, 64 columns, 8 channels); a wave moves one item per load
-        const int64_t items_per_wave = (items + WPX * WKO - 1) / (WPX * WKO);
         // Rows per workgroup: a workgroup walks RPW output rows as NFULL tiles of TR rows plus one
         // shorter tile.  Pick the RPW that minimises (rounds of workgroups over the compute units) x
         // (accumulator tiles a workgroup computes, plus a per-tile overhead worth half a tile column).
@@ -175,19 +172,17 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         tail_of(RPW, &TAIL_TRW, &TAIL_NT);
         const int64_t NFULL = RPW / TR;
         const int64_t TAIL_LROWS = TAIL_TRW ? lds_rows(TAIL_TRW) : 0;
-        const char* bq_env = getenv("MJT_CONV_BQ");
-        const int BQ = bq_env && *bq_env ? atoi(bq_env) : 3;   // B fragments requested ahead of use
         std::ostringstream key;
         const int64_t slab = 64 * 16 * MT * WKO;
-        const int64_t spare = 8 * 1024;
+        const int64_t spare = 1024;
         int64_t NSLAB = (lds_total - 2 * LROWS * LCOLS * CBLK * 2 - spare) / slab;
         if (NSLAB > 8) NSLAB = 8;
         if (const char* e = getenv("MJT_CONV_NS"))
             if (atoi(e) >= 3 && atoi(e) <= NSLAB) NSLAB = atoi(e);
         MJT_CHECK(NSLAB >= 3, "conv: internal: no room for the weight ring");
-        const bool tail_first = getenv("MJT_CONV_TAIL_FIRST") && atoi(getenv("MJT_CONV_TAIL_FIRST")) && TAIL_TRW > 0 && (RPW - NFULL * TR) % WPX == 0;
-        const int64_t slot_stride = getenv("MJT_CONV_SLOT_STRIDE") ? atoi(getenv("MJT_CONV_SLOT_STRIDE")) : cus / 8 > 0 ? cus / 8 : 1;
-        key << "mfma|" << half << "|" << BQ << "|" << geo.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT << "|" << WPS << "|" << tail_first << "|" << slot_stride << "|" << (getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0) << "|" << (getenv("MJT_CONV_SD") ? atoi(getenv("MJT_CONV_SD")) : 4) << "|" << (getenv("MJT_CONV_NT") ? atoi(getenv("MJT_CONV_NT")) : 0) << "|" << CBLK << "|" << NSLAB << "|" << (getenv("MJT_CONV_ROLES") ? atoi(getenv("MJT_CONV_ROLES")) : 0);
+        const int stage_depth = getenv("MJT_CONV_SD") && atoi(getenv("MJT_CONV_SD")) >= 2 && atoi(getenv("MJT_CONV_SD")) <= 8 ? atoi(getenv("MJT_CONV_SD")) : 4;
+        key << "mfma|" << half << "|" << geo.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT << "|" << WPS
+            << "|" << stage_depth << "|" << CBLK << "|" << NSLAB;
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
@@ -199,8 +194,8 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo.str()
                 << "#define MT " << MT << "\n#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
-                << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS  << "\n#define BQ_DIST " << BQ << "\n#define ITEMS_PER_WAVE " << items_per_wave << "\n#define Y_BF16 " << (y->dtype != MJT_FLOAT32 ? 1 : 0) << "\n#define IN_F16 " << (half ? 1 : 0)
-                << "\n#define WPS " << WPS << "\n#define TAIL_FIRST " << (tail_first ? 1 : 0) << "\n#define ROLES " << (getenv("MJT_CONV_ROLES") ? atoi(getenv("MJT_CONV_ROLES")) : 0) << "\n#define CB " << CBLK << "\n#define NS " << NSLAB << "\n#define STORE_NT " << (getenv("MJT_CONV_NT") ? atoi(getenv("MJT_CONV_NT")) : 0) << "\n#define STAGE_DEPTH " << (getenv("MJT_CONV_SD") ? atoi(getenv("MJT_CONV_SD")) : 4) << "\n#define SLOT_STRIDE " << slot_stride << "\n#define DBG " << (getenv("MJT_CONV_DBG") ? atoi(getenv("MJT_CONV_DBG")) : 0) << "\n";
+                << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS << "\n#define Y_BF16 " << (y->dtype != MJT_FLOAT32 ? 1 : 0) << "\n#define IN_F16 " << (half ? 1 : 0)
+                << "\n#define WPS " << WPS << "\n#define CB " << CBLK << "\n#define NS " << NSLAB << "\n#define STAGE_DEPTH " << stage_depth << "\n";
             src << embedded_source("conv_mfma.h") << "\n";
             k = jit_get(src.str(), name.str());
             kp = new JitKernel();

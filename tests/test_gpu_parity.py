@@ -499,6 +499,8 @@ def _conv_call(xbits, wbits, params, out_dtype="float32", in_dtype="bfloat16"):
     dict(x=(1, 64, 11, 70), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),        # 70 columns: a second staging segment of 6
     dict(x=(3, 64, 6, 6), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),          # rows shorter than one group of 8 columns
     dict(x=(2, 64, 5, 2), w=(64, 64, 1, 1), p=(1, 1, 0, 0, 1, 1)),          # two columns: a load spans four rows
+    dict(x=(2, 96, 12, 16), w=(64, 96, 3, 3), p=(1, 1, 1, 1, 1, 1)),        # 96 channels: three blocks of 32
+    dict(x=(1, 64, 30, 112), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),       # wide rows: one output row per wave, a short weight ring
 ])
 def test_conv_mfma_matches_oracle(gpu, case):
     from oracle import kernels as K
