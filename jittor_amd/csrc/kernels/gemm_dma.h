@@ -1,0 +1,214 @@
+// Matrix product on MFMA, both operands with k innermost in memory:  C[b][M][N] = sum_k A[b][M][K] * B[b][N][K]
+// (reference: the broadcast * broadcast -> reduce.add pattern that
+// python/jittor/src/opt/tuner/matmul_tuner.cc:16-104 relays to a library GEMM,
+// python/jittor/extern/cuda/cublas/ops/cublas_matmul_op.cc:27-126; this is the a x b^T case, the
+// forward product of a linear layer, python/jittor/nn.py:628-643).  bfloat16 / float16 operands with exact
+// products and float32 accumulation.
+//
+// Supplied by the host: IN (0 bfloat16, 1 float16), OUT (0 bfloat16 by truncation, 1 float16 rounded to
+// nearest even, 2 float32).  K is a multiple of 64, leading dimensions are multiples of 16 bytes and the
+// operand pointers 16-byte aligned (the host sends everything else to the general kernel).
+//
+// Mapping.  A workgroup of four waves (2 x 2, one wave per SIMD) owns a 256 x 256 tile of C; a wave owns
+// 128 x 128 of it as 4 x 4 accumulator tiles of v_mfma_f32_32x32x16, 256 accumulation registers.  K is walked in
+// stages of 64 (whole 128-byte lines of both operands): the 256 x 64 pieces of both operands (64 KB) alternate
+// between two buffers in LDS.  Nothing on that way passes through registers: a wave copies 8 rows x 128 bytes per
+// instruction straight from memory into LDS (lane i lands at byte 16 i of the 1 KB the instruction fills), a
+// stage ahead of their use.  A row of a stage is eight 16-byte chunks; chunk c of row r sits at position
+// c ^ (r / 2 % 8), which the copying lane arranges by choosing what it fetches.  The 16 lanes that read a
+// fragment together (16 neighbouring rows, one chunk) then touch 16 different bank groups.  Lane (row = lane % 32,
+// half = lane / 32) reads the 8 consecutive k of its row and half with one 16-byte LDS read; the fragments of
+// the next k-step are read while the 16 MFMAs of a k-step run.  One barrier per stage, before its last k-step,
+// hands over the next stage, which has landed by then, and frees the buffer of the current one, whose last
+// fragments are in registers.  Rows beyond M and N are read from the last valid row (their results are not stored).
+//
+// The MFMAs are spelled out, like the LDS reads and the waits, so that the order below is the schedule; the
+// accumulators live in the accumulation registers, which nothing but these MFMAs touches inside the loop (the
+// compiler takes a spelled-out MFMA for finished the moment it is issued).
+
+typedef float mjt_f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
+#if IN == 0
+#define MJT_MFMA_ASM "v_mfma_f32_32x32x16_bf16"
+#else
+#define MJT_MFMA_ASM "v_mfma_f32_32x32x16_f16"
+#endif
+#define TM 256
+#define TN 256
+#define KS 64
+#define STAGE_BYTES ((TM + TN) * 128)
+#define NTHR 256
+
+template <int V> struct mjt_ic { static constexpr int v = V; };
+template <int I, int N, class F> __device__ __forceinline__ void mjt_static_for(F&& f) {
+    if constexpr (I < N) {
+        f(mjt_ic<I>());
+        mjt_static_for<I + 1, N>(f);
+    }
+}
+template <int OFF> __device__ __forceinline__ void mjt_ds_read(mjt_u32x4v& dst, unsigned addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+__device__ __forceinline__ void mjt_mfma(mjt_f32x16& c, const mjt_u32x4v& a, const mjt_u32x4v& b) {
+    asm volatile(MJT_MFMA_ASM " %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mjt_keep(const mjt_u32x4v& x) { asm volatile("" : : "v"(x)); }     // x is in its registers up to here
+__device__ __forceinline__ void mjt_pin(mjt_f32x16& x) { asm volatile("" : "+a"(x)); }            // what reads x later comes after this point
+
+struct Params { void* a[12]; };
+
+extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu(1, 1))) void ENTRY(Params p) {
+    const int M = (int)(long long)p.a[3], N = (int)(long long)p.a[4], K = (int)(long long)p.a[5];
+    const long long lda = (long long)p.a[6], ldb = (long long)p.a[7], ldc = (long long)p.a[8];
+    const unsigned short* __restrict__ A = (const unsigned short*)p.a[0] + (long long)blockIdx.y * (long long)p.a[9];
+    const unsigned short* __restrict__ B = (const unsigned short*)p.a[1] + (long long)blockIdx.y * (long long)p.a[10];
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE_BYTES];
+
+    // Tile order: panels of 4 tile rows, inside a panel column by column.  Workgroups go round-robin over the
+    // 8 XCDs, so workgroup id takes tile (id % 8) * per_xcd + id / 8: every XCD works on a compact run of
+    // tiles and finds the operand rows and columns it shares in its own L2.
+    const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
+    const int tiles = tiles_m * tiles_n;
+    int L;
+    {
+        const int per_xcd = (tiles + 7) / 8;
+        L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if (L >= tiles || (int)(blockIdx.x >> 3) >= per_xcd) return;
+    }
+    int tm, tn;
+    {
+        const int panel = L / (4 * tiles_n);
+        const int rows_here = tiles_m - panel * 4 < 4 ? tiles_m - panel * 4 : 4;
+        const int within = L - panel * 4 * tiles_n;
+        tn = within / rows_here;
+        tm = panel * 4 + within - tn * rows_here;
+    }
+    const int m0 = tm * TM, n0 = tn * TN;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int nstages = K / KS;
+
+    // Copies.  A stage is 64 instructions of 1 KB (32 of A, 32 of B); wave w issues number 8w .. 8w+7 of each.
+    // Lane i of instruction j fills row 8 j + i / 8, position i % 8, with chunk (i % 8) ^ (row / 2 % 8).
+    // Descriptors start at the tile's first row; the lane offset is its row (clamped to the matrix) times the
+    // leading dimension plus its chunk, the stage adds 128 bytes per step through the scalar offset.
+    const int last_a = M - 1 - m0, last_b = N - 1 - n0;             // last valid row of the tile
+    unsigned voff_a[8], voff_b[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const int row = (wave * 8 + q) * 8 + (lane >> 3);
+        const unsigned chunk = (unsigned)((lane & 7) ^ ((row >> 1) & 7));
+        voff_a[q] = (unsigned)(row < last_a ? row : last_a) * (unsigned)(lda * 2) + chunk * 16;
+        voff_b[q] = (unsigned)(row < last_b ? row : last_b) * (unsigned)(ldb * 2) + chunk * 16;
+    }
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(A + (long long)m0 * lda), 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(B + (long long)n0 * ldb), 0, 0x7fffffff, 0x00020000);
+    // instruction q (0 .. 15: eight of A, eight of B) of this wave's share of stage s; s and slot uniform
+    auto copy_one = [&](auto qc, int s, int slot) {
+        constexpr int q = decltype(qc)::v;
+        const int st = s < nstages ? s : nstages - 1;               // past the end: a stage nobody reads
+        const int soff = st * (KS * 2);
+        __attribute__((address_space(3))) unsigned char* dst =
+            (__attribute__((address_space(3))) unsigned char*)&lds[0] + slot * STAGE_BYTES + wave * 8192;
+        // (an immediate offset would move the place in memory along with the place in LDS)
+        if constexpr (q < 8)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void*)(dst + q * 1024), 16, (int)voff_a[q], soff, 0, 0);
+        else
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void*)(dst + TM * 128 + (q - 8) * 1024), 16, (int)voff_b[q - 8], soff, 0, 0);
+    };
+    auto copy_stage = [&](int s, int slot) { mjt_static_for<0, 16>([&](auto qc) { copy_one(qc, s, slot); }); };
+
+    // Fragment addresses of this lane: row lane % 32 of each 32-row block of its wave's rows, chunk 2 * k-step +
+    // lane / 32 at position chunk ^ (row / 2 % 8): the position of k-step 0 with the k-step's bits flipped.
+    const int frow = lane & 31;
+    const unsigned pos0 = (unsigned)((lane >> 5) ^ ((frow >> 1) & 7));
+    const unsigned lds_base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned char*)&lds[0];
+    const unsigned a_lane = lds_base + (unsigned)((wm * 128 + frow) * 128);
+    const unsigned b_lane = lds_base + (unsigned)(TM * 128 + (wn * 128 + frow) * 128);
+    mjt_u32x4v fa[2][4], fb[2][4];
+    // fragment f (0 .. 7: four of A, four of B) of k-step kstep of the stage in slot, into set SET
+    auto request_one = [&](auto setc, auto fc, int slot, int kstep) {
+        constexpr int SET = decltype(setc)::v, f = decltype(fc)::v;
+        const unsigned off = (unsigned)(slot * STAGE_BYTES) + ((pos0 ^ (unsigned)(kstep * 2)) * 16);
+        if constexpr (f < 4) mjt_ds_read<f * 4096>(fa[SET][f], a_lane + off);
+        else mjt_ds_read<(f - 4) * 4096>(fb[SET][f - 4], b_lane + off);
+    };
+
+    mjt_f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+    // the zeros are written here, not next to the first MFMA that reads them
+    mjt_static_for<0, 16>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / 4][decltype(ic)::v % 4]); });
+    asm volatile("s_nop 7" : : : "memory");
+
+    // A k-step: 16 MFMAs on the fragments of set SET.  What else the wave has to issue goes between them, one
+    // instruction after each MFMA, where it costs no MFMA time (the wave is alone on its SIMD): the reads of the next
+    // k-step's fragments into the other set and, in the last k-step of a stage, the copies of the stage after the next.
+    auto kstep = [&](auto setc, int rd_slot, int rd_kstep, auto copyc, int cp_stage, int cp_slot) {
+        constexpr int SET = decltype(setc)::v;
+        constexpr bool COPY = decltype(copyc)::v != 0;
+        mjt_static_for<0, 16>([&](auto ic) {
+            constexpr int i = decltype(ic)::v;
+            mjt_mfma(acc[i / 4][i % 4], fa[SET][i / 4], fb[SET][i % 4]);
+            if constexpr (i < 8) request_one(mjt_ic<SET ^ 1>(), ic, rd_slot, rd_kstep);
+            if constexpr (COPY) copy_one(ic, cp_stage, cp_slot);
+        });
+    };
+    // stages 0 and 1 are asked for; stage 0 must have landed before the loop
+    copy_stage(0, 0);
+    copy_stage(1, 1);
+    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" : : : "memory");
+    mjt_static_for<0, 8>([&](auto fc) { request_one(mjt_ic<0>(), fc, 0, 0); });
+
+#pragma unroll 1
+    for (int s = 0; s < nstages; s++) {
+        const int slot = s & 1;
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+        kstep(mjt_ic<0>(), slot, 1, mjt_ic<0>(), 0, 0);
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+        kstep(mjt_ic<1>(), slot, 2, mjt_ic<0>(), 0, 0);
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+        kstep(mjt_ic<0>(), slot, 3, mjt_ic<0>(), 0, 0);
+        // Before the last k-step: its fragments are in registers, so nobody reads this stage's buffer any more once
+        // every wave is here, and the copies of the next stage, asked for one stage ago, have landed.
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" : : : "memory");
+        kstep(mjt_ic<1>(), slot ^ 1, 0, mjt_ic<1>(), s + 2, slot);
+    }
+    // The last MFMAs need time to read their operands and write their results; tie the registers to a point behind that.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" : : : "memory");
+    mjt_static_for<0, 4>([&](auto ic) { mjt_keep(fa[0][decltype(ic)::v]); mjt_keep(fa[1][decltype(ic)::v]); mjt_keep(fb[0][decltype(ic)::v]); mjt_keep(fb[1][decltype(ic)::v]); });
+    mjt_static_for<0, 16>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / 4][decltype(ic)::v % 4]); });
+
+    // D of a 32x32 tile: lane holds column lane % 32, rows 8 * (e / 4) + 4 * (lane / 32) + e % 4
+#if OUT == 2
+    float* __restrict__ C = (float*)p.a[2] + (long long)blockIdx.y * (long long)p.a[11];
+#else
+    unsigned short* __restrict__ C = (unsigned short*)p.a[2] + (long long)blockIdx.y * (long long)p.a[11];
+#endif
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int col = n0 + wn * 128 + j * 32 + (lane & 31);
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int row = m0 + wm * 128 + i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e & 3);
+                if (row < M && col < N) {
+                    const float v = acc[i][j][e];
+#if OUT == 2
+                    C[(long long)row * ldc + col] = v;
+#elif OUT == 0
+                    C[(long long)row * ldc + col] = (unsigned short)(__float_as_uint(v) >> 16);     // truncation (type/fp16_compute.h:238-241)
+#else
+                    const _Float16 h = (_Float16)v;                                                  // nearest even (type/fp16_compute.h:147-198)
+                    C[(long long)row * ldc + col] = __builtin_bit_cast(unsigned short, h);
+#endif
+                }
+            }
+        }
+}

@@ -59,6 +59,36 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
                       M < (int64_t(1) << 31) && N < (int64_t(1) << 31) && K < (int64_t(1) << 31) && batch < 65536;
     std::vector<uint64_t> args{bits_of_ptr(A), bits_of_ptr(B), bits_of_ptr(C), (uint64_t)M, (uint64_t)N, (uint64_t)K,
                                (uint64_t)lda, (uint64_t)ldb, (uint64_t)ldc, (uint64_t)sa, (uint64_t)sb, (uint64_t)sc};
+    // Both operands with k innermost, 16-bit, K a multiple of 64 and enough tiles of 256 x 256 to go round: the kernel
+    // whose operands reach LDS without passing through registers.  (Offsets inside a tile are 32-bit there.)
+    if (fast && a_kcont && b_kcont && esz == 2 && K % 64 == 0 && !getenv("MJT_GEMM_NO_DMA") && lda * 2 * 256 < (int64_t(1) << 31) &&
+        ldb * 2 * 256 < (int64_t(1) << 31)) {
+        const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
+        const int64_t tm = (M + 255) / 256, tn = (N + 255) / 256;
+        const double edge = ((double)M * N) / ((double)tm * 256 * tn * 256);
+        const double tiles = (double)tm * tn * batch;
+        const double util = tiles / (std::ceil(tiles / cus) * cus);
+        if ((edge >= 0.85 && util >= 0.7) || getenv("MJT_GEMM_DMA")) {
+            const int in = in_dtype == MJT_BFLOAT16 ? 0 : 1;
+            const int out = out_dtype == MJT_BFLOAT16 ? 0 : out_dtype == MJT_FLOAT16 ? 1 : 2;
+            std::ostringstream key;
+            key << "gemmd|" << in << out;
+            JitKernel* k = cached(key.str());
+            if (!k) {
+                std::ostringstream name;
+                name << "mjt_gemm_mfma_" << mjt_dtype_name(in_dtype) << "_" << mjt_dtype_name(out_dtype) << "_256x256_nt_direct";
+                std::ostringstream src;
+                src << "#define ENTRY " << name.str() << "\n#define IN " << in << "\n#define OUT " << out << "\n";
+                src << embedded_source("gemm_dma.h") << "\n";
+                k = jit_get(src.str(), name.str());
+                remember(key.str(), k);
+            }
+            const int64_t grid = (tm * tn + 7) / 8 * 8;
+            MJT_CHECK(grid < (int64_t(1) << 31), "matmul: launch too large");
+            jit_launch(k, (unsigned)grid, (unsigned)batch, 256, 0, args);
+            return;
+        }
+    }
     if (fast) {
         // Tile: the largest of 64 MI x 64 NI (MI, NI in 1, 2, 4) that still gives every compute unit work and wastes
         // little on the edges; larger tiles read each operand element less often.

@@ -89,6 +89,23 @@ def test_gemm_mfma_layouts_and_edges(gpu, dt, ta, tb):
         assert _run(lib, dt, "float32", 304, 200, 136, ta, tb).startswith("mjt_gemm_mfma_")
 
 
+@pytest.mark.parametrize("dt", ["bfloat16", "float16"])
+def test_gemm_direct_copy_kernel(gpu, dt, monkeypatch):
+    """a x b^T with 16-bit operands and K a multiple of 64 has a kernel of its own (operands go from memory to LDS
+    without passing through registers) once there are enough 256 x 256 tiles; here it is asked for by name so that
+    small shapes reach it too: tiles that hang over both edges, a single stage pair (K = 64), many stages, a
+    float32 result, a batch."""
+    lib = L.load()
+    monkeypatch.setenv("MJT_GEMM_DMA", "1")
+    for i, (M, K, N) in enumerate([(256, 64, 256), (512, 256, 256), (304, 128, 136), (1000, 192, 520), (8, 512, 8), (520, 2048, 264)]):
+        kern = _run(lib, dt, dt, M, K, N, 0, 1, seed=20 + i)
+        assert kern.endswith("_256x256_nt_direct"), kern
+    assert _run(lib, dt, "float32", 304, 128, 520, 0, 1, seed=30).endswith("_256x256_nt_direct")
+    assert _run(lib, dt, dt, 260, 64, 250, 0, 1, seed=31, batch=(3,)).endswith("_256x256_nt_direct")
+    # K = 96 is no multiple of 64: the general kernel
+    assert not _run(lib, dt, dt, 256, 96, 256, 0, 1, seed=32).endswith("_direct")
+
+
 def test_gemm_k_tail_inside_a_chunk(gpu):
     """k-innermost operands whose K is no multiple of the chunk: the row length (leading dimension) is what has to
     be aligned, and a product's operands are dense, so this route is only reachable with a K that is aligned;
