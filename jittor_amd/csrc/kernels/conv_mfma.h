@@ -7,7 +7,9 @@
 // (opt/kernel_ir.cc:958-968, ops/reduce_op.cc:259-266).  Taps outside the image
 // contribute 0 (overflow value 0 times w).
 //
-// All geometry is baked in by the host: C_, H_, W_, K_, R_, S_, OH_, OW_, SH, SW,
+// All geometry is baked in by the host: C_, H_, W_, K_ (input and output channels of the convolution: of one group when
+// it is grouped; XC_ and YK_ are then the channel counts of the whole x and y, whose pointers the host has moved to
+// the group's first channel), R_, S_, OH_, OW_, SH, SW,
 // PH, PW, DH, DW, WKO (groups of 16*MT output channels per workgroup), WPX (row
 // groups per workgroup), TRW / NT / LROWS (output rows per wave, 16-pixel tiles per
 // wave and input rows in LDS of a full tile), RPW (output rows a workgroup owns),
@@ -198,7 +200,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // buffer descriptors (base, size in bytes): addresses are a scalar offset plus a 32-bit lane offset,
     // so no per-item 64-bit address lives in vector registers
     const __amdgpu_buffer_rsrc_t x_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void*)(xp + (size_t)n * C_ * H_ * W_), 0, C_ * H_ * W_ * 2, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc((void*)(xp + (size_t)n * XC_ * H_ * W_), 0, C_ * H_ * W_ * 2, 0x00020000);
     const unsigned x_lane_off = (unsigned)sr * (H_ * W_ * 2);
     const unsigned as_spare = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned short*)&as_ring[0] + NS * KO_WG * 64;
     auto item_of = [&](int item, int& lr, int& seg, int& cg) {
@@ -228,7 +230,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // issued between two points is known and the waits can name exactly the loads that may still be under way.
     mjt_u32x4v x_desc;
     {
-        const unsigned long long base = (unsigned long long)(xp + (size_t)n * C_ * H_ * W_);
+        const unsigned long long base = (unsigned long long)(xp + (size_t)n * XC_ * H_ * W_);
         x_desc[0] = __builtin_amdgcn_readfirstlane((unsigned)base);
         x_desc[1] = __builtin_amdgcn_readfirstlane((unsigned)(base >> 32) & 0xffffu);
         x_desc[2] = C_ * H_ * W_ * 2;
@@ -527,7 +529,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                 y4[3] = b1 ? a3 : h1;
                 if (ok) {
                     const int ko = ko_base + m * 16 + lg * 4 + qj;
-                    const size_t o = (((size_t)n * K_ + ko) * OH_ + orow) * OW_ + col;
+                    const size_t o = (((size_t)n * YK_ + ko) * OH_ + orow) * OW_ + col;
 #if Y_BF16
                     mjt_u32x2 pk;
                     pk[0] = mjt_narrow2(y4[0], y4[1]);
@@ -551,7 +553,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         const int ko = ko_base + m * 16 + lg * 4 + i;
-                        const size_t o = (((size_t)n * K_ + ko) * OH_ + orow) * OW_ + col;
+                        const size_t o = (((size_t)n * YK_ + ko) * OH_ + orow) * OW_ + col;
 #if Y_BF16
                         ((unsigned short*)p.a[2])[o] = (unsigned short)mjt_narrow2(acc[m][t][i], 0.0f);
 #else

@@ -105,8 +105,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t max_px = WPX == 1 ? 224 : 112;            // pixels per wave: 16 per accumulator tile
     const int64_t WPS = max_px == 224 ? 1 : 2;              // waves per SIMD the register budget is set for
     // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
-    const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && K % 128 == 0 ? 8 : 4;
-    int64_t WKO = K % 256 == 0 ? 256 / (16 * MT) : K % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
+    const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && (K / G) % 128 == 0 ? 8 : 4;
+    const int64_t Kg = K / G;                                // output channels of one group: the K of the MFMA kernel
+    int64_t WKO = Kg % 256 == 0 ? 256 / (16 * MT) : Kg % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
     // LDS: two buffers of input rows (one block of CB channels each), a ring of NS weight slabs (64 bytes per output
     // channel of the workgroup each) and a spare KB that takes the writes of idle lanes.  Blocks of 32 channels
     // leave room for a deeper ring, which is what hides the latency of the slabs; the ring needs three slabs at least.
@@ -130,23 +131,24 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int64_t cus0 = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
         const int64_t tile_rows = WPX * (TRW > 0 ? TRW : 1);
         const int64_t min_ranges = N * ((OH + tile_rows - 1) / tile_rows);
-        while (WKO > 1 && 2 * min_ranges * (K / (16 * MT * WKO)) <= cus0) WKO /= 2;     // only while at most half of them would work
+        while (WKO > 1 && 2 * min_ranges * (Kg / (16 * MT * WKO)) <= cus0) WKO /= 2;     // only while at most half of them would work
         if (const char* e = getenv("MJT_CONV_WKO"))
-            if (atoi(e) >= 1 && atoi(e) <= WKO * 4 && K % (16 * MT * atoi(e)) == 0 && (atoi(e) & (atoi(e) - 1)) == 0 && atoi(e) <= 256 / (16 * MT)) WKO = atoi(e);
+            if (atoi(e) >= 1 && atoi(e) <= WKO * 4 && Kg % (16 * MT * atoi(e)) == 0 && (atoi(e) & (atoi(e) - 1)) == 0 && atoi(e) <= 256 / (16 * MT)) WKO = atoi(e);
     }
     const bool half = x->dtype == MJT_FLOAT16;
-    const bool mfma_ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % CBLK == 0 && K % 64 == 0 &&
+    // (a grouped convolution is one launch per group on the group's channels: worth it from 32 x 64 channels per group)
+    const bool mfma_ok = (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % CBLK == 0 && Kg % 64 == 0 && G <= 64 &&
                          W % 2 == 0 && TRW >= 1 && NT <= max_px / 16 && LROWS * LCOLS * CBLK * 2 <= tile_limit &&
                          // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
                          ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + (CBLK == 64 ? 4 * LROWS * LCOLS * 16 : 0) < 65536 &&
                          (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49 &&
                          // byte offsets inside one image and inside the weights are 32-bit in the kernel
-                         C * H * W * 2 < (int64_t(1) << 31) && K * OH * OW * 4 < (int64_t(1) << 31) && numel(w) * 2 < (int64_t(1) << 31);
+                         C * G * H * W * 2 < (int64_t(1) << 31) && K * OH * OW * 4 < (int64_t(1) << 31) && numel(w) * 2 < (int64_t(1) << 31);
     if (mfma_ok) {
         // Rows per workgroup: a workgroup walks RPW output rows as NFULL tiles of TR rows plus one
         // shorter tile.  Pick the RPW that minimises (rounds of workgroups over the compute units) x
         // (accumulator tiles a workgroup computes, plus a per-tile overhead worth half a tile column).
-        const int64_t TR = WPX * TRW, KPARTS = K / (16 * MT * WKO);
+        const int64_t TR = WPX * TRW, KPARTS = Kg / (16 * MT * WKO);
         const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
         auto tail_of = [&](int64_t rpw, int64_t* trw_t, int64_t* nt_t) {
             const int64_t t = rpw % TR;
@@ -181,17 +183,19 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             if (atoi(e) >= 3 && atoi(e) <= NSLAB) NSLAB = atoi(e);
         MJT_CHECK(NSLAB >= 3, "conv: internal: no room for the weight ring");
         const int stage_depth = getenv("MJT_CONV_SD") && atoi(getenv("MJT_CONV_SD")) >= 2 && atoi(getenv("MJT_CONV_SD")) <= 8 ? atoi(getenv("MJT_CONV_SD")) : 4;
-        key << "mfma|" << half << "|" << geo.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT << "|" << WPS
+        std::ostringstream geo_g;                        // the kernel's K_ is a group's; XC_ / YK_ are the strides of x and y between images
+        geo_g << geo.str() << "#undef K_\n#define K_ " << Kg << "\n#define XC_ " << C * G << "\n#define YK_ " << K << "\n";
+        key << "mfma|" << half << "|" << geo_g.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT << "|" << WPS
             << "|" << stage_depth << "|" << CBLK << "|" << NSLAB;
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
             std::ostringstream name;
-            name << "mjt_conv_mfma_" << (half ? "f16" : "bf16") << "_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s"
+            name << "mjt_conv_mfma_" << (half ? "f16" : "bf16") << "_c" << C << "_k" << Kg << (G > 1 ? "_g" + std::to_string(G) : std::string()) << "_" << H << "x" << W << "_r" << R << "x" << S << "_s"
                  << p->stride_h << "x" << p->stride_w << "_p" << p->pad_h << "x" << p->pad_w << "_d" << p->dil_h << "x"
                  << p->dil_w << "_rows" << RPW << (y->dtype == MJT_FLOAT32 ? "_of32" : half ? "_of16" : "_obf16");
             std::ostringstream src;
-            src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo.str()
+            src << "#define ENTRY " << name.str() << "\n#define ENTRY_PACK " << name.str() << "_pack\n" << geo_g.str()
                 << "#define MT " << MT << "\n#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
                 << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS << "\n#define Y_BF16 " << (y->dtype != MJT_FLOAT32 ? 1 : 0) << "\n#define IN_F16 " << (half ? 1 : 0)
@@ -214,16 +218,23 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             HIP_CHECK(hipMalloc(&g_wpack, wbytes));
             g_wpack_bytes = wbytes;
         }
-        std::vector<uint64_t> pa{bits_of_ptr(w->ptr), bits_of_ptr(g_wpack), 0, 0};
-        int64_t pblocks = (numel(w) + 255) / 256;
-        if (pblocks > 2048) pblocks = 2048;
-        jit_launch(kp, (unsigned)pblocks, 1, 256, 0, pa);
         const int64_t ranges = N * ((OH + RPW - 1) / RPW);
         const int64_t ranges8 = (ranges + 7) / 8 * 8;
         const int64_t blocks = ranges8 * KPARTS;
         MJT_CHECK(blocks < (int64_t(1) << 31), "conv: launch too large");
-        std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(g_wpack), bits_of_ptr(y->ptr), (uint64_t)N};
-        jit_launch(k, (unsigned)blocks, 1, (unsigned)(64 * WPX * WKO), 0, a);
+        const int64_t wg = Kg * C * R * S;               // weights of one group
+        int64_t pblocks = (wg + 255) / 256;
+        if (pblocks > 2048) pblocks = 2048;
+        const int64_t ysz = y->dtype == MJT_FLOAT32 ? 4 : 2;
+        for (int64_t g = 0; g < G; g++) {
+            const char* wsrc = (const char*)w->ptr + g * wg * 2;
+            char* wdst = (char*)g_wpack + g * wg * 2;
+            std::vector<uint64_t> pa{bits_of_ptr(wsrc), bits_of_ptr(wdst), 0, 0};
+            jit_launch(kp, (unsigned)pblocks, 1, 256, 0, pa);
+            std::vector<uint64_t> a{bits_of_ptr((const char*)x->ptr + g * C * H * W * 2), bits_of_ptr(wdst),
+                                    bits_of_ptr((char*)y->ptr + g * Kg * OH * OW * ysz), (uint64_t)N};
+            jit_launch(k, (unsigned)blocks, 1, (unsigned)(64 * WPX * WKO), 0, a);
+        }
         return;
     }
 

@@ -648,6 +648,35 @@ def test_conv_grouped_entry_and_front_end(gpu):
         jt.nn.conv2d(jt.array(x), jt.array(w), groups=4)
 
 
+@pytest.mark.parametrize("xs,ws,G,params,out", [
+    ((2, 128, 12, 16), (256, 64, 3, 3), 2, (1, 1, 1, 1, 1, 1), "float32"),      # two groups of 64 -> 128 channels
+    ((3, 128, 9, 24), (256, 32, 3, 3), 4, (1, 1, 1, 1, 1, 1), "bfloat16"),      # four groups of 32 -> 64, 16-bit result
+    ((2, 192, 10, 12), (192, 64, 1, 1), 3, (2, 2, 0, 0, 1, 1), "float32"),      # 1x1 stride 2, three groups
+])
+def test_conv_grouped_on_the_mfma_kernel(gpu, xs, ws, G, params, out):
+    """Groups of at least 32 input and 64 output channels run on the MFMA kernel, one launch per group on the group's
+    channels (python/jittor/nn.py:1272-1294): against the oracle's grouped convolution of the exact 16-bit operands,
+    per element within 1e-4 of the sum of its terms' magnitudes."""
+    rng = np.random.default_rng(41)
+    xb = O.f32_to_bf16_bits(rng.standard_normal(xs).astype(np.float32))
+    wb = O.f32_to_bf16_bits((rng.standard_normal(ws) * 0.1).astype(np.float32))
+    xf, wf = O.BF16(xb).to_f32(), O.BF16(wb).to_f32()
+    sh, sw, ph, pw, dh, dw = params
+    want = O.conv_meta_grouped(xf, wf, G, sh, ph, dh)
+    terms = O.conv_meta_grouped(np.abs(xf), np.abs(wf), G, sh, ph, dh)
+    x, w = jt.from_storage(xb, "bfloat16"), jt.from_storage(wb, "bfloat16")
+    y = jt.zeros(list(want.shape), out)
+    tx, tw, ty = L.tensor(x.raw_ptr(), "bfloat16", x.shape), L.tensor(w.raw_ptr(), "bfloat16", w.shape), L.tensor(y.raw_ptr(), out, y.shape)
+    p = L.ConvParams(*params)
+    L.check(L.load().mjt_conv2d_meta_grouped(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p), G))
+    kern = L.last_kernel()
+    assert kern.startswith("mjt_conv_mfma_bf16") and "_g%d_" % G in kern, kern
+    got = L.d2h(y.raw_ptr(), y.shape, L.NP_STORAGE[out])
+    got = O.BF16(got).to_f32().astype(np.float64) if out == "bfloat16" else got.astype(np.float64)
+    bound = 1e-4 * terms + (np.abs(want) * 2.0 ** -7 if out == "bfloat16" else 0.0)
+    assert (np.abs(got - want) <= bound).all(), float((np.abs(got - want) / np.maximum(bound, 1e-30)).max())
+
+
 def _wgrad_call(xbits, dybits, R, S, params, out_dtype="float32", in_dtype="bfloat16"):
     x, dy = jt.from_storage(xbits, in_dtype), jt.from_storage(dybits, in_dtype)
     dw = jt.zeros([dybits.shape[1], xbits.shape[1], R, S], out_dtype)
