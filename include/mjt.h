@@ -9,6 +9,9 @@
  * python/jittor/src/executor.cc:575-577, and kernels only read
  * Var::mem_ptr/shape/dtype, python/jittor/src/var.h:18-49).  Work is queued
  * on one stream per device and is asynchronous; mjt_sync() waits for it.
+ * Entry points may be called from several host threads: the library takes
+ * one lock per call, so the calls (and the kernels they queue) run one after
+ * the other.
  *
  * Paths in the citations below are relative to python/jittor/src/ of the
  * reference tree.

@@ -4,6 +4,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 #include <sstream>
@@ -40,8 +41,12 @@ struct Error {
     } while (0)
 
 // Every extern "C" entry point runs its body through this guard so that no
-// exception crosses the C boundary.
+// exception crosses the C boundary.  The guard also takes the library's one lock: the context, the scratch arena
+// and the growing device buffers of the convolution paths are process-wide, and work is queued on one stream, so
+// calls from several host threads run one after the other (the lock is recursive: an entry point may call another).
+std::recursive_mutex& api_mutex();
 template <class F> int guarded(F&& f) {
+    std::lock_guard<std::recursive_mutex> lock(api_mutex());
     try {
         f();
         return MJT_OK;

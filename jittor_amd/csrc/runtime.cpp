@@ -22,6 +22,11 @@ static std::mutex g_jit_mutex;
 static std::unordered_map<std::string, JitKernel*> g_jit_cache;
 static int64_t g_jit_compiled = 0, g_jit_hits = 0;
 
+std::recursive_mutex& api_mutex() {
+    static std::recursive_mutex m;
+    return m;
+}
+
 int set_error(int code, const std::string& msg) {
     g_error = msg;
     return code;
