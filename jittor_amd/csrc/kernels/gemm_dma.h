@@ -1,26 +1,34 @@
-// Matrix product on MFMA, both operands with k innermost in memory:  C[b][M][N] = sum_k A[b][M][K] * B[b][N][K]
+// Matrix product on MFMA for 16-bit operands, operands copied from memory straight into LDS:
+//   C[b][M][N] = sum_k A'[b][M][K] * B'[b][K][N]
 // (reference: the broadcast * broadcast -> reduce.add pattern that
 // python/jittor/src/opt/tuner/matmul_tuner.cc:16-104 relays to a library GEMM,
-// python/jittor/extern/cuda/cublas/ops/cublas_matmul_op.cc:27-126; this is the a x b^T case, the
-// forward product of a linear layer, python/jittor/nn.py:628-643).  bfloat16 / float16 operands with exact
+// python/jittor/extern/cuda/cublas/ops/cublas_matmul_op.cc:27-126; a x b^T is the forward product of a linear
+// layer, python/jittor/nn.py:628-643).  Row-major operands; A' is a, or a transposed when A_KCONT == 0 (memory
+// [K][M]); B' is b, or b transposed when B_KCONT == 1 (memory [N][K]).  bfloat16 / float16 operands with exact
 // products and float32 accumulation.
 //
 // Supplied by the host: IN (0 bfloat16, 1 float16), OUT (0 bfloat16 by truncation, 1 float16 rounded to
-// nearest even, 2 float32).  K is a multiple of 64, leading dimensions are multiples of 16 bytes and the
-// operand pointers 16-byte aligned (the host sends everything else to the general kernel).
+// nearest even, 2 float32), A_KCONT, B_KCONT (the operand's memory has k innermost).  K is a multiple of 64, leading
+// dimensions are multiples of 16 bytes and the operand pointers 16-byte aligned (the host sends everything else to the
+// general kernel).
 //
 // Mapping.  A workgroup of four waves (2 x 2, one wave per SIMD) owns a 256 x 256 tile of C; a wave owns
 // 128 x 128 of it as 4 x 4 accumulator tiles of v_mfma_f32_32x32x16, 256 accumulation registers.  K is walked in
 // stages of 64 (whole 128-byte lines of both operands): the 256 x 64 pieces of both operands (64 KB) alternate
-// between two buffers in LDS.  Nothing on that way passes through registers: a wave copies 8 rows x 128 bytes per
-// instruction straight from memory into LDS (lane i lands at byte 16 i of the 1 KB the instruction fills), a
-// stage ahead of their use.  A row of a stage is eight 16-byte chunks; chunk c of row r sits at position
-// c ^ (r / 2 % 8), which the copying lane arranges by choosing what it fetches.  The 16 lanes that read a
-// fragment together (16 neighbouring rows, one chunk) then touch 16 different bank groups.  Lane (row = lane % 32,
-// half = lane / 32) reads the 8 consecutive k of its row and half with one 16-byte LDS read; the fragments of
-// the next k-step are read while the 16 MFMAs of a k-step run.  One barrier per stage, before its last k-step,
-// hands over the next stage, which has landed by then, and frees the buffer of the current one, whose last
-// fragments are in registers.  Rows beyond M and N are read from the last valid row (their results are not stored).
+// between two buffers in LDS.  Nothing on that way passes through registers: a wave copies 1 KB per instruction
+// straight from memory into LDS (lane i lands at byte 16 i of that KB), a stage ahead of its use.  For an operand
+// with k innermost that is 8 rows x 128 bytes: a row of a stage is eight 16-byte chunks, chunk c of row r sits at
+// position c ^ (r / 2 % 8), which the copying lane arranges by choosing what it fetches; the 16 lanes that read a
+// fragment together (16 neighbouring rows, one chunk) then touch 16 different bank groups, and lane (row =
+// lane % 32, half = lane / 32) reads the 8 consecutive k of its row and half with one 16-byte LDS read.  An operand
+// with m or n innermost stays as it lies in memory, [64 k][256 columns], and the fragment is made by two transposing
+// LDS reads (ds_read_b64_tr_b16: the 16 lanes of a group present 16 8-byte pieces, four k-rows x 16 columns, and
+// each receives one column's four k); its 32-byte units are permuted within a row by the k-row so that the four
+// rows of a read fall into different banks.  The fragments of the next k-step are read while the 16 MFMAs of a
+// k-step run.  One barrier per stage, before its last k-step, hands over the next stage, which has landed by then,
+// and frees the buffer of the current one, whose last fragments are in registers.  Rows beyond M and N of an operand
+// with k innermost are read from the last valid row, columns beyond them of the other kind from whatever follows in
+// memory (zero past the operand's end); their results are not stored.
 //
 // The MFMAs are spelled out, like the LDS reads and the waits, so that the order below is the schedule; the
 // accumulators live in the accumulation registers, which nothing but these MFMAs touches inside the loop (the
@@ -46,13 +54,24 @@ template <int I, int N, class F> __device__ __forceinline__ void mjt_static_for(
         mjt_static_for<I + 1, N>(f);
     }
 }
-template <int OFF> __device__ __forceinline__ void mjt_ds_read(mjt_u32x4v& dst, unsigned addr) {
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+typedef unsigned mjt_u32x2 __attribute__((ext_vector_type(2)));
+// a 16-byte read delivered as two halves (so that fragments have one representation whichever read fills them)
+template <int OFF> __device__ __forceinline__ void mjt_ds_read_pair(mjt_u32x2& lo, mjt_u32x2& hi, unsigned addr) {
+    mjt_u32x4v v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    lo[0] = v[0]; lo[1] = v[1]; hi[0] = v[2]; hi[1] = v[3];
 }
-__device__ __forceinline__ void mjt_mfma(mjt_f32x16& c, const mjt_u32x4v& a, const mjt_u32x4v& b) {
+// transposing read: the lane receives four 16-bit values, one from each of four lanes' 8-byte pieces
+template <int OFF> __device__ __forceinline__ void mjt_ds_read_tr(mjt_u32x2& dst, unsigned addr) {
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+__device__ __forceinline__ void mjt_mfma2(mjt_f32x16& c, const mjt_u32x2& alo, const mjt_u32x2& ahi, const mjt_u32x2& blo, const mjt_u32x2& bhi) {
+    mjt_u32x4v a, b;
+    a[0] = alo[0]; a[1] = alo[1]; a[2] = ahi[0]; a[3] = ahi[1];
+    b[0] = blo[0]; b[1] = blo[1]; b[2] = bhi[0]; b[3] = bhi[1];
     asm volatile(MJT_MFMA_ASM " %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
-__device__ __forceinline__ void mjt_keep(const mjt_u32x4v& x) { asm volatile("" : : "v"(x)); }     // x is in its registers up to here
+__device__ __forceinline__ void mjt_keep2(const mjt_u32x2& x) { asm volatile("" : : "v"(x)); }     // x is in its registers up to here
 __device__ __forceinline__ void mjt_pin(mjt_f32x16& x) { asm volatile("" : "+a"(x)); }            // what reads x later comes after this point
 
 struct Params { void* a[12]; };
@@ -89,50 +108,107 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     const int wm = wave >> 1, wn = wave & 1;
     const int nstages = K / KS;
 
-    // Copies.  A stage is 64 instructions of 1 KB (32 of A, 32 of B); wave w issues number 8w .. 8w+7 of each.
-    // Lane i of instruction j fills row 8 j + i / 8, position i % 8, with chunk (i % 8) ^ (row / 2 % 8).
-    // Descriptors start at the tile's first row; the lane offset is its row (clamped to the matrix) times the
-    // leading dimension plus its chunk, the stage adds 128 bytes per step through the scalar offset.
+    // Copies.  A stage is 64 instructions of 1 KB (32 per operand); wave w issues number 8w .. 8w+7 of each operand.
+    // An operand with k innermost is staged [256 rows][64 k]: lane i of instruction j fills row 8 j + i / 8, position
+    // i % 8, with chunk (i % 8) ^ (row / 2 % 8); its descriptor starts at the tile's first row, the lane offset is its
+    // row (clamped to the matrix) times the leading dimension plus its chunk, and a stage adds 128 bytes through the
+    // scalar offset.  An operand with m (or n) innermost is staged as it lies in memory, [64 k][256 columns], 512-byte
+    // rows of sixteen 32-byte units: lane i of instruction j fills k-row 2 j + i / 32, 16-byte piece i % 32, and unit u of
+    // k-row r sits at position u ^ (r % 4).  Its descriptor starts at the tile's first column and ends with the operand,
+    // so whatever lies past the matrix reads as zero; a stage adds 64 rows through the scalar offset.
     const int last_a = M - 1 - m0, last_b = N - 1 - n0;             // last valid row of the tile
     unsigned voff_a[8], voff_b[8];
 #pragma unroll
     for (int q = 0; q < 8; q++) {
         const int row = (wave * 8 + q) * 8 + (lane >> 3);
         const unsigned chunk = (unsigned)((lane & 7) ^ ((row >> 1) & 7));
+        const int krow = (wave * 8 + q) * 2 + (lane >> 5);
+        const unsigned piece = (unsigned)(((((lane & 31) >> 1) ^ (krow & 3)) << 1) | (lane & 1));      // 16-byte piece of the k-row in memory
+#if A_KCONT
         voff_a[q] = (unsigned)(row < last_a ? row : last_a) * (unsigned)(lda * 2) + chunk * 16;
+#else
+        voff_a[q] = (unsigned)krow * (unsigned)(lda * 2) + piece * 16;
+#endif
+#if B_KCONT
         voff_b[q] = (unsigned)(row < last_b ? row : last_b) * (unsigned)(ldb * 2) + chunk * 16;
+#else
+        voff_b[q] = (unsigned)krow * (unsigned)(ldb * 2) + piece * 16;
+#endif
     }
+#if A_KCONT
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(A + (long long)m0 * lda), 0, 0x7fffffff, 0x00020000);
+    const int a_step = KS * 2;
+#else
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(A + m0), 0, (int)(((long long)(K - 1) * lda + (M - m0)) * 2), 0x00020000);
+    const int a_step = (int)(KS * lda * 2);
+#endif
+#if B_KCONT
     const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(B + (long long)n0 * ldb), 0, 0x7fffffff, 0x00020000);
+    const int b_step = KS * 2;
+#else
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(B + n0), 0, (int)(((long long)(K - 1) * ldb + (N - n0)) * 2), 0x00020000);
+    const int b_step = (int)(KS * ldb * 2);
+#endif
     // instruction q (0 .. 15: eight of A, eight of B) of this wave's share of stage s; s and slot uniform
     auto copy_one = [&](auto qc, int s, int slot) {
         constexpr int q = decltype(qc)::v;
         const int st = s < nstages ? s : nstages - 1;               // past the end: a stage nobody reads
-        const int soff = st * (KS * 2);
         __attribute__((address_space(3))) unsigned char* dst =
             (__attribute__((address_space(3))) unsigned char*)&lds[0] + slot * STAGE_BYTES + wave * 8192;
         // (an immediate offset would move the place in memory along with the place in LDS)
         if constexpr (q < 8)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void*)(dst + q * 1024), 16, (int)voff_a[q], soff, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void*)(dst + q * 1024), 16, (int)voff_a[q], st * a_step, 0, 0);
         else
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void*)(dst + TM * 128 + (q - 8) * 1024), 16, (int)voff_b[q - 8], soff, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void*)(dst + TM * 128 + (q - 8) * 1024), 16, (int)voff_b[q - 8], st * b_step, 0, 0);
     };
     auto copy_stage = [&](int s, int slot) { mjt_static_for<0, 16>([&](auto qc) { copy_one(qc, s, slot); }); };
 
-    // Fragment addresses of this lane: row lane % 32 of each 32-row block of its wave's rows, chunk 2 * k-step +
-    // lane / 32 at position chunk ^ (row / 2 % 8): the position of k-step 0 with the k-step's bits flipped.
+    // Fragments.  Lane (row = lane % 32, half = lane / 32) of v_mfma_f32_32x32x16 wants the 8 consecutive k of its row
+    // and half.  From a [rows][64 k] tile that is one 16-byte read: row lane % 32 of each 32-row block of the wave's
+    // rows, chunk 2 * k-step + half at position chunk ^ (row / 2 % 8), i.e. the position of k-step 0 with the k-step's
+    // bits flipped.  From a [64 k][256 columns] tile it is two transposing reads of four k each: the 16 lanes of a group
+    // point at four k-rows x four 8-byte pieces (lane i at k-row i / 4, piece i % 4 of the group's 16 columns) and
+    // receive column i of the group for those four k.
     const int frow = lane & 31;
     const unsigned pos0 = (unsigned)((lane >> 5) ^ ((frow >> 1) & 7));
     const unsigned lds_base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned char*)&lds[0];
+    const int ti = lane & 15, tg = (lane >> 4) & 1, tk = lane >> 5;
+#if A_KCONT
     const unsigned a_lane = lds_base + (unsigned)((wm * 128 + frow) * 128);
+#else
+    unsigned a_tr[4];
+#pragma unroll
+    for (int f = 0; f < 4; f++) a_tr[f] = lds_base + (unsigned)((tk * 8 + (ti >> 2)) * 512 + (((wm * 8 + 2 * f + tg) ^ (ti >> 2)) * 32) + (ti & 3) * 8);
+#endif
+#if B_KCONT
     const unsigned b_lane = lds_base + (unsigned)(TM * 128 + (wn * 128 + frow) * 128);
-    mjt_u32x4v fa[2][4], fb[2][4];
-    // fragment f (0 .. 7: four of A, four of B) of k-step kstep of the stage in slot, into set SET
-    auto request_one = [&](auto setc, auto fc, int slot, int kstep) {
-        constexpr int SET = decltype(setc)::v, f = decltype(fc)::v;
-        const unsigned off = (unsigned)(slot * STAGE_BYTES) + ((pos0 ^ (unsigned)(kstep * 2)) * 16);
-        if constexpr (f < 4) mjt_ds_read<f * 4096>(fa[SET][f], a_lane + off);
-        else mjt_ds_read<(f - 4) * 4096>(fb[SET][f - 4], b_lane + off);
+#else
+    unsigned b_tr[4];
+#pragma unroll
+    for (int f = 0; f < 4; f++) b_tr[f] = lds_base + (unsigned)(TM * 128 + (tk * 8 + (ti >> 2)) * 512 + (((wn * 8 + 2 * f + tg) ^ (ti >> 2)) * 32) + (ti & 3) * 8);
+#endif
+    mjt_u32x2 falo[2][4], fahi[2][4], fblo[2][4], fbhi[2][4];       // a fragment's four registers in two halves
+    constexpr int A_READS = A_KCONT ? 4 : 8, B_READS = B_KCONT ? 4 : 8, READS = A_READS + B_READS;
+    // read number r (0 .. READS-1) of the fragments of k-step kstep (compile-time) of the stage in slot, into set SET
+    auto request_one = [&](auto setc, auto rc, int slot, auto kc) {
+        constexpr int SET = decltype(setc)::v, r = decltype(rc)::v, kstep = decltype(kc)::v;
+        const unsigned soff = (unsigned)(slot * STAGE_BYTES);
+        if constexpr (r < A_READS) {
+#if A_KCONT
+            mjt_ds_read_pair<r * 4096>(falo[SET][r], fahi[SET][r], a_lane + soff + ((pos0 ^ (unsigned)(kstep * 2)) * 16));
+#else
+            if constexpr (r % 2 == 0) mjt_ds_read_tr<(kstep * 16) * 512>(falo[SET][r / 2], a_tr[r / 2] + soff);
+            else mjt_ds_read_tr<(kstep * 16 + 4) * 512>(fahi[SET][r / 2], a_tr[r / 2] + soff);
+#endif
+        } else {
+            constexpr int rb = r - A_READS;
+#if B_KCONT
+            mjt_ds_read_pair<rb * 4096>(fblo[SET][rb], fbhi[SET][rb], b_lane + soff + ((pos0 ^ (unsigned)(kstep * 2)) * 16));
+#else
+            if constexpr (rb % 2 == 0) mjt_ds_read_tr<(kstep * 16) * 512>(fblo[SET][rb / 2], b_tr[rb / 2] + soff);
+            else mjt_ds_read_tr<(kstep * 16 + 4) * 512>(fbhi[SET][rb / 2], b_tr[rb / 2] + soff);
+#endif
+        }
     };
 
     mjt_f32x16 acc[4][4];
@@ -149,13 +225,13 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // A k-step: 16 MFMAs on the fragments of set SET.  What else the wave has to issue goes between them, one
     // instruction after each MFMA, where it costs no MFMA time (the wave is alone on its SIMD): the reads of the next
     // k-step's fragments into the other set and, in the last k-step of a stage, the copies of the stage after the next.
-    auto kstep = [&](auto setc, int rd_slot, int rd_kstep, auto copyc, int cp_stage, int cp_slot) {
+    auto kstep = [&](auto setc, int rd_slot, auto rd_kstep, auto copyc, int cp_stage, int cp_slot) {
         constexpr int SET = decltype(setc)::v;
         constexpr bool COPY = decltype(copyc)::v != 0;
         mjt_static_for<0, 16>([&](auto ic) {
             constexpr int i = decltype(ic)::v;
-            mjt_mfma(acc[i / 4][i % 4], fa[SET][i / 4], fb[SET][i % 4]);
-            if constexpr (i < 8) request_one(mjt_ic<SET ^ 1>(), ic, rd_slot, rd_kstep);
+            mjt_mfma2(acc[i / 4][i % 4], falo[SET][i / 4], fahi[SET][i / 4], fblo[SET][i % 4], fbhi[SET][i % 4]);
+            if constexpr (i < READS) request_one(mjt_ic<SET ^ 1>(), ic, rd_slot, rd_kstep);
             if constexpr (COPY) copy_one(ic, cp_stage, cp_slot);
         });
     };
@@ -163,25 +239,28 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     copy_stage(0, 0);
     copy_stage(1, 1);
     asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" : : : "memory");
-    mjt_static_for<0, 8>([&](auto fc) { request_one(mjt_ic<0>(), fc, 0, 0); });
+    mjt_static_for<0, READS>([&](auto rc) { request_one(mjt_ic<0>(), rc, 0, mjt_ic<0>()); });
 
 #pragma unroll 1
     for (int s = 0; s < nstages; s++) {
         const int slot = s & 1;
         asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-        kstep(mjt_ic<0>(), slot, 1, mjt_ic<0>(), 0, 0);
+        kstep(mjt_ic<0>(), slot, mjt_ic<1>(), mjt_ic<0>(), 0, 0);
         asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-        kstep(mjt_ic<1>(), slot, 2, mjt_ic<0>(), 0, 0);
+        kstep(mjt_ic<1>(), slot, mjt_ic<2>(), mjt_ic<0>(), 0, 0);
         asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-        kstep(mjt_ic<0>(), slot, 3, mjt_ic<0>(), 0, 0);
+        kstep(mjt_ic<0>(), slot, mjt_ic<3>(), mjt_ic<0>(), 0, 0);
         // Before the last k-step: its fragments are in registers, so nobody reads this stage's buffer any more once
         // every wave is here, and the copies of the next stage, asked for one stage ago, have landed.
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" : : : "memory");
-        kstep(mjt_ic<1>(), slot ^ 1, 0, mjt_ic<1>(), s + 2, slot);
+        kstep(mjt_ic<1>(), slot ^ 1, mjt_ic<0>(), mjt_ic<1>(), s + 2, slot);
     }
     // The last MFMAs need time to read their operands and write their results; tie the registers to a point behind that.
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" : : : "memory");
-    mjt_static_for<0, 4>([&](auto ic) { mjt_keep(fa[0][decltype(ic)::v]); mjt_keep(fa[1][decltype(ic)::v]); mjt_keep(fb[0][decltype(ic)::v]); mjt_keep(fb[1][decltype(ic)::v]); });
+    mjt_static_for<0, 8>([&](auto ic) {
+        constexpr int st = decltype(ic)::v / 4, f = decltype(ic)::v % 4;
+        mjt_keep2(falo[st][f]); mjt_keep2(fahi[st][f]); mjt_keep2(fblo[st][f]); mjt_keep2(fbhi[st][f]);
+    });
     mjt_static_for<0, 16>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / 4][decltype(ic)::v % 4]); });
 
     // D of a 32x32 tile: lane holds column lane % 32, rows 8 * (e / 4) + 4 * (lane / 32) + e % 4

@@ -59,10 +59,11 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
                       M < (int64_t(1) << 31) && N < (int64_t(1) << 31) && K < (int64_t(1) << 31) && batch < 65536;
     std::vector<uint64_t> args{bits_of_ptr(A), bits_of_ptr(B), bits_of_ptr(C), (uint64_t)M, (uint64_t)N, (uint64_t)K,
                                (uint64_t)lda, (uint64_t)ldb, (uint64_t)ldc, (uint64_t)sa, (uint64_t)sb, (uint64_t)sc};
-    // Both operands with k innermost, 16-bit, K a multiple of 64 and enough tiles of 256 x 256 to go round: the kernel
-    // whose operands reach LDS without passing through registers.  (Offsets inside a tile are 32-bit there.)
-    if (fast && a_kcont && b_kcont && esz == 2 && K % 64 == 0 && !getenv("MJT_GEMM_NO_DMA") && lda * 2 * 256 < (int64_t(1) << 31) &&
-        ldb * 2 * 256 < (int64_t(1) << 31)) {
+    // 16-bit operands, K a multiple of 64 and enough tiles of 256 x 256 to go round: the kernel whose operands reach LDS
+    // without passing through registers (any of the four layouts).  Offsets inside an operand's tile are 32-bit there:
+    // 256 rows of an operand with k innermost, all K rows of one with m or n innermost.
+    auto fits32 = [&](bool kcont, int64_t ld) { return (kcont ? ld * 2 * 256 : ld * 2 * K) < (int64_t(1) << 31); };
+    if (fast && esz == 2 && K % 64 == 0 && !getenv("MJT_GEMM_NO_DMA") && fits32(a_kcont, lda) && fits32(b_kcont, ldb)) {
         const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
         const int64_t tm = (M + 255) / 256, tn = (N + 255) / 256;
         const double edge = ((double)M * N) / ((double)tm * 256 * tn * 256);
@@ -72,13 +73,15 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
             const int in = in_dtype == MJT_BFLOAT16 ? 0 : 1;
             const int out = out_dtype == MJT_BFLOAT16 ? 0 : out_dtype == MJT_FLOAT16 ? 1 : 2;
             std::ostringstream key;
-            key << "gemmd|" << in << out;
+            key << "gemmd|" << in << out << a_kcont << b_kcont;
             JitKernel* k = cached(key.str());
             if (!k) {
                 std::ostringstream name;
-                name << "mjt_gemm_mfma_" << mjt_dtype_name(in_dtype) << "_" << mjt_dtype_name(out_dtype) << "_256x256_nt_direct";
+                name << "mjt_gemm_mfma_" << mjt_dtype_name(in_dtype) << "_" << mjt_dtype_name(out_dtype) << "_256x256" << (a_kcont ? "_n" : "_t")
+                     << (b_kcont ? "t" : "n") << "_direct";
                 std::ostringstream src;
-                src << "#define ENTRY " << name.str() << "\n#define IN " << in << "\n#define OUT " << out << "\n";
+                src << "#define ENTRY " << name.str() << "\n#define IN " << in << "\n#define OUT " << out << "\n#define A_KCONT " << (a_kcont ? 1 : 0)
+                    << "\n#define B_KCONT " << (b_kcont ? 1 : 0) << "\n";
                 src << embedded_source("gemm_dma.h") << "\n";
                 k = jit_get(src.str(), name.str());
                 remember(key.str(), k);

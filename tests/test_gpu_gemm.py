@@ -90,20 +90,21 @@ def test_gemm_mfma_layouts_and_edges(gpu, dt, ta, tb):
 
 
 @pytest.mark.parametrize("dt", ["bfloat16", "float16"])
-def test_gemm_direct_copy_kernel(gpu, dt, monkeypatch):
-    """a x b^T with 16-bit operands and K a multiple of 64 has a kernel of its own (operands go from memory to LDS
-    without passing through registers) once there are enough 256 x 256 tiles; here it is asked for by name so that
-    small shapes reach it too: tiles that hang over both edges, a single stage pair (K = 64), many stages, a
-    float32 result, a batch."""
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+def test_gemm_direct_copy_kernel(gpu, dt, ta, tb, monkeypatch):
+    """16-bit operands with K a multiple of 64 have a kernel of their own (operands go from memory to LDS without
+    passing through registers; an operand whose memory has m or n innermost is read from LDS with transposing
+    reads) once there are enough 256 x 256 tiles; here it is asked for by name so that small shapes reach it too:
+    all four layouts, tiles that hang over both edges, a single stage (K = 64), many stages, a float32 result, a batch."""
     lib = L.load()
     monkeypatch.setenv("MJT_GEMM_DMA", "1")
     for i, (M, K, N) in enumerate([(256, 64, 256), (512, 256, 256), (304, 128, 136), (1000, 192, 520), (8, 512, 8), (520, 2048, 264)]):
-        kern = _run(lib, dt, dt, M, K, N, 0, 1, seed=20 + i)
-        assert kern.endswith("_256x256_nt_direct"), kern
-    assert _run(lib, dt, "float32", 304, 128, 520, 0, 1, seed=30).endswith("_256x256_nt_direct")
-    assert _run(lib, dt, dt, 260, 64, 250, 0, 1, seed=31, batch=(3,)).endswith("_256x256_nt_direct")
+        kern = _run(lib, dt, dt, M, K, N, ta, tb, seed=20 + i)
+        assert kern.endswith("_direct"), kern
+    assert _run(lib, dt, "float32", 304, 128, 520, ta, tb, seed=30).endswith("_direct")
+    assert _run(lib, dt, dt, 264, 64, 248, ta, tb, seed=31, batch=(3,)).endswith("_direct")
     # K = 96 is no multiple of 64: the general kernel
-    assert not _run(lib, dt, dt, 256, 96, 256, 0, 1, seed=32).endswith("_direct")
+    assert not _run(lib, dt, dt, 256, 96, 256, ta, tb, seed=32).endswith("_direct")
 
 
 def test_gemm_k_tail_inside_a_chunk(gpu):
