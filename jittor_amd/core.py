@@ -8,6 +8,7 @@ ops/reindex_op.cc:20-91, ops/reindex_reduce_op.cc:26-73, ops/array_op.cc:54-80).
 Nothing executes until a Var is synchronised (lazy_execution,
 var_holder.cc:25-33); execution is in executor.py.
 """
+import math
 import numbers
 import weakref
 
@@ -543,9 +544,21 @@ def unary_clone(x):
     return unary(x, "cast", force_dtype=x.dtype, allow_forward=False)
 
 
+_scalar_vars = {}        # (type, value, sign) -> the host Var of a Python number: `x * 2.0` builds no new array each time
+
+
 def _as_var(v):
     if isinstance(v, Var):
         return v
+    tv = type(v)
+    if tv is float or tv is int or tv is bool:
+        key = (tv, v, math.copysign(1.0, v) if tv is float else 0)
+        got = _scalar_vars.get(key)
+        if got is None:
+            if len(_scalar_vars) >= 4096:
+                _scalar_vars.clear()
+            got = _scalar_vars[key] = array(v)
+        return got
     if isinstance(v, (numbers.Number, np.generic, list, tuple, np.ndarray, bool)):
         return array(v)
     raise TypeError("cannot convert %r to a Var" % type(v))
