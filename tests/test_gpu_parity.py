@@ -573,6 +573,10 @@ def test_conv_direct_small_shapes_and_fp32(gpu):
     dict(dt="float32", x=(12, 24, 7, 7), w=(40, 24, 3, 3), p=(1, 1, 1, 1, 1, 1)),                      # 49 pixels: padded rows, k ends inside a stage
     dict(dt="bfloat16", x=(3, 72, 9, 11), w=(40, 72, 3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16"),
     dict(dt="float32", x=(5, 40, 16, 16), w=(96, 40, 1, 1), p=(1, 1, 0, 0, 1, 1), plain=True, chunk=2),
+    # the product on the direct-copy kernel (asked for by name: these shapes have too few tiles to get it by themselves):
+    # weights shared across the batch, column matrices with the pixels innermost read with transposing reads
+    dict(dt="bfloat16", x=(3, 64, 15, 15), w=(96, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), dma=True),
+    dict(dt="float16", x=(4, 64, 16, 16), w=(96, 64, 1, 1), p=(1, 1, 0, 0, 1, 1), out="float16", plain=True, dma=True),
 ])
 def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
     """Shapes the MFMA kernel does not take and that are large enough to matter run as column matrices (one reindex)
@@ -587,6 +591,8 @@ def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
     out = case.get("out", "float32")
     if "chunk" in case:
         monkeypatch.setenv("MJT_CONV_GEMM_CHUNK", str(case["chunk"]))
+    if case.get("dma"):
+        monkeypatch.setenv("MJT_GEMM_DMA", "1")
     got, kern = _conv_call(xb, wb, case["p"], out_dtype=out, in_dtype=dt)
     assert kern == ("conv_as_gemm" if case.get("plain") else "conv_as_reindex_gemm"), kern
     got = widen[out](got)
