@@ -107,6 +107,24 @@ def test_gemm_direct_copy_kernel(gpu, dt, ta, tb, monkeypatch):
     assert not _run(lib, dt, dt, 256, 96, 256, ta, tb, seed=32).endswith("_direct")
 
 
+def test_gemm_direct_copy_kernel_random_shapes(gpu, monkeypatch):
+    """Seeded sweep over shapes, layouts, result types and batches for the direct-copy kernel: M and N anywhere
+    between 1 and 700 (tiles cut on every side, operands whose last rows or columns end at the tensor's end),
+    K a multiple of 64 up to 1024."""
+    lib = L.load()
+    monkeypatch.setenv("MJT_GEMM_DMA", "1")
+    rng = np.random.default_rng(2024)
+    for i in range(24):
+        M, N = int(rng.integers(1, 88)) * 8, int(rng.integers(1, 88)) * 8       # rows of 16-byte multiples in every layout
+        K = 64 * int(rng.integers(1, 17))
+        ta, tb = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        dt = ("bfloat16", "float16")[i % 2]
+        odt = (dt, "float32")[int(rng.integers(0, 2))]
+        batch = () if i % 3 else (int(rng.integers(2, 4)),)
+        kern = _run(lib, dt, odt, M, K, N, ta, tb, seed=100 + i, batch=batch)
+        assert kern.endswith("_direct"), (kern, M, K, N, ta, tb)
+
+
 def test_gemm_k_tail_inside_a_chunk(gpu):
     """k-innermost operands whose K is no multiple of the chunk: the row length (leading dimension) is what has to
     be aligned, and a product's operands are dense, so this route is only reachable with a K that is aligned;

@@ -550,6 +550,43 @@ def test_conv_mfma_matches_oracle(gpu, case):
     assert np.abs(got2 - ref).max() <= 1e-4 * scale
 
 
+def test_conv_mfma_random_geometries(gpu):
+    """Seeded sweep over geometries for the MFMA kernel (channel counts, map sizes with even widths, taps, stride,
+    padding, dilation, 16-bit and float32 results): every case against a float64 sum of shifted products, per
+    element within 1e-4 of the sum of its terms' magnitudes (plus the result type's own rounding)."""
+    rng = np.random.default_rng(77)
+    taken = 0
+    for i in range(14):
+        C, K = int(rng.choice([32, 64, 96, 128])), int(rng.choice([64, 128, 192]))
+        R, S = int(rng.choice([1, 2, 3])), int(rng.choice([1, 3, 5]))
+        sh, sw = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))
+        dh, dw_ = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))
+        ph, pw = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+        H, W = int(rng.integers(4, 30)), 2 * int(rng.integers(3, 40))
+        N = int(rng.integers(1, 4))
+        if H + 2 * ph < dh * (R - 1) + 1 or W + 2 * pw < dw_ * (S - 1) + 1:
+            continue
+        out = ("float32", "bfloat16")[i % 2]
+        xb = O.f32_to_bf16_bits(rng.standard_normal((N, C, H, W)).astype(np.float32))
+        wb = O.f32_to_bf16_bits((rng.standard_normal((K, C, R, S)) * 0.1).astype(np.float32))
+        got, kern = _conv_call(xb, wb, (sh, sw, ph, pw, dh, dw_), out_dtype=out)
+        taken += kern.startswith("mjt_conv_mfma_bf16")
+        got = O.BF16(got).to_f32().astype(np.float64) if out == "bfloat16" else got.astype(np.float64)
+        xf, wf = O.BF16(xb).to_f32().astype(np.float64), O.BF16(wb).to_f32().astype(np.float64)
+        oh, ow = got.shape[2:]
+        xp = np.pad(xf, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+        ref, terms = np.zeros(got.shape), np.zeros(got.shape)
+        for r in range(R):
+            for s_ in range(S):
+                patch = xp[:, :, r * dh:r * dh + (oh - 1) * sh + 1:sh, s_ * dw_:s_ * dw_ + (ow - 1) * sw + 1:sw]
+                ref += np.einsum("nchw,kc->nkhw", patch, wf[:, :, r, s_])
+                terms += np.einsum("nchw,kc->nkhw", np.abs(patch), np.abs(wf[:, :, r, s_]))
+        bound = 1e-4 * terms + (np.abs(ref) * 2.0 ** -7 if out == "bfloat16" else 0.0) + 1e-30
+        assert (np.abs(got - ref) <= bound).all(), (kern, (N, C, H, W), (K, C, R, S), (sh, sw, ph, pw, dh, dw_),
+                                                    float((np.abs(got - ref) / bound).max()))
+    assert taken >= 8, taken          # most of the sweep runs on the MFMA kernel (the rest on the fallbacks, checked alike)
+
+
 def test_conv_direct_small_shapes_and_fp32(gpu):
     rng = np.random.default_rng(21)
     for xs, ws, st, pd, dl in [((2, 3, 9, 8), (4, 3, 3, 3), 1, 1, 1), ((2, 3, 9, 8), (4, 3, 3, 3), 2, 1, 1),
