@@ -18,8 +18,9 @@
 // weight ring), STAGE_DEPTH, WPS (waves per SIMD the register budget is for),
 // Y_BF16 (16-bit output in the operand type), IN_F16.
 //
-// Mapping.  v_mfma_f32_16x16x32_bf16 computes D[16 ko][16 px] += A[16 ko][32 c] *
-// B[32 c][16 px].  A workgroup of WPX*WKO waves owns 16*MT*WKO output channels x RPW
+// Mapping.  v_mfma_f32_16x16x32_bf16 computes D[16 px][16 ko] += A[16 px][32 c] *
+// B[32 c][16 ko]: the input fragment is the first operand, so that a lane ends up with
+// four consecutive pixels of one channel, which it stores as they are.  A workgroup of WPX*WKO waves owns 16*MT*WKO output channels x RPW
 // consecutive output rows of one image and walks them tile by tile (WPX*TRW rows
 // each), so that the number of workgroups can match the number of compute units
 // whatever the row count.  Within a tile wave (wko, wpx) owns 16*MT channels x TRW
@@ -474,7 +475,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                         // the next two passes
                         if constexpr (m == 0) mjt_lds_wait<(BULK ? 0 : NT_ - 1 - t + (P + 2 < PASSES ? 1 : 0))>(bfr[t]);
                         else if constexpr (t == 0) mjt_lds_wait<(P + 1 < PASSES ? 1 : 0) + (P + 2 < PASSES ? 1 : 0)>(afr[P % 3]);
-                        mjt_mfma(acc[m][t], afr[P % 3], bfr[t]);
+                        mjt_mfma(acc[m][t], bfr[t], afr[P % 3]);
                         if constexpr (m + 1 == MT && st + 1 < STEPS) mjt_ds_read<mjt_frag_off(st + 1)>(bfr[t], baddr[t]);
                         if constexpr (m == 0 && t == 0) issue_loads();
                         commit_stages(mjt_ic<m * NT_ + t + 1>());
@@ -491,7 +492,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
             }
         }
 
-        // epilogue: lane holds D[ko = 4*(lane/16)+i][px = lane%16] of each tile
+        // epilogue: lane holds D[px = 4*(lane/16)+i][ko = lane%16] of each tile
         // The compiler takes a spelled-out MFMA for finished the moment it is issued.  Give the last ones the
         // time to read their operands and write their results, and tie the registers to a point behind that:
         // the operands stay allocated up to here, and nothing reads an accumulator before.
@@ -501,68 +502,56 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         mjt_keep(afr[2]);
         mjt_static_for<0, NT_>([&](auto tc) { mjt_keep(bfr[decltype(tc)::v]); });
         mjt_static_for<0, MT * NT_>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / NT_][decltype(ic)::v % NT_]); });
-#if OW_ % 4 == 0
-        // The four lanes of a quad (4 pixels x 4 channels) transpose among themselves, after which lane j
-        // of the quad owns channel 4*(lane/16)+j for the quad's 4 consecutive pixels: one 16-byte (or
-        // 8-byte bfloat16) store instead of four scattered 4-byte stores.  Four pixels never straddle
-        // an output row because OW is a multiple of 4.
-        const int qj = lane & 3;
+        // (the lane's coordinates are taken from a copy of the lane number made here: what is worked out from it cannot
+        // be moved in front of the loop, where it would sit in registers the loop needs)
+        int lane_e = lane;
+        asm volatile("" : "+v"(lane_e));
+        const int l16_e = lane_e & 15, lg_e = lane_e >> 4;
 #pragma unroll
         for (int t = 0; t < NT_; t++) {
-            const int q0 = t * 16 + (l16 & ~3);
+#if OW_ % 4 == 0
+            // 16 bytes (8 as a 16-bit type) per lane: four pixels never straddle an output row because OW is a multiple
+            // of 4.  The four 16-lane rows of a register make up the 64 bytes of a pixel tile, for 16 channels.
+            // (Regrouping registers so that an instruction writes 256-byte runs of 4 channels, by quad transposes
+            // or row swaps, was no faster.)
+            const int q0 = t * 16 + lg_e * 4;
             const int r = q0 / OW_, col = q0 - r * OW_;
             const int orow = r0 + wpx * TRW_ + r;
-            const bool ok = q0 < TRW_ * OW_ && orow < row_lim;
+            if (q0 < TRW_ * OW_ && orow < row_lim) {
 #pragma unroll
-            for (int m = 0; m < MT; m++) {
-                const mjt_f32x4 v = acc[m][t];
-                // lane ^ 1: rows (0,1) and (2,3) trade pixels
-                const float g0 = mjt_xor1f(b0 ? v[0] : v[1]), g1 = mjt_xor1f(b0 ? v[2] : v[3]);
-                const float a0 = b0 ? g0 : v[0], a1 = b0 ? v[1] : g0;     // row (j & 1):     pixel pair of this lane pair
-                const float a2 = b0 ? g1 : v[2], a3 = b0 ? v[3] : g1;     // row (j & 1) + 2
-                // lane ^ 2: row pairs trade pixel pairs
-                const float h0 = mjt_xor2f(b1 ? a0 : a2), h1 = mjt_xor2f(b1 ? a1 : a3);
-                mjt_f32x4 y4;                                             // row j, pixels 0..3 of the quad
-                y4[0] = b1 ? h0 : a0;
-                y4[1] = b1 ? h1 : a1;
-                y4[2] = b1 ? a2 : h0;
-                y4[3] = b1 ? a3 : h1;
-                if (ok) {
-                    const int ko = ko_base + m * 16 + lg * 4 + qj;
-                    const size_t o = (((size_t)n * YK_ + ko) * OH_ + orow) * OW_ + col;
+                for (int m = 0; m < MT; m++) {
+                    const mjt_f32x4 v = acc[m][t];
+                    const size_t o = (((size_t)n * YK_ + ko_base + m * 16 + l16_e) * OH_ + orow) * OW_ + col;
 #if Y_BF16
                     mjt_u32x2 pk;
-                    pk[0] = mjt_narrow2(y4[0], y4[1]);
-                    pk[1] = mjt_narrow2(y4[2], y4[3]);
+                    pk[0] = mjt_narrow2(v[0], v[1]);
+                    pk[1] = mjt_narrow2(v[2], v[3]);
                     *(mjt_u32x2*)((unsigned short*)p.a[2] + o) = pk;
 #else
-                    *(mjt_f32x4*)((float*)p.a[2] + o) = y4;
+                    *(mjt_f32x4*)((float*)p.a[2] + o) = v;
 #endif
                 }
             }
-        }
 #else
 #pragma unroll
-        for (int t = 0; t < NT_; t++) {
-            const int q = t * 16 + l16;
-            const int r = q / OW_, col = q - r * OW_;
-            const int orow = r0 + wpx * TRW_ + r;
-            if (q < TRW_ * OW_ && orow < row_lim) {
+            for (int i = 0; i < 4; i++) {
+                const int q = t * 16 + lg_e * 4 + i;
+                const int r = q / OW_, col = q - r * OW_;
+                const int orow = r0 + wpx * TRW_ + r;
+                if (q < TRW_ * OW_ && orow < row_lim) {
 #pragma unroll
-                for (int m = 0; m < MT; m++)
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int ko = ko_base + m * 16 + lg * 4 + i;
-                        const size_t o = (((size_t)n * YK_ + ko) * OH_ + orow) * OW_ + col;
+                    for (int m = 0; m < MT; m++) {
+                        const size_t o = (((size_t)n * YK_ + ko_base + m * 16 + l16_e) * OH_ + orow) * OW_ + col;
 #if Y_BF16
                         ((unsigned short*)p.a[2])[o] = (unsigned short)mjt_narrow2(acc[m][t][i], 0.0f);
 #else
                         ((float*)p.a[2])[o] = acc[m][t][i];
 #endif
                     }
+                }
             }
-        }
 #endif
+        }
     };
     // tiles of this workgroup: full tiles while they start inside the row range, then the short one
     int nfull = (row_end - row_begin + TR - 1) / TR;
