@@ -282,6 +282,21 @@ int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* 
 int mjt_conv2d_meta_grouped(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y,
                             const mjt_conv_params* p, int groups);
 
+/* Input gradient of the same convolution (the pattern reindex_reduce.add of
+ * broadcast(dy) * broadcast(w) back into x's shape that jt.grad builds;
+ * opt/tuner/conv_tuner.cc:375-397 relays it to a backward-x library op,
+ * extern/cuda/cudnn/ops/cudnn_conv_backward_x_op.cc):
+ *   dx[n,c,h,w] = sum over (k,r,s) with h = oh*sh-ph+r*dh, w = ow*sw-pw+s*dw of dy[n,k,oh,ow] * w[k,c,r,s]
+ * dy [N,K,OH,OW] and w [K,C,R,S] bfloat16, float16 or float32 (same dtype), dx
+ * [N,C,H,W] float32 or their dtype; p is the forward convolution's.  Runs on
+ * the forward kernels: with transposed, flipped weights for stride 1; for a
+ * stride (no dilation, H and W multiples of it) as one stride-1 convolution
+ * per stride phase on that phase's taps, so that no product has a zero
+ * factor; otherwise on dy spread out with zeros.  Padding beyond the taps'
+ * reach (p > d*(R-1)) is rejected. */
+int mjt_conv2d_meta_dgrad(const mjt_tensor* dy, const mjt_tensor* w, const mjt_tensor* dx,
+                          const mjt_conv_params* p);
+
 /* Weight gradient of the same convolution (the pattern
  * reindex(x) * broadcast(dy) -> reduce.add over (n, oh, ow) that jt.grad builds;
  * opt/tuner/conv_tuner.cc:375-397 relays it to a backward-w library op,

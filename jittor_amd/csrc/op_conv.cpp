@@ -23,8 +23,10 @@ void* g_wpack = nullptr;
 size_t g_wpack_bytes = 0;
 void* g_wgrad_part = nullptr;      // per-slice partial weight gradients (its own buffer: the reduce that folds them uses the arena)
 size_t g_wgrad_bytes = 0;
-void* g_conv_scratch[2] = {nullptr, nullptr};   // column matrices of a chunk of images; float32 copy of a bfloat16 result
-size_t g_conv_scratch_bytes[2] = {0, 0};
+// column matrices of a chunk of images; float32 copy of a bfloat16 result; for the input gradient: rearranged weights,
+// and dy spread out with zeros or the results of the stride phases
+void* g_conv_scratch[4] = {nullptr, nullptr, nullptr, nullptr};
+size_t g_conv_scratch_bytes[4] = {0, 0, 0, 0};
 
 void forget() {
     std::lock_guard<std::mutex> lock(g_mu);
@@ -37,8 +39,12 @@ void forget() {
         for (void* b : g_conv_scratch)
             if (b) (void)hipFree(b);
     }
-    g_wpack = g_wgrad_part = g_conv_scratch[0] = g_conv_scratch[1] = nullptr;
-    g_wpack_bytes = g_wgrad_bytes = g_conv_scratch_bytes[0] = g_conv_scratch_bytes[1] = 0;
+    g_wpack = g_wgrad_part = nullptr;
+    g_wpack_bytes = g_wgrad_bytes = 0;
+    for (int i = 0; i < 4; i++) {
+        g_conv_scratch[i] = nullptr;
+        g_conv_scratch_bytes[i] = 0;
+    }
 }
 const bool g_registered = (at_shutdown(&forget), true);
 
@@ -66,7 +72,10 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
                  int64_t lda, int64_t ldb, int64_t ldc, int64_t sa, int64_t sb, int64_t sc, int64_t batch, bool a_kcont,
                  bool b_kcont);
 
-void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p, int64_t G) {
+// free_extent: y's rows and columns are taken as they are instead of checked against the extents that stride, padding and
+// taps give (output (oh, ow) reads x around (oh*sh - ph, ow*sw - pw) whatever oh and ow; outside the image x is 0): what the
+// stride phases of an input gradient need, whose zero margins differ between the two ends of an axis.
+void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p, int64_t G, bool free_extent = false) {
     require_init();
     check_tensor(x, "conv x");
     check_tensor(w, "conv w");
@@ -84,8 +93,8 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     MJT_CHECK(K % G == 0, "conv: " << K << " output channels do not divide into " << G << " groups");
     MJT_CHECK(p->stride_h >= 1 && p->stride_w >= 1 && p->dil_h >= 1 && p->dil_w >= 1 && p->pad_h >= 0 && p->pad_w >= 0,
               "conv: bad stride / padding / dilation");
-    const int64_t OH = (H + 2 * p->pad_h - p->dil_h * (R - 1) - 1) / p->stride_h + 1;
-    const int64_t OW = (W + 2 * p->pad_w - p->dil_w * (S - 1) - 1) / p->stride_w + 1;
+    const int64_t OH = free_extent ? y->shape[2] : (H + 2 * p->pad_h - p->dil_h * (R - 1) - 1) / p->stride_h + 1;
+    const int64_t OW = free_extent ? y->shape[3] : (W + 2 * p->pad_w - p->dil_w * (S - 1) - 1) / p->stride_w + 1;
     MJT_CHECK(OH >= 1 && OW >= 1, "conv: empty output");
     MJT_CHECK(y->shape[0] == N && y->shape[1] == K && y->shape[2] == OH && y->shape[3] == OW,
               "conv: y shape " << shape_str(y) << " != [" << N << "," << K << "," << OH << "," << OW << "]");
@@ -249,7 +258,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         P < (int64_t(1) << 31) && CRS < (int64_t(1) << 31) && matmul_available()) {
         const int64_t esz = dtype_size(x->dtype);
         const int64_t Ppad = (P * esz + 15) / 16 * 16 / esz;
-        const bool plain = R == 1 && S == 1 && p->stride_h == 1 && p->stride_w == 1 && p->pad_h == 0 && p->pad_w == 0 && Ppad == P;
+        const bool plain = R == 1 && S == 1 && p->stride_h == 1 && p->stride_w == 1 && p->pad_h == 0 && p->pad_w == 0 && Ppad == P && OH == H && OW == W;
         int64_t chunk = (int64_t(1) << 30) / (CRS * Ppad * esz);
         if (const char* e = getenv("MJT_CONV_GEMM_CHUNK"))      // images per chunk, for tests of the chunk loop
             if (atoi(e) >= 1) chunk = atoi(e);
@@ -497,6 +506,123 @@ extern "C" int mjt_conv2d_meta_wgrad(const mjt_tensor* x, const mjt_tensor* dy, 
 extern "C" int mjt_conv2d_meta_wgrad_grouped(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw, const mjt_conv_params* p,
                                              int groups) {
     return mjt::guarded([&] { mjt::conv_wgrad_impl(x, dy, dw, p, groups, true); });
+}
+
+namespace mjt {
+// Input gradient of the convolution y = conv(x, w): dx[n,c,h,w] = sum over (k, r, s) of dy[n,k,oh,ow] * w[k,c,r,s] with
+// h = oh*sh - ph + r*dh, w = ow*sw - pw + s*dw.  It is itself a convolution of dy, run on the forward kernels:
+//   * stride 1: with the weights transposed and their taps flipped, padding d*(R-1) - p;
+//   * a stride without dilation, H and W multiples of it: one stride-1 convolution per stride phase.  The rows
+//     h = sh*i + a of dx see only the taps r = r_a + sh*u (r_a = (a + ph) % sh, u = 0 .. U_a - 1) and
+//     dx[sh*i + a] = sum_u dy[i + d_a - u] * w[r_a + sh*u] with d_a = (a + ph) / sh: a convolution of dy with U_a taps
+//     (flipped) and left padding U_a - 1 - d_a, likewise for columns.  No product has a zero factor; the phases
+//     are written one after the other and interleaved by one reindex;
+//   * otherwise: dy with sh-1 (sw-1) zeros between its rows (columns), then as for stride 1.
+void conv_dgrad_impl(const mjt_tensor* dy, const mjt_tensor* w, const mjt_tensor* dx, const mjt_conv_params* p) {
+    require_init();
+    check_tensor(dy, "conv dgrad dy");
+    check_tensor(w, "conv dgrad w");
+    check_tensor(dx, "conv dgrad dx");
+    MJT_CHECK(p, "conv dgrad: null parameters");
+    MJT_CHECK(dy->ndim == 4 && w->ndim == 4 && dx->ndim == 4, "conv dgrad: dy, w and dx must have rank 4");
+    MJT_CHECK(dy->dtype == w->dtype && (dy->dtype == MJT_BFLOAT16 || dy->dtype == MJT_FLOAT16 || dy->dtype == MJT_FLOAT32),
+              "conv dgrad: dy and w must both be bfloat16, float16 or float32");
+    MJT_CHECK(dx->dtype == MJT_FLOAT32 || dx->dtype == dy->dtype, "conv dgrad: dx must be float32 or the operands' dtype");
+    const int64_t N = dx->shape[0], C = dx->shape[1], H = dx->shape[2], W = dx->shape[3];
+    const int64_t K = w->shape[0], R = w->shape[2], S = w->shape[3];
+    const int64_t sh = p->stride_h, sw = p->stride_w, ph = p->pad_h, pw = p->pad_w, dh = p->dil_h, dw = p->dil_w;
+    MJT_CHECK(sh >= 1 && sw >= 1 && dh >= 1 && dw >= 1 && ph >= 0 && pw >= 0, "conv dgrad: bad stride / padding / dilation");
+    MJT_CHECK(w->shape[1] == C, "conv dgrad: weight channels " << w->shape[1] << " != dx channels " << C);
+    const int64_t OH = (H + 2 * ph - dh * (R - 1) - 1) / sh + 1, OW = (W + 2 * pw - dw * (S - 1) - 1) / sw + 1;
+    MJT_CHECK(dy->shape[0] == N && dy->shape[1] == K && dy->shape[2] == OH && dy->shape[3] == OW,
+              "conv dgrad: dy shape " << shape_str(dy) << " != [" << N << "," << K << "," << OH << "," << OW << "]");
+    MJT_CHECK(dh * (R - 1) >= ph && dw * (S - 1) >= pw, "conv dgrad: padding beyond the taps' reach is not supported");
+    if (N == 0 || C == 0) return;
+    const int64_t esz = dtype_size(w->dtype);
+    auto view = [](void* ptr, int dtype, std::initializer_list<int64_t> shape) {
+        mjt_tensor t;
+        memset(&t, 0, sizeof(t));
+        t.ptr = ptr;
+        t.dtype = dtype;
+        for (int64_t e : shape) t.shape[t.ndim++] = e;
+        return t;
+    };
+    auto reindex = [&](const mjt_tensor& src, const mjt_tensor& dst, std::initializer_list<std::string> idx, std::initializer_list<std::string> over) {
+        std::vector<const char*> ip, op;
+        for (const std::string& e : idx) ip.push_back(e.c_str());
+        for (const std::string& e : over) op.push_back(e.c_str());
+        if (mjt_reindex(&src, &dst, (int)ip.size(), ip.data(), 0.0, (int)op.size(), op.data(), 0, nullptr) != MJT_OK)
+            MJT_FAIL(MJT_ERR_DEVICE, "conv dgrad: a rearrangement failed: " << mjt_last_error());
+    };
+    auto str = [](int64_t v) { return std::to_string(v); };
+    void* wbuf = conv_scratch(2, (size_t)(numel(w) * esz));
+
+    // the taps of each stride phase along one axis: first tap, number of taps, left padding (-1: not expressible)
+    struct Phase { int64_t first, taps, pad; };
+    auto phases = [](int64_t stride, int64_t pad, int64_t taps) {
+        std::vector<Phase> v;
+        for (int64_t a = 0; a < stride; a++) {
+            Phase q;
+            q.first = (a + pad) % stride;
+            q.taps = q.first < taps ? (taps - q.first + stride - 1) / stride : 0;
+            q.pad = q.taps ? q.taps - 1 - (a + pad) / stride : 0;
+            v.push_back(q);
+        }
+        return v;
+    };
+    bool by_phase = (sh > 1 || sw > 1) && dh == 1 && dw == 1 && H % sh == 0 && W % sw == 0 && !getenv("MJT_CONV_DGRAD_NO_PHASES");
+    std::vector<Phase> rows, cols;
+    if (by_phase) {
+        rows = phases(sh, ph, R);
+        cols = phases(sw, pw, S);
+        for (const Phase& q : rows) by_phase = by_phase && q.pad >= 0;
+        for (const Phase& q : cols) by_phase = by_phase && q.pad >= 0;
+    }
+    if (by_phase) {
+        const int64_t Hs = H / sh, Ws = W / sw, dsz = dtype_size(dx->dtype);
+        const int64_t plane = N * C * Hs * Ws;
+        char* part = (char*)conv_scratch(3, (size_t)(sh * sw * plane * dsz));
+        const mjt_conv_params unit = {1, 1, 0, 0, 1, 1};
+        std::string kernels;
+        for (int64_t a = 0; a < sh; a++)
+            for (int64_t b = 0; b < sw; b++) {
+                const Phase &qr = rows[a], &qc = cols[b];
+                mjt_tensor ty = view(part + (a * sw + b) * plane * dsz, dx->dtype, {N, C, Hs, Ws});
+                if (qr.taps == 0 || qc.taps == 0) {                 // no tap reaches these positions: zeros
+                    reindex(*dy, ty, {"0", "0", "0", "0"}, {"1"});
+                    continue;
+                }
+                // w [K,C,R,S] -> [C,K,U,V]: the phase's taps, flipped
+                mjt_tensor tw = view(wbuf, w->dtype, {C, K, qr.taps, qc.taps});
+                reindex(*w, tw, {"i1", "i0", str(qr.first) + "+" + str(sh) + "*(" + str(qr.taps - 1) + "-i2)",
+                                 str(qc.first) + "+" + str(sw) + "*(" + str(qc.taps - 1) + "-i3)"}, {});
+                mjt_conv_params q = unit;
+                q.pad_h = (int32_t)qr.pad;
+                q.pad_w = (int32_t)qc.pad;
+                conv_impl(dy, &tw, &ty, &q, 1, true);
+                if (kernels.empty()) kernels = mjt_last_kernel();
+            }
+        mjt_tensor tp = view(part, dx->dtype, {sh * sw, N, C, Hs, Ws});
+        reindex(tp, *dx, {"i2%" + str(sh) + "*" + str(sw) + "+i3%" + str(sw), "i0", "i1", "i2/" + str(sh), "i3/" + str(sw)}, {});
+        set_last_kernel(("conv_dgrad_phases:" + kernels).c_str());
+        return;
+    }
+    mjt_tensor tw = view(wbuf, w->dtype, {C, K, R, S});
+    reindex(*w, tw, {"i1", "i0", str(R - 1) + "-i2", str(S - 1) + "-i3"}, {});
+    const mjt_conv_params q = {1, 1, (int32_t)(dh * (R - 1) - ph), (int32_t)(dw * (S - 1) - pw), (int32_t)dh, (int32_t)dw};
+    if (sh == 1 && sw == 1) {
+        conv_impl(dy, &tw, dx, &q, 1);
+        return;
+    }
+    const int64_t ZH = H + 2 * ph - dh * (R - 1), ZW = W + 2 * pw - dw * (S - 1);
+    mjt_tensor tz = view(conv_scratch(3, (size_t)(N * K * ZH * ZW * esz)), dy->dtype, {N, K, ZH, ZW});
+    reindex(*dy, tz, {"i0", "i1", "i2/" + str(sh), "i3/" + str(sw)}, {"i2%" + str(sh) + "!=0", "i3%" + str(sw) + "!=0"});
+    conv_impl(&tz, &tw, dx, &q, 1);
+}
+}  // namespace mjt
+
+extern "C" int mjt_conv2d_meta_dgrad(const mjt_tensor* dy, const mjt_tensor* w, const mjt_tensor* dx, const mjt_conv_params* p) {
+    return mjt::guarded([&] { mjt::conv_dgrad_impl(dy, w, dx, p); });
 }
 
 extern "C" int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p) {

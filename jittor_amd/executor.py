@@ -816,6 +816,13 @@ def _run_single(op):
         sh, sw, ph, pw, dh, dw = op.params
         K, C, R, S = w.shape
         G = op.groups
+        if G == 1:
+            # the library's own entry: transposed, flipped weights for stride 1, one convolution per stride phase otherwise
+            td, tw = _tensor_of(dy), _tensor_of(w)
+            tx = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+            p = _lib.ConvParams(sh, sw, ph, pw, dh, dw)
+            _lib.check(lib.mjt_conv2d_meta_dgrad(ctypes.byref(td), ctypes.byref(tw), ctypes.byref(tx), ctypes.byref(p)))
+            return
         with core.no_grad():
             if G > 1:
                 # w [G*Kg, Cg, R, S] -> [G*Cg, Kg, R, S]: transposed within each group, taps flipped

@@ -587,6 +587,77 @@ def test_conv_mfma_random_geometries(gpu):
     assert taken >= 8, taken          # most of the sweep runs on the MFMA kernel (the rest on the fallbacks, checked alike)
 
 
+def _dgrad_reference(dy, w, H, W, params):
+    """The definition, in float64: every product dy[n,k,oh,ow] * w[k,c,r,s] is added at the input position the forward
+    window read (also returns the sum of the products' magnitudes, for the bound)."""
+    sh, sw, ph, pw, dh, dw_ = params
+    N, K, OH, OW = dy.shape
+    C, R, S = w.shape[1:]
+    dx, mag = np.zeros((N, C, H + 2 * ph, W + 2 * pw)), np.zeros((N, C, H + 2 * ph, W + 2 * pw))
+    for r in range(R):
+        for s_ in range(S):
+            rows, cols = slice(r * dh, r * dh + (OH - 1) * sh + 1, sh), slice(s_ * dw_, s_ * dw_ + (OW - 1) * sw + 1, sw)
+            dx[:, :, rows, cols] += np.einsum("nkhw,kc->nchw", dy, w[:, :, r, s_])
+            mag[:, :, rows, cols] += np.einsum("nkhw,kc->nchw", np.abs(dy), np.abs(w[:, :, r, s_]))
+    return dx[:, :, ph:ph + H, pw:pw + W], mag[:, :, ph:ph + H, pw:pw + W]
+
+
+@pytest.mark.parametrize("case", [
+    # x shape,         w shape,          (sh, sw, ph, pw, dh, dw), dtype,     result,    by phases
+    ((2, 8, 10, 12), (6, 8, 3, 3), (1, 1, 1, 1, 1, 1), "float32", "float32", False),
+    ((2, 8, 10, 12), (6, 8, 3, 3), (2, 2, 1, 1, 1, 1), "float32", "float32", True),
+    ((2, 8, 10, 12), (6, 8, 1, 1), (2, 2, 0, 0, 1, 1), "float32", "float32", True),      # phases no tap reaches: zeros
+    ((1, 4, 12, 12), (5, 4, 5, 5), (2, 2, 2, 2, 1, 1), "float32", "float32", True),
+    ((1, 4, 12, 9), (5, 4, 3, 3), (2, 3, 1, 0, 1, 1), "float32", "float32", True),
+    ((1, 4, 12, 12), (5, 4, 5, 3), (3, 2, 2, 1, 1, 1), "float32", "float32", True),
+    ((1, 4, 12, 12), (5, 4, 3, 2), (3, 2, 1, 1, 1, 1), "float32", "float32", False),     # a phase that starts past dy's first row
+    ((1, 4, 13, 12), (5, 4, 3, 3), (2, 2, 1, 1, 1, 1), "float32", "float32", False),     # 13 rows: dy spread out with zeros
+    ((1, 4, 12, 12), (5, 4, 3, 3), (2, 2, 2, 2, 2, 2), "float32", "float32", False),     # dilation: likewise
+    ((2, 64, 28, 28), (64, 64, 3, 3), (2, 2, 1, 1, 1, 1), "bfloat16", "bfloat16", True), # each phase on the MFMA kernel
+    ((2, 64, 28, 28), (128, 64, 3, 3), (2, 2, 1, 1, 1, 1), "float16", "float32", True),
+    ((2, 64, 28, 28), (64, 64, 3, 3), (1, 1, 1, 1, 1, 1), "bfloat16", "float32", False),
+], ids=lambda c: "x%s_w%s_p%s_%s" % ("x".join(map(str, c[0])), "x".join(map(str, c[1])), "".join(map(str, c[2])), c[3]))
+def test_conv_input_gradient_entry(gpu, case):
+    """mjt_conv2d_meta_dgrad against the definition of the gradient in float64 (per element within 1e-4 of the sum of
+    its terms' magnitudes, plus the result type's rounding), and for float32 against the oracle's gradient graph."""
+    xshape, wshape, params, dtype, out_dtype, phased = case
+    sh, sw, ph, pw, dh, dw_ = params
+    N, C, H, W = xshape
+    K, _, R, S = wshape
+    OH, OW = (H + 2 * ph - dh * (R - 1) - 1) // sh + 1, (W + 2 * pw - dw_ * (S - 1) - 1) // sw + 1
+    rng = np.random.default_rng(5)
+    dyf = rng.standard_normal((N, K, OH, OW)).astype(np.float32)
+    wf = (rng.standard_normal(wshape) * 0.2).astype(np.float32)
+    if dtype == "bfloat16":
+        dyb, wb = O.f32_to_bf16_bits(dyf), O.f32_to_bf16_bits(wf)
+        dyf, wf = O.BF16(dyb).to_f32(), O.BF16(wb).to_f32()
+    elif dtype == "float16":
+        dyb, wb = dyf.astype(np.float16), wf.astype(np.float16)
+        dyf, wf = dyb.astype(np.float32), wb.astype(np.float32)
+    else:
+        dyb, wb = dyf, wf
+    dy, w = jt.from_storage(np.ascontiguousarray(dyb), dtype), jt.from_storage(np.ascontiguousarray(wb), dtype)
+    dx = jt.zeros(list(xshape), out_dtype)
+    td, tw = L.tensor(dy.raw_ptr(), dtype, dy.shape), L.tensor(w.raw_ptr(), dtype, w.shape)
+    tx = L.tensor(dx.raw_ptr(), out_dtype, dx.shape)
+    p = L.ConvParams(*params)
+    L.check(L.load().mjt_conv2d_meta_dgrad(ctypes.byref(td), ctypes.byref(tw), ctypes.byref(tx), ctypes.byref(p)))
+    kern = L.last_kernel()
+    assert kern.startswith("conv_dgrad_phases:") == phased, kern
+    if dtype != "float32" and phased:
+        assert "mjt_conv_mfma" in kern, kern
+    raw = L.d2h(dx.raw_ptr(), dx.shape, L.NP_STORAGE[out_dtype])
+    got = (O.BF16(raw).to_f32() if out_dtype == "bfloat16" else raw).astype(np.float64)
+    ref, mag = _dgrad_reference(dyf.astype(np.float64), wf.astype(np.float64), H, W, params)
+    rounding = {"float32": 0.0, "bfloat16": 2.0 ** -7, "float16": 2.0 ** -10}[out_dtype]
+    bound = 1e-4 * mag + np.abs(ref) * rounding + 1e-30
+    assert (np.abs(got - ref) <= bound).all(), (kern, float((np.abs(got - ref) / bound).max()))
+    # the oracle's restatement of the gradient graph jt.grad builds (sequential float32 sums; small cases only)
+    if dtype == "float32":
+        odx, _ = O.conv_meta_grouped_grads(np.zeros(xshape, np.float32), wf, dyf, 1, (sh, sw), (ph, pw), (dh, dw_))
+        assert (np.abs(got - odx.astype(np.float64)) <= bound).all()
+
+
 def test_conv_direct_small_shapes_and_fp32(gpu):
     rng = np.random.default_rng(21)
     for xs, ws, st, pd, dl in [((2, 3, 9, 8), (4, 3, 3, 3), 1, 1, 1), ((2, 3, 9, 8), (4, 3, 3, 3), 2, 1, 1),

@@ -496,6 +496,34 @@ def test_shutdown_forgets_kernels_and_rebinding_compiles_again(compile_only, mon
     assert calls()[0] >= first + 3                           # compiled again, not taken from a stale table
 
 
+def test_conv_input_gradient_entry_validates_and_picks_its_path(compile_only):
+    """mjt_conv2d_meta_dgrad without a device: argument checks, and which of its three forms a geometry takes (one
+    convolution per stride phase, transposed flipped weights for stride 1, dy spread out with zeros otherwise)."""
+    lib = L.load()
+    P = 0x100000
+
+    def call(xs, ws, params, dys=None, dtype="bfloat16"):
+        N, C, H, W = xs
+        K, _, R, S = ws
+        sh, sw, ph, pw, dh, dw = params
+        oh, ow = (H + 2 * ph - dh * (R - 1) - 1) // sh + 1, (W + 2 * pw - dw * (S - 1) - 1) // sw + 1
+        dy, w = L.tensor(P, dtype, dys or (N, K, oh, ow)), L.tensor(P, dtype, ws)
+        dx, p = L.tensor(P, dtype, xs), L.ConvParams(*params)
+        return lib.mjt_conv2d_meta_dgrad(ctypes.byref(dy), ctypes.byref(w), ctypes.byref(dx), ctypes.byref(p))
+
+    assert call((2, 64, 28, 28), (64, 64, 3, 3), (2, 2, 1, 1, 1, 1)) == 0
+    assert L.last_kernel().startswith("conv_dgrad_phases:mjt_conv_mfma_bf16"), L.last_kernel()
+    assert call((2, 64, 28, 28), (64, 64, 3, 3), (1, 1, 1, 1, 1, 1)) == 0
+    assert L.last_kernel().startswith("mjt_conv_mfma_bf16"), L.last_kernel()
+    assert call((2, 64, 27, 28), (64, 64, 3, 3), (2, 2, 1, 1, 1, 1)) == 0          # 27 rows: no whole phases
+    assert not L.last_kernel().startswith("conv_dgrad_phases"), L.last_kernel()
+    assert call((2, 64, 28, 28), (64, 64, 3, 3), (2, 2, 1, 1, 1, 1), dys=(2, 64, 15, 14)) == -1
+    assert b"dy shape" in lib.mjt_last_error()
+    assert call((2, 64, 28, 28), (64, 32, 3, 3), (2, 2, 1, 1, 1, 1)) == -1         # weight channels != dx channels
+    assert call((2, 64, 28, 28), (64, 64, 1, 1), (1, 1, 1, 1, 1, 1)) == -1         # padding no tap reaches
+    assert b"padding" in lib.mjt_last_error()
+
+
 def test_conv_gradient_patterns_match_for_common_losses():
     """The two backward patterns are recognised whatever stands between the convolution and the loss: the loss may
     be the output itself (jt.grad seeds ones, test_conv_tuner.py:105-133), its sum or mean (for 16-bit outputs these
