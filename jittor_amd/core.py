@@ -17,6 +17,7 @@ import numpy as np
 from . import _lib
 from . import dtypes as dt
 from ._lib import MjtError
+from .flags import flags as _flags
 
 _next_id = [0]
 _grad_enabled = [True]
@@ -234,6 +235,8 @@ class Var:
         self.id = _new_id()
         self._name = None
         self._consumers = None   # ops that take this Var as an input (weakly)
+        # compile options: the flag's value at creation (var.cc:75)
+        self._compile_options = dict(_flags["compile_options"]) if _flags["compile_options"] else None
 
     # ---- properties ----
     @property
@@ -253,6 +256,24 @@ class Var:
 
     def numel(self):
         return self.num
+
+    @property
+    def compile_options(self):
+        """Options of the code generated for the op that makes this var: a dict name -> int
+        (var_holder.h:265-273; the fused group they end up in reads them through
+        FusedOp::get_loop_option, fused_op.cc:24-27,51-53).  nn.conv2d marks a grouped convolution with {"G": groups}
+        (nn.py:1278).  They are kept and handed on as the reference does; the kernels of this library take every
+        shape and layout decision from the operands themselves, so no option changes what runs."""
+        return dict(self._compile_options or {})
+
+    @compile_options.setter
+    def compile_options(self, options):
+        opts = {}
+        for k, v in dict(options).items():
+            if not isinstance(k, str) or isinstance(v, bool) or not isinstance(v, numbers.Integral):
+                raise TypeError("compile_options maps names to integers, got %r: %r" % (k, v))
+            opts[k] = int(v)
+        self._compile_options = opts or None
 
     def name(self, n=None):
         if n is None:

@@ -45,6 +45,7 @@ def conv2d(x, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
             "i4*%d-%d+i6*%d" % (stride[0], padding[0], dilation[0]),
             "i5*%d-%d+i7*%d" % (stride[1], padding[1], dilation[1]),
         ])
+        xx.compile_options = {"G": G}                      # nn.py:1278
         ww = weight.reindex([N, G, oc // G, CpG, oh, ow, Kh, Kw], ["i1*%d+i2" % (oc // G), "i3", "i6", "i7"])
         yy = xx * ww
         y = yy.reindex_reduce("add", [N, oc, oh, ow], ["i0", "i1*%d+i2" % (oc // G), "i4", "i5"])

@@ -524,6 +524,31 @@ def test_conv_input_gradient_entry_validates_and_picks_its_path(compile_only):
     assert b"padding" in lib.mjt_last_error()
 
 
+def test_compile_options_follow_the_flag_and_mark_grouped_convolutions():
+    """Var.compile_options (var_holder.h:265-273): a dict name -> int, initialised from the flag's value when the var is
+    created (var.cc:75); nn.conv2d marks the gathered input of a grouped convolution with {"G": groups} (nn.py:1278),
+    and the mark does not stand in the way of the matcher."""
+    import jittor_amd.executor as E
+    assert jt.zeros([2]).compile_options == {}
+    with jt.flag_scope(compile_options={"parallel": 0}):
+        v = jt.zeros([2])
+    assert v.compile_options == {"parallel": 0} and jt.zeros([2]).compile_options == {}
+    v.compile_options = {"G": 4, "C": 8}
+    assert v.compile_options == {"G": 4, "C": 8}
+    got = v.compile_options
+    got["G"] = 5                                       # a copy: the var keeps its own
+    assert v.compile_options["G"] == 4
+    with pytest.raises(TypeError):
+        v.compile_options = {"G": 1.5}
+    x, w = jt.zeros([1, 8, 6, 6]), jt.zeros([8, 2, 3, 3])
+    y = jt.nn.conv2d(x, w, padding=1, groups=4)
+    scatter = y._op
+    product = scatter.inputs[0]._op
+    assert product.inputs[0].compile_options == {"G": 4}
+    unit = E._match_conv_grouped(scatter)
+    assert unit is not None and unit.groups == 4
+
+
 def test_conv_gradient_patterns_match_for_common_losses():
     """The two backward patterns are recognised whatever stands between the convolution and the loss: the loss may
     be the output itself (jt.grad seeds ones, test_conv_tuner.py:105-133), its sum or mean (for 16-bit outputs these
