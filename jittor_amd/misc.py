@@ -8,6 +8,8 @@ Everything here only builds Var graphs; execution is the path's kernels.
 """
 import numbers
 
+import numpy as np
+
 from . import core
 from .core import Var, reindex, reindex_reduce, ternary, binary, array, broadcast
 
@@ -160,11 +162,15 @@ def reshape(x, *shape):
 
 def _parse_key(x, key):
     """Splits an index into, per axis of x, what selects it: returns (out_shape, exprs, extras) where exprs[d] is
-    the index expression of axis d of x in terms of the coordinates of the selection."""
+    the index expression of axis d of x in terms of the coordinates of the selection.  Integer Vars (also lists and
+    numpy integer arrays, of any rank) index their axes together: they are broadcast against each other, right
+    aligned, into one block of output dims that stands where the first of them stood
+    (python/jittor/src/ops/getitem_op.cc:76-113)."""
     if isinstance(key, Var) and key.dtype == "bool":
         raise IndexError("a boolean mask selects a data-dependent number of elements: use ternary(mask, a, b)")
     if not isinstance(key, tuple):
         key = (key,)
+    key = tuple(array(np.asarray(k)) if isinstance(k, (list, np.ndarray)) else k for k in key)
     if sum(1 for k in key if k is Ellipsis) > 1:
         raise IndexError("an index can only have a single ellipsis")
     n_real = sum(1 for k in key if k is not None and k is not Ellipsis)
@@ -177,9 +183,21 @@ def _parse_key(x, key):
         else:
             full.append(k)
     full.extend([slice(None)] * (x.ndim - sum(1 for k in full if k is not None)))
+    index_vars = [k for k in full if isinstance(k, Var)]
+    for k in index_vars:
+        if k.dtype == "bool" or k.is_float():
+            raise IndexError("only integer Vars index an axis, got %s" % k.dtype)
+    var_dim = max([k.ndim for k in index_vars], default=0)
+    block = [1] * var_dim                                  # the index Vars' common shape
+    for k in index_vars:
+        for j in range(k.ndim):
+            have, want = block[var_dim - 1 - j], k.shape[k.ndim - 1 - j]
+            if have != want and have != 1 and want != 1:
+                raise IndexError("index Vars of shapes %s do not broadcast" % [list(v.shape) for v in index_vars])
+            block[var_dim - 1 - j] = max(have, want)
     out_shape, exprs, extras = [], [], []
     axis = 0
-    var_axes = []
+    first_var_dim = -1                                     # output dim where the block starts
     for k in full:
         if k is None:
             out_shape.append(1)
@@ -196,12 +214,13 @@ def _parse_key(x, key):
             exprs.append("%d+i%d*(%d)" % (start, len(out_shape), step))
             out_shape.append(count)
         elif isinstance(k, Var):
-            if k.ndim != 1 or k.is_float():
-                raise IndexError("only 1-d integer Vars index an axis")
-            exprs.append("@e%d(i%d)" % (len(extras), len(out_shape)))
+            if first_var_dim < 0:
+                first_var_dim = len(out_shape)
+                out_shape.extend(block)
+            # the Var's own dims, right aligned in the block; an extent of 1 reads element 0 along that dim
+            coords = ["i%d" % (first_var_dim + var_dim - k.ndim + j) if k.shape[j] != 1 else "0" for j in range(k.ndim)]
+            exprs.append("@e%d(%s)" % (len(extras), ",".join(coords)))
             extras.append(k)
-            out_shape.append(k.shape[0])
-            var_axes.append(axis)
         else:
             raise IndexError("unsupported index %r" % (k,))
         axis += 1
@@ -209,8 +228,9 @@ def _parse_key(x, key):
 
 
 def getitem(x, key):
-    """Basic indexing with integers, slices (positive or negative step), None and Ellipsis, and one
-    integer Var per axis (gather along that axis); one reindex (python/jittor/src/ops/getitem_op.cc)."""
+    """Indexing with integers, slices (positive or negative step), None, Ellipsis and integer Vars / lists / numpy
+    arrays of any rank (broadcast against each other as in the reference); one reindex
+    (python/jittor/src/ops/getitem_op.cc)."""
     out_shape, exprs, extras = _parse_key(x, key)
     if not out_shape:
         out_shape = [1]

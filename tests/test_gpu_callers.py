@@ -87,6 +87,25 @@ def test_layout_ops_and_slicing(gpu):
     assert np.array_equal(v[:, None, 2].data, x[:, None, 2])
     idx = np.array([3, 0, 3, 1], np.int32)
     assert np.array_equal(v[:, jt.array(idx)].data, x[:, idx])
+    # integer Vars (lists, numpy arrays) of any rank; several of them index together, broadcast against each other into
+    # one block of dims where the first of them stood (getitem_op.cc:76-113) -- numpy's result when they are adjacent
+    i2 = np.array([[3, 0], [1, 2], [0, 0]], np.int32)
+    assert np.array_equal(v[jt.array(i2)].data, x[i2])
+    assert np.array_equal(v[:, jt.array(i2), 1].data, x[:, i2, 1])
+    a, b = np.array([0, 3, 1], np.int32), np.array([4, 4, 2], np.int32)
+    assert np.array_equal(v[jt.array(a), jt.array(b)].data, x[a, b])
+    assert np.array_equal(v[:, jt.array(a), jt.array(b), ::2].data, x[:, a, b, ::2])
+    col = np.array([[0], [3]], np.int32)
+    assert np.array_equal(v[jt.array(col), jt.array(b)].data, x[col, b])          # [2,1] with [3] -> a [2,3] block
+    assert np.array_equal(v[[1, 0, 1]].data, x[[1, 0, 1]])
+    assert np.array_equal(v[:, np.array([4, 1])].data, x[:, [4, 1]])
+    # separated by a slice: the block stays at the first index Var's place (numpy would move it to the front)
+    got = v[jt.array(a), :, jt.array(b)].data
+    assert np.array_equal(got, x[a, :, b])               # (the first one stands first here, so both agree)
+    got = v[:, jt.array(a), :, jt.array(b)].data
+    assert got.shape == (4, 3, 6) and np.array_equal(got, np.stack([x[:, a[i], :, b[i]] for i in range(3)], axis=1))
+    with pytest.raises(IndexError):
+        v[jt.array(a), jt.array(np.array([0, 1], np.int32))]                       # [3] and [2] do not broadcast
     with pytest.raises(IndexError):
         v[4]
     with pytest.raises(IndexError):
@@ -232,6 +251,14 @@ def test_setitem_and_assign(gpu):
     x[jt.array(idx)] = jt.array(v)
     want = a.copy()
     want[idx] = v
+    assert np.array_equal(x.data, want)
+    # two index Vars zipped (distinct positions), with a slice behind them
+    ia, ib = np.array([5, 0, 3], np.int32), np.array([6, 2, 2], np.int32)
+    v2 = rng.standard_normal((3, 2)).astype(np.float32)
+    x = jt.array(a)
+    x[jt.array(ia), jt.array(ib), 1:3] = jt.array(v2)
+    want = a.copy()
+    want[ia, ib, 1:3] = v2
     assert np.array_equal(x.data, want)
     # integer data, and a chain of writes
     b = np.arange(24, dtype=np.int32).reshape(4, 6)
