@@ -99,7 +99,12 @@ template <int ND> __device__ __forceinline__ index_t mjt_red_offset(const Params
 }
 
 #if ROW
-extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
+// G lanes share one output: up to a wave (shuffles only), or 128 .. 1024 lanes (whole waves; their results meet in
+// LDS).  Wide groups are for long rows streamed from memory: a lane then has one batch of UNR loads instead of
+// several, and the memory system serves many lanes with few loads each faster than few lanes with many
+// (a plain read of 134 MB: 64 lanes x 16 loads per workgroup 21.6 us, 128 x 8 20.4 us).
+#define BLK (G > 256 ? G : 256)
+extern "C" __global__ __launch_bounds__(BLK) void ENTRY(Params p) {
     const TX* __restrict__ xp = (const TX*)p.a[0];
     TY* __restrict__ yp = (TY*)p.a[1];
     const index_t O = (index_t)(unsigned long long)p.a[2];
@@ -109,7 +114,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     (void)xp;
     MJT_PRO_SCALARS
     const unsigned lane = threadIdx.x % G;
-    const index_t o = (index_t)blockIdx.x * (256 / G) + threadIdx.x / G;
+    const index_t o = (index_t)blockIdx.x * (BLK / G) + threadIdx.x / G;
     const index_t s = blockIdx.y;
     TACC acc[VEC];
 #pragma unroll
@@ -157,10 +162,19 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 #pragma unroll
     for (int k = 1; k < VEC; k++) r = (TACC)(MERGE(r, acc[k]));
 #pragma unroll
-    for (int off = G / 2; off > 0; off >>= 1) {
+    for (int off = (G < 64 ? G : 64) / 2; off > 0; off >>= 1) {
         TACC other = mjt_shfl_xor_any(r, off);
         r = (TACC)(MERGE(r, other));
     }
+#if G > 64
+    __shared__ TACC part[BLK / 64];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = r;
+    __syncthreads();
+    if (lane == 0) {
+#pragma unroll
+        for (int j = 1; j < G / 64; j++) r = (TACC)(MERGE(r, part[(threadIdx.x >> 6) + j]));
+    }
+#endif
     if (lane == 0 && o < O) yp[SPLIT ? o * S + s : o] = (TY)r;
 }
 #else
