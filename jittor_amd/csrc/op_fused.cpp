@@ -168,12 +168,15 @@ void fused_impl(const mjt_fused_desc* d) {
     while (vec > 1 && !aligned(vec)) vec /= 2;
     int64_t nvec = total / vec;
     auto env_int = [](const char* n, int d) { const char* v = getenv(n); return v && *v ? atoi(v) : d; };
-    int block = env_int("MJT_FUSED_BLOCK", 256);
     // measured on MI355X: one vector per lane is fastest for the chain workloads (more vectors per
     // lane cost registers and occupancy); outputs too large to be re-read from cache are stored
-    // non-temporally, loads stay plain
+    // non-temporally, loads stay plain; and such streams run best as single-wave workgroups, which the dispatcher
+    // hands out in address order 1 KB at a time (x[64,512,1024] float32 through an 11-op chain: 256 lanes 44.4 us,
+    // 128 lanes 44.1, 64 lanes 43.1, 512 lanes 45.2, 1024 lanes 49.9)
+    const bool streams = total * maxsize >= (int64_t(32) << 20);
+    int block = env_int("MJT_FUSED_BLOCK", streams ? 64 : 256);
     int unroll = env_int("MJT_FUSED_UNROLL", 1);
-    int nt = env_int("MJT_FUSED_NT", total * maxsize >= (int64_t(32) << 20) ? 2 : 0);   // bit 0: non-temporal loads, bit 1: non-temporal stores
+    int nt = env_int("MJT_FUSED_NT", streams ? 2 : 0);   // bit 0: non-temporal loads, bit 1: non-temporal stores
 
     // ---- parameter block layout ---------------------------------------------------
     // a[0] nvec | per merged axis: extent, divider | per var: pointer or scalar bits
