@@ -103,6 +103,37 @@ def test_reduce_other_dtypes(gpu):
     assert np.allclose(got, want, rtol=2 ** -7)
 
 
+@pytest.mark.parametrize("lanes", [128, 256, 512, 1024])
+def test_reduce_rows_shared_by_several_waves(gpu, lanes, monkeypatch):
+    """The row kernel with a row given to several whole waves (what long streamed rows take by themselves, forced here
+    on small inputs): every op family, ragged row lengths (lanes without an element, rows that end inside a vector
+    batch), row counts that do not fill the last workgroup, two reduced axes, 16-bit and integer inputs -- against
+    the oracle, exact for maximum / minimum / integers, 1e-5 for float sums."""
+    monkeypatch.setenv("MJT_REDUCE_G", str(lanes))
+    rng = np.random.default_rng(lanes)
+    # (few rows are split into partial sums and folded by a second launch; 2100 rows keep the chip busy by themselves)
+    for shape, dims in [((37, 5000), (1,)), ((5, 4096), (1,)), ((3, 7, 1031), (2,)), ((6, 3, 2048), (1, 2)), ((9, 640), (1,)),
+                        ((2100, 1100), (1,))]:
+        x = rng.uniform(-1, 1, shape).astype(np.float32)
+        n_red = x.size // int(np.prod(O.reduce_shape(shape, dims, False)[0]))
+        for op in ["add", "maximum", "minimum", "mean"]:
+            got = jt.reduce(jt.array(x), op, dims).data
+            assert ("g%d" % lanes) in L.last_kernel() or (shape[0] < 2100 and L.last_kernel().endswith("_fold")), L.last_kernel()
+            ref = O.reduce(x, op, dims)
+            if op in ("maximum", "minimum"):
+                assert exact(got, ref), (shape, op)
+            else:
+                assert np.allclose(got, ref, rtol=1e-5, atol=1e-5 * np.sqrt(n_red)), (shape, op, np.abs(got - ref).max())
+    xi = rng.integers(-1000, 1000, (11, 3000)).astype(np.int32)
+    for op in ["add", "maximum", "bitwise_xor"]:
+        assert exact(jt.reduce(jt.array(xi), op, 1).data, O.reduce(xi, op, 1)), op
+    h = rng.standard_normal((6, 2500)).astype(np.float32)
+    got = jt.array(h).bfloat16().sum(1).data          # cast -> float32 sum -> cast (truncation)
+    hb = O.BF16(O.f32_to_bf16_bits(h)).to_f32()
+    want = O.BF16(O.f32_to_bf16_bits(O.reduce(hb, "add", 1))).to_f32()
+    assert np.allclose(got, want, rtol=2 ** -7)
+
+
 def test_reduce_full_size_c1(gpu):
     x = np.random.default_rng(0).uniform(-1, 1, (8192, 4096)).astype(np.float32)
     got = jt.array(x).sum(1).data
