@@ -152,7 +152,13 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                          ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + (CBLK == 64 ? 4 * LROWS * LCOLS * 16 : 0) < 65536 &&
                          (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49 &&
                          // byte offsets inside one image and inside the weights are 32-bit in the kernel
-                         C * G * H * W * 2 < (int64_t(1) << 31) && K * OH * OW * 4 < (int64_t(1) << 31) && numel(w) * 2 < (int64_t(1) << 31);
+                         C * G * H * W * 2 < (int64_t(1) << 31) && K * OH * OW * 4 < (int64_t(1) << 31) && numel(w) * 2 < (int64_t(1) << 31) &&
+                         // a 1x1 convolution with many more input than output channels is a product with a long inner
+                         // dimension: with few output channels or a small map the matrix-product kernel below streams it
+                         // faster than this kernel walks one-step channel blocks (64 x 256 x 56 x 56 -> 64 channels: 31 us
+                         // against 73; 64 x 1024 x 14 x 14 -> 256: 50 against 142; but 64 x 512 x 28 x 28 -> 128: 50 against 41)
+                         !(R * S == 1 && G == 1 && C >= 4 * K && (K <= 64 || OH * OW <= 256) && p->stride_h == 1 && p->stride_w == 1 &&
+                           matmul_available() && !getenv("MJT_CONV_NO_GEMM"));
     if (mfma_ok) {
         // Rows per workgroup: a workgroup walks RPW output rows as NFULL tiles of TR rows plus one
         // shorter tile.  Pick the RPW that minimises (rounds of workgroups over the compute units) x

@@ -757,6 +757,25 @@ def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
     assert np.abs(widen[out](got2) - ref).max() <= tol * np.abs(ref).max()
 
 
+def test_conv_1x1_with_many_more_input_channels_runs_as_a_product(gpu, monkeypatch):
+    """A 1x1 convolution whose input channels outnumber its output channels 4 : 1 or more, with at most 64 output
+    channels or a map of at most 256 pixels, is handed to the matrix-product kernel although the MFMA convolution
+    kernel would take it (a long inner dimension in one-step channel blocks is that kernel's worst case); both
+    against a float64 product, same bound."""
+    rng = np.random.default_rng(43)
+    for xs, ws in (((2, 256, 16, 16), (64, 256, 1, 1)), ((3, 512, 14, 14), (128, 512, 1, 1))):
+        xb, wb = _bf16(rng.standard_normal(xs)), _bf16(rng.standard_normal(ws) * 0.1)
+        ref = np.einsum("nchw,kc->nkhw", O.BF16(xb).to_f32().astype(np.float64), O.BF16(wb).to_f32().astype(np.float64)[:, :, 0, 0])
+        got, kern = _conv_call(xb, wb, (1, 1, 0, 0, 1, 1))
+        assert kern in ("conv_as_gemm", "conv_as_reindex_gemm"), kern
+        assert np.abs(got - ref).max() <= 1e-4 * np.abs(ref).max()
+        monkeypatch.setenv("MJT_CONV_NO_GEMM", "1")
+        got2, kern2 = _conv_call(xb, wb, (1, 1, 0, 0, 1, 1))
+        monkeypatch.delenv("MJT_CONV_NO_GEMM")
+        assert kern2.startswith("mjt_conv_mfma_bf16"), kern2
+        assert np.abs(got2 - ref).max() <= 1e-4 * np.abs(ref).max()
+
+
 def test_conv_grouped_entry_and_front_end(gpu):
     """Grouped convolution (python/jittor/nn.py:1272-1294): the C entry point against the oracle's 8-d
     restatement, then nn.conv2d(groups=G) matched by the executor (one kernel, nothing of rank 8 in memory)
