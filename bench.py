@@ -440,6 +440,10 @@ def main():
     for k, f in fractions.items():
         by_config.setdefault(k[:2], []).append(f >= targets[k])
     met = sum(1 for v in by_config.values() if all(v))
+    # C5 is timed with the float32 accumulator stored; what the reference's graph hands on for bfloat16 inputs is that sum
+    # narrowed to bfloat16 (ops/reduce_op.cc:259-266), which the same kernel stores instead: shown beside it, not counted
+    if "C5bf16out" in results and "roofline" in results["C5bf16out"]:
+        fractions["C5bf16out"] = results["C5bf16out"]["roofline"]["frac"]
     line = {
         "metric": "achieved HBM GB/s (% peak) for reduce/reindex/fused ops; conv TFLOP/s",
         "value": head.get("roofline", {}).get("achieved"),
