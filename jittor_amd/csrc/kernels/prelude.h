@@ -92,11 +92,23 @@ __device__ __forceinline__ void mjt_store(T* p, const mjt_pack<T, N>& src) {
     typedef typename mjt_vec_t<sizeof(T) * N>::type V;
     *reinterpret_cast<V*>(p) = *reinterpret_cast<const V*>(&src);
 }
+// Streaming store: non-temporal and system scope (sc0 sc1 nt), for results that are written once and not read back by the
+// kernel.  On MI355X this is the fastest policy for large outputs (a fill of 231 MB: 6.9 TB/s against 6.6 for plain
+// non-temporal stores and 6.5 for ordinary ones).  Spelled out because the non-temporal builtin sets nt only.
 template <class T, int N>
 __device__ __forceinline__ void mjt_store_nt(T* p, const mjt_pack<T, N>& src) {
-    if constexpr (sizeof(T) * N <= 16) {
-        typedef typename mjt_vec_t<sizeof(T) * N>::type V;
-        __builtin_nontemporal_store(*reinterpret_cast<const V*>(&src), reinterpret_cast<V*>(p));
+    constexpr int BYTES = (int)(sizeof(T) * N);
+    if constexpr (BYTES == 16) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(*reinterpret_cast<const mjt_u32x4*>(&src)) : "memory");
+    } else if constexpr (BYTES == 8) {
+        typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+        asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(*reinterpret_cast<const u32x2*>(&src)) : "memory");
+    } else if constexpr (BYTES == 4) {
+        asm volatile("global_store_dword %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(*reinterpret_cast<const unsigned*>(&src)) : "memory");
+    } else if constexpr (BYTES == 2) {
+        asm volatile("global_store_short %0, %1, off sc0 sc1 nt" : : "v"(p), "v"((unsigned)*reinterpret_cast<const unsigned short*>(&src)) : "memory");
+    } else if constexpr (BYTES == 1) {
+        asm volatile("global_store_byte %0, %1, off sc0 sc1 nt" : : "v"(p), "v"((unsigned)*reinterpret_cast<const unsigned char*>(&src)) : "memory");
     } else {
         mjt_store(p, src);
     }
