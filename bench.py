@@ -352,7 +352,7 @@ def wl_copy(L, lib, steps, warmup, with_cpu):
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_workloads.txt"
 MEASURED_TRAFFIC = {
     "C1": ("mjt_reduce_row_add_float32_float32_k1r1v4g512", 2.0 * 65553.0 * 1024 + 256.0 * 1024),
-    "C2": ("mjt_window_gather_b4_56x56_k3x3_s1x1_d1x1_o56x56_t8x1", 2.0 * 15647.5 * 1024 + 225812.4 * 1024),
+    "C2": ("mjt_window_gather_b4_56x56_k3x3_s1x1_d1x1_o56x56_t8x1", 2.0 * 15647.5 * 1024 + 225792.0 * 1024),
     "C3add": ("mjt_scatter1d_add_float32_int32_w16384_b64_e8_s1920_main", 2.0 * 65688.8 * 1024 + 37617.6 * 1024),
     "C3max": ("mjt_scatter1d_maximum_float32_int32_w16384_b64_e8_s4096_main", 2.0 * 65690.2 * 1024 + 37642.0 * 1024),
     "C4": ("mjt_fused_11ops_caa413813b1db4ef", 2.0 * 65566.0 * 1024 + 131072.0 * 1024),
