@@ -143,7 +143,7 @@ void fill_axes(std::vector<uint64_t>& a, const std::vector<Axis>& kept, const st
 }
 
 // One launch of the row or column kernel.  Returns nothing; partials (when
-// S > 1) are written to `out` as [O, S] (row) or [S, O] (column).
+// S > 1) are written to `out` as [O, S] by both kernels.
 void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* out, int64_t O, int64_t S,
             const std::vector<Axis>& kept, const std::vector<Axis>& red, double rcount, bool use64, int vec, int g,
             int64_t per, int64_t total, bool stream = false, const Prologue* pro = nullptr, bool may_build = true) {
@@ -315,9 +315,13 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         } else {
             void* part = partials((size_t)O * S * asz);
             launch(false, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R, stream, pro, mb);
-            std::vector<Axis> k2{Axis{O, 1}}, r2{Axis{S, O}};
-            int vec2 = pick_vec(asz, O, part, y->ptr, tsz);
-            launch(false, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, 1, S, S, false, nullptr, mb);
+            // the partials are [O, S]: fold along the last axis with the row kernel
+            std::vector<Axis> k2{Axis{O, S}}, r2{Axis{S, 1}};
+            int vec2 = pick_vec(asz, S, part, nullptr, 0);
+            int g2 = 64;
+            while (g2 > 1 && (int64_t)(g2 / 2) * vec2 >= S) g2 /= 2;
+            int64_t nL2 = (S + (int64_t)g2 * vec2 - 1) / ((int64_t)g2 * vec2);
+            launch(true, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, g2, nL2, nL2, false, nullptr, mb);
         }
     }
 }
