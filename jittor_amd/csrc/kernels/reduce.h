@@ -186,9 +186,12 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     (void)rcount;
     (void)xp;
     MJT_PRO_SCALARS
-    const index_t o = ((index_t)blockIdx.x * 256 + threadIdx.x) * VEC;
-    const index_t s = blockIdx.y;
-    if (o >= O) return;
+    // G lanes across the outputs (a power of two up to 256, or 1 for 256): with fewer than 256 vectors of outputs the
+    // rest of the workgroup takes other slices of the rows instead of idling
+    constexpr int TXL = G > 1 ? G : 256;
+    const index_t o = ((index_t)blockIdx.x * TXL + threadIdx.x % TXL) * VEC;
+    const index_t s = (index_t)blockIdx.y * (256 / TXL) + threadIdx.x / TXL;
+    if (o >= O || (SPLIT && s >= (index_t)(unsigned long long)p.a[3])) return;
     MJT_PRO_PER_OUTPUT
     const index_t kbase = mjt_kept_offset(p, o);
     const index_t per = (index_t)(unsigned long long)p.a[5];

@@ -168,9 +168,11 @@ void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* 
     fill_axes(a, kept, red);
     if (pro) a.insert(a.end(), pro->args.begin(), pro->args.end());
     const int64_t blk = row && g > 256 ? g : 256;              // lanes per workgroup
-    int64_t blocks = row ? (O + (blk / g) - 1) / (blk / g) : ((O / vec) + 255) / 256;
-    MJT_CHECK(blocks < (int64_t(1) << 31) && S < 65536, "reduce: launch too large");
-    jit_launch(k, (unsigned)blocks, (unsigned)S, (unsigned)blk, 0, a);
+    const int64_t txl = !row && g > 1 ? g : 256;                // column kernel: lanes across the outputs
+    int64_t blocks = row ? (O + (blk / g) - 1) / (blk / g) : ((O / vec) + txl - 1) / txl;
+    const int64_t grid_y = row ? S : (S + 256 / txl - 1) / (256 / txl);
+    MJT_CHECK(blocks < (int64_t(1) << 31) && grid_y < 65536, "reduce: launch too large");
+    jit_launch(k, (unsigned)blocks, (unsigned)grid_y, (unsigned)blk, 0, a);
 }
 
 }  // namespace
@@ -313,8 +315,14 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         if (S == 1) {
             launch(false, tx, ty, op, false, x->ptr, y->ptr, O, 1, kept, red, rcount, use64, vec, 1, per, R, stream, pro, mb);
         } else {
+            // lanes across the outputs: all 256 (g = 1), or with fewer vectors of outputs the power of two that holds them
+            int gx = 1;
+            if (threads < 256) {
+                gx = 2;
+                while (gx < threads) gx *= 2;
+            }
             void* part = partials((size_t)O * S * asz);
-            launch(false, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, 1, per, R, stream, pro, mb);
+            launch(false, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, gx, per, R, stream, pro, mb);
             // the partials are [O, S]: fold along the last axis with the row kernel
             std::vector<Axis> k2{Axis{O, S}}, r2{Axis{S, 1}};
             int vec2 = pick_vec(asz, S, part, nullptr, 0);
