@@ -72,7 +72,10 @@ def test_reduce_integer_exact(gpu, keepdims):
 
 @pytest.mark.parametrize("shape,dims", [((64, 33, 5), (1,)), ((64, 33, 5), (0, 2)), ((64, 33, 5), ()),
                                         ((7, 1000), (1,)), ((1000, 7), (0,)), ((3, 5, 7, 9, 2), (1, 3)),
-                                        ((2, 70000), (1,)), ((70000, 4), (0,)), ((5, 0), (1,)), ((4, 6, 8), (2,))])
+                                        ((2, 70000), (1,)), ((70000, 4), (0,)), ((5, 0), (1,)), ((4, 6, 8), (2,)),
+                                        # column reduces whose rows are split among workgroups: few vectors of outputs (the
+                                        # workgroup's other lanes take other slices), partial sums folded by the row kernel
+                                        ((5000, 96), (0,)), ((3, 4000, 520), (0, 1)), ((2048, 1024), (0,)), ((40000, 20), (0,))])
 def test_reduce_float(gpu, shape, dims):
     rng = np.random.default_rng(7)
     x = rng.uniform(-1, 1, shape).astype(np.float32)
