@@ -209,17 +209,17 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 #pragma unroll
         for (int k = 0; k < VEC; k++) acc[k] = (TACC)(COMBINE(acc[k], v.v[k]));
     }
-#if SPLIT
-    // partial sums go out as [O, S], the layout the row kernel folds (S contiguous per output): a fold that walked S rows
-    // of an [S, O] array with one lane per output would be one long chain of dependent loads when O is small
+#if SPLIT && SPLIT_T
+    // many slices: partial sums go out as [O, S], the layout the row kernel folds (S contiguous per output): a fold that
+    // walked S rows of an [S, O] array with one lane per output would be one long chain of dependent loads
     const index_t S = (index_t)(unsigned long long)p.a[3];
 #pragma unroll
     for (int k = 0; k < VEC; k++) yp[(o + k) * S + s] = (TY)acc[k];
 #else
-    mjt_pack<TY, VEC> out;
+    mjt_pack<TY, VEC> out;                      // [O], or with a few slices [S, O], folded by this kernel
 #pragma unroll
     for (int k = 0; k < VEC; k++) out.v[k] = (TY)acc[k];
-    mjt_store(yp + o, out);
+    mjt_store(yp + (SPLIT ? s * O : 0) + o, out);
 #endif
 }
 #endif

@@ -4,7 +4,9 @@
 // anything they do not cover goes to the generic kernels.
 #include "common.h"
 #include "expr.h"
+#include <algorithm>
 #include <mutex>
+#include <sstream>
 #include <unordered_map>
 
 namespace mjt {
@@ -32,6 +34,101 @@ int env_int(const char* name, int dflt) {
     return v && *v ? atoi(v) : dflt;
 }
 }  // namespace
+
+// y = x with its axes in another order (every index expression is one output coordinate, each used once): tiles through
+// LDS when x's innermost axis is not y's (kernels/permute_tiles.h); otherwise the generic kernel already moves runs.
+bool try_permute(const mjt_tensor* x, const mjt_tensor* y, const std::vector<Affine>& aff) {
+    if (getenv("MJT_NO_FASTPATH") || getenv("MJT_NO_PERMUTE")) return false;
+    const int n = x->ndim;
+    if (n != y->ndim || n < 2) return false;
+    const int64_t esz = dtype_size(x->dtype);
+    if (esz != 2 && esz != 4 && esz != 8) return false;
+    // perm[d]: the output axis that indexes x's axis d
+    std::vector<int> perm(n, -1);
+    std::vector<bool> used(n, false);
+    for (int d = 0; d < n; d++) {
+        if (aff[d].c0 != 0) return false;
+        for (int j = 0; j < 10; j++) {
+            if (aff[d].coef[j] == 0) continue;
+            if (aff[d].coef[j] != 1 || perm[d] >= 0 || j >= n || used[j]) return false;
+            perm[d] = j;
+            used[j] = true;
+        }
+        if (perm[d] < 0 || y->shape[perm[d]] != x->shape[d]) return false;
+    }
+    if (numel(x) < (1 << 16) || numel(x) >= (int64_t(1) << 40)) return false;
+    // drop axes of extent 1; merge x axes d, d+1 that follow each other in y as well (only axes of extent 1 between them)
+    std::vector<int64_t> ext;        // extents of the merged x axes
+    std::vector<int> first_y, last_y;   // the output axes a merged x axis covers
+    for (int d = 0; d < n; d++) {
+        if (x->shape[d] == 1) continue;
+        bool merge = !ext.empty() && perm[d] > last_y.back();
+        for (int j = merge ? last_y.back() + 1 : 0; merge && j < perm[d]; j++) merge = y->shape[j] == 1;
+        if (merge) {
+            ext.back() *= x->shape[d];
+            last_y.back() = perm[d];
+        } else {
+            ext.push_back(x->shape[d]);
+            first_y.push_back(perm[d]);
+            last_y.push_back(perm[d]);
+        }
+    }
+    const int m = (int)ext.size();
+    if (m < 2 || m > 6) return false;
+    // order of the merged axes in y
+    std::vector<int> order(m);                       // order[k]: merged x axis that is k-th in y
+    for (int k = 0; k < m; k++) order[k] = k;
+    std::sort(order.begin(), order.end(), [&](int a, int b) { return first_y[a] < first_y[b]; });
+    std::vector<int64_t> xstr(m), ystr(m);
+    {
+        int64_t s = 1;
+        for (int d = m - 1; d >= 0; d--) { xstr[d] = s; s *= ext[d]; }
+        s = 1;
+        for (int k = m - 1; k >= 0; k--) { ystr[order[k]] = s; s *= ext[order[k]]; }
+    }
+    const int A = m - 1, B = order[m - 1];           // x's innermost axis; the x axis that is innermost in y
+    if (A == B) return false;                        // rows stay rows: nothing to transpose
+    if (ext[A] < 16 || ext[B] < 16) return false;    // thin tiles: the generic kernel does as well
+    std::ostringstream key;
+    key << "perm|" << esz;
+    for (int d = 0; d < m; d++) key << "|" << ext[d] << "," << ystr[d];
+    JitKernel* k = cached(key.str());
+    const int64_t TA = (ext[A] + 63) / 64, TBN = (ext[B] + 63) / 64;
+    int64_t others = 1;
+    if (!k) {
+        std::ostringstream oe, ox, oy, name;
+        int noth = 0;
+        for (int d = 0; d < m; d++) {
+            if (d == A || d == B) continue;
+            oe << (noth ? ", " : "") << ext[d];
+            ox << (noth ? ", " : "") << xstr[d];
+            oy << (noth ? ", " : "") << ystr[d];
+            noth++;
+        }
+        uint64_t h = 1469598103934665603ull;
+        for (unsigned char ch : key.str()) {
+            h ^= ch;
+            h *= 1099511628211ull;
+        }
+        char buf[32];
+        snprintf(buf, sizeof(buf), "%016llx", (unsigned long long)h);
+        name << "mjt_permute_b" << esz << "_" << ext[B] << "x" << ext[A] << "_" << buf;
+        std::ostringstream src;
+        src << "#define ENTRY " << name.str() << "\n#define TB " << (esz == 4 ? "unsigned" : esz == 2 ? "unsigned short" : "unsigned long long")
+            << "\n#define LA " << ext[A] << "LL\n#define LB " << ext[B] << "LL\n#define XSTR_B " << xstr[B] << "LL\n#define YSTR_A " << ystr[A]
+            << "LL\n#define NOTH " << noth << "\n#define OEXT " << oe.str() << "\n#define OXS " << ox.str() << "\n#define OYS " << oy.str() << "\n";
+        src << embedded_source("permute_tiles.h") << "\n";
+        k = jit_get(src.str(), name.str());
+        remember(key.str(), k);
+    }
+    for (int d = 0; d < m; d++)
+        if (d != A && d != B) others *= ext[d];
+    const int64_t blocks = TA * TBN * others;
+    if (blocks >= (int64_t(1) << 31)) return false;
+    std::vector<uint64_t> args{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), 0, 0};
+    jit_launch(k, (unsigned)blocks, 1, 256, 0, args);
+    return true;
+}
 
 // y[b.., oh, ow, kh, kw] = x[b.., oh*SH + kh*DH + CH, ow*SW + kw*DW + CW]
 bool try_window_gather(const mjt_tensor* x, const mjt_tensor* y, const std::vector<Affine>& aff, double overflow_value) {

@@ -59,13 +59,14 @@ struct Variant {
     int tx, ty, op, nk, nr, vec, g, unr, nt;
     bool row, split, use64, second;   // second: folding partials (TX == TY, plain merge)
     const Prologue* pro;
+    bool tsplit = false;              // column kernel: partials as [O, S] instead of [S, O]
 };
 
 // may_build == false: only a kernel that is already loaded is returned (no compiler, no module load)
 JitKernel* get_kernel(const Variant& v, bool may_build = true) {
     std::ostringstream key;
     key << v.tx << "," << v.ty << "," << v.op << "," << v.nk << "," << v.nr << "," << v.vec << "," << v.g << ","
-        << v.row << v.split << v.use64 << v.second << "," << v.unr << "," << v.nt;
+        << v.row << v.split << v.use64 << v.second << v.tsplit << "," << v.unr << "," << v.nt;
     if (v.pro) key << "|" << v.pro->key;
     std::lock_guard<std::mutex> lock(g_mu);
     auto it = g_kernels.find(key.str());
@@ -75,7 +76,7 @@ JitKernel* get_kernel(const Variant& v, bool may_build = true) {
     std::ostringstream name;
     name << "mjt_reduce_" << (v.row ? "row_" : "col_") << opn << "_" << mjt_dtype_name(v.tx) << "_"
          << mjt_dtype_name(v.ty) << "_k" << v.nk << "r" << v.nr << "v" << v.vec << "g" << v.g
-         << (v.split ? "_split" : "") << (v.second ? "_fold" : "") << (v.use64 ? "_i64" : "");
+         << (v.split ? (v.tsplit ? "_tsplit" : "_split") : "") << (v.second ? "_fold" : "") << (v.use64 ? "_i64" : "");
     if (v.pro) {
         uint64_t h = 1469598103934665603ull;
         for (unsigned char ch : v.pro->key) {
@@ -91,7 +92,7 @@ JitKernel* get_kernel(const Variant& v, bool may_build = true) {
     src << "#define TX " << dtype_cname(v.tx) << "\n#define TY " << dtype_cname(v.ty) << "\n#define TACC " << dtype_cname(acc_dtype(v.ty)) << "\n";
     src << "#define index_t " << (v.use64 ? "long long" : "int") << "\n#define USE64 " << (v.use64 ? 1 : 0) << "\n";
     src << "#define NK " << v.nk << "\n#define NR " << v.nr << "\n#define VEC " << v.vec << "\n#define G " << v.g
-        << "\n#define SPLIT " << (v.split ? 1 : 0) << "\n#define ROW " << (v.row ? 1 : 0) << "\n";
+        << "\n#define SPLIT " << (v.split ? 1 : 0) << "\n#define SPLIT_T " << (v.tsplit ? 1 : 0) << "\n#define ROW " << (v.row ? 1 : 0) << "\n";
     src << "#define UNR " << v.unr << "\n#define MJT_LD " << (v.nt ? "mjt_load_nt" : "mjt_load") << "\n";
     src << "#define MERGE(a, b) mjt_" << merge_op << "<TACC>((a), (b))\n";
     if (v.second || v.op != MJT_OP_MEAN)
@@ -146,7 +147,7 @@ void fill_axes(std::vector<uint64_t>& a, const std::vector<Axis>& kept, const st
 // S > 1) are written to `out` as [O, S] by both kernels.
 void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* out, int64_t O, int64_t S,
             const std::vector<Axis>& kept, const std::vector<Axis>& red, double rcount, bool use64, int vec, int g,
-            int64_t per, int64_t total, bool stream = false, const Prologue* pro = nullptr, bool may_build = true) {
+            int64_t per, int64_t total, bool stream = false, const Prologue* pro = nullptr, bool may_build = true, bool tsplit = false) {
     // inputs larger than the caches are streamed (read once, non-temporal loads)
     // loads in flight per lane: 8, or as many as a row gives a lane when that is fewer (the unrolled loop only takes whole batches)
     int unr = env_int("MJT_REDUCE_UNR", 8);
@@ -156,6 +157,7 @@ void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* 
     }
     Variant v{tx, ty, op, (int)kept.size(), (int)red.size(), vec, g, unr,
               env_int("MJT_REDUCE_NT", stream ? 1 : 0), row, S > 1, use64, second, pro};
+    v.tsplit = tsplit && !row && S > 1;
     JitKernel* k = get_kernel(v, may_build);
     std::vector<uint64_t> a(8 + 6 * 5, 0);
     a[0] = bits_of_ptr(x);
@@ -322,14 +324,20 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
                 while (gx < threads) gx *= 2;
             }
             void* part = partials((size_t)O * S * asz);
-            launch(false, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, gx, per, R, stream, pro, mb);
-            // the partials are [O, S]: fold along the last axis with the row kernel
-            std::vector<Axis> k2{Axis{O, S}}, r2{Axis{S, 1}};
-            int vec2 = pick_vec(asz, S, part, nullptr, 0);
-            int g2 = 64;
-            while (g2 > 1 && (int64_t)(g2 / 2) * vec2 >= S) g2 /= 2;
-            int64_t nL2 = (S + (int64_t)g2 * vec2 - 1) / ((int64_t)g2 * vec2);
-            launch(true, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, g2, nL2, nL2, false, nullptr, mb);
+            const bool tsplit = S >= 16;                 // many slices: partials as [O, S], folded by the row kernel
+            launch(false, tx, ta, op, false, x->ptr, part, O, S, kept, red, rcount, use64, vec, gx, per, R, stream, pro, mb, tsplit);
+            if (tsplit) {
+                std::vector<Axis> k2{Axis{O, S}}, r2{Axis{S, 1}};
+                int vec2 = pick_vec(asz, S, part, nullptr, 0);
+                int g2 = 64;
+                while (g2 > 1 && (int64_t)(g2 / 2) * vec2 >= S) g2 /= 2;
+                int64_t nL2 = (S + (int64_t)g2 * vec2 - 1) / ((int64_t)g2 * vec2);
+                launch(true, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, g2, nL2, nL2, false, nullptr, mb);
+            } else {                                     // a few slices [S, O]: each output's lane walks them
+                std::vector<Axis> k2{Axis{O, 1}}, r2{Axis{S, O}};
+                int vec2 = pick_vec(asz, O, part, y->ptr, tsz);
+                launch(false, ta, ty, op, true, part, y->ptr, O, 1, k2, r2, rcount, false, vec2, 1, S, S, false, nullptr, mb);
+            }
         }
     }
 }

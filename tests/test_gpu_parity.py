@@ -493,6 +493,42 @@ def test_lazy_graph_recomputes_fused_intermediates(gpu):
     assert np.array_equal(h, np.histogram(x, 10, (0, 1))[0].astype(np.float32))
 
 
+@pytest.mark.parametrize("shape,perm,dtype,tiled", [
+    ((300, 400), (1, 0), "float32", True),
+    ((7, 130, 97), (0, 2, 1), "float32", True),                  # ragged tiles in both directions
+    ((5, 33, 20, 24), (0, 2, 3, 1), "float32", True),            # NCHW -> NHWC: the two trailing axes move as one
+    ((5, 20, 24, 33), (0, 3, 1, 2), "bfloat16", True),           # NHWC -> NCHW, 2-byte elements
+    ((40, 3, 50, 64), (2, 1, 0, 3), "float32", False),           # the innermost axis stays: rows move as rows
+    ((64, 70, 1, 80), (3, 2, 1, 0), "int32", True),              # full reversal with an axis of extent 1
+    ((6, 500, 8), (2, 1, 0), "float64", False),                  # a thin axis becomes innermost: generic kernel
+    ((3, 200, 5, 300), (3, 2, 1, 0), "float64", False),          # y's innermost axis has extent 3
+    ((30, 200, 5, 70), (3, 2, 1, 0), "float64", True),
+    ((2, 3, 40, 50, 60), (0, 4, 2, 1, 3), "int16", True),
+])
+def test_permute_through_tiles(gpu, shape, perm, dtype, tiled):
+    """Axis permutations (every index expression is one output coordinate) bit for bit against numpy.transpose; where
+    x's innermost axis does not stay innermost and both tile axes are wide enough they run on the tile kernel."""
+    rng = np.random.default_rng(11)
+    if dtype == "bfloat16":
+        host = O.f32_to_bf16_bits(rng.standard_normal(shape).astype(np.float32))
+    elif dtype.startswith("float"):
+        host = rng.standard_normal(shape).astype(dtype)
+    else:
+        host = rng.integers(-30000, 30000, shape).astype(dtype)
+    x = jt.from_storage(host, dtype)
+    yshape = [shape[a] for a in perm]
+    # y[i0..] = x[...] : x's axis perm[j] is indexed by output coordinate j
+    idx = [None] * len(shape)
+    for j, a in enumerate(perm):
+        idx[a] = "i%d" % j
+    y = jt.zeros(yshape, dtype)
+    tx, ty = L.tensor(x.raw_ptr(), dtype, x.shape), L.tensor(y.raw_ptr(), dtype, y.shape)
+    L.check(L.load().mjt_reindex(ctypes.byref(tx), ctypes.byref(ty), len(shape), L.c_strings(idx), 0.0, 0, L.c_strings([]), 0, None))
+    assert L.last_kernel().startswith("mjt_permute_") == tiled, L.last_kernel()
+    got = L.d2h(y.raw_ptr(), y.shape, L.NP_STORAGE[dtype])
+    assert np.array_equal(got, np.transpose(host, perm))
+
+
 # ---- meta-op convolution ---------------------------------------------------------------------------------
 def _bf16(a):
     return O.f32_to_bf16_bits(np.asarray(a, np.float32))
