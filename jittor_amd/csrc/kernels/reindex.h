@@ -25,9 +25,13 @@ struct Params { void* a[NPARAM]; };   // 8-byte words; typed as pointers so load
 #if REDUCE_TAIL
 // Gather fused with the reduce that consumes it (the reference fuses a reindex with its consumer: it is a
 // broadcast-type op, executor.cc:555; the pooling group of python/jittor/pool.py:200-208): the loop space y is never
-// written.  One lane per output: it walks the RTAIL elements of y's last axes that fold into it, gathers each and
-// combines them in TACC.  Extra constants: TZ, TACC, COMBINE(a, x), INIT; a[1] is z, a[2] its element count,
-// P_RTAIL / P_RCOUNT the parameter words of the tail length and of 1 / tail length (mean).
+// written.  A lane owns OV adjacent outputs: for each it walks the elements of y's last axes that fold into it, gathers
+// them and combines them in TACC, in the order of the flat tail offset.  Extra constants: TZ, TACC, COMBINE(a, x), INIT;
+// a[1] is z, a[2] its element count, P_RTAIL / P_RCOUNT the parameter words of the tail length and of 1 / tail length
+// (mean); MJT_RX_DECODE_KEPT gives the kept coordinates of output o_, MJT_RX_DECODE_TAIL the folded ones of tail
+// offset r (extents as literals).  RTAIL_C > 0: the tail length, known when the kernel is built -- the walk is
+// unrolled, out-of-range elements load x[0] and are replaced afterwards, so that the loads of all OV * RTAIL_C
+// elements are in flight together (x is not empty then).  RTAIL_C == 0: a loop of the length given at launch.
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const TX* __restrict__ xp = (const TX*)p.a[0];
     TZ* __restrict__ zp = (TZ*)p.a[1];
@@ -36,19 +40,47 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const index_t rtail = (index_t)(unsigned long long)p.a[P_RTAIL];
     const TACC rcount = (TACC)__longlong_as_double((long long)(unsigned long long)p.a[P_RCOUNT]);
     (void)rcount;
+    (void)rtail;
     MJT_RX_SETUP
-    const index_t o = (index_t)blockIdx.x * 256 + threadIdx.x;
-    if (o >= nout) return;
+    const index_t o0 = ((index_t)blockIdx.x * 256 + threadIdx.x) * OV;
+    if (o0 >= nout) return;
+#if RTAIL_C
+    TX got[OV][RTAIL_C];
+    bool out_[OV][RTAIL_C];
+#pragma unroll
+    for (int k = 0; k < OV; k++) {
+        const index_t o_ = o0 + k < nout ? o0 + k : nout - 1;
+        MJT_RX_DECODE_KEPT
+#pragma unroll
+        for (int r = 0; r < RTAIL_C; r++) {
+            MJT_RX_DECODE_TAIL
+            MJT_RX_INDEX
+            out_[k][r] = ov_;
+            got[k][r] = xp[ov_ ? (index_t)0 : xid];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < OV; k++) {
+        TACC acc = INIT;
+#pragma unroll
+        for (int r = 0; r < RTAIL_C; r++) {
+            const TX v = out_[k][r] ? ovalue_ : got[k][r];
+            acc = (TACC)(COMBINE(acc, v));
+        }
+        if (o0 + k < nout) zp[o0 + k] = (TZ)acc;
+    }
+#else
+    const index_t o_ = o0;
+    MJT_RX_DECODE_KEPT
     TACC acc = INIT;
     for (index_t r = 0; r < rtail; r++) {
-        const index_t e = o * rtail + r;
-        MJT_RX_DECODE
-        const index_t MJT_RX_LASTVAR = ilast_;
+        MJT_RX_DECODE_TAIL
         MJT_RX_INDEX
         const TX v = ov_ ? ovalue_ : xp[xid];
         acc = (TACC)(COMBINE(acc, v));
     }
-    zp[o] = (TZ)acc;
+    zp[o_] = (TZ)acc;
+#endif
 }
 #else
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {

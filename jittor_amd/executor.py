@@ -389,6 +389,8 @@ def _match_gather_reduce(red, consumers, target_ids):
     # itself still runs if somebody needs its result in memory
     if ro is None or xx.id in target_ids or getattr(xx, "_stop_fuse", False):
         return None
+    if getattr(ro, "same_memory", False) and flags["reshape_shares_memory"]:
+        return None            # a reshape costs nothing by itself: the plain reduce kernels read its input's bytes
     nd, nred = xx.ndim, bin(red.reduce_mask).count("1")
     if nred < 1 or red.reduce_mask != ((1 << nred) - 1) << (nd - nred) or red.out.dtype == "bool":
         return None
@@ -768,6 +770,11 @@ def _run_single(op):
         _lib.check(lib.mjt_reduce(ctypes.byref(tx), ctypes.byref(ty), _lib.OP_CODE[op.op], op.reduce_mask))
     elif isinstance(op, ReindexOp):
         x, extras = op.inputs[0], op.inputs[1:]
+        if getattr(op, "same_memory", False) and flags["reshape_shares_memory"]:
+            x._device_ptr()                                    # a row-major reinterpretation: the same bytes
+            out._buf = x._buf
+            stats["launches"] -= 1
+            return
         tx = _tensor_of(x)
         ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
         ex = (_lib.Tensor * max(1, len(extras)))(*[_tensor_of(e) for e in extras])

@@ -124,8 +124,9 @@ def flip(x, dim=0):
 
 
 def reshape(x, *shape):
-    """Row-major reinterpretation: a reindex through the flat offset (the reference aliases the buffer,
-    python/jittor/src/ops/reshape_op.cc; a copy gives the same values)."""
+    """Row-major reinterpretation.  In the graph it is a reindex through the flat offset, so gradients and pattern
+    matching see an ordinary op; when it runs, the result shares its input's buffer and nothing is launched (the
+    reference aliases the buffer too, python/jittor/src/ops/reshape_op.cc)."""
     if len(shape) == 1 and isinstance(shape[0], (list, tuple)):
         shape = tuple(shape[0])
     shape = list(shape)
@@ -157,7 +158,9 @@ def reshape(x, *shape):
     for d in range(x.ndim - 1, -1, -1):
         idx.append("%s/%d%%%d" % (flat, stride, x.shape[d]))
         stride *= x.shape[d]
-    return reindex(x, shape, idx[::-1])
+    y = reindex(x, shape, idx[::-1])
+    y._op.same_memory = True             # values are functional (assign rebinds, nothing writes in place): sharing is safe
+    return y
 
 
 def _parse_key(x, key):

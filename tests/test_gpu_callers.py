@@ -72,6 +72,44 @@ def test_pool_against_numpy(gpu):
     assert np.array_equal(g, want)
 
 
+def test_reshape_shares_its_input_bytes(gpu):
+    """reshape launches nothing (python/jittor/src/ops/reshape_op.cc aliases the buffer); values, gradients and later
+    assignments to either Var behave as with a copy."""
+    from jittor_amd import executor as E
+    rng = np.random.default_rng(59)
+    x = rng.standard_normal((6, 8, 10)).astype(np.float32)
+    v = jt.array(x)
+    v.sync()
+    before = E.stats["launches"]
+    r = v.reshape(48, 10)
+    r.sync()
+    assert E.stats["launches"] == before and r._device_ptr() == v._device_ptr()
+    assert np.array_equal(r.data, x.reshape(48, 10))
+    # a computed input, a reshape in the middle of a chain, and a reduce over the reshaped axes
+    w = ((v * 2.0 + 1.0).reshape(6, 80) - 0.5).reshape(12, 40)
+    assert np.allclose(w.data, ((x * 2.0 + 1.0).reshape(6, 80) - 0.5).reshape(12, 40), rtol=1e-6, atol=1e-6)
+    s = (v * v).reshape(6, 4, 20).sum(2)
+    assert np.allclose(s.data, (x * x).reshape(6, 4, 20).sum(2), rtol=1e-5, atol=1e-5)
+    # functional values: rebinding one Var leaves the other's contents alone
+    v2 = jt.array(x)
+    r2 = v2.reshape(-1)
+    r2.sync()
+    v2.assign(v2 + 1.0)
+    v2.sync()
+    assert np.array_equal(r2.data, x.reshape(-1)) and np.allclose(v2.data, x + 1.0)
+    # gradient through a reshape
+    p = jt.array(x)
+    loss = (p.reshape(48, 10) * jt.array(np.arange(10, dtype=np.float32))).sum()
+    g = jt.grad(loss, [p])[0]
+    assert np.allclose(g.data, np.broadcast_to(np.arange(10, dtype=np.float32), (6, 8, 10)))
+    with jt.flag_scope(reshape_shares_memory=False):
+        before = E.stats["launches"]
+        c = v.reshape(10, 48)
+        c.sync()
+        assert E.stats["launches"] == before + 1 and c._device_ptr() != v._device_ptr()
+        assert np.array_equal(c.data, x.reshape(10, 48))
+
+
 def test_layout_ops_and_slicing(gpu):
     rng = np.random.default_rng(53)
     x = rng.standard_normal((4, 5, 6, 7)).astype(np.float32)

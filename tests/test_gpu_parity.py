@@ -1299,7 +1299,9 @@ def test_gather_fused_with_reduce(gpu):
             ("mean", [2, 3, 4, 5, 3, 2], ["i0", "i1", "i2*2-1+i4", "i3*2-0+i5"], 0.0, 2),
             ("add", [2, 9, 10, 3], ["i0", "i3", "i1", "i2"], 0.0, 1),                      # sum over channels, moved last
             ("minimum", [7, 2, 3, 9, 10], ["i1", "i2", "(i3+i0)%9", "i4"], 5.0, 4),        # keeps only the first axis
-            ("multiply", [4, 2, 3, 3, 3], ["i1", "i2", "i0+i3", "i4*5"], 1.0, 2)]:
+            ("multiply", [4, 2, 3, 3, 3], ["i1", "i2", "i0+i3", "i4*5"], 1.0, 2),
+            ("add", [3, 5, 3, 2], ["i0%2", "i1%3", "i2*3+i0", "i3*6"], 0.5, 2),            # an odd number of outputs, two per lane
+            ("maximum", [1, 1, 2, 3, 5, 3], ["i0", "i1", "i2*5+i4-1", "i3*3+i5"], -1e30, 4)]:  # 90 folded elements: the loop form
         want = O.reduce(O.reindex(x, shape, idx, ov), op, list(range(len(shape) - nred, len(shape))))
         vx, vz = jt.from_storage(x, "float32"), jt.zeros(list(want.shape), "float32")
         tx, ts = L.tensor(vx.raw_ptr(), "float32", vx.shape), L.tensor(0, "float32", shape)
