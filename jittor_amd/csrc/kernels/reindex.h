@@ -3,7 +3,7 @@
 // python/jittor/src/ops/reindex_reduce_op.cc:93-131).
 //
 // Constants and fragments supplied by the host:
-//   TX, index_t, VEC, NPARAM, SCATTER (0 gather, 1 scatter), LDIM
+//   TX, index_t, VEC, NPARAM, SCATTER (0 gather, 1 scatter), LDIM, FLAT_VEC and SAFE_LOAD (gather only)
 //   MJT_RX_SETUP    shapes, strides and extras pointers under the names the
 //                   index language uses (xshapeK, yshapeK, xstrideK, ystrideK,
 //                   XDIM, YDIM, eKp, eKstrideJ)
@@ -96,6 +96,28 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     MJT_RX_SETUP
     const index_t j = (index_t)blockIdx.x * 256 + threadIdx.x;
     if (j >= nvec) return;
+#if FLAT_VEC
+    // gather whose innermost extent does not divide into full vectors while y as a whole does: the lane's VEC elements
+    // are adjacent in y's memory and may lie in two rows, so each one is decoded by itself; out-of-range elements load
+    // x[0] and are replaced afterwards, which keeps the VEC loads in flight together (x is not empty)
+    const index_t ebase_ = j * VEC;
+    mjt_pack<TX, VEC> yv;
+    bool out_[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++) {
+        const index_t e = ebase_ + k;
+        MJT_RX_DECODE
+        const index_t MJT_RX_LASTVAR = ilast_;
+        MJT_RX_INDEX
+        out_[k] = ov_;
+        yv.v[k] = xp[ov_ ? (index_t)0 : xid];
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; k++)
+        if (out_[k]) yv.v[k] = ovalue_;
+    mjt_store(yp + ebase_, yv);
+    return;
+#else
     const index_t e = j * VEC;
     MJT_RX_DECODE
     mjt_pack<TX, VEC> yv;
@@ -121,11 +143,18 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 #elif SCATTER
         if (!ov_) { ATOMIC_UPDATE(xp + xid, yv.v[k]); }
 #else
+#if SAFE_LOAD
+        // x is not empty: an out-of-range element loads x[0] and is replaced, so no branch separates the lane's loads
+        const TX got_ = xp[ov_ ? (index_t)0 : xid];
+        yv.v[k] = ov_ ? ovalue_ : got_;
+#else
         if (ov_) yv.v[k] = ovalue_; else yv.v[k] = xp[xid];
+#endif
 #endif
     }
 #if !SCATTER
     mjt_store(yp + e, yv);
+#endif
 #endif
 }
 #endif

@@ -121,6 +121,16 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
     for (int i = 0; i < n_ex; i++) biggest = std::max(biggest, numel(&ex[i]));
     bool use64 = biggest >= (int64_t(1) << 31);   // index_t rule of op.cc:158-192
     int vec = z || sp ? 1 : pick_vec(dtype_size(x->dtype), y->shape[LD - 1], y->ptr);
+    // a gather into rows that do not divide into 16-byte vectors (a padded or cropped innermost axis) still stores 16 bytes
+    // per lane when y as a whole does: the kernel then decodes every element by itself
+    bool flat = false;
+    if (!z && !sp && !scatter && xn > 0 && vec * dtype_size(x->dtype) < 16 && !getenv("MJT_REINDEX_NO_FLAT")) {
+        const int fv = std::min(8, 16 / dtype_size(x->dtype));
+        if (yn % fv == 0 && (uintptr_t)y->ptr % 16 == 0) {
+            vec = fv;
+            flat = true;
+        }
+    }
     int64_t rtail = 1;
     for (int i = LD - nred; z && i < LD; i++) rtail *= y->shape[i];
 
@@ -157,7 +167,7 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
     // (neighbouring lanes then read further apart)
     const int rt_c = z && rtail <= 64 && xn > 0 && !getenv("MJT_GATHER_REDUCE_LOOP") ? (int)rtail : 0;
     const int ov = 1;
-    std::string vkey = std::to_string(vec) + (use64 ? "L" : "I");
+    std::string vkey = std::to_string(vec) + (use64 ? "L" : "I") + (flat ? "F" : "") + (xn > 0 ? "" : "E");
     if (sp) vkey += "|P" + sp->key;
     if (z) {
         vkey += "|R" + std::to_string(rop) + "," + std::to_string(z->dtype) + "," + std::to_string(nred) + "," + std::to_string(rt_c) + "," + std::to_string(ov);
@@ -234,9 +244,10 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
             index << "const index_t xid" << dd << " = (index_t)(" << emit_c(*plan->idx[dd]) << "); ";
         index << "const index_t xid = 0";
         for (int dd = 0; dd < XD; dd++) index << " + xid" << dd << " * xstride" << dd;
+        // combined without short-circuit evaluation: that would put a branch between the loads of a lane's elements
         index << "; bool ov_ = false";
-        for (int dd = 0; dd < XD; dd++) index << " || xid" << dd << " < 0 || xid" << dd << " >= xshape" << dd;
-        for (auto& c : plan->ofc) index << " || (" << emit_c(*c) << ")";
+        for (int dd = 0; dd < XD; dd++) index << " | (xid" << dd << " < 0) | (xid" << dd << " >= xshape" << dd << ")";
+        for (auto& c : plan->ofc) index << " | (bool)(" << emit_c(*c) << ")";
         index << "; ";
 
         std::ostringstream frag;
@@ -250,7 +261,8 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
                  << "\n#define RTAIL_C " << rt_c << "\n#define OV " << ov << "\n";
         frag << "#define MJT_RX_INDEX " << index.str() << "\n";
         if (scatter) frag << "#define ATOMIC_UPDATE(addr, v) mjt_atomic_" << mjt_op_name(op) << "<TX>((addr), (v))\n";
-        frag << "#define REDUCE_TAIL " << (z ? 1 : 0) << "\n";
+        frag << "#define REDUCE_TAIL " << (z ? 1 : 0) << "\n#define FLAT_VEC " << (flat ? 1 : 0) << "\n#define SAFE_LOAD "
+             << (xn > 0 ? 1 : 0) << "\n";
         if (sp) frag << sp->defs(p_sp);
         else frag << "#define SC_PROLOGUE 0\n";
         if (z) {

@@ -183,6 +183,36 @@ def test_reindex_extras_and_dtypes(gpu):
     assert jt.array(a).reindex([0, 4], ["i0", "i1"]).data.shape == (0, 4)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "int8", "int16", "float64", "bfloat16"])
+def test_reindex_rows_that_are_no_whole_vectors(gpu, dtype):
+    """A gather whose innermost extent does not divide into 16-byte vectors while the whole result does: every lane
+    still stores 16 bytes, its elements decoded one by one (they may lie in two rows).  Pads, crops with steps, a
+    flipped axis, an overflow condition; bit-exact against the oracle and against the one-element-per-lane form."""
+    rng = np.random.default_rng(12)
+    x = (rng.standard_normal((3, 5, 14, 9)) * 40).astype(np.float32)
+    xv = jt.array(x).cast(dtype)
+    ref_in = O.BF16(xv.raw()) if dtype == "bfloat16" else xv.data
+    for shape, idx, ov, ofc in [
+            ([3, 5, 16, 11], ["i0", "i1", "i2-1", "i3-1"], 0.0, []),                  # pad 1: rows of 11
+            ([3, 4, 8, 7], ["i0", "i1+1", "i2*2-1", "8-i3"], 2.0, []),                # steps, a flipped innermost axis
+            ([2, 5, 14, 13], ["i0+1", "i1", "13-i2", "i3-2"], -3.0, ["i3>10"]),       # an overflow condition
+            ([16, 1, 3, 5, 3], ["i2", "i3", "i0", "i4*4"], 1.0, []),                  # rows of 3, a permuted source
+            ([3, 5, 14, 5], ["i0", "i1", "i2", "i3+2"], 0.0, [])]:                    # 1050 elements: no vector fits the whole
+        want = O.reindex(ref_in, shape, idx, ov, ofc)
+        want = want.bits if dtype == "bfloat16" else want
+        got = xv.reindex(shape, idx, ov, ofc)
+        got = got.raw() if dtype == "bfloat16" else got.data
+        assert L.last_kernel().startswith("mjt_reindex_")
+        assert np.array_equal(got, want), (dtype, shape)
+        os.environ["MJT_REINDEX_NO_FLAT"] = "1"
+        try:
+            again = xv.reindex(shape, idx, ov, ofc)
+            again = again.raw() if dtype == "bfloat16" else again.data
+        finally:
+            del os.environ["MJT_REINDEX_NO_FLAT"]
+        assert np.array_equal(again, want), (dtype, shape)
+
+
 @pytest.mark.parametrize("case", [
     dict(x=(2, 3, 7, 6), k=(3, 3), s=(1, 1), d=(1, 1), p=(1, 1)),
     dict(x=(3, 9, 11), k=(3, 2), s=(2, 1), d=(1, 2), p=(0, 1)),
