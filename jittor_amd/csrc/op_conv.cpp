@@ -70,7 +70,7 @@ void matmul_impl(const mjt_tensor* a, const mjt_tensor* b, const mjt_tensor* c, 
 bool matmul_available();
 void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                  int64_t lda, int64_t ldb, int64_t ldc, int64_t sa, int64_t sb, int64_t sc, int64_t batch, bool a_kcont,
-                 bool b_kcont);
+                 bool b_kcont, int tile_m = 0, int tile_n = 0, bool allow_direct = true);
 
 // free_extent: y's rows and columns are taken as they are instead of checked against the extents that stride, padding and
 // taps give (output (oh, ow) reads x around (oh*sh - ph, ow*sw - pw) whatever oh and ow; outside the image x is 0): what the
@@ -153,12 +153,16 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                          (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && R * S <= 49 &&
                          // byte offsets inside one image and inside the weights are 32-bit in the kernel
                          C * G * H * W * 2 < (int64_t(1) << 31) && K * OH * OW * 4 < (int64_t(1) << 31) && numel(w) * 2 < (int64_t(1) << 31) &&
-                         // a 1x1 convolution with many more input than output channels is a product with a long inner
-                         // dimension: with few output channels or a small map the matrix-product kernel below streams it
-                         // faster than this kernel walks one-step channel blocks (64 x 256 x 56 x 56 -> 64 channels: 31 us
-                         // against 73; 64 x 1024 x 14 x 14 -> 256: 50 against 142; but 64 x 512 x 28 x 28 -> 128: 50 against 41)
-                         !(R * S == 1 && G == 1 && C >= 4 * K && (K <= 64 || OH * OW <= 256) && p->stride_h == 1 && p->stride_w == 1 &&
-                           matmul_available() && !getenv("MJT_CONV_NO_GEMM"));
+                         // a 1x1 convolution of stride 1 is a matrix product per image: when the rows of a plane are 16-byte
+                         // multiples the product kernel below reads x as it lies and is as fast or faster for every shape
+                         // measured (64 x 512 x 28 x 28 -> 128 channels: 22 us against 42; 64 x 256 x 56 x 56 -> 64: 31 against
+                         // 73; 64 x 1024 x 16 x 16 -> 2048: 82 against 387; closest 64 x 512 x 28 x 28 -> 512: 74 against 74),
+                         // this kernel walking one-step channel blocks.  With other plane sizes the product needs a padded
+                         // copy of x first, which pays with many more input than output channels and few output channels or
+                         // a small map (64 x 1024 x 14 x 14 -> 256: 50 against 142)
+                         !(R * S == 1 && G == 1 && p->stride_h == 1 && p->stride_w == 1 && matmul_available() && !getenv("MJT_CONV_NO_GEMM") &&
+                           ((p->pad_h == 0 && p->pad_w == 0 && OH == H && OW == W && (OH * OW * 2) % 16 == 0 && (uintptr_t)w->ptr % 16 == 0) ||
+                            (C >= 4 * K && (K <= 64 || OH * OW <= 256))));
     if (mfma_ok) {
         // Rows per workgroup: a workgroup walks RPW output rows as NFULL tiles of TR rows plus one
         // shorter tile.  Pick the RPW that minimises (rounds of workgroups over the compute units) x
@@ -303,7 +307,17 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                     MJT_FAIL(MJT_ERR_DEVICE, "conv: writing the column matrices failed: " << mjt_last_error());
             }
             char* yn = (char*)y->ptr + n0 * K * P * dtype_size(y->dtype);
-            gemm_launch(x->dtype, y->dtype, w->ptr, plain ? (void*)xn : cols, yn, K, P, CRS, CRS, Ppad, P, 0, CRS * Ppad, K * P, nb, true, false);
+            // a short sum (a 1x1 convolution, few channels) is bound by how many workgroups a compute unit holds, not by
+            // operand reuse: tiles of 128 x 128 (64 for at most 64 output channels or pixels, or when there would be fewer
+            // tiles than compute units), and the direct-copy kernel with its 256 x 256 tiles only from 256 summed elements on
+            // (16-bit operands; 64 x 512 x 28 x 28 -> 128 channels: 23 us against 48 with the tile the general rule picks;
+            // 64 x 64 x 56 x 56 -> 256: 45 against 54; 64 x 1024 x 28 x 28 -> 256: 63 against 113)
+            const bool short_sum = CRS <= 1024 && esz == 2 && !getenv("MJT_CONV_GEMM_NO_HINT");
+            const int64_t cus = ctx().dry_run || ctx().prop.multiProcessorCount <= 0 ? 256 : ctx().prop.multiProcessorCount;
+            const bool few = ((K + 127) / 128) * ((P + 127) / 128) * nb < cus;       // tiles of 128 x 128 would leave compute units idle
+            const int tile_m = !short_sum ? 0 : K <= 64 || few ? 64 : 128, tile_n = !short_sum ? 0 : P <= 64 || few ? 64 : 128;
+            gemm_launch(x->dtype, y->dtype, w->ptr, plain ? (void*)xn : cols, yn, K, P, CRS, CRS, Ppad, P, 0, CRS * Ppad, K * P, nb, true, false,
+                        tile_m, tile_n, !short_sum || CRS >= 256);
         }
         set_last_kernel(plain ? "conv_as_gemm" : "conv_as_reindex_gemm");
         return;

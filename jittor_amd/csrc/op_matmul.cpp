@@ -47,7 +47,7 @@ int env_int(const char* name, int dflt) {
 // k innermost (a as given, b transposed).
 void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                  int64_t lda, int64_t ldb, int64_t ldc, int64_t sa, int64_t sb, int64_t sc, int64_t batch, bool a_kcont,
-                 bool b_kcont) {
+                 bool b_kcont, int tile_m = 0, int tile_n = 0, bool allow_direct = true) {
     Context& c = ctx();
     const int esz = dtype_size(in_dtype);
     const bool mfma_type = in_dtype == MJT_BFLOAT16 || in_dtype == MJT_FLOAT16 || in_dtype == MJT_FLOAT32;
@@ -63,7 +63,7 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
     // without passing through registers (any of the four layouts).  Offsets inside an operand's tile are 32-bit there:
     // 256 rows of an operand with k innermost, all K rows of one with m or n innermost.
     auto fits32 = [&](bool kcont, int64_t ld) { return (kcont ? ld * 2 * 256 : ld * 2 * K) < (int64_t(1) << 31); };
-    if (fast && esz == 2 && K % 64 == 0 && !getenv("MJT_GEMM_NO_DMA") && fits32(a_kcont, lda) && fits32(b_kcont, ldb)) {
+    if (fast && allow_direct && esz == 2 && K % 64 == 0 && !getenv("MJT_GEMM_NO_DMA") && fits32(a_kcont, lda) && fits32(b_kcont, ldb)) {
         const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
         const int64_t tm = (M + 255) / 256, tn = (N + 255) / 256;
         const double edge = ((double)M * N) / ((double)tm * 256 * tn * 256);
@@ -109,6 +109,9 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
                 const double score = edge * util * (0.55 + 0.45 * reuse);
                 if (score > best) { best = score; best_mi = mi; best_ni = ni; }
             }
+        // the caller's tile, if it names one (tile_m x tile_n of 64, 128 or 256)
+        if (tile_m == 64 || tile_m == 128 || tile_m == 256) best_mi = tile_m / 64;
+        if (tile_n == 64 || tile_n == 128 || tile_n == 256) best_ni = tile_n / 64;
         int MI = env_int("MJT_GEMM_MI", best_mi), NI = env_int("MJT_GEMM_NI", best_ni);
         if ((MI != 1 && MI != 2 && MI != 4) || (NI != 1 && NI != 2 && NI != 4)) { MI = best_mi; NI = best_ni; }
         const int in = in_dtype == MJT_BFLOAT16 ? 0 : in_dtype == MJT_FLOAT16 ? 1 : 2;

@@ -585,7 +585,7 @@ def _conv_call(xbits, wbits, params, out_dtype="float32", in_dtype="bfloat16"):
     dict(x=(1, 128, 56, 56), w=(128, 128, 3, 3), p=(1, 1, 1, 1, 1, 1)),    # the benchmark geometry, fewer channels
     dict(x=(3, 64, 28, 24), w=(256, 64, 3, 3), p=(2, 2, 1, 1, 1, 1)),      # stride 2
     dict(x=(2, 64, 20, 32), w=(128, 64, 3, 3), p=(1, 1, 2, 2, 2, 2)),      # dilation 2
-    dict(x=(2, 192, 14, 8), w=(128, 192, 1, 1), p=(1, 1, 0, 0, 1, 1)),     # 1x1, three channel blocks
+    dict(x=(2, 192, 14, 8), w=(128, 192, 1, 1), p=(1, 1, 0, 0, 1, 1), nogemm=True),     # 1x1, three channel blocks (kept off the matrix-product route)
     dict(x=(1, 64, 9, 40), w=(128, 64, 5, 3), p=(1, 1, 2, 1, 1, 1)),       # 5x3 taps, odd height
     dict(x=(2, 64, 12, 72), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),       # 72 columns: two staging segments; 64 output channels
     dict(x=(2, 64, 10, 16), w=(128, 64, 3, 3), p=(1, 1, 0, 0, 1, 1)),      # output width 14: 4-byte store epilogue
@@ -610,6 +610,8 @@ def test_conv_mfma_matches_oracle(gpu, case):
     sh, sw, ph, pw, dh, dw = case["p"]
     if "rpw" in case:
         os.environ["MJT_CONV_RPW"] = str(case["rpw"])      # rows per workgroup, forced: the heuristic would pick it only for large batches
+    if case.get("nogemm"):
+        os.environ["MJT_CONV_NO_GEMM"] = "1"
     try:
         got, kern = _conv_call(xb, wb, case["p"])
         if "out" in case:                                  # narrower output = truncation of the same accumulators
@@ -617,6 +619,7 @@ def test_conv_mfma_matches_oracle(gpu, case):
             assert kern16.startswith("mjt_conv_mfma_bf16") and np.array_equal(got16, O.f32_to_bf16_bits(got))
     finally:
         os.environ.pop("MJT_CONV_RPW", None)
+        os.environ.pop("MJT_CONV_NO_GEMM", None)
     assert kern.startswith("mjt_conv_mfma_bf16"), kern
     if sh == sw and ph == pw and dh == dw:
         ref = K.conv_meta_bf16(xb, wb, sh, ph, dh, 8)
@@ -826,23 +829,33 @@ def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
     assert np.abs(widen[out](got2) - ref).max() <= tol * np.abs(ref).max()
 
 
-def test_conv_1x1_with_many_more_input_channels_runs_as_a_product(gpu, monkeypatch):
-    """A 1x1 convolution whose input channels outnumber its output channels 4 : 1 or more, with at most 64 output
-    channels or a map of at most 256 pixels, is handed to the matrix-product kernel although the MFMA convolution
-    kernel would take it (a long inner dimension in one-step channel blocks is that kernel's worst case); both
-    against a float64 product, same bound."""
+def test_conv_1x1_runs_as_a_product(gpu, monkeypatch):
+    """A 1x1 convolution of stride 1 is handed to the matrix-product kernel although the MFMA convolution kernel would
+    take it: always when a plane's rows are 16-byte multiples (the product then reads x as it lies, with tiles picked for
+    a short sum), and through a padded copy when its input channels outnumber its output channels 4 : 1 or more with at
+    most 64 output channels or a map of at most 256 pixels.  Both kernels against a float64 product, same bound; 16-bit
+    and float32 results."""
     rng = np.random.default_rng(43)
-    for xs, ws in (((2, 256, 16, 16), (64, 256, 1, 1)), ((3, 512, 14, 14), (128, 512, 1, 1))):
+    for xs, ws, out, want in (((2, 256, 16, 16), (64, 256, 1, 1), "float32", "conv_as_gemm"),
+                              ((3, 512, 14, 14), (128, 512, 1, 1), "float32", "conv_as_reindex_gemm"),
+                              ((3, 64, 24, 28), (256, 64, 1, 1), "bfloat16", "conv_as_gemm"),        # one step of the sum, tiles of 128
+                              ((5, 128, 12, 20), (192, 128, 1, 1), "float32", "conv_as_gemm"),       # 240 pixels, 192 channels: edge tiles
+                              ((2, 1024, 8, 8), (128, 1024, 1, 1), "bfloat16", "conv_as_gemm"),      # 64 pixels: narrow tiles
+                              ((70, 64, 16, 16), (192, 64, 1, 1), "bfloat16", "conv_as_gemm"),       # more tiles than compute units
+                              ((2, 64, 9, 12), (64, 64, 1, 1), "float32", "mjt_conv_mfma_bf16")):    # rows of 216 bytes: stays
         xb, wb = _bf16(rng.standard_normal(xs)), _bf16(rng.standard_normal(ws) * 0.1)
         ref = np.einsum("nchw,kc->nkhw", O.BF16(xb).to_f32().astype(np.float64), O.BF16(wb).to_f32().astype(np.float64)[:, :, 0, 0])
-        got, kern = _conv_call(xb, wb, (1, 1, 0, 0, 1, 1))
-        assert kern in ("conv_as_gemm", "conv_as_reindex_gemm"), kern
-        assert np.abs(got - ref).max() <= 1e-4 * np.abs(ref).max()
+        mag = np.einsum("nchw,kc->nkhw", np.abs(O.BF16(xb).to_f32().astype(np.float64)), np.abs(O.BF16(wb).to_f32().astype(np.float64))[:, :, 0, 0])
+        widen = (lambda a: O.BF16(a).to_f32().astype(np.float64)) if out == "bfloat16" else (lambda a: a.astype(np.float64))
+        bound = 1e-4 * mag + (np.abs(ref) * 2.0 ** -7 if out == "bfloat16" else 0.0) + 1e-30
+        got, kern = _conv_call(xb, wb, (1, 1, 0, 0, 1, 1), out_dtype=out)
+        assert kern.startswith(want), (kern, xs)
+        assert (np.abs(widen(got) - ref) <= bound).all(), (xs, ws)
         monkeypatch.setenv("MJT_CONV_NO_GEMM", "1")
-        got2, kern2 = _conv_call(xb, wb, (1, 1, 0, 0, 1, 1))
+        got2, kern2 = _conv_call(xb, wb, (1, 1, 0, 0, 1, 1), out_dtype=out)
         monkeypatch.delenv("MJT_CONV_NO_GEMM")
         assert kern2.startswith("mjt_conv_mfma_bf16"), kern2
-        assert np.abs(got2 - ref).max() <= 1e-4 * np.abs(ref).max()
+        assert (np.abs(widen(got2) - ref) <= bound).all(), (xs, ws)
 
 
 def test_conv_grouped_entry_and_front_end(gpu):
