@@ -29,9 +29,10 @@
 // hardware checks).  While the MFMAs of a step run, the loads of the next step fill a second set
 // of slots (when two sets fit into LDS; otherwise the same set, after a second barrier).
 //
-// A workgroup owns 64*KG output channels x 16*8/KG input channels x all taps, over the images
-// [slice*ips, slice*ips+ips): the partial sums of the slices go to partial[slice][k][c][r][s]
-// (float32) and are added up by a reduce launch.
+// A workgroup owns 64*KG output channels x 16*8/KG input channels x all taps, over the output rows
+// [slice*rps, slice*rps+rps) of the batch (row n*OH + oh: a slice may be a part of an image or span
+// several): the partial sums of the slices go to partial[slice][k][c][r][s] (float32) and are added
+// up by a reduce launch.
 
 #if IN_F16
 typedef _Float16 mjt_bf16x8 __attribute__((ext_vector_type(8)));
@@ -65,10 +66,11 @@ __device__ constexpr bool mjt_edge(int ch, int s) {
 
 extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     const int n_img = (int)(unsigned long long)p.a[3];
-    const int ips = (int)(unsigned long long)p.a[4];
+    const int rps = (int)(unsigned long long)p.a[4];                    // output rows (of all images, in order) per slice
     float* __restrict__ partial = (float*)p.a[2];
 
-    constexpr int KBLOCKS = K_ / (64 * KG), CBLOCKS = C_ / (16 * CTW);
+    // the last block of input channels may reach beyond C_ (a multiple of 16): its tiles there read zeros and write nothing
+    constexpr int KBLOCKS = K_ / (64 * KG), CBLOCKS = (C_ + 16 * CTW - 1) / (16 * CTW);
     // the workgroups of one slice read the same dy: they are 8 apart, so that they land on the same XCD
     // (workgroups go round-robin over the 8 XCDs) and share it through that XCD's L2
     const int id = blockIdx.x;
@@ -76,9 +78,11 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     const int kblock = j % KBLOCKS;
     const int cblock = (j / KBLOCKS) % CBLOCKS;
     const int slice = (j / (KBLOCKS * CBLOCKS)) * 8 + xcd;
-    if (slice * ips >= n_img) return;                       // the grid is padded to a multiple of 8 slices
-    const int img_begin = slice * ips;
-    const int img_end = img_begin + ips < n_img ? img_begin + ips : n_img;
+    const int n_rows = n_img * OH_;
+    if (slice * rps >= n_rows) return;                      // the grid is padded to a multiple of 8 slices
+    const int row_begin = slice * rps;
+    const int row_end = row_begin + rps < n_rows ? row_begin + rps : n_rows;
+    const int img_begin = row_begin / OH_, oh_begin = row_begin - img_begin * OH_;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -145,7 +149,7 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     const unsigned e_lane = (unsigned)(frow * H_ * W_ * 2) + (fpiece == 2 ? (unsigned)-4 : (unsigned)(64 + 4 * fpiece));
     auto fetch = [&](unsigned char* area, int img, int oh, int ch) -> int {
         int issued = 0;                                                  // by this wave
-        const bool img_ok = img < img_end && oh < OH_;
+        const bool img_ok = img * OH_ + oh < row_end;
 #pragma unroll
         for (int it0 = 0; it0 < NA + 2 * NB; it0 += 8) {
             const int it = it0 + wave;
@@ -160,8 +164,8 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
                 const int j = it - NA - (edge ? NB : 0);
                 const int tile = j / R_, r = j - tile * R_;
                 const int ih = oh * SH - PH + r * DH;
-                const bool ok = img_ok && ih >= 0 && ih < H_;
                 const int cc = (cblock * CTW + tile) * 16;
+                const bool ok = img_ok && ih >= 0 && ih < H_ && cc < C_;
                 const unsigned base = ok ? (unsigned)((((img * C_ + cc) * H_ + ih) * W_ + ch * 32) * 2) : 0u;
                 if (!edge) {
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + AREA_B + j * 1024), 16,
@@ -275,27 +279,30 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
             if (++oh >= OH_) { oh = 0; img++; }
         }
     };
-    fetch_unit(stage, img_begin, 0, 0);
+    fetch_unit(stage, img_begin, oh_begin, 0);
     if constexpr (NBUF == 3) {
-        int i1 = img_begin, o1 = 0, c1 = 0;
+        int i1 = img_begin, o1 = oh_begin, c1 = 0;
         advance(i1, o1, c1, 1);
         newest = fetch_unit(stage + UAREA, i1, o1, c1);
     }
-    for (int img = img_begin; img < img_end; img++) {
+    {
+        int img = img_begin, oh = oh_begin;
 #pragma unroll 1
-        for (int oh = 0; oh < OH_; oh++) {
+        for (int row = row_begin; row < row_end; row++) {
             mjt_static_for<0, NCHUNK / UNIT>([&](auto cc) {
                 constexpr int ch0 = decltype(cc)::v * UNIT;
                 int ni = img, no = oh, nc = ch0;
-                advance(ni, no, nc, AHEAD);                              // beyond the slice: img_end, read as zeros
+                advance(ni, no, nc, AHEAD);                              // beyond the slice: read as zeros
                 unit(mjt_ic<ch0>(), ni, no, nc);
             });
+            if (++oh >= OH_) { oh = 0; img++; }
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                     // nothing may arrive in LDS after the wave has ended
 
     // lane holds D[k = 4*lg + i][c = l16] of each (channel tile m, tap)
     const size_t KC = (size_t)K_ * C_;
+    if (c0 >= C_) return;
 #pragma unroll
     for (int m = 0; m < 4; m++)
 #pragma unroll

@@ -470,7 +470,7 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
     const int64_t CTW = 8 / KG;
     const bool half = x->dtype == MJT_FLOAT16;
     const bool ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && dy->dtype == x->dtype && (dw->dtype == MJT_FLOAT32 || dw->dtype == x->dtype) &&
-                    p->stride_w == 1 && p->pad_w <= 2 && (S - 1) * p->dil_w - p->pad_w <= 4 && K % 64 == 0 && C % (16 * CTW) == 0 && R * S <= 9 && OW % 8 == 0 &&
+                    p->stride_w == 1 && p->pad_w <= 2 && (S - 1) * p->dil_w - p->pad_w <= 4 && K % 64 == 0 && C % 16 == 0 && (C % (16 * CTW) == 0 || C % (16 * CTW) >= 8 * CTW) && R * S <= 9 && OW % 8 == 0 &&
                     W % 2 == 0 && N >= 1 && numel(x) * 2 < (int64_t(1) << 31) && numel(dy) * 2 < (int64_t(1) << 31) &&
                     (uintptr_t)x->ptr % 4 == 0 && (uintptr_t)dy->ptr % 16 == 0 &&
                     !getenv("MJT_NO_FASTPATH");
@@ -480,18 +480,23 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
     }
     if (!ok)
         MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: only bfloat16 or float16 operands with horizontal stride 1, column shifts of the taps within -2 .. 4, at most 9 taps, "
-                                      "K % 64 == 0, C % " << 16 * CTW << " == 0, OW % 8 == 0 and tensors below 2 GB run on the MFMA kernel");
+                                      "K % 64 == 0, C % 16 == 0 (the last block of " << 16 * CTW << " channels at least half full), OW % 8 == 0 and tensors below 2 GB run on the MFMA kernel");
     Context& c = ctx();
     const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
-    const int64_t blocks_per_slice = (K / (64 * KG)) * (C / (16 * CTW));
-    // slices of whole images: enough workgroups for every compute unit, at most one image per slice
+    const int64_t blocks_per_slice = (K / (64 * KG)) * ((C + 16 * CTW - 1) / (16 * CTW));   // the last block of channels may be partly idle
+    // slices of consecutive output rows of the batch (a part of an image, or several images): enough workgroups for every
+    // compute unit, at least 4 rows per slice (with whole images per slice, 64 x 64 x 56 x 56 with 3x3 taps ran 64
+    // workgroups: 158 us)
+    const int64_t rows = N * OH;
     int64_t slices = (cus + blocks_per_slice - 1) / blocks_per_slice;
-    if (slices > N) slices = N;
+    if (slices > (rows + 3) / 4) slices = (rows + 3) / 4;
     if (slices < 1) slices = 1;
-    int64_t ips = (N + slices - 1) / slices;
+    int64_t rps = (rows + slices - 1) / slices;
     if (const char* e = getenv("MJT_WGRAD_IPS"))             // images per slice, for experiments
-        if (atoi(e) >= 1) ips = atoi(e) < N ? atoi(e) : N;
-    slices = (N + ips - 1) / ips;
+        if (atoi(e) >= 1) rps = (atoi(e) < N ? atoi(e) : N) * OH;
+    if (const char* e = getenv("MJT_WGRAD_RPS"))             // rows per slice, likewise
+        if (atoi(e) >= 1) rps = atoi(e) < rows ? atoi(e) : rows;
+    slices = (rows + rps - 1) / rps;
 
     std::ostringstream key;
     key << "wgrad|" << C << "|" << H << "|" << W << "|" << K << "|" << R << "|" << S << "|" << OH << "|" << OW << "|" << p->stride_h << "|"
@@ -511,7 +516,7 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
         remember(key.str(), k);
     }
     void* part = wgrad_partials((size_t)slices * (size_t)numel(dw) * 4);
-    std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(dy->ptr), bits_of_ptr(part), (uint64_t)N, (uint64_t)ips, 0};
+    std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(dy->ptr), bits_of_ptr(part), (uint64_t)N, (uint64_t)rps, 0};
     jit_launch(k, (unsigned)((slices + 7) / 8 * 8 * blocks_per_slice), 1, 512, 0, a);
     fold_wgrad_slices(part, slices, dw);
     set_last_kernel(k->name.c_str());

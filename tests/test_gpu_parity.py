@@ -948,6 +948,12 @@ def _wgrad_call(xbits, dybits, R, S, params, out_dtype="float32", in_dtype="bflo
     dict(x=(2, 128, 8, 16), k=64, rs=(3, 3), p=(1, 1, 2, 2, 2, 2)),       # dilation 2, padding 2: shifts -2, 0, 2
     dict(x=(2, 128, 6, 12), k=64, rs=(2, 3), p=(1, 1, 0, 0, 1, 2)),       # horizontal dilation 2, no padding: shifts 0, 2, 4
     dict(x=(2, 32, 6, 16), k=256, rs=(3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16"),
+    dict(x=(3, 64, 10, 24), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),       # 64 of a block's 128 input channels: half of the waves idle
+    dict(x=(2, 192, 5, 8), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),        # a full block of input channels and half a block
+    dict(x=(2, 48, 6, 16), k=128, rs=(1, 1), p=(1, 1, 0, 0, 1, 1)),       # blocks of 64 channels: 48
+    dict(x=(3, 128, 9, 8), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1), rps=5),    # slices of 5 output rows: they start and end inside images
+    dict(x=(3, 128, 9, 40), k=64, rs=(3, 3), p=(2, 1, 1, 1, 1, 1), rps=4),   # 5 output rows per image (stride 2), slices of 4; two chunks
+    dict(x=(2, 128, 7, 8), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1), rps=1),    # one row per slice
 ])
 def test_conv_wgrad_mfma_matches_oracle(gpu, case, monkeypatch):
     """The weight gradient kernel through the C entry point against the oracle's restatement of the
@@ -963,6 +969,8 @@ def test_conv_wgrad_mfma_matches_oracle(gpu, case, monkeypatch):
     out = case.get("out", "float32")
     if "ips" in case:
         monkeypatch.setenv("MJT_WGRAD_IPS", str(case["ips"]))
+    if "rps" in case:
+        monkeypatch.setenv("MJT_WGRAD_RPS", str(case["rps"]))
     rc, got = _wgrad_call(xb, db, R, S, case["p"], out)
     assert rc == 0 and L.last_kernel().startswith("mjt_conv_wgrad_mfma_bf16")
     xf, df = O.BF16(xb).to_f32().astype(np.float64), O.BF16(db).to_f32().astype(np.float64)
