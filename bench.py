@@ -344,6 +344,116 @@ def wl_copy(L, lib, steps, warmup, with_cpu):
             "roofline": roofline("hbm", 2 * n, ms), **LAST_SPREAD}
 
 
+def _rotating(L, dev, nbytes_in, nbytes_out, make_call, fill=None):
+    """Enough (input, output) buffer pairs that a pass over them exceeds the memory-side cache."""
+    sets = max(2, CACHE_BYTES * 2 // max(nbytes_in + nbytes_out, 1) + 1)
+    calls = []
+    for s in range(sets):
+        pin = dev.put(fill) if fill is not None else dev.empty(nbytes_in)
+        calls.append(make_call(pin, dev.empty(nbytes_out)))
+    return calls
+
+
+def wl_callers(L, lib, steps, warmup, with_cpu):
+    """The callers either side of the five configurations, each as the one entry-point call the front end makes for it, on
+    buffers that rotate through more than the memory-side cache: layout changes, pad, crop, pooling, a column reduce, the
+    two gradients of a convolution and a 1x1 convolution.  Not part of the default run (--only CALLERS); no CPU legs."""
+    from jittor_amd.dtypes import f32_to_bf16_bits
+    rng = np.random.default_rng(0)
+    none, noex = L.c_strings([]), (L.Tensor * 1)()
+    out = {}
+
+    def reindex_case(name, xs, ys, idx, dtype="float32", esz=4):
+        dev = Dev(L)
+        nin, nout = int(np.prod(xs)) * esz, int(np.prod(ys)) * esz
+        x = rng.standard_normal(xs).astype(np.float32)
+        ci = L.c_strings(idx)
+
+        def make(pin, pout):
+            tx, ty = L.tensor(pin, dtype, xs), L.tensor(pout, dtype, ys)
+            return lambda: L.check(lib.mjt_reindex(ctypes.byref(tx), ctypes.byref(ty), len(idx), ci, 0.0, 0, none, 0, noex))
+        calls = _rotating(L, dev, nin, nout, make, fill=x)
+        ms, wall = time_calls(L, calls, steps, warmup)
+        work = min(nin, nout) + nout               # every output written once; no more input read than there is output
+        out[name] = {"workload": "%s: mjt_reindex %s -> %s %s" % (name, list(xs), list(ys), idx), "kernel": L.last_kernel(), "dtype": "f32",
+                     "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5), "roofline": roofline("hbm", work, ms), **LAST_SPREAD}
+        dev.release()
+
+    reindex_case("NHWC", (64, 128, 64, 64), (64, 64, 64, 128), ["i0", "i3", "i1", "i2"])
+    reindex_case("TRANSPOSE", (64, 512, 1024), (64, 1024, 512), ["i0", "i2", "i1"])
+    reindex_case("PAD", (64, 128, 64, 64), (64, 128, 66, 66), ["i0", "i1", "i2-1", "i3-1"])
+    reindex_case("CROP", (64, 512, 1024), (64, 256, 997), ["i0", "i1*2", "i2+3"])
+    reindex_case("FLIP", (64, 512, 1024), (64, 512, 1024), ["i0", "i1", "1023-i2"])
+
+    # 2 x 2 maximum pooling as the fused gather + reduce
+    dev = Dev(L)
+    xs, loop, zs = (64, 128, 64, 64), (64, 128, 32, 32, 2, 2), (64, 128, 32, 32)
+    x = rng.standard_normal(xs).astype(np.float32)
+    idx = ["i0", "i1", "i2*2+i4", "i3*2+i5"]
+    ci = L.c_strings(idx)
+
+    def make_pool(pin, pout):
+        tx, ts, tz = L.tensor(pin, "float32", xs), L.tensor(0, "float32", loop), L.tensor(pout, "float32", zs)
+        return lambda: L.check(lib.mjt_reindex_then_reduce(ctypes.byref(tx), ctypes.byref(ts), ctypes.byref(tz), L.OP_CODE["maximum"], 2,
+                                                           4, ci, -3.0e38, 0, none, 0, noex))
+    calls = _rotating(L, dev, x.nbytes, x.nbytes // 4, make_pool, fill=x)
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out["POOL"] = {"workload": "POOL: mjt_reindex_then_reduce maximum over 2x2 windows of fp32 [64,128,64,64]", "kernel": L.last_kernel(),
+                   "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+                   "roofline": roofline("hbm", x.nbytes + x.nbytes // 4, ms), **LAST_SPREAD}
+    dev.release()
+
+    # a column reduce: sum over axis 0 of [65536, 512]
+    dev = Dev(L)
+    x = rng.standard_normal((65536, 512)).astype(np.float32)
+
+    def make_col(pin, pout):
+        tx, ty = L.tensor(pin, "float32", x.shape), L.tensor(pout, "float32", [512])
+        return lambda: L.check(lib.mjt_reduce(ctypes.byref(tx), ctypes.byref(ty), L.OP_CODE["add"], 0b01))
+    calls = _rotating(L, dev, x.nbytes, 2048, make_col, fill=x)
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out["REDUCE_AXIS0"] = {"workload": "REDUCE_AXIS0: mjt_reduce sum over axis 0 of fp32 [65536,512]", "kernel": L.last_kernel(), "dtype": "f32",
+                           "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5), "roofline": roofline("hbm", x.nbytes + 2048, ms),
+                           **LAST_SPREAD, "note": "a step = the split kernel and the fold of its partial sums"}
+    dev.release()
+
+    # convolutions of a ResNet-50 stage-1 / stage-2 block at batch 64, bfloat16 operands and results
+    def conv_case(name, entry, xs, ws, params, bound, note):
+        dev = Dev(L)
+        N, C, H, W = xs
+        K, _, R, S = ws
+        sh, sw, ph, pw, dh, dw_ = params
+        OH, OW = (H + 2 * ph - dh * (R - 1) - 1) // sh + 1, (W + 2 * pw - dw_ * (S - 1) - 1) // sw + 1
+        ys = (N, K, OH, OW)
+        xb = f32_to_bf16_bits(rng.standard_normal(xs).astype(np.float32))
+        wb = f32_to_bf16_bits((rng.standard_normal(ws) * 0.05).astype(np.float32))
+        yb = f32_to_bf16_bits(rng.standard_normal(ys).astype(np.float32))
+        p = L.ConvParams(*params)
+        calls = []
+        for s in range(3):
+            tx, tw, ty = L.tensor(dev.put(xb), "bfloat16", xs), L.tensor(dev.put(wb), "bfloat16", ws), L.tensor(dev.put(yb), "bfloat16", ys)
+            if entry == "fwd":
+                calls.append(lambda tx=tx, tw=tw, ty=ty: L.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p))))
+            elif entry == "dgrad":
+                calls.append(lambda tx=tx, tw=tw, ty=ty: L.check(lib.mjt_conv2d_meta_dgrad(ctypes.byref(ty), ctypes.byref(tw), ctypes.byref(tx), ctypes.byref(p))))
+            else:
+                calls.append(lambda tx=tx, tw=tw, ty=ty: L.check(lib.mjt_conv2d_meta_wgrad(ctypes.byref(tx), ctypes.byref(ty), ctypes.byref(tw), ctypes.byref(p))))
+        ms, wall = time_calls(L, calls, steps, warmup)
+        flops = 2.0 * N * K * OH * OW * C * R * S
+        nbytes = xb.nbytes + yb.nbytes + wb.nbytes
+        out[name] = {"workload": "%s: %s of x bf16 %s, w bf16 %s, stride %d pad %d" % (name, entry, list(xs), list(ws), sh, ph),
+                     "kernel": L.last_kernel(), "dtype": "bf16", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+                     "roofline": roofline(bound, flops if bound == "mfma" else nbytes, ms), **LAST_SPREAD, "note": note}
+        dev.release()
+
+    conv_case("CONV1x1", "fwd", (64, 512, 28, 28), (128, 512, 1, 1), (1, 1, 0, 0, 1, 1), "hbm", "on the matrix-product kernel; bytes = x + w + y once")
+    conv_case("CONV1x1_UP", "fwd", (64, 64, 56, 56), (256, 64, 1, 1), (1, 1, 0, 0, 1, 1), "hbm", "on the matrix-product kernel; bytes = x + w + y once")
+    conv_case("DGRAD_S2", "dgrad", (64, 256, 56, 56), (256, 256, 3, 3), (2, 2, 1, 1, 1, 1), "mfma", "one convolution per stride phase, then the interleave")
+    conv_case("WGRAD_64", "wgrad", (64, 64, 56, 56), (64, 64, 3, 3), (1, 1, 1, 1, 1, 1), "hbm", "MFMA kernel over slices of output rows + fold; bytes = x + dy + dw once")
+    conv_case("WGRAD_1x1", "wgrad", (64, 64, 56, 56), (256, 64, 1, 1), (1, 1, 0, 0, 1, 1), "hbm", "MFMA kernel over slices of output rows + fold; bytes = x + dy + dw once")
+    return {"workload": "CALLERS", "cases": out}
+
+
 # HBM bytes per launch of the workload's kernels, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # runs of this file (KiB per dispatch), each scaled by what the same counter reads for the COPY workload
 # (FETCH_SIZE reads 131082 KiB for 262144 KiB fetched: factor 2.0; WRITE_SIZE reads 262144 KiB: factor 1.0).
@@ -400,6 +510,7 @@ WORKLOADS = {
     "GEMM": wl_gemm,
     "GEMMnn": lambda *a: wl_gemm(*a, trans_b=0),
     "COPY": wl_copy,
+    "CALLERS": wl_callers,
 }
 DEFAULT = ["C1", "C2", "C3add", "C3max", "C4", "C5", "C5bf16out"]
 
