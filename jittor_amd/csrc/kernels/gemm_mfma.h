@@ -46,6 +46,9 @@ typedef unsigned short TIN;
 #define TN (64 * NI)
 #define ROWB 144                 // bytes per LDS row: 8 chunks + 1 of padding
 #define NTHR 256
+#ifndef NBUF
+#define NBUF 2                   // staging buffers: 2, or 1 for a product of a single stage (K <= KS)
+#endif
 
 typedef float mjt_f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
@@ -204,7 +207,8 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const long long lda = (long long)p.a[6], ldb = (long long)p.a[7], ldc = (long long)p.a[8];
     const TIN* __restrict__ A = (const TIN*)p.a[0] + (long long)blockIdx.y * (long long)p.a[9];
     const TIN* __restrict__ B = (const TIN*)p.a[1] + (long long)blockIdx.y * (long long)p.a[10];
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2][(TM + TN) * ROWB];
+    // NBUF 1: the host promises K <= KS, a single stage -- one staging buffer, so twice as many workgroups fit a compute unit
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF][(TM + TN) * ROWB];
 
     // Tile order: panels of 4 tile rows, inside a panel column by column.  Workgroups go round-robin over the
     // 8 XCDs, so workgroup id takes tile (id % 8) * per_xcd + id / 8: every XCD works on a compact run of
@@ -249,10 +253,10 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
 
     // fragment addresses of this lane: row lane % 32 of its wave's tile rows, chunk lane / 32
     const int frow = lane & 31, fhalf = lane >> 5;
-    const int nstages = (K + KS - 1) / KS;
+    const int nstages = NBUF == 1 ? 1 : (K + KS - 1) / KS;
     for (int s = 0; s < nstages; s++) {
-        const unsigned char* la = &lds[s & 1][0] + (wm * 32 * MI + frow) * ROWB + fhalf * 16;
-        const unsigned char* lb = &lds[s & 1][TM * ROWB] + (wn * 32 * NI + frow) * ROWB + fhalf * 16;
+        const unsigned char* la = &lds[s & (NBUF - 1)][0] + (wm * 32 * MI + frow) * ROWB + fhalf * 16;
+        const unsigned char* lb = &lds[s & (NBUF - 1)][TM * ROWB] + (wn * 32 * NI + frow) * ROWB + fhalf * 16;
         if (s + 1 < nstages) {
             sa.fetch(A, lda, m0, arows, (s + 1) * KS, K, tid);
             sb.fetch(B, ldb, n0, brows, (s + 1) * KS, K, tid);
@@ -290,8 +294,8 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
 #endif
         });
         if (s + 1 < nstages) {
-            sa.commit(&lds[(s + 1) & 1][0], (s + 1) * KS, K, tid);             // the other buffer: nobody reads it now
-            sb.commit(&lds[(s + 1) & 1][TM * ROWB], (s + 1) * KS, K, tid);
+            sa.commit(&lds[(s + 1) & (NBUF - 1)][0], (s + 1) * KS, K, tid);             // the other buffer: nobody reads it now
+            sb.commit(&lds[(s + 1) & (NBUF - 1)][TM * ROWB], (s + 1) * KS, K, tid);
             __syncthreads();
         }
     }

@@ -116,14 +116,16 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
         if ((MI != 1 && MI != 2 && MI != 4) || (NI != 1 && NI != 2 && NI != 4)) { MI = best_mi; NI = best_ni; }
         const int in = in_dtype == MJT_BFLOAT16 ? 0 : in_dtype == MJT_FLOAT16 ? 1 : 2;
         const int out = out_dtype == MJT_BFLOAT16 ? 0 : out_dtype == MJT_FLOAT16 ? 1 : 2;
+        const bool one_stage = K <= (esz == 2 ? 64 : 32) && !getenv("MJT_GEMM_TWO_BUFFERS");       // a single stage of the kernel's k loop
         std::ostringstream key;
-        key << "gemm|" << in << out << MI << NI << a_kcont << b_kcont;
+        key << "gemm|" << in << out << MI << NI << a_kcont << b_kcont << one_stage;
         JitKernel* k = cached(key.str());
         if (!k) {
             std::ostringstream name;
             name << "mjt_gemm_mfma_" << mjt_dtype_name(in_dtype) << "_" << mjt_dtype_name(out_dtype) << "_" << 64 * MI << "x" << 64 * NI
-                 << (a_kcont ? "_n" : "_t") << (b_kcont ? "t" : "n");
+                 << (a_kcont ? "_n" : "_t") << (b_kcont ? "t" : "n") << (one_stage ? "_k1" : "");
             std::ostringstream src;
+            src << "#define NBUF " << (one_stage ? 1 : 2) << "\n";
             src << "#define ENTRY " << name.str() << "\n#define IN " << in << "\n#define OUT " << out << "\n#define MI " << MI
                 << "\n#define NI " << NI << "\n#define A_KCONT " << (a_kcont ? 1 : 0) << "\n#define B_KCONT " << (b_kcont ? 1 : 0) << "\n";
             src << embedded_source("gemm_mfma.h") << "\n";

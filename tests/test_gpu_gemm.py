@@ -135,6 +135,20 @@ def test_gemm_k_tail_inside_a_chunk(gpu):
     assert _run(lib, "float16", "float32", 96, 8, 64, 0, 1).startswith("mjt_gemm_mfma_")
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_single_stage_uses_one_staging_buffer(gpu, ta, tb, monkeypatch):
+    """A sum that fits one stage of the k loop (64 elements of 16 bits, 32 of float32) runs on a variant of the kernel
+    with one staging buffer; one element more and it is the two-buffer kernel again.  Tiles over every edge, a batch."""
+    lib = L.load()
+    for dt, K in (("bfloat16", 64), ("float16", 40), ("float32", 32), ("float32", 8)):
+        assert _run(lib, dt, dt, 304, K, 264, ta, tb, seed=K).endswith("_k1")
+        assert _run(lib, dt, "float32", 72, K, 520, ta, tb, seed=K + 1, batch=(3,)).endswith("_k1")
+    assert not _run(lib, "bfloat16", "bfloat16", 304, 72, 264, ta, tb, seed=3).endswith("_k1")
+    assert not _run(lib, "float32", "float32", 304, 36, 264, ta, tb, seed=4).endswith("_k1")
+    monkeypatch.setenv("MJT_GEMM_TWO_BUFFERS", "1")
+    assert not _run(lib, "bfloat16", "bfloat16", 304, 64, 264, ta, tb, seed=64).endswith("_k1")
+
+
 @pytest.mark.parametrize("dt", ["bfloat16", "float32", "float64"])
 def test_gemm_plain_unaligned_and_float64(gpu, dt):
     lib = L.load()
