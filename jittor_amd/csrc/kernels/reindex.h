@@ -96,25 +96,53 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     MJT_RX_SETUP
     const index_t j = (index_t)blockIdx.x * 256 + threadIdx.x;
     if (j >= nvec) return;
-#if FLAT_VEC
-    // gather whose innermost extent does not divide into full vectors while y as a whole does: the lane's VEC elements
-    // are adjacent in y's memory and may lie in two rows, so each one is decoded by itself; out-of-range elements load
-    // x[0] and are replaced afterwards, which keeps the VEC loads in flight together (x is not empty)
+#if !SCATTER && SAFE_LOAD && (FLAT_VEC || VEC > 1)
+    // A gather of a non-empty x with several elements per lane.  FLAT_VEC: the innermost extent does not divide into full
+    // vectors while y as a whole does -- the lane's VEC elements are adjacent in y's memory and may lie in two rows, so
+    // each one is decoded by itself; otherwise they share a row and differ in the innermost coordinate only.  When all
+    // of them are in range and adjacent in x as well (the inside of a padded, cropped or shifted row) they arrive as one
+    // load (a flipped row, descending addresses, gains nothing from the same: 45.9 us either way for [64,512,1024]);
+    // otherwise out-of-range elements load x[0] and are replaced afterwards, which keeps the VEC loads in flight together.
     const index_t ebase_ = j * VEC;
     mjt_pack<TX, VEC> yv;
     bool out_[VEC];
+    index_t at_[VEC];
+    bool run_ = true;                      // all in range and adjacent in x: one load of the whole vector
+#if !FLAT_VEC
+    const index_t e = ebase_;
+    MJT_RX_DECODE
+#endif
 #pragma unroll
     for (int k = 0; k < VEC; k++) {
+#if FLAT_VEC
         const index_t e = ebase_ + k;
         MJT_RX_DECODE
         const index_t MJT_RX_LASTVAR = ilast_;
+#else
+        const index_t MJT_RX_LASTVAR = ilast_ + k;
+#endif
         MJT_RX_INDEX
         out_[k] = ov_;
-        yv.v[k] = xp[ov_ ? (index_t)0 : xid];
+        at_[k] = ov_ ? (index_t)0 : xid;
+        run_ = run_ & !ov_ & (at_[k] == at_[0] + k);
     }
+    // decided for the wave as a whole: with both kinds of lanes in a wave it would walk both branches (rows of 66
+    // elements: nearly every wave has a lane at a row's end)
+    if (__builtin_amdgcn_ballot_w64(!run_) == 0) {
+        // x + at_[0] is aligned for one element only
+        struct __attribute__((packed, aligned(sizeof(TX)))) mjt_run { TX v[VEC]; };
+        index_t first_ = at_[0];
+        asm volatile("" : "+v"(first_));       // keeps the compiler from folding this branch into the element-wise one
+        const mjt_run got_ = *(const mjt_run*)(xp + first_);
 #pragma unroll
-    for (int k = 0; k < VEC; k++)
-        if (out_[k]) yv.v[k] = ovalue_;
+        for (int k = 0; k < VEC; k++) yv.v[k] = got_.v[k];
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC; k++) yv.v[k] = xp[at_[k]];
+#pragma unroll
+        for (int k = 0; k < VEC; k++)
+            if (out_[k]) yv.v[k] = ovalue_;
+    }
     mjt_store(yp + ebase_, yv);
     return;
 #else
