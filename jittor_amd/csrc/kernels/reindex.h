@@ -31,7 +31,9 @@ struct Params { void* a[NPARAM]; };   // 8-byte words; typed as pointers so load
 // (mean); MJT_RX_DECODE_KEPT gives the kept coordinates of output o_, MJT_RX_DECODE_TAIL the folded ones of tail
 // offset r (extents as literals).  RTAIL_C > 0: the tail length, known when the kernel is built -- the walk is
 // unrolled, out-of-range elements load x[0] and are replaced afterwards, so that the loads of all OV * RTAIL_C
-// elements are in flight together (x is not empty then).  RTAIL_C == 0: a loop of the length given at launch.
+// elements are in flight together (x is not empty then); TAIL_IN is the extent of the innermost folded axis (a window's
+// row), loaded as one vector when a wave finds all its rows in range and adjacent in x.  RTAIL_C == 0: a loop of the
+// length given at launch.
 extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     const TX* __restrict__ xp = (const TX*)p.a[0];
     TZ* __restrict__ zp = (TZ*)p.a[1];
@@ -47,6 +49,8 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
 #if RTAIL_C
     TX got[OV][RTAIL_C];
     bool out_[OV][RTAIL_C];
+    index_t at_[OV][RTAIL_C];
+    bool runs_ = TAIL_IN > 1;              // every row of the window (TAIL_IN elements, the innermost folded axis) in range and adjacent in x
 #pragma unroll
     for (int k = 0; k < OV; k++) {
         const index_t o_ = o0 + k < nout ? o0 + k : nout - 1;
@@ -56,8 +60,28 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
             MJT_RX_DECODE_TAIL
             MJT_RX_INDEX
             out_[k][r] = ov_;
-            got[k][r] = xp[ov_ ? (index_t)0 : xid];
+            at_[k][r] = ov_ ? (index_t)0 : xid;
+            runs_ = runs_ & !ov_ & (at_[k][r] == at_[k][r - r % TAIL_IN] + r % TAIL_IN);
         }
+    }
+    // decided for the wave as a whole, so that it walks one of the two branches
+    if (TAIL_IN > 1 && __builtin_amdgcn_ballot_w64(!runs_) == 0) {
+        struct __attribute__((packed, aligned(sizeof(TX)))) mjt_run { TX v[TAIL_IN]; };
+#pragma unroll
+        for (int k = 0; k < OV; k++)
+#pragma unroll
+            for (int r = 0; r < RTAIL_C; r += TAIL_IN) {
+                index_t first_ = at_[k][r];
+                asm volatile("" : "+v"(first_));       // keeps the compiler from folding this branch into the element-wise one
+                const mjt_run row_ = *(const mjt_run*)(xp + first_);
+#pragma unroll
+                for (int s = 0; s < TAIL_IN; s++) got[k][r + s] = row_.v[s];
+            }
+    } else {
+#pragma unroll
+        for (int k = 0; k < OV; k++)
+#pragma unroll
+            for (int r = 0; r < RTAIL_C; r++) got[k][r] = xp[at_[k][r]];
     }
 #pragma unroll
     for (int k = 0; k < OV; k++) {

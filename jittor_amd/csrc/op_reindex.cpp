@@ -162,7 +162,10 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
         p_sp = (int)args.size();
         args.insert(args.end(), sp->args.begin(), sp->args.end());
     }
-    // a short tail (a pooling window) is unrolled, the folded extents are literals in the kernel.  One output per lane:
+    // a short tail (a pooling window) is unrolled, the folded extents are literals in the kernel; window rows of 4 to 8
+    // elements are loaded as vectors where a wave finds them all in range and adjacent (8 x 8 mean over [64,128,64,64]:
+    // 59 -> 22.5 us; rows of 2 or 3 gain nothing: 25.9 against 25.7 us for 2 x 2, and with padding nearly every wave has a
+    // lane at the border).  One output per lane:
     // with 2 / 4 / 8 adjacent outputs per lane a 2 x 2 maximum over [64,128,64,64] took 36 / 65 / 79 us against 27
     // (neighbouring lanes then read further apart)
     const int rt_c = z && rtail <= 64 && xn > 0 && !getenv("MJT_GATHER_REDUCE_LOOP") ? (int)rtail : 0;
@@ -258,7 +261,8 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
         frag << "#define MJT_RX_DECODE " << dec.str() << "\n";
         if (z)
             frag << "#define MJT_RX_DECODE_KEPT " << dec_kept.str() << "\n#define MJT_RX_DECODE_TAIL " << dec_tail.str()
-                 << "\n#define RTAIL_C " << rt_c << "\n#define OV " << ov << "\n";
+                 << "\n#define RTAIL_C " << rt_c << "\n#define OV " << ov << "\n#define TAIL_IN "
+                 << (rt_c && y->shape[LD - 1] >= 4 && y->shape[LD - 1] <= 8 && !getenv("MJT_GATHER_REDUCE_NO_RUNS") ? y->shape[LD - 1] : 1) << "\n";
         frag << "#define MJT_RX_INDEX " << index.str() << "\n";
         if (scatter) frag << "#define ATOMIC_UPDATE(addr, v) mjt_atomic_" << mjt_op_name(op) << "<TX>((addr), (v))\n";
         frag << "#define REDUCE_TAIL " << (z ? 1 : 0) << "\n#define FLAT_VEC " << (flat ? 1 : 0) << "\n#define SAFE_LOAD "

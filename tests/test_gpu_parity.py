@@ -1352,6 +1352,9 @@ def test_gather_fused_with_reduce(gpu):
             ("minimum", [7, 2, 3, 9, 10], ["i1", "i2", "(i3+i0)%9", "i4"], 5.0, 4),        # keeps only the first axis
             ("multiply", [4, 2, 3, 3, 3], ["i1", "i2", "i0+i3", "i4*5"], 1.0, 2),
             ("add", [3, 5, 3, 2], ["i0%2", "i1%3", "i2*3+i0", "i3*6"], 0.5, 2),            # an odd number of outputs, two per lane
+            ("add", [2, 3, 2, 2, 4, 5], ["i0", "i1", "i2*4+i4", "i3*5+i5"], 0.0, 2),       # window rows of 5, all in range: loaded as vectors
+            ("maximum", [2, 3, 2, 2, 4, 5], ["i0", "i1", "i2*4+i4-1", "i3*5+i5"], -1e30, 2),  # the same with rows above the image
+            ("minimum", [2, 3, 9, 2, 4], ["i0", "i1", "i2", "i3*4+i4+1"], 7.0, 1),          # rows of 4 at odd offsets
             ("maximum", [1, 1, 2, 3, 5, 3], ["i0", "i1", "i2*5+i4-1", "i3*3+i5"], -1e30, 4)]:  # 90 folded elements: the loop form
         want = O.reduce(O.reindex(x, shape, idx, ov), op, list(range(len(shape) - nred, len(shape))))
         vx, vz = jt.from_storage(x, "float32"), jt.zeros(list(want.shape), "float32")
@@ -1372,6 +1375,13 @@ def test_gather_fused_with_reduce(gpu):
     assert np.array_equal(got.data, want) and jt.executor_stats["gather_reduces"] == before + 1
     # pooling through the front end, float32 and bfloat16 (the 16-bit mean's float32 casts are part of the group)
     xp = rng.standard_normal((3, 5, 11, 12)).astype(np.float32)
+    for dtype in ("float32", "bfloat16"):                      # windows of 4 x 4 without padding: rows loaded as vectors
+        v = jt.array(xp).cast(dtype)
+        y4 = jt.pool(v, 4, "maximum", 0, 4)
+        jt.sync([y4])
+        assert L.last_kernel().startswith("mjt_reindex_then_maximum"), L.last_kernel()
+        want = v.float32().data[:, :, :8, :12].reshape(3, 5, 2, 4, 3, 4).max(axis=(3, 5))
+        assert np.array_equal(y4.float32().data, want), dtype
     for dtype in ("float32", "bfloat16"):
         for op in ("maximum", "mean"):
             v = jt.array(xp).cast(dtype)
