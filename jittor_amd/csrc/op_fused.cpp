@@ -173,8 +173,17 @@ void fused_impl(const mjt_fused_desc* d) {
     // non-temporally, loads stay plain; and such streams run best as single-wave workgroups, which the dispatcher
     // hands out in address order 1 KB at a time (x[64,512,1024] float32 through an 11-op chain: 256 lanes 44.4 us,
     // 128 lanes 44.1, 64 lanes 43.1, 512 lanes 45.2, 1024 lanes 49.9)
+    // A kernel that streams no input of the output's size (a broadcast, a fill) is a pure store stream and wants 4 KB per
+    // workgroup: [512,1] spread over [64,512,1024] float32 takes 30.4 us with 64 lanes, 20.2 with 128 or 256
     const bool streams = total * maxsize >= (int64_t(32) << 20);
-    int block = env_int("MJT_FUSED_BLOCK", streams ? 64 : 256);
+    bool reads_stream = false;
+    for (size_t k = 0; k < inputs.size(); k++) {
+        bool full = true;
+        for (int a = 0; a < nd; a++)
+            if (dims[a].size > 1 && dims[a].bcast[k]) full = false;
+        reads_stream = reads_stream || full;
+    }
+    int block = env_int("MJT_FUSED_BLOCK", streams && reads_stream ? 64 : 256);
     int unroll = env_int("MJT_FUSED_UNROLL", 1);
     int nt = env_int("MJT_FUSED_NT", streams ? 2 : 0);   // bit 0: non-temporal loads, bit 1: non-temporal stores
 
