@@ -267,6 +267,57 @@ def test_reindex_reduce_pool(gpu, op):
         assert np.allclose(got, ref, rtol=1e-4)
 
 
+@pytest.mark.parametrize("case", [
+    # y's loop shape,           indexes into x,                               x shape
+    ([2, 3, 6, 7, 3, 3], ["i0", "i1", "i2*2+i4-1", "i3*2+i5-1"], [2, 3, 12, 14]),      # 3x3 stride 2 pad 1: windows overlap
+    ([2, 3, 6, 7, 2, 2], ["i0", "i1", "i2*2+i4", "i3*2+i5"], [2, 3, 12, 14]),          # 2x2 stride 2: every element once
+    ([4, 5, 5, 3, 2], ["i0", "i1*2+i3*2-2", "i2*3+i4-1"], [4, 11, 13]),               # one batch axis, dilation 2, elements no window reaches
+    ([9, 8, 3, 2], ["i0+i2-2", "i1*1+i3*3"], [9, 12]),                                 # no batch axis, stride 1, horizontal dilation 3
+    ([2, 4, 4, 3, 3], ["i0", "i1*4+i3", "i2*4+i4+1"], [2, 14, 20]),                    # stride beyond the window: gaps; rows the map never reaches
+    ([1, 2, 3, 3, 7, 1], ["i0", "i1", "i2*3+i4-3", "i3+i5"], [1, 2, 8, 3]),            # a window taller than the image
+])
+@pytest.mark.parametrize("op,dtype", [("add", "float32"), ("maximum", "float32"), ("add", "int32"), ("minimum", "int16"),
+                                      ("multiply", "float64"), ("add", "bfloat16")])
+def test_window_scatter_runs_as_a_gather(gpu, case, op, dtype, monkeypatch):
+    """reindex_reduce through a window pattern (the gradient of pooling): every element of x folds the windows that
+    reach it, no atomic update.  Against the oracle, and against the atomic kernel on the same input; integers, maximum
+    and minimum bit-exact, float sums within 1e-4 of the sum of magnitudes (another order of addition)."""
+    shape, idx, xshape = case
+    rng = np.random.default_rng(61)
+    if dtype in ("float32", "float64", "bfloat16"):
+        y = (rng.standard_normal(shape) * (0.2 if op == "multiply" else 2.0) + (1.0 if op == "multiply" else 0.0)).astype(np.float32)
+    else:
+        y = rng.integers(-3, 4, shape).astype(np.float32)
+    vy = jt.array(y).cast(dtype)
+    jt.sync([vy])
+    ref_in = O.BF16(vy.raw()) if dtype == "bfloat16" else vy.data
+    got_v = vy.reindex_reduce(op, xshape, idx)
+    jt.sync([got_v])
+    assert L.last_kernel().startswith("mjt_window_scatter_" + op), L.last_kernel()
+    monkeypatch.setenv("MJT_NO_WINDOW_SCATTER", "1")
+    atomic_v = vy.reindex_reduce(op, xshape, idx)
+    jt.sync([atomic_v])
+    assert L.last_kernel().startswith("mjt_reindex_reduce_" + op), L.last_kernel()
+    monkeypatch.delenv("MJT_NO_WINDOW_SCATTER")
+    if dtype == "bfloat16":
+        # 16-bit sums: one rounding here (float32 accumulator), one per update in the atomic kernel and in the oracle
+        ref = O.reindex_reduce(ref_in.to_f32(), op, xshape, idx)
+        mag = O.reindex_reduce(np.abs(ref_in.to_f32()), op, xshape, idx)
+        got = O.BF16(got_v.raw()).to_f32()
+        assert (np.abs(got - ref) <= 2.0 ** -7 * mag + 1e-30).all()
+        return
+    ref = O.reindex_reduce(ref_in, op, xshape, idx)
+    got, atomic = got_v.data, atomic_v.data
+    assert got.dtype == ref.dtype
+    if dtype in ("int32", "int16") or op in ("maximum", "minimum"):
+        assert np.array_equal(got, ref) and np.array_equal(atomic, ref)
+    elif op == "add":
+        mag = O.reindex_reduce(np.abs(ref_in), op, xshape, idx)
+        assert (np.abs(got - ref) <= 1e-4 * mag + 1e-30).all() and (np.abs(atomic - ref) <= 1e-4 * mag + 1e-30).all()
+    else:
+        assert np.allclose(got, ref, rtol=1e-9) and np.allclose(atomic, ref, rtol=1e-9)
+
+
 def test_reindex_reduce_dtypes_and_overflow(gpu):
     rng = np.random.default_rng(13)
     n, bins = 4000, 50
@@ -1440,10 +1491,18 @@ def test_scatter_with_element_wise_prologue(gpu):
         d.shape[i] = s_
     d.n_vars, d.vars, d.n_ops, d.ops = len(spec), va, len(ops), oa
     tx = L.tensor(vx.raw_ptr(), "float32", xshape)
-    L.check(lib.mjt_fused_reindex_reduce(ctypes.byref(d), ctypes.byref(tx), L.OP_CODE["add"], 4, L.c_strings(idx), 0, L.c_strings([]),
-                                         0, (L.Tensor * 1)()))
-    assert L.last_kernel().startswith("mjt_reindex_reduce_add_")
-    got = L.d2h(vx.raw_ptr(), xshape, np.float32)
-    assert np.allclose(got, want, rtol=1e-4, atol=1e-5)
+    # the window pattern runs as a gather over x; with that path switched off, as atomic updates
+    for env, kernel in ((None, "mjt_window_scatter_add_"), ("MJT_NO_WINDOW_SCATTER", "mjt_reindex_reduce_add_")):
+        if env:
+            os.environ[env] = "1"
+        try:
+            L.check(lib.mjt_fused_reindex_reduce(ctypes.byref(d), ctypes.byref(tx), L.OP_CODE["add"], 4, L.c_strings(idx), 0, L.c_strings([]),
+                                                 0, (L.Tensor * 1)()))
+        finally:
+            if env:
+                del os.environ[env]
+        assert L.last_kernel().startswith(kernel), L.last_kernel()
+        got = L.d2h(vx.raw_ptr(), xshape, np.float32)
+        assert np.allclose(got, want, rtol=1e-4, atol=1e-5), kernel
     # a gathered var is refused where it has no meaning
     assert lib.mjt_fused_elementwise(ctypes.byref(d)) < 0 and "role" in lib.mjt_last_error().decode()
