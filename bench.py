@@ -403,6 +403,25 @@ def wl_callers(L, lib, steps, warmup, with_cpu):
                    "roofline": roofline("hbm", x.nbytes + x.nbytes // 4, ms), **LAST_SPREAD}
     dev.release()
 
+    # the scatter of a pooling gradient: 3x3 windows of stride 2 added back into fp32 [64,64,112,112]
+    dev = Dev(L)
+    ys, xs = (64, 64, 56, 56, 3, 3), (64, 64, 112, 112)
+    y = rng.standard_normal(ys).astype(np.float32)
+    idx = ["i0", "i1", "i2*2+i4-1", "i3*2+i5-1"]
+    ci = L.c_strings(idx)
+    xbytes = int(np.prod(xs)) * 4
+    calls = []
+    py = dev.put(y)
+    for s in range(2):
+        ty, tx = L.tensor(py, "float32", ys), L.tensor(dev.empty(xbytes), "float32", xs)
+        calls.append(lambda ty=ty, tx=tx: L.check(lib.mjt_reindex_reduce(ctypes.byref(ty), ctypes.byref(tx), L.OP_CODE["add"], 4, ci, 0, none, 0, noex)))
+    ms, wall = time_calls(L, calls, steps, warmup)
+    out["SCATTER_WINDOW"] = {"workload": "SCATTER_WINDOW: mjt_reindex_reduce add of fp32 [64,64,56,56,3,3] into [64,64,112,112] through 3x3 stride-2 windows",
+                             "kernel": L.last_kernel(), "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+                             "roofline": roofline("hbm", y.nbytes + xbytes, ms), **LAST_SPREAD,
+                             "note": "as a gather over x: no atomic updates, no identity fill"}
+    dev.release()
+
     # a column reduce: sum over axis 0 of [65536, 512]
     dev = Dev(L)
     x = rng.standard_normal((65536, 512)).astype(np.float32)
