@@ -304,8 +304,7 @@ void run_generic(Plan* plan, bool scatter, int op, const mjt_tensor* x, const mj
 // A scatter through a window pattern (x[b.., oh*SH + kh*DH + CH, ow*SW + kw*DW + CW] op= y[b.., oh, ow, kh, kw], no
 // overflow conditions, no extras: the gradient of pooling) runs as a gather over x: every element of x folds the windows
 // that reach it (kernels/window_scatter.h) -- no atomic updates, no identity fill.  Measured on the gradient of a 3x3
-// stride-2 maximum pooling of [64,64,112,112] float32: 1042 us of queued atomic adds (plus 20 us of fill) against the
-// time below.  Returns false when the pattern is another one; the caller then fills and scatters.
+// stride-2 maximum pooling of [64,64,112,112] float32: 1042 us of queued atomic adds (plus 20 us of fill) against 139 us.  Returns false when the pattern is another one; the caller then fills and scatters.
 bool try_window_scatter(Plan* plan, int op, const mjt_tensor* x, const mjt_tensor* y, int n_ofc, int n_ex, const ScatterPrologue* sp) {
     if (getenv("MJT_NO_FASTPATH") || getenv("MJT_NO_WINDOW_SCATTER")) return false;
     if (n_ofc != 0 || n_ex != 0 || !plan->all_affine) return false;
@@ -349,8 +348,16 @@ bool try_window_scatter(Plan* plan, int op, const mjt_tensor* x, const mjt_tenso
     const int p_sp = (int)args.size();
     if (sp) args.insert(args.end(), sp->args.begin(), sp->args.end());
 
+    // elements of a row of x per lane: one 16-byte store when the rows and the pointer allow it
+    int wvec = std::min(8, 16 / dtype_size(x->dtype));
+    while (wvec > 1 && (x->shape[XD - 1] % wvec != 0 || (uintptr_t)x->ptr % (size_t)(wvec * dtype_size(x->dtype)) != 0)) wvec /= 2;
+    while (wvec > 1 && NCH * NCW * wvec > 32) wvec /= 2;                  // at most 32 candidate windows per lane
+    if (const char* e = getenv("MJT_WINDOW_SCATTER_VEC")) {               // 1, 2, 4 or 8, for experiments
+        const int v = atoi(e);
+        if (v >= 1 && v <= wvec && (v & (v - 1)) == 0) wvec = v;
+    }
     std::ostringstream vk;
-    vk << "WS" << op << (use64 ? "L" : "I") << "|" << SH << "," << SW << "," << DH << "," << DW << "," << CH << "," << CW << "," << KH << "," << KW;
+    vk << "WS" << op << (use64 ? "L" : "I") << wvec << "|" << SH << "," << SW << "," << DH << "," << DW << "," << CH << "," << CW << "," << KH << "," << KW;
     for (int i = 0; i < XD; i++) vk << "," << x->shape[i];
     vk << "," << y->shape[a_oh] << "," << y->shape[a_ow];
     if (sp) vk << "|P" << sp->key;
@@ -384,8 +391,8 @@ bool try_window_scatter(Plan* plan, int op, const mjt_tensor* x, const mjt_tenso
         }
         const int ta = x->dtype == MJT_FLOAT16 || x->dtype == MJT_BFLOAT16 ? MJT_FLOAT32 : x->dtype;
         std::ostringstream frag;
-        frag << "#define TX " << dtype_cname(x->dtype) << "\n#define TACC " << dtype_cname(ta) << "\n#define index_t " << IT << "\n#define NPARAM "
-             << args.size() << "\n#define NB " << nb << "\n#define KH " << KH << "\n#define KW " << KW << "\n#define SH " << SH << "\n#define SW " << SW
+        frag << "#define TX " << dtype_cname(x->dtype) << "\n#define TACC " << dtype_cname(ta) << "\n#define index_t " << IT << "\n#define VEC " << wvec
+             << "\n#define NPARAM " << args.size() << "\n#define NB " << nb << "\n#define KH " << KH << "\n#define KW " << KW << "\n#define SH " << SH << "\n#define SW " << SW
              << "\n#define DH " << DH << "\n#define DW " << DW << "\n#define CH " << CH << "\n#define CW " << CW << "\n#define NCH " << NCH
              << "\n#define NCW " << NCW << "\n";
         // extents as literals: the lane's coordinates come from divisions by them
@@ -409,7 +416,7 @@ bool try_window_scatter(Plan* plan, int op, const mjt_tensor* x, const mjt_tenso
         std::lock_guard<std::mutex> lock(g_mu);
         plan->kernels.emplace(vkey, kern);
     }
-    const int64_t blocks = (xn + 255) / 256;
+    const int64_t blocks = (xn / wvec + 255) / 256;
     if (blocks >= (int64_t(1) << 31)) return false;
     jit_launch(kern, (unsigned)blocks, 1, 256, 0, args);
     return true;
