@@ -525,6 +525,51 @@ def test_conv_input_gradient_entry_validates_and_picks_its_path(compile_only):
     assert b"padding" in lib.mjt_last_error()
 
 
+def test_scatter_and_gather_entries_pick_their_kernels(compile_only, monkeypatch):
+    """Without a device: which kernel skeleton a reindex_reduce, a reindex and a fused gather + reduce take.  A scatter
+    through a window pattern is a gather over x unless it has overflow conditions, extras or too many candidate windows
+    per element; a gather into rows that are no whole vectors keeps 16-byte stores; axis permutations go through tiles."""
+    lib = L.load()
+    P = 0x100000
+    e, noex = L.c_strings([]), (L.Tensor * 1)()
+
+    def scatter(ys, xs, idx, op="add", ofc=(), dtype="float32"):
+        ty, tx = L.tensor(P, dtype, ys), L.tensor(P, dtype, xs)
+        rc = lib.mjt_reindex_reduce(ctypes.byref(ty), ctypes.byref(tx), L.OP_CODE[op], len(idx), L.c_strings(idx), len(ofc),
+                                    L.c_strings(list(ofc)), 0, noex)
+        assert rc == 0, lib.mjt_last_error()
+        return L.last_kernel()
+
+    pool = ([4, 8, 16, 16, 3, 3], [4, 8, 32, 32], ["i0", "i1", "i2*2+i4-1", "i3*2+i5-1"])
+    assert scatter(*pool).startswith("mjt_window_scatter_add_")
+    assert scatter(*pool, op="maximum", dtype="bfloat16").startswith("mjt_window_scatter_maximum_")
+    assert scatter(*pool, ofc=["i4>1"]).startswith("mjt_reindex_reduce_add_")                      # an overflow condition
+    assert scatter(*pool, op="bitwise_or", dtype="int32").startswith("mjt_reindex_reduce_bitwise_or_")
+    assert scatter([4, 8, 30, 30, 7, 7], [4, 8, 36, 36], ["i0", "i1", "i2+i4", "i3+i5"]).startswith("mjt_reindex_reduce_add_")   # 49 windows reach an element
+    assert scatter([4, 8, 16, 16, 3, 3], [4, 8, 32, 32], ["i0", "i1", "i3*2+i4-1", "i2*2+i5-1"]).startswith("mjt_reindex_reduce_add_")  # rows from the column axis
+    monkeypatch.setenv("MJT_NO_WINDOW_SCATTER", "1")
+    assert scatter(*pool).startswith("mjt_reindex_reduce_add_")
+    monkeypatch.delenv("MJT_NO_WINDOW_SCATTER")
+
+    def gather(xs, ys, idx):
+        tx, ty = L.tensor(P, "float32", xs), L.tensor(P, "float32", ys)
+        assert lib.mjt_reindex(ctypes.byref(tx), ctypes.byref(ty), len(idx), L.c_strings(idx), 0.0, 0, e, 0, noex) == 0, lib.mjt_last_error()
+        return L.last_kernel()
+
+    assert gather([8, 16, 64, 64], [8, 64, 64, 16], ["i0", "i3", "i1", "i2"]).startswith("mjt_permute_b4_")
+    assert gather([8, 16, 64, 64], [8, 16, 66, 66], ["i0", "i1", "i2-1", "i3-1"]).startswith("mjt_reindex_")
+    a = L.jit_stats()[0]
+    monkeypatch.setenv("MJT_REINDEX_NO_FLAT", "1")
+    assert gather([8, 16, 64, 64], [8, 16, 66, 66], ["i0", "i1", "i2-1", "i3-1"]).startswith("mjt_reindex_")
+    assert L.jit_stats()[0] == a + 1                         # another kernel: two elements per lane instead of four
+
+    loop, z = L.tensor(0, "float32", [8, 16, 32, 32, 2, 2]), L.tensor(P, "float32", [8, 16, 32, 32])
+    tx = L.tensor(P, "float32", [8, 16, 64, 64])
+    assert lib.mjt_reindex_then_reduce(ctypes.byref(tx), ctypes.byref(loop), ctypes.byref(z), L.OP_CODE["maximum"], 2, 4,
+                                       L.c_strings(["i0", "i1", "i2*2+i4", "i3*2+i5"]), 0.0, 0, e, 0, noex) == 0
+    assert L.last_kernel().startswith("mjt_reindex_then_maximum_")
+
+
 def test_compile_options_follow_the_flag_and_mark_grouped_convolutions():
     """Var.compile_options (var_holder.h:265-273): a dict name -> int, initialised from the flag's value when the var is
     created (var.cc:75); nn.conv2d marks the gathered input of a grouped convolution with {"G": groups} (nn.py:1278),
