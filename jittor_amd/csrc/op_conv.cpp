@@ -2,6 +2,7 @@
 // python/jittor/nn.py:1251-1262 builds; parameters as solved by
 // python/jittor/src/opt/tuner/conv_tuner.cc:312-356).
 #include "common.h"
+#include <array>
 #include <mutex>
 #include <unordered_map>
 
@@ -609,6 +610,37 @@ void conv_dgrad_impl(const mjt_tensor* dy, const mjt_tensor* w, const mjt_tensor
         char* part = (char*)conv_scratch(3, (size_t)(sh * sw * plane * dsz));
         const mjt_conv_params unit = {1, 1, 0, 0, 1, 1};
         std::string kernels;
+        // The weights of all phases in one pass (the phases partition the taps): w [K,C,R,S] -> one block [C,K,U,V] per
+        // phase, the phase's taps flipped, the blocks one after the other.  Seen from the flat offset i0 of that buffer,
+        // block p covers [off_p, off_p + C*K*U*V) and its element (c, k, u, v) reads w[k, c, first_r + sh*(U-1-u),
+        // first_c + sw*(V-1-v)]: four index expressions, each a chain of conditions on i0.
+        std::vector<int64_t> woff((size_t)(sh * sw), -1);
+        {
+            std::string ek = "0", ec = "0", er = "0", es = "0";
+            int64_t off = 0;
+            std::vector<std::array<std::string, 4>> pieces;
+            std::vector<int64_t> ends;
+            for (int64_t a = 0; a < sh; a++)
+                for (int64_t b = 0; b < sw; b++) {
+                    const Phase &qr = rows[a], &qc = cols[b];
+                    if (qr.taps == 0 || qc.taps == 0) continue;
+                    woff[(size_t)(a * sw + b)] = off;
+                    const int64_t U = qr.taps, V = qc.taps;
+                    const std::string l = "(i0-" + str(off) + ")";
+                    pieces.push_back({l + "/" + str(U * V) + "%" + str(K), l + "/" + str(K * U * V),
+                                      str(qr.first) + "+" + str(sh) + "*(" + str(U - 1) + "-" + l + "/" + str(V) + "%" + str(U) + ")",
+                                      str(qc.first) + "+" + str(sw) + "*(" + str(V - 1) + "-" + l + "%" + str(V) + ")"});
+                    off += C * K * U * V;
+                    ends.push_back(off);
+                }
+            if (!pieces.empty()) {
+                std::array<std::string, 4> e = pieces.back();
+                for (int i = (int)pieces.size() - 2; i >= 0; i--)
+                    for (int j = 0; j < 4; j++) e[j] = "(i0<" + str(ends[i]) + " ? " + pieces[i][j] + " : " + e[j] + ")";
+                mjt_tensor tall = view(wbuf, w->dtype, {off});
+                reindex(*w, tall, {e[0], e[1], e[2], e[3]}, {});
+            }
+        }
         for (int64_t a = 0; a < sh; a++)
             for (int64_t b = 0; b < sw; b++) {
                 const Phase &qr = rows[a], &qc = cols[b];
@@ -617,10 +649,7 @@ void conv_dgrad_impl(const mjt_tensor* dy, const mjt_tensor* w, const mjt_tensor
                     reindex(*dy, ty, {"0", "0", "0", "0"}, {"1"});
                     continue;
                 }
-                // w [K,C,R,S] -> [C,K,U,V]: the phase's taps, flipped
-                mjt_tensor tw = view(wbuf, w->dtype, {C, K, qr.taps, qc.taps});
-                reindex(*w, tw, {"i1", "i0", str(qr.first) + "+" + str(sh) + "*(" + str(qr.taps - 1) + "-i2)",
-                                 str(qc.first) + "+" + str(sw) + "*(" + str(qc.taps - 1) + "-i3)"}, {});
+                mjt_tensor tw = view((char*)wbuf + woff[(size_t)(a * sw + b)] * esz, w->dtype, {C, K, qr.taps, qc.taps});
                 mjt_conv_params q = unit;
                 q.pad_h = (int32_t)qr.pad;
                 q.pad_w = (int32_t)qc.pad;
