@@ -126,12 +126,15 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
     // each one is decoded by itself; otherwise they share a row and differ in the innermost coordinate only.  When all
     // of them are in range and adjacent in x as well (the inside of a padded, cropped or shifted row) they arrive as one
     // load (a flipped row, descending addresses, gains nothing from the same: 45.9 us either way for [64,512,1024]);
-    // otherwise out-of-range elements load x[0] and are replaced afterwards, which keeps the VEC loads in flight together.
+    // when the even and the odd ones are each adjacent (two sources woven column by column, or every source element
+    // taken twice) they arrive as two loads of half a vector; otherwise out-of-range elements load x[0] and are
+    // replaced afterwards, which keeps the VEC loads in flight together.
     const index_t ebase_ = j * VEC;
     mjt_pack<TX, VEC> yv;
     bool out_[VEC];
     index_t at_[VEC];
     bool run_ = true;                      // all in range and adjacent in x: one load of the whole vector
+    bool twin_ = VEC >= 4;                 // all in range, the even and the odd ones each adjacent in x: two loads of half a vector
 #if !FLAT_VEC
     const index_t e = ebase_;
     MJT_RX_DECODE
@@ -149,6 +152,7 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
         out_[k] = ov_;
         at_[k] = ov_ ? (index_t)0 : xid;
         run_ = run_ & !ov_ & (at_[k] == at_[0] + k);
+        twin_ = twin_ & !ov_ & (k < 2 || at_[k] == at_[k - 2] + 1);
     }
     // decided for the wave as a whole: with both kinds of lanes in a wave it would walk both branches (rows of 66
     // elements: nearly every wave has a lane at a row's end)
@@ -160,6 +164,15 @@ extern "C" __global__ __launch_bounds__(256) void ENTRY(Params p) {
         const mjt_run got_ = *(const mjt_run*)(xp + first_);
 #pragma unroll
         for (int k = 0; k < VEC; k++) yv.v[k] = got_.v[k];
+    } else if (VEC >= 4 && __builtin_amdgcn_ballot_w64(!twin_) == 0) {
+        // two runs woven into each other (columns interleaved from two sources, every source element taken twice)
+        struct __attribute__((packed, aligned(sizeof(TX)))) mjt_half_run { TX v[VEC / 2 > 0 ? VEC / 2 : 1]; };
+        index_t even_ = at_[0], odd_ = at_[1];
+        asm volatile("" : "+v"(even_), "+v"(odd_));
+        const mjt_half_run a_ = *(const mjt_half_run*)(xp + even_);
+        const mjt_half_run b_ = *(const mjt_half_run*)(xp + odd_);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) yv.v[k] = (k & 1) ? b_.v[k / 2] : a_.v[k / 2];
     } else {
 #pragma unroll
         for (int k = 0; k < VEC; k++) yv.v[k] = xp[at_[k]];

@@ -352,6 +352,9 @@ bool try_window_scatter(Plan* plan, int op, const mjt_tensor* x, const mjt_tenso
     int wvec = std::min(8, 16 / dtype_size(x->dtype));
     while (wvec > 1 && (x->shape[XD - 1] % wvec != 0 || (uintptr_t)x->ptr % (size_t)(wvec * dtype_size(x->dtype)) != 0)) wvec /= 2;
     while (wvec > 1 && NCH * NCW * wvec > 32) wvec /= 2;                  // at most 32 candidate windows per lane
+    // without a prologue the candidates are loads from y itself, far apart for neighbouring elements of x: more of them
+    // per lane coalesce worse (3x3 stride-2 windows into [64,64,112,112]: 230 us with four elements per lane, 175 with one)
+    if (!sp) wvec = 1;
     if (const char* e = getenv("MJT_WINDOW_SCATTER_VEC")) {               // 1, 2, 4 or 8, for experiments
         const int v = atoi(e);
         if (v >= 1 && v <= wvec && (v & (v - 1)) == 0) wvec = v;

@@ -213,6 +213,28 @@ def test_reindex_rows_that_are_no_whole_vectors(gpu, dtype):
         assert np.array_equal(again, want), (dtype, shape)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "int8", "float64"])
+def test_reindex_two_runs_woven_into_each_other(gpu, dtype):
+    """A lane whose even and odd elements are each adjacent in x loads them as two half vectors: every source element
+    taken twice (nearest-neighbour upsampling), columns interleaved from several sources (the stride phases of an input
+    gradient), and the same with rows where only some waves qualify; bit-exact against the oracle."""
+    rng = np.random.default_rng(14)
+    x = (rng.standard_normal((4, 3, 5, 6, 8)) * 40).astype(np.float32)
+    xv = jt.array(x).cast(dtype)
+    ref_in = O.BF16(xv.raw()) if dtype == "bfloat16" else xv.data
+    for shape, idx, ov in [
+            ([3, 5, 12, 16], ["i2%2*2+i3%2", "i0", "i1", "i2/2", "i3/2"], 0.0),      # four sources woven by rows and columns
+            ([4, 3, 5, 6, 16], ["i0", "i1", "i2", "i3", "i4/2"], 0.0),              # every element twice
+            ([4, 3, 5, 6, 16], ["i0", "i1", "i2", "i3", "i4/2+1"], -2.0),            # the same, shifted: the last pair out of range
+            ([2, 3, 5, 6, 16], ["i0*2+i4%2", "i1", "i2", "i3", "i4/2"], 0.0)]:       # two sources far apart
+        want = O.reindex(ref_in, shape, idx, ov)
+        want = want.bits if dtype == "bfloat16" else want
+        got = xv.reindex(shape, idx, ov)
+        got = got.raw() if dtype == "bfloat16" else got.data
+        assert L.last_kernel().startswith("mjt_reindex_")
+        assert np.array_equal(got, want), (dtype, shape, idx)
+
+
 @pytest.mark.parametrize("case", [
     dict(x=(2, 3, 7, 6), k=(3, 3), s=(1, 1), d=(1, 1), p=(1, 1)),
     dict(x=(3, 9, 11), k=(3, 2), s=(2, 1), d=(1, 2), p=(0, 1)),
