@@ -197,12 +197,12 @@ def wl_c3(L, lib, steps, warmup, with_cpu, op):
             ctypes.byref(tv), ctypes.byref(tx), L.OP_CODE[op], 1, s1, 0, e, 1, ti)))
     ms, wall = time_calls(L, calls, steps, warmup)
     last = L.last_kernel()
-    main_kernel = last[:-len("_final")] + "_main" if last.endswith("_final") else last
+    main_kernel = last[:-len("_tail")] + "_main" if last.endswith("_tail") else last
     out = {"workload": "C3 ReindexReduceOp scatter-%s, 2^24 fp32 values into 2^20 bins, int32 Zipf(1.1) indices" % op,
            "kernel": main_kernel, "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
            "roofline": roofline("hbm", work, ms), **LAST_SPREAD,
-           "note": "a step = the four launches of the 1-d scatter (main, plan, cold, final); the bins need no prior fill; "
-                   "`kernel` names the dominant one (the main pass), `kernel_ms` is the four together"}
+           "note": "a step = the two launches of the 1-d scatter (main, tail); the bins need no prior fill; "
+                   "`kernel` names the dominant one (the main pass), `kernel_ms` is the two together"}
     dev.release()
     if with_cpu:
         t1 = cpu_time(lambda: K.scatter_1d(v, idx, bins, op))

@@ -95,6 +95,7 @@ struct JitKernel {
     hipModule_t module = nullptr;
     hipFunction_t fn = nullptr;
     std::string name;
+    uint64_t state[2] = {0, 0};   // for the launcher of kernels that keep state in their code object's device memory
 };
 // Compiles `source` (which must define extern "C" __global__ `entry`) for the
 // current device, or returns the cached kernel for an identical source.

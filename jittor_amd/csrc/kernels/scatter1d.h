@@ -4,8 +4,10 @@
 // python/jittor/src/ops/reindex_reduce_op.cc:93-131).
 //
 // Scattered global atomics run at about 2e10 updates/s on this chip whatever
-// their scope, and a hot bin serialises them further, so this path uses none.
-// The bin axis is cut into buckets of WBINS bins (one bucket fits in LDS):
+// their scope (contiguous ones, 64 neighbouring bins per wave instruction, at
+// 2-4e11/s), and a hot bin serialises them further, so no update of the input
+// is a global atomic.  The bin axis is cut into buckets of WBINS bins (one
+// bucket fits in LDS); two launches:
 //   main    every workgroup streams its share of (idx, y) in rounds of
 //           NP*EPT elements.  A sample of its own indices picks the bucket
 //           that receives most of its updates (its "hot" bucket); updates of
@@ -13,39 +15,68 @@
 //           into an LDS staging area (a wave takes its slots of a round with
 //           one LDS atomic), and a few waves that load no input append what
 //           the previous round staged to the workgroup's per-bucket lists in
-//           scratch memory.  At the end the private copy, the list lengths and
-//           the hot bucket's number are written out;
-//   plan    one workgroup sums the list lengths per bucket and lays out the
-//           work of the cold pass;
-//   cold    a fixed number of workgroups walks the work items.  A list item
-//           (bucket, split) folds the lists of its bucket written by main
-//           workgroups split, split + nsplit, ... into a private LDS copy and
-//           writes it out; the number of list items per bucket follows the
+//           scratch memory.  Those waves also write the identity into the
+//           workgroup's slice of x.  At the end the private copy, the list
+//           lengths and the hot bucket's number are written out, and the
+//           lengths and the hot bucket are added to the tallies below;
+//   tail    every workgroup reads the tallies (list entries and private
+//           copies per bucket), lays out the work items from them and walks
+//           its items.  A list item (bucket, split) folds the lists of its
+//           bucket written by main workgroups split, split + nsplit, ... into
+//           an LDS copy; the number of list items per bucket follows the
 //           bucket's population.  Entries that did not fit a list (rare: a
 //           second hot region) sit in per-workgroup overflow lists that item
-//           (bucket, 0) scans.  A merge item merges a segment of the private
-//           copies of 32 main workgroups that had the same hot bucket;
-//   final   x[bin] = merge of the partial copies of its bucket (plain stores:
-//           x needs no prior fill).
-// Workgroups of one launch share nothing, so no buffer has to be cleared
-// beforehand and no global atomic is issued.
+//           (bucket, 0) scans.  A merge item merges a segment of MB bins of
+//           all private copies of the bucket.  An item that is the only one
+//           to reach its bins stores them; otherwise the items of a bucket
+//           combine in x through contiguous atomics (a wave instruction
+//           updates 64 neighbouring bins) on top of the identity.
+// The tallies are two sets of counters in device memory that belong to this
+// code object: a call uses set `slot` (its number modulo 2), and the tail pass
+// of a call clears the other set, so the counters are zero when main starts
+// and nothing has to be cleared in a launch of its own (ENTRY_RESET clears
+// both: first call, and after a call that did not finish).
 //
 // Supplied by the host: TX (4-byte element type), TE (index type), WBINS
-// (power of two), LOGW, NBMAX (power of two >= bucket count, <= NTHREADS),
+// (power of two), LOGW, NBMAX (power of two >= bucket count, <= NTHREADS / 2),
 // NTHREADS, NFLUSH (threads that only store), EPT (elements per thread and
 // round, multiple of 4), SCAP (entries of each of the two staging areas), MODE (0 add, 1 maximum, 2 minimum), ACC64, COLD_TARGET,
 // EXACT_BINS (the bin count is a multiple of WBINS),
 // IDENT_BITS (bit pattern of the identity).
 
+// ABL (0 in production): timing-only ablations, results are wrong with any bit set.  1 the tail pass stores
+// instead of combining through atomics, 2 list items read no lists, 4 no merge items, 8 the main pass
+// stores no list entries, 16 stages none, 32 leaves the private copy alone, 64 neither fills x nor tallies.
+#ifndef ABL
+#define ABL 0
+#endif
+#ifndef MDEPTH
+#define MDEPTH 8
+#endif
+#ifndef LDEPTH
+#define LDEPTH 16
+#endif
+
 struct Params { void* a[20]; };   // 8-byte words; typed as pointers so loads/stores use the global address space
 // a[0] x          a[1] y           a[2] idx        a[3] n          a[4] bins
-// a[5] plan (written by the plan kernel)
+// a[5] fill (1: main writes the identity into x)
 // a[6] per (elements per main workgroup)           a[7] G1 (main workgroups)
 // a[8] NB (buckets)  a[9] CAP (list capacity)  a[10] counts[G1][NB]  a[11] lists[NB][G1][CAP]
-// a[12] partial_main[G1][WBINS]  a[13] partial_cold[items][WBINS]  a[14] hotof[G1]
+// a[12] partial_main[MSEG][G1][MB]  a[13] slot (tally set of this call)  a[14] hotof[G1]
 // a[15] overflow lists[G1][per]   a[16] novf[G1]
 
+// Tallies of the main pass: [set][b] list entries of bucket b, [set][NBMAX + b] main workgroups whose hot bucket
+// was b, [set][2 * NBMAX] main workgroups that wrote an overflow list.
+// Each set exists TSUB times (a main workgroup adds to copy number blockIdx % TSUB, the tail pass sums the
+// copies): hundreds of atomics on one address queue up at the memory.
+constexpr int TSUB = 16, TALLY = 2 * NBMAX + 1;
+__device__ unsigned mjt_tally[2][TSUB][TALLY];
+
 struct mjt_pair { int bin; TX val; };
+// The private copies in memory: partial_main[segment][main workgroup][MB] -- a merge item reads segment s of every
+// copy, which is one contiguous piece this way (as rows of whole copies its reads were 1 KB pieces 64 KB apart).
+constexpr int MB = WBINS < 256 ? WBINS : 256;                 // bins of a merge item
+constexpr int MSEG = WBINS / MB;
 
 // TA: type partial results are merged in.  TW: type of the private copies in LDS.
 // add: a float LDS add costs 3 cycles per lane on this chip, a double one 0.25 (0.6 with the same-address
@@ -123,10 +154,12 @@ template <bool V> struct mjt_flag { static constexpr bool value = V; };
 constexpr int NP = NTHREADS - NFLUSH;                        // threads that load input; the others append to the lists
 
 extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
+    TX* __restrict__ xp = (TX*)p.a[0];
     const TX* __restrict__ yp = (const TX*)p.a[1];
     const TE* __restrict__ ip = (const TE*)p.a[2];
     const long long n = (long long)(unsigned long long)p.a[3];
     const long long bins = (long long)(unsigned long long)p.a[4];
+    const bool fill = p.a[5] != nullptr;
     const long long per = (long long)(unsigned long long)p.a[6];
     const int NB = (int)(unsigned long long)p.a[8];
     const unsigned CAP = (unsigned)(unsigned long long)p.a[9];
@@ -170,6 +203,11 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
     constexpr long long STEP = (long long)NP * EPT;
     const int rounds = 2 * (int)((end4 - begin + 2 * STEP - 1) / (2 * STEP)) + (end4 < end ? 1 : 0);
     if (threadIdx.x >= NP) {
+        if (fill && !(ABL & 64)) {                            // the identity into this workgroup's slice of x
+            const long long slice = (bins + gridDim.x - 1) / gridDim.x;
+            const long long f0 = (long long)blockIdx.x * slice, f1 = f0 + slice < bins ? f0 + slice : bins;
+            for (long long t = f0 + (threadIdx.x - NP); t < f1; t += NFLUSH) xp[t] = ident;
+        }
         __syncthreads();                                      // the three barriers of the producers' vote
         __syncthreads();
         __syncthreads();
@@ -195,7 +233,7 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
 #pragma unroll
                     for (int u = 0; u < FDEPTH; u++) {
                         const int b = e[u].bin >> LOGW;
-                        if (b < NBMAX) {
+                        if (b < NBMAX && !(ABL & 8)) {
                             if (pos[u] < CAP) mylists[(size_t)b * bucket_stride + pos[u]] = e[u];
                             else ovf[atomicAdd(&ovf_len, 1u)] = e[u];
                         }
@@ -219,8 +257,8 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
 #pragma unroll
             for (int k = 0; k < EPT; k++) {
                 const unsigned bucket = idx[k] >> LOGW;
-                if (bucket == hot) mjt_win_update(&win[idx[k] & (WBINS - 1)], val[k]);
-                cold[k] = bucket != hot && bucket < (unsigned)NB;
+                if (bucket == hot && !(ABL & 32)) mjt_win_update(&win[idx[k] & (WBINS - 1)], val[k]);
+                cold[k] = bucket != hot && bucket < (unsigned)NB && !(ABL & 16);
                 mask[k] = __builtin_amdgcn_ballot_w64(cold[k]);
                 before[k] = total;
                 total += (unsigned)__popcll(mask[k]);
@@ -329,115 +367,74 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_MAIN(Params p) {
         __syncthreads();                                      // the flushers have drained the last round
     }
     __syncthreads();
-    TX* __restrict__ out = pmain + (size_t)blockIdx.x * WBINS;
     for (int t = threadIdx.x * 4; t < WBINS; t += NTHREADS * 4) {
         mjt_pack<TX, 4> o;
 #pragma unroll
         for (int k = 0; k < 4; k++) o.v[k] = mjt_win_read(win[t + k]);
-        mjt_store(out + t, o);
+        mjt_store(pmain + ((size_t)(t / MB) * gridDim.x + blockIdx.x) * MB + t % MB, o);
     }
+    unsigned* __restrict__ tally = mjt_tally[(unsigned)(unsigned long long)p.a[13] & 1u][blockIdx.x % TSUB];
     for (int t = threadIdx.x; t < NB; t += NTHREADS) {
-        const unsigned c = cursor[t];
-        counts[(size_t)blockIdx.x * NB + t] = c < CAP ? c : CAP;
+        const unsigned c = cursor[t] < CAP ? cursor[t] : CAP;
+        counts[(size_t)blockIdx.x * NB + t] = c;
+        if (c && !(ABL & 64)) atomicAdd(&tally[t], c);
     }
     if (threadIdx.x == 0) {
         hotof[blockIdx.x] = (int)hot;
         novf[blockIdx.x] = ovf_len;
+        atomicAdd(&tally[NBMAX + hot], 1u);
+        if (ovf_len) atomicAdd(&tally[2 * NBMAX], 1u);
     }
 }
 
-// Work plan of the cold pass, computed identically by every cold workgroup.  Bucket b has nsplit[b] list
-// items (list entries / COLD_TARGET, at least 1 when it has entries, at most G1), each producing one
-// partial copy, followed by nmerge[b] * MSEG merge items: the partial copies of MERGE_ROWS main workgroups
-// whose hot bucket it was are merged into one, MSEG items sharing the work by segments of MBINS bins (one
-// compute unit pulls little more than 100 GB/s: an item should not read more than about 100 KB).
-// first[b] is the number of the bucket's first item, pfirst[b] of its first partial copy; first[NBMAX] and
-// pfirst[NBMAX] are the totals.
-constexpr int MERGE_ROWS = 32;
-constexpr int MBINS = WBINS < 2048 ? WBINS : 2048;
-constexpr int MSEG = WBINS / MBINS;
+// ---- updates of x by the tail pass ------------------------------------------------------------------------
+// x holds the identity or what other items have put there; float maxima and minima go through the
+// order-preserving integer view of IEEE floats (non-negative floats order like signed integers, negative
+// ones inversely like unsigned integers).
+#if MODE == 0
+__device__ __forceinline__ void mjt_x_update(float* a, float v) { unsafeAtomicAdd(a, v); }
+__device__ __forceinline__ void mjt_x_update(int* a, int v) { atomicAdd(a, v); }
+__device__ __forceinline__ void mjt_x_update(unsigned* a, unsigned v) { atomicAdd(a, v); }
+#elif MODE == 1
+__device__ __forceinline__ void mjt_x_update(float* a, float v) {
+    const unsigned b = __float_as_uint(v);
+    if (b >> 31) atomicMin((unsigned*)a, b); else atomicMax((int*)a, (int)b);
+}
+__device__ __forceinline__ void mjt_x_update(int* a, int v) { atomicMax(a, v); }
+__device__ __forceinline__ void mjt_x_update(unsigned* a, unsigned v) { atomicMax(a, v); }
+#else
+__device__ __forceinline__ void mjt_x_update(float* a, float v) {
+    const unsigned b = __float_as_uint(v);
+    if (b >> 31) atomicMax((unsigned*)a, b); else atomicMin((int*)a, (int)b);
+}
+__device__ __forceinline__ void mjt_x_update(int* a, int v) { atomicMin(a, v); }
+__device__ __forceinline__ void mjt_x_update(unsigned* a, unsigned v) { atomicMin(a, v); }
+#endif
+
+// ---- reset: both tally sets to zero ----------------------------------------------------------------------
+extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_RESET(Params) {
+    unsigned* t = &mjt_tally[0][0][0];
+    for (int i = threadIdx.x; i < 2 * TSUB * TALLY; i += NTHREADS) t[i] = 0;
+}
+
+// ---- tail: folds the lists and merges the private copies of main into x -----------------------------------
+// Work plan, computed identically by every workgroup from the tallies.  Bucket b has nsplit[b] list items
+// (list entries / COLD_TARGET, at least 1 when it has entries, at most G1) followed, when main workgroups had
+// it as their hot bucket, by MSEG merge items: one per segment of MB bins, each over all private copies of
+// the bucket (one compute unit pulls little more than 100 GB/s: an item should not read more than a few
+// hundred KB).  The list items of all buckets come first (they take longest), the merge items after them:
+// first[b] is the number of the bucket's first list item, mfirst[b] of its first merge item; first[NBMAX] is
+// the number of list items, mfirst[NBMAX] the total.
 struct mjt_plan {
     unsigned nsplit[NBMAX];
-    unsigned nmerge[NBMAX];
+    unsigned nrows[NBMAX];
     unsigned first[NBMAX + 1];
-    unsigned pfirst[NBMAX + 1];
+    unsigned mfirst[NBMAX + 1];
 };
 
-__device__ __forceinline__ void mjt_make_plan(mjt_plan& plan, const unsigned* __restrict__ counts,
-                                              const int* __restrict__ hotof, int G1, int NB, unsigned long long* wsum) {
-    for (int b = threadIdx.x; b < NBMAX; b += NTHREADS) { plan.nsplit[b] = 0; plan.nmerge[b] = 0; }   // populations first
-    __syncthreads();
-    {
-        const int b = threadIdx.x & (NBMAX - 1);
-        unsigned sum = 0;
-        if (b < NB) {                                         // independent loads, several in flight
-            constexpr int RSTEP = NTHREADS / NBMAX;
-            for (int r0 = threadIdx.x / NBMAX; r0 < G1; r0 += 16 * RSTEP) {
-                unsigned c[16];
-#pragma unroll
-                for (int u = 0; u < 16; u++) c[u] = r0 + u * RSTEP < G1 ? counts[(size_t)(r0 + u * RSTEP) * NB + b] : 0u;
-#pragma unroll
-                for (int u = 0; u < 16; u++) sum += c[u];
-            }
-        }
-        if (sum) atomicAdd(&plan.nsplit[b], sum);
-        for (int j = threadIdx.x; j < G1; j += NTHREADS) atomicAdd(&plan.nmerge[hotof[j]], 1u);
-    }
-    __syncthreads();
-    const int b = threadIdx.x;
-    unsigned k = 0, m = 0;
-    if (b < NBMAX) {
-        k = (plan.nsplit[b] + COLD_TARGET - 1) / COLD_TARGET;
-        if (k > (unsigned)G1) k = (unsigned)G1;
-        m = (plan.nmerge[b] + MERGE_ROWS - 1) / MERGE_ROWS;
-    }
-    // items in the low word, partial copies in the high word
-    const unsigned long long mine = (unsigned long long)(k + m * MSEG) | ((unsigned long long)(k + m) << 32);
-    const unsigned long long incl = mjt_block_scan_value(mine, wsum);
-    if (b < NBMAX) {
-        plan.nsplit[b] = k;
-        plan.nmerge[b] = m;
-        plan.first[b] = (unsigned)incl - (k + m * MSEG);
-        plan.pfirst[b] = (unsigned)(incl >> 32) - (k + m);
-    }
-    if (b == NBMAX - 1) {
-        plan.first[NBMAX] = (unsigned)incl;
-        plan.pfirst[NBMAX] = (unsigned)(incl >> 32);
-    }
-    __syncthreads();
-}
-
-// ---- plan: one workgroup computes the work plan of the cold pass -------------------------------------------
-// layout of the plan in memory, in words: nsplit[NBMAX], nmerge[NBMAX], first[NBMAX + 1], pfirst[NBMAX + 1], any_ovf
-extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_PLAN(Params p) {
-    unsigned* __restrict__ planout = (unsigned*)p.a[5];
-    const int G1 = (int)(unsigned long long)p.a[7];
-    const int NB = (int)(unsigned long long)p.a[8];
-    const unsigned* __restrict__ counts = (const unsigned*)p.a[10];
-    const int* __restrict__ hotof = (const int*)p.a[14];
-    const unsigned* __restrict__ novf = (const unsigned*)p.a[16];
-    __shared__ mjt_plan plan;
-    __shared__ unsigned long long wsum[16];
-    __shared__ unsigned any_ovf;
-    if (threadIdx.x == 0) any_ovf = 0;
-    mjt_make_plan(plan, counts, hotof, G1, NB, wsum);
-    for (int w = threadIdx.x; w < G1; w += NTHREADS)
-        if (novf[w]) any_ovf = 1;
-    __syncthreads();
-    for (int t = threadIdx.x; t < NBMAX; t += NTHREADS) {
-        planout[t] = plan.nsplit[t];
-        planout[NBMAX + t] = plan.nmerge[t];
-    }
-    for (int t = threadIdx.x; t <= NBMAX; t += NTHREADS) {
-        planout[2 * NBMAX + t] = plan.first[t];
-        planout[3 * NBMAX + 1 + t] = plan.pfirst[t];
-    }
-    if (threadIdx.x == 0) planout[4 * NBMAX + 2] = any_ovf;
-}
-
-// ---- cold: folds the lists into partial copies, and the partial copies of main MERGE_ROWS at a time ----------
-extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_COLD(Params p) {
-    const unsigned* __restrict__ planin = (const unsigned*)p.a[5];
+extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_TAIL(Params p) {
+    TX* __restrict__ xp = (TX*)p.a[0];
+    const long long bins = (long long)(unsigned long long)p.a[4];
     const long long per = (long long)(unsigned long long)p.a[6];
     const int G1 = (int)(unsigned long long)p.a[7];
     const int NB = (int)(unsigned long long)p.a[8];
@@ -445,126 +442,184 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_COLD(Params p) {
     const unsigned* __restrict__ counts = (const unsigned*)p.a[10];
     const mjt_pair* __restrict__ lists = (const mjt_pair*)p.a[11];
     const TX* __restrict__ pmain = (const TX*)p.a[12];
-    TX* __restrict__ pcold = (TX*)p.a[13];
+    const unsigned slot = (unsigned)(unsigned long long)p.a[13] & 1u;
     const int* __restrict__ hotof = (const int*)p.a[14];
     const mjt_pair* __restrict__ ovf = (const mjt_pair*)p.a[15];
     const unsigned* __restrict__ novf = (const unsigned*)p.a[16];
-    // the private copy of a list item, or the rows of a merge item on their way to being combined
-    constexpr size_t WIN_BYTES = sizeof(TW) * WBINS > sizeof(TA) * NTHREADS * 4 ? sizeof(TW) * WBINS : sizeof(TA) * NTHREADS * 4;
-    __shared__ __attribute__((aligned(16))) unsigned char win_bytes[WIN_BYTES];
+#if ABL & 256
+    unsigned long long* dbg = (unsigned long long*)p.a[17] + (size_t)blockIdx.x * 8;
+    const unsigned long long dbg_t0 = wall_clock64();
+    unsigned long long dbg_t1 = 0, dbg_kind = 0, dbg_t2 = 0;
+#endif
+    // the private copy of a list item, or the partial results of a merge item on their way to being combined
+    constexpr int GROUPS = NTHREADS / (MB / 4);               // a merge item: MB / 4 threads across, GROUPS sets of rows
+    constexpr size_t WIN_BYTES = sizeof(TW) * WBINS > sizeof(TA) * GROUPS * MB ? sizeof(TW) * WBINS : sizeof(TA) * GROUPS * MB;
+    // At least half of a compute unit's LDS, so that a compute unit takes one workgroup: the dispatcher fills a
+    // compute unit before it goes to the next, and two items on one compute unit share its path to memory
+    // while other compute units have none (measured with 64 KB copies: 24 us instead of 15).
+    constexpr size_t WIN_ALLOC = WIN_BYTES > 84 * 1024 ? WIN_BYTES : 84 * 1024;
+    __shared__ __attribute__((aligned(16))) unsigned char win_bytes[WIN_ALLOC];
     TW* win = (TW*)win_bytes;
     __shared__ mjt_plan plan;
     __shared__ unsigned length[512];                          // lengths of the lists of an item (G1 <= 512)
-    __shared__ int rows[MERGE_ROWS];
+    __shared__ int rows[512];                                 // main workgroups whose private copies an item merges
     __shared__ unsigned novf_s[512];                          // entries of each main workgroup's overflow list
     __shared__ unsigned long long wsum[16];
     __shared__ unsigned any_ovf, nmatch;
+    for (int t = threadIdx.x; t < TALLY; t += NTHREADS) {     // the copies of a counter: loads in flight together
+        unsigned c[TSUB], sum = 0;
+#pragma unroll
+        for (int u = 0; u < TSUB; u++) c[u] = mjt_tally[slot][u][t];
+#pragma unroll
+        for (int u = 0; u < TSUB; u++) sum += c[u];
+        if (t < NBMAX) plan.nsplit[t] = sum;
+        else if (t < 2 * NBMAX) plan.nrows[t - NBMAX] = sum;
+        else any_ovf = sum;
+    }
     for (int t = threadIdx.x; t < G1; t += NTHREADS) novf_s[t] = novf[t];
-    for (int t = threadIdx.x; t < NBMAX; t += NTHREADS) {
-        plan.nsplit[t] = planin[t];
-        plan.nmerge[t] = planin[NBMAX + t];
-    }
-    for (int t = threadIdx.x; t <= NBMAX; t += NTHREADS) {
-        plan.first[t] = planin[2 * NBMAX + t];
-        plan.pfirst[t] = planin[3 * NBMAX + 1 + t];
-    }
-    if (threadIdx.x == 0) any_ovf = planin[4 * NBMAX + 2];
-    // fetched together with the plan: a merge item then has one memory round trip less in front of its rows
+    // fetched together with the tallies: a merge item then has one memory round trip less in front of its rows
     const int my_hot = (int)threadIdx.x < G1 ? hotof[threadIdx.x] : -1;
+    if (blockIdx.x == 0)                                      // the next call's set: nobody reads or adds to it now
+        for (int t = threadIdx.x; t < TSUB * TALLY; t += NTHREADS) (&mjt_tally[slot ^ 1u][0][0])[t] = 0;
     __syncthreads();
+    {
+        const int b = threadIdx.x;
+        unsigned k = 0, m = 0;
+        if (b < NBMAX) {
+            k = (plan.nsplit[b] + COLD_TARGET - 1) / COLD_TARGET;
+            if (k > (unsigned)G1) k = (unsigned)G1;
+            m = plan.nrows[b] ? (unsigned)MSEG : 0u;
+        }
+        // list items in the low word, merge items in the high word
+        const unsigned long long incl = mjt_block_scan_value((unsigned long long)k | ((unsigned long long)m << 32), wsum);
+        if (b < NBMAX) {
+            plan.nsplit[b] = k;
+            plan.first[b] = (unsigned)incl - k;
+            plan.mfirst[b] = (unsigned)(incl >> 32) - m;
+        }
+        if (b == NBMAX - 1) {
+            plan.first[NBMAX] = (unsigned)incl;
+            plan.mfirst[NBMAX] = (unsigned)(incl >> 32);
+        }
+        __syncthreads();
+        if (b < NBMAX + 1) plan.mfirst[b] += plan.first[NBMAX];
+        __syncthreads();
+    }
     const TX ident = mjt_ident();
-    for (unsigned item = blockIdx.x; item < plan.first[NBMAX]; item += gridDim.x) {
+#if ABL & 256
+    dbg_t1 = wall_clock64();
+#endif
+    for (unsigned item = blockIdx.x; item < plan.mfirst[NBMAX]; item += gridDim.x) {
+        const bool merge = item >= plan.first[NBMAX];
+#if ABL & 256
+        dbg_kind = merge ? 2 : 1;
+#endif
+        const unsigned* __restrict__ firsts = merge ? plan.mfirst : plan.first;
         int bucket;
         {
             int lo = 0, hi = NBMAX - 1;                       // the last bucket whose first item is <= item: it has items,
             while (lo < hi) {                                 // buckets without share `first` with their successor
                 const int mid = (lo + hi + 1) >> 1;
-                if (plan.first[mid] <= item) lo = mid; else hi = mid - 1;
+                if (firsts[mid] <= item) lo = mid; else hi = mid - 1;
             }
             bucket = lo;
         }
-        const int within = (int)(item - plan.first[bucket]);
+        const int within = (int)(item - firsts[bucket]);
         const int SPLIT = (int)plan.nsplit[bucket];
-        if (within >= SPLIT) {
-            // merge item: segment sgm of the partial copies of main workgroups number g*MERGE_ROWS ... of this bucket
-            const int g = (within - SPLIT) / MSEG, sgm = (within - SPLIT) - g * MSEG;
+        // more than one item reaches the bins of this bucket: they combine in x through atomics
+        const bool shared = SPLIT + (plan.nrows[bucket] ? 1 : 0) > 1;
+        const long long bin0 = (long long)bucket * WBINS;
+        if (merge) {
+            // merge item: segment sgm of all private copies of this bucket
+            if (ABL & 4) continue;
+            const int sgm = within;
             const unsigned match = my_hot == bucket ? 1u : 0u;
             const unsigned incl = (unsigned)mjt_block_scan_value(match, wsum);
-            if (match && (int)(incl - 1) / MERGE_ROWS == g) rows[(incl - 1) % MERGE_ROWS] = threadIdx.x;
+            if (match) rows[incl - 1] = threadIdx.x;
             if (threadIdx.x == NTHREADS - 1) nmatch = incl;
             __syncthreads();
-            const int nrows = (int)nmatch - g * MERGE_ROWS < MERGE_ROWS ? (int)nmatch - g * MERGE_ROWS : MERGE_ROWS;
-            // MBINS / 4 threads across, the rows dealt to the groups of MBINS / 4 threads; combined through LDS
-            constexpr int ACROSS = MBINS / 4, GROUPS = NTHREADS / ACROSS;
+            const int nrows = (int)nmatch;
+            constexpr int ACROSS = MB / 4;
             const int col = threadIdx.x % ACROSS, grp = threadIdx.x / ACROSS;
-            const int t = sgm * MBINS + col * 4;
             TA acc[4] = {(TA)ident, (TA)ident, (TA)ident, (TA)ident};
-            // all rows of the thread in flight at once
-            constexpr int RPT = (MERGE_ROWS + GROUPS - 1) / GROUPS;
-            mjt_pack<TX, 4> v[RPT];
+            constexpr int RPT = MDEPTH;                       // rows of a thread in flight at once
+            for (int r0 = 0; r0 < nrows; r0 += GROUPS * RPT) {
+                mjt_pack<TX, 4> v[RPT];
 #pragma unroll
-            for (int j = 0; j < RPT; j++) {
-                const int r = grp + j * GROUPS;
-                mjt_load(v[j], pmain + (size_t)rows[r < nrows ? r : 0] * WBINS + t);
+                for (int j = 0; j < RPT; j++) {
+                    const int r = r0 + grp + j * GROUPS;
+                    mjt_load(v[j], pmain + ((size_t)sgm * G1 + rows[r < nrows ? r : 0]) * MB + col * 4);
+                }
+#pragma unroll
+                for (int j = 0; j < RPT; j++)
+                    if (r0 + grp + j * GROUPS < nrows) {
+#pragma unroll
+                        for (int k = 0; k < 4; k++) acc[k] = MERGE2(acc[k], (TA)v[j].v[k]);
+                    }
             }
+            TA* comb = (TA*)win_bytes;                        // GROUPS x MB values
 #pragma unroll
-            for (int j = 0; j < RPT; j++)
-                if (grp + j * GROUPS < nrows) {
-#pragma unroll
-                    for (int k = 0; k < 4; k++) acc[k] = MERGE2(acc[k], (TA)v[j].v[k]);
-                }
-            TA* comb = (TA*)win_bytes;                        // GROUPS x MBINS = NTHREADS * 4 values
-#pragma unroll
-            for (int k = 0; k < 4; k++) comb[grp * MBINS + col * 4 + k] = acc[k];
+            for (int k = 0; k < 4; k++) comb[grp * MB + col * 4 + k] = acc[k];
             __syncthreads();
-            if (grp == 0) {
-                mjt_pack<TX, 4> o;
-#pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    TA r = comb[col * 4 + k];
-                    for (int q = 1; q < GROUPS; q++) r = MERGE2(r, comb[q * MBINS + col * 4 + k]);
-                    o.v[k] = (TX)r;
+            if (threadIdx.x < MB) {                           // one bin per thread: neighbouring lanes, neighbouring bins
+                TA r = comb[threadIdx.x];
+                for (int q = 1; q < GROUPS; q++) r = MERGE2(r, comb[q * MB + threadIdx.x]);
+                const long long bin = bin0 + sgm * MB + threadIdx.x;
+                if (EXACT_BINS || bin < bins) {
+                    if (!shared || (ABL & 1)) xp[bin] = (TX)r;
+                    else if ((TX)r != ident) mjt_x_update(xp + bin, (TX)r);
                 }
-                mjt_store(pcold + (size_t)(plan.pfirst[bucket] + SPLIT + g) * WBINS + t, o);
             }
             __syncthreads();
             continue;
         }
         const int split = within;
-        TX* __restrict__ out = pcold + (size_t)(plan.pfirst[bucket] + split) * WBINS;
         for (int t = threadIdx.x; t < WBINS; t += NTHREADS) win[t] = mjt_win_from(ident);
         const int nsrc = (G1 - split + SPLIT - 1) / SPLIT;       // lists this item folds
         for (int t = threadIdx.x; t < nsrc; t += NTHREADS) length[t] = counts[(size_t)(split + t * SPLIT) * NB + bucket];
         __syncthreads();
-        // Each wave walks whole lists (no search for the list an entry belongs to), 64 consecutive entries per
-        // load and DEPTH loads in flight; when the item has fewer lists than waves, several waves share a list.
+        // Each wave walks whole lists (no search for the list an entry belongs to), 128 consecutive entries per
+        // load (two per lane: a list starts at a multiple of 16 bytes) and all of DEPTH loads in flight before
+        // the first is used: the pass is bound by memory round trips, not by bandwidth.  When the item has fewer
+        // lists than waves, several waves share a list.
         {
-            constexpr int WAVES = NTHREADS / 64, DEPTH = 8;
+            constexpr int WAVES = NTHREADS / 64, DEPTH = LDEPTH;
             const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
             int wpl = 1;                                          // waves per list
             while (wpl * 2 * nsrc <= WAVES) wpl *= 2;
-            const unsigned first_off = (unsigned)(wave % wpl) * 64u, off_step = (unsigned)wpl * 64u;
+            const unsigned first_off = (unsigned)(wave % wpl) * 128u, off_step = (unsigned)wpl * 128u;
             const int list_step = WAVES / wpl;
             int li = wave / wpl;
             unsigned off = first_off;
-            while (li < nsrc) {
-                mjt_pair e[DEPTH];
+            const mjt_pair* __restrict__ blists = lists + (size_t)bucket * G1 * CAP;   // G1 * CAP < 2^29 entries
+            while (li < nsrc && !(ABL & 2)) {
+                mjt_pack<mjt_pair, 2> e[DEPTH];
 #pragma unroll
                 for (int d = 0; d < DEPTH; d++) {
-                    e[d].bin = -1;
+                    e[d].v[0].bin = -1;
+                    e[d].v[1].bin = -1;
                     if (li < nsrc) {
                         const unsigned c = length[li];
-                        const unsigned q = off + lane;
-                        if (q < c) e[d] = lists[((size_t)bucket * G1 + (split + li * SPLIT)) * CAP + q];
+                        const unsigned q = off + 2 * lane;
+                        // (nothing loaded is modified afterwards: that would be a wait for the load)
+                        const mjt_pair* src = blists + ((unsigned)(split + li * SPLIT) * CAP + q);
+                        if (q + 1 < c) mjt_load(e[d], src);
+                        else if (q < c) e[d].v[0] = *src;
                         off += off_step;
                         if (off >= c) { li += list_step; off = first_off; }
                     }
                 }
 #pragma unroll
-                for (int d = 0; d < DEPTH; d++)
-                    if (e[d].bin >= 0) mjt_win_update(&win[e[d].bin & (WBINS - 1)], e[d].val);
+                for (int d = 0; d < DEPTH; d++) {
+                    if (e[d].v[0].bin >= 0) mjt_win_update(&win[e[d].v[0].bin & (WBINS - 1)], e[d].v[0].val);
+                    if (e[d].v[1].bin >= 0) mjt_win_update(&win[e[d].v[1].bin & (WBINS - 1)], e[d].v[1].val);
+                }
             }
         }
+#if ABL & 256
+        __syncthreads();
+        dbg_t2 = wall_clock64();
+#endif
         // entries that did not fit a list: the first item of the bucket scans the overflow lists
         if (split == 0 && any_ovf) {
             for (int w = 0; w < G1; w++) {
@@ -577,51 +632,24 @@ extern "C" __global__ __launch_bounds__(NTHREADS) void ENTRY_COLD(Params p) {
             }
         }
         __syncthreads();
-        for (int t = threadIdx.x * 4; t < WBINS; t += NTHREADS * 4) {
-            mjt_pack<TX, 4> o;
-#pragma unroll
-            for (int k = 0; k < 4; k++) o.v[k] = mjt_win_read(win[t + k]);
-            mjt_store(out + t, o);
+        for (int t = threadIdx.x; t < WBINS; t += NTHREADS) {
+            const long long bin = bin0 + t;
+            if (EXACT_BINS || bin < bins) {
+                const TW w = win[t];
+                if (!shared || (ABL & 1)) xp[bin] = mjt_win_read(w);
+                else if (w != mjt_win_from(ident)) mjt_x_update(xp + bin, mjt_win_read(w));
+            }
         }
         __syncthreads();
     }
-}
-
-// ---- final: x[bin] = merge of the partial copies of its bucket --------------------------------
-// workgroup = (bucket, segment of 256 bins); 64 lanes x 4 bins across, 4 groups of partial copies down
-extern "C" __global__ __launch_bounds__(256) void ENTRY_FINAL(Params p) {
-    TX* __restrict__ xp = (TX*)p.a[0];
-    const long long bins = (long long)(unsigned long long)p.a[4];
-    const unsigned* __restrict__ planin = (const unsigned*)p.a[5];
-    const TX* __restrict__ pcold = (const TX*)p.a[13];
-    constexpr int SEGS = WBINS / 256;
-    const int bucket = blockIdx.x / SEGS, seg = blockIdx.x - bucket * SEGS;
-    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
-    const int t = seg * 256 + lane * 4;
-    const int P = (int)(planin[bucket] + planin[NBMAX + bucket]);
-    const size_t first = planin[3 * NBMAX + 1 + bucket];
-    const TA ident = (TA)mjt_ident();
-    TA acc[4] = {ident, ident, ident, ident};
-#pragma unroll 8
-    for (int j = grp; j < P; j += 4) {
-        mjt_pack<TX, 4> v;
-        mjt_load(v, pcold + (first + j) * WBINS + t);
-#pragma unroll
-        for (int k = 0; k < 4; k++) acc[k] = MERGE2(acc[k], (TA)v.v[k]);
+#if ABL & 256
+    if (threadIdx.x == 0) {
+        dbg[0] = dbg_t0; dbg[1] = dbg_t1; dbg[2] = wall_clock64(); dbg[3] = dbg_kind; dbg[4] = dbg_t2;
+        unsigned smid;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(smid));
+        dbg[5] = smid;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(smid));
+        dbg[6] = smid;
     }
-    __shared__ TA comb[4][256];
-#pragma unroll
-    for (int k = 0; k < 4; k++) comb[grp][lane * 4 + k] = acc[k];
-    __syncthreads();
-    if (grp == 0) {
-        const long long b0 = (long long)bucket * WBINS + t;
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            TA r = comb[0][lane * 4 + k];
-            r = MERGE2(r, comb[1][lane * 4 + k]);
-            r = MERGE2(r, comb[2][lane * 4 + k]);
-            r = MERGE2(r, comb[3][lane * 4 + k]);
-            if (b0 + k < bins) xp[b0 + k] = (TX)r;
-        }
-    }
+#endif
 }

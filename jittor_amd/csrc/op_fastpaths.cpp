@@ -246,7 +246,7 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     if (bins >= (int64_t(1) << 31) || n >= (int64_t(1) << 36)) return false;
     if ((uintptr_t)y->ptr % 16 || (uintptr_t)index->ptr % 32 || (uintptr_t)x->ptr % 4) return false;
     Context& c = ctx();
-    int logw = env_int("MJT_SCATTER_LOGW", 14);              // 16384 bins: 64 KB (128 KB for float sums) of LDS per private copy
+    int logw = 14;                                            // 16384 bins: 64 KB (128 KB for float sums) of LDS per private copy
     while (logw > 8 && (int64_t(1) << (logw - 1)) >= bins) logw--;
     const int64_t W = int64_t(1) << logw;
     const int64_t NB = (bins + W - 1) / W;
@@ -254,18 +254,19 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     if (NB > 512) return false;                               // per-bucket tables live in LDS, one loading thread per bucket
     int64_t nbmax = 1;
     while (nbmax < NB) nbmax *= 2;
-    const int per_cu = env_int("MJT_SCATTER_WG_PER_CU", 1);
-    const int64_t cold_target = env_int("MJT_SCATTER_COLD_TARGET", 24576);   // list entries per cold item
-    const int acc64 = mode == 0 && x->dtype == MJT_FLOAT32 && env_int("MJT_SCATTER_ACC64", 1);
-    const int ept = env_int("MJT_SCATTER_EPT", 8);           // elements per thread and round
-    if (ept < 4 || ept % 4 || ept > 32) return false;
-    const int nflush = env_int("MJT_SCATTER_NFLUSH", 256);    // threads of a main workgroup that only append to the lists
-    if (nflush < 64 || nflush % 64 || nflush > 512) return false;
+    // Measured on the 2^24 -> 2^20 Zipf(1.1) scatter; every neighbouring value was slower.  list entries per list
+    // item of the tail pass: 16384 -> 23 us, 24576 -> 17.5, 32768 -> 18.3, 40960 -> 22 (tail pass); loads in flight
+    // per thread there: 8 (16 and 24 spill registers); threads of a main workgroup that only append to the lists:
+    // 64 -> 48 us, 128 -> 41, 256 -> 40 (main pass); elements per thread and round: 4 -> 44-48 us, 8 -> 40.
+    const int64_t cold_target = 24576;
+    const int ldepth = 8, mdepth = 8;
+    const int ept = 8, nflush = 256;
+    const int abl = env_int("MJT_ABLATE_SCATTER", 0);      // timing-only ablations (bench.py --ablate): results are wrong
+    const int acc64 = mode == 0 && x->dtype == MJT_FLOAT32;  // float sums in double: the one fast float atomic of the LDS
     // staging entries: what the private copy and the per-bucket table leave of the 160 KB of LDS, in two areas
     const int64_t lds_left = 160 * 1024 - 1024 - W * (acc64 ? 8 : 4) - (nbmax + 1) * 4;
     int64_t scap = lds_left / 16 / 64 * 64;
     if (scap > 4096) scap = 4096;
-    scap = env_int("MJT_SCATTER_SCAP", (int)scap);
     if (scap < 64 || scap * 16 > lds_left) return false;
     // identity
     uint32_t ident = 0;
@@ -275,43 +276,46 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
         else ident = mode == 1 ? 0u : 0xffffffffu;
     }
     // geometry of the main pass
-    int64_t G1 = (int64_t)c.prop.multiProcessorCount * per_cu;
+    int64_t G1 = (int64_t)c.prop.multiProcessorCount;
     if (G1 > 512) G1 = 512;
     const int64_t chunk = (int64_t)nthreads * 4;
     const int64_t per = ((n + G1 - 1) / G1 + chunk - 1) / chunk * chunk;
     G1 = n ? (n + per - 1) / per : 1;
-    // cold items: at most one per bucket plus population / cold_target (see mjt_make_plan)
-    // plus the partial copies of the merge items: at most one per 16 main workgroups of a bucket and one per bucket
-    const int64_t cold_items = NB + n / cold_target + 1 + G1 / 16 + (NB < G1 ? NB : G1) + 1;
-    int64_t cold_wgs = (int64_t)c.prop.multiProcessorCount * (acc64 ? 1 : 2);
-    if (cold_wgs > cold_items) cold_wgs = cold_items;
+    // items of the tail pass: at most one list item per bucket plus population / cold_target, and the merge items
+    // (bins of a bucket / 256 per bucket that was some main workgroup's hot one)
+    const int64_t mseg = W < 256 ? 1 : W / 256;
+    const int64_t tail_items = NB + n / cold_target + 1 + (NB < G1 ? NB : G1) * mseg;
+    int64_t tail_wgs = (int64_t)c.prop.multiProcessorCount;   // one per compute unit (by its LDS)
+    if (tail_wgs > tail_items) tail_wgs = tail_items;
     // A list holds four times its share of a uniformly spread input, plus 512 bytes: all workgroups append to
     // the lists of one bucket at about the same position, and lists that lie a power of two apart (32 KB for
     // 2^24 elements into 2^20 bins) put those appends into the same memory channels (main pass 40 instead of 44 us).
+    // Three times the share is as fast, twice overflows the Zipf head's lists (tail pass 37 us), eight times spreads
+    // the appends over 1 GB and the main pass takes 59 us.
     int64_t CAP = NB > 1 ? (4 * per / NB + 63) / 64 * 64 + 64 : 64;
     if (CAP > per) CAP = (per + 63) / 64 * 64;
 
     std::ostringstream key;
     key << "sc1|" << x->dtype << "|" << index->dtype << "|" << mode << "|" << logw << "|" << nbmax << "|" << nthreads << "|" << nflush << "|" << ept
-        << "|" << scap << "|" << cold_target << "|" << acc64 << "|" << (bins % W == 0);
-    static const char* parts[] = {"main", "plan", "cold", "final"};
-    JitKernel* ks[4];
+        << "|" << scap << "|" << cold_target << "|" << acc64 << "|" << (bins % W == 0) << "|" << abl << "|" << ldepth << "|" << mdepth;
+    static const char* parts[] = {"main", "tail", "reset"};
+    JitKernel* ks[3];
     bool have = true;
-    for (int i = 0; i < 4; i++) have = (ks[i] = cached(key.str() + "|" + parts[i])) != nullptr && have;
+    for (int i = 0; i < 3; i++) have = (ks[i] = cached(key.str() + "|" + parts[i])) != nullptr && have;
     if (!have) {
         std::ostringstream name;
         name << "mjt_scatter1d_" << mjt_op_name(op) << "_" << mjt_dtype_name(x->dtype) << "_" << mjt_dtype_name(index->dtype)
              << "_w" << W << "_b" << nbmax << "_e" << ept << "_s" << scap;
         std::ostringstream src;
-        src << "#define ENTRY_MAIN " << name.str() << "_main\n#define ENTRY_PLAN " << name.str() << "_plan\n#define ENTRY_COLD "
-            << name.str() << "_cold\n#define ENTRY_FINAL " << name.str() << "_final\n#define COLD_TARGET " << cold_target
+        src << "#define ENTRY_MAIN " << name.str() << "_main\n#define ENTRY_TAIL " << name.str() << "_tail\n#define ENTRY_RESET "
+            << name.str() << "_reset\n#define LDEPTH " << ldepth << "\n#define MDEPTH " << mdepth << "\n#define ABL " << abl << "\n#define COLD_TARGET " << cold_target
             << "u\n#define TX " << dtype_cname(x->dtype) << "\n#define TE " << dtype_cname(index->dtype) << "\n#define WBINS "
             << W << "\n#define LOGW " << logw << "\n#define NBMAX " << nbmax << "\n#define NTHREADS " << nthreads
             << "\n#define EXACT_BINS " << (bins % W == 0 ? 1 : 0) << "\n#define NFLUSH " << nflush << "\n#define EPT " << ept << "\n#define SCAP " << scap << "\n#define ACC64 " << acc64
             << "\n#define MODE " << mode << "\n#define IDENT_BITS " << ident << "u\n";
         src << embedded_source("prelude.h") << "\n" << embedded_source("scatter1d.h") << "\n";
         JitKernel* first = jit_get(src.str(), name.str() + "_main");
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < 3; i++) {
             JitKernel* k = i == 0 ? first : new JitKernel();
             if (i) {
                 k->name = name.str() + "_" + parts[i];
@@ -324,14 +328,14 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
     }
     // scratch layout
     auto align = [](size_t v) { return (v + 255) / 256 * 256; };
-    const size_t off_hotof = align((size_t)(4 * nbmax + 3) * 4);          // after the plan
+    const size_t off_hotof = 0;
     const size_t off_novf = off_hotof + align((size_t)G1 * 4);
     const size_t off_counts = off_novf + align((size_t)G1 * 4);
     const size_t off_pmain = off_counts + align((size_t)G1 * NB * 4);
-    const size_t off_pcold = off_pmain + align((size_t)G1 * W * 4);
-    const size_t off_lists = off_pcold + align((size_t)cold_items * W * 4);
+    const size_t off_lists = off_pmain + align((size_t)G1 * W * 4);
     const size_t off_ovf = off_lists + align(NB > 1 ? (size_t)G1 * NB * CAP * 8 : 0);
-    const size_t total = off_ovf + align(NB > 1 ? (size_t)G1 * per * 8 : 0);
+    const size_t off_dbg = off_ovf + align(NB > 1 ? (size_t)G1 * per * 8 : 0);
+    const size_t total = off_dbg + ((abl & 256) ? 512 * 64 : 0);
     // about 40 bytes of scratch per input element: when that is more than a sixteenth of the device's memory, or
     // the arena cannot grow, the generic kernel (global atomics, no scratch) takes the call
     if (!c.dry_run && total > c.prop.totalGlobalMem / 16) return false;
@@ -342,15 +346,35 @@ bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_
         (void)hipGetLastError();
         return false;
     }
+    // The main pass writes the identity into x beside its stream (each workgroup a slice); with few main
+    // workgroups and many bins that would take longer than the stream, and a launch of its own fills x.
+    const bool fill_in_main = bins <= G1 * 65536;
+    // ks[0]->state: [0] calls completed with this code object (its parity names the tally set of the next call),
+    // [1] 1 when both tally sets are known to be zero or about to be cleared by a tail pass that was launched
+    JitKernel* owner = ks[0];
     std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), bits_of_ptr(index->ptr), (uint64_t)n, (uint64_t)bins,
-                            bits_of_ptr(base), (uint64_t)per, (uint64_t)G1, (uint64_t)NB, (uint64_t)CAP,
+                            (uint64_t)(fill_in_main ? 1 : 0), (uint64_t)per, (uint64_t)G1, (uint64_t)NB, (uint64_t)CAP,
                             bits_of_ptr(base + off_counts), bits_of_ptr(base + off_lists), bits_of_ptr(base + off_pmain),
-                            bits_of_ptr(base + off_pcold), bits_of_ptr(base + off_hotof), bits_of_ptr(base + off_ovf),
-                            bits_of_ptr(base + off_novf), 0, 0, 0};
+                            owner->state[0] & 1, bits_of_ptr(base + off_hotof), bits_of_ptr(base + off_ovf),
+                            bits_of_ptr(base + off_novf), bits_of_ptr(base + off_dbg), 0, 0};
+    if (!owner->state[1]) jit_launch(ks[2], 1, 1, (unsigned)nthreads, 0, a);
+    owner->state[1] = 0;                                      // until the tail pass of this call is under way
+    if (!fill_in_main) launch_fill_pattern(x->ptr, ident, 4, (size_t)bins);
     jit_launch(ks[0], (unsigned)G1, 1, (unsigned)nthreads, 0, a);
-    jit_launch(ks[1], 1, 1, (unsigned)nthreads, 0, a);
-    jit_launch(ks[2], (unsigned)cold_wgs, 1, (unsigned)nthreads, 0, a);
-    jit_launch(ks[3], (unsigned)(NB * (W / 256)), 1, 256, 0, a);
+    jit_launch(ks[1], (unsigned)tail_wgs, 1, (unsigned)nthreads, 0, a);
+    owner->state[0]++;
+    owner->state[1] = 1;
+    if ((abl & 256) && !c.dry_run && owner->state[0] == 30) {   // development only: when each tail workgroup did what
+        HIP_CHECK(hipStreamSynchronize(c.stream));
+        std::vector<uint64_t> d((size_t)tail_wgs * 8);
+        HIP_CHECK(hipMemcpy(d.data(), base + off_dbg, d.size() * 8, hipMemcpyDeviceToHost));
+        uint64_t t0 = ~0ull;
+        for (int64_t i = 0; i < tail_wgs; i++) t0 = std::min(t0, d[i * 8]);
+        for (int64_t i = 0; i < tail_wgs; i++)
+            fprintf(stderr, "tailwg %3d kind %d start %6.2f plan %6.2f lists %6.2f end %6.2f xcc %d hwid %08x\n", (int)i, (int)d[i * 8 + 3],
+                    (d[i * 8] - t0) * 0.01, (d[i * 8 + 1] - t0) * 0.01, d[i * 8 + 4] ? (d[i * 8 + 4] - t0) * 0.01 : 0.0, (d[i * 8 + 2] - t0) * 0.01,
+                    (int)d[i * 8 + 5], (unsigned)d[i * 8 + 6]);
+    }
     return true;
 }
 

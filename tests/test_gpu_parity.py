@@ -380,6 +380,30 @@ def test_scatter_1d_fast_path(gpu, n, bins):
     assert np.array_equal(got, np.bincount(idx[ok], minlength=bins).astype(np.int32))
 
 
+def test_scatter_1d_add_propagates_nan(gpu):
+    """The reference's loop is x[idx] = x[idx] + y (reindex_reduce_op.cc:123-130): one NaN update makes its bin
+    NaN and leaves every other bin alone.  The bins are chosen so that NaNs pass through each route of the 1-d
+    scatter: the LDS copy of the hot bucket, the lists of the other buckets (several list items combining in x
+    through atomics for the well-filled bucket, a single storing item for the others), and a bin nobody else updates."""
+    rng = np.random.default_rng(23)
+    n, bins = 1 << 21, 1 << 18
+    v = rng.random(n, dtype=np.float32)
+    idx = np.where(rng.random(n) < 0.6, rng.integers(0, 3000, n),
+                   np.where(rng.random(n) < 0.5, rng.integers(16384, 32768, n), rng.integers(0, bins - 1, n))).astype(np.int32)
+    nan_bins = np.array([5, 2999, 20000, 32767, 100000, 200001, bins - 1], np.int64)
+    where = rng.choice(n, nan_bins.size * 3, replace=False)
+    idx[where] = np.repeat(nan_bins, 3)
+    v[where] = np.nan
+    got = jt.array(v).reindex_reduce("add", [bins], ["@e0(i0)"], extras=[jt.array(idx)]).data
+    assert L.last_kernel().startswith("mjt_scatter1d_add")
+    want = O.reindex_reduce(v, "add", [bins], ["@e0(i0)"], extras=[idx])
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.isnan(got).sum() == nan_bins.size
+    assert np.isnan(got[nan_bins]).all()
+    fin = ~np.isnan(want)
+    ref = np.bincount(idx[~np.isnan(v)], weights=v[~np.isnan(v)].astype(np.float64), minlength=bins)
+    assert np.allclose(got[fin], ref[fin], rtol=1e-4, atol=1e-6)
+
+
 def _scatter_check(v, idx, bins, ops=("add", "maximum", "minimum")):
     ok = (idx >= 0) & (idx < bins)
     jv, ji = jt.array(v), jt.array(idx, "int64" if idx.dtype == np.int64 else "int32")
