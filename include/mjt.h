@@ -274,6 +274,28 @@ typedef struct {
 int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y,
                     const mjt_conv_params* p);
 
+/* The same convolution with the weights prepared once.  The reference's relay
+ * target prepares per jit key and keeps what it prepared across calls
+ * (extern/cuda/cudnn/ops/cudnn_conv_op.cc:218-299: the algorithm found for a
+ * key is cached and reused); here what can be kept is the rearrangement of w
+ * into the order the MFMA kernel consumes, which mjt_conv2d_meta otherwise
+ * repeats on every call.
+ *   mjt_conv2d_meta_pack    writes that rearrangement of w into `packed`
+ *                           (device memory, 16-byte aligned, at least as many
+ *                           bytes as w; x and y give the shapes of the calls
+ *                           that will follow, their data is not touched);
+ *   mjt_conv2d_meta_packed  is mjt_conv2d_meta on weights packed by
+ *                           mjt_conv2d_meta_pack for the same shapes, dtypes
+ *                           and parameters (w gives the shape; its data is
+ *                           not read).
+ * Both return MJT_ERR_UNSUPPORTED for a convolution that does not run on
+ * packed weights (float32, channel counts or widths the MFMA kernel does not
+ * take, 1x1 convolutions sent to the matrix product): call mjt_conv2d_meta. */
+int mjt_conv2d_meta_pack(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y,
+                         const mjt_conv_params* p, void* packed, size_t packed_bytes);
+int mjt_conv2d_meta_packed(const mjt_tensor* x, const mjt_tensor* w, const void* packed,
+                           const mjt_tensor* y, const mjt_conv_params* p);
+
 /* The grouped form (python/jittor/nn.py:1272-1294: reindex(x) * reindex(w) ->
  * reindex_reduce.add, the group count handed to the tuner as compile option
  * "G"): x [N, groups*Cg, H, W], w [K, Cg, R, S], y [N, K, OH, OW]; output

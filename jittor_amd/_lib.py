@@ -91,7 +91,7 @@ EXPORTS = ["mjt_init", "mjt_shutdown", "mjt_last_error", "mjt_get_device_info",
            "mjt_alloc", "mjt_free", "mjt_h2d", "mjt_d2h", "mjt_d2d", "mjt_fill_u32",
            "mjt_sync", "mjt_event_create", "mjt_event_record", "mjt_event_elapsed_ms",
            "mjt_event_destroy", "mjt_reduce", "mjt_reduce_static", "mjt_reindex", "mjt_reindex_reduce",
-           "mjt_fused_elementwise", "mjt_fused_reduce", "mjt_conv2d_meta", "mjt_conv2d_meta_grouped", "mjt_conv2d_meta_dgrad", "mjt_conv2d_meta_wgrad", "mjt_conv2d_meta_wgrad_grouped",
+           "mjt_fused_elementwise", "mjt_fused_reduce", "mjt_conv2d_meta", "mjt_conv2d_meta_pack", "mjt_conv2d_meta_packed", "mjt_conv2d_meta_grouped", "mjt_conv2d_meta_dgrad", "mjt_conv2d_meta_wgrad", "mjt_conv2d_meta_wgrad_grouped",
            "mjt_reindex_then_reduce", "mjt_fused_reindex_reduce", "mjt_matmul", "mjt_matmul_available",
            "mjt_expr_affine",
            "mjt_jit_stats", "mjt_last_kernel"]
@@ -141,6 +141,10 @@ def load():
     lib.mjt_fused_reduce.argtypes = [ctypes.POINTER(FusedDesc), ctypes.POINTER(Tensor), ctypes.c_int, ctypes.c_uint32]
     lib.mjt_conv2d_meta.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.POINTER(Tensor),
                                     ctypes.POINTER(ConvParams)]
+    lib.mjt_conv2d_meta_pack.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.POINTER(Tensor),
+                                         ctypes.POINTER(ConvParams), ctypes.c_void_p, ctypes.c_size_t]
+    lib.mjt_conv2d_meta_packed.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.c_void_p, ctypes.POINTER(Tensor),
+                                           ctypes.POINTER(ConvParams)]
     lib.mjt_conv2d_meta_grouped.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.POINTER(Tensor),
                                             ctypes.POINTER(ConvParams), ctypes.c_int]
     lib.mjt_conv2d_meta_dgrad.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.POINTER(Tensor),

@@ -72,6 +72,14 @@ typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
 
 struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as pointers: global address space)
 
+// ABL (0 in production): timing-only ablations, results are wrong with any bit set.  1 no output stores, 2 no input
+// rows (neither loaded nor written to LDS), 4 (only together with 1 and 2) no weight slabs copied, no fragment reads
+// from LDS and no barrier per step: 7 leaves the MFMAs alone, 16 no MFMAs: leaves the data movement alone.  The host
+// admits 0, 1, 2, 3, 7, 16 and 17 only.
+#ifndef ABL
+#define ABL 0
+#endif
+
 #define KSTEPS (CB / 32)                    // MFMA k-steps per tap in a channel block of CB (32 or 64) channels
 #define KO_WG (16 * MT * WKO)
 #define NWAVES (WPX * WKO)
@@ -122,12 +130,20 @@ __device__ __forceinline__ unsigned mjt_xor4(unsigned v) {
 // use for them, and no copies are made to feed an MFMA); before and after the loop they are tied to points
 // behind explicit idle cycles.
 __device__ __forceinline__ void mjt_mfma(mjt_f32x4& c, const mjt_u32x4v& a, const mjt_u32x4v& b) {
+#if ABL & 16
+    asm volatile("" : "+a"(c) : "v"(a), "v"(b));
+#else
     asm volatile(MJT_MFMA_ASM " %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+#endif
 }
 __device__ __forceinline__ void mjt_keep(const mjt_u32x4v& x) { asm volatile("" : : "v"(x)); }     // x is in its registers up to here
 __device__ __forceinline__ void mjt_pin(mjt_f32x4& x) { asm volatile("" : "+a"(x)); }             // what reads x later comes after this point
 template <int OFF> __device__ __forceinline__ void mjt_ds_read(mjt_u32x4v& dst, unsigned addr) {
+#if ABL & 4
+    asm volatile("" : "+v"(dst) : "v"(addr));
+#else
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+#endif
 }
 // wait until at most N LDS operations issued after the one that fills x are outstanding (LDS returns in order)
 template <int N> __device__ __forceinline__ void mjt_lds_wait(mjt_u32x4v& x) {
@@ -310,6 +326,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         __attribute__((address_space(3))) unsigned short* dst =
             (__attribute__((address_space(3))) unsigned short*)&as_ring[0] + (slot * SLAB + wave * (FPL * 1024)) / 2;
         const unsigned voff = (unsigned)lane * 16;
+        if (ABL & 4) return;
         mjt_static_for<0, FPL>([&](auto fc) {
             constexpr int f = decltype(fc)::v;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (__attribute__((address_space(3))) void*)(dst + (f >> 2) * 2048), 16, (int)voff,
@@ -330,7 +347,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // in the loop, so their number is known).
     auto step_sync = [&](auto nc) {                  // nc: loads issued in the last NS - 3 steps, this one included
         asm volatile("s_waitcnt vmcnt(%0)" : : "n"(decltype(nc)::v < 63 ? decltype(nc)::v : 63) : "memory");
-        asm volatile("s_barrier" : : : "memory");
+        if (!(ABL & 4)) asm volatile("s_barrier" : : : "memory");
     };
 
     int buf = 0;                                  // LDS buffer that holds the current channel block
@@ -396,7 +413,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
 #pragma unroll 1
         for (int cb = 0; cb < NCB; cb++) {
             const bool more = cb + 1 < NCB;
-            const bool feed = more || next_lrows;                // somebody needs another block of input rows
+            const bool feed = (more || next_lrows) && !(ABL & 2);   // somebody needs another block of input rows
             const int f_r0 = more ? r0 : next_r0, f_lrows = more ? LR_ : next_lrows, f_cb = more ? cb + 1 : 0;
             const int my_first = wave * IPW, my_limit = (wave + 1) * IPW < ITEMS ? (wave + 1) * IPW : ITEMS;
             // nothing is under way here
@@ -517,7 +534,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
             const int q0 = t * 16 + lg_e * 4;
             const int r = q0 / OW_, col = q0 - r * OW_;
             const int orow = r0 + wpx * TRW_ + r;
-            if (q0 < TRW_ * OW_ && orow < row_lim) {
+            if (q0 < TRW_ * OW_ && orow < row_lim && !(ABL & 1)) {
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
                     const mjt_f32x4 v = acc[m][t];
@@ -538,7 +555,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                 const int q = t * 16 + lg_e * 4 + i;
                 const int r = q / OW_, col = q - r * OW_;
                 const int orow = r0 + wpx * TRW_ + r;
-                if (q < TRW_ * OW_ && orow < row_lim) {
+                if (q < TRW_ * OW_ && orow < row_lim && !(ABL & 1)) {
 #pragma unroll
                     for (int m = 0; m < MT; m++) {
                         const size_t o = (((size_t)n * YK_ + ko_base + m * 16 + l16_e) * OH_ + orow) * OW_ + col;

@@ -76,7 +76,11 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
 // free_extent: y's rows and columns are taken as they are instead of checked against the extents that stride, padding and
 // taps give (output (oh, ow) reads x around (oh*sh - ph, ow*sw - pw) whatever oh and ow; outside the image x is 0): what the
 // stride phases of an input gradient need, whose zero margins differ between the two ends of an axis.
-void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p, int64_t G, bool free_extent = false) {
+// packed / pack_mode: 0 the call packs the weights itself (into the library's buffer) and runs; 1 it only packs them
+// into `packed`; 2 it runs on weights packed by an earlier call of mode 1 for the same shapes and parameters.  Modes 1
+// and 2 exist for the MFMA kernel only and fail with MJT_ERR_UNSUPPORTED for a convolution that takes another route.
+void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p, int64_t G, bool free_extent = false,
+               int pack_mode = 0, void* packed = nullptr) {
     require_init();
     check_tensor(x, "conv x");
     check_tensor(w, "conv w");
@@ -203,10 +207,13 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             if (atoi(e) >= 3 && atoi(e) <= NSLAB) NSLAB = atoi(e);
         MJT_CHECK(NSLAB >= 3, "conv: internal: no room for the weight ring");
         const int stage_depth = getenv("MJT_CONV_SD") && atoi(getenv("MJT_CONV_SD")) >= 2 && atoi(getenv("MJT_CONV_SD")) <= 8 ? atoi(getenv("MJT_CONV_SD")) : 4;
+        const int abl = getenv("MJT_ABLATE_CONV") ? atoi(getenv("MJT_ABLATE_CONV")) : 0;   // timing-only ablations (bench.py --ablate): results are wrong
+        MJT_CHECK(abl == 0 || abl == 1 || abl == 2 || abl == 3 || abl == 7 || abl == 16 || abl == 17,
+                  "conv: MJT_ABLATE_CONV must be one of 0, 1, 2, 3, 7, 16, 17");
         std::ostringstream geo_g;                        // the kernel's K_ is a group's; XC_ / YK_ are the strides of x and y between images
         geo_g << geo.str() << "#undef K_\n#define K_ " << Kg << "\n#define XC_ " << C * G << "\n#define YK_ " << K << "\n";
         key << "mfma|" << half << "|" << geo_g.str() << TRW << "|" << (y->dtype != MJT_FLOAT32) << "|" << WKO << "|" << WPX << "|" << RPW << "|" << MT << "|" << WPS
-            << "|" << stage_depth << "|" << CBLK << "|" << NSLAB;
+            << "|" << stage_depth << "|" << CBLK << "|" << NSLAB << "|" << abl;
         JitKernel* k = cached(key.str());
         JitKernel* kp = cached(key.str() + "|pack");
         if (!k || !kp) {
@@ -219,7 +226,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                 << "#define MT " << MT << "\n#define WKO " << WKO << "\n#define WPX " << WPX << "\n#define TRW " << TRW << "\n#define NT " << NT << "\n#define LROWS " << LROWS << "\n#define LCOLS " << LCOLS
                 << "\n#define RPW " << RPW << "\n#define NFULL " << NFULL << "\n#define TAIL_TRW " << TAIL_TRW << "\n#define TAIL_NT "
                 << TAIL_NT << "\n#define TAIL_LROWS " << TAIL_LROWS << "\n#define Y_BF16 " << (y->dtype != MJT_FLOAT32 ? 1 : 0) << "\n#define IN_F16 " << (half ? 1 : 0)
-                << "\n#define WPS " << WPS << "\n#define CB " << CBLK << "\n#define NS " << NSLAB << "\n#define STAGE_DEPTH " << stage_depth << "\n";
+                << "\n#define ABL " << abl << "\n#define WPS " << WPS << "\n#define CB " << CBLK << "\n#define NS " << NSLAB << "\n#define STAGE_DEPTH " << stage_depth << "\n";
             src << embedded_source("conv_mfma.h") << "\n";
             k = jit_get(src.str(), name.str());
             kp = new JitKernel();
@@ -230,7 +237,8 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             remember(key.str() + "|pack", kp);
         }
         size_t wbytes = (size_t)numel(w) * 2;
-        if (!c.dry_run && wbytes > g_wpack_bytes) {
+        if (pack_mode) MJT_CHECK(packed && (uintptr_t)packed % 16 == 0, "conv: packed weights must be a 16-byte aligned device buffer");
+        if (!pack_mode && !c.dry_run && wbytes > g_wpack_bytes) {
             if (g_wpack) {
                 HIP_CHECK(hipStreamSynchronize(c.stream));
                 HIP_CHECK(hipFree(g_wpack));
@@ -248,15 +256,20 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int64_t ysz = y->dtype == MJT_FLOAT32 ? 4 : 2;
         for (int64_t g = 0; g < G; g++) {
             const char* wsrc = (const char*)w->ptr + g * wg * 2;
-            char* wdst = (char*)g_wpack + g * wg * 2;
-            std::vector<uint64_t> pa{bits_of_ptr(wsrc), bits_of_ptr(wdst), 0, 0};
-            jit_launch(kp, (unsigned)pblocks, 1, 256, 0, pa);
+            char* wdst = (char*)(pack_mode ? packed : g_wpack) + g * wg * 2;
+            if (pack_mode != 2) {
+                std::vector<uint64_t> pa{bits_of_ptr(wsrc), bits_of_ptr(wdst), 0, 0};
+                jit_launch(kp, (unsigned)pblocks, 1, 256, 0, pa);
+            }
+            if (pack_mode == 1) continue;
             std::vector<uint64_t> a{bits_of_ptr((const char*)x->ptr + g * C * H * W * 2), bits_of_ptr(wdst),
                                     bits_of_ptr((char*)y->ptr + g * Kg * OH * OW * ysz), (uint64_t)N};
             jit_launch(k, (unsigned)blocks, 1, (unsigned)(64 * WPX * WKO), 0, a);
         }
         return;
     }
+
+    if (pack_mode) MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv: this convolution does not run on packed weights (mjt_conv2d_meta takes it)");
 
     // ---- column matrices x weights on the GEMM kernel -----------------------------------
     // What the MFMA convolution kernel does not take (float32, odd widths, channel counts that are no multiple of 64,
@@ -681,6 +694,20 @@ extern "C" int mjt_conv2d_meta_dgrad(const mjt_tensor* dy, const mjt_tensor* w, 
 
 extern "C" int mjt_conv2d_meta(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p) {
     return mjt::guarded([&] { mjt::conv_impl(x, w, y, p, 1); });
+}
+
+extern "C" int mjt_conv2d_meta_pack(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p,
+                                    void* packed, size_t packed_bytes) {
+    return mjt::guarded([&] {
+        mjt::check_tensor(w, "conv w");
+        MJT_CHECK(packed_bytes >= (size_t)mjt::numel(w) * mjt::dtype_size(w->dtype), "conv: the packed weights need as many bytes as w");
+        mjt::conv_impl(x, w, y, p, 1, false, 1, packed);
+    });
+}
+
+extern "C" int mjt_conv2d_meta_packed(const mjt_tensor* x, const mjt_tensor* w, const void* packed, const mjt_tensor* y,
+                                      const mjt_conv_params* p) {
+    return mjt::guarded([&] { mjt::conv_impl(x, w, y, p, 1, false, 2, const_cast<void*>(packed)); });
 }
 
 extern "C" int mjt_conv2d_meta_grouped(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, const mjt_conv_params* p,

@@ -750,6 +750,45 @@ def test_conv_mfma_matches_oracle(gpu, case):
     assert np.abs(got2 - ref).max() <= 1e-4 * scale
 
 
+def test_conv_packed_weights_entry(gpu):
+    """mjt_conv2d_meta_pack + mjt_conv2d_meta_packed (weights rearranged once, several calls on them) give the bits
+    of mjt_conv2d_meta, which test_conv_mfma_matches_oracle holds against the oracle; the weights' own buffer may
+    change after packing without effect; a convolution that takes another route is refused."""
+    import ctypes
+    lib = L.load()
+    rng = np.random.default_rng(21)
+    for xs, ws, params, out in (((3, 64, 28, 24), (256, 64, 3, 3), (2, 2, 1, 1, 1, 1), "float32"),
+                                ((2, 128, 24, 24), (128, 128, 3, 3), (1, 1, 1, 1, 1, 1), "bfloat16")):
+        wb = _bf16(rng.standard_normal(ws) * 0.05)
+        w = jt.from_storage(wb, "bfloat16")
+        packed = jt.zeros([int(np.prod(ws))], "bfloat16")
+        p = L.ConvParams(*params)
+        for trial in range(2):                              # two inputs on the same packed weights
+            xb = _bf16(rng.standard_normal(xs))
+            want, kern = _conv_call(xb, wb, params, out_dtype=out)
+            assert kern.startswith("mjt_conv_mfma_bf16")
+            x = jt.from_storage(xb, "bfloat16")
+            y = jt.zeros(list(want.shape), out)
+            tx, tw = L.tensor(x.raw_ptr(), "bfloat16", x.shape), L.tensor(w.raw_ptr(), "bfloat16", w.shape)
+            ty = L.tensor(y.raw_ptr(), out, y.shape)
+            if trial == 0:
+                L.check(lib.mjt_conv2d_meta_pack(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p),
+                                                 packed.raw_ptr(), int(np.prod(ws)) * 2))
+                assert L.last_kernel().endswith("_pack")
+                L.check(lib.mjt_fill_u32(w.raw_ptr(), 0x7fc07fc0, int(np.prod(ws)) // 2))      # w itself is not read any more
+            L.check(lib.mjt_conv2d_meta_packed(ctypes.byref(tx), ctypes.byref(tw), packed.raw_ptr(), ctypes.byref(ty), ctypes.byref(p)))
+            assert L.last_kernel() == kern
+            got = L.d2h(y.raw_ptr(), y.shape, L.NP_STORAGE[out])
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (xs, trial)
+    # float32 takes another route: no packed form
+    x, w = jt.array(rng.standard_normal((1, 8, 6, 6)).astype(np.float32)), jt.array(rng.standard_normal((4, 8, 3, 3)).astype(np.float32))
+    y, buf = jt.zeros([1, 4, 6, 6], "float32"), jt.zeros([4 * 8 * 9], "float32")
+    tx, tw, ty = (L.tensor(v.raw_ptr(), "float32", v.shape) for v in (x, w, y))
+    p = L.ConvParams(1, 1, 1, 1, 1, 1)
+    assert lib.mjt_conv2d_meta_pack(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p), buf.raw_ptr(), 4 * 8 * 9 * 4) == -2
+    assert lib.mjt_conv2d_meta_packed(ctypes.byref(tx), ctypes.byref(tw), buf.raw_ptr(), ctypes.byref(ty), ctypes.byref(p)) == -2
+
+
 def test_conv_mfma_random_geometries(gpu):
     """Seeded sweep over geometries for the MFMA kernel (channel counts, map sizes with even widths, taps, stride,
     padding, dilation, 16-bit and float32 results): every case against a float64 sum of shifted products, per
