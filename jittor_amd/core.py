@@ -424,7 +424,9 @@ class Var:
     def assign(self, other):
         """This Var becomes `other` (shape, dtype and value), as VarHolder::assign rebinds a holder
         (python/jittor/src/var_holder.cc).  Ops built from the old value keep reading the old value."""
-        other = _as_var(other)
+        # a Python number becomes an array of its own: the Vars _as_var keeps per number are shared by every
+        # expression that names that number and must never be rebound
+        other = other if isinstance(other, Var) else array(other)
         if other is self:
             return self
         if self._op is not None or self._buf is not None or self._host is not None:

@@ -26,8 +26,9 @@ void* g_wgrad_part = nullptr;      // per-slice partial weight gradients (its ow
 size_t g_wgrad_bytes = 0;
 // column matrices of a chunk of images; float32 copy of a bfloat16 result; for the input gradient: rearranged weights,
 // and dy spread out with zeros or the results of the stride phases
-void* g_conv_scratch[4] = {nullptr, nullptr, nullptr, nullptr};
-size_t g_conv_scratch_bytes[4] = {0, 0, 0, 0};
+// [4]: weights with rows padded to 16 bytes for the product
+void* g_conv_scratch[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+size_t g_conv_scratch_bytes[5] = {0, 0, 0, 0, 0};
 
 void forget() {
     std::lock_guard<std::mutex> lock(g_mu);
@@ -42,7 +43,7 @@ void forget() {
     }
     g_wpack = g_wgrad_part = nullptr;
     g_wpack_bytes = g_wgrad_bytes = 0;
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < 5; i++) {
         g_conv_scratch[i] = nullptr;
         g_conv_scratch_bytes[i] = 0;
     }
@@ -288,6 +289,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             if (atoi(e) >= 1) chunk = atoi(e);
         if (chunk < 1) chunk = 1;
         if (chunk > N) chunk = N;
+        if (chunk > 65535) chunk = 65535;                       // the images of a chunk are the batch of one product launch
         void* cols = plain ? nullptr : conv_scratch(0, (size_t)(chunk * CRS * Ppad * esz));
         auto view = [](void* ptr, int dtype, std::initializer_list<int64_t> shape) {
             mjt_tensor t;
@@ -311,6 +313,19 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         }
         const char* idx[4] = {"i0", "i1", sh.c_str(), sw.c_str()};
         const char* ovc[1] = {over.c_str()};
+        // The product's MFMA kernel wants operand rows that are 16-byte multiples at 16-byte aligned addresses.  Weight
+        // rows that are not (3 x 7 x 7 float32 taps: 588 bytes) are copied into rows padded with zeros once per call.
+        const void* wmat = w->ptr;
+        int64_t lda = CRS;
+        if ((CRS * esz) % 16 || (uintptr_t)w->ptr % 16) {
+            lda = (CRS * esz + 15) / 16 * 16 / esz;
+            void* wpad = conv_scratch(4, (size_t)(K * lda * esz));
+            mjt_tensor tw = view(w->ptr, w->dtype, {K, CRS}), tp = view(wpad, w->dtype, {K, lda});
+            const char* widx[2] = {"i0", "i1"};                 // columns past CRS lie outside w: overflow value 0
+            if (mjt_reindex(&tw, &tp, 2, widx, 0.0, 0, nullptr, 0, nullptr) != MJT_OK)
+                MJT_FAIL(MJT_ERR_DEVICE, "conv: padding the weight rows failed: " << mjt_last_error());
+            wmat = wpad;
+        }
         for (int64_t n0 = 0; n0 < N; n0 += chunk) {
             const int64_t nb = N - n0 < chunk ? N - n0 : chunk;
             char* xn = (char*)x->ptr + n0 * C * H * W * esz;
@@ -330,7 +345,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             const int64_t cus = ctx().dry_run || ctx().prop.multiProcessorCount <= 0 ? 256 : ctx().prop.multiProcessorCount;
             const bool few = ((K + 127) / 128) * ((P + 127) / 128) * nb < cus;       // tiles of 128 x 128 would leave compute units idle
             const int tile_m = !short_sum ? 0 : K <= 64 || few ? 64 : 128, tile_n = !short_sum ? 0 : P <= 64 || few ? 64 : 128;
-            gemm_launch(x->dtype, y->dtype, w->ptr, plain ? (void*)xn : cols, yn, K, P, CRS, CRS, Ppad, P, 0, CRS * Ppad, K * P, nb, true, false,
+            gemm_launch(x->dtype, y->dtype, wmat, plain ? (void*)xn : cols, yn, K, P, CRS, lda, Ppad, P, 0, CRS * Ppad, K * P, nb, true, false,
                         tile_m, tile_n, !short_sum || CRS >= 256);
         }
         set_last_kernel(plain ? "conv_as_gemm" : "conv_as_reindex_gemm");

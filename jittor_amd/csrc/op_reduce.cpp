@@ -348,11 +348,15 @@ void reduce_impl(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
 
 // Looks up where this device keeps the fixed scratch array.  Runs once per device, with that device current
 // (mjt_init calls it after hipSetDevice).
+// Never fails: a device outside the table, or one whose copy of the array cannot be found, leaves its entry null, and
+// mjt_reduce_static then reports MJT_ERR_NOT_INIT for that device while every other entry point works.
 void reduce_static_setup(int device) {
-    MJT_CHECK(device >= 0 && device < kMaxDevices, "device " << device << " is outside the table of fixed scratch arrays");
-    if (g_static_ptr[device]) return;
+    if (device < 0 || device >= kMaxDevices || g_static_ptr[device]) return;
     void* ptr = nullptr;
-    HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch)));
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch)) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
     g_static_ptr[device] = ptr;
 }
 

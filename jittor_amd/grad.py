@@ -134,6 +134,9 @@ def _op_grad(op, inputs, out, dout, index):
     if isinstance(op, ReindexOp):                       # ops/reindex_op.cc:76-80: no gradient for the extras
         if index:
             return None
+        if getattr(op, "same_memory", False):           # a reshape: its gradient is the reshape back (ops/reshape_op.cc),
+            from . import misc                          # which shares dout's buffer, instead of a scatter with atomics
+            return misc.reshape(dout, list(x.shape))
         return reindex_reduce(dout, "add", x.shape, op.indexes, op.overflow_conditions, inputs[1:])
     if isinstance(op, ReindexReduceOp):                 # ops/reindex_reduce_op.cc:45-63
         if index:

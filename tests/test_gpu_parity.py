@@ -920,6 +920,7 @@ def test_conv_direct_small_shapes_and_fp32(gpu):
     dict(dt="float32", x=(12, 24, 7, 7), w=(40, 24, 3, 3), p=(1, 1, 1, 1, 1, 1)),                      # 49 pixels: padded rows, k ends inside a stage
     dict(dt="bfloat16", x=(3, 72, 9, 11), w=(40, 72, 3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16"),
     dict(dt="float32", x=(5, 40, 16, 16), w=(96, 40, 1, 1), p=(1, 1, 0, 0, 1, 1), plain=True, chunk=2),
+    dict(dt="float32", x=(8, 3, 64, 64), w=(32, 3, 7, 7), p=(2, 2, 3, 3, 1, 1)),      # a stem: weight rows of 588 bytes are padded to 16-byte multiples
     # the product on the direct-copy kernel (asked for by name: these shapes have too few tiles to get it by themselves):
     # weights shared across the batch, column matrices with the pixels innermost read with transposing reads
     dict(dt="bfloat16", x=(3, 64, 15, 15), w=(96, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), dma=True),

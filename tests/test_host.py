@@ -324,6 +324,29 @@ def test_grad_graph_is_built_from_path_ops():
     assert (x * 2).stop_grad()._history is None
     with jt.no_grad():
         assert (x * 2)._history is None
+    # the gradient of a reshape is the reshape back (ops/reshape_op.cc): again a reindex that shares memory, no scatter
+    g = jt.grad((x.reshape([6, 64]) * 3.0).sum(), x)
+    assert isinstance(g._op, core.ReindexOp) and getattr(g._op, "same_memory", False) and g.shape == x.shape
+
+
+def test_assign_of_a_python_number_leaves_the_shared_scalar_alone():
+    """Python numbers are kept as one host Var per value; x.assign(2.0) must rebind x to an array of its own and
+    leave that shared Var a plain constant: a later `w * 2.0` does not depend on x (its gradient w.r.t. x is the
+    zeros of an untouched target), and the constant stays a by-value scalar without a producing op."""
+    import jittor_amd as jt
+    from jittor_amd import core
+    x = jt.array(np.ones(3, np.float32))
+    w = jt.array(np.ones(3, np.float32))
+    shared = core._as_var(2.0)
+    x.assign(2.0)
+    assert core._as_var(2.0) is shared and shared._op is None and shared._history is None
+    assert x.shape == [1] and not any(v is x for v in (shared._op.inputs if shared._op else ()))
+    loss = (w * 2.0).sum()
+    g = jt.grad(loss, [x])[0]
+    assert g.shape == x.shape and not isinstance(g._op, (core.ReindexReduceOp, core.ReindexOp))   # zeros, not a gradient path
+    z = jt.array(np.zeros(2, np.float32))
+    z.assign(2.0)
+    assert z._op is None or z._op.inputs == []          # an array of its own, not an alias of x
 
 
 def test_fused_reduce_descriptor_checks_and_specialisation(compile_only):

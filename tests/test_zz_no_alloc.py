@@ -36,6 +36,13 @@ def test_reduce_static_matches_reduce_on_two_calls_in_a_row(gpu):
             L.check(_reduce(lib, lib.mjt_reduce, dx[s], dy_ref, s, [s[0]], "float32", "float32", "add", 0b10))
             assert "split" in L.last_kernel() or "fold" in L.last_kernel(), L.last_kernel()
             refs[s] = L.d2h(dy_ref, [s[0]], np.float32)
+        # what the entry point exists for: between here and the end of its calls no kernel is built or loaded and
+        # no device memory is taken (the free memory the runtime reports stays what it was)
+        hip = ctypes.CDLL("libamdhip64.so")
+        free0, free1, total = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+        L.sync()
+        assert hip.hipMemGetInfo(ctypes.byref(free0), ctypes.byref(total)) == 0
+        stats0 = L.jit_stats()
         # two calls in a row of the variant that allocates nothing, the second with the smaller input
         for s in (big, small):
             L.h2d(dy_new, np.full(64, np.nan, np.float32))
@@ -45,6 +52,9 @@ def test_reduce_static_matches_reduce_on_two_calls_in_a_row(gpu):
             assert np.allclose(got, refs[s], rtol=1e-5, atol=0), (s, got, refs[s])
             assert np.array_equal(got, refs[s]), (s, got, refs[s])
             assert np.allclose(got, exact, rtol=1e-5, atol=1e-5 * np.sqrt(s[1])), (s, got, exact)
+        assert L.jit_stats() == stats0, (stats0, L.jit_stats())
+        assert hip.hipMemGetInfo(ctypes.byref(free1), ctypes.byref(total)) == 0
+        assert free1.value == free0.value, (free0.value, free1.value)
     finally:
         for p in list(dx.values()) + [dy_ref, dy_new]:
             L.free(p)
