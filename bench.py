@@ -474,6 +474,33 @@ def wl_callers(L, lib, steps, warmup, with_cpu):
                      "roofline": roofline(bound, flops if bound == "mfma" else nbytes, ms), **LAST_SPREAD, "note": note}
         dev.release()
 
+    # float32 convolutions: the product kernel gathers its operand from x (no column matrices); against the fp32 MFMA peak
+    def conv_f32_case(name, xs, ws, params):
+        dev = Dev(L)
+        N, C, H, W = xs
+        K, _, R, S = ws
+        sh, sw, ph, pw, dh, dw_ = params
+        OH, OW = (H + 2 * ph - dh * (R - 1) - 1) // sh + 1, (W + 2 * pw - dw_ * (S - 1) - 1) // sw + 1
+        ys = (N, K, OH, OW)
+        xf, wf = rng.standard_normal(xs).astype(np.float32), (rng.standard_normal(ws) * 0.05).astype(np.float32)
+        p = L.ConvParams(*params)
+        calls = []
+        for s in range(3):
+            tx, tw = L.tensor(dev.put(xf), "float32", xs), L.tensor(dev.put(wf), "float32", ws)
+            ty = L.tensor(dev.empty(int(np.prod(ys)) * 4), "float32", ys)
+            calls.append(lambda tx=tx, tw=tw, ty=ty: L.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p))))
+        ms, wall = time_calls(L, calls, steps, warmup)
+        flops = 2.0 * N * K * OH * OW * C * R * S
+        r = roofline("mfma", flops, ms)
+        r["peak"], r["frac"] = 157.3, round(r["achieved"] / 157.3, 4)          # float32 MFMA peak, TFLOP/s
+        out[name] = {"workload": "%s: conv of x fp32 %s, w fp32 %s, stride %d pad %d" % (name, list(xs), list(ws), sh, ph),
+                     "kernel": L.last_kernel(), "dtype": "f32", "ms_per_step": round(wall, 5), "kernel_ms": round(ms, 5),
+                     "roofline": r, **LAST_SPREAD}
+        dev.release()
+
+    conv_f32_case("CONV_F32_3x3", (64, 64, 56, 56), (64, 64, 3, 3), (1, 1, 1, 1, 1, 1))
+    conv_f32_case("CONV_F32_STEM", (64, 3, 224, 224), (64, 3, 7, 7), (2, 2, 3, 3, 1, 1))
+    conv_f32_case("CONV_F32_7x7MAP", (64, 512, 7, 7), (512, 512, 3, 3), (1, 1, 1, 1, 1, 1))
     conv_case("CONV1x1", "fwd", (64, 512, 28, 28), (128, 512, 1, 1), (1, 1, 0, 0, 1, 1), "hbm", "on the matrix-product kernel; bytes = x + w + y once")
     conv_case("CONV1x1_UP", "fwd", (64, 64, 56, 56), (256, 64, 1, 1), (1, 1, 0, 0, 1, 1), "hbm", "on the matrix-product kernel; bytes = x + w + y once")
     conv_case("DGRAD_S2", "dgrad", (64, 256, 56, 56), (256, 256, 3, 3), (2, 2, 1, 1, 1, 1), "mfma", "one convolution per stride phase, then the interleave")

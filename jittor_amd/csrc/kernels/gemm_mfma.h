@@ -28,6 +28,14 @@
 // four MFMAs (lanes 32..63 read the next chunk, so that an MFMA sums k and k + 4 of a
 // chunk pair; any pairing is right as long as both operands use the same one).
 //
+// CONV = 1 (float32 only) makes the kernel an implicit-GEMM convolution, the meta-op group of
+// python/jittor/nn.py:1251-1262 that opt/tuner/conv_tuner.cc:233-240,365-373 relays for every float type:
+// A = the weights [K_][C_*R_*S_] (rows padded to 16 bytes by the host), B'[k = (c, r, s)][j = (image, oh, ow)] =
+// x[image][c][oh*SH-PH+r*DH][ow*SW-PW+s*DW] (0 outside the image) is never written to memory -- the B tile of a
+// stage is gathered from x element by element on its way to LDS (a float32 MFMA runs at a sixteenth of the 16-bit
+// rate, so the gather's address arithmetic hides behind it) -- and C[k][j] is stored as y[image][k][oh][ow].
+// Geometry comes as C_, H_, W_, K_, R_, S_, OH_, OW_, SH, SW, PH, PW, DH, DW; N = images * OH_ * OW_.
+//
 // Rows of A' and columns of B' beyond M and N are read from the last valid row (their
 // results are not stored); k beyond K is zeroed in both operands.  Leading dimensions are
 // multiples of 16 bytes and the operand pointers 16-byte aligned (the host sends
@@ -46,6 +54,9 @@ typedef unsigned short TIN;
 #define TN (64 * NI)
 #define ROWB 144                 // bytes per LDS row: 8 chunks + 1 of padding
 #define NTHR 256
+#ifndef CONV
+#define CONV 0
+#endif
 #ifndef NBUF
 #define NBUF 2                   // staging buffers: 2, or 1 for a product of a single stage (K <= KS)
 #endif
@@ -202,6 +213,68 @@ template <int ROWS, bool KCONT> struct mjt_stager {
     }
 };
 
+#if CONV
+// The B tile of a stage of the implicit-GEMM convolution.  Same blocks as mjt_stager<TN, false>: 4 lanes hold 4
+// k-rows x 4 columns, lane tid % 4 the k-row.  What depends on a column alone (its image and pixel) is worked out once
+// per workgroup (mjt_conv_cols): base = element offset of x[image][0][oh*SH-PH][ow*SW-PW], hw = that row and column,
+// both biased by 0x4000, in one word (0 for a column past N: every tap of it then fails the range check).
+struct mjt_conv_cols {
+    static constexpr int PER = TN * KC / NTHR;
+    int base[PER][4];
+    unsigned hw[PER][4];
+    // (compile-time loop indices throughout: with run-time ones the compiler keeps these arrays in scratch memory
+    // once the loops are too long for it to unroll them itself)
+    __device__ __forceinline__ void init(int n0, int N, int tid) {
+        mjt_static_for<0, PER * 4>([&](auto ic) {
+            constexpr int i = decltype(ic)::v / 4, e = decltype(ic)::v % 4;
+            const int b = tid / 4 + i * (NTHR / 4);
+            const int j = n0 + (b % (TN / 4)) * 4 + e;
+            const int img = j / (OH_ * OW_), px = j - img * (OH_ * OW_);
+            const int oh = px / OW_, ow = px - oh * OW_;
+            const int ih = oh * SH - PH, iw = ow * SW - PW;
+            base[i][e] = j < N ? (img * C_ * H_ + ih) * W_ + iw : 0;
+            hw[i][e] = j < N ? ((unsigned)(ih + 0x4000) << 16) | (unsigned)(iw + 0x4000) : 0u;
+        });
+    }
+};
+struct mjt_conv_stager {
+    static constexpr int PER = TN * KC / NTHR;
+    static constexpr int RS = R_ * S_, CRS = C_ * R_ * S_;
+    mjt_u32x4v reg[PER];
+
+    __device__ __forceinline__ void fetch(const float* __restrict__ x, const mjt_conv_cols& cols, int k0, int tid) {
+        mjt_static_for<0, PER>([&](auto ic) {
+            constexpr int i = decltype(ic)::v;
+            const int b = tid / 4 + i * (NTHR / 4);
+            const int k = k0 + (b / (TN / 4)) * 4 + tid % 4;
+            const bool kvalid = k < CRS;
+            const int kk = kvalid ? k : 0;
+            const int c = kk / RS, rs = kk - c * RS;
+            const int r = rs / S_, t = rs - r * S_;
+            const int koff = (c * H_ + r * DH) * W_ + t * DW;
+            const unsigned dhw = ((unsigned)(r * DH) << 16) | (unsigned)(t * DW);
+            mjt_static_for<0, 4>([&](auto ec) {
+                constexpr int e = decltype(ec)::v;
+                const unsigned q = cols.hw[i][e] + dhw;
+                const bool ok = kvalid && (q >> 16) - 0x4000u < (unsigned)H_ && (q & 0xffffu) - 0x4000u < (unsigned)W_;
+                // an unconditional load from a valid address, zeroed afterwards: a load under a condition is a branch per
+                // element
+                const unsigned v = __float_as_uint(x[ok ? cols.base[i][e] + koff : 0]);
+                reg[i][e] = ok ? v : 0u;
+            });
+        });
+    }
+    __device__ __forceinline__ void commit(unsigned char* lds, int tid) const {
+        mjt_static_for<0, PER>([&](auto ic) {
+            constexpr int i = decltype(ic)::v;
+            const int b = tid / 4 + i * (NTHR / 4);
+            const int row = (b % (TN / 4)) * 4 + tid % 4, kc = b / (TN / 4);
+            *(mjt_u32x4v*)(lds + row * ROWB + kc * 16) = mjt_transpose4x4_b32(reg[i], tid);
+        });
+    }
+};
+#endif
+
 extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const int M = (int)(long long)p.a[3], N = (int)(long long)p.a[4], K = (int)(long long)p.a[5];
     const long long lda = (long long)p.a[6], ldb = (long long)p.a[7], ldc = (long long)p.a[8];
@@ -233,11 +306,43 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
 
-    mjt_stager<TM, A_KCONT> sa;
-    mjt_stager<TN, B_KCONT> sb;
+    // The operand tiles of a stage are asked for NSET stages ahead: one stage of 16-bit MFMAs on tiles up to 128 x 128
+    // is shorter than a trip to memory, so those keep two stages in registers (2048^3 bfloat16: 31.7 -> 30.6 us; tiles
+    // of 64 x 64: 40.8 -> 38.6 us).  Larger tiles have no registers to spare, and float32 stages are long enough (two
+    // sets: 153 -> 159 us for 2048^3).
+    constexpr int NSET = (NBUF > 1 && MI * NI <= 4 && IN != 2 && !CONV) ? 2 : 1;
+    const int nstages = NBUF == 1 ? 1 : (K + KS - 1) / KS;
+    mjt_stager<TM, A_KCONT> sa[NSET];
     const int arows = M, brows = N;
-    sa.fetch(A, lda, m0, arows, 0, K, tid);
-    sb.fetch(B, ldb, n0, brows, 0, K, tid);
+#if CONV
+    mjt_conv_cols cols;
+    cols.init(n0, N, tid);
+    mjt_conv_stager sb[NSET];
+#else
+    mjt_stager<TN, B_KCONT> sb[NSET];
+#endif
+    auto fetch = [&](auto setc, int stage) {
+        constexpr int SET = decltype(setc)::v;
+        sa[SET].fetch(A, lda, m0, arows, stage * KS, K, tid);
+#if CONV
+        sb[SET].fetch(B, cols, stage * KS, tid);
+#else
+        sb[SET].fetch(B, ldb, n0, brows, stage * KS, K, tid);
+#endif
+    };
+    auto commit = [&](auto setc, int stage) {
+        constexpr int SET = decltype(setc)::v;
+        unsigned char* buf = &lds[stage & (NBUF - 1)][0];
+        sa[SET].commit(buf, stage * KS, K, tid);
+#if CONV
+        sb[SET].commit(buf + TM * ROWB, tid);
+#else
+        sb[SET].commit(buf + TM * ROWB, stage * KS, K, tid);
+#endif
+    };
+    mjt_static_for<0, NSET>([&](auto tc) {
+        if (decltype(tc)::v < nstages) fetch(tc, decltype(tc)::v);
+    });
 
     mjt_f32x16 acc[MI][NI];
 #pragma unroll
@@ -247,20 +352,18 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    sa.commit(&lds[0][0], 0, K, tid);
-    sb.commit(&lds[0][TM * ROWB], 0, K, tid);
+    commit(mjt_ic<0>(), 0);
     __syncthreads();
 
     // fragment addresses of this lane: row lane % 32 of its wave's tile rows, chunk lane / 32
     const int frow = lane & 31, fhalf = lane >> 5;
-    const int nstages = NBUF == 1 ? 1 : (K + KS - 1) / KS;
-    for (int s = 0; s < nstages; s++) {
+    // stage s: its tiles sit in LDS buffer s % NBUF; the registers of set s % NSET are free (committed before the
+    // stage began) and take stage s + NSET; at the end stage s + 1 goes from set (s + 1) % NSET to the other buffer
+    auto run_stage = [&](auto parc, const int s) {
+        constexpr int PAR = decltype(parc)::v;
         const unsigned char* la = &lds[s & (NBUF - 1)][0] + (wm * 32 * MI + frow) * ROWB + fhalf * 16;
         const unsigned char* lb = &lds[s & (NBUF - 1)][TM * ROWB] + (wn * 32 * NI + frow) * ROWB + fhalf * 16;
-        if (s + 1 < nstages) {
-            sa.fetch(A, lda, m0, arows, (s + 1) * KS, K, tid);
-            sb.fetch(B, ldb, n0, brows, (s + 1) * KS, K, tid);
-        }
+        if (s + NSET < nstages) fetch(parc, s + NSET);
         // a pair of chunks per step; the fragments of the next step are requested before the MFMAs of this one
         mjt_u32x4v fa[2][MI], fb[2][NI];
         const unsigned la_addr = (unsigned)(unsigned long long)(__attribute__((address_space(3))) const unsigned char*)la;
@@ -294,11 +397,14 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
 #endif
         });
         if (s + 1 < nstages) {
-            sa.commit(&lds[(s + 1) & (NBUF - 1)][0], (s + 1) * KS, K, tid);             // the other buffer: nobody reads it now
-            sb.commit(&lds[(s + 1) & (NBUF - 1)][TM * ROWB], (s + 1) * KS, K, tid);
+            commit(mjt_ic<(PAR + 1) % NSET>(), s + 1);           // the other buffer: nobody reads it now
             __syncthreads();
         }
-    }
+    };
+    for (int s0 = 0; s0 < nstages; s0 += NSET)
+        mjt_static_for<0, NSET>([&](auto parc) {
+            if (s0 + decltype(parc)::v < nstages) run_stage(parc, s0 + decltype(parc)::v);
+        });
 
     // D of a 32x32 tile: lane holds column lane % 32, rows 8 * (e / 4) + 4 * (lane / 32) + e % 4
 #if OUT == 2
@@ -311,12 +417,17 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
 #pragma unroll
         for (int j = 0; j < NI; j++) {
             const int col = n0 + wn * 32 * NI + j * 32 + (lane & 31);
+#if CONV
+            const int img = col / (OH_ * OW_), px = col - img * (OH_ * OW_);      // y[img][row][px]
+#endif
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int row = m0 + wm * 32 * MI + i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e & 3);
                 if (row < M && col < N) {
                     const float v = acc[i][j][e];
-#if OUT == 2
+#if CONV
+                    C[((long long)img * K_ + row) * (OH_ * OW_) + px] = v;
+#elif OUT == 2
                     C[(long long)row * ldc + col] = v;
 #elif OUT == 0
                     C[(long long)row * ldc + col] = (unsigned short)(__float_as_uint(v) >> 16);     // truncation (type/fp16_compute.h:238-241)

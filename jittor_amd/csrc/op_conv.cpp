@@ -284,13 +284,6 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int64_t esz = dtype_size(x->dtype);
         const int64_t Ppad = (P * esz + 15) / 16 * 16 / esz;
         const bool plain = R == 1 && S == 1 && p->stride_h == 1 && p->stride_w == 1 && p->pad_h == 0 && p->pad_w == 0 && Ppad == P && OH == H && OW == W;
-        int64_t chunk = (int64_t(1) << 30) / (CRS * Ppad * esz);
-        if (const char* e = getenv("MJT_CONV_GEMM_CHUNK"))      // images per chunk, for tests of the chunk loop
-            if (atoi(e) >= 1) chunk = atoi(e);
-        if (chunk < 1) chunk = 1;
-        if (chunk > N) chunk = N;
-        if (chunk > 65535) chunk = 65535;                       // the images of a chunk are the batch of one product launch
-        void* cols = plain ? nullptr : conv_scratch(0, (size_t)(chunk * CRS * Ppad * esz));
         auto view = [](void* ptr, int dtype, std::initializer_list<int64_t> shape) {
             mjt_tensor t;
             memset(&t, 0, sizeof(t));
@@ -299,6 +292,65 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             for (int64_t e : shape) t.shape[t.ndim++] = e;
             return t;
         };
+        // The product's MFMA kernel wants operand rows that are 16-byte multiples at 16-byte aligned addresses.  Weight
+        // rows that are not (3 x 7 x 7 float32 taps: 588 bytes) are copied into rows padded with zeros once per call.
+        const void* wmat = w->ptr;
+        int64_t lda = CRS;
+        if ((CRS * esz) % 16 || (uintptr_t)w->ptr % 16) {
+            lda = (CRS * esz + 15) / 16 * 16 / esz;
+            void* wpad = conv_scratch(4, (size_t)(K * lda * esz));
+            mjt_tensor tw = view(w->ptr, w->dtype, {K, CRS}), tp = view(wpad, w->dtype, {K, lda});
+            const char* widx[2] = {"i0", "i1"};                 // columns past CRS lie outside w: overflow value 0
+            if (mjt_reindex(&tw, &tp, 2, widx, 0.0, 0, nullptr, 0, nullptr) != MJT_OK)
+                MJT_FAIL(MJT_ERR_DEVICE, "conv: padding the weight rows failed: " << mjt_last_error());
+            wmat = wpad;
+        }
+        // float32: the product kernel gathers its second operand from x on the fly (kernels/gemm_mfma.h with CONV): no
+        // column matrices.  Offsets inside x and y and the column number are 32-bit there, rows and columns of the
+        // image and the reach of the taps 14-bit.
+        if (!plain && x->dtype == MJT_FLOAT32 && y->dtype == MJT_FLOAT32 && !getenv("MJT_CONV_NO_IGEMM") &&
+            numel(x) < (int64_t(1) << 31) && numel(y) < (int64_t(1) << 31) && H < 16384 && W < 16384 &&
+            (R - 1) * p->dil_h < 16384 && (S - 1) * p->dil_w < 16384 && p->pad_h < 16384 && p->pad_w < 16384 &&
+            OH * p->stride_h < 16384 && OW * p->stride_w < 16384) {
+            const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
+            const int64_t NP = N * P;
+            // Tile: 64 output channels x 64 pixels, or 128 x 128 when there are more than 64 output channels and enough
+            // tiles of that size for every compute unit.  Measured (us, tiles 64x64 / 64x128 / 128x64 / 128x128):
+            // 64x64x56x56 3x3 -> 64: 202 / 244 / 381 / 365; 64x3x224x224 7x7 stride 2 -> 64: 228 / 254 / 426 / 379;
+            // 64x128x28x28 3x3 -> 128: 208 / 246 / 214 / 192; 64x512x7x7 3x3 -> 512: 272 / 335 / 273 / 469.  Small tiles
+            // win because four workgroups then share a compute unit: the gather's address arithmetic of one overlaps the
+            // MFMAs of another.
+            const bool big = K > 64 && ((K + 127) / 128) * ((NP + 127) / 128) >= cus;
+            const int MI = big ? 2 : 1, NI = big ? 2 : 1;
+            std::ostringstream key;
+            key << "igemm|" << geo.str() << MI << NI;
+            JitKernel* k = cached(key.str());
+            if (!k) {
+                std::ostringstream name;
+                name << "mjt_conv_igemm_float32_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s" << p->stride_h << "x"
+                     << p->stride_w << "_p" << p->pad_h << "x" << p->pad_w << "_d" << p->dil_h << "x" << p->dil_w << "_" << 64 * MI << "x" << 64 * NI;
+                std::ostringstream src;
+                src << "#define ENTRY " << name.str() << "\n#define CONV 1\n#define IN 2\n#define OUT 2\n#define MI " << MI << "\n#define NI " << NI
+                    << "\n#define A_KCONT 1\n#define B_KCONT 0\n" << geo.str();
+                src << embedded_source("gemm_mfma.h") << "\n";
+                k = jit_get(src.str(), name.str());
+                remember(key.str(), k);
+            }
+            const int64_t tiles = ((K + 64 * MI - 1) / (64 * MI)) * ((NP + 64 * NI - 1) / (64 * NI));
+            const int64_t grid = (tiles + 7) / 8 * 8;
+            MJT_CHECK(grid < (int64_t(1) << 31), "conv: launch too large");
+            std::vector<uint64_t> a{bits_of_ptr(wmat), bits_of_ptr(x->ptr), bits_of_ptr(y->ptr), (uint64_t)K, (uint64_t)NP, (uint64_t)CRS,
+                                    (uint64_t)lda, 0, 0, 0, 0, 0};
+            jit_launch(k, (unsigned)grid, 1, 256, 0, a);
+            return;
+        }
+        int64_t chunk = (int64_t(1) << 30) / (CRS * Ppad * esz);
+        if (const char* e = getenv("MJT_CONV_GEMM_CHUNK"))      // images per chunk, for tests of the chunk loop
+            if (atoi(e) >= 1) chunk = atoi(e);
+        if (chunk < 1) chunk = 1;
+        if (chunk > N) chunk = N;
+        if (chunk > 65535) chunk = 65535;                       // the images of a chunk are the batch of one product launch
+        void* cols = plain ? nullptr : conv_scratch(0, (size_t)(chunk * CRS * Ppad * esz));
         // index strings of the column matrices: [n, c, kh, kw, oh, ow] when a row needs no padding (the window
         // pattern of the reindex fast path), else [n, c, kh, kw, pixel] with the pixel split by division and
         // remainder and the padding marked as overflow
@@ -313,19 +365,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         }
         const char* idx[4] = {"i0", "i1", sh.c_str(), sw.c_str()};
         const char* ovc[1] = {over.c_str()};
-        // The product's MFMA kernel wants operand rows that are 16-byte multiples at 16-byte aligned addresses.  Weight
-        // rows that are not (3 x 7 x 7 float32 taps: 588 bytes) are copied into rows padded with zeros once per call.
-        const void* wmat = w->ptr;
-        int64_t lda = CRS;
-        if ((CRS * esz) % 16 || (uintptr_t)w->ptr % 16) {
-            lda = (CRS * esz + 15) / 16 * 16 / esz;
-            void* wpad = conv_scratch(4, (size_t)(K * lda * esz));
-            mjt_tensor tw = view(w->ptr, w->dtype, {K, CRS}), tp = view(wpad, w->dtype, {K, lda});
-            const char* widx[2] = {"i0", "i1"};                 // columns past CRS lie outside w: overflow value 0
-            if (mjt_reindex(&tw, &tp, 2, widx, 0.0, 0, nullptr, 0, nullptr) != MJT_OK)
-                MJT_FAIL(MJT_ERR_DEVICE, "conv: padding the weight rows failed: " << mjt_last_error());
-            wmat = wpad;
-        }
+
         for (int64_t n0 = 0; n0 < N; n0 += chunk) {
             const int64_t nb = N - n0 < chunk ? N - n0 : chunk;
             char* xn = (char*)x->ptr + n0 * C * H * W * esz;

@@ -921,6 +921,11 @@ def test_conv_direct_small_shapes_and_fp32(gpu):
     dict(dt="bfloat16", x=(3, 72, 9, 11), w=(40, 72, 3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16"),
     dict(dt="float32", x=(5, 40, 16, 16), w=(96, 40, 1, 1), p=(1, 1, 0, 0, 1, 1), plain=True, chunk=2),
     dict(dt="float32", x=(8, 3, 64, 64), w=(32, 3, 7, 7), p=(2, 2, 3, 3, 1, 1)),      # a stem: weight rows of 588 bytes are padded to 16-byte multiples
+    dict(dt="float32", x=(8, 3, 64, 64), w=(32, 3, 7, 7), p=(2, 2, 3, 3, 1, 1), cols=True),      # the same through column matrices
+    dict(dt="float32", x=(4, 32, 28, 28), w=(48, 32, 3, 3), p=(1, 1, 1, 1, 1, 1), cols=True),
+    dict(dt="float32", x=(3, 80, 19, 23), w=(136, 80, 3, 3), p=(1, 2, 2, 0, 2, 1)),                 # 136 output channels: two row tiles, the second mostly empty; mixed strides
+    dict(dt="float32", x=(70, 16, 7, 7), w=(24, 16, 3, 3), p=(1, 1, 1, 1, 1, 1)),                    # 7 x 7 maps: a tile of pixels spans several images
+    dict(dt="float32", x=(2, 8, 40, 130), w=(16, 8, 1, 5), p=(1, 1, 0, 2, 1, 1)),                    # wide rows, taps along the row only
     # the product on the direct-copy kernel (asked for by name: these shapes have too few tiles to get it by themselves):
     # weights shared across the batch, column matrices with the pixels innermost read with transposing reads
     dict(dt="bfloat16", x=(3, 64, 15, 15), w=(96, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), dma=True),
@@ -941,8 +946,13 @@ def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
         monkeypatch.setenv("MJT_CONV_GEMM_CHUNK", str(case["chunk"]))
     if case.get("dma"):
         monkeypatch.setenv("MJT_GEMM_DMA", "1")
+    if case.get("cols"):
+        monkeypatch.setenv("MJT_CONV_NO_IGEMM", "1")
     got, kern = _conv_call(xb, wb, case["p"], out_dtype=out, in_dtype=dt)
-    assert kern == ("conv_as_gemm" if case.get("plain") else "conv_as_reindex_gemm"), kern
+    if dt == "float32" and not case.get("plain") and not case.get("cols"):
+        assert kern.startswith("mjt_conv_igemm_float32"), kern      # float32: the product gathers its operand from x itself
+    else:
+        assert kern == ("conv_as_gemm" if case.get("plain") else "conv_as_reindex_gemm"), kern
     got = widen[out](got)
     xf, wf = widen[dt](xb).astype(np.float64), widen[dt](wb).astype(np.float64)
     K, _, R, S = wf.shape
