@@ -98,6 +98,34 @@ def pool(x, kernel_size, op, padding=0, stride=None):
     return core.reduce(xx, op, [4, 5])
 
 
+def concat(arr, dim=0):
+    """jt.concat (python/jittor/contrib.py:22-58): every part is reindexed into the result's shape at its offset
+    along `dim` (0 elsewhere) and the parts are added."""
+    arr = [core._as_var(a) for a in arr]
+    if not arr:
+        raise ValueError("concat: empty list")
+    nd = arr[0].ndim
+    if dim < 0:
+        dim += nd
+    if not 0 <= dim < nd:
+        raise ValueError("concat: dim %d out of range for rank %d" % (dim, nd))
+    total = sum(a.shape[dim] for a in arr)
+    indexes = ["i%d" % i for i in range(nd)]
+    out, at = None, 0
+    for a in arr:
+        if a.ndim != nd or any(a.shape[i] != arr[0].shape[i] for i in range(nd) if i != dim):
+            raise ValueError("concat: shapes %s and %s differ outside dim %d" % (list(arr[0].shape), list(a.shape), dim))
+        shape = list(a.shape)
+        shape[dim] = total
+        indexes[dim] = "i%d-%d" % (dim, at)
+        b = a.reindex(shape, list(indexes))
+        if len(arr) >= 100:
+            b.stop_fuse()
+        out = b if out is None else out + b
+        at += a.shape[dim]
+    return out
+
+
 def permute(x, *dims):
     if len(dims) == 1 and isinstance(dims[0], (list, tuple)):
         dims = tuple(dims[0])

@@ -69,6 +69,84 @@ def conv2d(x, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
     return y
 
 
+def conv_transpose(x, weight, bias=None, stride=1, padding=0, output_padding=0, groups=1, dilation=1):
+    """The transposed convolution as python/jittor/nn.py:1535-1577 writes it (groups == 1): x [N, i, H, W] and
+    weight [i, o, h, w] broadcast into [N, i, o, H, W, h, w], multiplied, and scattered with reindex_reduce.add
+    into [N, o, h_out, w_out].  That graph is the input gradient of the convolution whose output x would be
+    (conv_tuner.cc:375-397 relays it to the library's backward-data call); the executor recognises it the same
+    way and runs it on the convolution kernels."""
+    if groups != 1:
+        raise NotImplementedError("conv_transpose: groups > 1")
+    if x.ndim != 4:
+        raise RuntimeError("Expected 4D input to conv_transpose, but got input of size: %s" % list(x.shape))
+    stride, padding, dilation, output_padding = _pair(stride), _pair(padding), _pair(dilation), _pair(output_padding)
+    N, C, H, W = x.shape
+    i, o, h, w = weight.shape
+    assert C == i, (C, i)
+    if stride[0] <= 0 or stride[1] <= 0:
+        raise RuntimeError("non-positive stride is not supported")
+    assert output_padding[0] < max(stride[0], dilation[0]) and output_padding[1] < max(stride[1], dilation[1]), \
+        "output padding must be smaller than max(stride, dilation)"
+    h_out = (H - 1) * stride[0] + output_padding[0] - 2 * padding[0] + 1 + (h - 1) * dilation[0]
+    w_out = (W - 1) * stride[1] + output_padding[1] - 2 * padding[1] + 1 + (w - 1) * dilation[1]
+    shape = [N, i, o, H, W, h, w]
+    with flag_scope(amp_reg=flags.amp_reg | 36):
+        xx = x.broadcast(shape, [2, 5, 6])
+        ww = weight.broadcast(shape, [0, 3, 4])
+        y = (ww * xx).reindex_reduce("add", [N, o, h_out, w_out], [
+            "i0",
+            "i2",
+            "i3*%d-%d+i5*%d" % (stride[0], padding[0], dilation[0]),
+            "i4*%d-%d+i6*%d" % (stride[1], padding[1], dilation[1]),
+        ])
+    if bias is not None:
+        y = y + bias.broadcast(y.shape, [0, 2, 3])
+    return y
+
+
+conv_transpose2d = conv_transpose
+
+
+def unfold(x, kernel_size, dilation=1, padding=0, stride=1):
+    """Sliding windows as columns, [n, c, h, w] -> [n, c * kh * kw, blocks] (python/jittor/nn.py:2450-2477): a
+    padding reindex, then one reindex whose index expressions divide and take remainders."""
+    assert x.ndim == 4
+    kernel_size, dilation, padding, stride = _pair(kernel_size), _pair(dilation), _pair(padding), _pair(stride)
+    assert kernel_size[0] > 0 and kernel_size[1] > 0, "kernel size must be positive"
+    assert dilation[0] > 0 and dilation[1] > 0, "dilation must be positive"
+    assert padding[0] >= 0 and padding[1] >= 0, "padding must be non-negative"
+    assert stride[0] > 0 and stride[1] > 0, "stride must be positive"
+    n, c, h, w = x.shape
+    area = kernel_size[0] * kernel_size[1]
+    blocks = [(x.shape[i] + 2 * padding[i - 2] - dilation[i - 2] * (kernel_size[i - 2] - 1) - 1) // stride[i - 2] + 1 for i in (2, 3)]
+    if padding[0] != 0 or padding[1] != 0:
+        x = x.reindex([n, c, h + padding[0] * 2, w + padding[1] * 2], ["i0", "i1", "i2-%d" % padding[0], "i3-%d" % padding[1]])
+    return x.reindex([n, c * area, blocks[0] * blocks[1]], [
+        "i0", "i1/%d" % area,
+        "i2/%d*%d+(i1%%%d)/%d*%d" % (blocks[1], stride[0], area, kernel_size[1], dilation[0]),
+        "i2%%%d*%d+(i1%%%d)%%%d*%d" % (blocks[1], stride[1], area, kernel_size[1], dilation[1])])
+
+
+def fold(x, output_size, kernel_size, dilation=1, padding=0, stride=1):
+    """Columns summed back into an image, [n, c * kh * kw, blocks] -> [n, c, H, W] (python/jittor/nn.py:2480-2501):
+    one reindex_reduce.add with unfold's index expressions, then the crop of the padding."""
+    assert x.ndim == 3
+    assert output_size[0] > 0 and output_size[1] > 0, "output size must be positive."
+    kernel_size, dilation, padding, stride = _pair(kernel_size), _pair(dilation), _pair(padding), _pair(stride)
+    assert kernel_size[0] > 0 and kernel_size[1] > 0, "kernel size must be positive"
+    assert dilation[0] > 0 and dilation[1] > 0, "dilation must be positive"
+    assert padding[0] >= 0 and padding[1] >= 0, "padding must be non-negative"
+    assert stride[0] > 0 and stride[1] > 0, "stride must be positive"
+    n, cl, num = x.shape
+    area = kernel_size[0] * kernel_size[1]
+    blocks = [(output_size[i] + 2 * padding[i] - dilation[i] * (kernel_size[i] - 1) - 1) // stride[i] + 1 for i in (0, 1)]
+    out = x.reindex_reduce("add", [n, cl // area, output_size[0] + 2 * padding[0], output_size[1] + 2 * padding[1]], [
+        "i0", "i1/%d" % area,
+        "i2/%d*%d+(i1%%%d)/%d*%d" % (blocks[1], stride[0], area, kernel_size[1], dilation[0]),
+        "i2%%%d*%d+(i1%%%d)%%%d*%d" % (blocks[1], stride[1], area, kernel_size[1], dilation[1])])
+    return out[:, :, padding[0]:padding[0] + output_size[0], padding[1]:padding[1] + output_size[1]]
+
+
 def pad(x, padding, mode="constant", value=0):
     from .misc import pad as _pad
     return _pad(x, padding, mode, value)

@@ -324,3 +324,78 @@ def test_setitem_and_assign(gpu):
     assert np.array_equal(p.data, a[::-1] * 2) and np.array_equal(s_old.data, a + 1)
     with pytest.raises(IndexError):
         jt.array(a)[jt.array(a > 0)]
+
+
+def _conv_transpose_ref(x, w, stride, padding, output_padding, dilation):
+    """Direct statement of the scatter python/jittor/nn.py:1556-1568 builds, in float64."""
+    N, C, H, W = x.shape
+    _, O_, kh, kw = w.shape
+    ho = (H - 1) * stride + output_padding - 2 * padding + 1 + (kh - 1) * dilation
+    wo = (W - 1) * stride + output_padding - 2 * padding + 1 + (kw - 1) * dilation
+    full = np.zeros((N, O_, ho + 2 * padding + stride, wo + 2 * padding + stride))
+    for r in range(kh):
+        for s in range(kw):
+            contrib = np.einsum("nihw,io->nohw", x.astype(np.float64), w[:, :, r, s].astype(np.float64))
+            full[:, :, r * dilation:r * dilation + (H - 1) * stride + 1:stride, s * dilation:s * dilation + (W - 1) * stride + 1:stride] += contrib
+    return full[:, :, padding:padding + ho, padding:padding + wo]
+
+
+def test_conv_transpose_runs_as_the_input_gradient_pattern(gpu):
+    """nn.conv_transpose builds the reference's graph (broadcast x, broadcast w, multiply, reindex_reduce.add); the
+    executor takes it for the backward-data pattern and runs it on the convolution kernels: float32 (through the
+    product kernel) and bfloat16 (MFMA convolution kernel, one convolution per stride phase), with bias."""
+    rng = np.random.default_rng(61)
+    for dt, xs, ws, st, pd, op, dl, tol in (("float32", (2, 8, 5, 7), (8, 6, 3, 3), 2, 1, 1, 1, 1e-4),
+                                            ("float32", (3, 16, 9, 9), (16, 12, 3, 2), 1, 0, 0, 2, 1e-4),
+                                            # bfloat16: the sum and the sum plus bias are each truncated to 8 bits
+                                            ("bfloat16", (2, 64, 14, 14), (64, 64, 3, 3), 2, 1, 1, 1, 2.0 ** -6),
+                                            ("bfloat16", (2, 64, 12, 16), (64, 128, 3, 3), 1, 1, 0, 1, 2.0 ** -6)):
+        x = rng.standard_normal(xs).astype(np.float32)
+        w = (rng.standard_normal(ws) * 0.1).astype(np.float32)
+        b = rng.standard_normal(ws[1]).astype(np.float32)
+        if dt == "bfloat16":
+            x, w, b = (O.BF16(O.f32_to_bf16_bits(v)).to_f32() for v in (x, w, b))
+        jx, jw, jb = jt.array(x), jt.array(w), jt.array(b)
+        if dt == "bfloat16":
+            jx, jw, jb = jx.bfloat16(), jw.bfloat16(), jb.bfloat16()
+        before = jt.executor_stats["conv_matches"]
+        y = jt.nn.conv_transpose(jx, jw, jb, stride=st, padding=pd, output_padding=op, dilation=dl)
+        assert y.dtype == dt
+        got = y.numpy().astype(np.float32)
+        assert jt.executor_stats["conv_matches"] == before + 1, "not taken for the backward-data pattern"
+        ref = _conv_transpose_ref(x, w, st, pd, op, dl) + b[None, :, None, None]
+        assert got.shape == ref.shape and np.abs(got - ref).max() <= tol * np.abs(ref).max(), (dt, xs)
+
+
+def test_concat_unfold_fold(gpu):
+    rng = np.random.default_rng(62)
+    parts = [rng.standard_normal((3, n, 5)).astype(np.float32) for n in (2, 4, 1)]
+    assert np.array_equal(jt.concat([jt.array(p) for p in parts], 1).data, np.concatenate(parts, 1))
+    assert np.array_equal(jt.concat([jt.array(p) for p in parts], -2).data, np.concatenate(parts, 1))
+    assert jt.concat([jt.array([[1], [2]]), jt.array([[2], [2]])], dim=1).data.tolist() == [[1, 2], [2, 2]]    # contrib.py:33-35
+    with pytest.raises(ValueError):
+        jt.concat([jt.array(parts[0]), jt.array(parts[1])], 0)
+    # unfold against windows cut with numpy; fold(unfold(x)) counts how many windows cover each element
+    x = rng.standard_normal((2, 3, 9, 8)).astype(np.float32)
+    for k, d, p, s in ((3, 1, 1, 2), ((2, 3), (2, 1), (0, 1), (1, 2))):
+        kh, kw = (k, k) if isinstance(k, int) else k
+        dh, dw = (d, d) if isinstance(d, int) else d
+        ph, pw = (p, p) if isinstance(p, int) else p
+        sh, sw = (s, s) if isinstance(s, int) else s
+        u = jt.nn.unfold(jt.array(x), k, d, p, s)
+        xp = np.pad(x, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+        bh = (x.shape[2] + 2 * ph - dh * (kh - 1) - 1) // sh + 1
+        bw = (x.shape[3] + 2 * pw - dw * (kw - 1) - 1) // sw + 1
+        want = np.zeros((2, 3 * kh * kw, bh * bw), np.float32)
+        for c in range(3):
+            for r in range(kh):
+                for t in range(kw):
+                    want[:, (c * kh + r) * kw + t] = xp[:, c, r * dh:r * dh + (bh - 1) * sh + 1:sh, t * dw:t * dw + (bw - 1) * sw + 1:sw].reshape(2, -1)
+        assert np.array_equal(u.data, want), (k, d, p, s)
+        back = jt.nn.fold(u, (9, 8), k, d, p, s).data
+        cover = np.zeros_like(xp)
+        for r in range(kh):
+            for t in range(kw):
+                cover[:, :, r * dh:r * dh + (bh - 1) * sh + 1:sh, t * dw:t * dw + (bw - 1) * sw + 1:sw] += 1
+        cover = cover[:, :, ph:ph + 9, pw:pw + 8]
+        assert np.allclose(back, x * cover, rtol=1e-5, atol=1e-6), (k, d, p, s)
