@@ -258,6 +258,18 @@ int mjt_fused_reindex_reduce(const mjt_fused_desc* desc, const mjt_tensor* x, in
                              int n_overflow_conditions, const char* const* overflow_conditions,
                              int n_extras, const mjt_tensor* extras);
 
+/* ---- where ------------------------------------------------------------
+ * The positions of the non-zero elements of `cond` (any dtype; -0.0 is zero,
+ * NaN is not), in row-major order, as one int32 tensor per axis of cond
+ * (python/jittor/src/ops/where_op.cc:20-60; what x[mask] and x[mask] = v with a
+ * boolean mask are built from).  The length of the result depends on the
+ * data: mjt_where_count returns it (one counting pass and a synchronous
+ * 8-byte copy, as the reference's executor fixes the op's uncertain shape once
+ * it has run), the caller allocates cond->ndim tensors int32 [count] and
+ * passes them to mjt_where, which writes at most `count` positions. */
+int mjt_where_count(const mjt_tensor* cond, int64_t* count);
+int mjt_where(const mjt_tensor* cond, int64_t count, const mjt_tensor* outs);
+
 /* ---- meta-op convolution ----------------------------------------------
  * The group reindex + broadcast + multiply + reduce.add that
  * python/jittor/nn.py:1251-1262 builds and opt/tuner/conv_tuner.cc:218-411

@@ -23,14 +23,14 @@ from .grad import grad
 from . import misc
 from . import profiler
 from .profiler import profile_scope
-from .misc import gather, scatter, pad, pool, permute, transpose, reshape, flip, concat
+from .misc import gather, scatter, pad, pool, permute, transpose, reshape, flip, concat, where
 from .nn import matmul
 from .core import no_grad
 
 __all__ = ["Var", "array", "unary", "binary", "ternary", "broadcast", "broadcast_var",
            "reduce", "reindex", "reindex_var", "reindex_reduce", "nn", "sync", "sync_all",
            "fetch_sync", "grad", "no_grad", "gather", "scatter", "pad", "pool", "permute", "transpose", "reshape",
-           "flip", "concat", "matmul", "profile_scope", "MjtError"]
+           "flip", "concat", "where", "matmul", "profile_scope", "MjtError"]
 
 
 def sync(vars, device_sync=False):

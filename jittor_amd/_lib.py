@@ -93,7 +93,7 @@ EXPORTS = ["mjt_init", "mjt_shutdown", "mjt_last_error", "mjt_get_device_info",
            "mjt_event_destroy", "mjt_reduce", "mjt_reduce_static", "mjt_reindex", "mjt_reindex_reduce",
            "mjt_fused_elementwise", "mjt_fused_reduce", "mjt_conv2d_meta", "mjt_conv2d_meta_pack", "mjt_conv2d_meta_packed", "mjt_conv2d_meta_grouped", "mjt_conv2d_meta_dgrad", "mjt_conv2d_meta_wgrad", "mjt_conv2d_meta_wgrad_grouped",
            "mjt_reindex_then_reduce", "mjt_fused_reindex_reduce", "mjt_matmul", "mjt_matmul_available",
-           "mjt_expr_affine",
+           "mjt_expr_affine", "mjt_where_count", "mjt_where",
            "mjt_jit_stats", "mjt_last_kernel"]
 
 _lib = None
@@ -155,6 +155,8 @@ def load():
                                                   ctypes.POINTER(ConvParams), ctypes.c_int]
     lib.mjt_matmul.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.POINTER(Tensor), ctypes.c_int, ctypes.c_int]
     lib.mjt_matmul_available.argtypes = []
+    lib.mjt_where_count.argtypes = [ctypes.POINTER(Tensor), ctypes.POINTER(ctypes.c_int64)]
+    lib.mjt_where.argtypes = [ctypes.POINTER(Tensor), ctypes.c_int64, ctypes.POINTER(Tensor)]
     lib.mjt_expr_affine.argtypes = [ctypes.c_char_p, ctypes.POINTER(Tensor), ctypes.POINTER(Tensor),
                                     ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)]
     lib.mjt_jit_stats.argtypes = [ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)]

@@ -98,6 +98,39 @@ def pool(x, kernel_size, op, padding=0, stride=None):
     return core.reduce(xx, op, [4, 5])
 
 
+def _lib_storage(dtype):
+    from . import _lib
+    return _lib.NP_STORAGE[dtype]
+
+
+def where(cond, x=None, y=None):
+    """jt.where(cond) -> one int32 index Var per axis of cond holding the positions where cond is non-zero, in
+    row-major order (python/jittor/src/ops/where_op.cc:20-60; the result's length depends on the data, so cond is
+    computed here); jt.where(cond, x, y) = ternary(cond, x, y) (:42-45)."""
+    cond = core._as_var(cond)
+    if x is not None or y is not None:
+        if x is None or y is None:
+            raise ValueError("where: give both x and y, or neither")
+        return ternary(cond, x, y)
+    import ctypes
+    from . import _lib
+    cond.sync()
+    lib = _lib.ensure_init()
+    tc = _lib.tensor(cond.raw_ptr(), cond.dtype, cond.shape)
+    count = ctypes.c_int64()
+    _lib.check(lib.mjt_where_count(ctypes.byref(tc), ctypes.byref(count)))
+    n = count.value
+    outs = [array(np.zeros(n, np.int32)) for _ in range(cond.ndim)]
+    if n:
+        to = (_lib.Tensor * cond.ndim)(*[_lib.tensor(o.raw_ptr(), "int32", [n]) for o in outs])
+        _lib.check(lib.mjt_where(ctypes.byref(tc), n, to))
+        for o in outs:
+            o._host = None                              # the device buffer now holds the value
+    for o in outs:
+        o.is_scalar = False                             # an index list of one entry is no fused number
+    return tuple(outs)
+
+
 def concat(arr, dim=0):
     """jt.concat (python/jittor/contrib.py:22-58): every part is reindexed into the result's shape at its offset
     along `dim` (0 elsewhere) and the parts are added."""
@@ -197,22 +230,32 @@ def _parse_key(x, key):
     numpy integer arrays, of any rank) index their axes together: they are broadcast against each other, right
     aligned, into one block of output dims that stands where the first of them stood
     (python/jittor/src/ops/getitem_op.cc:76-113)."""
-    if isinstance(key, Var) and key.dtype == "bool":
-        raise IndexError("a boolean mask selects a data-dependent number of elements: use ternary(mask, a, b)")
     if not isinstance(key, tuple):
         key = (key,)
     key = tuple(array(np.asarray(k)) if isinstance(k, (list, np.ndarray)) else k for k in key)
     if sum(1 for k in key if k is Ellipsis) > 1:
         raise IndexError("an index can only have a single ellipsis")
-    n_real = sum(1 for k in key if k is not None and k is not Ellipsis)
+    # a boolean mask stands for as many axes as it has dims
+    width = lambda k: 0 if k is None or k is Ellipsis else k.ndim if isinstance(k, Var) and k.dtype == "bool" else 1
+    n_real = sum(width(k) for k in key)
     if n_real > x.ndim:
         raise IndexError("too many indices for a Var of rank %d" % x.ndim)
-    full = []
+    full, axis = [], 0
     for k in key:
         if k is Ellipsis:
             full.extend([slice(None)] * (x.ndim - n_real))
+            axis += x.ndim - n_real
+        elif isinstance(k, Var) and k.dtype == "bool":
+            # a boolean mask selects the positions where it is true: the index Vars of where(mask), one per axis it covers
+            # (the result's size depends on the data; python/jittor/src/ops/where_op.cc)
+            if list(k.shape) != list(x.shape[axis:axis + k.ndim]):
+                raise IndexError("boolean mask of shape %s does not match axes %d..%d of shape %s"
+                                 % (list(k.shape), axis, axis + k.ndim - 1, list(x.shape)))
+            full.extend(where(k))
+            axis += k.ndim
         else:
             full.append(k)
+            axis += width(k)
     full.extend([slice(None)] * (x.ndim - sum(1 for k in full if k is not None)))
     index_vars = [k for k in full if isinstance(k, Var)]
     for k in index_vars:
@@ -225,7 +268,7 @@ def _parse_key(x, key):
             have, want = block[var_dim - 1 - j], k.shape[k.ndim - 1 - j]
             if have != want and have != 1 and want != 1:
                 raise IndexError("index Vars of shapes %s do not broadcast" % [list(v.shape) for v in index_vars])
-            block[var_dim - 1 - j] = max(have, want)
+            block[var_dim - 1 - j] = want if have == 1 else have      # (an extent of 0 stays 0: an empty selection)
     out_shape, exprs, extras = [], [], []
     axis = 0
     first_var_dim = -1                                     # output dim where the block starts
@@ -265,6 +308,8 @@ def getitem(x, key):
     out_shape, exprs, extras = _parse_key(x, key)
     if not out_shape:
         out_shape = [1]
+    if 0 in out_shape:                                  # an empty selection (a mask that is false everywhere): nothing to launch
+        return array(np.zeros(out_shape, _lib_storage(x.dtype)), x.dtype)
     return reindex(x, out_shape, exprs, extras=extras)
 
 
@@ -277,6 +322,8 @@ def setitem(x, key, value):
     out_shape, exprs, extras = _parse_key(x, key)
     if not out_shape:
         out_shape = [1]
+    if 0 in out_shape:                                  # nothing selected: x stays as it is
+        return x
     value = core._as_var(value)
     if value.dtype != x.dtype:
         value = value.cast(x.dtype)
@@ -302,3 +349,4 @@ Var.flip = flip
 Var.__getitem__ = getitem
 Var.__setitem__ = lambda self, key, value: (setitem(self, key, value), None)[1]
 Var.setitem = setitem
+Var.where = where

@@ -322,8 +322,7 @@ def test_setitem_and_assign(gpu):
     s_old = p + 1
     p.assign(q * 2)
     assert np.array_equal(p.data, a[::-1] * 2) and np.array_equal(s_old.data, a + 1)
-    with pytest.raises(IndexError):
-        jt.array(a)[jt.array(a > 0)]
+    assert np.array_equal(jt.array(a)[jt.array(a > 0)].data, a[a > 0])      # a boolean mask: where(mask) as index Vars
 
 
 def _conv_transpose_ref(x, w, stride, padding, output_padding, dilation):
@@ -399,3 +398,58 @@ def test_concat_unfold_fold(gpu):
                 cover[:, :, r * dh:r * dh + (bh - 1) * sh + 1:sh, t * dw:t * dw + (bw - 1) * sw + 1:sw] += 1
         cover = cover[:, :, ph:ph + 9, pw:pw + 8]
         assert np.allclose(back, x * cover, rtol=1e-5, atol=1e-6), (k, d, p, s)
+
+
+def test_where_and_boolean_masks(gpu):
+    """jt.where(cond) against np.nonzero for several dtypes, ranks and sizes (tile edges of the compaction kernel,
+    all-false and all-true inputs); x[mask] and x[mask] = v with boolean masks as the reference's tests use them
+    (test/test_setitem.py:204-221)."""
+    rng = np.random.default_rng(63)
+    for shape, dtype, p in (((10,), "bool", 0.5), ((4096,), "int32", 0.3), ((4097,), "float32", 0.9), ((3, 5, 7), "bool", 0.5),
+                            ((70, 300), "float32", 0.01), ((1 << 20,), "bool", 0.5), ((9, 1000), "int8", 1.0), ((5, 5), "bool", 0.0),
+                            ((33, 129), "bfloat16", 0.5)):
+        m = rng.random(shape) < p
+        host = m.astype(np.float32)
+        if dtype == "float32":
+            host = np.where(m, rng.standard_normal(shape), 0.0).astype(np.float32)
+            host.reshape(-1)[::7] *= -0.0                        # -0.0 counts as zero
+            if m.any():
+                host[tuple(i[0] for i in np.nonzero(m))] = np.nan      # NaN counts as non-zero
+        v = jt.array(host.astype(np.float32) if dtype in ("float32", "bfloat16") else m.astype(L.NP_STORAGE[dtype]))
+        if dtype == "bfloat16":
+            v = v.bfloat16()
+        got = jt.where(v)
+        want = np.nonzero(host != 0) if dtype == "float32" else np.nonzero(m)
+        assert len(got) == len(shape)
+        for g, w in zip(got, want):
+            assert g.dtype == "int32" and list(g.shape) == [w.size] and np.array_equal(g.numpy(), w.astype(np.int32)), (shape, dtype)
+    # where(cond, x, y) is the ternary
+    c = jt.array([True, False, True])
+    assert jt.where(c, jt.array([1, 2, 3]), jt.array([7, 8, 9])).data.tolist() == [1, 8, 3]
+    # masks as keys
+    a = jt.array([1, 2, 3, 4])
+    b = jt.array([True, False, True, False])
+    a[b] = jt.array([-1, -2])
+    assert a.data.tolist() == [-1, 2, -2, 4]
+    a = jt.array([1, 2, 3, 4])
+    a[b] = jt.array([-1])
+    assert a.data.tolist() == [-1, 2, -1, 4]
+    a = jt.array([1, 2, 3, 4])
+    a[b] = -1
+    assert a.data.tolist() == [-1, 2, -1, 4]
+    x = rng.standard_normal((6, 5, 4)).astype(np.float32)
+    jx = jt.array(x)
+    assert np.array_equal(jx[jx > 0.5].data, x[x > 0.5])
+    rows = x[:, 0, 0] > 0
+    assert np.array_equal(jx[jt.array(rows)].data, x[rows])
+    assert np.array_equal(jx[jt.array(rows), 1:3].data, x[rows, 1:3])
+    m2 = x[0] > 0
+    assert np.array_equal(jx[2, jt.array(m2)].data, x[2, m2])
+    assert np.array_equal(jx[..., jt.array(m2[0])].data, x[..., m2[0]])
+    assert list(jx[jx > 100.0].shape) == [0]
+    with pytest.raises(IndexError):
+        jx[jt.array(m2)]                                         # [5, 4] does not match axes 0..1 of [6, 5, 4]
+    y = x.copy()
+    y[y < 0] = 0.0
+    jx[jx < 0] = 0.0
+    assert np.array_equal(jx.data, y)
