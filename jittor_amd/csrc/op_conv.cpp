@@ -115,19 +115,18 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         << p->dil_h << "\n#define DW " << p->dil_w << "\n";
 
     // ---- MFMA path ----------------------------------------------------------------
-    const char* wpx_env = getenv("MJT_CONV_WPX");
-    const int64_t WPX = wpx_env && atoi(wpx_env) == 1 ? 1 : 2;
+    const int64_t WPX = 2;                                  // pixel halves per workgroup (1: one wave per SIMD with 224-pixel wave tiles, 224-227 us on the 3x3 256-channel 56x56 layer against 215)
     const int64_t max_px = WPX == 1 ? 224 : 112;            // pixels per wave: 16 per accumulator tile
     const int64_t WPS = max_px == 224 ? 1 : 2;              // waves per SIMD the register budget is set for
     // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
-    const int64_t MT = getenv("MJT_CONV_MT") && atoi(getenv("MJT_CONV_MT")) == 8 && (K / G) % 128 == 0 ? 8 : 4;
+    const int64_t MT = 4;
     const int64_t Kg = K / G;                                // output channels of one group: the K of the MFMA kernel
     int64_t WKO = Kg % 256 == 0 ? 256 / (16 * MT) : Kg % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
     // LDS: two buffers of input rows (one block of CB channels each), a ring of NS weight slabs (64 bytes per output
     // channel of the workgroup each) and a spare KB that takes the writes of idle lanes.  Blocks of 32 channels
     // leave room for a deeper ring, which is what hides the latency of the slabs; the ring needs three slabs at least.
     const int64_t lds_total = 160 * 1024;
-    const int64_t CBLK = getenv("MJT_CONV_CB") && atoi(getenv("MJT_CONV_CB")) == 64 ? 64 : 32;
+    const int64_t CBLK = 32;
     const int64_t slab0 = 64 * 16 * MT * WKO, spare0 = 1024;
     const int64_t tile_limit = (lds_total - 4 * slab0 - spare0) / 2;         // leaves room for four slabs of the widest workgroup
     int64_t TRW = OW <= max_px ? max_px / OW : 0;
@@ -147,8 +146,6 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int64_t tile_rows = WPX * (TRW > 0 ? TRW : 1);
         const int64_t min_ranges = N * ((OH + tile_rows - 1) / tile_rows);
         while (WKO > 1 && 2 * min_ranges * (Kg / (16 * MT * WKO)) <= cus0) WKO /= 2;     // only while at most half of them would work
-        if (const char* e = getenv("MJT_CONV_WKO"))
-            if (atoi(e) >= 1 && atoi(e) <= WKO * 4 && Kg % (16 * MT * atoi(e)) == 0 && (atoi(e) & (atoi(e) - 1)) == 0 && atoi(e) <= 256 / (16 * MT)) WKO = atoi(e);
     }
     const bool half = x->dtype == MJT_FLOAT16;
     // (a grouped convolution is one launch per group on the group's channels: worth it from 32 x 64 channels per group)
@@ -204,10 +201,8 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int64_t spare = 1024;
         int64_t NSLAB = (lds_total - 2 * LROWS * LCOLS * CBLK * 2 - spare) / slab;
         if (NSLAB > 8) NSLAB = 8;
-        if (const char* e = getenv("MJT_CONV_NS"))
-            if (atoi(e) >= 3 && atoi(e) <= NSLAB) NSLAB = atoi(e);
         MJT_CHECK(NSLAB >= 3, "conv: internal: no room for the weight ring");
-        const int stage_depth = getenv("MJT_CONV_SD") && atoi(getenv("MJT_CONV_SD")) >= 2 && atoi(getenv("MJT_CONV_SD")) <= 8 ? atoi(getenv("MJT_CONV_SD")) : 4;
+        const int stage_depth = 4;                          // steps between asking for an input row and writing it to LDS (2-7: +-2 us)
         const int abl = getenv("MJT_ABLATE_CONV") ? atoi(getenv("MJT_ABLATE_CONV")) : 0;   // timing-only ablations (bench.py --ablate): results are wrong
         MJT_CHECK(abl == 0 || abl == 1 || abl == 2 || abl == 3 || abl == 7 || abl == 16 || abl == 17,
                   "conv: MJT_ABLATE_CONV must be one of 0, 1, 2, 3, 7, 16, 17");

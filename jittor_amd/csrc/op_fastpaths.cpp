@@ -169,7 +169,7 @@ bool try_window_gather(const mjt_tensor* x, const mjt_tensor* y, const std::vect
     // lanes of the last store round busy, and start every workgroup's run of y on a vector boundary
     const int64_t LW = (OW - 1) * SW + (KW - 1) * DW + 1;
     auto tile_rows = [&](int64_t th) { return (th - 1) * SH + (KH - 1) * DH + 1; };
-    const int wthreads = env_int("MJT_WINDOW_THREADS", 256);
+    const int wthreads = 256;
     int64_t TH = 0;
     double best = -1.0;
     for (int64_t th = 1; th <= OH; th++) {

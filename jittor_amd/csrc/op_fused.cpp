@@ -167,7 +167,6 @@ void fused_impl(const mjt_fused_desc* d) {
     };
     while (vec > 1 && !aligned(vec)) vec /= 2;
     int64_t nvec = total / vec;
-    auto env_int = [](const char* n, int d) { const char* v = getenv(n); return v && *v ? atoi(v) : d; };
     // measured on MI355X: one vector per lane is fastest for the chain workloads (more vectors per
     // lane cost registers and occupancy); outputs too large to be re-read from cache are stored
     // non-temporally, loads stay plain; and such streams run best as single-wave workgroups, which the dispatcher
@@ -183,9 +182,9 @@ void fused_impl(const mjt_fused_desc* d) {
             if (dims[a].size > 1 && dims[a].bcast[k]) full = false;
         reads_stream = reads_stream || full;
     }
-    int block = env_int("MJT_FUSED_BLOCK", streams && reads_stream ? 64 : 256);
-    int unroll = env_int("MJT_FUSED_UNROLL", 1);
-    int nt = env_int("MJT_FUSED_NT", streams ? 2 : 0);   // bit 0: non-temporal loads, bit 1: non-temporal stores
+    int block = streams && reads_stream ? 64 : 256;
+    int unroll = 1;
+    int nt = streams ? 2 : 0;   // bit 0: non-temporal loads, bit 1: non-temporal stores
 
     // ---- parameter block layout ---------------------------------------------------
     // a[0] nvec | per merged axis: extent, divider | per var: pointer or scalar bits

@@ -112,8 +112,7 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
         // the caller's tile, if it names one (tile_m x tile_n of 64, 128 or 256)
         if (tile_m == 64 || tile_m == 128 || tile_m == 256) best_mi = tile_m / 64;
         if (tile_n == 64 || tile_n == 128 || tile_n == 256) best_ni = tile_n / 64;
-        int MI = env_int("MJT_GEMM_MI", best_mi), NI = env_int("MJT_GEMM_NI", best_ni);
-        if ((MI != 1 && MI != 2 && MI != 4) || (NI != 1 && NI != 2 && NI != 4)) { MI = best_mi; NI = best_ni; }
+        const int MI = best_mi, NI = best_ni;
         const int in = in_dtype == MJT_BFLOAT16 ? 0 : in_dtype == MJT_FLOAT16 ? 1 : 2;
         const int out = out_dtype == MJT_BFLOAT16 ? 0 : out_dtype == MJT_FLOAT16 ? 1 : 2;
         const bool one_stage = K <= (esz == 2 ? 64 : 32) && !getenv("MJT_GEMM_TWO_BUFFERS");       // a single stage of the kernel's k loop

@@ -150,13 +150,13 @@ void launch(bool row, int tx, int ty, int op, bool second, const void* x, void* 
             int64_t per, int64_t total, bool stream = false, const Prologue* pro = nullptr, bool may_build = true, bool tsplit = false) {
     // inputs larger than the caches are streamed (read once, non-temporal loads)
     // loads in flight per lane: 8, or as many as a row gives a lane when that is fewer (the unrolled loop only takes whole batches)
-    int unr = env_int("MJT_REDUCE_UNR", 8);
+    int unr = 8;
     if (row && !red.empty()) {
         const int64_t per_lane = red.back().size / ((int64_t)g * vec);
         while (unr > 1 && unr > per_lane) unr /= 2;
     }
     Variant v{tx, ty, op, (int)kept.size(), (int)red.size(), vec, g, unr,
-              env_int("MJT_REDUCE_NT", stream ? 1 : 0), row, S > 1, use64, second, pro};
+              stream ? 1 : 0, row, S > 1, use64, second, pro};
     v.tsplit = tsplit && !row && S > 1;
     JitKernel* k = get_kernel(v, may_build);
     std::vector<uint64_t> a(8 + 6 * 5, 0);
@@ -267,8 +267,8 @@ void reduce_core(const mjt_tensor* x, const mjt_tensor* y, int op, uint32_t redu
         // long rows streamed from memory: up to eight waves per row while every lane keeps at least two loads (measured
         // on an [8192, 4096] float32 sum: 64 lanes per row 22.3 us, 128 21.1, 256 20.8, 512 20.2; with a single load per
         // lane the fixed cost of a lane dominates: [65536, 1024] with 256 lanes 48 us against 39)
-        if (stream && g == 64 && env_int("MJT_REDUCE_WIDE", 1))
-            while (g < env_int("MJT_REDUCE_GMAX", 512) && (int64_t)g * 2 * vec * 2 <= L) g *= 2;
+        if (stream && g == 64)
+            while (g < 512 && (int64_t)g * 2 * vec * 2 <= L) g *= 2;
         if (env_int("MJT_REDUCE_G", 0) >= 64) g = env_int("MJT_REDUCE_G", 0);
         int64_t nL = (L + (int64_t)g * vec - 1) / ((int64_t)g * vec);
         int64_t total = (R / L) * nL;

@@ -355,10 +355,6 @@ bool try_window_scatter(Plan* plan, int op, const mjt_tensor* x, const mjt_tenso
     // without a prologue the candidates are loads from y itself, far apart for neighbouring elements of x: more of them
     // per lane coalesce worse (3x3 stride-2 windows into [64,64,112,112]: 230 us with four elements per lane, 175 with one)
     if (!sp) wvec = 1;
-    if (const char* e = getenv("MJT_WINDOW_SCATTER_VEC")) {               // 1, 2, 4 or 8, for experiments
-        const int v = atoi(e);
-        if (v >= 1 && v <= wvec && (v & (v - 1)) == 0) wvec = v;
-    }
     std::ostringstream vk;
     vk << "WS" << op << (use64 ? "L" : "I") << wvec << "|" << SH << "," << SW << "," << DH << "," << DW << "," << CH << "," << CW << "," << KH << "," << KW;
     for (int i = 0; i < XD; i++) vk << "," << x->shape[i];
