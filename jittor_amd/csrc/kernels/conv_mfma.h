@@ -8,8 +8,8 @@
 // contribute 0 (overflow value 0 times w).
 //
 // All geometry is baked in by the host: C_, H_, W_, K_ (input and output channels of the convolution: of one group when
-// it is grouped; XC_ and YK_ are then the channel counts of the whole x and y, whose pointers the host has moved to
-// the group's first channel), R_, S_, OH_, OW_, SH, SW,
+// it is grouped; XC_ and YK_ are then the channel counts of the whole x and y, and blockIdx.y is the group),
+// R_, S_, OH_, OW_, SH, SW,
 // PH, PW, DH, DW, WKO (groups of 16*MT output channels per workgroup), WPX (row
 // groups per workgroup), TRW / NT / LROWS (output rows per wave, 16-pixel tiles per
 // wave and input rows in LDS of a full tile), RPW (output rows a workgroup owns),
@@ -151,8 +151,10 @@ template <int N> __device__ __forceinline__ void mjt_lds_wait(mjt_u32x4v& x) {
 }
 
 extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu(WPS, WPS))) void ENTRY(Params p) {
-    const unsigned short* __restrict__ xp = (const unsigned short*)p.a[0];
-    const unsigned short* __restrict__ wp = (const unsigned short*)p.a[1];
+    // blockIdx.y = group of a grouped convolution (0 otherwise): its channels of x, its weights, its channels of y
+    const unsigned short* __restrict__ xp = (const unsigned short*)p.a[0] + (size_t)blockIdx.y * (C_ * H_ * W_);
+    const unsigned short* __restrict__ wp = (const unsigned short*)p.a[1] + (size_t)blockIdx.y * (K_ * C_ * R_ * S_);
+    const int y_k0 = blockIdx.y * K_;
     const int n_img = (int)(unsigned long long)p.a[3];
     __shared__ __attribute__((aligned(16))) unsigned short xs[2][TILE_ELEMS];
     __shared__ __attribute__((aligned(16))) unsigned short as_ring[NS * KO_WG * 32 + 512];   // ring of weight slabs and a spare KB, see below
@@ -538,7 +540,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
                     const mjt_f32x4 v = acc[m][t];
-                    const size_t o = (((size_t)n * YK_ + ko_base + m * 16 + l16_e) * OH_ + orow) * OW_ + col;
+                    const size_t o = (((size_t)n * YK_ + y_k0 + ko_base + m * 16 + l16_e) * OH_ + orow) * OW_ + col;
 #if Y_BF16
                     mjt_u32x2 pk;
                     pk[0] = mjt_narrow2(v[0], v[1]);
@@ -558,7 +560,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
                 if (q < TRW_ * OW_ && orow < row_lim && !(ABL & 1)) {
 #pragma unroll
                     for (int m = 0; m < MT; m++) {
-                        const size_t o = (((size_t)n * YK_ + ko_base + m * 16 + l16_e) * OH_ + orow) * OW_ + col;
+                        const size_t o = (((size_t)n * YK_ + y_k0 + ko_base + m * 16 + l16_e) * OH_ + orow) * OW_ + col;
 #if Y_BF16
                         ((unsigned short*)p.a[2])[o] = (unsigned short)mjt_narrow2(acc[m][t][i], 0.0f);
 #else
@@ -615,9 +617,9 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
 
 // Weight re-pack: w[ko][c][kh][kw] -> Wp[tap][c/CB][k-step][ko/16][lg][l16][8 c] (c = CB block + 32 k-step + 8 lg + ..)
 extern "C" __global__ __launch_bounds__(256) void ENTRY_PACK(Params p) {
-    const unsigned short* __restrict__ w = (const unsigned short*)p.a[0];
-    unsigned short* __restrict__ wp = (unsigned short*)p.a[1];
-    const int total = K_ * C_ * R_ * S_;
+    const int total = K_ * C_ * R_ * S_;                      // of one group: blockIdx.y
+    const unsigned short* __restrict__ w = (const unsigned short*)p.a[0] + (size_t)blockIdx.y * total;
+    unsigned short* __restrict__ wp = (unsigned short*)p.a[1] + (size_t)blockIdx.y * total;
     for (int o = blockIdx.x * 256 + threadIdx.x; o < total; o += gridDim.x * 256) {
         int c8 = o & 7, l16 = (o >> 3) & 15, lg = (o >> 7) & 3;
         int rest = o >> 9;

@@ -249,18 +249,15 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int64_t wg = Kg * C * R * S;               // weights of one group
         int64_t pblocks = (wg + 255) / 256;
         if (pblocks > 2048) pblocks = 2048;
-        const int64_t ysz = y->dtype == MJT_FLOAT32 ? 4 : 2;
-        for (int64_t g = 0; g < G; g++) {
-            const char* wsrc = (const char*)w->ptr + g * wg * 2;
-            char* wdst = (char*)(pack_mode ? packed : g_wpack) + g * wg * 2;
-            if (pack_mode != 2) {
-                std::vector<uint64_t> pa{bits_of_ptr(wsrc), bits_of_ptr(wdst), 0, 0};
-                jit_launch(kp, (unsigned)pblocks, 1, 256, 0, pa);
-            }
-            if (pack_mode == 1) continue;
-            std::vector<uint64_t> a{bits_of_ptr((const char*)x->ptr + g * C * H * W * 2), bits_of_ptr(wdst),
-                                    bits_of_ptr((char*)y->ptr + g * Kg * OH * OW * ysz), (uint64_t)N};
-            jit_launch(k, (unsigned)blocks, 1, (unsigned)(64 * WPX * WKO), 0, a);
+        // one launch for all groups (the group is the grid's second axis)
+        char* wdst = (char*)(pack_mode ? packed : g_wpack);
+        if (pack_mode != 2) {
+            std::vector<uint64_t> pa{bits_of_ptr(w->ptr), bits_of_ptr(wdst), 0, 0};
+            jit_launch(kp, (unsigned)pblocks, (unsigned)G, 256, 0, pa);
+        }
+        if (pack_mode != 1) {
+            std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(wdst), bits_of_ptr(y->ptr), (uint64_t)N};
+            jit_launch(k, (unsigned)blocks, (unsigned)G, (unsigned)(64 * WPX * WKO), 0, a);
         }
         return;
     }
