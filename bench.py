@@ -518,11 +518,12 @@ TRAFFIC_SOURCE = "profiles/hbm_traffic_all_workloads.txt"
 MEASURED_TRAFFIC = {
     "C1": ("mjt_reduce_row_add_float32_float32_k1r1v4g512", 2.0 * 65553.0 * 1024 + 256.0 * 1024),
     "C2": ("mjt_window_gather_b4_56x56_k3x3_s1x1_d1x1_o56x56_t8x1", 2.0 * 15647.5 * 1024 + 225792.0 * 1024),
-    "C3add": ("mjt_scatter1d_add_float32_int32_w16384_b64_e8_s1920_main", 2.0 * 65688.8 * 1024 + 37617.6 * 1024),
-    "C3max": ("mjt_scatter1d_maximum_float32_int32_w16384_b64_e8_s4096_main", 2.0 * 65690.2 * 1024 + 37642.0 * 1024),
+    # C3: main pass + tail pass (the two launches of a step)
+    "C3add": ("mjt_scatter1d_add_float32_int32_w16384_b64_e8_s1920_main", 2.0 * (65715.7 + 19497.6) * 1024 + (41766.6 + 9030.9) * 1024),
+    "C3max": ("mjt_scatter1d_maximum_float32_int32_w16384_b64_e8_s4096_main", 2.0 * (65708.2 + 19490.9) * 1024 + (41772.3 + 9030.9) * 1024),
     "C4": ("mjt_fused_11ops_caa413813b1db4ef", 2.0 * 65566.0 * 1024 + 131072.0 * 1024),
-    "C5": ("mjt_conv_mfma_bf16_c256_k256_56x56_r3x3_s1x1_p1x1_d1x1_rows14_of32", 2.0 * 113243.4 * 1024 + 211680.1 * 1024),
-    "C5bf16out": ("mjt_conv_mfma_bf16_c256_k256_56x56_r3x3_s1x1_p1x1_d1x1_rows14_obf16", 2.0 * 112271.2 * 1024 + 112708.6 * 1024),
+    "C5": ("mjt_conv_mfma_bf16_c256_k256_56x56_r3x3_s1x1_p1x1_d1x1_rows14_of32", 2.0 * 113300.0 * 1024 + 211215.0 * 1024),
+    "C5bf16out": ("mjt_conv_mfma_bf16_c256_k256_56x56_r3x3_s1x1_p1x1_d1x1_rows14_obf16", 2.0 * 112314.9 * 1024 + 112340.4 * 1024),
 }
 
 
