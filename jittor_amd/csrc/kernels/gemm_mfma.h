@@ -28,12 +28,14 @@
 // four MFMAs (lanes 32..63 read the next chunk, so that an MFMA sums k and k + 4 of a
 // chunk pair; any pairing is right as long as both operands use the same one).
 //
-// CONV = 1 (float32 only) makes the kernel an implicit-GEMM convolution, the meta-op group of
+// CONV = 1 makes the kernel an implicit-GEMM convolution, the meta-op group of
 // python/jittor/nn.py:1251-1262 that opt/tuner/conv_tuner.cc:233-240,365-373 relays for every float type:
 // A = the weights [K_][C_*R_*S_] (rows padded to 16 bytes by the host), B'[k = (c, r, s)][j = (image, oh, ow)] =
 // x[image][c][oh*SH-PH+r*DH][ow*SW-PW+s*DW] (0 outside the image) is never written to memory -- the B tile of a
 // stage is gathered from x element by element on its way to LDS (a float32 MFMA runs at a sixteenth of the 16-bit
-// rate, so the gather's address arithmetic hides behind it) -- and C[k][j] is stored as y[image][k][oh][ow].
+// rate, so the gather's address arithmetic hides behind it; with 16-bit operands the gather is what bounds the
+// kernel, which then serves the shapes the MFMA convolution kernel does not take) -- and C[k][j] is stored as
+// y[image][k][oh][ow].
 // Geometry comes as C_, H_, W_, K_, R_, S_, OH_, OW_, SH, SW, PH, PW, DH, DW; N = images * OH_ * OW_.
 //
 // Rows of A' and columns of B' beyond M and N are read from the last valid row (their
@@ -214,21 +216,22 @@ template <int ROWS, bool KCONT> struct mjt_stager {
 };
 
 #if CONV
-// The B tile of a stage of the implicit-GEMM convolution.  Same blocks as mjt_stager<TN, false>: 4 lanes hold 4
-// k-rows x 4 columns, lane tid % 4 the k-row.  What depends on a column alone (its image and pixel) is worked out once
-// per workgroup (mjt_conv_cols): base = element offset of x[image][0][oh*SH-PH][ow*SW-PW], hw = that row and column,
-// both biased by 0x4000, in one word (0 for a column past N: every tap of it then fails the range check).
+// The B tile of a stage of the implicit-GEMM convolution.  Same blocks as mjt_stager<TN, false>: EPC lanes hold EPC
+// k-rows x EPC columns (4 x 4 float32 values, 8 x 8 16-bit ones), lane tid % EPC the k-row.  What depends on a column
+// alone (its image and pixel) is worked out once per workgroup (mjt_conv_cols): base = element offset of
+// x[image][0][oh*SH-PH][ow*SW-PW], hw = that row and column, both biased by 0x4000, in one word (0 for a column past
+// N: every tap of it then fails the range check).
 struct mjt_conv_cols {
     static constexpr int PER = TN * KC / NTHR;
-    int base[PER][4];
-    unsigned hw[PER][4];
+    int base[PER][EPC];
+    unsigned hw[PER][EPC];
     // (compile-time loop indices throughout: with run-time ones the compiler keeps these arrays in scratch memory
     // once the loops are too long for it to unroll them itself)
     __device__ __forceinline__ void init(int n0, int N, int tid) {
-        mjt_static_for<0, PER * 4>([&](auto ic) {
-            constexpr int i = decltype(ic)::v / 4, e = decltype(ic)::v % 4;
-            const int b = tid / 4 + i * (NTHR / 4);
-            const int j = n0 + (b % (TN / 4)) * 4 + e;
+        mjt_static_for<0, PER * EPC>([&](auto ic) {
+            constexpr int i = decltype(ic)::v / EPC, e = decltype(ic)::v % EPC;
+            const int b = tid / EPC + i * (NTHR / EPC);
+            const int j = n0 + (b % (TN / EPC)) * EPC + e;
             const int img = j / (OH_ * OW_), px = j - img * (OH_ * OW_);
             const int oh = px / OW_, ow = px - oh * OW_;
             const int ih = oh * SH - PH, iw = ow * SW - PW;
@@ -242,34 +245,48 @@ struct mjt_conv_stager {
     static constexpr int RS = R_ * S_, CRS = C_ * R_ * S_;
     mjt_u32x4v reg[PER];
 
-    __device__ __forceinline__ void fetch(const float* __restrict__ x, const mjt_conv_cols& cols, int k0, int tid) {
+    __device__ __forceinline__ void fetch(const TIN* __restrict__ x, const mjt_conv_cols& cols, int k0, int tid) {
         mjt_static_for<0, PER>([&](auto ic) {
             constexpr int i = decltype(ic)::v;
-            const int b = tid / 4 + i * (NTHR / 4);
-            const int k = k0 + (b / (TN / 4)) * 4 + tid % 4;
+            const int b = tid / EPC + i * (NTHR / EPC);
+            const int k = k0 + (b / (TN / EPC)) * EPC + tid % EPC;
             const bool kvalid = k < CRS;
             const int kk = kvalid ? k : 0;
             const int c = kk / RS, rs = kk - c * RS;
             const int r = rs / S_, t = rs - r * S_;
             const int koff = (c * H_ + r * DH) * W_ + t * DW;
             const unsigned dhw = ((unsigned)(r * DH) << 16) | (unsigned)(t * DW);
-            mjt_static_for<0, 4>([&](auto ec) {
+            unsigned v[EPC];
+            mjt_static_for<0, EPC>([&](auto ec) {
                 constexpr int e = decltype(ec)::v;
                 const unsigned q = cols.hw[i][e] + dhw;
                 const bool ok = kvalid && (q >> 16) - 0x4000u < (unsigned)H_ && (q & 0xffffu) - 0x4000u < (unsigned)W_;
                 // an unconditional load from a valid address, zeroed afterwards: a load under a condition is a branch per
                 // element
-                const unsigned v = __float_as_uint(x[ok ? cols.base[i][e] + koff : 0]);
-                reg[i][e] = ok ? v : 0u;
+#if IN == 2
+                const unsigned ld = __float_as_uint(x[ok ? cols.base[i][e] + koff : 0]);
+#else
+                const unsigned ld = x[ok ? cols.base[i][e] + koff : 0];
+#endif
+                v[e] = ok ? ld : 0u;
             });
+#if IN == 2
+            reg[i][0] = v[0]; reg[i][1] = v[1]; reg[i][2] = v[2]; reg[i][3] = v[3];
+#else
+            reg[i][0] = v[0] | (v[1] << 16); reg[i][1] = v[2] | (v[3] << 16); reg[i][2] = v[4] | (v[5] << 16); reg[i][3] = v[6] | (v[7] << 16);
+#endif
         });
     }
     __device__ __forceinline__ void commit(unsigned char* lds, int tid) const {
         mjt_static_for<0, PER>([&](auto ic) {
             constexpr int i = decltype(ic)::v;
-            const int b = tid / 4 + i * (NTHR / 4);
-            const int row = (b % (TN / 4)) * 4 + tid % 4, kc = b / (TN / 4);
+            const int b = tid / EPC + i * (NTHR / EPC);
+            const int row = (b % (TN / EPC)) * EPC + tid % EPC, kc = b / (TN / EPC);
+#if IN == 2
             *(mjt_u32x4v*)(lds + row * ROWB + kc * 16) = mjt_transpose4x4_b32(reg[i], tid);
+#else
+            *(mjt_u32x4v*)(lds + row * ROWB + kc * 16) = mjt_transpose8x8_b16(reg[i], tid);
+#endif
         });
     }
 };
@@ -426,14 +443,17 @@ extern "C" __global__ __launch_bounds__(NTHR) void ENTRY(Params p) {
                 if (row < M && col < N) {
                     const float v = acc[i][j][e];
 #if CONV
-                    C[((long long)img * K_ + row) * (OH_ * OW_) + px] = v;
-#elif OUT == 2
-                    C[(long long)row * ldc + col] = v;
-#elif OUT == 0
-                    C[(long long)row * ldc + col] = (unsigned short)(__float_as_uint(v) >> 16);     // truncation (type/fp16_compute.h:238-241)
+                    const long long at = ((long long)img * K_ + row) * (OH_ * OW_) + px;
 #else
-                    const _Float16 h = (_Float16)v;                                                  // nearest even (type/fp16_compute.h:147-198)
-                    C[(long long)row * ldc + col] = __builtin_bit_cast(unsigned short, h);
+                    const long long at = (long long)row * ldc + col;
+#endif
+#if OUT == 2
+                    C[at] = v;
+#elif OUT == 0
+                    C[at] = (unsigned short)(__float_as_uint(v) >> 16);     // truncation (type/fp16_compute.h:238-241)
+#else
+                    const _Float16 h = (_Float16)v;                        // nearest even (type/fp16_compute.h:147-198)
+                    C[at] = __builtin_bit_cast(unsigned short, h);
 #endif
                 }
             }

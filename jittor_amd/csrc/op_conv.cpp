@@ -160,12 +160,14 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                          // multiples the product kernel below reads x as it lies and is as fast or faster for every shape
                          // measured (64 x 512 x 28 x 28 -> 128 channels: 22 us against 42; 64 x 256 x 56 x 56 -> 64: 31 against
                          // 73; 64 x 1024 x 16 x 16 -> 2048: 82 against 387; closest 64 x 512 x 28 x 28 -> 512: 74 against 74),
-                         // this kernel walking one-step channel blocks.  With other plane sizes the product needs a padded
-                         // copy of x first, which pays with many more input than output channels and few output channels or
-                         // a small map (64 x 1024 x 14 x 14 -> 256: 50 against 142)
+                         // this kernel walking one-step channel blocks.  With other plane sizes the product kernel gathers x
+                         // (its CONV mode), which wins with more than 64 output channels and enough 128 x 64 tiles for the chip
+                         // (64 x 512 x 14 x 14 -> 512: 36 against 61; 64 x 1024 x 14 x 14 -> 512: 63 against 100; -> 256: 37
+                         // against 142) and with many more input than output channels and few output channels or a small map
                          !(R * S == 1 && G == 1 && p->stride_h == 1 && p->stride_w == 1 && matmul_available() && !getenv("MJT_CONV_NO_GEMM") &&
                            ((p->pad_h == 0 && p->pad_w == 0 && OH == H && OW == W && (OH * OW * 2) % 16 == 0 && (uintptr_t)w->ptr % 16 == 0) ||
-                            (C >= 4 * K && (K <= 64 || OH * OW <= 256))));
+                            (C >= 4 * K && (K <= 64 || OH * OW <= 256)) ||
+                            (K > 64 && !getenv("MJT_CONV_NO_IGEMM") && ((K + 127) / 128) * ((N * OH * OW + 63) / 64) >= 256)));
     if (mfma_ok) {
         // Rows per workgroup: a workgroup walks RPW output rows as NFULL tiles of TR rows plus one
         // shorter tile.  Pick the RPW that minimises (rounds of workgroups over the compute units) x
@@ -297,32 +299,44 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
                 MJT_FAIL(MJT_ERR_DEVICE, "conv: padding the weight rows failed: " << mjt_last_error());
             wmat = wpad;
         }
-        // float32: the product kernel gathers its second operand from x on the fly (kernels/gemm_mfma.h with CONV): no
-        // column matrices.  Offsets inside x and y and the column number are 32-bit there, rows and columns of the
-        // image and the reach of the taps 14-bit.
-        if (!plain && x->dtype == MJT_FLOAT32 && y->dtype == MJT_FLOAT32 && !getenv("MJT_CONV_NO_IGEMM") &&
+        // The product kernel gathers its second operand from x on the fly (kernels/gemm_mfma.h with CONV): no column
+        // matrices.  float32 convolutions, and the 16-bit ones the MFMA convolution kernel above does not take (odd widths,
+        // channel counts that are no multiple of 32 / 64, long rows).  Offsets inside x and y and the column number are
+        // 32-bit there, rows and columns of the image and the reach of the taps 14-bit.
+        const bool ig16 = x->dtype == MJT_BFLOAT16 || x->dtype == MJT_FLOAT16;
+        const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
+        const int64_t NP = N * P, tiles64 = ((K + 63) / 64) * ((NP + 63) / 64);
+        // (16-bit operands with a long sum and fewer 64 x 64 tiles than compute units stay on the column matrices, whose
+        // product picks its tiles for a part-filled chip: 32 x 512 x 7 x 7 3x3 -> 512, 200 tiles: 102 us here, 71 there)
+        const bool ig_fits = !ig16 || tiles64 >= cus || CRS <= 1024;
+        if (!plain && ((x->dtype == MJT_FLOAT32 && y->dtype == MJT_FLOAT32) || ig16) && ig_fits && !getenv("MJT_CONV_NO_IGEMM") &&
             numel(x) < (int64_t(1) << 31) && numel(y) < (int64_t(1) << 31) && H < 16384 && W < 16384 &&
             (R - 1) * p->dil_h < 16384 && (S - 1) * p->dil_w < 16384 && p->pad_h < 16384 && p->pad_w < 16384 &&
             OH * p->stride_h < 16384 && OW * p->stride_w < 16384) {
-            const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
-            const int64_t NP = N * P;
-            // Tile: 64 output channels x 64 pixels, or 128 x 128 when there are more than 64 output channels and enough
-            // tiles of that size for every compute unit.  Measured (us, tiles 64x64 / 64x128 / 128x64 / 128x128):
+            // Tile, float32: 64 output channels x 64 pixels, or 128 x 128 when there are more than 64 output channels and
+            // enough tiles of that size for every compute unit.  Measured (us, tiles 64x64 / 64x128 / 128x64 / 128x128):
             // 64x64x56x56 3x3 -> 64: 202 / 244 / 381 / 365; 64x3x224x224 7x7 stride 2 -> 64: 228 / 254 / 426 / 379;
             // 64x128x28x28 3x3 -> 128: 208 / 246 / 214 / 192; 64x512x7x7 3x3 -> 512: 272 / 335 / 273 / 469.  Small tiles
             // win because four workgroups then share a compute unit: the gather's address arithmetic of one overlaps the
             // MFMAs of another.
-            const bool big = K > 64 && ((K + 127) / 128) * ((NP + 127) / 128) >= cus;
-            const int MI = big ? 2 : 1, NI = big ? 2 : 1;
+            // 16-bit: the gather bounds the kernel and every 64 rows of output channels repeat it, so 128 x 64 when
+            // such tiles fill the chip (us, 64x64 / 128x64 / 256x64 / column matrices: 64x1024x14x14 1x1 -> 256: 51 / 37 /
+            // 36 / 68; 64x256x13x13 3x3 -> 384: 116 / 76 / 139 / 103; 64x64x27x27 3x3 stride 2 -> 128: 20 / 18 / 23 / 29;
+            // 64x48x28x28 3x3 -> 96: 40 / 35 / 67 / 69; 64x3x224x224 7x7 stride 2 -> 64: 136 / - / - / 285).
+            const bool big = !ig16 && K > 64 && ((K + 127) / 128) * ((NP + 127) / 128) >= cus;
+            const bool tall = ig16 && K > 64 && ((K + 127) / 128) * ((NP + 63) / 64) >= cus;
+            const int MI = big || tall ? 2 : 1, NI = big ? 2 : 1;
+            const int in = x->dtype == MJT_BFLOAT16 ? 0 : x->dtype == MJT_FLOAT16 ? 1 : 2;
+            const int out = y->dtype == MJT_BFLOAT16 ? 0 : y->dtype == MJT_FLOAT16 ? 1 : 2;
             std::ostringstream key;
-            key << "igemm|" << geo.str() << MI << NI;
+            key << "igemm|" << geo.str() << MI << NI << in << out;
             JitKernel* k = cached(key.str());
             if (!k) {
                 std::ostringstream name;
-                name << "mjt_conv_igemm_float32_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s" << p->stride_h << "x"
+                name << "mjt_conv_igemm_" << mjt_dtype_name(x->dtype) << (y->dtype != x->dtype ? "_of32" : "") << "_c" << C << "_k" << K << "_" << H << "x" << W << "_r" << R << "x" << S << "_s" << p->stride_h << "x"
                      << p->stride_w << "_p" << p->pad_h << "x" << p->pad_w << "_d" << p->dil_h << "x" << p->dil_w << "_" << 64 * MI << "x" << 64 * NI;
                 std::ostringstream src;
-                src << "#define ENTRY " << name.str() << "\n#define CONV 1\n#define IN 2\n#define OUT 2\n#define MI " << MI << "\n#define NI " << NI
+                src << "#define ENTRY " << name.str() << "\n#define CONV 1\n#define IN " << in << "\n#define OUT " << out << "\n#define MI " << MI << "\n#define NI " << NI
                     << "\n#define A_KCONT 1\n#define B_KCONT 0\n" << geo.str();
                 src << embedded_source("gemm_mfma.h") << "\n";
                 k = jit_get(src.str(), name.str());

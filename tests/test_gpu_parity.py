@@ -923,12 +923,23 @@ def test_conv_direct_small_shapes_and_fp32(gpu):
     dict(dt="float32", x=(8, 3, 64, 64), w=(32, 3, 7, 7), p=(2, 2, 3, 3, 1, 1)),      # a stem: weight rows of 588 bytes are padded to 16-byte multiples
     dict(dt="float32", x=(8, 3, 64, 64), w=(32, 3, 7, 7), p=(2, 2, 3, 3, 1, 1), cols=True),      # the same through column matrices
     dict(dt="float32", x=(4, 32, 28, 28), w=(48, 32, 3, 3), p=(1, 1, 1, 1, 1, 1), cols=True),
+    dict(dt="bfloat16", x=(2, 64, 27, 27), w=(128, 64, 3, 3), p=(2, 2, 1, 1, 1, 1), out="bfloat16", cols=True),
+    dict(dt="float16", x=(4, 64, 14, 14), w=(96, 64, 1, 1), p=(1, 1, 0, 0, 1, 1), out="float16", cols=True),
+    dict(dt="bfloat16", x=(3, 40, 13, 9), w=(72, 40, 5, 3), p=(1, 1, 2, 1, 1, 1)),                 # 40 channels, 13 x 9 maps, 5 x 3 taps: weight rows of 1200 bytes
+    dict(dt="float16", x=(2, 16, 10, 130), w=(24, 16, 3, 3), p=(1, 1, 1, 1, 1, 1), out="float16"),   # rows of 130 outputs
     dict(dt="float32", x=(3, 80, 19, 23), w=(136, 80, 3, 3), p=(1, 2, 2, 0, 2, 1)),                 # 136 output channels: two row tiles, the second mostly empty; mixed strides
     dict(dt="float32", x=(70, 16, 7, 7), w=(24, 16, 3, 3), p=(1, 1, 1, 1, 1, 1)),                    # 7 x 7 maps: a tile of pixels spans several images
     dict(dt="float32", x=(2, 8, 40, 130), w=(16, 8, 1, 5), p=(1, 1, 0, 2, 1, 1)),                    # wide rows, taps along the row only
+    # 16-bit with more than 64 output channels and enough tiles: 128 x 64 tiles (200 and 136 rows: part-filled row tiles)
+    dict(dt="bfloat16", x=(50, 32, 13, 13), w=(200, 32, 3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16", tile="128x64"),
+    dict(dt="float16", x=(80, 24, 15, 17), w=(136, 24, 3, 3), p=(2, 1, 1, 1, 1, 1), tile="128x64"),
+    # float32 with more than 64 output channels and enough tiles: 128 x 128 tiles (72 rows: a part-filled row tile)
+    dict(dt="float32", x=(42, 8, 28, 28), w=(72, 8, 3, 3), p=(1, 1, 1, 1, 1, 1), tile="128x128"),
+    # 16-bit with a long sum and few tiles: stays on the column matrices
+    dict(dt="bfloat16", x=(2, 128, 7, 7), w=(128, 128, 3, 3), p=(1, 1, 1, 1, 1, 1), stays=True),
     # the product on the direct-copy kernel (asked for by name: these shapes have too few tiles to get it by themselves):
     # weights shared across the batch, column matrices with the pixels innermost read with transposing reads
-    dict(dt="bfloat16", x=(3, 64, 15, 15), w=(96, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), dma=True),
+    dict(dt="bfloat16", x=(3, 64, 15, 15), w=(96, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), dma=True, cols=True),
     dict(dt="float16", x=(4, 64, 16, 16), w=(96, 64, 1, 1), p=(1, 1, 0, 0, 1, 1), out="float16", plain=True, dma=True),
 ])
 def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
@@ -949,8 +960,9 @@ def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
     if case.get("cols"):
         monkeypatch.setenv("MJT_CONV_NO_IGEMM", "1")
     got, kern = _conv_call(xb, wb, case["p"], out_dtype=out, in_dtype=dt)
-    if dt == "float32" and not case.get("plain") and not case.get("cols"):
-        assert kern.startswith("mjt_conv_igemm_float32"), kern      # float32: the product gathers its operand from x itself
+    if not case.get("plain") and not case.get("cols") and not case.get("dma") and not case.get("stays"):
+        assert kern.startswith("mjt_conv_igemm_" + dt), kern        # the product kernel gathers its operand from x itself
+        assert kern.endswith(case.get("tile", "64x64")), kern
     else:
         assert kern == ("conv_as_gemm" if case.get("plain") else "conv_as_reindex_gemm"), kern
     got = widen[out](got)
@@ -979,12 +991,15 @@ def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
 def test_conv_1x1_runs_as_a_product(gpu, monkeypatch):
     """A 1x1 convolution of stride 1 is handed to the matrix-product kernel although the MFMA convolution kernel would
     take it: always when a plane's rows are 16-byte multiples (the product then reads x as it lies, with tiles picked for
-    a short sum), and through a padded copy when its input channels outnumber its output channels 4 : 1 or more with at
-    most 64 output channels or a map of at most 256 pixels.  Both kernels against a float64 product, same bound; 16-bit
-    and float32 results."""
+    a short sum); with other plane sizes the product kernel gathers x itself, when the input channels outnumber the output
+    channels 4 : 1 or more with at most 64 output channels or a map of at most 256 pixels, or when there are more than 64
+    output channels and enough 128 x 64 tiles for every compute unit.  Both kernels against a float64 product, same
+    bound; 16-bit and float32 results."""
     rng = np.random.default_rng(43)
     for xs, ws, out, want in (((2, 256, 16, 16), (64, 256, 1, 1), "float32", "conv_as_gemm"),
-                              ((3, 512, 14, 14), (128, 512, 1, 1), "float32", "conv_as_reindex_gemm"),
+                              ((3, 512, 14, 14), (128, 512, 1, 1), "float32", "mjt_conv_igemm_bfloat16_of32"),
+                              ((48, 128, 14, 14), (256, 128, 1, 1), "bfloat16", "mjt_conv_igemm_bfloat16_c128_k256_14x14_r1x1_s1x1_p0x0_d1x1_128x64"),
+                              ((20, 128, 14, 14), (256, 128, 1, 1), "bfloat16", "mjt_conv_mfma_bf16"),   # too few tiles: stays
                               ((3, 64, 24, 28), (256, 64, 1, 1), "bfloat16", "conv_as_gemm"),        # one step of the sum, tiles of 128
                               ((5, 128, 12, 20), (192, 128, 1, 1), "float32", "conv_as_gemm"),       # 240 pixels, 192 channels: edge tiles
                               ((2, 1024, 8, 8), (128, 1024, 1, 1), "bfloat16", "conv_as_gemm"),      # 64 pixels: narrow tiles
