@@ -41,11 +41,24 @@ typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
 #else
 #define MJT_MFMA_ASM "v_mfma_f32_32x32x16_f16"
 #endif
-#define TM 256
-#define TN 256
+#ifndef TILE
+#define TILE 256
+#endif
+#ifndef NBUF
+#define NBUF 2
+#endif
+#define TM TILE
+#define TN TILE
 #define KS 64
 #define STAGE_BYTES ((TM + TN) * 128)
 #define NTHR 256
+#define FR (TILE / 64)          // 32 x 32 accumulator tiles per wave along each axis
+#define NM (FR * FR)            // MFMAs of a k-step
+#define WT (TILE / 2)           // rows and columns of C per wave
+#define CPW (TILE / 32)         // 1 KB copies per wave, operand and stage
+#define ROWB (TILE * 2)         // bytes of a k-row of an operand staged with m or n innermost
+#define RPI (1024 / ROWB)       // k-rows of such an operand per copy
+#define PPR (ROWB / 16)         // 16-byte pieces of such a k-row
 
 template <int V> struct mjt_ic { static constexpr int v = V; };
 template <int I, int N, class F> __device__ __forceinline__ void mjt_static_for(F&& f) {
@@ -81,7 +94,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     const long long lda = (long long)p.a[6], ldb = (long long)p.a[7], ldc = (long long)p.a[8];
     const unsigned short* __restrict__ A = (const unsigned short*)p.a[0] + (long long)blockIdx.y * (long long)p.a[9];
     const unsigned short* __restrict__ B = (const unsigned short*)p.a[1] + (long long)blockIdx.y * (long long)p.a[10];
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE_BYTES];
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NBUF * STAGE_BYTES];
 
     // Tile order: panels of 4 tile rows, inside a panel column by column.  Workgroups go round-robin over the
     // 8 XCDs, so workgroup id takes tile (id % 8) * per_xcd + id / 8: every XCD works on a compact run of
@@ -117,13 +130,14 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // k-row r sits at position u ^ (r % 4).  Its descriptor starts at the tile's first column and ends with the operand,
     // so whatever lies past the matrix reads as zero; a stage adds 64 rows through the scalar offset.
     const int last_a = M - 1 - m0, last_b = N - 1 - n0;             // last valid row of the tile
-    unsigned voff_a[8], voff_b[8];
+    unsigned voff_a[CPW], voff_b[CPW];
 #pragma unroll
-    for (int q = 0; q < 8; q++) {
-        const int row = (wave * 8 + q) * 8 + (lane >> 3);
+    for (int q = 0; q < CPW; q++) {
+        const int row = (wave * CPW + q) * 8 + (lane >> 3);
         const unsigned chunk = (unsigned)((lane & 7) ^ ((row >> 1) & 7));
-        const int krow = (wave * 8 + q) * 2 + (lane >> 5);
-        const unsigned piece = (unsigned)(((((lane & 31) >> 1) ^ (krow & 3)) << 1) | (lane & 1));      // 16-byte piece of the k-row in memory
+        const int krow = (wave * CPW + q) * RPI + lane / PPR;
+        const int pl = lane % PPR;
+        const unsigned piece = (unsigned)((((pl >> 1) ^ (krow & 3)) << 1) | (pl & 1));                  // 16-byte piece of the k-row in memory
 #if A_KCONT
         voff_a[q] = (unsigned)(row < last_a ? row : last_a) * (unsigned)(lda * 2) + chunk * 16;
 #else
@@ -154,14 +168,14 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         constexpr int q = decltype(qc)::v;
         const int st = s < nstages ? s : nstages - 1;               // past the end: a stage nobody reads
         __attribute__((address_space(3))) unsigned char* dst =
-            (__attribute__((address_space(3))) unsigned char*)&lds[0] + slot * STAGE_BYTES + wave * 8192;
+            (__attribute__((address_space(3))) unsigned char*)&lds[0] + slot * STAGE_BYTES + wave * (CPW * 1024);
         // (an immediate offset would move the place in memory along with the place in LDS)
-        if constexpr (q < 8)
+        if constexpr (q < CPW)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void*)(dst + q * 1024), 16, (int)voff_a[q], st * a_step, 0, 0);
         else
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void*)(dst + TM * 128 + (q - 8) * 1024), 16, (int)voff_b[q - 8], st * b_step, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void*)(dst + TM * 128 + (q - CPW) * 1024), 16, (int)voff_b[q - CPW], st * b_step, 0, 0);
     };
-    auto copy_stage = [&](int s, int slot) { mjt_static_for<0, 16>([&](auto qc) { copy_one(qc, s, slot); }); };
+    auto copy_stage = [&](int s, int slot) { mjt_static_for<0, 2 * CPW>([&](auto qc) { copy_one(qc, s, slot); }); };
 
     // Fragments.  Lane (row = lane % 32, half = lane / 32) of v_mfma_f32_32x32x16 wants the 8 consecutive k of its row
     // and half.  From a [rows][64 k] tile that is one 16-byte read: row lane % 32 of each 32-row block of the wave's
@@ -174,21 +188,21 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     const unsigned lds_base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned char*)&lds[0];
     const int ti = lane & 15, tg = (lane >> 4) & 1, tk = lane >> 5;
 #if A_KCONT
-    const unsigned a_lane = lds_base + (unsigned)((wm * 128 + frow) * 128);
+    const unsigned a_lane = lds_base + (unsigned)((wm * WT + frow) * 128);
 #else
-    unsigned a_tr[4];
+    unsigned a_tr[FR];
 #pragma unroll
-    for (int f = 0; f < 4; f++) a_tr[f] = lds_base + (unsigned)((tk * 8 + (ti >> 2)) * 512 + (((wm * 8 + 2 * f + tg) ^ (ti >> 2)) * 32) + (ti & 3) * 8);
+    for (int f = 0; f < FR; f++) a_tr[f] = lds_base + (unsigned)((tk * 8 + (ti >> 2)) * ROWB + (((wm * (WT / 16) + 2 * f + tg) ^ (ti >> 2)) * 32) + (ti & 3) * 8);
 #endif
 #if B_KCONT
-    const unsigned b_lane = lds_base + (unsigned)(TM * 128 + (wn * 128 + frow) * 128);
+    const unsigned b_lane = lds_base + (unsigned)(TM * 128 + (wn * WT + frow) * 128);
 #else
-    unsigned b_tr[4];
+    unsigned b_tr[FR];
 #pragma unroll
-    for (int f = 0; f < 4; f++) b_tr[f] = lds_base + (unsigned)(TM * 128 + (tk * 8 + (ti >> 2)) * 512 + (((wn * 8 + 2 * f + tg) ^ (ti >> 2)) * 32) + (ti & 3) * 8);
+    for (int f = 0; f < FR; f++) b_tr[f] = lds_base + (unsigned)(TM * 128 + (tk * 8 + (ti >> 2)) * ROWB + (((wn * (WT / 16) + 2 * f + tg) ^ (ti >> 2)) * 32) + (ti & 3) * 8);
 #endif
-    mjt_u32x2 falo[2][4], fahi[2][4], fblo[2][4], fbhi[2][4];       // a fragment's four registers in two halves
-    constexpr int A_READS = A_KCONT ? 4 : 8, B_READS = B_KCONT ? 4 : 8, READS = A_READS + B_READS;
+    mjt_u32x2 falo[2][FR], fahi[2][FR], fblo[2][FR], fbhi[2][FR];       // a fragment's four registers in two halves
+    constexpr int A_READS = A_KCONT ? FR : 2 * FR, B_READS = B_KCONT ? FR : 2 * FR, READS = A_READS + B_READS;
     // read number r (0 .. READS-1) of the fragments of k-step kstep (compile-time) of the stage in slot, into set SET
     auto request_one = [&](auto setc, auto rc, int slot, auto kc) {
         constexpr int SET = decltype(setc)::v, r = decltype(rc)::v, kstep = decltype(kc)::v;
@@ -197,29 +211,29 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
 #if A_KCONT
             mjt_ds_read_pair<r * 4096>(falo[SET][r], fahi[SET][r], a_lane + soff + ((pos0 ^ (unsigned)(kstep * 2)) * 16));
 #else
-            if constexpr (r % 2 == 0) mjt_ds_read_tr<(kstep * 16) * 512>(falo[SET][r / 2], a_tr[r / 2] + soff);
-            else mjt_ds_read_tr<(kstep * 16 + 4) * 512>(fahi[SET][r / 2], a_tr[r / 2] + soff);
+            if constexpr (r % 2 == 0) mjt_ds_read_tr<(kstep * 16) * ROWB>(falo[SET][r / 2], a_tr[r / 2] + soff);
+            else mjt_ds_read_tr<(kstep * 16 + 4) * ROWB>(fahi[SET][r / 2], a_tr[r / 2] + soff);
 #endif
         } else {
             constexpr int rb = r - A_READS;
 #if B_KCONT
             mjt_ds_read_pair<rb * 4096>(fblo[SET][rb], fbhi[SET][rb], b_lane + soff + ((pos0 ^ (unsigned)(kstep * 2)) * 16));
 #else
-            if constexpr (rb % 2 == 0) mjt_ds_read_tr<(kstep * 16) * 512>(fblo[SET][rb / 2], b_tr[rb / 2] + soff);
-            else mjt_ds_read_tr<(kstep * 16 + 4) * 512>(fbhi[SET][rb / 2], b_tr[rb / 2] + soff);
+            if constexpr (rb % 2 == 0) mjt_ds_read_tr<(kstep * 16) * ROWB>(fblo[SET][rb / 2], b_tr[rb / 2] + soff);
+            else mjt_ds_read_tr<(kstep * 16 + 4) * ROWB>(fbhi[SET][rb / 2], b_tr[rb / 2] + soff);
 #endif
         }
     };
 
-    mjt_f32x16 acc[4][4];
+    mjt_f32x16 acc[FR][FR];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < FR; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < FR; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
     // the zeros are written here, not next to the first MFMA that reads them
-    mjt_static_for<0, 16>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / 4][decltype(ic)::v % 4]); });
+    mjt_static_for<0, NM>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / FR][decltype(ic)::v % FR]); });
     asm volatile("s_nop 7" : : : "memory");
 
     // A k-step: 16 MFMAs on the fragments of set SET.  What else the wave has to issue goes between them, one
@@ -228,22 +242,29 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     auto kstep = [&](auto setc, int rd_slot, auto rd_kstep, auto copyc, int cp_stage, int cp_slot) {
         constexpr int SET = decltype(setc)::v;
         constexpr bool COPY = decltype(copyc)::v != 0;
-        mjt_static_for<0, 16>([&](auto ic) {
+        constexpr int RPM = (READS + NM - 1) / NM, CPM = (2 * CPW + NM - 1) / NM;       // reads and copies behind one MFMA
+        mjt_static_for<0, NM>([&](auto ic) {
             constexpr int i = decltype(ic)::v;
-            mjt_mfma2(acc[i / 4][i % 4], falo[SET][i / 4], fahi[SET][i / 4], fblo[SET][i % 4], fbhi[SET][i % 4]);
-            if constexpr (i < READS) request_one(mjt_ic<SET ^ 1>(), ic, rd_slot, rd_kstep);
-            if constexpr (COPY) copy_one(ic, cp_stage, cp_slot);
+            mjt_mfma2(acc[i / FR][i % FR], falo[SET][i / FR], fahi[SET][i / FR], fblo[SET][i % FR], fbhi[SET][i % FR]);
+            mjt_static_for<0, RPM>([&](auto jc) {
+                constexpr int r = i * RPM + decltype(jc)::v;
+                if constexpr (r < READS) request_one(mjt_ic<SET ^ 1>(), mjt_ic<r>(), rd_slot, rd_kstep);
+            });
+            if constexpr (COPY)
+                mjt_static_for<0, CPM>([&](auto jc) {
+                    constexpr int q = i * CPM + decltype(jc)::v;
+                    if constexpr (q < 2 * CPW) copy_one(mjt_ic<q>(), cp_stage, cp_slot);
+                });
         });
     };
-    // stages 0 and 1 are asked for; stage 0 must have landed before the loop
-    copy_stage(0, 0);
-    copy_stage(1, 1);
-    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" : : : "memory");
+    // the first NBUF stages are asked for; stage 0 must have landed before the loop (a wave's copies land in order)
+    mjt_static_for<0, NBUF>([&](auto sc) { copy_stage(decltype(sc)::v, decltype(sc)::v); });
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"((NBUF - 1) * 2 * CPW) : "memory");
     mjt_static_for<0, READS>([&](auto rc) { request_one(mjt_ic<0>(), rc, 0, mjt_ic<0>()); });
 
 #pragma unroll 1
     for (int s = 0; s < nstages; s++) {
-        const int slot = s & 1;
+        const int slot = s & (NBUF - 1), next_slot = (s + 1) & (NBUF - 1);
         asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
         kstep(mjt_ic<0>(), slot, mjt_ic<1>(), mjt_ic<0>(), 0, 0);
         asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
@@ -252,16 +273,16 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         kstep(mjt_ic<0>(), slot, mjt_ic<3>(), mjt_ic<0>(), 0, 0);
         // Before the last k-step: its fragments are in registers, so nobody reads this stage's buffer any more once
         // every wave is here, and the copies of the next stage, asked for one stage ago, have landed.
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" : : : "memory");
-        kstep(mjt_ic<1>(), slot ^ 1, mjt_ic<0>(), mjt_ic<1>(), s + 2, slot);
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"((NBUF - 2) * 2 * CPW) : "memory");
+        kstep(mjt_ic<1>(), next_slot, mjt_ic<0>(), mjt_ic<1>(), s + NBUF, slot);
     }
     // The last MFMAs need time to read their operands and write their results; tie the registers to a point behind that.
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" : : : "memory");
-    mjt_static_for<0, 8>([&](auto ic) {
-        constexpr int st = decltype(ic)::v / 4, f = decltype(ic)::v % 4;
+    mjt_static_for<0, 2 * FR>([&](auto ic) {
+        constexpr int st = decltype(ic)::v / FR, f = decltype(ic)::v % FR;
         mjt_keep2(falo[st][f]); mjt_keep2(fahi[st][f]); mjt_keep2(fblo[st][f]); mjt_keep2(fbhi[st][f]);
     });
-    mjt_static_for<0, 16>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / 4][decltype(ic)::v % 4]); });
+    mjt_static_for<0, NM>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / FR][decltype(ic)::v % FR]); });
 
     // D of a 32x32 tile: lane holds column lane % 32, rows 8 * (e / 4) + 4 * (lane / 32) + e % 4
 #if OUT == 2
@@ -270,13 +291,13 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     unsigned short* __restrict__ C = (unsigned short*)p.a[2] + (long long)blockIdx.y * (long long)p.a[11];
 #endif
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < FR; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int col = n0 + wn * 128 + j * 32 + (lane & 31);
+        for (int j = 0; j < FR; j++) {
+            const int col = n0 + wn * WT + j * 32 + (lane & 31);
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                const int row = m0 + wm * 128 + i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e & 3);
+                const int row = m0 + wm * WT + i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e & 3);
                 if (row < M && col < N) {
                     const float v = acc[i][j][e];
 #if OUT == 2

@@ -65,23 +65,32 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
     auto fits32 = [&](bool kcont, int64_t ld) { return (kcont ? ld * 2 * 256 : ld * 2 * K) < (int64_t(1) << 31); };
     if (fast && allow_direct && esz == 2 && K % 64 == 0 && !getenv("MJT_GEMM_NO_DMA") && fits32(a_kcont, lda) && fits32(b_kcont, ldb)) {
         const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
-        const int64_t tm = (M + 255) / 256, tn = (N + 255) / 256;
-        const double edge = ((double)M * N) / ((double)tm * 256 * tn * 256);
-        const double tiles = (double)tm * tn * batch;
-        const double util = tiles / (std::ceil(tiles / cus) * cus);
-        if ((edge >= 0.85 && util >= 0.7) || getenv("MJT_GEMM_DMA")) {
+        // 256 x 256 tiles on two stage buffers, or 128 x 128 tiles on a ring of four (a 128-tile's stage is a quarter of
+        // the MFMA time, so more stages have to be on their way): the smaller tile where the larger one leaves compute
+        // units without work
+        int tile = 0;
+        for (int t = 256; t >= (tile_m || tile_n ? 256 : 128) && !tile; t /= 2) {       // a caller that names its tile has measured the general kernel
+            const int64_t tm = (M + t - 1) / t, tn = (N + t - 1) / t;
+            const double edge = ((double)M * N) / ((double)tm * t * tn * t);
+            const double tiles = (double)tm * tn * batch;
+            const double util = tiles / (std::ceil(tiles / cus) * cus);
+            if (edge >= 0.85 && util >= (t == 256 ? 0.7 : 0.25)) tile = t;
+        }
+        if (const char* e = getenv("MJT_GEMM_DMA")) tile = atoi(e) == 128 ? 128 : 256;
+        if (tile) {
+            const int64_t tm = (M + tile - 1) / tile, tn = (N + tile - 1) / tile;
             const int in = in_dtype == MJT_BFLOAT16 ? 0 : 1;
             const int out = out_dtype == MJT_BFLOAT16 ? 0 : out_dtype == MJT_FLOAT16 ? 1 : 2;
             std::ostringstream key;
-            key << "gemmd|" << in << out << a_kcont << b_kcont;
+            key << "gemmd|" << in << out << a_kcont << b_kcont << tile;
             JitKernel* k = cached(key.str());
             if (!k) {
                 std::ostringstream name;
-                name << "mjt_gemm_mfma_" << mjt_dtype_name(in_dtype) << "_" << mjt_dtype_name(out_dtype) << "_256x256" << (a_kcont ? "_n" : "_t")
+                name << "mjt_gemm_mfma_" << mjt_dtype_name(in_dtype) << "_" << mjt_dtype_name(out_dtype) << "_" << tile << "x" << tile << (a_kcont ? "_n" : "_t")
                      << (b_kcont ? "t" : "n") << "_direct";
                 std::ostringstream src;
                 src << "#define ENTRY " << name.str() << "\n#define IN " << in << "\n#define OUT " << out << "\n#define A_KCONT " << (a_kcont ? 1 : 0)
-                    << "\n#define B_KCONT " << (b_kcont ? 1 : 0) << "\n";
+                    << "\n#define B_KCONT " << (b_kcont ? 1 : 0) << "\n#define TILE " << tile << "\n#define NBUF " << (tile == 256 ? 2 : 4) << "\n";
                 src << embedded_source("gemm_dma.h") << "\n";
                 k = jit_get(src.str(), name.str());
                 remember(key.str(), k);

@@ -89,30 +89,33 @@ def test_gemm_mfma_layouts_and_edges(gpu, dt, ta, tb):
         assert _run(lib, dt, "float32", 304, 200, 136, ta, tb).startswith("mjt_gemm_mfma_")
 
 
+@pytest.mark.parametrize("tile", ["256", "128"])
 @pytest.mark.parametrize("dt", ["bfloat16", "float16"])
 @pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
-def test_gemm_direct_copy_kernel(gpu, dt, ta, tb, monkeypatch):
+def test_gemm_direct_copy_kernel(gpu, dt, ta, tb, tile, monkeypatch):
     """16-bit operands with K a multiple of 64 have a kernel of their own (operands go from memory to LDS without
     passing through registers; an operand whose memory has m or n innermost is read from LDS with transposing
-    reads) once there are enough 256 x 256 tiles; here it is asked for by name so that small shapes reach it too:
-    all four layouts, tiles that hang over both edges, a single stage (K = 64), many stages, a float32 result, a batch."""
+    reads) once there are enough 256 x 256 tiles (two stage buffers) or 128 x 128 tiles (a ring of four); here it is
+    asked for by name and tile so that small shapes reach it too: all four layouts, tiles that hang over both edges, fewer
+    stages than buffers (K = 64, 128, 192), many stages, a float32 result, a batch."""
     lib = L.load()
-    monkeypatch.setenv("MJT_GEMM_DMA", "1")
+    monkeypatch.setenv("MJT_GEMM_DMA", tile)
     for i, (M, K, N) in enumerate([(256, 64, 256), (512, 256, 256), (304, 128, 136), (1000, 192, 520), (8, 512, 8), (520, 2048, 264)]):
         kern = _run(lib, dt, dt, M, K, N, ta, tb, seed=20 + i)
-        assert kern.endswith("_direct"), kern
+        assert kern.endswith("%sx%s_%s%s_direct" % (tile, tile, "nt"[ta], "nt"[tb])), kern
     assert _run(lib, dt, "float32", 304, 128, 520, ta, tb, seed=30).endswith("_direct")
     assert _run(lib, dt, dt, 264, 64, 248, ta, tb, seed=31, batch=(3,)).endswith("_direct")
     # K = 96 is no multiple of 64: the general kernel
     assert not _run(lib, dt, dt, 256, 96, 256, ta, tb, seed=32).endswith("_direct")
 
 
-def test_gemm_direct_copy_kernel_random_shapes(gpu, monkeypatch):
+@pytest.mark.parametrize("tile", ["256", "128"])
+def test_gemm_direct_copy_kernel_random_shapes(gpu, tile, monkeypatch):
     """Seeded sweep over shapes, layouts, result types and batches for the direct-copy kernel: M and N anywhere
     between 1 and 700 (tiles cut on every side, operands whose last rows or columns end at the tensor's end),
     K a multiple of 64 up to 1024."""
     lib = L.load()
-    monkeypatch.setenv("MJT_GEMM_DMA", "1")
+    monkeypatch.setenv("MJT_GEMM_DMA", tile)
     rng = np.random.default_rng(2024)
     for i in range(24):
         M, N = int(rng.integers(1, 88)) * 8, int(rng.integers(1, 88)) * 8       # rows of 16-byte multiples in every layout
@@ -184,6 +187,16 @@ def test_gemm_is_the_meta_op_expression(gpu):
         for p in (pa, pb, pc):
             L.free(p)
     assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+
+
+def test_gemm_2048_runs_on_128_tiles_of_the_direct_copy_kernel(gpu):
+    """2048^3 has 64 tiles of 256 x 256 for 256 compute units: the direct-copy kernel takes it on 128 x 128 tiles (a ring
+    of four stages), in every layout; 1536^3 (144 such tiles) too; the whole result against float64."""
+    lib = L.load()
+    for ta, tb in ((0, 1), (0, 0), (1, 0), (1, 1)):
+        kern = _run(lib, "bfloat16", "bfloat16", 2048, 2048, 2048, ta, tb, seed=40 + 2 * ta + tb)
+        assert kern.endswith("128x128_%s%s_direct" % ("nt"[ta], "nt"[tb])), kern
+    assert _run(lib, "float16", "float32", 1536, 1536, 1536, 0, 1, seed=44).endswith("128x128_nt_direct")
 
 
 def test_gemm_full_size_4096_bf16_properties(gpu):
