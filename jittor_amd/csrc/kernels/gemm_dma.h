@@ -59,6 +59,8 @@ typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
 #define ROWB (TILE * 2)         // bytes of a k-row of an operand staged with m or n innermost
 #define RPI (1024 / ROWB)       // k-rows of such an operand per copy
 #define PPR (ROWB / 16)         // 16-byte pieces of such a k-row
+#define PFD (TILE == 256 ? 1 : 2)                   // how many k-steps ahead the fragments are read
+#define NSETS (PFD == 1 ? 2 : 4)                    // fragment sets
 
 template <int V> struct mjt_ic { static constexpr int v = V; };
 template <int I, int N, class F> __device__ __forceinline__ void mjt_static_for(F&& f) {
@@ -201,7 +203,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
     for (int f = 0; f < FR; f++) b_tr[f] = lds_base + (unsigned)(TM * 128 + (tk * 8 + (ti >> 2)) * ROWB + (((wn * (WT / 16) + 2 * f + tg) ^ (ti >> 2)) * 32) + (ti & 3) * 8);
 #endif
-    mjt_u32x2 falo[2][FR], fahi[2][FR], fblo[2][FR], fbhi[2][FR];       // a fragment's four registers in two halves
+    mjt_u32x2 falo[NSETS][FR], fahi[NSETS][FR], fblo[NSETS][FR], fbhi[NSETS][FR];       // a fragment's four registers in two halves
     constexpr int A_READS = A_KCONT ? FR : 2 * FR, B_READS = B_KCONT ? FR : 2 * FR, READS = A_READS + B_READS;
     // read number r (0 .. READS-1) of the fragments of k-step kstep (compile-time) of the stage in slot, into set SET
     auto request_one = [&](auto setc, auto rc, int slot, auto kc) {
@@ -236,49 +238,56 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     mjt_static_for<0, NM>([&](auto ic) { mjt_pin(acc[decltype(ic)::v / FR][decltype(ic)::v % FR]); });
     asm volatile("s_nop 7" : : : "memory");
 
-    // A k-step: 16 MFMAs on the fragments of set SET.  What else the wave has to issue goes between them, one
-    // instruction after each MFMA, where it costs no MFMA time (the wave is alone on its SIMD): the reads of the next
-    // k-step's fragments into the other set and, in the last k-step of a stage, the copies of the stage after the next.
-    auto kstep = [&](auto setc, int rd_slot, auto rd_kstep, auto copyc, int cp_stage, int cp_slot) {
-        constexpr int SET = decltype(setc)::v;
-        constexpr bool COPY = decltype(copyc)::v != 0;
-        constexpr int RPM = (READS + NM - 1) / NM, CPM = (2 * CPW + NM - 1) / NM;       // reads and copies behind one MFMA
+    // A k-step: NM MFMAs on the fragments of set SET.  What else the wave has to issue goes between them, behind the
+    // MFMAs, where it costs no MFMA time (the wave is alone on its SIMD): the reads of the fragments of the k-step PFD
+    // steps ahead into that step's set and, in the last PFD k-steps of a stage, the copies of the stage NBUF stages ahead
+    // (COPY0 .. COPY0 + COPYN - 1 of the wave's 2 CPW).  With 256 x 256 tiles a k-step is 16 MFMAs and hides the reads of
+    // the next one (PFD 1, two sets); the 4 MFMAs of a 128 x 128 tile's k-step do not, so there the reads run two k-steps
+    // ahead (PFD 2, a set per k-step of a stage) and a k-step waits for all but the latest READS of them.
+    auto kstep = [&](auto setc, auto rdsetc, int rd_slot, auto rd_kstep, auto copy0c, auto copync, int cp_stage, int cp_slot) {
+        constexpr int SET = decltype(setc)::v, RDSET = decltype(rdsetc)::v;
+        constexpr int COPY0 = decltype(copy0c)::v, COPYN = decltype(copync)::v;
+        constexpr int RPM = (READS + NM - 1) / NM, CPM = (COPYN + NM - 1) / NM;       // reads and copies behind one MFMA
         mjt_static_for<0, NM>([&](auto ic) {
             constexpr int i = decltype(ic)::v;
             mjt_mfma2(acc[i / FR][i % FR], falo[SET][i / FR], fahi[SET][i / FR], fblo[SET][i % FR], fbhi[SET][i % FR]);
             mjt_static_for<0, RPM>([&](auto jc) {
                 constexpr int r = i * RPM + decltype(jc)::v;
-                if constexpr (r < READS) request_one(mjt_ic<SET ^ 1>(), mjt_ic<r>(), rd_slot, rd_kstep);
+                if constexpr (r < READS) request_one(mjt_ic<RDSET>(), mjt_ic<r>(), rd_slot, rd_kstep);
             });
-            if constexpr (COPY)
-                mjt_static_for<0, CPM>([&](auto jc) {
-                    constexpr int q = i * CPM + decltype(jc)::v;
-                    if constexpr (q < 2 * CPW) copy_one(mjt_ic<q>(), cp_stage, cp_slot);
-                });
+            mjt_static_for<0, CPM>([&](auto jc) {
+                constexpr int q = i * CPM + decltype(jc)::v;
+                if constexpr (q < COPYN) copy_one(mjt_ic<COPY0 + q>(), cp_stage, cp_slot);
+            });
         });
     };
     // the first NBUF stages are asked for; stage 0 must have landed before the loop (a wave's copies land in order)
     mjt_static_for<0, NBUF>([&](auto sc) { copy_stage(decltype(sc)::v, decltype(sc)::v); });
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"((NBUF - 1) * 2 * CPW) : "memory");
-    mjt_static_for<0, READS>([&](auto rc) { request_one(mjt_ic<0>(), rc, 0, mjt_ic<0>()); });
+    mjt_static_for<0, PFD>([&](auto kc) {
+        mjt_static_for<0, READS>([&](auto rc) { request_one(kc, rc, 0, kc); });
+    });
 
 #pragma unroll 1
     for (int s = 0; s < nstages; s++) {
         const int slot = s & (NBUF - 1), next_slot = (s + 1) & (NBUF - 1);
-        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-        kstep(mjt_ic<0>(), slot, mjt_ic<1>(), mjt_ic<0>(), 0, 0);
-        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-        kstep(mjt_ic<1>(), slot, mjt_ic<2>(), mjt_ic<0>(), 0, 0);
-        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-        kstep(mjt_ic<0>(), slot, mjt_ic<3>(), mjt_ic<0>(), 0, 0);
-        // Before the last k-step: its fragments are in registers, so nobody reads this stage's buffer any more once
-        // every wave is here, and the copies of the next stage, asked for one stage ago, have landed.
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"((NBUF - 2) * 2 * CPW) : "memory");
-        kstep(mjt_ic<1>(), next_slot, mjt_ic<0>(), mjt_ic<1>(), s + NBUF, slot);
+        mjt_static_for<0, 4>([&](auto jc) {
+            constexpr int j = decltype(jc)::v, ahead = j + PFD;                 // this k-step, and the one whose fragments it asks for
+            constexpr int COPYN = j >= 4 - PFD ? 2 * CPW / PFD : 0, COPY0 = j >= 4 - PFD ? (j - (4 - PFD)) * COPYN : 0;
+            // Before the first k-step that reads the next stage (PFD steps before the stage's end): every fragment of
+            // this stage is in registers, so nobody reads its buffer any more once every wave is here, and the copies of
+            // the next stage, asked for NBUF - 1 stages ago, have landed.
+            if constexpr (j == 4 - PFD)
+                asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"((NBUF - 2) * 2 * CPW) : "memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(%0)" : : "n"((PFD - 1) * READS) : "memory");
+            kstep(mjt_ic<j % NSETS>(), mjt_ic<ahead % NSETS>(), ahead < 4 ? slot : next_slot, mjt_ic<ahead % 4>(), mjt_ic<COPY0>(), mjt_ic<COPYN>(),
+                  s + NBUF, slot);
+        });
     }
     // The last MFMAs need time to read their operands and write their results; tie the registers to a point behind that.
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" : : : "memory");
-    mjt_static_for<0, 2 * FR>([&](auto ic) {
+    mjt_static_for<0, NSETS * FR>([&](auto ic) {
         constexpr int st = decltype(ic)::v / FR, f = decltype(ic)::v % FR;
         mjt_keep2(falo[st][f]); mjt_keep2(fahi[st][f]); mjt_keep2(fblo[st][f]); mjt_keep2(fbhi[st][f]);
     });
