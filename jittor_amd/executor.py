@@ -19,7 +19,7 @@ from . import profiler as _profiler
 from .flags import flags
 
 stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0, "matmul_matches": 0,
-         "wgrad_kernel": 0, "gather_reduces": 0, "fused_scatters": 0}
+         "wgrad_kernel": 0, "gather_reduces": 0, "fused_scatters": 0, "plans": 0, "replays": 0}
 
 
 class ConvUnit:
@@ -445,13 +445,246 @@ def _match_matmul(red):
     return None
 
 
+# ---- replay of a graph that was executed before -----------------------------------------------------
+# The reference keeps what it worked out for a fused group and finds it again by the group's key
+# (executor.cc:55-110, load_fused_op and the jit cache behind it); a training step asks for the same graph every time.
+# Here the first execution of a graph records what it handed to the library: every call with its argument objects,
+# and for every pointer and by-value scalar inside them the var it came from.  A later graph with the same signature
+# (ops, their attributes, shapes, types, wiring, which results are asked for, flags) skips matching, partitioning and
+# descriptor building: its vars get their buffers the way the recorded run gave them out, the pointers and scalars
+# are written into the recorded argument objects, and the recorded calls are issued again.
+class _VarPtr(int):
+    """A device address that remembers the var (and the offset inside it) it was taken from."""
+
+    def __new__(cls, value, var, off=0):
+        o = int.__new__(cls, value)
+        o.var, o.off = var, off
+        return o
+
+    def __add__(self, n):
+        return _VarPtr(int(self) + n, self.var, self.off + n)
+
+    __radd__ = __add__
+
+
+class _Capture:
+    def __init__(self, lib):
+        self.lib = lib
+        self.calls = []          # (library function, argument tuple) of every call that succeeded
+        self.ptrs = []           # (struct or array, index or None, var, offset): a pointer field and where it came from
+        self.scalars = []        # (FusedVar array, index, var): a by-value scalar and the host var it came from
+
+    def __getattr__(self, name):                             # stands in for the library while recording
+        fn = getattr(self.lib, name)
+        if name == "mjt_matmul_available":
+            return fn
+
+        def call(*args):
+            rc = fn(*args)
+            if rc == 0:
+                self.calls.append((fn, args))
+            return rc
+        return call
+
+
+class _Plan:
+    __slots__ = ("slots", "needs_ptr", "produce", "ptrs", "scalars", "calls", "stats", "cleared")
+
+
+_cap = None
+_plans = {}
+_PLAN_LIMIT = 512
+
+
+def _libh():
+    return _cap if _cap is not None else _lib.ensure_init()
+
+
+def _op_sig(op):
+    if isinstance(op, (UnaryOp, BinaryOp)):
+        return (op.kind, op.op)
+    if isinstance(op, TernaryOp):
+        return (op.kind,)
+    if isinstance(op, BroadcastOp):
+        return (op.kind, op.bcast_mask, op.keepdims_mask)
+    if isinstance(op, ReduceOp):
+        return (op.kind, op.op, op.reduce_mask, op.keepdims_mask)
+    if isinstance(op, ReindexOp):
+        return (op.kind, tuple(op.indexes), op.overflow_value, tuple(op.overflow_conditions), getattr(op, "same_memory", False))
+    if isinstance(op, ReindexReduceOp):
+        return (op.kind, op.op, tuple(op.indexes), tuple(op.overflow_conditions))
+    return None
+
+
+def _signature(ops, target_ids):
+    """Hashable description of everything the execution of `ops` depends on besides the data, or None."""
+    pos, leaf, parts = {}, {}, []
+    for i, op in enumerate(ops):
+        sig = _op_sig(op)
+        out = op.out
+        if sig is None or out is None:
+            return None
+        ins = []
+        for u in op.inputs:
+            k = pos.get(u.id)
+            if k is not None:
+                ins.append(k)
+                continue
+            l = leaf.get(u.id)
+            if l is None:
+                l = leaf[u.id] = len(leaf)
+                ins.append((l, tuple(u.shape), u.dtype, u._op is None, u._buf is None, u._host is not None,
+                            getattr(u, "_stop_fuse", False)))
+            else:
+                ins.append(-1 - l)
+        pos[out.id] = i
+        parts.append((sig, tuple(out.shape), out.dtype, out.id in target_ids, out._buf is None, getattr(out, "_stop_fuse", False),
+                      tuple(ins)))
+    return (tuple(parts), tuple(sorted((k, str(v)) for k, v in flags.items())), dt_amp())
+
+
+def dt_amp():
+    from . import dtypes
+    return dtypes.amp_reg
+
+
+def _capture(ops, target_ids, sig):
+    """Executes `ops` and records the execution as a plan under `sig` (or marks the signature as not replayable)."""
+    global _cap
+    # a var's place in the graph: result of op i, or input j of op i (the first place it is seen at)
+    slot_of, slots, held = {}, [], []
+    made = {op.out.id for op in ops}
+    for i, op in enumerate(ops):
+        for j, u in enumerate(op.inputs):
+            if u.id not in made and id(u) not in slot_of:
+                slot_of[id(u)] = len(slots)
+                slots.append(("in", i, j))
+                held.append(u)
+        slot_of[id(op.out)] = len(slots)
+        slots.append(("out", i))
+        held.append(op.out)
+    had_inputs = [bool(op.inputs) for op in ops]
+    before = dict(stats)
+    cap = _cap = _Capture(_lib.ensure_init())
+    try:
+        _execute(ops, target_ids)
+    finally:
+        _cap = None
+    plan = _Plan()
+    # vars made during the execution (rearranged weights, column matrices, partial sums): a buffer of their own per replay
+    def slot(v):
+        k = slot_of.get(id(v))
+        if k is None:
+            if v._buf is None:
+                return None
+            k = slot_of[id(v)] = len(slots)
+            slots.append(("tmp", v._buf.size))
+            held.append(v)
+        return k
+    plan.ptrs, plan.scalars, needs_ptr = [], [], set()
+    for obj, idx, v, off in cap.ptrs:
+        k = slot(v)
+        if k is None:
+            _plans[sig] = False
+            return
+        plan.ptrs.append((obj, idx, k, off))
+        needs_ptr.add(k)
+    for arr, idx, v in cap.scalars:
+        k = slot_of.get(id(v))
+        if k is None or slots[k][0] != "in":
+            _plans[sig] = False
+            return
+        plan.scalars.append((arr, idx, k))
+    # who owns which buffer: inputs first, then the vars made on the way, then the results in the order of the ops
+    owner, produce = {}, []
+    for k, d in enumerate(slots):
+        if d[0] != "out" and held[k]._buf is not None:
+            owner.setdefault(id(held[k]._buf), k)
+    for k, d in enumerate(slots):
+        if d[0] != "out":
+            continue
+        buf = held[k]._buf
+        if buf is None:
+            continue
+        src = owner.get(id(buf))
+        if src is None:
+            owner[id(buf)] = k
+            produce.append((k, -1))
+        else:
+            produce.append((k, src))
+            needs_ptr.add(src)
+    plan.slots, plan.needs_ptr, plan.produce, plan.calls = slots, needs_ptr, produce, cap.calls
+    plan.stats = [(key, stats[key] - before[key]) for key in stats if stats[key] != before[key]]
+    plan.cleared = [(i, had_inputs[i] and not op.inputs) for i, op in enumerate(ops) if op.out is not None and op.out._op is None]
+    if len(_plans) >= _PLAN_LIMIT:
+        _plans.clear()
+    _plans[sig] = plan
+    stats["plans"] += 1
+
+
+def _replay(plan, ops):
+    slots = plan.slots
+    n = len(slots)
+    var, buf, base = [None] * n, [None] * n, [0] * n
+    needs_ptr = plan.needs_ptr
+    for k, d in enumerate(slots):
+        kind = d[0]
+        if kind == "in":
+            v = var[k] = ops[d[1]].inputs[d[2]]
+            if k in needs_ptr:
+                base[k] = v._device_ptr()
+                buf[k] = v._buf
+        elif kind == "out":
+            var[k] = ops[d[1]].out
+        else:
+            b = buf[k] = Buffer(d[1])
+            base[k] = b.ptr
+    for k, src in plan.produce:
+        v = var[k]
+        if src >= 0:
+            v._buf = buf[src]
+        elif v._buf is None:
+            v._buf = Buffer(max(v.nbytes, 1))
+        buf[k] = v._buf
+        base[k] = v._buf.ptr
+    for obj, idx, k, off in plan.ptrs:
+        if idx is None:
+            obj.ptr = base[k] + off
+        else:
+            obj[idx].ptr = base[k] + off
+    for arr, idx, k in plan.scalars:
+        fv = arr[idx]
+        fv.fvalue, fv.ivalue = _scalar_value(var[k])
+    check = _lib.check
+    for fn, args in plan.calls:
+        rc = fn(*args)
+        if rc:
+            check(rc)
+    for key, d in plan.stats:
+        stats[key] += d
+    for i, clear_inputs in plan.cleared:
+        op = ops[i]
+        op.out._op = None
+        if clear_inputs:
+            op.inputs = []
+    stats["replays"] += 1
+
+
 def run_sync(targets, device_sync=False):
     targets = [t for t in targets if isinstance(t, Var)]
     stats["syncs"] += 1
     _lib.ensure_init()
     ops = _pending_ops(targets)
     if ops:
-        _execute(ops, {t.id for t in targets})
+        target_ids = {t.id for t in targets}
+        sig = _signature(ops, target_ids) if flags["enable_replay"] and _cap is None and _profiler.active() is None else None
+        plan = _plans.get(sig) if sig is not None else False
+        if plan is None:
+            _capture(ops, target_ids, sig)
+        elif plan is False:
+            _execute(ops, target_ids)
+        else:
+            _replay(plan, ops)
     for t in targets:
         t._device_ptr()
     if device_sync:
@@ -752,21 +985,50 @@ def _execute(ops, target_ids):
 def _alloc_out(v):
     if v._buf is None:
         v._buf = Buffer(max(v.nbytes, 1))
-    return v._buf.ptr
+    return v._buf.ptr if _cap is None else _VarPtr(v._buf.ptr, v)
+
+
+def _ptr_of(v):
+    p = v._device_ptr()
+    return p if _cap is None else _VarPtr(p, v)
+
+
+def _tensor(ptr, dtype, shape):
+    t = _lib.tensor(ptr, dtype, shape)
+    if _cap is not None and isinstance(ptr, _VarPtr):
+        _cap.ptrs.append((t, None, ptr.var, ptr.off))
+    return t
 
 
 def _tensor_of(v):
-    return _lib.tensor(v._device_ptr(), v.dtype, v.shape)
+    return _tensor(_ptr_of(v), v.dtype, v.shape)
+
+
+def _tensor_array(vs):
+    arr = (_lib.Tensor * max(1, len(vs)))(*[_lib.tensor(v._device_ptr(), v.dtype, v.shape) for v in vs])
+    if _cap is not None:
+        for i, v in enumerate(vs):
+            _cap.ptrs.append((arr, i, v, 0))
+    return arr
+
+
+def _scalar_value(u):
+    """(fvalue, ivalue) of a one-element host array that goes into a kernel by value (ops/array_op.cc:56-60)"""
+    if u.dtype == "bfloat16":
+        from .dtypes import bf16_bits_to_f32
+        return float(bf16_bits_to_f32(u._host).reshape(-1)[0]), 0
+    h = u._host.reshape(-1)[0]
+    return (float(h), 0) if u.is_float() else (0.0, int(h))
 
 
 def _run_single(op):
-    lib = _lib.ensure_init()
+    lib = _libh()
     out = op.out
     stats["launches"] += 1
     if isinstance(op, ReduceOp):
         x = op.inputs[0]
         tx = _tensor_of(x)
-        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        ty = _tensor(_alloc_out(out), out.dtype, out.shape)
         _lib.check(lib.mjt_reduce(ctypes.byref(tx), ctypes.byref(ty), _lib.OP_CODE[op.op], op.reduce_mask))
     elif isinstance(op, ReindexOp):
         x, extras = op.inputs[0], op.inputs[1:]
@@ -776,23 +1038,23 @@ def _run_single(op):
             stats["launches"] -= 1
             return
         tx = _tensor_of(x)
-        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
-        ex = (_lib.Tensor * max(1, len(extras)))(*[_tensor_of(e) for e in extras])
+        ty = _tensor(_alloc_out(out), out.dtype, out.shape)
+        ex = _tensor_array(extras)
         _lib.check(lib.mjt_reindex(ctypes.byref(tx), ctypes.byref(ty), len(op.indexes), _lib.c_strings(op.indexes),
                                    op.overflow_value, len(op.overflow_conditions),
                                    _lib.c_strings(op.overflow_conditions), len(extras), ex))
     elif isinstance(op, ReindexReduceOp):
         y, extras = op.inputs[0], op.inputs[1:]
         ty = _tensor_of(y)
-        tx = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
-        ex = (_lib.Tensor * max(1, len(extras)))(*[_tensor_of(e) for e in extras])
+        tx = _tensor(_alloc_out(out), out.dtype, out.shape)
+        ex = _tensor_array(extras)
         _lib.check(lib.mjt_reindex_reduce(ctypes.byref(ty), ctypes.byref(tx), _lib.OP_CODE[op.op], len(op.indexes),
                                           _lib.c_strings(op.indexes), len(op.overflow_conditions),
                                           _lib.c_strings(op.overflow_conditions), len(extras), ex))
     elif isinstance(op, ConvUnit):
         x, w = op.inputs
         tx, tw = _tensor_of(x), _tensor_of(w)
-        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        ty = _tensor(_alloc_out(out), out.dtype, out.shape)
         p = _lib.ConvParams(*op.params)
         if op.groups > 1:
             _lib.check(lib.mjt_conv2d_meta_grouped(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p),
@@ -803,9 +1065,9 @@ def _run_single(op):
         ro = op.reindex
         x, extras = ro.inputs[0], ro.inputs[1:]
         tx = _tensor_of(x)
-        ts = _lib.tensor(0, x.dtype, ro.out.shape)                       # the reindex result: its shape only
-        tz = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
-        ex = (_lib.Tensor * max(1, len(extras)))(*[_tensor_of(e) for e in extras])
+        ts = _tensor(0, x.dtype, ro.out.shape)                       # the reindex result: its shape only
+        tz = _tensor(_alloc_out(out), out.dtype, out.shape)
+        ex = _tensor_array(extras)
         _lib.check(lib.mjt_reindex_then_reduce(ctypes.byref(tx), ctypes.byref(ts), ctypes.byref(tz), _lib.OP_CODE[op.op], op.nred,
                                                len(ro.indexes), _lib.c_strings(ro.indexes), ro.overflow_value,
                                                len(ro.overflow_conditions), _lib.c_strings(ro.overflow_conditions),
@@ -816,7 +1078,7 @@ def _run_single(op):
         k = b.shape[-2] if op.trans[1] else b.shape[-1]
         ta, tb = _tensor_of(a), _tensor_of(b)
         # a kept reduced axis of extent 1 changes nothing in memory
-        tc = _lib.tensor(_alloc_out(out), out.dtype, list(a.shape[:-2]) + [n, k])
+        tc = _tensor(_alloc_out(out), out.dtype, list(a.shape[:-2]) + [n, k])
         _lib.check(lib.mjt_matmul(ctypes.byref(ta), ctypes.byref(tb), ctypes.byref(tc), int(op.trans[0]), int(op.trans[1])))
     elif isinstance(op, ConvBwdDataUnit):
         dy, w = op.inputs
@@ -826,7 +1088,7 @@ def _run_single(op):
         if G == 1:
             # the library's own entry: transposed, flipped weights for stride 1, one convolution per stride phase otherwise
             td, tw = _tensor_of(dy), _tensor_of(w)
-            tx = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+            tx = _tensor(_alloc_out(out), out.dtype, out.shape)
             p = _lib.ConvParams(sh, sw, ph, pw, dh, dw)
             _lib.check(lib.mjt_conv2d_meta_dgrad(ctypes.byref(td), ctypes.byref(tw), ctypes.byref(tx), ctypes.byref(p)))
             return
@@ -847,7 +1109,7 @@ def _run_single(op):
                                   ["i0", "i1", "i2/%d" % sh, "i3/%d" % sw], 0.0, ["i2%%%d!=0" % sh, "i3%%%d!=0" % sw])
             _run_single(dy._op)
         tx, tw = _tensor_of(dy), _tensor_of(wt)
-        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        ty = _tensor(_alloc_out(out), out.dtype, out.shape)
         p = _lib.ConvParams(1, 1, dh * (R - 1) - ph, dw * (S - 1) - pw, dh, dw)
         if G > 1:
             _lib.check(lib.mjt_conv2d_meta_grouped(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(ty), ctypes.byref(p), G))
@@ -856,7 +1118,7 @@ def _run_single(op):
     elif isinstance(op, ConvBwdWeightUnit) and op.groups > 1:
         x, dy = op.inputs
         tx, td = _tensor_of(x), _tensor_of(dy)
-        tw = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        tw = _tensor(_alloc_out(out), out.dtype, out.shape)
         p = _lib.ConvParams(*op.params)
         _lib.check(lib.mjt_conv2d_meta_wgrad_grouped(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p), op.groups))
     elif isinstance(op, ConvBwdWeightUnit):
@@ -868,7 +1130,7 @@ def _run_single(op):
         if x.dtype in ("bfloat16", "float16") and flags["enable_conv_wgrad_kernel"]:
             # the MFMA kernel; shapes it does not cover come back as unsupported and take the paths below
             tx, td = _tensor_of(x), _tensor_of(dy)
-            tw = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+            tw = _tensor(_alloc_out(out), out.dtype, out.shape)
             p = _lib.ConvParams(sh, sw, ph, pw, dh, dw)
             rc = lib.mjt_conv2d_meta_wgrad(ctypes.byref(tx), ctypes.byref(td), ctypes.byref(tw), ctypes.byref(p))
             if rc == 0:
@@ -894,17 +1156,17 @@ def _run_single(op):
             psz = _lib.DTYPE_SIZE[pdt]
             for n0 in range(0, N, chunk):
                 nb = min(chunk, N - n0)
-                tx = _lib.tensor(x._device_ptr() + n0 * C * H * W * esz, x.dtype, [nb, C, H, W])
-                tc = _lib.tensor(cols_ptr, x.dtype, [nb, C, R, S, OH, OW])
+                tx = _tensor(_ptr_of(x) + n0 * C * H * W * esz, x.dtype, [nb, C, H, W])
+                tc = _tensor(cols_ptr, x.dtype, [nb, C, R, S, OH, OW])
                 _lib.check(lib.mjt_reindex(ctypes.byref(tx), ctypes.byref(tc), 4, idx, 0.0, 0, none, 0, ex))
-                ta = _lib.tensor(dy._device_ptr() + n0 * K * P * esz, dy.dtype, [nb, K, P])
-                tb = _lib.tensor(cols_ptr, x.dtype, [nb, CRS, P])
-                tp = _lib.tensor(part_ptr + n0 * K * CRS * psz, pdt, [nb, K, CRS])
+                ta = _tensor(_ptr_of(dy) + n0 * K * P * esz, dy.dtype, [nb, K, P])
+                tb = _tensor(cols_ptr, x.dtype, [nb, CRS, P])
+                tp = _tensor(part_ptr + n0 * K * CRS * psz, pdt, [nb, K, CRS])
                 _lib.check(lib.mjt_matmul(ctypes.byref(ta), ctypes.byref(tb), ctypes.byref(tp), 0, 1))
                 stats["launches"] += 2
             acc = out if out.dtype == pdt else Var([K, C, R, S], pdt)
-            tpart = _lib.tensor(part_ptr, pdt, [N, K * CRS])
-            tacc = _lib.tensor(_alloc_out(acc), pdt, [K * CRS])
+            tpart = _tensor(part_ptr, pdt, [N, K * CRS])
+            tacc = _tensor(_alloc_out(acc), pdt, [K * CRS])
             _lib.check(lib.mjt_reduce(ctypes.byref(tpart), ctypes.byref(tacc), _lib.OP_CODE["add"], 0b01))
             if acc is not out:                                 # narrow the float32 sum to the weights' dtype
                 with core.no_grad():
@@ -921,10 +1183,10 @@ def _run_single(op):
         # the stride never reaches make its output larger than R x S: the reindex below keeps the first R x S taps
         tmp = Var([C, K, (H + 2 * ph - sh * (OH - 1) - 1) // dh + 1, (W + 2 * pw - sw * (OW - 1) - 1) // dw + 1], out.dtype)
         tx, tw = _tensor_of(xt), _tensor_of(dyt)
-        tt = _lib.tensor(_alloc_out(tmp), tmp.dtype, tmp.shape)
+        tt = _tensor(_alloc_out(tmp), tmp.dtype, tmp.shape)
         p = _lib.ConvParams(dh, dw, ph, pw, sh, sw)              # stride and dilation trade places
         _lib.check(lib.mjt_conv2d_meta(ctypes.byref(tx), ctypes.byref(tw), ctypes.byref(tt), ctypes.byref(p)))
-        ty = _lib.tensor(_alloc_out(out), out.dtype, out.shape)
+        ty = _tensor(_alloc_out(out), out.dtype, out.shape)
         idx, none = _lib.c_strings(["i1", "i0", "i2", "i3"]), _lib.c_strings([])
         ex = (_lib.Tensor * 1)()
         _lib.check(lib.mjt_reindex(ctypes.byref(tt), ctypes.byref(ty), 4, idx, 0.0, 0, none, 0, ex))
@@ -936,18 +1198,20 @@ def _run_group(members, consumers, target_ids, reduce=None, pre=None, scatter=No
     """One launch for a group of element / broadcast ops.  With `reduce` (the ReduceOp that consumes the
     group's only result) the group runs as that reduce's prologue; returns False when the library does
     not take the group in that form (a tensor broadcast inside it), True otherwise."""
-    lib = _lib.ensure_init()
+    lib = _libh()
     member_ids = {op.id for op in members}
     shape = members[-1].out.shape
-    fvars, fops = [], []
+    fvars, fops, prov = [], [], []
     index = {}           # (var id, bcast mask) -> fused var index
     keep = []            # keeps arrays alive
 
-    def add_var(role, dtype, ptr=None, fvalue=0.0, ivalue=0, mask=0):
+    def add_var(role, dtype, ptr=None, fvalue=0.0, ivalue=0, mask=0, scalar=None):
         fv = _lib.FusedVar()
         fv.role, fv.dtype, fv.ptr = role, _lib.DTYPE_CODE[dtype], ptr
         fv.fvalue, fv.ivalue, fv.bcast_mask = float(fvalue), int(ivalue), mask
         fvars.append(fv)
+        if _cap is not None:                                  # where the pointer / the value came from, for replays
+            prov.append((len(fvars) - 1, ptr.var, ptr.off) if isinstance(ptr, _VarPtr) else (len(fvars) - 1, scalar, None) if scalar is not None else None)
         return len(fvars) - 1
 
     def external(u, mask):
@@ -955,22 +1219,15 @@ def _run_group(members, consumers, target_ids, reduce=None, pre=None, scatter=No
         if key in index:
             return index[key]
         if gathered and u.id in gathered:
-            i = add_var(_lib.VAR_GATHERED, u.dtype, ptr=gathered[u.id].inputs[0]._device_ptr())
+            i = add_var(_lib.VAR_GATHERED, u.dtype, ptr=_ptr_of(gathered[u.id].inputs[0]))
             index[key] = i
             return i
         if u._op is None and u._host is not None and u.num == 1:
             # one-element host array: by-value kernel argument (ops/array_op.cc:56-60)
-            h = u._host.reshape(-1)[0]
-            if u.dtype == "bfloat16":
-                from .dtypes import bf16_bits_to_f32
-                val = float(bf16_bits_to_f32(u._host).reshape(-1)[0])
-                i = add_var(_lib.VAR_SCALAR, u.dtype, fvalue=val)
-            elif u.is_float():
-                i = add_var(_lib.VAR_SCALAR, u.dtype, fvalue=float(h))
-            else:
-                i = add_var(_lib.VAR_SCALAR, u.dtype, ivalue=int(h))
+            fval, ival = _scalar_value(u)
+            i = add_var(_lib.VAR_SCALAR, u.dtype, fvalue=fval, ivalue=ival, scalar=u)
         else:
-            i = add_var(_lib.VAR_INPUT, u.dtype, ptr=u._device_ptr(), mask=mask)
+            i = add_var(_lib.VAR_INPUT, u.dtype, ptr=_ptr_of(u), mask=mask)
         index[key] = i
         return i
 
@@ -1032,11 +1289,17 @@ def _run_group(members, consumers, target_ids, reduce=None, pre=None, scatter=No
     varr = (_lib.FusedVar * len(fvars))(*fvars)
     oarr = (_lib.FusedOp * len(fops))(*fops)
     desc.n_vars, desc.vars, desc.n_ops, desc.ops = len(fvars), varr, len(fops), oarr
+    if _cap is not None:
+        for pv in prov:
+            if pv is not None and pv[2] is not None:
+                _cap.ptrs.append((varr, pv[0], pv[1], pv[2]))
+            elif pv is not None:
+                _cap.scalars.append((varr, pv[0], pv[1]))
     if scatter is not None:
         rout, extras = scatter.out, scatter.inputs[1:]
         had_buf = rout._buf is not None
-        tx = _lib.tensor(_alloc_out(rout), rout.dtype, rout.shape)
-        ex = (_lib.Tensor * max(1, len(extras)))(*[_tensor_of(e) for e in extras])
+        tx = _tensor(_alloc_out(rout), rout.dtype, rout.shape)
+        ex = _tensor_array(extras)
         rc = lib.mjt_fused_reindex_reduce(ctypes.byref(desc), ctypes.byref(tx), _lib.OP_CODE[scatter.op], len(scatter.indexes),
                                           _lib.c_strings(scatter.indexes), len(scatter.overflow_conditions),
                                           _lib.c_strings(scatter.overflow_conditions), len(extras), ex)
@@ -1051,7 +1314,7 @@ def _run_group(members, consumers, target_ids, reduce=None, pre=None, scatter=No
     if reduce is not None:
         rout = reduce.out
         had_buf = rout._buf is not None
-        ty = _lib.tensor(_alloc_out(rout), rout.dtype, rout.shape)
+        ty = _tensor(_alloc_out(rout), rout.dtype, rout.shape)
         rc = lib.mjt_fused_reduce(ctypes.byref(desc), ctypes.byref(ty), _lib.OP_CODE[reduce.op], reduce.reduce_mask)
         if rc == -2:                                   # MJT_ERR_UNSUPPORTED: run the two kernels instead
             if not had_buf:

@@ -46,7 +46,7 @@ class Flags(dict):
 
 flags = Flags()
 for _name, _value in (("enable_conv_match", True), ("enable_reduce_fusion", True), ("enable_broadcast_sink", True),
-                      ("enable_matmul_match", True), ("enable_conv_wgrad_kernel", True), ("enable_gather_reduce", True), ("enable_scatter_fusion", True), ("reshape_shares_memory", True), ("auto_mixed_precision_level", 0),
+                      ("enable_matmul_match", True), ("enable_conv_wgrad_kernel", True), ("enable_gather_reduce", True), ("enable_scatter_fusion", True), ("reshape_shares_memory", True), ("enable_replay", True), ("auto_mixed_precision_level", 0),
                       # default compile options of new vars (python/jittor/src/var.cc:19,75): a dict name -> int
                       ("compile_options", {})):
     dict.__setitem__(flags, _name, _value)
