@@ -554,6 +554,72 @@ def wl_gemm(L, lib, steps, warmup, with_cpu, trans_b=1):
     return out
 
 
+def wl_steps(L, lib, steps, warmup, with_cpu, which=("bottleneck_bf16", "small_cnn_f32")):
+    """Two training steps through the Python front end (graph construction, gradient graph, executor, library calls):
+    a ResNet-50 stage-1 bottleneck block at batch 64 in bfloat16 and a small float32 CNN, forward and every gradient,
+    with the executor's replay of a graph it has seen before switched off and on.  ms_per_step is host wall time per
+    step over `steps` steps issued back to back (best of 5 blocks); the kernels' own time is what
+    `rocprofv3 --kernel-trace --stats` sums for the same run over the steps_run of both modes (--only STEP_BOTTLENECK or
+    STEP_SMALL_CNN runs one of the two).  Not part of the default run (--only STEPS)."""
+    import jittor_amd as jt
+    from jittor_amd import executor
+    rng = np.random.default_rng(13)
+    bf = lambda a: jt.array(a.astype(np.float32)).bfloat16()
+    x = bf(rng.standard_normal((64, 256, 56, 56)))
+    w1, w2, w3 = bf(rng.standard_normal((64, 256, 1, 1)) * 0.05), bf(rng.standard_normal((64, 64, 3, 3)) * 0.05), bf(rng.standard_normal((256, 64, 1, 1)) * 0.05)
+    jt.sync([x, w1, w2, w3])
+
+    def bottleneck():
+        h = jt.nn.relu(jt.nn.conv2d(x, w1))
+        h = jt.nn.relu(jt.nn.conv2d(h, w2, padding=1))
+        h = jt.nn.conv2d(h, w3)
+        loss = jt.nn.relu(h + x).float32().sum()
+        jt.sync([loss] + jt.grad(loss, [x, w1, w2, w3]))
+
+    xs = rng.standard_normal((4, 8, 12, 12)).astype(np.float32)
+    v1, v2 = (rng.standard_normal((16, 8, 3, 3)) * 0.2).astype(np.float32), (rng.standard_normal((16, 16, 3, 3)) * 0.2).astype(np.float32)
+    wl, bl = (rng.standard_normal((5, 16)) * 0.3).astype(np.float32), rng.standard_normal(5).astype(np.float32)
+    onehot = np.eye(5, dtype=np.float32)[rng.integers(0, 5, 4)]
+
+    def small_cnn():
+        ax, a1, a2, al, ab = (jt.array(a) for a in (xs, v1, v2, wl, bl))
+        h = jt.nn.relu(jt.nn.conv2d(ax, a1, padding=1))
+        h = jt.nn.max_pool2d(h, 3, 2, 1)
+        h = jt.nn.relu(jt.nn.conv2d(h, a2, stride=2, padding=1))
+        logits = jt.nn.linear(h.mean([2, 3]), al, ab)
+        m = logits.max([1], keepdims=True)
+        logp = logits - m - jt.unary(jt.unary(logits - m, "exp").sum([1], keepdims=True), "log")
+        loss = (logp * jt.array(onehot)).sum() * (-1.0 / 4)
+        jt.sync([loss] + jt.grad(loss, [ax, a1, a2, al, ab]))
+
+    out = {}
+    saved = jt.flags["enable_replay"]
+    try:
+        for name, step in (("bottleneck_bf16", bottleneck), ("small_cnn_f32", small_cnn)):
+            if name not in which:
+                continue
+            for replay in (False, True):
+                jt.flags["enable_replay"] = replay
+                for i in range(max(warmup, 3)):
+                    step()
+                L.sync()
+                before = dict(executor.stats)
+                best = None
+                for block in range(5):
+                    t0 = time.perf_counter()
+                    for i in range(steps):
+                        step()
+                    L.sync()
+                    t = (time.perf_counter() - t0) * 1e3 / steps
+                    best = t if best is None else min(best, t)
+                out["%s_%s" % (name, "replay" if replay else "fresh")] = {
+                    "steps_run": max(warmup, 3) + 5 * steps, "ms_per_step": round(best, 4), "launches_per_step": (executor.stats["launches"] - before["launches"]) / (5.0 * steps),
+                    "replays_per_step": (executor.stats["replays"] - before["replays"]) / (5.0 * steps)}
+    finally:
+        jt.flags["enable_replay"] = saved
+    return {"workload": "STEPS", "cases": out}
+
+
 WORKLOADS = {
     "C1": wl_c1,
     "C2": wl_c2,
@@ -568,6 +634,9 @@ WORKLOADS = {
     "GEMMnn": lambda *a: wl_gemm(*a, trans_b=0),
     "COPY": wl_copy,
     "CALLERS": wl_callers,
+    "STEPS": wl_steps,
+    "STEP_BOTTLENECK": lambda *a: wl_steps(*a, which=("bottleneck_bf16",)),
+    "STEP_SMALL_CNN": lambda *a: wl_steps(*a, which=("small_cnn_f32",)),
 }
 DEFAULT = ["C1", "C2", "C3add", "C3max", "C4", "C5", "C5bf16out"]
 

@@ -112,10 +112,15 @@ class Op:
 
     def __init__(self, inputs):
         self.inputs = list(inputs)
-        for v in self.inputs:              # who reads a Var: Var.assign moves them to the old value
-            if v._consumers is None:
-                v._consumers = weakref.WeakSet()
-            v._consumers.add(self)
+        me = weakref.ref(self)
+        for v in self.inputs:              # who reads a Var (weakly): Var.assign moves them to the old value
+            lst = v._consumers
+            if lst is None:
+                v._consumers = [me]
+            else:
+                lst.append(me)
+                if len(lst) > 64 and len(lst) & (len(lst) - 1) == 0:     # a long-lived var (a weight): drop the dead readers now and then
+                    lst[:] = [r for r in lst if r() is not None]
         self.id = _new_id()
         self._out_ref = None
         self.amp = dt.amp_reg & 63          # the register at creation; its gradient is built under it (op.cc:38, grad.cc:48-55)
@@ -221,6 +226,10 @@ class Var:
             if s < 0:
                 raise ValueError("Shape should greater than 0: %r" % (shape,))
         self.shape = shape
+        n = 1
+        for e in shape:
+            n *= e
+        self._num = n
         self.dtype = dtype
         self._op = op
         if op is not None:
@@ -241,10 +250,7 @@ class Var:
     # ---- properties ----
     @property
     def num(self):
-        n = 1
-        for s in self.shape:
-            n *= s
-        return n
+        return self._num
 
     @property
     def ndim(self):
@@ -414,7 +420,10 @@ class Var:
         self._op = self._history = self._buf = self._host = None     # nothing left here until assign() fills it
         if old._op is not None:
             old._op.out = old
-        for op in list(old._consumers or ()):
+        for ref in list(old._consumers or ()):
+            op = ref()
+            if op is None:
+                continue
             op.inputs = [old if v is self else v for v in op.inputs]
             out = op.out
             if out is not None and out._history is not None:
