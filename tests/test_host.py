@@ -658,3 +658,69 @@ def test_grouped_conv_and_its_gradients_are_matched_by_role():
     a = jt.zeros([2, 2, 3, 2, 4, 4, 3, 3])
     z = (a * a).reindex_reduce("add", [2, 6, 4, 4], ["i0", "i1*3+i2", "i5", "i4"])
     assert E._match_conv_grouped(z._op) is None
+
+
+def test_executor_replays_a_graph_it_has_seen(compile_only, monkeypatch):
+    """The second execution of a graph with the same signature re-issues the recorded library calls: same number of calls
+    and the same counters, every pointer inside the recorded descriptors is the new graph's (input, result or a buffer
+    made on the way), a by-value scalar is the new graph's value, computed vars become leaves; another shape, another
+    wiring or a switched flag is another signature.  Compile-only mode with addresses handed out by a counter: no device."""
+    from jittor_amd import core, executor
+    nxt = [0x10000000]
+
+    def fake_alloc(nbytes):
+        size = core._Pool._round(nbytes)
+        nxt[0] += size
+        return nxt[0] - size, size
+
+    monkeypatch.setattr(core.pool, "alloc", fake_alloc)
+    monkeypatch.setattr(core.pool, "free", lambda ptr, size: None)
+    monkeypatch.setattr(L, "h2d", lambda ptr, arr: None)
+    monkeypatch.setitem(executor.flags, "enable_replay", True)
+    executor._plans.clear()
+
+    def step(lr, shape=(3, 6, 10, 10), twice=False):
+        x = jt.array(np.ones(shape, np.float32))
+        w = jt.array(np.ones((8, shape[1], 3, 3), np.float32))
+        y = jt.nn.conv2d(x, w, padding=1)
+        gw, = jt.grad((y * y).sum(), [w])                    # float32 weight gradient: column matrices and partial sums on the way
+        new_w = w - gw * jt.array(np.float32(lr))            # a by-value scalar
+        flat = jt.reshape(y, [shape[0], -1])                 # shares y's buffer
+        out = (flat + flat) if twice else (flat + 1.0)
+        before = dict(executor.stats)
+        jt.sync([new_w, out, y])
+        return {k: executor.stats[k] - before[k] for k in before}, (x, w, y, new_w, out, flat)
+
+    d1, keep1 = step(0.5)
+    assert d1["plans"] == 1 and d1["replays"] == 0
+    plan = next(iter(executor._plans.values()))
+    ncalls = len(plan.calls)
+    d2, keep2 = step(0.25)
+    assert d2["replays"] == 1 and d2["plans"] == 0
+    for k in d1:
+        if k not in ("plans", "replays"):
+            assert d1[k] == d2[k], k
+    assert len(plan.calls) == ncalls and ncalls == d1["launches"]
+    # every recorded pointer now points into a buffer of the second graph (or one made during the replay), none into the first's
+    x1, w1, y1, nw1, out1, flat1 = keep1
+    x2, w2, y2, nw2, out2, flat2 = keep2
+    first = {v._buf.ptr for v in keep1}
+    second = {v._buf.ptr for v in keep2}
+    assert not first & second and flat2._buf is y2._buf and flat1._buf is y1._buf
+    seen = set()
+    for obj, idx, slot, off in plan.ptrs:
+        ptr = (obj if idx is None else obj[idx]).ptr
+        assert ptr - off not in first
+        seen.add(ptr - off)
+    assert second - {flat2._buf.ptr} <= seen | {y2._buf.ptr}
+    assert all(v._op is None for v in (y2, nw2, out2))
+    vals = [arr[i].fvalue for arr, i, _ in plan.scalars]
+    assert 0.25 in vals and 0.5 not in vals
+    # other signatures: a shape, the wiring of a leaf, a flag
+    assert step(0.5, shape=(3, 6, 12, 10))[0]["plans"] == 1
+    assert step(0.5, twice=True)[0]["plans"] == 1
+    monkeypatch.setitem(executor.flags, "enable_reduce_fusion", False)
+    assert step(0.5)[0]["plans"] == 1
+    monkeypatch.setitem(executor.flags, "enable_replay", False)
+    d = step(0.5)[0]
+    assert d["plans"] == 0 and d["replays"] == 0
