@@ -91,7 +91,10 @@ __device__ __forceinline__ void mjt_pin(mjt_f32x16& x) { asm volatile("" : "+a"(
 
 struct Params { void* a[12]; };
 
-extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu(1, 1))) void ENTRY(Params p) {
+#ifndef WPE
+#define WPE 1                   // workgroups (of one wave per SIMD) a compute unit is meant to hold
+#endif
+extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu(1, WPE))) void ENTRY(Params p) {
     const int M = (int)(long long)p.a[3], N = (int)(long long)p.a[4], K = (int)(long long)p.a[5];
     const long long lda = (long long)p.a[6], ldb = (long long)p.a[7], ldc = (long long)p.a[8];
     const unsigned short* __restrict__ A = (const unsigned short*)p.a[0] + (long long)blockIdx.y * (long long)p.a[9];

@@ -384,15 +384,20 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             char* yn = (char*)y->ptr + n0 * K * P * dtype_size(y->dtype);
             // a short sum (a 1x1 convolution, few channels) is bound by how many workgroups a compute unit holds, not by
             // operand reuse: tiles of 128 x 128 (64 for at most 64 output channels or pixels, or when there would be fewer
-            // tiles than compute units), and the direct-copy kernel with its 256 x 256 tiles only from 256 summed elements on
-            // (16-bit operands; 64 x 512 x 28 x 28 -> 128 channels: 23 us against 48 with the tile the general rule picks;
-            // 64 x 64 x 56 x 56 -> 256: 45 against 54; 64 x 1024 x 28 x 28 -> 256: 63 against 113)
+            // tiles than compute units; at most 64 output channels with four or more 64 x 128 tiles per compute unit:
+            // 64 x 64), and the direct-copy kernel from two stages of the sum on, its 256 x 256 tiles from four
+            // (16-bit operands, us with / without the tile named here: 64 x 64 x 56 x 56 -> 256: 43 / 55;
+            // 64 x 512 x 28 x 28 -> 64: 19 / 37; 64 x 256 x 56 x 56 -> 64: 37 / 44 with 64 x 128;
+            // general kernel / direct-copy kernel on 128 x 128 tiles: 64 x 512 x 28 x 28 -> 128: 21.8 / 19.8; -> 512: 77 / 64;
+            // 64 x 256 x 56 x 56 -> 128: 56 / 47; 64 x 128 x 28 x 28 -> 512: 32 / 26)
             const bool short_sum = CRS <= 1024 && esz == 2 && !getenv("MJT_CONV_GEMM_NO_HINT");
             const int64_t cus = ctx().dry_run || ctx().prop.multiProcessorCount <= 0 ? 256 : ctx().prop.multiProcessorCount;
             const bool few = ((K + 127) / 128) * ((P + 127) / 128) * nb < cus;       // tiles of 128 x 128 would leave compute units idle
-            const int tile_m = !short_sum ? 0 : K <= 64 || few ? 64 : 128, tile_n = !short_sum ? 0 : P <= 64 || few ? 64 : 128;
+            const bool many = ((P + 127) / 128) * nb >= 4 * cus;                     // plenty of 64 x 128 tiles
+            const int tile_m = !short_sum ? 0 : K <= 64 || few ? 64 : 128;
+            const int tile_n = !short_sum ? 0 : P <= 64 || few || (K <= 64 && many) ? 64 : 128;
             gemm_launch(x->dtype, y->dtype, wmat, plain ? (void*)xn : cols, yn, K, P, CRS, lda, Ppad, P, 0, CRS * Ppad, K * P, nb, true, false,
-                        tile_m, tile_n, !short_sum || CRS >= 256);
+                        tile_m, tile_n, !short_sum || CRS >= 128);
         }
         set_last_kernel(plain ? "conv_as_gemm" : "conv_as_reindex_gemm");
         return;

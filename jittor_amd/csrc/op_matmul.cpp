@@ -69,28 +69,41 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
         // the MFMA time, so more stages have to be on their way): the smaller tile where the larger one leaves compute
         // units without work
         int tile = 0;
-        for (int t = 256; t >= (tile_m || tile_n ? 256 : 128) && !tile; t /= 2) {       // a caller that names its tile has measured the general kernel
+        // a caller that names its tile has measured the general kernel against the 256 x 256 tiles; 128 x 128 tiles of this
+        // kernel are still better than the general kernel's from two stages on (measured on 1x1 convolutions below)
+        const bool hinted = tile_m || tile_n;
+        const int smallest = hinted && !(tile_m == 128 && tile_n == 128 && K >= 128) ? 256 : 128;
+        for (int t = 256; t >= smallest && !tile; t /= 2) {
             const int64_t tm = (M + t - 1) / t, tn = (N + t - 1) / t;
             const double edge = ((double)M * N) / ((double)tm * t * tn * t);
             const double tiles = (double)tm * tn * batch;
             const double util = tiles / (std::ceil(tiles / cus) * cus);
-            if (edge >= 0.85 && util >= (t == 256 ? 0.7 : 0.25)) tile = t;
+            // (a sum of fewer than four stages does not fill the time a 256 x 256 tile's operands take to arrive, and only
+            // one such workgroup fits a compute unit)
+            if (edge >= 0.85 && util >= (t == 256 ? 0.7 : 0.25) && (t == 128 || K >= 256)) tile = t;
         }
         if (const char* e = getenv("MJT_GEMM_DMA")) tile = atoi(e) == 128 ? 128 : 256;
         if (tile) {
             const int64_t tm = (M + tile - 1) / tile, tn = (N + tile - 1) / tile;
             const int in = in_dtype == MJT_BFLOAT16 ? 0 : 1;
             const int out = out_dtype == MJT_BFLOAT16 ? 0 : out_dtype == MJT_FLOAT16 ? 1 : 2;
+            // a short sum on 128 x 128 tiles: two stage buffers, so that a compute unit holds two workgroups and one
+            // computes or stores while the other waits for its operands
+            // 128 x 128 tiles: with more tiles than compute units two stage buffers, so that a compute unit holds two
+            // workgroups and one computes or stores while the other waits for its operands (us, ring of four / two
+            // workgroups: 3072 x 3072 x 1024 35.4 / 31.7; 8192 x 1024 x 1024 26.8 / 22.1; 64 x 512 x 28 x 28 -> 512 as a
+            // product 82.3 / 63.7); with at most one tile each a ring of four (2048^3 21.7 / 24.8; 1536^3 15.3 / 20.5)
+            const int nbuf = tile == 256 ? 2 : (double)tm * tn * batch > (double)cus ? 2 : 4, wpe = tile == 128 && nbuf == 2 ? 2 : 1;
             std::ostringstream key;
-            key << "gemmd|" << in << out << a_kcont << b_kcont << tile;
+            key << "gemmd|" << in << out << a_kcont << b_kcont << tile << nbuf;
             JitKernel* k = cached(key.str());
             if (!k) {
                 std::ostringstream name;
                 name << "mjt_gemm_mfma_" << mjt_dtype_name(in_dtype) << "_" << mjt_dtype_name(out_dtype) << "_" << tile << "x" << tile << (a_kcont ? "_n" : "_t")
-                     << (b_kcont ? "t" : "n") << "_direct";
+                     << (b_kcont ? "t" : "n") << "_direct" << (wpe == 2 ? "2" : "");
                 std::ostringstream src;
                 src << "#define ENTRY " << name.str() << "\n#define IN " << in << "\n#define OUT " << out << "\n#define A_KCONT " << (a_kcont ? 1 : 0)
-                    << "\n#define B_KCONT " << (b_kcont ? 1 : 0) << "\n#define TILE " << tile << "\n#define NBUF " << (tile == 256 ? 2 : 4) << "\n";
+                    << "\n#define B_KCONT " << (b_kcont ? 1 : 0) << "\n#define TILE " << tile << "\n#define NBUF " << nbuf << "\n#define WPE " << wpe << "\n";
                 src << embedded_source("gemm_dma.h") << "\n";
                 k = jit_get(src.str(), name.str());
                 remember(key.str(), k);

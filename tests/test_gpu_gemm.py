@@ -199,6 +199,19 @@ def test_gemm_2048_runs_on_128_tiles_of_the_direct_copy_kernel(gpu):
     assert _run(lib, "float16", "float32", 1536, 1536, 1536, 0, 1, seed=44).endswith("128x128_nt_direct")
 
 
+def test_gemm_more_128_tiles_than_compute_units_run_two_workgroups_per_unit(gpu):
+    """With more 128 x 128 tiles than compute units (and too few 256 x 256 ones, or a sum too short for those) the
+    direct-copy kernel runs on two stage buffers, two workgroups per compute unit: every layout, one to five stages of
+    the sum, tiles hanging over both edges, a batch; the whole result against float64."""
+    lib = L.load()
+    for i, (ta, tb) in enumerate(((0, 1), (0, 0), (1, 0), (1, 1))):
+        kern = _run(lib, "bfloat16", "bfloat16", 2176, 128, 2120, ta, tb, seed=50 + i)
+        assert kern.endswith("128x128_%s%s_direct2" % ("nt"[ta], "nt"[tb])), kern
+    assert _run(lib, "float16", "float16", 2304, 320, 2200, 0, 1, seed=54).endswith("128x128_nt_direct2")
+    assert _run(lib, "bfloat16", "float32", 2304, 64, 2304, 1, 0, seed=55).endswith("128x128_tn_direct2")
+    assert _run(lib, "bfloat16", "bfloat16", 640, 192, 904, 0, 0, seed=56, batch=(9,)).endswith("128x128_nn_direct2")
+
+
 def test_gemm_full_size_4096_bf16_properties(gpu):
     """4096^3 in bfloat16 (the shape the throughput figure is quoted on): rows of the result against float64 on a
     sample, and linearity in b, which holds exactly for power-of-two factors."""
