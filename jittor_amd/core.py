@@ -222,13 +222,12 @@ class Var:
             shape = [1]
         if len(shape) > _lib.MAX_DIM:
             raise ValueError("at most %d dims are supported" % _lib.MAX_DIM)
-        for s in shape:
-            if s < 0:
-                raise ValueError("Shape should greater than 0: %r" % (shape,))
-        self.shape = shape
         n = 1
         for e in shape:
+            if e < 0:
+                raise ValueError("Shape should greater than 0: %r" % (shape,))
             n *= e
+        self.shape = shape
         self._num = n
         self.dtype = dtype
         self._op = op
@@ -245,7 +244,8 @@ class Var:
         self._name = None
         self._consumers = None   # ops that take this Var as an input (weakly)
         # compile options: the flag's value at creation (var.cc:75)
-        self._compile_options = dict(_flags["compile_options"]) if _flags["compile_options"] else None
+        co = dict.__getitem__(_flags, "compile_options")
+        self._compile_options = dict(co) if co else None
 
     # ---- properties ----
     @property
