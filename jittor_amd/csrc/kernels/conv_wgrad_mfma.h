@@ -46,6 +46,12 @@ typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
 
 struct Params { void* a[6]; };   // x, dy, partial, number of images, images per slice (typed as pointers: 8-byte words)
 
+// ABL (0 in production): timing-only ablations, results are wrong with any bit set.  1: the loads of dy fetch nothing
+// (offsets beyond the buffer: zeros, no memory traffic), 2: likewise the loads of x, 4: no MFMAs, 8: no fragment reads
+// from LDS, 16: no loads issued at all.
+#ifndef ABL
+#define ABL 0
+#endif
 #define TAPS (R_ * S_)
 #define NCHUNK ((OW_ + 31) / 32)
 #define CTW (8 / KG)
@@ -63,6 +69,19 @@ __device__ constexpr int mjt_col_shift(int s) { return s * DW - PW; }      // in
 __device__ constexpr bool mjt_edge(int ch, int s) {
     return ch * 32 + mjt_col_shift(s) < 0 || ch * 32 + 31 + mjt_col_shift(s) >= W_ || ch * 32 + 31 >= OW_;
 }
+
+typedef unsigned mjt_u32x2 __attribute__((ext_vector_type(2)));
+template <int OFF> __device__ __forceinline__ void mjt_ds_read128(mjt_u32x4v& dst, unsigned addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+__device__ __forceinline__ void mjt_no_mfma(mjt_f32x4& c, const mjt_u32x4v& a, const mjt_u32x4v& b) { asm volatile("" : "+v"(c) : "v"(a), "v"(b)); }
+__device__ __forceinline__ void mjt_pin_acc(mjt_f32x4& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void mjt_ds_read32(unsigned& dst, unsigned addr) { asm volatile("ds_read_b32 %0, %1" : "=v"(dst) : "v"(addr) : "memory"); }
+__device__ __forceinline__ void mjt_ds_read64(mjt_u32x2& dst, unsigned addr) { asm volatile("ds_read_b64 %0, %1" : "=v"(dst) : "v"(addr) : "memory"); }
+// wait until at most N LDS operations issued after the one that fills x are outstanding (the counter has four bits)
+template <int N> __device__ __forceinline__ void mjt_lds_wait(mjt_u32x4v& x) { asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N < 15 ? N : 15)); }
+template <int N> __device__ __forceinline__ void mjt_lds_wait1(unsigned& x) { asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N < 15 ? N : 15)); }
+template <int N> __device__ __forceinline__ void mjt_lds_wait2(mjt_u32x2& x) { asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N < 15 ? N : 15)); }
 
 extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     const int n_img = (int)(unsigned long long)p.a[3];
@@ -122,18 +141,22 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     // the fetch at byte 16 i) and, for each of its CTW channel tiles and each tap row, the 32 columns of the chunk of that
     // input row (1 KB, same order) plus the 4 columns after and the 2 before (16 B per channel: dwords right0, right1,
     // left, unused), from which the fragments of all tap columns are cut.
-    // Three areas when they fit (the loads of a step are then requested two steps ahead: memory latency under
-    // load is longer than one step), else two, else one.
+    // Four areas when they fit (the loads of a step are then requested three steps ahead: memory latency under load is
+    // longer than a step), else three, two, one.  A unit, what lies between two hand-over barriers, is one chunk.
     constexpr int NA = 4 * KG, NB = CTW * R_;
     constexpr int AREA_B = NA * 1024, AREA_X = AREA_B + NB * 1024, AREA = AREA_X + NB * 256;
-    // A unit is what lies between two barriers: a whole row of chunks when three units of that size fit, else a chunk.
-    constexpr int UNIT = NCHUNK <= 2 && 3 * NCHUNK * AREA <= 150 * 1024 ? NCHUNK : 1;
+    constexpr int UNIT = 1;
     constexpr int UAREA = UNIT * AREA;
-    constexpr int NBUF = 3 * UAREA <= 150 * 1024 ? 3 : 2 * UAREA <= 150 * 1024 ? 2 : 1;
+    constexpr int NBUF = 4 * UAREA <= 150 * 1024 ? 4 : 3 * UAREA <= 150 * 1024 ? 3 : 2 * UAREA <= 150 * 1024 ? 2 : 1;
+    // With three or more areas the two waves of a SIMD (wave w and w + 4) work in opposite phases: while one reads the
+    // fragments of a unit from LDS, the other runs the MFMAs of the unit before.  With every wave in the same phase a
+    // step was the sum of the two: all eight waves read (about 100 KB per chunk, LDS-bound), then all eight multiply.
+    constexpr bool SPLIT = NBUF >= 3;
     __shared__ __attribute__((aligned(16))) unsigned char stage[NBUF * UAREA];
     typedef __attribute__((address_space(3))) void* mjt_lds_ptr;
     // fragment order: lane (l16, lg) wants row l16, piece lg
     const int rd = (l16 * 4 + lg) * 16;
+    const unsigned stage_base = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned char*)&stage[0];
 
     mjt_f32x4 acc[4][TAPS];
 #pragma unroll
@@ -147,38 +170,86 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     // edge dwords: lane i fetches for channel i / 4 one of the two dwords right of the chunk (i % 4 = 0, 1) or the dword
     // left of it (i % 4 = 2); 16 B per channel: right0, right1, left, unused
     const unsigned e_lane = (unsigned)(frow * H_ * W_ * 2) + (fpiece == 2 ? (unsigned)-4 : (unsigned)(64 + 4 * fpiece));
-    auto fetch = [&](unsigned char* area, int img, int oh, int ch) -> int {
-        int issued = 0;                                                  // by this wave
-        const bool img_ok = img * OH_ + oh < row_end;
-#pragma unroll
-        for (int it0 = 0; it0 < NA + 2 * NB; it0 += 8) {
-            const int it = it0 + wave;
-            if (it < NA) {
-                const int kk = (kblock * KG + it / 4) * 64 + (it & 3) * 16;
-                const unsigned base = img_ok ? (unsigned)((((img * K_ + kk) * OH_ + oh) * OW_ + ch * 32) * 2) : 0u;
-                const unsigned flag = (img_ok ? 0u : INVALID) | (ch * 32 + fpiece * 8 < OW_ ? 0u : INVALID);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(y_rsrc, (mjt_lds_ptr)(area + it * 1024), 16, (int)((a_lane + base) | flag), 0, 0, 0);
-                issued++;
-            } else if (it < NA + 2 * NB) {
-                const bool edge = it >= NA + NB;
-                const int j = it - NA - (edge ? NB : 0);
-                const int tile = j / R_, r = j - tile * R_;
-                const int ih = oh * SH - PH + r * DH;
-                const int cc = (cblock * CTW + tile) * 16;
-                const bool ok = img_ok && ih >= 0 && ih < H_ && cc < C_;
-                const unsigned base = ok ? (unsigned)((((img * C_ + cc) * H_ + ih) * W_ + ch * 32) * 2) : 0u;
-                if (!edge) {
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + AREA_B + j * 1024), 16,
-                                                             (int)((b_lane + base) | (ok ? 0u : INVALID)), 0, 0, 0);
-                } else {
-                    // at the very start of the tensor the left dword lies in front of it: its offset wraps, out of range, zeros
-                    const unsigned flag = (ok ? 0u : INVALID) | (fpiece == 3 ? INVALID : 0u);
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + AREA_X + j * 256), 4, (int)((e_lane + base) | flag), 0, 0, 0);
-                }
-                issued++;
-            }
+    // Which loads a wave issues is fixed: fragment q * 8 + wave of dy, row chunk q * 8 + wave of x, edge set
+    // q * 8 + (wave + 6) % 8; what depends on that alone is worked out here, so that a unit's loads are a few scalar
+    // additions and one branch per slot (with the items dealt round-robin over one combined list the loads of a unit were
+    // 200 instructions with 30 branches, a fifth of the kernel's time).
+    constexpr int QA = (NA + 7) / 8, QB = (NB + 7) / 8;
+    // the fewest loads any wave issues per unit: the wait for a unit's loads names that many per unit still under way
+    // (a wave that issues more waits for a few loads of a later unit as well)
+    constexpr auto min_per_unit = []() {
+        int best = 1 << 30;
+        for (int w = 0; w < 8; w++) {
+            int n = 0;
+            for (int q = 0; q < (NA + 7) / 8; q++) n += q * 8 + w < NA ? 1 : 0;
+            for (int q = 0; q < (NB + 7) / 8; q++) n += (q * 8 + w < NB ? 1 : 0) + (q * 8 + ((w + 6) & 7) < NB ? 1 : 0);
+            best = n < best ? n : best;
         }
-        return issued;
+        return best;
+    };
+    constexpr int MINPER = min_per_unit();
+    bool a_on[QA], b_on[QB], e_on[QB], b_cok[QB], e_cok[QB];
+    unsigned a_off[QA], b_off[QB], e_off[QB];                            // byte offset inside the image's dy / x
+    int a_dst[QA], b_dst[QB], e_dst[QB], b_dih[QB], e_dih[QB];
+#pragma unroll
+    for (int q = 0; q < QA; q++) {
+        const int it = q * 8 + wave;
+        a_on[q] = it < NA;
+        a_off[q] = (unsigned)(((kblock * KG + it / 4) * 64 + (it & 3) * 16) * (OH_ * OW_ * 2));
+        a_dst[q] = it * 1024;
+    }
+#pragma unroll
+    for (int q = 0; q < QB; q++) {
+        const int j = q * 8 + wave, je = q * 8 + ((wave + 6) & 7);
+        const int tile = j / R_, r = j - tile * R_, tile_e = je / R_, r_e = je - tile_e * R_;
+        const int cc = (cblock * CTW + tile) * 16, cc_e = (cblock * CTW + tile_e) * 16;
+        b_on[q] = j < NB;
+        e_on[q] = je < NB;
+        b_cok[q] = cc < C_;
+        e_cok[q] = cc_e < C_;
+        b_dih[q] = r * DH;
+        e_dih[q] = r_e * DH;
+        b_off[q] = (unsigned)((cc * H_ + r * DH) * (W_ * 2));
+        e_off[q] = (unsigned)((cc_e * H_ + r_e * DH) * (W_ * 2));
+        b_dst[q] = AREA_B + j * 1024;
+        e_dst[q] = AREA_X + je * 256;
+    }
+    int per_unit = 0;                                                    // loads this wave issues per unit
+#pragma unroll
+    for (int q = 0; q < QA; q++) per_unit += a_on[q] ? 1 : 0;
+#pragma unroll
+    for (int q = 0; q < QB; q++) per_unit += (b_on[q] ? 1 : 0) + (e_on[q] ? 1 : 0);
+    auto fetch = [&](unsigned char* area, int img, int oh, int ch) -> int {
+        if (ABL & 16) return 0;
+        const bool img_ok = img * OH_ + oh < row_end;
+        const int ih0 = oh * SH - PH;
+        // of the unit: (image, row 0 of the taps, chunk) inside dy and x, bytes (unsigned arithmetic: a row above the image
+        // wraps and is never used)
+        const unsigned dy_unit = ((unsigned)img * (unsigned)(K_ * OH_ * OW_) + (unsigned)(oh * OW_ + ch * 32)) * 2u;
+        const unsigned x_unit = ((unsigned)img * (unsigned)(C_ * H_ * W_) + (unsigned)(ih0 * W_ + ch * 32)) * 2u;
+        const unsigned a_flag = (img_ok && !(ABL & 1) ? 0u : INVALID) | (ch * 32 + fpiece * 8 < OW_ ? 0u : INVALID);
+        mjt_static_for<0, QA>([&](auto qc) {
+            constexpr int q = decltype(qc)::v;
+            if (a_on[q])
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(y_rsrc, (mjt_lds_ptr)(area + a_dst[q]), 16, (int)((a_lane + dy_unit + a_off[q]) | a_flag), 0, 0, 0);
+        });
+        mjt_static_for<0, QB>([&](auto qc) {
+            constexpr int q = decltype(qc)::v;
+            if (b_on[q]) {
+                const int ih = ih0 + b_dih[q];
+                const bool ok = img_ok && ih >= 0 && ih < H_ && b_cok[q] && !(ABL & 2);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + b_dst[q]), 16,
+                                                         (int)((b_lane + x_unit + b_off[q]) | (ok ? 0u : INVALID)), 0, 0, 0);
+            }
+            if (e_on[q]) {
+                const int ih = ih0 + e_dih[q];
+                const bool ok = img_ok && ih >= 0 && ih < H_ && e_cok[q] && !(ABL & 2);
+                // at the very start of the tensor the left dword lies in front of it: its offset wraps, out of range, zeros
+                const unsigned flag = (ok ? 0u : INVALID) | (fpiece == 3 ? INVALID : 0u);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (mjt_lds_ptr)(area + e_dst[q]), 4, (int)((e_lane + x_unit + e_off[q]) | flag), 0, 0, 0);
+            }
+        });
+        return per_unit;
     };
     // wait until at most n of this wave's loads are outstanding (they complete in order)
     auto wait_loads = [&](int n) {
@@ -208,49 +279,55 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
         for (int u = 0; u < UNIT; u++) issued += fetch(uarea + u * AREA, img, oh, ch0 + u);
         return issued;
     };
-    // One unit: its fragments are in unit area `cur` once every wave's loads have arrived; request those of the unit
-    // NBUF - 1 ahead (nimg, noh, nch) into the area that was read last (with a single area: into the same, after
-    // everybody has read it), run the MFMAs chunk by chunk.
-    int cur = 0, newest = 0;                                             // newest: loads of this wave's latest request
-    auto unit = [&](auto ch_c, const int nimg, const int noh, const int nch) {
-        constexpr int CH0 = decltype(ch_c)::v;
-        unsigned char* const uarea = stage + cur * UAREA;
-        wait_loads(NBUF == 3 ? newest : 0);                              // this wave's loads for this unit have arrived
-        __syncthreads();                                                 // ... everybody's; and the area read last is free
-        if constexpr (NBUF >= 2) newest = fetch_unit(stage + (cur == 0 ? NBUF - 1 : cur - 1) * UAREA, nimg, noh, nch);
-        mjt_static_for<0, UNIT>([&](auto uc) {
-        constexpr int CH = CH0 + decltype(uc)::v;
-        unsigned char* const area = uarea + decltype(uc)::v * AREA;
-        mjt_u32x4v afrag[4], bd[R_];                                     // per tap row: columns 8 lg .. 8 lg + 7 of the chunk
-        unsigned bp[R_];                                                 // ... the two columns before them
-        unsigned long long bn[R_];                                       // ... the four after them
-        const unsigned char* const my_a = area + kg * 4096 + rd;
-        const unsigned char* const my_b = area + AREA_B + ct * (R_ * 1024);
-        const unsigned char* const my_x = area + AREA_X + ct * (R_ * 256);
-        // a lane's neighbours are in the previous / next piece of the row, or among the edge dwords (pieces of the rows of
-        // a tile are 1 KB apart per tap row, their edge dwords 256 B)
-        const unsigned char* const prev0 = lg > 0 ? my_b + rd - 4 : my_x + l16 * 16 + 8;
-        const unsigned char* const next0 = lg < 3 ? my_b + rd + 16 : my_x + l16 * 16;
-        const int prev_step = lg > 0 ? 1024 : 256, next_step = lg < 3 ? 1024 : 256;
+    // The fragments of a chunk: per tap row the lane's columns 8 lg .. 8 lg + 7, the two columns before them and the four
+    // after them; four fragments of dy.  (Zero at first: the second wave group multiplies what it read a unit earlier.)
+    mjt_u32x4v afrag[4], bd[R_];
+    unsigned bp[R_];
+    mjt_u32x2 bn[R_];
 #pragma unroll
-        for (int m = 0; m < 4; m++) afrag[m] = *(const mjt_u32x4v*)(my_a + m * 1024);
+    for (int m = 0; m < 4; m++) afrag[m] = (mjt_u32x4v)(0u);
+#pragma unroll
+    for (int r = 0; r < R_; r++) { bd[r] = (mjt_u32x4v)(0u); bp[r] = 0u; bn[r] = (mjt_u32x2)(0u); }
+    int cur = 0, newest = 0;                                             // newest: loads of this wave's latest request
+    // All reads of a chunk are issued at once, in the order of their use, and spelled out (the compiler sees no latency in
+    // an LDS read and would otherwise issue them one by one between the MFMAs, each with a full wait).  LDS addresses
+    // (bytes): the fragments of dy, the lane's piece of each tap row of x, and its neighbours: the previous / next piece
+    // of the row, or the edge dwords (pieces of the rows of a tile are 1 KB apart per tap row, their edge dwords 256 B).
+    auto read_frags = [&]() {
+        if (ABL & 8) return;
+        const unsigned area_at = stage_base + (unsigned)(cur * UAREA);
+        const unsigned my_a = area_at + (unsigned)(kg * 4096 + rd);
+        const unsigned my_b = area_at + (unsigned)(AREA_B + ct * (R_ * 1024) + rd);
+        const unsigned my_x = area_at + (unsigned)(AREA_X + ct * (R_ * 256) + l16 * 16);
+        const unsigned prev0 = lg > 0 ? my_b - 4 : my_x + 8;
+        const unsigned next0 = lg < 3 ? my_b + 16 : my_x;
+        const unsigned prev_step = lg > 0 ? 1024 : 256, next_step = lg < 3 ? 1024 : 256;
+        mjt_static_for<0, 4>([&](auto mc) { mjt_ds_read128<decltype(mc)::v * 1024>(afrag[decltype(mc)::v], my_a); });
         mjt_static_for<0, R_>([&](auto rc) {
             constexpr int r = decltype(rc)::v;
-            bd[r] = *(const mjt_u32x4v*)(my_b + r * 1024 + rd);
-            bp[r] = *(const unsigned*)(prev0 + r * prev_step);
-            bn[r] = *(const unsigned long long*)(next0 + r * next_step);
+            mjt_ds_read128<r * 1024>(bd[r], my_b);
+            mjt_ds_read32(bp[r], prev0 + r * prev_step);
+            mjt_ds_read64(bn[r], next0 + r * next_step);
         });
-        if constexpr (NBUF == 1) {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");           // read by this wave
-            __syncthreads();                                             // ... by everybody: the area may be refilled
-            fetch(area, nimg, noh, nch);
-        }
+    };
+    const int grp = wave >> 2;                                           // waves w and w + 4 share a SIMD
+    // The MFMAs of chunk CH on the fragments in registers.  LDS operations of a wave complete in order: the wait in front
+    // of a tap row names the reads of the later rows (the waits also tie the MFMAs to a place behind the reads).
+    auto mfmas = [&](auto ch_c) {
+        constexpr int CH = decltype(ch_c)::v;
         mjt_static_for<0, TAPS>([&](auto tc) {
             constexpr int t = decltype(tc)::v;
             constexpr int r = t / S_, s = t % S_;
             constexpr int off = mjt_col_shift(s);                        // -2 .. 4: the host admits nothing else
+            if constexpr (s == 0) {                                      // the reads of this tap row (and, in front of them, of dy) have arrived
+                constexpr int later = 3 * (R_ - 1 - r);
+                if constexpr (r == 0) mjt_static_for<0, 4>([&](auto mc) { mjt_lds_wait<later + 3>(afrag[decltype(mc)::v]); });
+                mjt_lds_wait<later + 2>(bd[r]);
+                mjt_lds_wait1<later + 1>(bp[r]);
+                mjt_lds_wait2<later>(bn[r]);
+            }
             // the seven dwords around the lane's columns: elements 8 lg - 2 .. 8 lg + 11
-            const unsigned w[7] = {bp[r], bd[r][0], bd[r][1], bd[r][2], bd[r][3], (unsigned)bn[r], (unsigned)(bn[r] >> 32)};
+            const unsigned w[7] = {bp[r], bd[r][0], bd[r][1], bd[r][2], bd[r][3], bn[r][0], bn[r][1]};
             constexpr int first = (off + 2) >> 1;                        // dword of element 8 lg + off
             mjt_u32x4v v;
             if constexpr (off & 1) {
@@ -261,12 +338,48 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
                 for (int j = 0; j < 4; j++) v[j] = w[first + j];
             }
             if constexpr (mjt_edge(CH, s)) v &= masks[CH * S_ + s];
-            const mjt_bf16x8 b = __builtin_bit_cast(mjt_bf16x8, v);
 #pragma unroll
-            for (int m = 0; m < 4; m++)
-                acc[m][t] = MJT_MFMA(__builtin_bit_cast(mjt_bf16x8, afrag[m]), b, acc[m][t], 0, 0, 0);
+            for (int m = 0; m < 4; m++) {
+#if ABL & 4
+                mjt_no_mfma(acc[m][t], afrag[m], v);
+#else
+                acc[m][t] = MJT_MFMA(__builtin_bit_cast(mjt_bf16x8, afrag[m]), __builtin_bit_cast(mjt_bf16x8, v), acc[m][t], 0, 0, 0);
+#endif
+            }
         });
-        });
+    };
+    // the MFMAs issued so far stay in front of this point
+    auto pin_acc = [&]() {
+        mjt_static_for<0, 4 * TAPS>([&](auto ic) { mjt_pin_acc(acc[decltype(ic)::v / TAPS][decltype(ic)::v % TAPS]); });
+    };
+    // One unit (chunk CH): its data is in area `cur` once every wave's loads have
+    // arrived; the loads of the unit NBUF - 1 ahead (nimg, noh, nch) go into the area that was read last (with a single
+    // area: into the same, after everybody has read it).
+    auto unit = [&](auto ch_c, const int nimg, const int noh, const int nch) {
+        if constexpr (SPLIT) {
+            // Every wave runs: barrier P, loads of the unit NBUF - 1 ahead, LDS reads of this unit, barrier Q, MFMAs.  The
+            // second group enters one barrier late (and the first leaves one barrier late), so one group's P meets the
+            // other's Q: while a wave reads, the other wave of its SIMD multiplies.  A wave waits for its loads of the
+            // *next* unit before Q: whichever barrier the other group is at when it passes, those loads have landed
+            // before anybody reads them, and everybody has read the area of the unit before this one when a wave passes P.
+            asm volatile("s_barrier" ::: "memory");
+            newest = fetch_unit(stage + (cur == 0 ? NBUF - 1 : cur - 1) * UAREA, nimg, noh, nch);
+            read_frags();
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(MINPER * (NBUF - 2) < 63 ? MINPER * (NBUF - 2) : 63) : "memory");
+            mfmas(ch_c);
+            pin_acc();
+        } else {
+            wait_loads(0);                                               // this wave's loads for this unit have arrived
+            __syncthreads();                                             // ... everybody's; and the area read last is free
+            if constexpr (NBUF >= 2) newest = fetch_unit(stage + (cur == 0 ? NBUF - 1 : cur - 1) * UAREA, nimg, noh, nch);
+            read_frags();
+            if constexpr (NBUF == 1) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // read by this wave
+                __syncthreads();                                         // ... by everybody: the area may be refilled
+                fetch(stage, nimg, noh, nch);
+            }
+            mfmas(ch_c);
+        }
         if constexpr (NBUF >= 2) cur = cur + 1 == NBUF ? 0 : cur + 1;
     };
 
@@ -279,18 +392,22 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
             if (++oh >= OH_) { oh = 0; img++; }
         }
     };
-    fetch_unit(stage, img_begin, oh_begin, 0);
-    if constexpr (NBUF == 3) {
+    mjt_static_for<0, AHEAD>([&](auto ac) {
         int i1 = img_begin, o1 = oh_begin, c1 = 0;
-        advance(i1, o1, c1, 1);
-        newest = fetch_unit(stage + UAREA, i1, o1, c1);
+        advance(i1, o1, c1, decltype(ac)::v);
+        newest = fetch_unit(stage + decltype(ac)::v * UAREA, i1, o1, c1);
+    });
+    if constexpr (SPLIT) {
+        // this wave's loads of the first unit have landed; the second group runs half a unit behind
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MINPER * (NBUF - 2) < 63 ? MINPER * (NBUF - 2) : 63) : "memory");
+        if (grp == 1) asm volatile("s_barrier" ::: "memory");
     }
     {
         int img = img_begin, oh = oh_begin;
 #pragma unroll 1
         for (int row = row_begin; row < row_end; row++) {
-            mjt_static_for<0, NCHUNK / UNIT>([&](auto cc) {
-                constexpr int ch0 = decltype(cc)::v * UNIT;
+            mjt_static_for<0, NCHUNK>([&](auto cc) {
+                constexpr int ch0 = decltype(cc)::v;
                 int ni = img, no = oh, nc = ch0;
                 advance(ni, no, nc, AHEAD);                              // beyond the slice: read as zeros
                 unit(mjt_ic<ch0>(), ni, no, nc);
@@ -298,6 +415,8 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
             if (++oh >= OH_) { oh = 0; img++; }
         }
     }
+    if constexpr (SPLIT)
+        if (grp == 0) asm volatile("s_barrier" ::: "memory");            // the second group's last barrier
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                     // nothing may arrive in LDS after the wave has ended
 
     // lane holds D[k = 4*lg + i][c = l16] of each (channel tile m, tap)

@@ -578,8 +578,10 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
         if (atoi(e) >= 1) rps = atoi(e) < rows ? atoi(e) : rows;
     slices = (rows + rps - 1) / rps;
 
+    const int abl = getenv("MJT_ABLATE_WGRAD") ? atoi(getenv("MJT_ABLATE_WGRAD")) : 0;    // timing-only ablations (bench.py --ablate): results are wrong
+    MJT_CHECK(abl >= 0 && abl <= 31, "conv wgrad: MJT_ABLATE_WGRAD must be 0 .. 31");
     std::ostringstream key;
-    key << "wgrad|" << C << "|" << H << "|" << W << "|" << K << "|" << R << "|" << S << "|" << OH << "|" << OW << "|" << p->stride_h << "|"
+    key << "wgrad|" << abl << "|" << C << "|" << H << "|" << W << "|" << K << "|" << R << "|" << S << "|" << OH << "|" << OW << "|" << p->stride_h << "|"
         << p->pad_h << "|" << p->pad_w << "|" << p->dil_h << "|" << p->dil_w << "|" << KG << "|" << half;
     JitKernel* k = cached(key.str());
     if (!k) {
@@ -590,7 +592,7 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
         src << "#define ENTRY " << name.str() << "\n#define C_ " << C << "\n#define H_ " << H << "\n#define W_ " << W << "\n#define K_ " << K
             << "\n#define R_ " << R << "\n#define S_ " << S << "\n#define OH_ " << OH << "\n#define OW_ " << OW << "\n#define SH "
             << p->stride_h << "\n#define PH " << p->pad_h << "\n#define PW " << p->pad_w << "\n#define DH " << p->dil_h << "\n#define DW "
-            << p->dil_w << "\n#define KG " << KG << "\n#define IN_F16 " << (half ? 1 : 0) << "\n";
+            << p->dil_w << "\n#define KG " << KG << "\n#define IN_F16 " << (half ? 1 : 0) << "\n#define ABL " << abl << "\n";
         src << embedded_source("conv_wgrad_mfma.h") << "\n";
         k = jit_get(src.str(), name.str());
         remember(key.str(), k);
