@@ -48,7 +48,7 @@ struct Params { void* a[6]; };   // x, dy, partial, number of images, images per
 
 // ABL (0 in production): timing-only ablations, results are wrong with any bit set.  1: the loads of dy fetch nothing
 // (offsets beyond the buffer: zeros, no memory traffic), 2: likewise the loads of x, 4: no MFMAs, 8: no fragment reads
-// from LDS, 16: no loads issued at all.
+// from LDS, 16: no loads issued at all, 32: the partial sums are not stored.
 #ifndef ABL
 #define ABL 0
 #endif
@@ -145,7 +145,12 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     // longer than a step), else three, two, one.  A unit, what lies between two hand-over barriers, is one chunk.
     constexpr int NA = 4 * KG, NB = CTW * R_;
     constexpr int AREA_B = NA * 1024, AREA_X = AREA_B + NB * 1024, AREA = AREA_X + NB * 256;
-    constexpr int UNIT = 1;
+#ifndef WG_UNIT2
+#define WG_UNIT2 1
+#endif
+    // two chunks per unit (half the barriers, and the MFMAs of a unit then last as long as its loads and reads) when three
+    // such units fit and a row splits into pairs of chunks; their fragments are all in registers at once
+    constexpr int UNIT = WG_UNIT2 && NCHUNK % 2 == 0 && 3 * 2 * AREA <= 150 * 1024 ? 2 : 1;
     constexpr int UAREA = UNIT * AREA;
     constexpr int NBUF = 4 * UAREA <= 150 * 1024 ? 4 : 3 * UAREA <= 150 * 1024 ? 3 : 2 * UAREA <= 150 * 1024 ? 2 : 1;
     // With three or more areas the two waves of a SIMD (wave w and w + 4) work in opposite phases: while one reads the
@@ -188,6 +193,8 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
         return best;
     };
     constexpr int MINPER = min_per_unit();
+    // loads of the later units that may still be under way when a unit's own have to have landed
+    constexpr int LOADS_AHEAD = UNIT * MINPER * (NBUF - 2) < 63 ? (NBUF >= 2 ? UNIT * MINPER * (NBUF - 2) : 0) : 63;
     bool a_on[QA], b_on[QB], e_on[QB], b_cok[QB], e_cok[QB];
     unsigned a_off[QA], b_off[QB], e_off[QB];                            // byte offset inside the image's dy / x
     int a_dst[QA], b_dst[QB], e_dst[QB], b_dih[QB], e_dih[QB];
@@ -281,53 +288,58 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     };
     // The fragments of a chunk: per tap row the lane's columns 8 lg .. 8 lg + 7, the two columns before them and the four
     // after them; four fragments of dy.  (Zero at first: the second wave group multiplies what it read a unit earlier.)
-    mjt_u32x4v afrag[4], bd[R_];
-    unsigned bp[R_];
-    mjt_u32x2 bn[R_];
+    mjt_u32x4v afrag[UNIT][4], bd[UNIT][R_];
+    unsigned bp[UNIT][R_];
+    mjt_u32x2 bn[UNIT][R_];
 #pragma unroll
-    for (int m = 0; m < 4; m++) afrag[m] = (mjt_u32x4v)(0u);
+    for (int u = 0; u < UNIT; u++) {
 #pragma unroll
-    for (int r = 0; r < R_; r++) { bd[r] = (mjt_u32x4v)(0u); bp[r] = 0u; bn[r] = (mjt_u32x2)(0u); }
+        for (int m = 0; m < 4; m++) afrag[u][m] = (mjt_u32x4v)(0u);
+#pragma unroll
+        for (int r = 0; r < R_; r++) { bd[u][r] = (mjt_u32x4v)(0u); bp[u][r] = 0u; bn[u][r] = (mjt_u32x2)(0u); }
+    }
     int cur = 0, newest = 0;                                             // newest: loads of this wave's latest request
     // All reads of a chunk are issued at once, in the order of their use, and spelled out (the compiler sees no latency in
     // an LDS read and would otherwise issue them one by one between the MFMAs, each with a full wait).  LDS addresses
     // (bytes): the fragments of dy, the lane's piece of each tap row of x, and its neighbours: the previous / next piece
     // of the row, or the edge dwords (pieces of the rows of a tile are 1 KB apart per tap row, their edge dwords 256 B).
-    auto read_frags = [&]() {
+    auto read_frags = [&](auto uc) {
+        constexpr int U = decltype(uc)::v;                               // chunk of the unit
         if (ABL & 8) return;
-        const unsigned area_at = stage_base + (unsigned)(cur * UAREA);
+        const unsigned area_at = stage_base + (unsigned)(cur * UAREA + U * AREA);
         const unsigned my_a = area_at + (unsigned)(kg * 4096 + rd);
         const unsigned my_b = area_at + (unsigned)(AREA_B + ct * (R_ * 1024) + rd);
         const unsigned my_x = area_at + (unsigned)(AREA_X + ct * (R_ * 256) + l16 * 16);
         const unsigned prev0 = lg > 0 ? my_b - 4 : my_x + 8;
         const unsigned next0 = lg < 3 ? my_b + 16 : my_x;
         const unsigned prev_step = lg > 0 ? 1024 : 256, next_step = lg < 3 ? 1024 : 256;
-        mjt_static_for<0, 4>([&](auto mc) { mjt_ds_read128<decltype(mc)::v * 1024>(afrag[decltype(mc)::v], my_a); });
+        mjt_static_for<0, 4>([&](auto mc) { mjt_ds_read128<decltype(mc)::v * 1024>(afrag[U][decltype(mc)::v], my_a); });
         mjt_static_for<0, R_>([&](auto rc) {
             constexpr int r = decltype(rc)::v;
-            mjt_ds_read128<r * 1024>(bd[r], my_b);
-            mjt_ds_read32(bp[r], prev0 + r * prev_step);
-            mjt_ds_read64(bn[r], next0 + r * next_step);
+            mjt_ds_read128<r * 1024>(bd[U][r], my_b);
+            mjt_ds_read32(bp[U][r], prev0 + r * prev_step);
+            mjt_ds_read64(bn[U][r], next0 + r * next_step);
         });
     };
     const int grp = wave >> 2;                                           // waves w and w + 4 share a SIMD
     // The MFMAs of chunk CH on the fragments in registers.  LDS operations of a wave complete in order: the wait in front
     // of a tap row names the reads of the later rows (the waits also tie the MFMAs to a place behind the reads).
-    auto mfmas = [&](auto ch_c) {
-        constexpr int CH = decltype(ch_c)::v;
+    auto mfmas = [&](auto ch_c, auto uc) {
+        constexpr int CH = decltype(ch_c)::v, U = decltype(uc)::v;
+        constexpr int AFTER = (UNIT - 1 - U) * (4 + 3 * R_);             // reads of the unit's later chunks
         mjt_static_for<0, TAPS>([&](auto tc) {
             constexpr int t = decltype(tc)::v;
             constexpr int r = t / S_, s = t % S_;
             constexpr int off = mjt_col_shift(s);                        // -2 .. 4: the host admits nothing else
             if constexpr (s == 0) {                                      // the reads of this tap row (and, in front of them, of dy) have arrived
-                constexpr int later = 3 * (R_ - 1 - r);
-                if constexpr (r == 0) mjt_static_for<0, 4>([&](auto mc) { mjt_lds_wait<later + 3>(afrag[decltype(mc)::v]); });
-                mjt_lds_wait<later + 2>(bd[r]);
-                mjt_lds_wait1<later + 1>(bp[r]);
-                mjt_lds_wait2<later>(bn[r]);
+                constexpr int later = 3 * (R_ - 1 - r) + AFTER;
+                if constexpr (r == 0) mjt_static_for<0, 4>([&](auto mc) { mjt_lds_wait<later + 3>(afrag[U][decltype(mc)::v]); });
+                mjt_lds_wait<later + 2>(bd[U][r]);
+                mjt_lds_wait1<later + 1>(bp[U][r]);
+                mjt_lds_wait2<later>(bn[U][r]);
             }
             // the seven dwords around the lane's columns: elements 8 lg - 2 .. 8 lg + 11
-            const unsigned w[7] = {bp[r], bd[r][0], bd[r][1], bd[r][2], bd[r][3], bn[r][0], bn[r][1]};
+            const unsigned w[7] = {bp[U][r], bd[U][r][0], bd[U][r][1], bd[U][r][2], bd[U][r][3], bn[U][r][0], bn[U][r][1]};
             constexpr int first = (off + 2) >> 1;                        // dword of element 8 lg + off
             mjt_u32x4v v;
             if constexpr (off & 1) {
@@ -341,9 +353,9 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
 #pragma unroll
             for (int m = 0; m < 4; m++) {
 #if ABL & 4
-                mjt_no_mfma(acc[m][t], afrag[m], v);
+                mjt_no_mfma(acc[m][t], afrag[U][m], v);
 #else
-                acc[m][t] = MJT_MFMA(__builtin_bit_cast(mjt_bf16x8, afrag[m]), __builtin_bit_cast(mjt_bf16x8, v), acc[m][t], 0, 0, 0);
+                acc[m][t] = MJT_MFMA(__builtin_bit_cast(mjt_bf16x8, afrag[U][m]), __builtin_bit_cast(mjt_bf16x8, v), acc[m][t], 0, 0, 0);
 #endif
             }
         });
@@ -364,21 +376,21 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
             // before anybody reads them, and everybody has read the area of the unit before this one when a wave passes P.
             asm volatile("s_barrier" ::: "memory");
             newest = fetch_unit(stage + (cur == 0 ? NBUF - 1 : cur - 1) * UAREA, nimg, noh, nch);
-            read_frags();
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(MINPER * (NBUF - 2) < 63 ? MINPER * (NBUF - 2) : 63) : "memory");
-            mfmas(ch_c);
+            mjt_static_for<0, UNIT>([&](auto uc) { read_frags(uc); });
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(LOADS_AHEAD) : "memory");
+            mjt_static_for<0, UNIT>([&](auto uc) { mfmas(mjt_ic<decltype(ch_c)::v + decltype(uc)::v>(), uc); });
             pin_acc();
         } else {
             wait_loads(0);                                               // this wave's loads for this unit have arrived
             __syncthreads();                                             // ... everybody's; and the area read last is free
             if constexpr (NBUF >= 2) newest = fetch_unit(stage + (cur == 0 ? NBUF - 1 : cur - 1) * UAREA, nimg, noh, nch);
-            read_frags();
+            read_frags(mjt_ic<0>());
             if constexpr (NBUF == 1) {
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // read by this wave
                 __syncthreads();                                         // ... by everybody: the area may be refilled
                 fetch(stage, nimg, noh, nch);
             }
-            mfmas(ch_c);
+            mfmas(ch_c, mjt_ic<0>());
         }
         if constexpr (NBUF >= 2) cur = cur + 1 == NBUF ? 0 : cur + 1;
     };
@@ -399,15 +411,15 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     });
     if constexpr (SPLIT) {
         // this wave's loads of the first unit have landed; the second group runs half a unit behind
-        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MINPER * (NBUF - 2) < 63 ? MINPER * (NBUF - 2) : 63) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(LOADS_AHEAD) : "memory");
         if (grp == 1) asm volatile("s_barrier" ::: "memory");
     }
     {
         int img = img_begin, oh = oh_begin;
 #pragma unroll 1
         for (int row = row_begin; row < row_end; row++) {
-            mjt_static_for<0, NCHUNK>([&](auto cc) {
-                constexpr int ch0 = decltype(cc)::v;
+            mjt_static_for<0, NCHUNK / UNIT>([&](auto cc) {
+                constexpr int ch0 = decltype(cc)::v * UNIT;
                 int ni = img, no = oh, nc = ch0;
                 advance(ni, no, nc, AHEAD);                              // beyond the slice: read as zeros
                 unit(mjt_ic<ch0>(), ni, no, nc);
@@ -419,16 +431,31 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
         if (grp == 0) asm volatile("s_barrier" ::: "memory");            // the second group's last barrier
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                     // nothing may arrive in LDS after the wave has ended
 
-    // lane holds D[k = 4*lg + i][c = l16] of each (channel tile m, tap)
+    // lane holds D[k = 4*lg + i][c = l16] of each (channel tile m, tap): the taps of one (k, c) are neighbours in
+    // partial[slice][k][c][tap], and the 16 lanes of a row hold 16 neighbouring c, so a row writes one contiguous run of
+    // 16 * TAPS floats, each lane its TAPS of them (with one store per element the stores were a fifth of the kernel)
+    typedef float mjt_f4u __attribute__((ext_vector_type(4), aligned(4)));
+    typedef float mjt_f2u __attribute__((ext_vector_type(2), aligned(4)));
     const size_t KC = (size_t)K_ * C_;
-    if (c0 >= C_) return;
+    if (c0 >= C_ || (ABL & 32)) return;
 #pragma unroll
     for (int m = 0; m < 4; m++)
 #pragma unroll
-        for (int t = 0; t < TAPS; t++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const size_t k = (size_t)(k0 + m * 16 + lg * 4 + i);
-                partial[((size_t)slice * KC + k * C_ + (size_t)(c0 + l16)) * TAPS + t] = acc[m][t][i];
+        for (int i = 0; i < 4; i++) {
+            const size_t k = (size_t)(k0 + m * 16 + lg * 4 + i);
+            float* const dst = partial + ((size_t)slice * KC + k * C_ + (size_t)(c0 + l16)) * TAPS;
+            mjt_static_for<0, TAPS / 4>([&](auto qc) {
+                constexpr int t0 = decltype(qc)::v * 4;
+                mjt_f4u v;
+                v[0] = acc[m][t0][i]; v[1] = acc[m][t0 + 1][i]; v[2] = acc[m][t0 + 2][i]; v[3] = acc[m][t0 + 3][i];
+                *(mjt_f4u*)(dst + t0) = v;
+            });
+            constexpr int T4 = TAPS / 4 * 4;
+            if constexpr (TAPS - T4 >= 2) {
+                mjt_f2u v;
+                v[0] = acc[m][T4][i]; v[1] = acc[m][T4 + 1][i];
+                *(mjt_f2u*)(dst + T4) = v;
             }
+            if constexpr ((TAPS - T4) & 1) dst[TAPS - 1] = acc[m][TAPS - 1][i];
+        }
 }

@@ -579,7 +579,7 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
     slices = (rows + rps - 1) / rps;
 
     const int abl = getenv("MJT_ABLATE_WGRAD") ? atoi(getenv("MJT_ABLATE_WGRAD")) : 0;    // timing-only ablations (bench.py --ablate): results are wrong
-    MJT_CHECK(abl >= 0 && abl <= 31, "conv wgrad: MJT_ABLATE_WGRAD must be 0 .. 31");
+    MJT_CHECK(abl >= 0 && abl <= 63, "conv wgrad: MJT_ABLATE_WGRAD must be 0 .. 63");
     std::ostringstream key;
     key << "wgrad|" << abl << "|" << C << "|" << H << "|" << W << "|" << K << "|" << R << "|" << S << "|" << OH << "|" << OW << "|" << p->stride_h << "|"
         << p->pad_h << "|" << p->pad_w << "|" << p->dil_h << "|" << p->dil_w << "|" << KG << "|" << half;
