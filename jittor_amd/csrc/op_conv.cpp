@@ -26,9 +26,9 @@ void* g_wgrad_part = nullptr;      // per-slice partial weight gradients (its ow
 size_t g_wgrad_bytes = 0;
 // column matrices of a chunk of images; float32 copy of a bfloat16 result; for the input gradient: rearranged weights,
 // and dy spread out with zeros or the results of the stride phases
-// [4]: weights with rows padded to 16 bytes for the product
-void* g_conv_scratch[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
-size_t g_conv_scratch_bytes[5] = {0, 0, 0, 0, 0};
+// [4]: weights with rows padded to 16 bytes for the product; [5]: the product of a whole batch, channels outermost
+void* g_conv_scratch[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+size_t g_conv_scratch_bytes[6] = {0, 0, 0, 0, 0, 0};
 
 void forget() {
     std::lock_guard<std::mutex> lock(g_mu);
@@ -43,7 +43,7 @@ void forget() {
     }
     g_wpack = g_wgrad_part = nullptr;
     g_wpack_bytes = g_wgrad_bytes = 0;
-    for (int i = 0; i < 5; i++) {
+    for (int i = 0; i < 6; i++) {
         g_conv_scratch[i] = nullptr;
         g_conv_scratch_bytes[i] = 0;
     }
@@ -148,8 +148,26 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         while (WKO > 1 && 2 * min_ranges * (Kg / (16 * MT * WKO)) <= cus0) WKO /= 2;     // only while at most half of them would work
     }
     const bool half = x->dtype == MJT_FLOAT16;
+    // Small maps with long sums that the MFMA kernel below does not take (7 x 7 and 13 x 13 maps: odd widths): one
+    // product for the whole batch, y'[K][N * P] = w [K][C*R*S] x cols [C*R*S][N * P], on column matrices with the images
+    // side by side, then y' -> y [N][K][P] by one permutation.  The gather of the implicit GEMM is paid once per 64 or
+    // 128 output channels, the column matrices once (us, bf16, gather / per-image column matrices / this:
+    // 64 x 512 x 7 x 7 3x3 -> 512: 126 / 85 / 60; 64 x 256 x 13 x 13 3x3 -> 384: 76 / 103 / 69; 1x1 on 7 x 7 maps,
+    // gather / this: 2048 -> 512: 60 / 35; 1024 -> 1024: 38 / 29; 512 -> 2048: 38 / 31; on 14 x 14: 1024 -> 512: 63 / 51;
+    // 512 -> 512: 36 / 36; 1024 -> 256: 36 / 41; short sums, few output channels and larger maps stay with the gather:
+    // 64 x 48 x 28 x 28 3x3 -> 96: 35 / 69 / 62; with fewer than 64 tiles of 128 x 128 the per-image matrices win:
+    // 32 x 512 x 7 x 7 3x3 -> 512: 70 against 79; where the MFMA kernel applies it wins: 64 x 256 x 14 x 14 3x3 -> 256:
+    // 61 against 71).  MJT_CONV_FLAT=1 sends every eligible shape this way, =0 none.
+    const int64_t esz0 = dtype_size(x->dtype), NP0 = N * OH * OW, CRS0 = C * R * S;
+    const bool flat_ok = G == 1 && pack_mode == 0 && esz0 == 2 && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_GEMM") && matmul_available() &&
+                         (NP0 * esz0) % 16 == 0 && (uintptr_t)x->ptr % 16 == 0 && (uintptr_t)y->ptr % 16 == 0 && NP0 < (int64_t(1) << 31) &&
+                         CRS0 * NP0 * esz0 <= (int64_t(1) << 30) && CRS0 * esz0 >= 128 && (double)N * K * OH * OW * CRS0 >= (double)(1 << 22);
+    const char* flat_env = getenv("MJT_CONV_FLAT");
+    const bool flat_forced = flat_ok && flat_env && atoi(flat_env) != 0;
+    const bool flat = flat_forced || (flat_ok && !flat_env && OH * OW <= 256 && ((K + 127) / 128) * ((NP0 + 127) / 128) >= 64 &&
+                                      ((K >= 512 && CRS0 >= 512) || (K >= 256 && CRS0 >= 2048)));
     // (a grouped convolution is one launch per group on the group's channels: worth it from 32 x 64 channels per group)
-    const bool mfma_ok = (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % CBLK == 0 && Kg % 64 == 0 && G <= 64 &&
+    const bool mfma_ok = !flat_forced && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % CBLK == 0 && Kg % 64 == 0 && G <= 64 &&
                          W % 2 == 0 && TRW >= 1 && NT <= max_px / 16 && LROWS * LCOLS * CBLK * 2 <= tile_limit &&
                          // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
                          ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + (CBLK == 64 ? 4 * LROWS * LCOLS * 16 : 0) < 65536 &&
@@ -298,6 +316,24 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             if (mjt_reindex(&tw, &tp, 2, widx, 0.0, 0, nullptr, 0, nullptr) != MJT_OK)
                 MJT_FAIL(MJT_ERR_DEVICE, "conv: padding the weight rows failed: " << mjt_last_error());
             wmat = wpad;
+        }
+        if (flat && !plain) {
+            const int64_t osz = dtype_size(y->dtype);
+            void* cols = conv_scratch(0, (size_t)(CRS * NP0 * esz));
+            void* yt = conv_scratch(5, (size_t)(K * NP0 * osz));
+            const std::string ih = "i4*" + std::to_string(p->stride_h) + "-" + std::to_string(p->pad_h) + "+i1*" + std::to_string(p->dil_h);
+            const std::string iw = "i5*" + std::to_string(p->stride_w) + "-" + std::to_string(p->pad_w) + "+i2*" + std::to_string(p->dil_w);
+            const char* cidx[4] = {"i3", "i0", ih.c_str(), iw.c_str()};
+            mjt_tensor tx = view(x->ptr, x->dtype, {N, C, H, W}), tc = view(cols, x->dtype, {C, R, S, N, OH, OW});
+            if (mjt_reindex(&tx, &tc, 4, cidx, 0.0, 0, nullptr, 0, nullptr) != MJT_OK)
+                MJT_FAIL(MJT_ERR_DEVICE, "conv: writing the column matrices failed: " << mjt_last_error());
+            gemm_launch(x->dtype, y->dtype, wmat, cols, yt, K, NP0, CRS, lda, NP0, NP0, 0, 0, 0, 1, true, false);
+            const char* pidx[3] = {"i1", "i0", "i2"};
+            mjt_tensor tt = view(yt, y->dtype, {K, N, P}), ty = view(y->ptr, y->dtype, {N, K, P});
+            if (mjt_reindex(&tt, &ty, 3, pidx, 0.0, 0, nullptr, 0, nullptr) != MJT_OK)
+                MJT_FAIL(MJT_ERR_DEVICE, "conv: rearranging the product failed: " << mjt_last_error());
+            set_last_kernel("conv_as_batch_gemm");
+            return;
         }
         // The product kernel gathers its second operand from x on the fly (kernels/gemm_mfma.h with CONV): no column
         // matrices.  float32 convolutions, and the 16-bit ones the MFMA convolution kernel above does not take (odd widths,

@@ -937,6 +937,12 @@ def test_conv_direct_small_shapes_and_fp32(gpu):
     dict(dt="float32", x=(42, 8, 28, 28), w=(72, 8, 3, 3), p=(1, 1, 1, 1, 1, 1), tile="128x128"),
     # 16-bit with a long sum and few tiles: stays on the column matrices
     dict(dt="bfloat16", x=(2, 128, 7, 7), w=(128, 128, 3, 3), p=(1, 1, 1, 1, 1, 1), stays=True),
+    # small maps with long sums and many output channels: one product for the whole batch on column matrices with the
+    # images side by side, then a permutation (by the rule; asked for by name with strides, dilation and a float32 result)
+    dict(dt="bfloat16", x=(48, 64, 7, 7), w=(512, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16", batch=True),
+    dict(dt="float16", x=(48, 512, 7, 7), w=(512, 512, 1, 1), p=(1, 1, 0, 0, 1, 1), batch=True),
+    dict(dt="bfloat16", x=(16, 32, 12, 10), w=(40, 32, 3, 3), p=(2, 1, 1, 0, 1, 2), batch=True, flat="1"),
+    dict(dt="bfloat16", x=(48, 64, 7, 7), w=(512, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), out="bfloat16", flat="0"),
     # the product on the direct-copy kernel (asked for by name: these shapes have too few tiles to get it by themselves):
     # weights shared across the batch, column matrices with the pixels innermost read with transposing reads
     dict(dt="bfloat16", x=(3, 64, 15, 15), w=(96, 64, 3, 3), p=(1, 1, 1, 1, 1, 1), dma=True, cols=True),
@@ -959,8 +965,12 @@ def test_conv_as_reindex_and_gemm(gpu, case, monkeypatch):
         monkeypatch.setenv("MJT_GEMM_DMA", "1")
     if case.get("cols"):
         monkeypatch.setenv("MJT_CONV_NO_IGEMM", "1")
+    if "flat" in case:
+        monkeypatch.setenv("MJT_CONV_FLAT", case["flat"])
     got, kern = _conv_call(xb, wb, case["p"], out_dtype=out, in_dtype=dt)
-    if not case.get("plain") and not case.get("cols") and not case.get("dma") and not case.get("stays"):
+    if case.get("batch"):
+        assert kern == "conv_as_batch_gemm", kern
+    elif not case.get("plain") and not case.get("cols") and not case.get("dma") and not case.get("stays"):
         assert kern.startswith("mjt_conv_igemm_" + dt), kern        # the product kernel gathers its operand from x itself
         assert kern.endswith(case.get("tile", "64x64")), kern
     else:
