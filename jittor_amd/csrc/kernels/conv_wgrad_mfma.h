@@ -144,10 +144,15 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
     // Four areas when they fit (the loads of a step are then requested three steps ahead: memory latency under load is
     // longer than a step), else three, two, one.  A unit, what lies between two hand-over barriers, is one chunk.
     constexpr int NA = 4 * KG, NB = CTW * R_;
-    constexpr int AREA_B = NA * 1024, AREA_X = AREA_B + NB * 1024, AREA = AREA_X + NB * 256;
 #ifndef WG_UNIT2
 #define WG_UNIT2 1
 #endif
+    // WHOLE_ROW: a unit holds every chunk of its row (rows of at most 32 / 64 outputs).  What lies left of its first and
+    // right of its last chunk is outside the image and cleared by the edge masks whatever is read there, and the columns
+    // between two chunks of the unit are in the neighbouring chunk's piece: no edge dwords are loaded at all.
+    constexpr bool WHOLE_ROW = NCHUNK <= 2 && (NCHUNK == 1 || (NCHUNK == 2 && WG_UNIT2 && 3 * 2 * (NA * 1024 + NB * 1024) <= 150 * 1024)) &&
+                               NCHUNK * 32 >= W_;
+    constexpr int AREA_B = NA * 1024, AREA_X = AREA_B + NB * 1024, AREA = AREA_X + (WHOLE_ROW ? 0 : NB * 256);
     // two chunks per unit (half the barriers, and the MFMAs of a unit then last as long as its loads and reads) when three
     // such units fit and a row splits into pairs of chunks; their fragments are all in registers at once
     constexpr int UNIT = WG_UNIT2 && NCHUNK % 2 == 0 && 3 * 2 * AREA <= 150 * 1024 ? 2 : 1;
@@ -211,7 +216,7 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
         const int tile = j / R_, r = j - tile * R_, tile_e = je / R_, r_e = je - tile_e * R_;
         const int cc = (cblock * CTW + tile) * 16, cc_e = (cblock * CTW + tile_e) * 16;
         b_on[q] = j < NB;
-        e_on[q] = je < NB;
+        e_on[q] = je < NB && !WHOLE_ROW;
         b_cok[q] = cc < C_;
         e_cok[q] = cc_e < C_;
         b_dih[q] = r * DH;
@@ -309,10 +314,20 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
         const unsigned area_at = stage_base + (unsigned)(cur * UAREA + U * AREA);
         const unsigned my_a = area_at + (unsigned)(kg * 4096 + rd);
         const unsigned my_b = area_at + (unsigned)(AREA_B + ct * (R_ * 1024) + rd);
-        const unsigned my_x = area_at + (unsigned)(AREA_X + ct * (R_ * 256) + l16 * 16);
-        const unsigned prev0 = lg > 0 ? my_b - 4 : my_x + 8;
-        const unsigned next0 = lg < 3 ? my_b + 16 : my_x;
-        const unsigned prev_step = lg > 0 ? 1024 : 256, next_step = lg < 3 ? 1024 : 256;
+        unsigned prev0, next0, prev_step, next_step;
+        if constexpr (WHOLE_ROW) {
+            // the last dword of the piece before / the first two of the piece after: in this chunk, or (for the first and
+            // the last lane group) in the same row of the chunk before / after; at the ends of the row anything (masked)
+            prev0 = lg > 0 ? my_b - 4 : U > 0 ? my_b - AREA + 3 * 16 + 12 : my_b;
+            next0 = lg < 3 ? my_b + 16 : U + 1 < UNIT ? my_b + AREA - 3 * 16 : my_b;
+            prev_step = next_step = 1024;
+        } else {
+            const unsigned my_x = area_at + (unsigned)(AREA_X + ct * (R_ * 256) + l16 * 16);
+            prev0 = lg > 0 ? my_b - 4 : my_x + 8;
+            next0 = lg < 3 ? my_b + 16 : my_x;
+            prev_step = lg > 0 ? 1024 : 256;
+            next_step = lg < 3 ? 1024 : 256;
+        }
         mjt_static_for<0, 4>([&](auto mc) { mjt_ds_read128<decltype(mc)::v * 1024>(afrag[U][decltype(mc)::v], my_a); });
         mjt_static_for<0, R_>([&](auto rc) {
             constexpr int r = decltype(rc)::v;
