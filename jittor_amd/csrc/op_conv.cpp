@@ -145,7 +145,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int64_t cus0 = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
         const int64_t tile_rows = WPX * (TRW > 0 ? TRW : 1);
         const int64_t min_ranges = N * ((OH + tile_rows - 1) / tile_rows);
-        while (WKO > 1 && 2 * min_ranges * (Kg / (16 * MT * WKO)) <= cus0) WKO /= 2;     // only while at most half of them would work
+        // (down to 128 channels per workgroup, four waves, never to workgroups of two waves: 64 x 256 x 14 x 14 3x3 -> 256 on 128
+        // workgroups of four waves 48 us, on 256 of two waves 61, on 64 of eight 65; with 8 images 48 against 58)
+        while (WKO > 2 && 2 * min_ranges * (Kg / (16 * MT * WKO)) <= cus0) WKO /= 2;
     }
     const bool half = x->dtype == MJT_FLOAT16;
     // Small maps with long sums that the MFMA kernel below does not take (7 x 7 and 13 x 13 maps: odd widths): one
