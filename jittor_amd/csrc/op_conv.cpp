@@ -119,8 +119,13 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const int64_t max_px = WPX == 1 ? 224 : 112;            // pixels per wave: 16 per accumulator tile
     const int64_t WPS = max_px == 224 ? 1 : 2;              // waves per SIMD the register budget is set for
     // output channels per wave: 16 per accumulator-tile row; per workgroup: up to 256
-    const int64_t MT = 4;
     const int64_t Kg = K / G;                                // output channels of one group: the K of the MFMA kernel
+    // accumulator-tile rows (of 16 output channels) per wave: 4; 2 for groups of 64 or 128 output channels, which then have four
+    // waves share an input tile instead of two (64 x 64 x 56 x 56 3x3 -> 64: 42.9 -> 31.7 us; 64 x 256 x 56 x 56 -> 64:
+    // 124 -> 86; 64 x 64 x 28 x 28 -> 64: 20.8 -> 14.3)
+    // (groups of 128: eight waves of 32 channels instead of four of 64: 64 x 128 x 28 x 28 3x3 -> 128: 25.4 -> 24.6 us,
+    // with 8 images 23.0 -> 18.4)
+    const int64_t MT = Kg == 64 || Kg == 128 ? 2 : 4;
     int64_t WKO = Kg % 256 == 0 ? 256 / (16 * MT) : Kg % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
     // LDS: two buffers of input rows (one block of CB channels each), a ring of NS weight slabs (64 bytes per output
     // channel of the workgroup each) and a spare KB that takes the writes of idle lanes.  Blocks of 32 channels
