@@ -125,8 +125,12 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     // 124 -> 86; 64 x 64 x 28 x 28 -> 64: 20.8 -> 14.3)
     // (groups of 128: eight waves of 32 channels instead of four of 64: 64 x 128 x 28 x 28 3x3 -> 128: 25.4 -> 24.6 us,
     // with 8 images 23.0 -> 18.4)
-    const int64_t MT = Kg == 64 || Kg == 128 ? 2 : 4;
-    int64_t WKO = Kg % 256 == 0 ? 256 / (16 * MT) : Kg % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
+    int64_t MT = Kg == 64 || Kg == 128 ? 2 : 4;
+    auto widest = [&]() {                                   // groups of output channels per workgroup: up to 256 channels, eight waves
+        const int64_t v = Kg % 256 == 0 ? 256 / (16 * MT) : Kg % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
+        return v > 4 ? int64_t(4) : v;
+    };
+    int64_t WKO = widest();
     // LDS: two buffers of input rows (one block of CB channels each), a ring of NS weight slabs (64 bytes per output
     // channel of the workgroup each) and a spare KB that takes the writes of idle lanes.  Blocks of 32 channels
     // leave room for a deeper ring, which is what hides the latency of the slabs; the ring needs three slabs at least.
@@ -152,7 +156,15 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         const int64_t min_ranges = N * ((OH + tile_rows - 1) / tile_rows);
         // (down to 128 channels per workgroup, four waves, never to workgroups of two waves: 64 x 256 x 14 x 14 3x3 -> 256 on 128
         // workgroups of four waves 48 us, on 256 of two waves 61, on 64 of eight 65; with 8 images 48 against 58)
+        const int64_t before = WKO;
         while (WKO > 2 && 2 * min_ranges * (Kg / (16 * MT * WKO)) <= cus0) WKO /= 2;
+        // such a small grid with more channels: wave tiles of 32 channels as well, so that twice as many workgroups of four
+        // waves share the work (64 x 256 x 14 x 14 3x3 -> 256: 48 -> 39 us; 64 x 256 x 14 x 14 3x3 stride 2 -> 512: 42 -> 37)
+        if (WKO < before && MT == 4) {
+            MT = 2;
+            WKO = widest();
+            while (WKO > 2 && 2 * min_ranges * (Kg / (16 * MT * WKO)) <= cus0) WKO /= 2;
+        }
     }
     const bool half = x->dtype == MJT_FLOAT16;
     // Small maps with long sums that the MFMA kernel below does not take (7 x 7 and 13 x 13 maps: odd widths): one
