@@ -125,9 +125,9 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     // 124 -> 86; 64 x 64 x 28 x 28 -> 64: 20.8 -> 14.3)
     // (groups of 128: eight waves of 32 channels instead of four of 64: 64 x 128 x 28 x 28 3x3 -> 128: 25.4 -> 24.6 us,
     // with 8 images 23.0 -> 18.4)
-    int64_t MT = Kg == 64 || Kg == 128 ? 2 : 4;
+    int64_t MT = Kg == 32 || Kg == 64 || Kg == 128 ? 2 : 4;
     auto widest = [&]() {                                   // groups of output channels per workgroup: up to 256 channels, eight waves
-        const int64_t v = Kg % 256 == 0 ? 256 / (16 * MT) : Kg % 128 == 0 ? 128 / (16 * MT) : 64 / (16 * MT);
+        const int64_t v = Kg % 256 == 0 ? 256 / (16 * MT) : Kg % 128 == 0 ? 128 / (16 * MT) : Kg % 64 == 0 ? 64 / (16 * MT) : 32 / (16 * MT);
         return v > 4 ? int64_t(4) : v;
     };
     int64_t WKO = widest();
@@ -186,7 +186,7 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
     const bool flat = flat_forced || (flat_ok && !flat_env && OH * OW <= 256 && ((K + 127) / 128) * ((NP0 + 127) / 128) >= 64 &&
                                       ((K >= 512 && CRS0 >= 512) || (K >= 256 && CRS0 >= 2048)));
     // (a grouped convolution is one launch per group on the group's channels: worth it from 32 x 64 channels per group)
-    const bool mfma_ok = !flat_forced && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % CBLK == 0 && Kg % 64 == 0 && G <= 64 &&
+    const bool mfma_ok = !flat_forced && (x->dtype == MJT_BFLOAT16 || half) && !getenv("MJT_NO_FASTPATH") && !getenv("MJT_CONV_NO_MFMA") && C % CBLK == 0 && (Kg % 64 == 0 || Kg == 32) && G <= 64 &&
                          W % 2 == 0 && TRW >= 1 && NT <= max_px / 16 && LROWS * LCOLS * CBLK * 2 <= tile_limit &&
                          // tap shift + k-step plane offset of a fragment read must fit the 16-bit offset field
                          ((R - 1) * p->dil_h * LCOLS + (S - 1) * p->dil_w) * 16 + (CBLK == 64 ? 4 * LROWS * LCOLS * 16 : 0) < 65536 &&

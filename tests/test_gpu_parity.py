@@ -1070,9 +1070,11 @@ def test_conv_grouped_entry_and_front_end(gpu):
     ((2, 128, 12, 16), (256, 64, 3, 3), 2, (1, 1, 1, 1, 1, 1), "float32"),      # two groups of 64 -> 128 channels
     ((3, 128, 9, 24), (256, 32, 3, 3), 4, (1, 1, 1, 1, 1, 1), "bfloat16"),      # four groups of 32 -> 64, 16-bit result
     ((2, 192, 10, 12), (192, 64, 1, 1), 3, (2, 2, 0, 0, 1, 1), "float32"),      # 1x1 stride 2, three groups
+    ((2, 128, 12, 16), (128, 32, 3, 3), 4, (1, 1, 1, 1, 1, 1), "float32"),      # four groups of 32 -> 32: workgroups of two waves, 16 channels each
+    ((3, 256, 14, 14), (256, 32, 3, 3), 8, (2, 2, 1, 1, 1, 1), "bfloat16"),     # eight groups of 32 -> 32, stride 2
 ])
 def test_conv_grouped_on_the_mfma_kernel(gpu, xs, ws, G, params, out):
-    """Groups of at least 32 input and 64 output channels run on the MFMA kernel, one launch per group on the group's
+    """Groups of at least 32 input and 32 output channels run on the MFMA kernel, all groups in one launch, each on its own
     channels (python/jittor/nn.py:1272-1294): against the oracle's grouped convolution of the exact 16-bit operands,
     per element within 1e-4 of the sum of its terms' magnitudes."""
     rng = np.random.default_rng(41)
