@@ -96,6 +96,9 @@ struct JitKernel {
     hipFunction_t fn = nullptr;
     std::string name;
     uint64_t state[2] = {0, 0};   // for the launcher of kernels that keep state in their code object's device memory
+    // what the code object's metadata says of the entry point: accumulation registers in use and vector registers
+    // moved to scratch memory (-1: not found)
+    int agprs = -1, spilled = -1;
 };
 // Compiles `source` (which must define extern "C" __global__ `entry`) for the
 // current device, or returns the cached kernel for an identical source.

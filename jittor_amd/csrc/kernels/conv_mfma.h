@@ -208,10 +208,19 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // When the steps of a block are too few for that (more than SGMAX items per step), the items of a step go in
     // rounds of at most SGMAX instead, each written as soon as it has arrived, the last one at the end of the step.
     constexpr int SGMAX = 8;
-    constexpr int SD0 = STEPS < STAGE_DEPTH ? STEPS : STAGE_DEPTH;
-    constexpr bool BULK = (IPW + (STEPS - SD0 + 1) - 1) / (STEPS - SD0 + 1) > SGMAX;
+    // Rows on their way occupy registers the compiler knows nothing about (it takes a spelled-out load for finished when it
+    // is issued): were it to run out of registers and move one of them aside, it would move what the load has not written
+    // yet.  So their number stays inside what the loop leaves free of the 128 registers of a wave (B fragments and their
+    // addresses: 5 per accumulator tile; A fragments, descriptors, selectors and addresses: 44), by way of a shorter flight.
+    constexpr int SQMAX = (84 - 5 * NT) / 4;
+    constexpr int SD1 = STEPS < STAGE_DEPTH ? STEPS : STAGE_DEPTH;
+    constexpr auto sg_of = [](int sd) { return (IPW + (STEPS - sd + 1) - 1) / (STEPS - sd + 1); };
+    constexpr auto sq_of = [=](int sd) { return sg_of(sd) * sd < IPW ? sg_of(sd) * sd : IPW; };
+    constexpr auto fits = [=](int sd) { return sg_of(sd) <= SGMAX && sq_of(sd) <= SQMAX; };
+    constexpr int SD0 = fits(SD1) ? SD1 : SD1 > 2 && fits(SD1 - 1) ? SD1 - 1 : SD1 > 3 && fits(SD1 - 2) ? SD1 - 2 : 0;
+    constexpr bool BULK = SD0 == 0;
     constexpr int SD = BULK ? 1 : SD0;
-    constexpr int SG = (IPW + (STEPS - SD + 1) - 1) / (STEPS - SD + 1);
+    constexpr int SG = sg_of(SD);
     constexpr int RPS = BULK ? (SG + SGMAX - 1) / SGMAX : 1;      // rounds per step
     constexpr int RS = (SG + RPS - 1) / RPS;                      // items per round
     constexpr int SQ = BULK ? RS : SG * SD < IPW ? SG * SD : IPW;
@@ -269,6 +278,10 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     };
     auto commit_stage = [&](auto sc, bool live, mjt_u32x4v& d, int r0, int lrows, int buf, int item, int limit) {
         constexpr int stg = decltype(sc)::v;
+        // (the item number is made opaque here: what follows from it is worked out in place, with scalar instructions,
+        // instead of once per item in front of the loop, where every item's address would hold a register for good)
+        item = __builtin_amdgcn_readfirstlane(item);         // (it is the same in every lane)
+        asm volatile("" : "+s"(item));
         int lr, seg, cg;
         item_of(item, lr, seg, cg);
         if constexpr (stg == 0) {
@@ -363,12 +376,16 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         constexpr int TRW_ = decltype(trw_c)::v, NT_ = decltype(nt_c)::v, LR_ = decltype(lr_c)::v;
         // per-lane pixel of each of the NT_ tiles
         unsigned baddr[NT_];                                 // LDS byte address of the fragment at tap (0,0), k-step 0, in the current buffer
+        // (from a copy of the lane number made here: worked out per tile, the addresses of the full and of the short tile do
+        // not both hold registers for the whole kernel)
+        int lane_t = lane;
+        asm volatile("" : "+v"(lane_t));
 #pragma unroll
         for (int t = 0; t < NT_; t++) {
-            int q = t * 16 + l16;
+            int q = t * 16 + (lane_t & 15);
             int r = q / OW_, col = q - r * OW_;
             if (q >= TRW_ * OW_) { r = 0; col = 0; }
-            baddr[t] = xs_base + (unsigned)(buf * TILE_ELEMS * 2) + (unsigned)mjt_lds_off(((wpx * TRW_ + r) * SH) * LCOLS + col * SW, lg) * 2;
+            baddr[t] = xs_base + (unsigned)(buf * TILE_ELEMS * 2) + (unsigned)mjt_lds_off(((wpx * TRW_ + r) * SH) * LCOLS + col * SW, lane_t >> 4) * 2;
         }
         mjt_f32x4 acc[MT][NT_];
 #pragma unroll

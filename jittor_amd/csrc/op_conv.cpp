@@ -271,34 +271,41 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
             remember(key.str(), k);
             remember(key.str() + "|pack", kp);
         }
-        size_t wbytes = (size_t)numel(w) * 2;
-        if (pack_mode) MJT_CHECK(packed && (uintptr_t)packed % 16 == 0, "conv: packed weights must be a 16-byte aligned device buffer");
-        if (!pack_mode && !c.dry_run && wbytes > g_wpack_bytes) {
-            if (g_wpack) {
-                HIP_CHECK(hipStreamSynchronize(c.stream));
-                HIP_CHECK(hipFree(g_wpack));
+        // The kernel keeps loads and LDS reads under way in registers behind the compiler's back (it takes a spelled-out load
+        // for finished when issued).  That is sound while the compiler moves no register aside; a build that needed more
+        // registers than a wave has (accumulation registers beyond the accumulators, scratch memory) may have moved one
+        // whose load had not landed, so such a build is not run: the convolution takes the routes below.
+        const bool regs_ok = k->spilled == 0 && k->agprs >= 0 && k->agprs <= MT * NT * 4;
+        if (regs_ok) {
+            size_t wbytes = (size_t)numel(w) * 2;
+            if (pack_mode) MJT_CHECK(packed && (uintptr_t)packed % 16 == 0, "conv: packed weights must be a 16-byte aligned device buffer");
+            if (!pack_mode && !c.dry_run && wbytes > g_wpack_bytes) {
+                if (g_wpack) {
+                    HIP_CHECK(hipStreamSynchronize(c.stream));
+                    HIP_CHECK(hipFree(g_wpack));
+                }
+                HIP_CHECK(hipMalloc(&g_wpack, wbytes));
+                g_wpack_bytes = wbytes;
             }
-            HIP_CHECK(hipMalloc(&g_wpack, wbytes));
-            g_wpack_bytes = wbytes;
+            const int64_t ranges = N * ((OH + RPW - 1) / RPW);
+            const int64_t ranges8 = (ranges + 7) / 8 * 8;
+            const int64_t blocks = ranges8 * KPARTS;
+            MJT_CHECK(blocks < (int64_t(1) << 31), "conv: launch too large");
+            const int64_t wg = Kg * C * R * S;               // weights of one group
+            int64_t pblocks = (wg + 255) / 256;
+            if (pblocks > 2048) pblocks = 2048;
+            // one launch for all groups (the group is the grid's second axis)
+            char* wdst = (char*)(pack_mode ? packed : g_wpack);
+            if (pack_mode != 2) {
+                std::vector<uint64_t> pa{bits_of_ptr(w->ptr), bits_of_ptr(wdst), 0, 0};
+                jit_launch(kp, (unsigned)pblocks, (unsigned)G, 256, 0, pa);
+            }
+            if (pack_mode != 1) {
+                std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(wdst), bits_of_ptr(y->ptr), (uint64_t)N};
+                jit_launch(k, (unsigned)blocks, (unsigned)G, (unsigned)(64 * WPX * WKO), 0, a);
+            }
+            return;
         }
-        const int64_t ranges = N * ((OH + RPW - 1) / RPW);
-        const int64_t ranges8 = (ranges + 7) / 8 * 8;
-        const int64_t blocks = ranges8 * KPARTS;
-        MJT_CHECK(blocks < (int64_t(1) << 31), "conv: launch too large");
-        const int64_t wg = Kg * C * R * S;               // weights of one group
-        int64_t pblocks = (wg + 255) / 256;
-        if (pblocks > 2048) pblocks = 2048;
-        // one launch for all groups (the group is the grid's second axis)
-        char* wdst = (char*)(pack_mode ? packed : g_wpack);
-        if (pack_mode != 2) {
-            std::vector<uint64_t> pa{bits_of_ptr(w->ptr), bits_of_ptr(wdst), 0, 0};
-            jit_launch(kp, (unsigned)pblocks, (unsigned)G, 256, 0, pa);
-        }
-        if (pack_mode != 1) {
-            std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(wdst), bits_of_ptr(y->ptr), (uint64_t)N};
-            jit_launch(k, (unsigned)blocks, (unsigned)G, (unsigned)(64 * WPX * WKO), 0, a);
-        }
-        return;
     }
 
     if (pack_mode) MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv: this convolution does not run on packed weights (mjt_conv2d_meta takes it)");
@@ -651,6 +658,14 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
         src << embedded_source("conv_wgrad_mfma.h") << "\n";
         k = jit_get(src.str(), name.str());
         remember(key.str(), k);
+    }
+    // (as in the forward kernel: a build that had to move registers aside is not run; its accumulators are vector registers)
+    if (k->spilled != 0 || k->agprs != 0) {
+        if (any_shape) {
+            conv_wgrad_direct(x, dy, dw, p, G);
+            return;
+        }
+        MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: the MFMA kernel for this shape needs more registers than a wave has");
     }
     void* part = wgrad_partials((size_t)slices * (size_t)numel(dw) * 4);
     std::vector<uint64_t> a{bits_of_ptr(x->ptr), bits_of_ptr(dy->ptr), bits_of_ptr(part), (uint64_t)N, (uint64_t)rps, 0};

@@ -108,10 +108,15 @@ void gemm_launch(int in_dtype, int out_dtype, const void* A, const void* B, void
                 k = jit_get(src.str(), name.str());
                 remember(key.str(), k);
             }
-            const int64_t grid = (tm * tn + 7) / 8 * 8;
-            MJT_CHECK(grid < (int64_t(1) << 31), "matmul: launch too large");
-            jit_launch(k, (unsigned)grid, (unsigned)batch, 256, 0, args);
-            return;
+            // (the kernel keeps LDS reads under way in registers behind the compiler's back: a build that had to move
+            // registers aside, into accumulation registers beyond the tile / 256 accumulators or into scratch memory,
+            // is not run; the general kernel below takes the product)
+            if (k->spilled == 0 && k->agprs >= 0 && k->agprs <= tile * tile / 256) {
+                const int64_t grid = (tm * tn + 7) / 8 * 8;
+                MJT_CHECK(grid < (int64_t(1) << 31), "matmul: launch too large");
+                jit_launch(k, (unsigned)grid, (unsigned)batch, 256, 0, args);
+                return;
+            }
         }
     }
     if (fast) {

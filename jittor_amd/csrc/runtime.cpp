@@ -191,6 +191,40 @@ static void store_code(const std::string& path, const std::vector<char>& code) {
     else unlink(tmp.c_str());
 }
 
+// The register figures of `entry` in a code object's metadata (a MessagePack map per kernel whose keys come in
+// alphabetical order: .agpr_count first, .symbol and .vgpr_spill_count behind it).
+static void read_register_use(const std::vector<char>& code, const std::string& entry, int* agprs, int* spilled) {
+    *agprs = *spilled = -1;
+    const std::string blob(code.begin(), code.end());
+    auto value_at = [&](size_t pos) -> int {                  // an unsigned integer of up to 16 bits
+        if (pos >= blob.size()) return -1;
+        const unsigned char t = (unsigned char)blob[pos];
+        if (t < 0x80) return t;
+        if (t == 0xcc && pos + 1 < blob.size()) return (unsigned char)blob[pos + 1];
+        if (t == 0xcd && pos + 2 < blob.size()) return ((unsigned char)blob[pos + 1] << 8) | (unsigned char)blob[pos + 2];
+        return -1;
+    };
+    const std::string k_agpr = "\xab.agpr_count", k_sym = "\xa7.symbol", k_spill = "\xb1.vgpr_spill_count";
+    const std::string want = entry + ".kd";
+    for (size_t at = blob.find(k_agpr); at != std::string::npos; at = blob.find(k_agpr, at + 1)) {
+        const size_t next = blob.find(k_agpr, at + 1);
+        const size_t sym = blob.find(k_sym, at), sp = blob.find(k_spill, at);
+        if (sym == std::string::npos || sp == std::string::npos || (next != std::string::npos && (sym > next || sp > next))) continue;
+        size_t v = sym + k_sym.size();                        // the name: a string of up to 31, 255 or 65535 bytes
+        if (v >= blob.size()) continue;
+        const unsigned char t = (unsigned char)blob[v];
+        size_t len = 0;
+        if ((t & 0xe0) == 0xa0) { len = t & 0x1f; v += 1; }
+        else if (t == 0xd9 && v + 1 < blob.size()) { len = (unsigned char)blob[v + 1]; v += 2; }
+        else if (t == 0xda && v + 2 < blob.size()) { len = ((unsigned char)blob[v + 1] << 8) | (unsigned char)blob[v + 2]; v += 3; }
+        else continue;
+        if (len != want.size() || blob.compare(v, len, want) != 0) continue;
+        *agprs = value_at(at + k_agpr.size());
+        *spilled = value_at(sp + k_spill.size());
+        return;
+    }
+}
+
 JitKernel* jit_get(const std::string& source, const std::string& entry) {
     require_init();
     std::lock_guard<std::mutex> lock(g_jit_mutex);
@@ -226,6 +260,7 @@ JitKernel* jit_get(const std::string& source, const std::string& entry) {
     }
     JitKernel* k = new JitKernel();
     k->name = entry;
+    read_register_use(code, entry, &k->agprs, &k->spilled);
     if (!ctx().dry_run) {
         hipError_t e = hipModuleLoadData(&k->module, code.data());
         if (e != hipSuccess && from_disk) {
@@ -236,6 +271,7 @@ JitKernel* jit_get(const std::string& source, const std::string& entry) {
             code = compile_source(source, entry + ".hip");
             g_jit_compiled++;
             store_code(path, code);
+            read_register_use(code, entry, &k->agprs, &k->spilled);
             e = hipModuleLoadData(&k->module, code.data());
         }
         if (e != hipSuccess) {

@@ -698,6 +698,9 @@ def _conv_call(xbits, wbits, params, out_dtype="float32", in_dtype="bfloat16"):
     dict(x=(2, 64, 5, 2), w=(64, 64, 1, 1), p=(1, 1, 0, 0, 1, 1)),          # two columns: a load spans four rows
     dict(x=(2, 96, 12, 16), w=(64, 96, 3, 3), p=(1, 1, 1, 1, 1, 1)),        # 96 channels: three blocks of 32
     dict(x=(1, 64, 30, 112), w=(64, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),       # wide rows: one output row per wave, a short weight ring
+    dict(x=(2, 64, 16, 16), w=(32, 64, 3, 3), p=(1, 1, 1, 1, 1, 1)),        # 32 output channels: workgroups of two waves that stage 32 items each, two channel blocks
+    dict(x=(2, 128, 40, 16), w=(32, 128, 3, 3), p=(1, 1, 1, 1, 1, 1), rpw=40, out="bfloat16"),   # the same with two full tiles and a short one per workgroup, four blocks
+    dict(x=(2, 64, 31, 10), w=(32, 64, 3, 3), p=(2, 2, 1, 1, 1, 1)),        # 32 output channels, stride 2, odd height
 ])
 def test_conv_mfma_matches_oracle(gpu, case):
     from oracle import kernels as K
@@ -789,14 +792,16 @@ def test_conv_packed_weights_entry(gpu):
     assert lib.mjt_conv2d_meta_packed(ctypes.byref(tx), ctypes.byref(tw), buf.raw_ptr(), ctypes.byref(ty), ctypes.byref(p)) == -2
 
 
-def test_conv_mfma_random_geometries(gpu):
+@pytest.mark.parametrize("seed,ks,at_least", [(77, [64, 128, 192], 8), (78, [32, 32, 64], 8)])
+def test_conv_mfma_random_geometries(gpu, seed, ks, at_least):
     """Seeded sweep over geometries for the MFMA kernel (channel counts, map sizes with even widths, taps, stride,
     padding, dilation, 16-bit and float32 results): every case against a float64 sum of shifted products, per
-    element within 1e-4 of the sum of its terms' magnitudes (plus the result type's own rounding)."""
-    rng = np.random.default_rng(77)
+    element within 1e-4 of the sum of its terms' magnitudes (plus the result type's own rounding).  The second sweep
+    is mostly on 32 output channels (workgroups of two waves, each staging twice the input rows)."""
+    rng = np.random.default_rng(seed)
     taken = 0
     for i in range(14):
-        C, K = int(rng.choice([32, 64, 96, 128])), int(rng.choice([64, 128, 192]))
+        C, K = int(rng.choice([32, 64, 96, 128])), int(rng.choice(ks))
         R, S = int(rng.choice([1, 2, 3])), int(rng.choice([1, 3, 5]))
         sh, sw = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))
         dh, dw_ = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))
@@ -823,7 +828,7 @@ def test_conv_mfma_random_geometries(gpu):
         bound = 1e-4 * terms + (np.abs(ref) * 2.0 ** -7 if out == "bfloat16" else 0.0) + 1e-30
         assert (np.abs(got - ref) <= bound).all(), (kern, (N, C, H, W), (K, C, R, S), (sh, sw, ph, pw, dh, dw_),
                                                     float((np.abs(got - ref) / bound).max()))
-    assert taken >= 8, taken          # most of the sweep runs on the MFMA kernel (the rest on the fallbacks, checked alike)
+    assert taken >= at_least, taken   # most of the sweep runs on the MFMA kernel (the rest on the fallbacks, checked alike)
 
 
 def _dgrad_reference(dy, w, H, W, params):

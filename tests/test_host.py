@@ -548,6 +548,38 @@ def test_conv_input_gradient_entry_validates_and_picks_its_path(compile_only):
     assert b"padding" in lib.mjt_last_error()
 
 
+def test_conv_builds_that_ran_out_of_registers_are_not_run(compile_only):
+    """The MFMA convolution keeps loads under way in registers the compiler does not track, which is sound only while the
+    compiler moves no register aside.  The library reads each build's register figures from the code object: a geometry
+    whose build stays within a wave's registers runs on the kernel (among them 32 output channels on two waves, which once
+    did not), one whose build needs more (4-column maps: 58 staging items per wave) takes another route.  That the first
+    group still names the MFMA kernel also shows that the figures are found at all."""
+    lib = L.load()
+    P = 0x100000
+
+    def call(xs, ws, params=(1, 1, 1, 1, 1, 1)):
+        N, C, H, W = xs
+        K, _, R, S = ws
+        sh, sw, ph, pw, dh, dw = params
+        oh, ow = (H + 2 * ph - dh * (R - 1) - 1) // sh + 1, (W + 2 * pw - dw * (S - 1) - 1) // sw + 1
+        x, w, y = L.tensor(P, "bfloat16", xs), L.tensor(P, "bfloat16", ws), L.tensor(P, "bfloat16", (N, K, oh, ow))
+        p = L.ConvParams(*params)
+        assert lib.mjt_conv2d_meta(ctypes.byref(x), ctypes.byref(w), ctypes.byref(y), ctypes.byref(p)) == 0
+        return L.last_kernel()
+
+    assert call((2, 64, 16, 16), (32, 64, 3, 3)).startswith("mjt_conv_mfma_bf16")
+    assert call((2, 64, 16, 16), (64, 64, 3, 3)).startswith("mjt_conv_mfma_bf16")
+    assert call((2, 32, 40, 4), (64, 32, 3, 3)).startswith("mjt_conv_igemm")
+    # the weight gradient kernel likewise: rows of 104 columns need more registers than there are
+    x, dy = L.tensor(P, "bfloat16", (4, 64, 10, 104)), L.tensor(P, "bfloat16", (4, 64, 10, 104))
+    dw, p = L.tensor(P, "float32", (64, 64, 3, 3)), L.ConvParams(1, 1, 1, 1, 1, 1)
+    assert lib.mjt_conv2d_meta_wgrad(ctypes.byref(x), ctypes.byref(dy), ctypes.byref(dw), ctypes.byref(p)) == -2
+    assert b"registers" in lib.mjt_last_error()
+    x, dy = L.tensor(P, "bfloat16", (4, 64, 16, 16)), L.tensor(P, "bfloat16", (4, 64, 16, 16))
+    assert lib.mjt_conv2d_meta_wgrad(ctypes.byref(x), ctypes.byref(dy), ctypes.byref(dw), ctypes.byref(p)) == 0
+    assert L.last_kernel().startswith("mjt_conv_wgrad_mfma_bf16")
+
+
 def test_scatter_and_gather_entries_pick_their_kernels(compile_only, monkeypatch):
     """Without a device: which kernel skeleton a reindex_reduce, a reindex and a fused gather + reduce take.  A scatter
     through a window pattern is a gather over x unless it has overflow conditions, extras or too many candidate windows
