@@ -9,6 +9,7 @@ new one), recognise the convolution pattern the way ConvTuner does
 once.  Everything runs on the device; there is no host path.
 """
 import ctypes
+import math
 
 from . import _lib
 from . import core
@@ -19,7 +20,7 @@ from . import profiler as _profiler
 from .flags import flags
 
 stats = {"launches": 0, "fused_groups": 0, "fused_reduces": 0, "conv_matches": 0, "syncs": 0, "sunk_ops": 0, "matmul_matches": 0,
-         "wgrad_kernel": 0, "gather_reduces": 0, "fused_scatters": 0, "plans": 0, "replays": 0}
+         "wgrad_kernel": 0, "wgrad_chunked": 0, "gather_reduces": 0, "fused_scatters": 0, "plans": 0, "replays": 0}
 
 
 class ConvUnit:
@@ -1146,8 +1147,51 @@ def _run_single(op):
             # batched GEMM per chunk, one sum over the images.
             esz = _lib.DTYPE_SIZE[x.dtype]
             P, CRS = OH * OW, C * R * S
-            chunk = max(1, min(N, (1 << 30) // max(1, CRS * P * esz)))
             pdt = "float32" if x.dtype in ("float16", "bfloat16") else x.dtype
+            # 16-bit planes that are no 16-byte multiples (14 x 14, 7 x 7, 13 x 13 maps) would send every image's
+            # product to the kernel without MFMAs.  The sum over images and pixels is one contraction: with the images of
+            # a chunk side by side, dw = sum over chunks of dy' [K, nb*P] times cols' [(c,r,s), nb*P]^T, where nb images
+            # make nb*P a multiple of 64 elements (the product kernel that copies its operands straight into LDS wants
+            # that), or of 8.  Few chunks: long sums on large tiles and few partial results (us of kernels, bf16, 3x3,
+            # 64 images: 256 x 14 x 14 -> 256: 441 -> 99; 512 x 7 x 7 -> 512: 632 -> 61).  Planes that are 16-byte
+            # multiples stay with the product per image (128 x 28 x 28 -> 128: 159 us against 165 this way).
+            nb0 = next((a // math.gcd(P, a) for a in (64, 8) if N % (a // math.gcd(P, a)) == 0), 0)
+            if esz == 2 and (P * esz) % 16 != 0 and nb0 and CRS * N * P * esz <= (1 << 30):
+                tiles = -(-K // 128) * -(-CRS // 128)
+                chunks = N // nb0                                  # most chunks there can be
+                while chunks % 2 == 0 and (chunks // 2) * tiles >= 256:
+                    chunks //= 2
+                nb = N // chunks
+                L = nb * P
+                stats["wgrad_chunked"] += 1
+                with core.no_grad():
+                    dyc = core.reindex(dy, [chunks, K, nb, OH, OW], ["i0*%d+i2" % nb, "i1", "i3", "i4"])
+                    colsc = core.reindex(x, [chunks, C, R, S, nb, OH, OW],
+                                         ["i0*%d+i4" % nb, "i1", "i5*%d-%d+i2*%d" % (sh, ph, dh), "i6*%d-%d+i3*%d" % (sw, pw, dw)], 0.0)
+                _run_single(dyc._op)
+                _run_single(colsc._op)
+                ta = _tensor(_ptr_of(dyc), dy.dtype, [chunks, K, L])
+                tb = _tensor(_ptr_of(colsc), x.dtype, [chunks, CRS, L])
+                if chunks == 1:                                    # the product is the result, in the weights' dtype
+                    tp = _tensor(_alloc_out(out), out.dtype, [1, K, CRS])
+                    _lib.check(lib.mjt_matmul(ctypes.byref(ta), ctypes.byref(tb), ctypes.byref(tp), 0, 1))
+                    stats["launches"] += 1
+                    return
+                part = Var([chunks, K, CRS], pdt)
+                tp = _tensor(_alloc_out(part), pdt, [chunks, K, CRS])
+                _lib.check(lib.mjt_matmul(ctypes.byref(ta), ctypes.byref(tb), ctypes.byref(tp), 0, 1))
+                stats["launches"] += 1
+                acc = out if out.dtype == pdt else Var([K, C, R, S], pdt)
+                tpart = _tensor(_ptr_of(part), pdt, [chunks, K * CRS])
+                tacc = _tensor(_alloc_out(acc), pdt, [K * CRS])
+                _lib.check(lib.mjt_reduce(ctypes.byref(tpart), ctypes.byref(tacc), _lib.OP_CODE["add"], 0b01))
+                if acc is not out:                                 # narrow the float32 sum to the weights' dtype
+                    with core.no_grad():
+                        narrowed = core.unary(acc, out.dtype)
+                    _run_group([narrowed._op], {}, {narrowed.id})
+                    out._buf = narrowed._buf
+                return
+            chunk = max(1, min(N, (1 << 30) // max(1, CRS * P * esz)))
             cols = Var([chunk, C, R, S, OH, OW], x.dtype)
             part = Var([N, K, CRS], pdt)
             cols_ptr, part_ptr = _alloc_out(cols), _alloc_out(part)

@@ -246,6 +246,37 @@ def test_grad_meta_conv_bfloat16(gpu, xs, ws, wgrad_kernel):
             stack.extend(v._history[1])
 
 
+@pytest.mark.parametrize("xs,k,rs,stride,pad,dtype,chunked", [
+    ((8, 32, 14, 14), 64, 3, 1, 1, "bfloat16", 1),      # 196-pixel planes: pairs of images make 16-byte multiples, four chunks
+    ((16, 64, 7, 7), 96, 3, 1, 1, "float16", 1),        # 49 pixels: eight images per chunk
+    ((64, 32, 7, 7), 64, 3, 1, 1, "bfloat16", 1),       # 64 images of 49 pixels: one chunk of 3136, the product is the result
+    ((6, 32, 27, 27), 64, 3, 2, 1, "bfloat16", 1),      # stride 2 onto 14 x 14; three chunks
+    ((8, 48, 13, 13), 40, 1, 1, 0, "bfloat16", 1),      # 1x1 taps on 169 pixels: all eight images in one chunk
+    ((3, 32, 14, 14), 64, 3, 1, 1, "bfloat16", 0),      # three images never make a multiple of 8 elements: the product per image
+])
+def test_grad_conv_weight_16bit_maps_with_unaligned_planes(gpu, xs, k, rs, stride, pad, dtype, chunked):
+    """Weight gradient of 16-bit convolutions on maps whose planes are no 16-byte multiples (14 x 14, 7 x 7, 13 x 13): one
+    product over chunks of images laid side by side instead of one product per image on the kernel without MFMAs
+    (executor.py, ConvBwdWeightUnit); against the float64 gradient of the exact 16-bit operands."""
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal((k, xs[1], rs, rs)) * 0.05).astype(np.float32)
+    vx, vw = jt.array(x).cast(dtype), jt.array(w).cast(dtype)
+    jt.sync([vx, vw])
+    xe = vx.float32().numpy()
+    we = vw.float32().numpy()
+    y = jt.nn.conv2d(vx, vw, stride=stride, padding=pad)
+    r = (rng.integers(-2, 3, y.shape) * 0.5).astype(np.float32)            # exact in both 16-bit types
+    gw, = jt.grad((y * jt.array(r).cast(dtype)).sum(), [vw])
+    assert gw.dtype == dtype
+    before = jt.executor_stats["wgrad_chunked"]
+    jt.sync([gw])
+    assert jt.executor_stats["wgrad_chunked"] - before == chunked
+    _, dW = _conv_grads_ref(xe, we, r, stride, pad, 1)
+    tol = 2.0 ** -7 if dtype == "bfloat16" else 2.0 ** -10                 # results are rounded to the 16-bit type
+    assert np.abs(gw.float32().numpy() - dW).max() <= tol * np.abs(dW).max()
+
+
 def test_grad_stop_grad_and_no_grad(gpu):
     x = jt.array(np.arange(1, 7, dtype=np.float32))
     y = (x * 2).stop_grad()

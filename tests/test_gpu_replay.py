@@ -109,6 +109,24 @@ def test_replay_float32_weight_gradient_through_column_matrices(gpu):
     assert replays >= 1
 
 
+def test_replay_16bit_weight_gradient_over_chunks_of_images(gpu):
+    """The weight gradient on 14 x 14 maps (planes that are no 16-byte multiples) is one product over chunks of images
+    laid side by side: two reindexes into buffers of their own, a batched product, a sum over the chunks."""
+    def step(seed):
+        rng = np.random.default_rng(400 + seed)
+        x = jt.array(rng.standard_normal((8, 32, 14, 14)).astype(np.float32)).cast("bfloat16")
+        w = jt.array((rng.standard_normal((64, 32, 3, 3)) * 0.1).astype(np.float32)).cast("bfloat16")
+        y = jt.nn.conv2d(x, w, padding=1)
+        gx, gw = jt.grad((y * y).sum(), [x, w])
+        jt.sync([y, gx, gw])
+        return [y.raw(), gx.raw(), gw.raw()]
+
+    before = executor.stats["wgrad_chunked"]
+    fresh, again, replays = _both_ways(step)
+    _same(fresh, again)
+    assert replays >= 2 and executor.stats["wgrad_chunked"] > before
+
+
 def test_replay_keeps_the_graph_bookkeeping(gpu):
     """After a replayed execution the vars are leaves with buffers of their own, exactly as after a fresh one: a result
     can be reused by a later graph, and two replays never share a result buffer."""
