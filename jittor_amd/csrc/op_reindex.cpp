@@ -19,6 +19,7 @@ namespace mjt {
 // fast paths, aot_kernels.hip
 bool try_window_gather(const mjt_tensor* x, const mjt_tensor* y, const std::vector<Affine>& aff, double overflow_value);
 bool try_permute(const mjt_tensor* x, const mjt_tensor* y, const std::vector<Affine>& aff);
+bool try_im2col_planes(const mjt_tensor* x, const mjt_tensor* y, const std::vector<Affine>& aff, double overflow_value);
 bool try_scatter_1d(const mjt_tensor* y, const mjt_tensor* x, int op, const mjt_tensor* index);
 void launch_fill_pattern(void* dst, uint64_t pattern, int elem_size, size_t n);
 
@@ -489,6 +490,7 @@ void reindex_impl(const mjt_tensor* x, const mjt_tensor* y, int n_idx, const cha
         for (int i = 0; i < n_idx && ok; i++) ok = affine_of(*plan->idx[i], xs, ys, &aff[i]);
         if (ok && n_ofc == 0 && try_permute(x, y, aff)) return;
         if (ok && try_window_gather(x, y, aff, overflow_value)) return;
+        if (ok && try_im2col_planes(x, y, aff, overflow_value)) return;
     }
     run_generic(plan, false, 0, x, y, overflow_value, n_ex, ex);
 }

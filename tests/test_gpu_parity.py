@@ -268,6 +268,54 @@ def test_window_gather_fast_path_matches_oracle_and_generic(gpu, case, dtype):
     assert fast.startswith("mjt_window_gather"), fast
 
 
+@pytest.mark.parametrize("case", [
+    # x [N, C, H, W],  taps,   stride, dilation, padding, images per chunk (None: one image per group; 0: the whole batch is one group)
+    dict(x=(3, 5, 9, 10), k=(3, 3), s=(1, 1), d=(1, 1), p=(1, 1), nb=None),
+    dict(x=(4, 3, 14, 14), k=(3, 3), s=(1, 1), d=(1, 1), p=(1, 1), nb=2),             # 196-pixel planes in pairs: vectors of 8 cross image borders
+    dict(x=(8, 4, 7, 7), k=(3, 3), s=(1, 1), d=(1, 1), p=(1, 1), nb=0),               # 49-pixel planes, the whole batch side by side
+    dict(x=(6, 2, 27, 27), k=(3, 3), s=(2, 2), d=(1, 1), p=(1, 1), nb=3),             # stride 2; three images: vectors of 4
+    dict(x=(2, 3, 14, 13), k=(2, 3), s=(1, 2), d=(2, 1), p=(0, 2), nb=None),          # mixed stride / dilation, no vertical padding
+    dict(x=(3, 2, 9, 9), k=(1, 1), s=(1, 1), d=(1, 1), p=(0, 0), nb=None),            # 1x1 taps, 81 pixels per run: single elements
+    # (maps of up to 64 pixels read the other way round, taps as pixels and pixels as taps, are the sliding-window gather's)
+    dict(x=(2, 2, 40, 56), k=(5, 5), s=(1, 1), d=(1, 1), p=(2, 2), nb=None),          # 25 taps on a larger plane
+])
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32", "float16"])
+def test_im2col_planes_fast_path_matches_oracle_and_generic(gpu, case, dtype):
+    """The column matrices of a convolution with the pixels innermost (kernels/im2col_planes.h), per image, for the whole
+    batch and per chunk of images: bit for bit against the oracle's reindex and against the generic gather."""
+    rng = np.random.default_rng(14)
+    (N, C, H, W), (kh, kw), (sh, sw), (dh, dw), (ph, pw), nb = case["x"], case["k"], case["s"], case["d"], case["p"], case["nb"]
+    oh = (H + 2 * ph - dh * (kh - 1) - 1) // sh + 1
+    ow = (W + 2 * pw - dw * (kw - 1) - 1) // sw + 1
+    store = L.NP_STORAGE[dtype]
+    x32 = (rng.standard_normal(case["x"]) * 4).astype(np.float32)
+    x = O.f32_to_bf16_bits(x32) if dtype == "bfloat16" else x32.astype(store)
+    if nb is None:
+        shape, a = [N, C, kh, kw, oh, ow], 2
+        idx = ["i0", "i1"]
+    elif nb == 0:
+        shape, a = [C, kh, kw, N, oh, ow], 1
+        idx = ["i3", "i0"]
+    else:
+        shape, a = [N // nb, C, kh, kw, nb, oh, ow], 2
+        idx = ["i0*%d+i4" % nb, "i1"]
+    o = len(shape) - 2
+    idx += ["i%d*%d-%d+i%d*%d" % (o, sh, ph, a, dh), "i%d*%d-%d+i%d*%d" % (o + 1, sw, pw, a + 1, dw)]
+    ref = O.reindex(x, shape, idx, 0)
+    vx = jt.from_storage(x, dtype) if dtype != "float32" else jt.array(x)
+    got = vx.reindex(shape, idx, 0).raw()
+    fast = L.last_kernel()
+    assert exact(got, ref)
+    os.environ["MJT_NO_FASTPATH"] = "1"
+    try:
+        got2 = vx.reindex(shape, idx, 0).raw()
+        assert L.last_kernel().startswith("mjt_reindex_")
+    finally:
+        del os.environ["MJT_NO_FASTPATH"]
+    assert exact(got2, ref)
+    assert fast.startswith("mjt_im2col_planes"), fast
+
+
 def test_reindex_full_size_c2_bit_exact(gpu):
     x = np.random.default_rng(0).standard_normal((32, 64, 56, 56)).astype(np.float32)
     y = jt.array(x).reindex([32, 64, 56, 56, 3, 3], ["i0", "i1", "i2+i4-1", "i3+i5-1"], 0).data

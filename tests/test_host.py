@@ -617,6 +617,13 @@ def test_scatter_and_gather_entries_pick_their_kernels(compile_only, monkeypatch
     rows = gather([8, 16, 64, 64], [8, 16, 66, 66], ["i0", "i1", "i2-1", "i3-1"])
     monkeypatch.delenv("MJT_REINDEX_NO_FLAT")
     assert flat.startswith("mjt_reindex_") and rows.startswith("mjt_reindex_") and flat != rows      # four elements per lane, or two
+    # column matrices with the pixels innermost: per image, the whole batch as one group, chunks of images; a stride the
+    # pattern does not have (the image index times 3 for chunks of 2) stays on the generic kernel
+    taps = ["i4-1+i2", "i5-1+i3"]
+    assert gather([8, 16, 28, 28], [8, 16, 3, 3, 28, 28], ["i0", "i1"] + taps).startswith("mjt_im2col_planes_b4_28x28_k3x3")
+    assert gather([8, 16, 7, 7], [16, 3, 3, 8, 7, 7], ["i3", "i0", "i4-1+i1", "i5-1+i2"]).endswith("_n8_v4")
+    assert gather([8, 16, 29, 29], [4, 16, 3, 3, 2, 14, 14], ["i0*2+i4", "i1", "i5*2-1+i2", "i6*2-1+i3"]).endswith("_n2_v4")
+    assert gather([12, 16, 14, 14], [4, 16, 3, 3, 2, 14, 14], ["i0*3+i4", "i1", "i5-1+i2", "i6-1+i3"]).startswith("mjt_reindex_")
 
     loop, z = L.tensor(0, "float32", [8, 16, 32, 32, 2, 2]), L.tensor(P, "float32", [8, 16, 32, 32])
     tx = L.tensor(P, "float32", [8, 16, 64, 64])
