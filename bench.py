@@ -620,6 +620,46 @@ def wl_steps(L, lib, steps, warmup, with_cpu, which=("bottleneck_bf16", "small_c
     return {"workload": "STEPS", "cases": out}
 
 
+def wl_layers(L, lib, steps, warmup, with_cpu, which=None):
+    """The 3x3 convolutions of a ResNet's four stages and the two strided ones between them, batch 64, bfloat16: forward,
+    input gradient and weight gradient of one layer through the Python front end (replayed), host wall time per step over
+    `steps` steps issued back to back (best of 5 blocks; the steps are bound by the GPU).  Per-kernel times are what
+    `rocprofv3 --kernel-trace` shows for the same run.  Not part of the default run (--only LAYERS, or one layer by name:
+    LAYER_56, LAYER_28, LAYER_14, LAYER_7, LAYER_56S2, LAYER_28S2)."""
+    import jittor_amd as jt
+    rng = np.random.default_rng(17)
+    bf = lambda a: jt.array(a.astype(np.float32)).bfloat16()
+    layers = {"56": ((64, 64, 56, 56), 64, 1), "28": ((64, 128, 28, 28), 128, 1), "14": ((64, 256, 14, 14), 256, 1), "7": ((64, 512, 7, 7), 512, 1),
+              "56S2": ((64, 128, 56, 56), 128, 2), "28S2": ((64, 256, 28, 28), 256, 2)}
+    out = {}
+    for name, (xs, k, stride) in layers.items():
+        if which and name not in which:
+            continue
+        x, w = bf(rng.standard_normal(xs)), bf(rng.standard_normal((k, xs[1], 3, 3)) * 0.05)
+        jt.sync([x, w])
+
+        def step():
+            y = jt.nn.conv2d(x, w, stride=stride, padding=1)
+            jt.sync(jt.grad((y * y).sum(), [x, w]))
+
+        for i in range(max(warmup, 3)):
+            step()
+        L.sync()
+        best = None
+        for block in range(5):
+            t0 = time.perf_counter()
+            for i in range(steps):
+                step()
+            L.sync()
+            t = (time.perf_counter() - t0) * 1e3 / steps
+            best = t if best is None else min(best, t)
+        oh = (xs[2] + 2 - 3) // stride + 1
+        flops = 3 * 2.0 * xs[0] * k * oh * oh * xs[1] * 9
+        out["conv3x3_%dx%dx%dx%d_to_%d_s%d" % (xs + (k, stride))] = {"ms_per_step": round(best, 4), "tflops_fwd_bwd": round(flops / best / 1e9, 1),
+                                                                        "steps_run": max(warmup, 3) + 5 * steps}
+    return {"workload": "LAYERS", "cases": out}
+
+
 WORKLOADS = {
     "C1": wl_c1,
     "C2": wl_c2,
@@ -637,6 +677,13 @@ WORKLOADS = {
     "STEPS": wl_steps,
     "STEP_BOTTLENECK": lambda *a: wl_steps(*a, which=("bottleneck_bf16",)),
     "STEP_SMALL_CNN": lambda *a: wl_steps(*a, which=("small_cnn_f32",)),
+    "LAYERS": wl_layers,
+    "LAYER_56": lambda *a: wl_layers(*a, which=("56",)),
+    "LAYER_28": lambda *a: wl_layers(*a, which=("28",)),
+    "LAYER_14": lambda *a: wl_layers(*a, which=("14",)),
+    "LAYER_7": lambda *a: wl_layers(*a, which=("7",)),
+    "LAYER_56S2": lambda *a: wl_layers(*a, which=("56S2",)),
+    "LAYER_28S2": lambda *a: wl_layers(*a, which=("28S2",)),
 }
 DEFAULT = ["C1", "C2", "C3add", "C3max", "C4", "C5", "C5bf16out"]
 
