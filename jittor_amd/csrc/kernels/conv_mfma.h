@@ -67,6 +67,7 @@ __device__ __forceinline__ unsigned mjt_narrow2(float lo, float hi) {
 }
 #endif
 typedef float mjt_f32x4 __attribute__((ext_vector_type(4)));
+typedef float mjt_f32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned mjt_u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned mjt_u32x4v __attribute__((ext_vector_type(4)));
 
@@ -88,7 +89,13 @@ struct Params { void* a[4]; };   // x, packed w, y, number of images (typed as p
 #define SPLITS ((OH_ + RPW - 1) / RPW)      // row ranges per image
 #define NCB (C_ / CB)
 #define GROUPS ((W_ + 7) / 8)           // groups of 8 columns; the last one may reach past the row: what it reads there is never written
-#define SEGS ((GROUPS + 7) / 8)         // segments of 64 columns
+// An item of the staging is what one load instruction of a wave brings: 8 channels x 8 groups of 8 columns.  Rows of more than
+// 32 columns take SEGS items of 64 columns each; narrower rows share an item, RPI of them with GP2 groups each, since on a
+// 14-column map an item of one row would use a quarter of its lanes and cost the same instructions.
+#define GP2 (GROUPS <= 1 ? 1 : GROUPS <= 2 ? 2 : GROUPS <= 4 ? 4 : 8)       // groups that a row takes in an item
+#define RPI (8 / GP2)                                                        // rows per item
+#define SEGS (RPI > 1 ? 1 : (GROUPS + 7) / 8)                                // segments of 64 columns
+#define ROWITEMS ((LROWS + RPI - 1) / RPI)                                   // items along the rows of a full tile
 #define TILE_ELEMS (LROWS * LCOLS * CB)
 
 // LDS tile: 8 planes, one per group of 8 channels, each [row][col][8 c] (16 bytes per position).  The 16 lanes
@@ -200,7 +207,7 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
     // Every wave moves its share of the input rows of a block and of every weight slab.  Vector memory
     // operations of a wave complete in order: the ring is deep enough that the wait for a slab, which also waits
     // for every older load, never asks for an input row earlier than the row is needed itself.
-    constexpr int ITEMS = LROWS * SEGS * (CB / 8);                       // of a full tile
+    constexpr int ITEMS = ROWITEMS * SEGS * (CB / 8);                    // of a full tile
     constexpr int IPW = (ITEMS + NWAVES - 1) / NWAVES;            // items of one wave per channel block
     // A wave asks for item k of its share at the start of step fetch_step(k) and writes it to LDS at the end
     // of step fetch_step(k) + SD - 1: SD steps for the row to arrive from HBM, SG items per step, SQ registers.
@@ -236,7 +243,10 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         const int rest = item / (CB / 8);
         lr = rest / SEGS;
         seg = rest - lr * SEGS;
+        lr *= RPI;                                           // the item's first row
     };
+    // the lane's row inside an item and its group of 8 columns inside the row
+    const int row_in_item = RPI > 1 ? sg / GP2 : 0, grp_in_row = RPI > 1 ? sg % GP2 : sg;
     // The loads are unconditional instructions (rows outside the image and idle lanes read a clamped address and
     // are zeroed or skipped when written; a wave whose role this is not reads beyond the descriptor's range, which
     // costs no memory traffic): around a load under a branch the compiler no longer knows how many loads are under
@@ -245,12 +255,21 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         const int ir0 = r0 * SH - PH;
         int lr, seg, cg;
         item_of(item, lr, seg, cg);
-        int ir = ir0 + (lr < lrows ? lr : lrows - 1);
-        ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
-        const int soff = __builtin_amdgcn_readfirstlane((((cb * CB + cg * 8) * H_ + ir) * W_) * 2);     // uniform: channel group and row inside the image
-        int grp = seg * 8 + sg;
-        grp = grp < GROUPS ? grp : GROUPS - 1;
-        return __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)((live ? x_lane_off : 0x80000000u) + (unsigned)grp * 16), soff, 0);
+        if constexpr (RPI > 1) {                             // the row differs between lanes
+            lr += row_in_item;
+            int ir = ir0 + (lr < lrows ? lr : lrows - 1);
+            ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
+            const int soff = __builtin_amdgcn_readfirstlane(((cb * CB + cg * 8) * H_ * W_) * 2);      // uniform: the channel group
+            const int grp = grp_in_row < GROUPS ? grp_in_row : GROUPS - 1;
+            return __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)((live ? x_lane_off : 0x80000000u) + (unsigned)(ir * W_ * 2 + grp * 16)), soff, 0);
+        } else {
+            int ir = ir0 + (lr < lrows ? lr : lrows - 1);
+            ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
+            const int soff = __builtin_amdgcn_readfirstlane((((cb * CB + cg * 8) * H_ + ir) * W_) * 2);     // uniform: channel group and row inside the image
+            int grp = seg * 8 + sg;
+            grp = grp < GROUPS ? grp : GROUPS - 1;
+            return __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)((live ? x_lane_off : 0x80000000u) + (unsigned)grp * 16), soff, 0);
+        }
     };
     // Writing an item to LDS, in four stages that work in place on its four registers (the main loop spreads them
     // between its MFMAs): three exchanges, then the write.
@@ -268,12 +287,23 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         const int ir0 = r0 * SH - PH;
         int lr, seg, cg;
         item_of(item, lr, seg, cg);
-        int ir = ir0 + (lr < lrows ? lr : lrows - 1);
-        ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
-        const int soff = __builtin_amdgcn_readfirstlane((((cb * CB + cg * 8) * H_ + ir) * W_) * 2);
-        int grp = seg * 8 + sg;
-        grp = grp < GROUPS ? grp : GROUPS - 1;
-        const unsigned voff = (live ? x_lane_off : 0x80000000u) + (unsigned)grp * 16;
+        int soff;
+        unsigned voff;
+        if constexpr (RPI > 1) {
+            lr += row_in_item;
+            int ir = ir0 + (lr < lrows ? lr : lrows - 1);
+            ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
+            soff = __builtin_amdgcn_readfirstlane(((cb * CB + cg * 8) * H_ * W_) * 2);
+            const int grp = grp_in_row < GROUPS ? grp_in_row : GROUPS - 1;
+            voff = (live ? x_lane_off : 0x80000000u) + (unsigned)(ir * W_ * 2 + grp * 16);
+        } else {
+            int ir = ir0 + (lr < lrows ? lr : lrows - 1);
+            ir = ir < 0 ? 0 : ir >= H_ ? H_ - 1 : ir;
+            soff = __builtin_amdgcn_readfirstlane((((cb * CB + cg * 8) * H_ + ir) * W_) * 2);
+            int grp = seg * 8 + sg;
+            grp = grp < GROUPS ? grp : GROUPS - 1;
+            voff = (live ? x_lane_off : 0x80000000u) + (unsigned)grp * 16;
+        }
         asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(dst) : "v"(voff), "s"(x_desc), "s"(soff) : "memory");
     };
     auto commit_stage = [&](auto sc, bool live, mjt_u32x4v& d, int r0, int lrows, int buf, int item, int limit) {
@@ -287,7 +317,12 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
         if constexpr (stg == 0) {
             // d[k] = columns 2k (low half), 2k+1 (high half) of channel r
             const int ir0 = r0 * SH - PH;
-            if (ir0 + lr < 0 || ir0 + lr >= H_) d = (mjt_u32x4v)(0u);   // uniform: a row outside the image
+            if constexpr (RPI > 1) {                         // per lane: the rows of an item
+                const bool outside = ir0 + lr + row_in_item < 0 || ir0 + lr + row_in_item >= H_;
+                d[0] = outside ? 0u : d[0]; d[1] = outside ? 0u : d[1]; d[2] = outside ? 0u : d[2]; d[3] = outside ? 0u : d[3];
+            } else {
+                if (ir0 + lr < 0 || ir0 + lr >= H_) d = (mjt_u32x4v)(0u);   // uniform: a row outside the image
+            }
             // lane ^ 4: keep one half of the columns, get the same half from the channel 4 away
             const unsigned g0 = mjt_xor4(b2 ? d[0] : d[2]), g1 = mjt_xor4(b2 ? d[1] : d[3]);
             const unsigned a0 = b2 ? g0 : d[0], a1 = b2 ? g1 : d[1];      // channel r & 3:       column pairs 0, 1 of the half
@@ -313,8 +348,10 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
             // rows outside the image carry zeros; columns past the row end are not the row's; what is not to be written
             // goes to the spare piece of LDS.  The write is spelled out: a compiler-made LDS access after the copies
             // into the slab ring would wait for all of those first.
-            const bool wr = live && item < limit && lr < lrows && seg * 64 + lane < W_;
-            const unsigned dst = wr ? xs_base + (unsigned)(buf * TILE_ELEMS + mjt_lds_off(lr * LCOLS + PW + seg * 64 + lane, cg)) * 2
+            // (after the exchanges the lane holds column 8 * group + lane % 8 of its row)
+            const int lrow = lr + row_in_item, col = RPI > 1 ? grp_in_row * 8 + sr : seg * 64 + lane;
+            const bool wr = live && item < limit && lrow < lrows && col < W_;
+            const unsigned dst = wr ? xs_base + (unsigned)(buf * TILE_ELEMS + mjt_lds_off(lrow * LCOLS + PW + col, cg)) * 2
                                     : as_spare + (unsigned)lane * 16;
             asm volatile("ds_write_b128 %0, %1" : : "v"(dst), "v"(d) : "memory");
         }
@@ -566,6 +603,28 @@ extern "C" __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu
 #else
                     *(mjt_f32x4*)((float*)p.a[2] + o) = v;
 #endif
+                }
+            }
+#elif OW_ % 2 == 0
+            // an even width: pairs of pixels never straddle an output row (widths of 14: half the stores of single pixels)
+#pragma unroll
+            for (int i = 0; i < 4; i += 2) {
+                const int q = t * 16 + lg_e * 4 + i;
+                const int r = q / OW_, col = q - r * OW_;
+                const int orow = r0 + wpx * TRW_ + r;
+                if (q < TRW_ * OW_ && orow < row_lim && !(ABL & 1)) {
+#pragma unroll
+                    for (int m = 0; m < MT; m++) {
+                        const size_t o = (((size_t)n * YK_ + y_k0 + ko_base + m * 16 + l16_e) * OH_ + orow) * OW_ + col;
+#if Y_BF16
+                        *(unsigned*)((unsigned short*)p.a[2] + o) = mjt_narrow2(acc[m][t][i], acc[m][t][i + 1]);
+#else
+                        mjt_f32x2 pr;
+                        pr[0] = acc[m][t][i];
+                        pr[1] = acc[m][t][i + 1];
+                        *(mjt_f32x2*)((float*)p.a[2] + o) = pr;
+#endif
+                    }
                 }
             }
 #else
