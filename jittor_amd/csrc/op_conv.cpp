@@ -218,14 +218,25 @@ void conv_impl(const mjt_tensor* x, const mjt_tensor* w, const mjt_tensor* y, co
         };
         int64_t RPW = TR;
         {
+            // Workgroups of at most four waves whose LDS is at most half a compute unit's run two to a compute unit, each
+            // SIMD then holding two waves that fill each other's gaps: a pair gets through its work in 1.4 times the time
+            // of one workgroup alone (64 x 64 x 56 x 56 3x3 -> 64: 256 workgroups of 14 rows 29.7 us, 448 of 8 rows 25.1,
+            // 896 of 4 rows 28.4; 64 x 256 x 56 x 56 -> 64: 91.9 -> 75.9 us per call).  Such a grid pays for more, shorter
+            // workgroups; a workgroup's set-up counts as one accumulator tile there, a short last tile as half a one more.
+            const int64_t lds_need = 2 * LROWS * LCOLS * CBLK * 2 + 8 * (64 * 16 * MT * WKO) + 1024;
+            const bool pairs = WPX * WKO <= 4 && lds_need <= lds_total / 2;
             double best = 1e300;
             for (int64_t r = TR; r <= OH || r == TR; r++) {
                 int64_t trw_t, nt_t;
                 tail_of(r, &trw_t, &nt_t);
                 const int64_t wgs = N * ((OH + r - 1) / r) * KPARTS;
-                const int64_t rounds = (wgs + cus - 1) / cus;
                 const int64_t ntiles = r / TR + (trw_t ? 1 : 0);
-                const double cost = (double)rounds * ((double)(r / TR) * NT + nt_t + 0.5 * ntiles);
+                const double work = (double)(r / TR) * NT + nt_t + 0.5 * ntiles;
+                double cost;
+                if (pairs && wgs > cus)
+                    cost = (double)((wgs + 2 * cus - 1) / (2 * cus)) * 1.4 * (work + 1.0 + (trw_t ? 0.5 : 0.0));
+                else
+                    cost = (double)((wgs + cus - 1) / cus) * work;
                 if (cost < best - 1e-9) { best = cost; RPW = r; }
             }
             const char* e = getenv("MJT_CONV_RPW");
