@@ -130,6 +130,22 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
         }
     });
 
+    // An output width that is no multiple of 8: the last piece of dy that a row has ends in the next row's first columns.
+    // The fragments of x are zero there (the masks above), but a product with zero is only zero for finite values, so the
+    // lane group that holds that piece clears what lies beyond the row in dy as well.
+    constexpr bool DY_TAIL = OW_ % 8 != 0;
+    mjt_u32x4v dy_mask = (mjt_u32x4v)(0xffffffffu);
+    if constexpr (DY_TAIL) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            unsigned v = 0;
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                if ((NCHUNK - 1) * 32 + lg * 8 + 2 * j + h < OW_) v |= h ? 0xffff0000u : 0x0000ffffu;
+            dy_mask[j] = v;
+        }
+    }
+
     // buffer descriptors over the whole tensors; every offset is a lane offset, so the range check sees all of it
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.a[0], 0, n_img * (C_ * H_ * W_ * 2), 0x00020000);
     const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.a[1], 0, n_img * (K_ * OH_ * OW_ * 2), 0x00020000);
@@ -349,6 +365,7 @@ extern "C" __global__ __launch_bounds__(512) void ENTRY(Params p) {
             if constexpr (s == 0) {                                      // the reads of this tap row (and, in front of them, of dy) have arrived
                 constexpr int later = 3 * (R_ - 1 - r) + AFTER;
                 if constexpr (r == 0) mjt_static_for<0, 4>([&](auto mc) { mjt_lds_wait<later + 3>(afrag[U][decltype(mc)::v]); });
+                if constexpr (r == 0 && DY_TAIL && CH == NCHUNK - 1) mjt_static_for<0, 4>([&](auto mc) { afrag[U][decltype(mc)::v] &= dy_mask; });
                 mjt_lds_wait<later + 2>(bd[U][r]);
                 mjt_lds_wait1<later + 1>(bp[U][r]);
                 mjt_lds_wait2<later>(bn[U][r]);

@@ -623,7 +623,7 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
     const int64_t CTW = 8 / KG;
     const bool half = x->dtype == MJT_FLOAT16;
     const bool ok = G == 1 && (x->dtype == MJT_BFLOAT16 || half) && dy->dtype == x->dtype && (dw->dtype == MJT_FLOAT32 || dw->dtype == x->dtype) &&
-                    p->stride_w == 1 && p->pad_w <= 2 && (S - 1) * p->dil_w - p->pad_w <= 4 && K % 64 == 0 && C % 16 == 0 && (C % (16 * CTW) == 0 || C % (16 * CTW) >= 8 * CTW) && R * S <= 9 && OW % 8 == 0 &&
+                    p->stride_w == 1 && p->pad_w <= 2 && (S - 1) * p->dil_w - p->pad_w <= 4 && K % 64 == 0 && C % 16 == 0 && (C % (16 * CTW) == 0 || C % (16 * CTW) >= 8 * CTW) && R * S <= 9 && OW % 2 == 0 &&
                     W % 2 == 0 && N >= 1 && numel(x) * 2 < (int64_t(1) << 31) && numel(dy) * 2 < (int64_t(1) << 31) &&
                     (uintptr_t)x->ptr % 4 == 0 && (uintptr_t)dy->ptr % 16 == 0 &&
                     !getenv("MJT_NO_FASTPATH");
@@ -633,7 +633,7 @@ void conv_wgrad_impl(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor
     }
     if (!ok)
         MJT_FAIL(MJT_ERR_UNSUPPORTED, "conv wgrad: only bfloat16 or float16 operands with horizontal stride 1, column shifts of the taps within -2 .. 4, at most 9 taps, "
-                                      "K % 64 == 0, C % 16 == 0 (the last block of " << 16 * CTW << " channels at least half full), OW % 8 == 0 and tensors below 2 GB run on the MFMA kernel");
+                                      "K % 64 == 0, C % 16 == 0 (the last block of " << 16 * CTW << " channels at least half full), even OW and tensors below 2 GB run on the MFMA kernel");
     Context& c = ctx();
     const int64_t cus = c.dry_run || c.prop.multiProcessorCount <= 0 ? 256 : c.prop.multiProcessorCount;
     const int64_t blocks_per_slice = (K / (64 * KG)) * ((C + 16 * CTW - 1) / (16 * CTW));   // the last block of channels may be partly idle

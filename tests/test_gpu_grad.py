@@ -209,11 +209,12 @@ def test_grad_meta_conv(gpu, case):
 
 
 @pytest.mark.parametrize("xs,ws,wgrad_kernel", [((2, 32, 16, 16), (64, 32, 3, 3), 0), ((2, 64, 16, 16), (64, 64, 3, 3), 1),
-                                                    ((2, 128, 8, 16), (64, 128, 3, 3), 1)])
+                                                    ((2, 128, 8, 16), (64, 128, 3, 3), 1), ((2, 64, 28, 28), (64, 64, 3, 3), 1)])
 def test_grad_meta_conv_bfloat16(gpu, xs, ws, wgrad_kernel):
     """The same three units for bfloat16 operands (conv2d builds them under amp_reg | 36, so the sums keep
     16 bit without casts): the MFMA kernel runs forward and input gradient; the weight gradient runs on its
-    own MFMA kernel where that applies (64 input channels: half a block of its workgroup; 128: a whole one) and as
+    own MFMA kernel where that applies (64 input channels: half a block of its workgroup; 128: a whole one; 28 columns: rows
+    whose last piece is shared with the next row) and as
     a batched GEMM over shifted input planes otherwise (first case: 32 input channels); gradients keep the dtype of
     their variable."""
     rng = np.random.default_rng(8)

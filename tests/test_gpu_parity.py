@@ -1181,6 +1181,13 @@ def _wgrad_call(xbits, dybits, R, S, params, out_dtype="float32", in_dtype="bflo
     dict(x=(3, 128, 9, 8), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1), rps=5),    # slices of 5 output rows: they start and end inside images
     dict(x=(3, 128, 9, 40), k=64, rs=(3, 3), p=(2, 1, 1, 1, 1, 1), rps=4),   # 5 output rows per image (stride 2), slices of 4; two chunks
     dict(x=(2, 128, 7, 8), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1), rps=1),    # one row per slice
+    dict(x=(3, 128, 28, 28), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),      # 28 output columns: the row's last piece of dy is half the next row's
+    dict(x=(4, 64, 14, 14), k=128, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),      # 14 columns: six of the second piece
+    dict(x=(2, 128, 9, 36), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),       # 36 columns: a second chunk of four
+    dict(x=(2, 64, 12, 12), k=64, rs=(1, 3), p=(1, 1, 0, 1, 1, 1), out="bfloat16"),
+    dict(x=(3, 128, 7, 6), k=64, rs=(3, 3), p=(1, 1, 1, 1, 1, 1)),        # six columns: rows shorter than a piece
+    dict(x=(2, 128, 27, 30), k=64, rs=(3, 3), p=(2, 1, 1, 1, 1, 1)),      # vertical stride 2 onto 14 rows of 30 columns
+    dict(x=(2, 128, 10, 22), k=64, rs=(3, 3), p=(1, 1, 2, 2, 2, 2)),      # dilation 2 on 22 columns
 ])
 def test_conv_wgrad_mfma_matches_oracle(gpu, case, monkeypatch):
     """The weight gradient kernel through the C entry point against the oracle's restatement of the
@@ -1215,6 +1222,33 @@ def test_conv_wgrad_mfma_matches_oracle(gpu, case, monkeypatch):
     if N * K * C * OH * OW * R * S <= 4e7 and sh == sw and ph == pw and dh == dw_:
         ref = O.conv_meta_wgrad(O.BF16(xb), O.BF16(db), R, S, sh, ph, dh)     # the reference's own summation order
         assert np.abs(got - ref).max() <= (1e-4 if out == "float32" else 2.0 ** -7) * np.abs(ref).max()
+
+
+def test_conv_wgrad_mfma_keeps_an_infinite_dy_in_its_row(gpu):
+    """With 28 output columns a row's last 16-byte piece of dy holds the first four values of the next row.  An infinity
+    there must not reach the sums of the row before it (0 x inf is NaN): the non-finite entries of dw are exactly those of
+    the float64 evaluation, with their signs, and the finite ones agree."""
+    rng = np.random.default_rng(33)
+    N, C, K, H = 2, 128, 64, 28
+    xb = _bf16(rng.standard_normal((N, C, H, H)) + 3.0)        # no zeros and no sign changes: every product with inf is +inf or -inf
+    d = rng.standard_normal((N, K, H, H)).astype(np.float32)
+    d[0, 3, 5, 0] = np.inf                                     # first column of a row: in the tail of the piece that ends row 4
+    d[1, 9, 0, 2] = -np.inf
+    db = _bf16(d)
+    rc, got = _wgrad_call(xb, db, 3, 3, (1, 1, 1, 1, 1, 1))
+    assert rc == 0 and L.last_kernel().startswith("mjt_conv_wgrad_mfma_bf16")
+    xf, df = O.BF16(xb).to_f32().astype(np.float64), O.BF16(db).to_f32().astype(np.float64)
+    xp = np.pad(xf, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    want = np.zeros((K, C, 3, 3))
+    with np.errstate(invalid="ignore"):
+        for r in range(3):
+            for s in range(3):
+                want[:, :, r, s] = np.einsum("nkhw,nchw->kc", df, xp[:, :, r:r + H, s:s + H])
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(np.isposinf(got), np.isposinf(want)) and np.array_equal(np.isneginf(got), np.isneginf(want))
+    fin = np.isfinite(want)
+    assert fin.sum() > 0.9 * want.size and not fin.all()
+    assert np.abs(got[fin] - want[fin]).max() <= 1e-4 * np.abs(want[fin]).max()
 
 
 @pytest.mark.parametrize("case", [
