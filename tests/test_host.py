@@ -551,9 +551,10 @@ def test_conv_input_gradient_entry_validates_and_picks_its_path(compile_only):
 def test_conv_builds_that_ran_out_of_registers_are_not_run(compile_only):
     """The MFMA convolution keeps loads under way in registers the compiler does not track, which is sound only while the
     compiler moves no register aside.  The library reads each build's register figures from the code object: a geometry
-    whose build stays within a wave's registers runs on the kernel (among them 32 output channels on two waves, which once
-    did not), one whose build needs more (4-column maps: 58 staging items per wave) takes another route.  That the first
-    group still names the MFMA kernel also shows that the figures are found at all."""
+    whose build stays within a wave's registers runs on the kernel (among them 32 output channels on two waves and 4-column
+    maps, whose builds once did not), one whose build needs more takes another route (the weight-gradient kernel on rows of
+    104 columns).  That the first group names the MFMA kernel also shows that the figures are found at all: a build whose
+    figures are missing is not run either."""
     lib = L.load()
     P = 0x100000
 
@@ -569,7 +570,7 @@ def test_conv_builds_that_ran_out_of_registers_are_not_run(compile_only):
 
     assert call((2, 64, 16, 16), (32, 64, 3, 3)).startswith("mjt_conv_mfma_bf16")
     assert call((2, 64, 16, 16), (64, 64, 3, 3)).startswith("mjt_conv_mfma_bf16")
-    assert call((2, 32, 40, 4), (64, 32, 3, 3)).startswith("mjt_conv_igemm")
+    assert call((2, 32, 40, 4), (64, 32, 3, 3)).startswith("mjt_conv_mfma_bf16")
     # the weight gradient kernel likewise: rows of 104 columns need more registers than there are
     x, dy = L.tensor(P, "bfloat16", (4, 64, 10, 104)), L.tensor(P, "bfloat16", (4, 64, 10, 104))
     dw, p = L.tensor(P, "float32", (64, 64, 3, 3)), L.ConvParams(1, 1, 1, 1, 1, 1)
