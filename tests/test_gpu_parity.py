@@ -275,7 +275,8 @@ def test_window_gather_fast_path_matches_oracle_and_generic(gpu, case, dtype):
     dict(x=(8, 4, 7, 7), k=(3, 3), s=(1, 1), d=(1, 1), p=(1, 1), nb=0),               # 49-pixel planes, the whole batch side by side
     dict(x=(6, 2, 27, 27), k=(3, 3), s=(2, 2), d=(1, 1), p=(1, 1), nb=3),             # stride 2; three images: vectors of 4
     dict(x=(2, 3, 14, 13), k=(2, 3), s=(1, 2), d=(2, 1), p=(0, 2), nb=None),          # mixed stride / dilation, no vertical padding
-    dict(x=(3, 2, 9, 9), k=(1, 1), s=(1, 1), d=(1, 1), p=(0, 0), nb=None),            # 1x1 taps, 81 pixels per run: single elements
+    dict(x=(3, 2, 9, 9), k=(1, 2), s=(1, 1), d=(1, 1), p=(0, 0), nb=None),            # 1x2 taps, 72 pixels per run
+    dict(x=(3, 2, 9, 9), k=(3, 3), s=(1, 1), d=(1, 1), p=(1, 1), nb=None),            # 81 pixels per run: single elements
     # (maps of up to 64 pixels read the other way round, taps as pixels and pixels as taps, are the sliding-window gather's)
     dict(x=(2, 2, 40, 56), k=(5, 5), s=(1, 1), d=(1, 1), p=(2, 2), nb=None),          # 25 taps on a larger plane
 ])
