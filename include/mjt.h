@@ -339,7 +339,8 @@ int mjt_conv2d_meta_dgrad(const mjt_tensor* dy, const mjt_tensor* w, const mjt_t
  * x [N,C,H,W] and dy [N,K,OH,OW] bfloat16 or float16, dw [K,C,R,S] float32 or their dtype
  * (float32 accumulation, rounded once).  One MFMA kernel plus a reduce over
  * slices of images; shapes it does not cover (horizontal stride > 1, more
- * than 9 taps, left padding > 2, K % 64 != 0, ...) return MJT_ERR_UNSUPPORTED
+ * than 9 taps, left padding > 2, K % 64 != 0, an odd OW or W, a geometry whose
+ * kernel would need more registers than a wave has, ...) return MJT_ERR_UNSUPPORTED
  * and are the caller's to run through mjt_matmul or mjt_conv2d_meta. */
 int mjt_conv2d_meta_wgrad(const mjt_tensor* x, const mjt_tensor* dy, const mjt_tensor* dw,
                           const mjt_conv_params* p);
